@@ -1,0 +1,63 @@
+// Shared host/device helpers for the gfx950 matrix backend.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "../../include/cudamat_amd.h"
+
+#define WAVE 64
+
+// One CU count for launch sizing; MI355X has 256 CUs in 8 XCDs.  Queried once.
+int dn_num_cus();
+
+// Records the launch status of the kernel just queued; returns CUDA_ERROR or 0.
+static inline int dn_launch_status() {
+  return hipPeekAtLastError() == hipSuccess ? 0 : CUDA_ERROR;
+}
+
+static inline bool dn_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+static inline long long dn_len(const cudamat* m) { return (long long)m->size[0] * (long long)m->size[1]; }
+
+// Division of a 32-bit index by a run-time constant without the hardware-less
+// integer divide: q = (n * magic) >> 32 >> shift for n < 2^31.
+struct FastDiv {
+  uint32_t magic;
+  uint32_t shift;
+  uint32_t d;
+};
+
+static inline FastDiv make_fastdiv(uint32_t d) {
+  FastDiv f;
+  f.d = d;
+  if (d <= 1) { f.magic = 0; f.shift = 0; return f; }
+  uint32_t s = 0;
+  while ((1ull << s) < d) ++s;            // s = ceil(log2 d)
+  uint64_t m = ((1ull << 32) * ((1ull << s) - d)) / d + 1;
+  f.magic = (uint32_t)m;
+  f.shift = s;
+  return f;
+}
+
+// Exact for every 32-bit n (round-up method: q = (hi + ((n - hi) >> 1)) >> (s-1)).
+__device__ __forceinline__ uint32_t fd_div(uint32_t n, const FastDiv& f) {
+  if (f.d <= 1) return n;
+  uint32_t hi = __umulhi(n, f.magic);
+  return (hi + ((n - hi) >> 1)) >> (f.shift - 1);
+}
+
+// Wave-wide reductions through cross-lane shuffles (wave64).
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, WAVE));
+  return v;
+}
+__device__ __forceinline__ double wave_sum_d(double v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+  return v;
+}

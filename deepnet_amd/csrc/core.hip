@@ -1,0 +1,254 @@
+// Handle lifetime, device memory, transfers, views, row slices and transpose.
+// Replaces cudamat/cudamat.cu:25-53, 87-123, 153-186, 217-434 and the copy
+// kernels cudamat_kernels.cu:247-294.
+#include "common.h"
+#include <stdio.h>
+#include <string.h>
+
+static int g_num_cus = 0;
+
+int dn_num_cus() {
+  if (g_num_cus == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+      g_num_cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+    else
+      g_num_cus = 256;
+  }
+  return g_num_cus;
+}
+
+// ------------------------------------------------------------------ kernels
+
+// Column-major row-band copy: dst(r, c) = src(r + row0, c) for a band of `rows`
+// rows; threads run down a column so both sides are read/written in 256-byte
+// runs.  src_ld / dst_ld are the two leading dimensions.
+__global__ void k_copy_rows(const float* src, float* dst, int rows, int cols, int src_ld, int dst_ld,
+                            int src_row0, int dst_row0) {
+  const int r = blockIdx.x * blockDim.x + threadIdx.x;
+  if (r >= rows) return;
+  for (int c = blockIdx.y; c < cols; c += gridDim.y)
+    dst[(size_t)c * dst_ld + dst_row0 + r] = src[(size_t)c * src_ld + src_row0 + r];
+}
+
+// Out-of-place transpose through a 64x64 LDS tile (+1 column of padding so the
+// transposed read walks distinct banks).  in is h x w column-major, out is w x h.
+#define TR_TILE 64
+__global__ void __launch_bounds__(256) k_transpose(const float* in, float* out, int h, int w) {
+  __shared__ float tile[TR_TILE][TR_TILE + 1];
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;  // 64 x 4
+  const int r0 = blockIdx.x * TR_TILE, c0 = blockIdx.y * TR_TILE;
+#pragma unroll
+  for (int j = ty; j < TR_TILE; j += 4) {
+    const int r = r0 + tx, c = c0 + j;
+    if (r < h && c < w) tile[j][tx] = in[(size_t)c * h + r];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int j = ty; j < TR_TILE; j += 4) {
+    const int c = c0 + tx, r = r0 + j;  // out(c, r) = in(r, c)
+    if (r < h && c < w) out[(size_t)r * w + c] = tile[tx][j];
+  }
+}
+
+// ------------------------------------------------------------------ C ABI
+
+extern "C" {
+
+const char* get_last_cuda_error(void) { return hipGetErrorString(hipGetLastError()); }
+
+int cublas_init(void) {
+  // Nothing to create: the contraction kernels are part of this library.  Touch
+  // the device so a missing GPU is reported here rather than at the first op.
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess || n <= 0) return CUBLAS_ERROR;
+  return 0;
+}
+
+int cublas_shutdown(void) {
+  hipDeviceSynchronize();
+  return 0;
+}
+
+int cuda_set_device(int deviceId) {
+  if (hipSetDevice(deviceId) != hipSuccess) return CUDA_ERROR;
+  g_num_cus = 0;
+  return 0;
+}
+
+void cuda_sync_threads(void) { hipDeviceSynchronize(); }
+
+int get_leading_dimension(cudamat* mat) { return mat->is_trans ? mat->size[1] : mat->size[0]; }
+int get_nonleading_dimension(cudamat* mat) { return mat->is_trans ? mat->size[0] : mat->size[1]; }
+void set_transpose(cudamat* mat, int is_trans) { mat->is_trans = is_trans; }
+
+int allocate_device_memory(cudamat* mat) {
+  const long long len = dn_len(mat);
+  void* p = nullptr;
+  // A 0-element matrix still gets a distinct, valid pointer.
+  const size_t bytes = (size_t)(len > 0 ? len : 1) * sizeof(float);
+  if (hipMalloc(&p, bytes) != hipSuccess) {
+    hipGetLastError();
+    return CUBLAS_ERROR;
+  }
+  mat->data_device = (float*)p;
+  mat->on_device = 1;
+  return 0;
+}
+
+int copy_to_host(cudamat* mat) {
+  if (!mat->on_device) return ERROR_NOT_ON_DEVICE;
+  const long long len = dn_len(mat);
+  if (len > 0 &&
+      hipMemcpy(mat->data_host, mat->data_device, (size_t)len * sizeof(float), hipMemcpyDeviceToHost) != hipSuccess)
+    return CUBLAS_ERROR;
+  return 0;
+}
+
+int copy_to_device(cudamat* mat) {
+  if (!mat->on_device) {
+    int err = allocate_device_memory(mat);
+    if (err) return err;
+  }
+  const long long len = dn_len(mat);
+  if (len > 0 &&
+      hipMemcpy(mat->data_device, mat->data_host, (size_t)len * sizeof(float), hipMemcpyHostToDevice) != hipSuccess)
+    return CUBLAS_ERROR;
+  return 0;
+}
+
+int copy_on_device(cudamat* mat1, cudamat* mat2) {
+  if (mat1->size[0] != mat2->size[0] || mat1->size[1] != mat2->size[1]) return ERROR_INCOMPATIBLE_DIMENSIONS;
+  const long long len = dn_len(mat1);
+  if (len > 0 && mat1->data_device != mat2->data_device &&
+      hipMemcpyAsync(mat2->data_device, mat1->data_device, (size_t)len * sizeof(float), hipMemcpyDeviceToDevice,
+                     0) != hipSuccess)
+    return CUBLAS_ERROR;
+  return 0;
+}
+
+int free_device_memory(cudamat* mat) {
+  if (mat->owns_data && mat->on_device) {
+    hipError_t e = hipFree(mat->data_device);
+    mat->on_device = 0;
+    if (e != hipSuccess) return CUBLAS_ERROR;
+  }
+  return 0;
+}
+
+int set_shape(cudamat* mat, unsigned int m, unsigned int n) {
+  mat->size[0] = m;
+  mat->size[1] = n;
+  return 0;
+}
+
+int reshape(cudamat* mat, unsigned int m, unsigned int n) {
+  if ((unsigned int)(mat->size[0] * mat->size[1]) != m * n) return ERROR_INCOMPATIBLE_DIMENSIONS;
+  mat->size[0] = m;
+  mat->size[1] = n;
+  return 0;
+}
+
+int get_slice(cudamat* source, cudamat* target, unsigned int first_col, unsigned int last_col) {
+  if (source->is_trans) return ERROR_TRANSPOSED;
+  if (!source->on_device) return ERROR_NOT_ON_DEVICE;
+  if (last_col > (unsigned int)source->size[1] || first_col >= last_col) return ERROR_INCOMPATIBLE_DIMENSIONS;
+  const int num_rows = source->size[0];
+  target->data_host = 0;
+  target->data_device = source->data_device + (size_t)first_col * num_rows;
+  target->on_device = 1;
+  target->on_host = 0;
+  target->size[0] = source->size[0];
+  target->size[1] = last_col - first_col;
+  target->is_trans = 0;
+  target->owns_data = 0;
+  return 0;
+}
+
+int get_vector_slice(cudamat* source, cudamat* target, unsigned int first_ind, unsigned int last_ind) {
+  if (source->size[0] > 1 && source->size[1] > 1) return ERROR_GENERIC;
+  if (source->is_trans) return ERROR_TRANSPOSED;
+  if (!source->on_device) return ERROR_NOT_ON_DEVICE;
+  if (first_ind >= last_ind) return ERROR_INCOMPATIBLE_DIMENSIONS;
+  const int num_rows = source->size[0];
+  // The reference offsets by first_ind * num_rows for both orientations
+  // (cudamat.cu:369-372); for a column vector that walks first_ind whole
+  // columns, i.e. past the data for any first_ind > 0.  Offset by elements.
+  (void)num_rows;
+  target->data_host = 0;
+  target->data_device = source->data_device + first_ind;
+  target->on_device = 1;
+  target->on_host = 0;
+  target->is_trans = 0;
+  target->owns_data = 0;
+  if (source->size[0] > 1) {
+    if (last_ind > (unsigned int)source->size[0]) return ERROR_INCOMPATIBLE_DIMENSIONS;
+    target->size[0] = last_ind - first_ind;
+    target->size[1] = 1;
+  } else {
+    if (last_ind > (unsigned int)source->size[1]) return ERROR_INCOMPATIBLE_DIMENSIONS;
+    target->size[0] = 1;
+    target->size[1] = last_ind - first_ind;
+  }
+  return 0;
+}
+
+void init_from_array(cudamat* mat, float* data, int m, int n) {
+  mat->data_host = data;
+  mat->size[0] = m;
+  mat->size[1] = n;
+  mat->on_device = 0;
+  mat->on_host = 1;
+  mat->is_trans = 0;
+  mat->owns_data = 1;
+}
+
+void set_on_device(cudamat* mat) { mat->on_device = 1; }
+
+int init_empty(cudamat* mat, int m, int n) {
+  mat->size[0] = m;
+  mat->size[1] = n;
+  mat->on_device = 0;
+  mat->on_host = 0;
+  mat->is_trans = 0;
+  mat->owns_data = 1;
+  return allocate_device_memory(mat);
+}
+
+int get_row_slice(cudamat* source, cudamat* target, unsigned int start, unsigned int end) {
+  const int height = source->size[0], width = source->size[1];
+  if ((end - start) != (unsigned int)target->size[0] || source->size[1] != target->size[1] || start >= end ||
+      end > (unsigned int)height)
+    return ERROR_INCOMPATIBLE_DIMENSIONS;
+  const int rows = end - start;
+  if (width == 0) return 0;
+  dim3 grid((rows + 255) / 256, width < 4096 ? width : 4096);
+  hipLaunchKernelGGL(k_copy_rows, grid, dim3(256), 0, 0, source->data_device, target->data_device, rows, width,
+                     height, rows, (int)start, 0);
+  return dn_launch_status();
+}
+
+int set_row_slice(cudamat* source, cudamat* target, unsigned int start, unsigned int end) {
+  const int height = target->size[0], width = target->size[1];
+  if ((end - start) != (unsigned int)source->size[0] || source->size[1] != target->size[1] || start >= end ||
+      end > (unsigned int)height)
+    return ERROR_INCOMPATIBLE_DIMENSIONS;
+  const int rows = end - start;
+  if (width == 0) return 0;
+  dim3 grid((rows + 255) / 256, width < 4096 ? width : 4096);
+  hipLaunchKernelGGL(k_copy_rows, grid, dim3(256), 0, 0, source->data_device, target->data_device, rows, width, rows,
+                     height, 0, (int)start);
+  return dn_launch_status();
+}
+
+int copy_transpose(cudamat* source, cudamat* target) {
+  const int height = source->size[0], width = source->size[1];
+  if (source->size[0] != target->size[1] || source->size[1] != target->size[0]) return ERROR_INCOMPATIBLE_DIMENSIONS;
+  if (height == 0 || width == 0) return 0;
+  dim3 grid((height + TR_TILE - 1) / TR_TILE, (width + TR_TILE - 1) / TR_TILE);
+  hipLaunchKernelGGL(k_transpose, grid, dim3(256), 0, 0, source->data_device, target->data_device, height, width);
+  return dn_launch_status();
+}
+
+}  // extern "C"

@@ -1,0 +1,482 @@
+// Elementwise, scalar, comparison and broadcast ops over column-major fp32.
+// Replaces the grid-stride kernels of cudamat/cudamat_kernels.cu:298-716 and
+// their wrappers cudamat/cudamat.cu:592-1146, 1318-1669, 1763-2102.
+//
+// All of these are HBM-bound.  One templated kernel moves 16-byte vectors with
+// four independent loads in flight per lane; operands that are not 16-byte
+// aligned (column views) are peeled to alignment when they share the same
+// offset and fall back to 4-byte accesses otherwise.
+#include "common.h"
+#include <math.h>
+
+// ------------------------------------------------------------------ functors
+// f(a, b): a = first input, b = second input (unused for unary ops).
+
+#define DN_FUNCTOR0(NAME, EXPR)                                           \
+  struct NAME {                                                           \
+    __device__ __forceinline__ float operator()(float a, float b) const { \
+      (void)a; (void)b;                                                   \
+      return (EXPR);                                                      \
+    }                                                                     \
+  };
+#define DN_FUNCTOR1(NAME, EXPR)                                           \
+  struct NAME {                                                           \
+    float s;                                                              \
+    __device__ __forceinline__ float operator()(float a, float b) const { \
+      (void)a; (void)b;                                                   \
+      return (EXPR);                                                      \
+    }                                                                     \
+  };
+
+// unary (cudamat_kernels.cu:386-506)
+DN_FUNCTOR0(FSign, a ? copysignf(1.f, a) : 0.f)
+DN_FUNCTOR0(FCos, cosf(a))
+DN_FUNCTOR0(FSin, sinf(a))
+DN_FUNCTOR0(FSigmoid, 1.f / (1.f + expf(-a)))
+// 1 - 2/(exp(2x)+1) is tanh(x); evaluated as tanhf so the result carries the accuracy of
+// the formula itself rather than the cancellation of its fp32 steps near 0.
+DN_FUNCTOR0(FTanh, tanhf(a))
+DN_FUNCTOR0(FAbs, a * (float)((a > 0.f) - (a < 0.f)))
+DN_FUNCTOR0(FLog1pExp, a > 0.f ? (log1pf(expf(-a)) + a) : log1pf(expf(a)))
+DN_FUNCTOR1(FLog, logf(a + s))
+DN_FUNCTOR0(FExp, expf(a))
+DN_FUNCTOR0(FCeil, ceilf(a))
+DN_FUNCTOR0(FFloor, floorf(a))
+DN_FUNCTOR0(FSqrt, sqrtf(a))
+DN_FUNCTOR1(FPow, powf(a, s))
+DN_FUNCTOR0(FRecip, (float)(1.0 / (double)a))
+// binary (cudamat_kernels.cu:298-364, 476-500, 600-685)
+DN_FUNCTOR0(FLt, a < b ? 1.f : 0.f)
+DN_FUNCTOR0(FLe, a <= b ? 1.f : 0.f)
+DN_FUNCTOR0(FGt, a > b ? 1.f : 0.f)
+DN_FUNCTOR0(FGe, a >= b ? 1.f : 0.f)
+DN_FUNCTOR0(FUpper, a > b ? b : a)
+DN_FUNCTOR0(FLower, a < b ? b : a)
+DN_FUNCTOR0(FAdd, a + b)
+DN_FUNCTOR0(FSub, a - b)
+DN_FUNCTOR0(FDiv, a / b)
+DN_FUNCTOR0(FMul, a * b)
+DN_FUNCTOR0(FPowMat, powf(a, b))
+DN_FUNCTOR0(FCosDeriv, -a * sinf(b))
+DN_FUNCTOR0(FSinDeriv, a * cosf(b))
+DN_FUNCTOR0(FLogisticDeriv, (float)((double)(a * b) * (1.0 - (double)b)))
+DN_FUNCTOR0(FTanhDeriv, (float)((double)a * (1.0 + (double)b) * (1.0 - (double)b) * 0.5))
+DN_FUNCTOR0(FReluDeriv, a * (b > 0.f ? 1.f : 0.f))
+DN_FUNCTOR0(FReluSmoothDeriv, a * -expm1f(-b))
+DN_FUNCTOR1(FAxpy, a + s * b)
+DN_FUNCTOR1(FAddMultSign, a + ((b > 0.f) ? s : ((b < 0.f) ? -s : 0.f)))
+DN_FUNCTOR1(FCrossEntropy, -a * logf(b + s))
+DN_FUNCTOR1(FCrossEntropyBernoulli, -a * logf(b + s) - (1.f - a) * logf(1.f - b + s))
+DN_FUNCTOR1(FCorrectPreds, a * (float)(b >= s) + (1.f - a) * (float)(b < s))
+// matrix (op) scalar (cudamat_kernels.cu:310-364, 687-716)
+DN_FUNCTOR1(FLtS, a < s ? 1.f : 0.f)
+DN_FUNCTOR1(FLeS, a <= s ? 1.f : 0.f)
+DN_FUNCTOR1(FGtS, a > s ? 1.f : 0.f)
+DN_FUNCTOR1(FGeS, a >= s ? 1.f : 0.f)
+DN_FUNCTOR1(FUpperS, a > s ? s : a)
+DN_FUNCTOR1(FLowerS, a < s ? s : a)
+DN_FUNCTOR1(FMulS, s * a)
+DN_FUNCTOR1(FDivS, a / s)
+DN_FUNCTOR1(FAddS, a + s)
+DN_FUNCTOR1(FAssignS, s)
+
+// ------------------------------------------------------------------ kernels
+
+#define EW_THREADS 256
+#define EW_UNROLL 4
+
+// NIN inputs (0, 1 or 2) -> one output.  [head, head + 4*n4) is moved as
+// 16-byte vectors; the up-to-3 leading and trailing elements by single lanes.
+template <int NIN, class F>
+__global__ void __launch_bounds__(EW_THREADS)
+k_ew(const float* a, const float* b, float* t, long long n, int head, long long n4, F f) {
+  const long long tid = (long long)blockIdx.x * EW_THREADS + threadIdx.x;
+  const long long stride = (long long)gridDim.x * EW_THREADS;
+  const float4* a4 = reinterpret_cast<const float4*>(a + head);
+  const float4* b4 = reinterpret_cast<const float4*>(b + head);
+  float4* t4 = reinterpret_cast<float4*>(t + head);
+  for (long long i = tid; i < n4; i += stride * EW_UNROLL) {
+    float4 va[EW_UNROLL], vb[EW_UNROLL];
+#pragma unroll
+    for (int u = 0; u < EW_UNROLL; ++u) {
+      const long long j = i + u * stride;
+      if (j < n4) {
+        if (NIN >= 1) va[u] = a4[j];
+        if (NIN >= 2) vb[u] = b4[j];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < EW_UNROLL; ++u) {
+      const long long j = i + u * stride;
+      if (j < n4) {
+        float4 r;
+        r.x = f(va[u].x, vb[u].x);
+        r.y = f(va[u].y, vb[u].y);
+        r.z = f(va[u].z, vb[u].z);
+        r.w = f(va[u].w, vb[u].w);
+        t4[j] = r;
+      }
+    }
+  }
+  // ragged ends
+  const long long tail0 = head + 4 * n4;
+  if (tid < head) {
+    t[tid] = f(NIN >= 1 ? a[tid] : 0.f, NIN >= 2 ? b[tid] : 0.f);
+  } else if (tid - head < n - tail0) {
+    const long long j = tail0 + (tid - head);
+    t[j] = f(NIN >= 1 ? a[j] : 0.f, NIN >= 2 ? b[j] : 0.f);
+  }
+}
+
+// Fallback for operands whose 16-byte phases differ: 4-byte accesses.
+template <int NIN, class F>
+__global__ void __launch_bounds__(EW_THREADS) k_ew_scalar(const float* a, const float* b, float* t, long long n, F f) {
+  const long long stride = (long long)gridDim.x * EW_THREADS;
+  for (long long i = (long long)blockIdx.x * EW_THREADS + threadIdx.x; i < n; i += stride)
+    t[i] = f(NIN >= 1 ? a[i] : 0.f, NIN >= 2 ? b[i] : 0.f);
+}
+
+static inline int head_of(const void* p) {  // elements until the next 16-byte boundary
+  return (int)(((16u - (reinterpret_cast<uintptr_t>(p) & 15u)) & 15u) >> 2);
+}
+
+template <int NIN, class F>
+static int launch_ew(const float* a, const float* b, float* t, long long n, F f) {
+  if (n <= 0) return 0;
+  const int cus = dn_num_cus();
+  const int ht = head_of(t);
+  const bool same_phase = (NIN < 1 || head_of(a) == ht) && (NIN < 2 || head_of(b) == ht) &&
+                          ((reinterpret_cast<uintptr_t>(t) & 3u) == 0);
+  if (same_phase) {
+    const int head = (int)(ht < n ? ht : n);
+    const long long n4 = (n - head) / 4;
+    long long blocks = (n4 + (long long)EW_THREADS * EW_UNROLL - 1) / ((long long)EW_THREADS * EW_UNROLL);
+    const long long cap = (long long)cus * 16;
+    if (blocks > cap) blocks = cap;
+    if (blocks < 1) blocks = 1;
+    hipLaunchKernelGGL((k_ew<NIN, F>), dim3((unsigned)blocks), dim3(EW_THREADS), 0, 0, a, b, t, n, head, n4, f);
+  } else {
+    long long blocks = (n + EW_THREADS - 1) / EW_THREADS;
+    const long long cap = (long long)cus * 32;
+    if (blocks > cap) blocks = cap;
+    hipLaunchKernelGGL((k_ew_scalar<NIN, F>), dim3((unsigned)blocks), dim3(EW_THREADS), 0, 0, a, b, t, n, f);
+  }
+  return dn_launch_status();
+}
+
+// Broadcast of a vector along rows (vec[i % h], a column vector) or along
+// columns (vec[i / h], a row vector) into a flat pass over the matrix.  The
+// row / column of the first element of each 16-byte group comes from one
+// multiply-high; the other three follow by increment-and-wrap.
+template <bool COLVEC, class F>
+__global__ void __launch_bounds__(EW_THREADS)
+k_bcast(const float* a, const float* vec, float* t, long long n, int head, long long n4, FastDiv fd, F f) {
+  const long long tid = (long long)blockIdx.x * EW_THREADS + threadIdx.x;
+  const long long stride = (long long)gridDim.x * EW_THREADS;
+  const uint32_t h = fd.d;
+  if (n4 > 0) {
+    const float4* a4 = reinterpret_cast<const float4*>(a + head);
+    float4* t4 = reinterpret_cast<float4*>(t + head);
+    for (long long i = tid; i < n4; i += stride * EW_UNROLL) {
+      float4 va[EW_UNROLL];
+#pragma unroll
+      for (int u = 0; u < EW_UNROLL; ++u) {
+        const long long j = i + u * stride;
+        if (j < n4) va[u] = a4[j];
+      }
+#pragma unroll
+      for (int u = 0; u < EW_UNROLL; ++u) {
+        const long long j = i + u * stride;
+        if (j < n4) {
+          const uint32_t e = (uint32_t)(head + 4 * j);
+          uint32_t q = fd_div(e, fd);
+          uint32_t r = e - q * h;
+          float v[4];
+          const float x[4] = {va[u].x, va[u].y, va[u].z, va[u].w};
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            v[k] = f(x[k], vec[COLVEC ? r : q]);
+            if (++r == h) { r = 0; ++q; }
+          }
+          t4[j] = make_float4(v[0], v[1], v[2], v[3]);
+        }
+      }
+    }
+  }
+  const long long tail0 = head + 4 * n4;
+  long long j = -1;
+  if (tid < head) j = tid;
+  else if (tid - head < n - tail0) j = tail0 + (tid - head);
+  if (j >= 0) {
+    const uint32_t q = fd_div((uint32_t)j, fd);
+    const uint32_t r = (uint32_t)j - q * h;
+    t[j] = f(a[j], vec[COLVEC ? r : q]);
+  }
+}
+
+template <bool COLVEC, class F>
+__global__ void __launch_bounds__(EW_THREADS)
+k_bcast_scalar(const float* a, const float* vec, float* t, long long n, FastDiv fd, F f) {
+  const long long stride = (long long)gridDim.x * EW_THREADS;
+  for (long long i = (long long)blockIdx.x * EW_THREADS + threadIdx.x; i < n; i += stride) {
+    const uint32_t q = fd_div((uint32_t)i, fd);
+    const uint32_t r = (uint32_t)i - q * fd.d;
+    t[i] = f(a[i], vec[COLVEC ? r : q]);
+  }
+}
+
+template <bool COLVEC, class F>
+static int launch_bcast(const float* a, const float* vec, float* t, int h, int w, F f) {
+  const long long n = (long long)h * w;
+  if (n <= 0) return 0;
+  if (n >= (1ll << 32)) return ERROR_UNSUPPORTED;  // 32-bit element index inside the kernel
+  const FastDiv fd = make_fastdiv((uint32_t)h);
+  const int cus = dn_num_cus();
+  const int ht = head_of(t);
+  if (head_of(a) == ht) {
+    const int head = (int)(ht < n ? ht : n);
+    const long long n4 = (n - head) / 4;
+    long long blocks = (n4 + (long long)EW_THREADS * EW_UNROLL - 1) / ((long long)EW_THREADS * EW_UNROLL);
+    const long long cap = (long long)cus * 16;
+    if (blocks > cap) blocks = cap;
+    if (blocks < 1) blocks = 1;
+    hipLaunchKernelGGL((k_bcast<COLVEC, F>), dim3((unsigned)blocks), dim3(EW_THREADS), 0, 0, a, vec, t, n, head, n4,
+                       fd, f);
+  } else {
+    long long blocks = (n + EW_THREADS - 1) / EW_THREADS;
+    const long long cap = (long long)cus * 32;
+    if (blocks > cap) blocks = cap;
+    hipLaunchKernelGGL((k_bcast_scalar<COLVEC, F>), dim3((unsigned)blocks), dim3(EW_THREADS), 0, 0, a, vec, t, n, fd,
+                       f);
+  }
+  return dn_launch_status();
+}
+
+// Diagonal of a square w x w matrix: element i*(w+1).  vec may be null (scalar form).
+template <class F>
+__global__ void k_diag(const float* a, const float* vec, float* t, int w, F f) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < w) {
+    const size_t p = (size_t)i * w + i;
+    t[p] = f(a[p], vec ? vec[i] : 0.f);
+  }
+}
+
+template <class F>
+static int launch_diag(const float* a, const float* vec, float* t, int w, F f) {
+  if (w <= 0) return 0;
+  hipLaunchKernelGGL((k_diag<F>), dim3((w + 255) / 256), dim3(256), 0, 0, a, vec, t, w, f);
+  return dn_launch_status();
+}
+
+// ------------------------------------------------------------------ argument checks
+// Each family keeps the order of checks of the wrappers it replaces.
+
+static inline bool same_dims(const cudamat* a, const cudamat* b) {
+  return a->size[0] == b->size[0] && a->size[1] == b->size[1];
+}
+
+// unary math (cudamat.cu:1339-1546): device, then dims.
+static inline int check_unary(const cudamat* mat, const cudamat* target) {
+  if (!mat->on_device || !target->on_device) return ERROR_NOT_ON_DEVICE;
+  if (!same_dims(mat, target)) return ERROR_INCOMPATIBLE_DIMENSIONS;
+  return 0;
+}
+// sign and matrix-vs-scalar comparisons (cudamat.cu:923-966, 1060-1146, 1318-1338):
+// device, transposedness of mat vs target, dims.
+static inline int check_unary_trans(const cudamat* mat, const cudamat* target) {
+  if (!mat->on_device || !target->on_device) return ERROR_NOT_ON_DEVICE;
+  if (mat->is_trans != target->is_trans) return ERROR_TRANSPOSEDNESS;
+  if (!same_dims(mat, target)) return ERROR_INCOMPATIBLE_DIMENSIONS;
+  return 0;
+}
+// binary elementwise (cudamat.cu:878-1059, 1803-2030): device, transposedness
+// of the two inputs, dims.
+static inline int check_binary(const cudamat* m1, const cudamat* m2, const cudamat* target) {
+  if (!m1->on_device || !m2->on_device || !target->on_device) return ERROR_NOT_ON_DEVICE;
+  if (m1->is_trans != m2->is_trans) return ERROR_TRANSPOSEDNESS;
+  if (!same_dims(m1, m2) || !same_dims(m1, target)) return ERROR_INCOMPATIBLE_DIMENSIONS;
+  return 0;
+}
+// pow_matrix / cross-entropy family (cudamat.cu:1566-1650): device of mat and
+// target, dims of target, dims of the second input.
+static inline int check_binary_notrans(const cudamat* mat, const cudamat* p, const cudamat* target) {
+  if (!mat->on_device || !target->on_device || !p->on_device) return ERROR_NOT_ON_DEVICE;
+  if (!same_dims(mat, target)) return ERROR_INCOMPATIBLE_DIMENSIONS;
+  if (!same_dims(mat, p)) return ERROR_INCOMPATIBLE_DIMENSIONS;
+  return 0;
+}
+// column-vector broadcasts (cudamat.cu:592-639, 783-853): device, mat not
+// transposed, vec is h x 1 and target matches.
+static inline int check_colvec(const cudamat* mat, const cudamat* vec, const cudamat* target) {
+  if (!mat->on_device || !vec->on_device || !target->on_device) return ERROR_NOT_ON_DEVICE;
+  if (mat->is_trans) return ERROR_TRANSPOSED;
+  if (mat->size[0] != vec->size[0] || vec->size[1] != 1 || !same_dims(mat, target))
+    return ERROR_INCOMPATIBLE_DIMENSIONS;
+  return 0;
+}
+// row-vector broadcasts (cudamat.cu:735-781, 807-877): vec is 1 x w.
+static inline int check_rowvec(const cudamat* mat, const cudamat* vec, const cudamat* target) {
+  if (!mat->on_device || !vec->on_device || !target->on_device) return ERROR_NOT_ON_DEVICE;
+  if (mat->is_trans) return ERROR_TRANSPOSED;
+  if (mat->size[1] != vec->size[1] || vec->size[0] != 1 || !same_dims(mat, target))
+    return ERROR_INCOMPATIBLE_DIMENSIONS;
+  return 0;
+}
+
+#define DN_UNARY(NAME, CHECK, FUNCTOR)                                                        \
+  int NAME(cudamat* mat, cudamat* target) {                                                   \
+    if (int e = CHECK(mat, target)) return e;                                                 \
+    return launch_ew<1>(mat->data_device, nullptr, target->data_device, dn_len(mat), FUNCTOR); \
+  }
+#define DN_BINARY(NAME, CHECK, FUNCTOR)                                                                   \
+  int NAME(cudamat* mat1, cudamat* mat2, cudamat* target) {                                               \
+    if (int e = CHECK(mat1, mat2, target)) return e;                                                      \
+    return launch_ew<2>(mat1->data_device, mat2->data_device, target->data_device, dn_len(mat1), FUNCTOR); \
+  }
+#define DN_SCALAR(NAME, CHECK, FUNCTOR)                                                                 \
+  int NAME(cudamat* mat, float val, cudamat* target) {                                                  \
+    if (int e = CHECK(mat, target)) return e;                                                           \
+    return launch_ew<1>(mat->data_device, nullptr, target->data_device, dn_len(mat), FUNCTOR{val});      \
+  }
+#define DN_BINARY_PARAM(NAME, FUNCTOR)                                                                          \
+  int NAME(cudamat* mat, cudamat* p, cudamat* target, float s) {                                                \
+    if (int e = check_binary_notrans(mat, p, target)) return e;                                                 \
+    return launch_ew<2>(mat->data_device, p->data_device, target->data_device, dn_len(mat), FUNCTOR{s});         \
+  }
+#define DN_COLVEC(NAME, FUNCTOR)                                                                   \
+  int NAME(cudamat* mat, cudamat* vec, cudamat* target) {                                          \
+    if (int e = check_colvec(mat, vec, target)) return e;                                          \
+    return launch_bcast<true>(mat->data_device, vec->data_device, target->data_device, mat->size[0], \
+                              mat->size[1], FUNCTOR);                                              \
+  }
+#define DN_ROWVEC(NAME, FUNCTOR)                                                                    \
+  int NAME(cudamat* mat, cudamat* vec, cudamat* target) {                                           \
+    if (int e = check_rowvec(mat, vec, target)) return e;                                           \
+    return launch_bcast<false>(mat->data_device, vec->data_device, target->data_device, mat->size[0], \
+                               mat->size[1], FUNCTOR);                                              \
+  }
+
+extern "C" {
+
+// ---- unary
+DN_UNARY(sign, check_unary_trans, FSign{})
+DN_UNARY(apply_cos, check_unary, FCos{})
+DN_UNARY(apply_sin, check_unary, FSin{})
+DN_UNARY(apply_sigmoid, check_unary, FSigmoid{})
+DN_UNARY(apply_tanh, check_unary, FTanh{})
+DN_UNARY(apply_abs, check_unary, FAbs{})
+DN_UNARY(apply_log_1_plus_exp, check_unary, FLog1pExp{})
+DN_UNARY(apply_exp, check_unary, FExp{})
+DN_UNARY(apply_ceil, check_unary, FCeil{})
+DN_UNARY(apply_floor, check_unary, FFloor{})
+DN_UNARY(apply_sqrt, check_unary, FSqrt{})
+DN_UNARY(reciprocal, check_unary, FRecip{})
+
+int apply_log(cudamat* mat, cudamat* target, float tiny) {
+  if (int e = check_unary(mat, target)) return e;
+  return launch_ew<1>(mat->data_device, nullptr, target->data_device, dn_len(mat), FLog{tiny});
+}
+
+// ---- matrix (op) scalar
+DN_SCALAR(apply_pow, check_unary, FPow)
+DN_SCALAR(less_than_eq_scalar, check_unary_trans, FLeS)
+DN_SCALAR(less_than_scalar, check_unary_trans, FLtS)
+DN_SCALAR(greater_than_eq_scalar, check_unary_trans, FGeS)
+DN_SCALAR(greater_than_scalar, check_unary_trans, FGtS)
+DN_SCALAR(upper_bound_scalar, check_unary_trans, FUpperS)
+DN_SCALAR(lower_bound_scalar, check_unary_trans, FLowerS)
+DN_SCALAR(mult_by_scalar, check_unary, FMulS)
+DN_SCALAR(divide_by_scalar, check_unary, FDivS)
+DN_SCALAR(add_scalar, check_unary, FAddS)
+
+int assign_scalar(cudamat* mat, float alpha) {
+  if (!mat->on_device) return ERROR_NOT_ON_DEVICE;
+  return launch_ew<0>(nullptr, nullptr, mat->data_device, dn_len(mat), FAssignS{alpha});
+}
+
+// ---- binary
+DN_BINARY(less_than_eq, check_binary, FLe{})
+DN_BINARY(less_than, check_binary, FLt{})
+DN_BINARY(greater_than_eq, check_binary, FGe{})
+DN_BINARY(greater_than, check_binary, FGt{})
+DN_BINARY(upper_bound, check_binary, FUpper{})
+DN_BINARY(lower_bound, check_binary, FLower{})
+DN_BINARY(add_elementwise, check_binary, FAdd{})
+DN_BINARY(subtract_elementwise, check_binary, FSub{})
+DN_BINARY(divide_elementwise, check_binary, FDiv{})
+DN_BINARY(mult_elementwise, check_binary, FMul{})
+DN_BINARY(apply_sin_deriv, check_binary, FSinDeriv{})
+DN_BINARY(apply_cos_deriv, check_binary, FCosDeriv{})
+DN_BINARY(apply_logistic_deriv, check_binary, FLogisticDeriv{})
+DN_BINARY(apply_tanh_deriv, check_binary, FTanhDeriv{})
+DN_BINARY(apply_rectified_linear_deriv, check_binary, FReluDeriv{})
+DN_BINARY(apply_rectified_linear_smooth_deriv, check_binary, FReluSmoothDeriv{})
+DN_BINARY(apply_pow_matrix, check_binary_notrans, FPowMat{})
+DN_BINARY_PARAM(compute_cross_entropy, FCrossEntropy)
+DN_BINARY_PARAM(compute_cross_entropy_bernoulli, FCrossEntropyBernoulli)
+DN_BINARY_PARAM(correct_preds, FCorrectPreds)
+
+// mat1 += alpha * mat2 (cudamat.cu:1763-1781): device, transposedness, dims; no target.
+int add_mult(cudamat* mat1, cudamat* mat2, float alpha) {
+  if (!mat1->on_device || !mat2->on_device) return ERROR_NOT_ON_DEVICE;
+  if (mat1->is_trans != mat2->is_trans) return ERROR_TRANSPOSEDNESS;
+  if (!same_dims(mat1, mat2)) return ERROR_INCOMPATIBLE_DIMENSIONS;
+  return launch_ew<2>(mat1->data_device, mat2->data_device, mat1->data_device, dn_len(mat1), FAxpy{alpha});
+}
+
+int add_mult_sign(cudamat* mat1, cudamat* mat2, float mult) {
+  if (!mat1->on_device || !mat2->on_device) return ERROR_NOT_ON_DEVICE;
+  if (mat1->is_trans != mat2->is_trans) return ERROR_TRANSPOSEDNESS;
+  if (!same_dims(mat1, mat2)) return ERROR_INCOMPATIBLE_DIMENSIONS;
+  return launch_ew<2>(mat1->data_device, mat2->data_device, mat1->data_device, dn_len(mat1), FAddMultSign{mult});
+}
+
+// ---- broadcasts
+DN_COLVEC(add_col_vec, FAdd{})
+DN_COLVEC(mult_by_col_vec, FMul{})
+DN_COLVEC(div_by_col_vec, FDiv{})
+DN_ROWVEC(add_row_vec, FAdd{})
+DN_ROWVEC(mult_by_row_vec, FMul{})
+DN_ROWVEC(div_by_row_vec, FDiv{})
+
+int add_col_mult(cudamat* mat, cudamat* vec, cudamat* target, float mult) {
+  if (int e = check_colvec(mat, vec, target)) return e;
+  return launch_bcast<true>(mat->data_device, vec->data_device, target->data_device, mat->size[0], mat->size[1],
+                            FAxpy{mult});
+}
+
+int add_row_mult(cudamat* mat, cudamat* vec, cudamat* target, float mult) {
+  if (int e = check_rowvec(mat, vec, target)) return e;
+  return launch_bcast<false>(mat->data_device, vec->data_device, target->data_device, mat->size[0], mat->size[1],
+                             FAxpy{mult});
+}
+
+// ---- diagonal (cudamat.cu:641-733): only the w diagonal entries of target are written.
+static inline int check_diag(const cudamat* mat, const cudamat* vec, const cudamat* target) {
+  if (!mat->on_device || (vec && !vec->on_device) || !target->on_device) return ERROR_NOT_ON_DEVICE;
+  if (mat->is_trans) return ERROR_TRANSPOSED;
+  if ((vec && mat->size[0] != vec->size[1] * vec->size[0]) || !same_dims(mat, target))
+    return ERROR_INCOMPATIBLE_DIMENSIONS;
+  if (mat->size[0] < mat->size[1]) return ERROR_INCOMPATIBLE_DIMENSIONS;  // diagonal index i*w+i must stay inside
+  return 0;
+}
+
+int mult_diagonal_scalar(cudamat* mat, float val, cudamat* target) {
+  if (int e = check_diag(mat, nullptr, target)) return e;
+  return launch_diag(mat->data_device, nullptr, target->data_device, mat->size[1], FMulS{val});
+}
+int add_diagonal_scalar(cudamat* mat, float val, cudamat* target) {
+  if (int e = check_diag(mat, nullptr, target)) return e;
+  return launch_diag(mat->data_device, nullptr, target->data_device, mat->size[1], FAddS{val});
+}
+int mult_diagonal(cudamat* mat, cudamat* vec, cudamat* target) {
+  if (int e = check_diag(mat, vec, target)) return e;
+  return launch_diag(mat->data_device, vec->data_device, target->data_device, mat->size[1], FMul{});
+}
+int add_diagonal(cudamat* mat, cudamat* vec, cudamat* target) {
+  if (int e = check_diag(mat, vec, target)) return e;
+  return launch_diag(mat->data_device, vec->data_device, target->data_device, mat->size[1], FAdd{});
+}
+
+}  // extern "C"

@@ -1,0 +1,657 @@
+// Reductions: per-column / per-row max, argmax, sum of squares, norm clipping,
+// column softmax and its loss helpers, weighted sums (matrix-vector products),
+// flat dot product and Euclidean norm.
+// Replaces cudamat/cudamat.cu:1148-1315, 1733-1761, 2104-2118, 2192-2346 and
+// the kernels cudamat_kernels.cu:5-92, 819-1088.
+//
+// A column is h contiguous floats.  One wavefront (or one 256-lane workgroup
+// for tall, few columns) streams a column with 16-byte loads and finishes with
+// cross-lane shuffles; rows are reduced by tiles of 64 rows x 4 wavefronts with
+// the lanes running down the rows so every load is a 256-byte run.
+#include "common.h"
+#include <float.h>
+#include <math.h>
+
+// ------------------------------------------------------------------ scratch
+// Grow-only device workspace for two-stage reductions (partials + result).
+static void* g_scratch = nullptr;
+static size_t g_scratch_bytes = 0;
+
+void* dn_scratch(size_t bytes) {
+  if (bytes > g_scratch_bytes) {
+    if (g_scratch) {
+      hipDeviceSynchronize();
+      hipFree(g_scratch);
+    }
+    size_t want = bytes < (1u << 20) ? (1u << 20) : bytes;
+    if (hipMalloc(&g_scratch, want) != hipSuccess) {
+      g_scratch = nullptr;
+      g_scratch_bytes = 0;
+      hipGetLastError();
+      return nullptr;
+    }
+    g_scratch_bytes = want;
+  }
+  return g_scratch;
+}
+
+// ------------------------------------------------------------------ column walkers
+
+// Visit every element of one column with TPC cooperating lanes: fn(row, value).
+template <int TPC, class Fn>
+__device__ __forceinline__ void for_each_in_col(const float* c, int h, int lane, Fn fn) {
+  int head = (int)(((16u - (unsigned)(reinterpret_cast<uintptr_t>(c) & 15u)) & 15u) >> 2);
+  if (head > h) head = h;
+  if (lane < head) fn(lane, c[lane]);
+  const float4* c4 = reinterpret_cast<const float4*>(c + head);
+  const int n4 = (h - head) >> 2;
+  for (int j = lane; j < n4; j += TPC) {
+    const float4 v = c4[j];
+    const int b = head + 4 * j;
+    fn(b, v.x);
+    fn(b + 1, v.y);
+    fn(b + 2, v.z);
+    fn(b + 3, v.w);
+  }
+  const int t0 = head + 4 * n4;
+  if (lane < h - t0) fn(t0 + lane, c[t0 + lane]);
+}
+
+// Combine one float per lane across the TPC lanes that share a column.
+// TPC == 64: shuffles only.  TPC == 256: shuffles, then 4 partials through LDS.
+template <int TPC, bool IS_MAX>
+__device__ __forceinline__ float col_combine(float v, float* lds4) {
+  v = IS_MAX ? wave_max(v) : wave_sum(v);
+  if (TPC == 64) return v;
+  const int wv = threadIdx.x >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) lds4[wv] = v;
+  __syncthreads();
+  const float a = lds4[0], b = lds4[1], c = lds4[2], d = lds4[3];
+  return IS_MAX ? fmaxf(fmaxf(a, b), fmaxf(c, d)) : ((a + b) + (c + d));
+}
+
+// Arg-max candidate.  The reference scans a column with 32 lanes, lane t taking
+// rows t, t+32, ..., keeps the first strictly larger value per lane and then
+// the first strictly larger lane (cudamat_kernels.cu:1020-1050); among equal
+// maxima that selects the smallest (row % 32, row).  key reproduces that order;
+// the start value (-FLT_MAX, row 0) wins every tie, as it does there.
+struct ArgCand {
+  float v;
+  long long key;  // -1 for the start value, else ((row % 32) << 32) | row
+  int row;
+};
+__device__ __forceinline__ bool arg_better(float v1, long long k1, float v2, long long k2) {
+  return v1 > v2 || (v1 == v2 && k1 < k2);
+}
+__device__ __forceinline__ void arg_visit(ArgCand& c, int row, float v) {
+  const long long k = ((long long)(row & 31) << 32) | (long long)row;
+  if (arg_better(v, k, c.v, c.key)) { c.v = v; c.key = k; c.row = row; }
+}
+template <int TPC>
+__device__ __forceinline__ ArgCand arg_combine(ArgCand c, ArgCand* lds4) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float v = __shfl_xor(c.v, o, WAVE);
+    const long long k = __shfl_xor(c.key, o, WAVE);
+    const int r = __shfl_xor(c.row, o, WAVE);
+    if (arg_better(v, k, c.v, c.key)) { c.v = v; c.key = k; c.row = r; }
+  }
+  if (TPC == 64) return c;
+  const int wv = threadIdx.x >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) lds4[wv] = c;
+  __syncthreads();
+  ArgCand best = lds4[0];
+#pragma unroll
+  for (int i = 1; i < 4; ++i)
+    if (arg_better(lds4[i].v, lds4[i].key, best.v, best.key)) best = lds4[i];
+  return best;
+}
+
+#define COL_SETUP(TPC)                                                 \
+  const int cols_per_block = 256 / TPC;                                \
+  const int col = blockIdx.x * cols_per_block + (int)threadIdx.x / TPC; \
+  const int lane = (int)threadIdx.x % TPC;                             \
+  const bool active = col < w;
+
+// ------------------------------------------------------------------ column kernels (axis 0)
+
+template <int TPC>
+__global__ void __launch_bounds__(256) k_col_max(const float* mat, float* target, int w, int h) {
+  __shared__ float lds4[4];
+  COL_SETUP(TPC)
+  float m = -FLT_MAX;
+  if (active) for_each_in_col<TPC>(mat + (size_t)col * h, h, lane, [&](int, float v) { if (v > m) m = v; });
+  m = col_combine<TPC, true>(m, lds4);
+  if (active && lane == 0) target[col] = m;
+}
+
+// mode 0: target[col] = argmax; 1: one-hot column into target; 2: target(argmax, col) += 1;
+// 3: target[col] = (argmax == (int)labels[col]).
+template <int TPC>
+__global__ void __launch_bounds__(256)
+k_col_argmax(const float* mat, float* target, const float* labels, int w, int h, int mode) {
+  __shared__ ArgCand lds4[4];
+  COL_SETUP(TPC)
+  ArgCand c;
+  c.v = -FLT_MAX; c.key = -1; c.row = 0;
+  if (active) for_each_in_col<TPC>(mat + (size_t)col * h, h, lane, [&](int r, float v) { arg_visit(c, r, v); });
+  c = arg_combine<TPC>(c, lds4);
+  if (!active) return;
+  if (mode == 0) {
+    if (lane == 0) target[col] = (float)c.row;
+  } else if (mode == 1) {
+    float* t = target + (size_t)col * h;
+    for (int i = lane; i < h; i += TPC) t[i] = (i == c.row) ? 1.f : 0.f;
+  } else if (mode == 2) {
+    if (lane == 0) target[(size_t)col * h + c.row] += 1.f;
+  } else {
+    if (lane == 0) target[col] = (c.row == (int)labels[col]) ? 1.f : 0.f;
+  }
+}
+
+template <int TPC>
+__global__ void __launch_bounds__(256) k_col_sqsum(const float* mat, float* target, int w, int h, float mult, float p) {
+  __shared__ float lds4[4];
+  COL_SETUP(TPC)
+  float s = 0.f;
+  if (active) for_each_in_col<TPC>(mat + (size_t)col * h, h, lane, [&](int, float v) { s += v * v; });
+  s = col_combine<TPC, false>(s, lds4);
+  // p == 0 overwrites: the previous contents (possibly uninitialised) are not read.
+  if (active && lane == 0) target[col] = (p == 0.f ? 0.f : p * target[col]) + mult * s;
+}
+
+template <int TPC>
+__global__ void __launch_bounds__(256) k_col_normlimit(const float* mat, float* target, int w, int h, float norm) {
+  __shared__ float lds4[4];
+  COL_SETUP(TPC)
+  float s = 0.f;
+  const float* c = mat + (size_t)col * h;
+  if (active) for_each_in_col<TPC>(c, h, lane, [&](int, float v) { s += v * v; });
+  s = col_combine<TPC, false>(s, lds4);
+  if (!active) return;
+  float scale = sqrtf(s);
+  scale = (scale < norm) ? 1.f : (norm / scale);
+  float* t = target + (size_t)col * h;
+  for_each_in_col<TPC>(c, h, lane, [&](int r, float v) { t[r] = v * scale; });
+}
+
+// Column softmax: max, sum of exp(x - max), divide (cudamat_kernels.cu:868-934).
+// The column is re-read from cache for the second and third pass.
+template <int TPC>
+__global__ void __launch_bounds__(256) k_col_softmax(const float* mat, float* target, int w, int h) {
+  __shared__ float lds4[4];
+  COL_SETUP(TPC)
+  const float* c = mat + (size_t)col * h;
+  float* t = target + (size_t)col * h;
+  float m = -FLT_MAX;
+  if (active) for_each_in_col<TPC>(c, h, lane, [&](int, float v) { if (v > m) m = v; });
+  m = col_combine<TPC, true>(m, lds4);
+  float s = 0.f;
+  if (active) for_each_in_col<TPC>(c, h, lane, [&](int, float v) { s += expf(v - m); });
+  s = col_combine<TPC, false>(s, lds4);
+  if (active) for_each_in_col<TPC>(c, h, lane, [&](int r, float v) { t[r] = expf(v - m) / s; });
+}
+
+// Columns of at most 64 * 4 * NV floats stay in registers between the passes:
+// one read and one write of HBM per element.  Requires h % 4 == 0 and 16-byte
+// aligned columns.
+template <int NV>
+__global__ void __launch_bounds__(256) k_col_softmax_reg(const float* mat, float* target, int w, int h) {
+  const int col = blockIdx.x * 4 + (int)(threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (col >= w) return;
+  const float4* c4 = reinterpret_cast<const float4*>(mat + (size_t)col * h);
+  float4* t4 = reinterpret_cast<float4*>(target + (size_t)col * h);
+  const int n4 = h >> 2;
+  float4 v[NV];
+  float m = -FLT_MAX;
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    const int j = lane + k * 64;
+    if (j < n4) {
+      v[k] = c4[j];
+      m = fmaxf(m, fmaxf(fmaxf(v[k].x, v[k].y), fmaxf(v[k].z, v[k].w)));
+    }
+  }
+  m = wave_max(m);
+  float s = 0.f;
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    const int j = lane + k * 64;
+    if (j < n4) {
+      v[k].x = expf(v[k].x - m); v[k].y = expf(v[k].y - m);
+      v[k].z = expf(v[k].z - m); v[k].w = expf(v[k].w - m);
+      s += (v[k].x + v[k].y) + (v[k].z + v[k].w);
+    }
+  }
+  s = wave_sum(s);
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    const int j = lane + k * 64;
+    if (j < n4) t4[j] = make_float4(v[k].x / s, v[k].y / s, v[k].z / s, v[k].w / s);
+  }
+}
+
+__global__ void k_softmax_grad(const float* mat, const float* labels, float* target, int w, int h, FastDiv fd) {
+  const size_t n = (size_t)w * h;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+    const uint32_t q = fd_div((uint32_t)i, fd);
+    const uint32_t r = (uint32_t)i - q * (uint32_t)h;
+    target[i] = mat[i] - (((int)labels[q] == (int)r) ? 1.f : 0.f);
+  }
+}
+
+__global__ void k_softmax_ce(const float* mat, const float* labels, float* target, int w, int h, float tiny) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < w) target[i] = -logf(mat[(size_t)h * i + (int)labels[i]] + tiny);
+}
+
+// ------------------------------------------------------------------ row kernels (axis 1)
+// 64 rows per workgroup, lanes down the rows, the 4 wavefronts take columns
+// j = wave, wave + 4, ... and meet in LDS.  First-occurrence ties and a start
+// value taken "before column 0", as in eigenmat/eigenmat.cc:617-731.
+
+// op 0: max, 1: argmax, 2: one-hot row into target, 3: sqsum (target = p*target + mult*sum)
+__global__ void __launch_bounds__(256)
+k_row_reduce(const float* mat, float* target, int w, int h, int op, float mult, float p) {
+  __shared__ float sv[4][64];
+  __shared__ int si[4][64];
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int row = blockIdx.x * 64 + lane;
+  float acc = (op == 3) ? 0.f : -INFINITY;
+  int idx = 0;
+  if (row < h) {
+    for (int j = wv; j < w; j += 4) {
+      const float v = mat[(size_t)j * h + row];
+      if (op == 3) acc += v * v;
+      else if (v > acc) { acc = v; idx = j; }
+    }
+  }
+  sv[wv][lane] = acc;
+  si[wv][lane] = idx;
+  __syncthreads();
+  if (row >= h) return;
+  float best = sv[0][lane];
+  int bidx = si[0][lane];
+  if (op == 3) {
+    best = (sv[0][lane] + sv[1][lane]) + (sv[2][lane] + sv[3][lane]);
+  } else {
+#pragma unroll
+    for (int k = 1; k < 4; ++k) {
+      const float v = sv[k][lane];
+      const int i2 = si[k][lane];
+      if (v > best || (v == best && i2 < bidx)) { best = v; bidx = i2; }
+    }
+  }
+  if (op == 0) { if (wv == 0) target[row] = best; }
+  else if (op == 1) { if (wv == 0) target[row] = (float)bidx; }
+  else if (op == 3) { if (wv == 0) target[row] = (p == 0.f ? 0.f : p * target[row]) + mult * best; }
+  else { for (int j = wv; j < w; j += 4) target[(size_t)j * h + row] = (j == bidx) ? 1.f : 0.f; }
+}
+
+__global__ void __launch_bounds__(256) k_row_normlimit(const float* mat, float* target, int w, int h, float norm) {
+  __shared__ float sv[4][64];
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int row = blockIdx.x * 64 + lane;
+  float acc = 0.f;
+  if (row < h)
+    for (int j = wv; j < w; j += 4) { const float v = mat[(size_t)j * h + row]; acc += v * v; }
+  sv[wv][lane] = acc;
+  __syncthreads();
+  if (row >= h) return;
+  float scale = sqrtf((sv[0][lane] + sv[1][lane]) + (sv[2][lane] + sv[3][lane]));
+  scale = (scale < norm) ? 1.f : (norm / scale);
+  for (int j = wv; j < w; j += 4) target[(size_t)j * h + row] = mat[(size_t)j * h + row] * scale;
+}
+
+// ------------------------------------------------------------------ weighted sums (matrix-vector)
+
+// y[j] = beta*y[j] + alpha * sum_i M[i + j*ld] * x[i]   (one output per contiguous column)
+template <int TPC>
+__global__ void __launch_bounds__(256)
+k_gemv_cols(const float* M, int ld, int h, int w, const float* x, float* y, float alpha, float beta) {
+  __shared__ float lds4[4];
+  COL_SETUP(TPC)
+  float s = 0.f;
+  if (active) for_each_in_col<TPC>(M + (size_t)col * ld, h, lane, [&](int r, float v) { s += v * x[r]; });
+  s = col_combine<TPC, false>(s, lds4);
+  if (active && lane == 0) y[col] = (beta == 0.f ? 0.f : beta * y[col]) + alpha * s;
+}
+
+// Stage 1 of y[i] = beta*y[i] + alpha * sum_j M[i + j*ld] * x[j]: workgroup (bx, by)
+// reduces columns [by*cps, (by+1)*cps) for rows 256*bx .. 256*bx+255 (4 rows per
+// lane as one 16-byte load when vec, else 64 rows per workgroup).  With one
+// split the result goes straight to y.
+template <bool VEC>
+__global__ void __launch_bounds__(256)
+k_gemv_rows(const float* M, int ld, int h, int w, int cps, const float* x, float* y, float* partial, float alpha,
+            float beta) {
+  constexpr int RPL = VEC ? 4 : 1;
+  __shared__ float sv[4][64 * RPL];
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int row0 = (blockIdx.x * 64 + lane) * RPL;
+  const int j0 = blockIdx.y * cps;
+  const int j1 = (j0 + cps < w) ? j0 + cps : w;
+  float acc[RPL];
+#pragma unroll
+  for (int k = 0; k < RPL; ++k) acc[k] = 0.f;
+  if (row0 < h) {
+    if constexpr (VEC) {
+      for (int j = j0 + wv; j < j1; j += 4) {
+        const float4 v = *reinterpret_cast<const float4*>(M + (size_t)j * ld + row0);
+        const float xj = x[j];
+        acc[0] += v.x * xj; acc[1] += v.y * xj; acc[2] += v.z * xj; acc[3] += v.w * xj;
+      }
+    } else {
+      for (int j = j0 + wv; j < j1; j += 4) acc[0] += M[(size_t)j * ld + row0] * x[j];
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < RPL; ++k) sv[wv][lane * RPL + k] = acc[k];
+  __syncthreads();
+  // 256 lanes finish 64*RPL rows.
+  for (int r = threadIdx.x; r < 64 * RPL; r += 256) {
+    const int row = blockIdx.x * 64 * RPL + r;
+    if (row < h) {
+      const float s = (sv[0][r] + sv[1][r]) + (sv[2][r] + sv[3][r]);
+      if (partial) partial[(size_t)blockIdx.y * h + row] = s;
+      else y[row] = (beta == 0.f ? 0.f : beta * y[row]) + alpha * s;
+    }
+  }
+}
+
+__global__ void k_gemv_rows_finish(const float* partial, int splits, int h, float* y, float alpha, float beta) {
+  const int row = blockIdx.x * blockDim.x + threadIdx.x;
+  if (row >= h) return;
+  float s = 0.f;
+  for (int k = 0; k < splits; ++k) s += partial[(size_t)k * h + row];
+  y[row] = (beta == 0.f ? 0.f : beta * y[row]) + alpha * s;
+}
+
+// Host entry points used by dot() for vector-shaped products.
+int dn_gemv_cols(const float* M, int ld, int h, int w, const float* x, float* y, float alpha, float beta) {
+  if (w <= 0) return 0;
+  const int cus = dn_num_cus();
+  if (w < cus * 2 && h >= 4096) {
+    hipLaunchKernelGGL((k_gemv_cols<256>), dim3(w), dim3(256), 0, 0, M, ld, h, w, x, y, alpha, beta);
+  } else {
+    hipLaunchKernelGGL((k_gemv_cols<64>), dim3((w + 3) / 4), dim3(256), 0, 0, M, ld, h, w, x, y, alpha, beta);
+  }
+  return dn_launch_status();
+}
+
+int dn_gemv_rows(const float* M, int ld, int h, int w, const float* x, float* y, float alpha, float beta) {
+  if (h <= 0) return 0;
+  const bool vec = dn_aligned16(M) && (ld % 4 == 0) && (h % 4 == 0) && h >= 1024;
+  const int rows_per_block = vec ? 256 : 64;
+  const int bx = (h + rows_per_block - 1) / rows_per_block;
+  int splits = (4 * dn_num_cus()) / bx;
+  if (splits > (w + 31) / 32) splits = (w + 31) / 32;
+  if (splits < 1) splits = 1;
+  int cps = (w + splits - 1) / splits;
+  if (cps < 1) cps = 1;
+  splits = w > 0 ? (w + cps - 1) / cps : 1;
+  float* partial = nullptr;
+  if (splits > 1) {
+    partial = (float*)dn_scratch((size_t)splits * h * sizeof(float));
+    if (!partial) return CUDA_ERROR;
+  }
+  dim3 grid(bx, splits);
+  if (vec)
+    hipLaunchKernelGGL((k_gemv_rows<true>), grid, dim3(256), 0, 0, M, ld, h, w, cps, x, y, partial, alpha, beta);
+  else
+    hipLaunchKernelGGL((k_gemv_rows<false>), grid, dim3(256), 0, 0, M, ld, h, w, cps, x, y, partial, alpha, beta);
+  if (splits > 1)
+    hipLaunchKernelGGL(k_gemv_rows_finish, dim3((h + 255) / 256), dim3(256), 0, 0, partial, splits, h, y, alpha, beta);
+  return dn_launch_status();
+}
+
+// ------------------------------------------------------------------ flat dot / norm
+
+// partial[block] = sum over a grid-stride slice of a[i]*b[i], accumulated in
+// fp32 per lane and in fp64 across lanes and workgroups.
+__global__ void __launch_bounds__(256) k_dot_partial(const float* a, const float* b, long long n, double* partial) {
+  __shared__ double lds[4];
+  const long long stride = (long long)gridDim.x * 256;
+  float s0 = 0.f, s1 = 0.f;
+  long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  for (; i + stride < n; i += 2 * stride) {
+    s0 += a[i] * b[i];
+    s1 += a[i + stride] * b[i + stride];
+  }
+  if (i < n) s0 += a[i] * b[i];
+  double s = wave_sum_d((double)s0 + (double)s1);
+  if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = s;
+  __syncthreads();
+  if (threadIdx.x == 0) partial[blockIdx.x] = (lds[0] + lds[1]) + (lds[2] + lds[3]);
+}
+
+__global__ void __launch_bounds__(256) k_dot_finish(const double* partial, int nblocks, float* out, int take_sqrt) {
+  __shared__ double lds[4];
+  double s = 0.0;
+  for (int i = threadIdx.x; i < nblocks; i += 256) s += partial[i];
+  s = wave_sum_d(s);
+  if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = s;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const double t = (lds[0] + lds[1]) + (lds[2] + lds[3]);
+    out[0] = (float)(take_sqrt ? sqrt(t) : t);
+  }
+}
+
+static int flat_dot(const float* a, const float* b, long long n, int take_sqrt, float* result) {
+  *result = 0.f;
+  if (n <= 0) return 0;
+  long long nb = (n + 2047) / 2048;
+  const long long cap = (long long)dn_num_cus() * 8;
+  if (nb > cap) nb = cap;
+  char* ws = (char*)dn_scratch((size_t)nb * sizeof(double) + 16);
+  if (!ws) return CUDA_ERROR;
+  double* partial = (double*)ws;
+  float* out = (float*)(ws + (size_t)nb * sizeof(double));
+  hipLaunchKernelGGL(k_dot_partial, dim3((unsigned)nb), dim3(256), 0, 0, a, b, n, partial);
+  hipLaunchKernelGGL(k_dot_finish, dim3(1), dim3(256), 0, 0, partial, (int)nb, out, take_sqrt);
+  if (hipMemcpy(result, out, sizeof(float), hipMemcpyDeviceToHost) != hipSuccess) return CUDA_ERROR;
+  return 0;
+}
+
+// ------------------------------------------------------------------ C ABI
+
+template <class K64, class K256, class... Args>
+static int launch_cols(K64 k64, K256 k256, int w, int h, Args... args) {
+  if (w <= 0) return 0;
+  if (w < dn_num_cus() * 2 && h >= 4096)
+    hipLaunchKernelGGL(k256, dim3(w), dim3(256), 0, 0, args...);
+  else
+    hipLaunchKernelGGL(k64, dim3((w + 3) / 4), dim3(256), 0, 0, args...);
+  return dn_launch_status();
+}
+
+static inline int check_axis_common(const cudamat* mat, const cudamat* target) {
+  if (!mat->on_device || !target->on_device) return ERROR_NOT_ON_DEVICE;
+  if (mat->is_trans) return ERROR_TRANSPOSED;
+  return 0;
+}
+
+extern "C" {
+
+int max_by_axis(cudamat* mat, cudamat* target, int axis) {
+  const int h = mat->size[0], w = mat->size[1];
+  if (int e = check_axis_common(mat, target)) return e;
+  if (axis == 0) {
+    if (target->size[0] != 1 || target->size[1] != w) return ERROR_INCOMPATIBLE_DIMENSIONS;
+    return launch_cols(k_col_max<64>, k_col_max<256>, w, h, (const float*)mat->data_device, target->data_device, w, h);
+  } else if (axis == 1) {
+    if (target->size[0] != h || target->size[1] != 1) return ERROR_INCOMPATIBLE_DIMENSIONS;
+    if (h <= 0) return 0;
+    hipLaunchKernelGGL(k_row_reduce, dim3((h + 63) / 64), dim3(256), 0, 0, (const float*)mat->data_device,
+                       target->data_device, w, h, 0, 0.f, 0.f);
+    return dn_launch_status();
+  }
+  return ERROR_UNSUPPORTED;
+}
+
+int argmax_by_axis(cudamat* mat, cudamat* target, int axis) {
+  const int h = mat->size[0], w = mat->size[1];
+  if (int e = check_axis_common(mat, target)) return e;
+  if (axis == 0) {
+    if (target->size[0] != 1 || target->size[1] != w) return ERROR_INCOMPATIBLE_DIMENSIONS;
+    return launch_cols(k_col_argmax<64>, k_col_argmax<256>, w, h, (const float*)mat->data_device,
+                       target->data_device, (const float*)nullptr, w, h, 0);
+  } else if (axis == 1) {
+    if (target->size[0] != h || target->size[1] != 1) return ERROR_INCOMPATIBLE_DIMENSIONS;
+    if (h <= 0) return 0;
+    hipLaunchKernelGGL(k_row_reduce, dim3((h + 63) / 64), dim3(256), 0, 0, (const float*)mat->data_device,
+                       target->data_device, w, h, 1, 0.f, 0.f);
+    return dn_launch_status();
+  }
+  return ERROR_UNSUPPORTED;
+}
+
+// One-hot of the arg-max of every column (axis 0) or row (axis 1).  The reference
+// kernel clears rows of column 0 instead of the column it is working on
+// (cudamat_kernels.cu:980); every column is cleared here.
+int choose_max_by_axis(cudamat* mat, cudamat* target, int axis) {
+  const int h = mat->size[0], w = mat->size[1];
+  if (int e = check_axis_common(mat, target)) return e;
+  if (target->size[0] != h || target->size[1] != w) return ERROR_INCOMPATIBLE_DIMENSIONS;
+  if (axis == 0) {
+    return launch_cols(k_col_argmax<64>, k_col_argmax<256>, w, h, (const float*)mat->data_device,
+                       target->data_device, (const float*)nullptr, w, h, 1);
+  } else if (axis == 1) {
+    if (h <= 0) return 0;
+    hipLaunchKernelGGL(k_row_reduce, dim3((h + 63) / 64), dim3(256), 0, 0, (const float*)mat->data_device,
+                       target->data_device, w, h, 2, 0.f, 0.f);
+    return dn_launch_status();
+  }
+  return ERROR_UNSUPPORTED;
+}
+
+int choose_max_and_accumulate(cudamat* mat, cudamat* acc) {
+  const int h = mat->size[0], w = mat->size[1];
+  if (int e = check_axis_common(mat, acc)) return e;
+  if (acc->size[0] != h || acc->size[1] != w) return ERROR_INCOMPATIBLE_DIMENSIONS;
+  return launch_cols(k_col_argmax<64>, k_col_argmax<256>, w, h, (const float*)mat->data_device, acc->data_device,
+                     (const float*)nullptr, w, h, 2);
+}
+
+int sqsum_by_axis(cudamat* mat, cudamat* target, int axis, float mult, float p) {
+  const int h = mat->size[0], w = mat->size[1];
+  if (int e = check_axis_common(mat, target)) return e;
+  if (axis == 0) {
+    if (target->size[0] != 1 || target->size[1] != w) return ERROR_INCOMPATIBLE_DIMENSIONS;
+    return launch_cols(k_col_sqsum<64>, k_col_sqsum<256>, w, h, (const float*)mat->data_device, target->data_device,
+                       w, h, mult, p);
+  } else if (axis == 1) {
+    if (target->size[0] != h || target->size[1] != 1) return ERROR_INCOMPATIBLE_DIMENSIONS;
+    if (h <= 0) return 0;
+    hipLaunchKernelGGL(k_row_reduce, dim3((h + 63) / 64), dim3(256), 0, 0, (const float*)mat->data_device,
+                       target->data_device, w, h, 3, mult, p);
+    return dn_launch_status();
+  }
+  return ERROR_UNSUPPORTED;
+}
+
+int normlimit_by_axis(cudamat* mat, cudamat* target, int axis, float norm) {
+  const int h = mat->size[0], w = mat->size[1];
+  if (int e = check_axis_common(mat, target)) return e;
+  if (target->size[0] != h || target->size[1] != w) return ERROR_INCOMPATIBLE_DIMENSIONS;
+  if (axis == 0) {
+    return launch_cols(k_col_normlimit<64>, k_col_normlimit<256>, w, h, (const float*)mat->data_device,
+                       target->data_device, w, h, norm);
+  } else if (axis == 1) {
+    if (h <= 0) return 0;
+    hipLaunchKernelGGL(k_row_normlimit, dim3((h + 63) / 64), dim3(256), 0, 0, (const float*)mat->data_device,
+                       target->data_device, w, h, norm);
+    return dn_launch_status();
+  }
+  return ERROR_UNSUPPORTED;
+}
+
+static int softmax_impl(const float* in, float* out, int w, int h) {
+  if (w <= 0 || h <= 0) return 0;
+  const bool reg_ok = (h % 4 == 0) && dn_aligned16(in) && dn_aligned16(out) && h <= 64 * 4 * 16;
+  if (reg_ok) {
+    const int n4 = h / 4;
+    dim3 grid((w + 3) / 4), block(256);
+    if (n4 <= 64) hipLaunchKernelGGL((k_col_softmax_reg<1>), grid, block, 0, 0, in, out, w, h);
+    else if (n4 <= 128) hipLaunchKernelGGL((k_col_softmax_reg<2>), grid, block, 0, 0, in, out, w, h);
+    else if (n4 <= 256) hipLaunchKernelGGL((k_col_softmax_reg<4>), grid, block, 0, 0, in, out, w, h);
+    else if (n4 <= 512) hipLaunchKernelGGL((k_col_softmax_reg<8>), grid, block, 0, 0, in, out, w, h);
+    else hipLaunchKernelGGL((k_col_softmax_reg<16>), grid, block, 0, 0, in, out, w, h);
+    return dn_launch_status();
+  }
+  return launch_cols(k_col_softmax<64>, k_col_softmax<256>, w, h, in, out, w, h);
+}
+
+int softmax(cudamat* mat, cudamat* target) {
+  const int h = mat->size[0], w = mat->size[1];
+  if (int e = check_axis_common(mat, target)) return e;
+  if (target->size[0] != h || target->size[1] != w) return ERROR_INCOMPATIBLE_DIMENSIONS;
+  return softmax_impl(mat->data_device, target->data_device, w, h);
+}
+
+int softmax_overwrite(cudamat* mat) {
+  if (!mat->on_device) return ERROR_NOT_ON_DEVICE;
+  if (mat->is_trans) return ERROR_TRANSPOSED;
+  return softmax_impl(mat->data_device, mat->data_device, mat->size[1], mat->size[0]);
+}
+
+int apply_softmax_grad(cudamat* mat, cudamat* labels, cudamat* target) {
+  const int h = mat->size[0], w = mat->size[1];
+  if (int e = check_axis_common(mat, target)) return e;
+  if (target->size[0] != h || target->size[1] != w) return ERROR_INCOMPATIBLE_DIMENSIONS;
+  if (labels->size[0] != 1 || labels->size[1] != w) return ERROR_INCOMPATIBLE_DIMENSIONS;
+  const long long n = (long long)h * w;
+  if (n <= 0) return 0;
+  if (n >= (1ll << 32)) return ERROR_UNSUPPORTED;
+  long long blocks = (n + 255) / 256;
+  if (blocks > dn_num_cus() * 32ll) blocks = dn_num_cus() * 32ll;
+  hipLaunchKernelGGL(k_softmax_grad, dim3((unsigned)blocks), dim3(256), 0, 0, (const float*)mat->data_device,
+                     (const float*)labels->data_device, target->data_device, w, h, make_fastdiv((uint32_t)h));
+  return dn_launch_status();
+}
+
+int get_softmax_correct(cudamat* mat, cudamat* labels, cudamat* target) {
+  const int h = mat->size[0], w = mat->size[1];
+  if (int e = check_axis_common(mat, target)) return e;
+  if (target->size[0] != 1 || target->size[1] != w) return ERROR_INCOMPATIBLE_DIMENSIONS;
+  if (labels->size[0] != 1 || labels->size[1] != w) return ERROR_INCOMPATIBLE_DIMENSIONS;
+  return launch_cols(k_col_argmax<64>, k_col_argmax<256>, w, h, (const float*)mat->data_device, target->data_device,
+                     (const float*)labels->data_device, w, h, 3);
+}
+
+int get_softmax_cross_entropy(cudamat* mat, cudamat* labels, cudamat* target, float tiny) {
+  const int h = mat->size[0], w = mat->size[1];
+  if (int e = check_axis_common(mat, target)) return e;
+  if (target->size[0] != 1 || target->size[1] != w) return ERROR_INCOMPATIBLE_DIMENSIONS;
+  if (labels->size[0] != 1 || labels->size[1] != w) return ERROR_INCOMPATIBLE_DIMENSIONS;
+  if (w <= 0) return 0;
+  hipLaunchKernelGGL(k_softmax_ce, dim3((w + 255) / 256), dim3(256), 0, 0, (const float*)mat->data_device,
+                     (const float*)labels->data_device, target->data_device, w, h, tiny);
+  return dn_launch_status();
+}
+
+float vdot(cudamat* mat1, cudamat* mat2, int* err_code) {
+  const long long len = dn_len(mat1);
+  if (!mat1->on_device || !mat2->on_device) { *err_code = ERROR_NOT_ON_DEVICE; return 0.f; }
+  if (mat1->is_trans != mat2->is_trans) { *err_code = ERROR_TRANSPOSEDNESS; return 0.f; }
+  if (dn_len(mat2) != len) { *err_code = ERROR_INCOMPATIBLE_DIMENSIONS; return 0.f; }
+  float res = 0.f;
+  const int e = flat_dot(mat1->data_device, mat2->data_device, len, 0, &res);
+  *err_code = e;
+  return e ? -1.f : res;
+}
+
+float euclid_norm(cudamat* mat, int* err_code) {
+  if (!mat->on_device) { *err_code = ERROR_NOT_ON_DEVICE; return 0.f; }
+  float res = 0.f;
+  const int e = flat_dot(mat->data_device, mat->data_device, dn_len(mat), 1, &res);
+  *err_code = e;
+  return e ? -1.f : res;
+}
+
+}  // extern "C"

@@ -1,0 +1,200 @@
+/*
+ * C ABI of the MI355X matrix backend (libcudamat.so).
+ *
+ * Every entry point keeps the name, argument order, argument meaning and error
+ * code of the function it replaces in the reference's cudamat/cudamat.cu (cited
+ * per group as file:line), so the reference's cudamat.py binds it unchanged
+ * through ctypes.  All matrices are fp32, column-major, leading dimension
+ * size[0], no padding.  Work is queued on the NULL HIP stream; only the calls
+ * that hand a value back to the host (copy_to_host, vdot, euclid_norm,
+ * cuda_sync_threads) wait for the device.
+ */
+#ifndef CUDAMAT_AMD_H_
+#define CUDAMAT_AMD_H_
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Error codes: cudamat/cudamat.cuh:1-9. */
+#define ERROR_INCOMPATIBLE_DIMENSIONS -1
+#define CUBLAS_ERROR -2
+#define CUDA_ERROR -3
+#define VIEW_ERROR -4
+#define ERROR_TRANSPOSED -5
+#define ERROR_GENERIC -6
+#define ERROR_TRANSPOSEDNESS -7
+#define ERROR_NOT_ON_DEVICE -8
+#define ERROR_UNSUPPORTED -9
+
+/* Matrix handle: cudamat/cudamat.cuh:21-29 (ctypes mirror cudamat.py:126-133). */
+typedef struct cudamat {
+  float* data_host;
+  float* data_device;
+  int on_device;
+  int on_host;
+  int size[2];
+  int is_trans; /* 0 or 1 */
+  int owns_data;
+} cudamat;
+
+/* RNG state: cudamat/cudamat.cuh:31-34.  12288 multipliers and 12288 64-bit words. */
+typedef struct rnd_struct {
+  unsigned int* dev_mults;
+  unsigned long long* dev_words;
+} rnd_struct;
+
+#define NUM_RND_STREAMS 12288 /* cudamat_kernels.cuh:4-6 */
+#define NUM_RND_BURNIN 100    /* cudamat_kernels.cuh:18 */
+
+/* ---- device / library lifetime: cudamat.cu:25-53, 103-105 ---- */
+const char* get_last_cuda_error(void);
+int cublas_init(void);
+int cublas_shutdown(void);
+int cuda_set_device(int deviceId);
+void cuda_sync_threads(void);
+
+/* ---- handle fields and views: cudamat.cu:87-101, 312-434 ---- */
+int get_leading_dimension(cudamat* mat);
+int get_nonleading_dimension(cudamat* mat);
+void set_transpose(cudamat* mat, int is_trans);
+int set_shape(cudamat* mat, unsigned int m, unsigned int n);
+int reshape(cudamat* mat, unsigned int m, unsigned int n);
+int get_slice(cudamat* source, cudamat* target, unsigned int first_col, unsigned int last_col);
+int get_vector_slice(cudamat* source, cudamat* target, unsigned int first_ind, unsigned int last_ind);
+void init_from_array(cudamat* mat, float* data, int m, int n);
+void set_on_device(cudamat* mat);
+int init_empty(cudamat* mat, int m, int n);
+
+/* ---- allocation and transfers: cudamat.cu:109-123, 153-186, 217-229, 298-310 ---- */
+int allocate_device_memory(cudamat* mat);
+int copy_to_host(cudamat* mat);
+int copy_to_device(cudamat* mat);
+int copy_on_device(cudamat* mat1, cudamat* mat2);
+int free_device_memory(cudamat* mat);
+
+/* ---- row slices and transpose: cudamat.cu:231-296 ---- */
+int get_row_slice(cudamat* source, cudamat* target, unsigned int start, unsigned int end);
+int set_row_slice(cudamat* source, cudamat* target, unsigned int start, unsigned int end);
+int copy_transpose(cudamat* source, cudamat* target);
+
+/* ---- multiply-with-carry RNG: cudamat.cu:55-83, 437-588; kernels cudamat_kernels.cu:96-239 ---- */
+int init_random(rnd_struct* rnd_state, int seed, char* cudamatpath);
+int fill_with_rand(rnd_struct* rnd_state, cudamat* mat);
+int fill_with_randn(rnd_struct* rnd_state, cudamat* mat);
+int sample_bernoulli(rnd_struct* rnd_state, cudamat* mat, cudamat* target);
+int sample_bernoulli_tanh(rnd_struct* rnd_state, cudamat* mat, cudamat* target);
+int sample_poisson(rnd_struct* rnd_state, cudamat* mat, cudamat* target);
+int sample_gaussian(rnd_struct* rnd_state, cudamat* mat, cudamat* target, float mult);
+int perturb_energy(rnd_struct* rnd_state, cudamat* mat, cudamat* target);
+int perturb_prob(rnd_struct* rnd_state, cudamat* mat, cudamat* target);
+int dropout(rnd_struct* rnd_state, cudamat* mat, float dropprob, float val);
+
+/* ---- broadcasts of a row / column / diagonal vector: cudamat.cu:592-877 ---- */
+int add_col_vec(cudamat* mat, cudamat* vec, cudamat* target);
+int add_col_mult(cudamat* mat, cudamat* vec, cudamat* target, float mult);
+int add_row_vec(cudamat* mat, cudamat* vec, cudamat* target);
+int add_row_mult(cudamat* mat, cudamat* vec, cudamat* target, float mult);
+int mult_by_col_vec(cudamat* mat, cudamat* vec, cudamat* target);
+int mult_by_row_vec(cudamat* mat, cudamat* vec, cudamat* target);
+int div_by_col_vec(cudamat* mat, cudamat* vec, cudamat* target);
+int div_by_row_vec(cudamat* mat, cudamat* vec, cudamat* target);
+int mult_diagonal_scalar(cudamat* mat, float val, cudamat* target);
+int add_diagonal_scalar(cudamat* mat, float val, cudamat* target);
+int mult_diagonal(cudamat* mat, cudamat* vec, cudamat* target);
+int add_diagonal(cudamat* mat, cudamat* vec, cudamat* target);
+
+/* ---- comparisons and clamps: cudamat.cu:878-1146 ---- */
+int less_than_eq(cudamat* mat1, cudamat* mat2, cudamat* target);
+int less_than(cudamat* mat1, cudamat* mat2, cudamat* target);
+int less_than_eq_scalar(cudamat* mat, float val, cudamat* target);
+int less_than_scalar(cudamat* mat, float val, cudamat* target);
+int greater_than_eq(cudamat* mat1, cudamat* mat2, cudamat* target);
+int greater_than(cudamat* mat1, cudamat* mat2, cudamat* target);
+int greater_than_eq_scalar(cudamat* mat, float val, cudamat* target);
+int greater_than_scalar(cudamat* mat, float val, cudamat* target);
+int upper_bound(cudamat* mat1, cudamat* mat2, cudamat* target);
+int lower_bound(cudamat* mat1, cudamat* mat2, cudamat* target);
+int upper_bound_scalar(cudamat* mat, float val, cudamat* target);
+int lower_bound_scalar(cudamat* mat, float val, cudamat* target);
+
+/* ---- reductions along an axis: cudamat.cu:1148-1315.
+ * axis 0 reduces each column (the reference's only supported case).  axis 1,
+ * which the reference answers with ERROR_UNSUPPORTED, reduces each row here with
+ * the semantics of eigenmat/eigenmat.cc:617-731. ---- */
+int max_by_axis(cudamat* mat, cudamat* target, int axis);
+int argmax_by_axis(cudamat* mat, cudamat* target, int axis);
+int choose_max_by_axis(cudamat* mat, cudamat* target, int axis);
+int choose_max_and_accumulate(cudamat* mat, cudamat* acc);
+int sqsum_by_axis(cudamat* mat, cudamat* target, int axis, float mult, float p);
+int normlimit_by_axis(cudamat* mat, cudamat* target, int axis, float norm);
+
+/* ---- unary math: cudamat.cu:1318-1669 ---- */
+int sign(cudamat* mat, cudamat* target);
+int apply_cos(cudamat* mat, cudamat* target);
+int apply_sin(cudamat* mat, cudamat* target);
+int apply_sigmoid(cudamat* mat, cudamat* target);
+int apply_tanh(cudamat* mat, cudamat* target);
+int apply_abs(cudamat* mat, cudamat* target);
+int apply_log_1_plus_exp(cudamat* mat, cudamat* target);
+int apply_log(cudamat* mat, cudamat* target, float tiny);
+int apply_exp(cudamat* mat, cudamat* target);
+int apply_ceil(cudamat* mat, cudamat* target);
+int apply_floor(cudamat* mat, cudamat* target);
+int apply_sqrt(cudamat* mat, cudamat* target);
+int apply_pow(cudamat* mat, float pow, cudamat* target);
+int apply_pow_matrix(cudamat* mat, cudamat* pow, cudamat* target);
+int compute_cross_entropy(cudamat* mat, cudamat* p, cudamat* target, float tiny);
+int compute_cross_entropy_bernoulli(cudamat* mat, cudamat* p, cudamat* target, float tiny);
+int correct_preds(cudamat* mat, cudamat* p, cudamat* target, float cutoff);
+int reciprocal(cudamat* mat, cudamat* target);
+
+/* ---- dense contraction and BLAS-1: cudamat.cu:1671-1781, 2104-2118.
+ * dot: target = beta*target + alpha*op(mat1)*op(mat2), op chosen by is_trans;
+ * the target's is_trans flag is ignored (beta comes before alpha). ---- */
+int dot(cudamat* mat1, cudamat* mat2, cudamat* target, float beta, float alpha);
+float vdot(cudamat* mat1, cudamat* mat2, int* err_code);
+int add_mult(cudamat* mat1, cudamat* mat2, float alpha);
+float euclid_norm(cudamat* mat, int* err_code);
+
+/* ---- binary elementwise and activation derivatives: cudamat.cu:1782-2030 ---- */
+int add_mult_sign(cudamat* mat1, cudamat* mat2, float mult);
+int add_elementwise(cudamat* mat1, cudamat* mat2, cudamat* target);
+int subtract_elementwise(cudamat* mat1, cudamat* mat2, cudamat* target);
+int divide_elementwise(cudamat* mat1, cudamat* mat2, cudamat* target);
+int mult_elementwise(cudamat* mat1, cudamat* mat2, cudamat* target);
+int apply_sin_deriv(cudamat* mat1, cudamat* mat2, cudamat* target);
+int apply_cos_deriv(cudamat* mat1, cudamat* mat2, cudamat* target);
+int apply_logistic_deriv(cudamat* mat1, cudamat* mat2, cudamat* target);
+int apply_tanh_deriv(cudamat* mat1, cudamat* mat2, cudamat* target);
+int apply_rectified_linear_deriv(cudamat* mat1, cudamat* mat2, cudamat* target);
+int apply_rectified_linear_smooth_deriv(cudamat* mat1, cudamat* mat2, cudamat* target);
+
+/* ---- scalar ops: cudamat.cu:2031-2102 ---- */
+int assign_scalar(cudamat* mat, float alpha);
+int mult_by_scalar(cudamat* mat, float alpha, cudamat* target);
+int divide_by_scalar(cudamat* mat, float alpha, cudamat* target);
+int add_scalar(cudamat* mat, float alpha, cudamat* target);
+
+/* ---- column gather / scatter with float-encoded indices: cudamat.cu:2120-2189, 2295-2399 ---- */
+int selectRows(cudamat* source, cudamat* target, cudamat* indices);
+int swapColumns(cudamat* source, cudamat* target, cudamat* indices1, cudamat* indices2);
+int setSelectedRows(cudamat* target, cudamat* source, cudamat* indices);
+int generate_translations_big_var_off(cudamat* source, cudamat* target, cudamat* off_x, cudamat* off_y,
+                                      int source_w, int target_w, int num_channels);
+int blockify(cudamat* source, cudamat* target, int blocksize);
+int accumulate_columns(cudamat* mat, cudamat* indices, cudamat* target, float mult, int avg);
+int expand(cudamat* source, cudamat* indices, cudamat* target);
+int expand_and_add(cudamat* source, cudamat* mat, cudamat* indices, cudamat* target, float mult);
+
+/* ---- column softmax and its loss helpers: cudamat.cu:2192-2346 ---- */
+int softmax(cudamat* mat, cudamat* target);
+int softmax_overwrite(cudamat* mat);
+int apply_softmax_grad(cudamat* mat, cudamat* labels, cudamat* target);
+int get_softmax_correct(cudamat* mat, cudamat* labels, cudamat* target);
+int get_softmax_cross_entropy(cudamat* mat, cudamat* labels, cudamat* target, float tiny);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CUDAMAT_AMD_H_ */

@@ -1,0 +1,117 @@
+"""GPU parity of dot / add_dot / subtract_dot (fp32 MFMA kernel and the
+matrix-vector paths) against np.dot in float64: 1e-4 relative."""
+import numpy as np
+import pytest
+
+from oracle import cudamat_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+REL = 1e-4
+
+
+def _rand(rng, shape):
+    return np.asarray(rng.standard_normal(shape), dtype=np.float32, order='F')
+
+
+def _relerr(got, want, A, B):
+    """Error relative to |A|.|B| elementwise bound (robust to cancellation)."""
+    bound = np.abs(A).astype(np.float64) @ np.abs(B).astype(np.float64)
+    return np.max(np.abs(np.asarray(got, np.float64) - want) / (bound + 1e-30))
+
+
+# (m, k, n): test_cudamat.py:796-880 uses 128x256x64-like shapes, eigenmat/test.py:23-47
+# 500x1000x600; the rest are the benchmark's step shapes and ragged edges.
+SHAPES = [(64, 128, 32), (128, 256, 64), (500, 1000, 600), (500, 784, 100), (784, 500, 100),
+          (784, 100, 500), (1024, 784, 128), (10, 1024, 128), (1024, 128, 1024), (1, 5, 1),
+          (33, 17, 65), (130, 1, 70), (129, 257, 131), (1, 300, 40), (300, 40, 1), (5, 7, 3)]
+
+
+@pytest.mark.parametrize("m,k,n", SHAPES)
+@pytest.mark.parametrize("ta,tb", [(False, False), (True, False), (False, True), (True, True)])
+def test_dot_all_transpose_combinations(cm, rng, m, k, n, ta, tb):
+    A, B = _rand(rng, (m, k)), _rand(rng, (k, n))
+    a = cm.CUDAMatrix(np.asfortranarray(A.T)) if ta else cm.CUDAMatrix(A)
+    b = cm.CUDAMatrix(np.asfortranarray(B.T)) if tb else cm.CUDAMatrix(B)
+    t = cm.dot(a.T if ta else a, b.T if tb else b)
+    assert t.shape == (m, n)
+    want = A.astype(np.float64) @ B.astype(np.float64)
+    assert _relerr(t.asarray(), want, A, B) < REL
+    for h in (a, b, t):
+        h.free_device_memory()
+
+
+@pytest.mark.parametrize("alpha,beta", [(1.0, 0.0), (1.0, 1.0), (-1.0, 1.0), (np.pi, -1.0), (0.0, 1.0)])
+def test_alpha_beta(cm, rng, alpha, beta):
+    A, B, C = _rand(rng, (128, 256)), _rand(rng, (256, 64)), _rand(rng, (128, 64))
+    a, b, c = cm.CUDAMatrix(A), cm.CUDAMatrix(B), cm.CUDAMatrix(C)
+    cm._check(cm._cudamat.dot(a.p_mat, b.p_mat, c.p_mat, beta, alpha))
+    want = orc.dot(A, B, C, beta=beta, alpha=alpha)
+    bound = abs(alpha) * (np.abs(A).astype(np.float64) @ np.abs(B)) + abs(beta) * np.abs(C) + 1e-30
+    assert np.max(np.abs(c.asarray() - want) / bound) < REL
+
+
+def test_beta_zero_ignores_garbage_in_target(cm, rng):
+    A, B = _rand(rng, (70, 30)), _rand(rng, (30, 50))
+    t = cm.CUDAMatrix(np.full((70, 50), np.nan, dtype=np.float32))
+    cm.dot(cm.CUDAMatrix(A), cm.CUDAMatrix(B), target=t)
+    assert np.all(np.isfinite(t.asarray()))
+
+
+def test_add_dot_subtract_dot_and_mult(cm, rng):
+    A, B, C = _rand(rng, (784, 100)), _rand(rng, (500, 100)), _rand(rng, (784, 500))
+    a, b, c = cm.CUDAMatrix(A), cm.CUDAMatrix(B), cm.CUDAMatrix(C)
+    c.add_dot(a, b.T, mult=0.01)
+    want = C + 0.01 * (A.astype(np.float64) @ B.T)
+    assert np.max(np.abs(c.asarray() - want)) < 1e-4
+    c.subtract_dot(a, b.T)
+    want = want - A.astype(np.float64) @ B.T
+    assert np.max(np.abs(c.asarray() - want) / (np.abs(A).astype(np.float64) @ np.abs(B.T) + 1)) < REL
+    d = a.dot(b.T, mult=2.0)
+    assert _relerr(d.asarray(), 2.0 * (A.astype(np.float64) @ B.T), 2 * A, B.T) < REL
+
+
+def test_dot_on_column_views(cm, rng):
+    # operands that start 37*k floats into a buffer: unaligned loads inside the tile loader
+    A, B = _rand(rng, (37, 90)), _rand(rng, (37, 50))
+    a, b = cm.CUDAMatrix(A), cm.CUDAMatrix(B)
+    va, vb = a.slice(5, 85), b.slice(3, 47)
+    t = cm.dot(va.T, vb)
+    want = A[:, 5:85].astype(np.float64).T @ B[:, 3:47]
+    assert _relerr(t.asarray(), want, A[:, 5:85].T, B[:, 3:47]) < REL
+
+
+def test_dot_error_codes(cm, rng):
+    a, b = cm.CUDAMatrix(_rand(rng, (8, 6))), cm.CUDAMatrix(_rand(rng, (5, 4)))
+    with pytest.raises(cm.CUDAMatException, match="Incompatible matrix dimensions"):
+        cm.dot(a, b)
+    with pytest.raises(cm.CUDAMatException, match="Incompatible matrix dimensions"):
+        cm.dot(a, cm.CUDAMatrix(_rand(rng, (6, 4))), target=cm.empty((8, 5)))
+    host_only = cm.CUDAMatrix(_rand(rng, (6, 4)), copy_to_device=False)
+    with pytest.raises(cm.CUDAMatException, match="not in device memory"):
+        cm.dot(a, host_only, target=cm.empty((8, 4)))
+
+
+@pytest.mark.parametrize("n", [2048, 4096])
+def test_large_square_products(cm, rng, n):
+    """Checked on sampled rows/columns against float64 and through the identity
+    (A B) x = A (B x) on the whole product."""
+    A = np.asarray(rng.uniform(-1, 1, (n, n)), dtype=np.float32, order='F')
+    B = np.asarray(rng.uniform(-1, 1, (n, n)), dtype=np.float32, order='F')
+    a, b = cm.CUDAMatrix(A), cm.CUDAMatrix(B)
+    c = cm.dot(a, b)
+    got = c.asarray()
+    rows = np.arange(0, n, 211); cols = np.arange(0, n, 173)
+    want = A[rows, :].astype(np.float64) @ B[:, cols].astype(np.float64)
+    bound = np.abs(A[rows, :]).astype(np.float64) @ np.abs(B[:, cols]).astype(np.float64)
+    assert np.max(np.abs(got[np.ix_(rows, cols)] - want) / bound) < REL
+    x = rng.uniform(-1, 1, (n,))
+    lhs = got.astype(np.float64) @ x
+    rhs = A.astype(np.float64) @ (B.astype(np.float64) @ x)
+    assert np.max(np.abs(lhs - rhs)) / np.max(np.abs(rhs)) < 1e-4
+    ct_ = cm.dot(a.T, b.T)
+    want_t = A[:, rows].astype(np.float64).T @ B[cols, :].astype(np.float64).T
+    bound_t = np.abs(A[:, rows]).astype(np.float64).T @ np.abs(B[cols, :]).astype(np.float64).T
+    assert np.max(np.abs(ct_.asarray()[np.ix_(rows, cols)] - want_t) / bound_t) < REL
+    for h in (a, b, c, ct_):
+        h.free_device_memory()

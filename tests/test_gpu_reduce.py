@@ -1,0 +1,175 @@
+"""GPU parity of reductions, softmax and the sum path (dot with ones):
+1e-5 relative for sums / sums of squares / softmax, exact for max / argmax."""
+import numpy as np
+import pytest
+
+from oracle import cudamat_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+REL = 1e-5
+SHAPES = [(256, 128), (37, 53), (1, 7), (7, 1), (4100, 3), (3, 4100), (10, 128), (1000, 1000)]
+
+
+def _rand(rng, shape, lo=-1.0, hi=1.0):
+    return np.asarray(rng.uniform(lo, hi, shape), dtype=np.float32, order='F')
+
+
+def _rel(got, want, scale=None):
+    want = np.asarray(want, dtype=np.float64)
+    scale = np.maximum(np.abs(want), 1e-30) if scale is None else scale
+    return np.max(np.abs(np.asarray(got, np.float64) - want) / scale)
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("axis", [0, 1])
+def test_sum(cm, rng, shape, axis):
+    x = _rand(rng, shape)
+    a = cm.CUDAMatrix(x)
+    got = a.sum(axis=axis).asarray()
+    want = x.astype(np.float64).sum(axis=axis, keepdims=True)
+    # error relative to the sum of magnitudes (sums of signed values can cancel)
+    assert _rel(got, want, np.abs(x).astype(np.float64).sum(axis=axis, keepdims=True) + 1e-30) < REL
+    assert got.shape == want.shape
+
+
+def test_sum_of_transposed_and_add_sums_and_total(cm, rng):
+    x = _rand(rng, (300, 200), 0.0, 1.0)
+    a = cm.CUDAMatrix(x)
+    # test_cudamat.py:298-327: sums of a.T are the sums of the transpose
+    assert _rel(cm.sum(a.T, axis=0).asarray(), x.T.astype(np.float64).sum(axis=0, keepdims=True)) < REL
+    assert _rel(cm.sum(a.T, axis=1).asarray(), x.T.astype(np.float64).sum(axis=1, keepdims=True)) < REL
+    t0 = _rand(rng, (300, 1)); t = cm.CUDAMatrix(t0)
+    t.add_sums(a, axis=1, mult=-0.5)
+    assert _rel(t.asarray(), t0 - 0.5 * x.astype(np.float64).sum(axis=1, keepdims=True)) < 2e-5
+    t1 = _rand(rng, (1, 200)); t = cm.CUDAMatrix(t1)
+    t.add_sums(a, axis=0, mult=2.0)
+    assert _rel(t.asarray(), t1 + 2.0 * x.astype(np.float64).sum(axis=0, keepdims=True)) < REL
+    assert abs(a.sum() - x.astype(np.float64).sum()) / x.astype(np.float64).sum() < REL
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("axis", [0, 1])
+def test_max_argmax(cm, rng, shape, axis):
+    x = _rand(rng, shape)
+    a = cm.CUDAMatrix(x)
+    assert np.array_equal(a.max(axis=axis).asarray(), orc.max_by_axis(x, axis).astype(np.float32))
+    assert np.array_equal(a.argmax(axis=axis).asarray(), orc.argmax_by_axis(x, axis).astype(np.float32))
+
+
+def test_argmax_ties_follow_the_reference_scan_order(cm):
+    # equal maxima at rows 2 and 33: the reference's 32-lane scan reports 33
+    # (lane 33 % 32 = 1 is visited before lane 2), cudamat_kernels.cu:1020-1050
+    x = np.zeros((70, 3), dtype=np.float32, order='F')
+    x[2, 0] = x[33, 0] = 5.0
+    x[64, 1] = x[0, 1] = x[32, 1] = 1.0      # lane 0 holds rows 0, 32, 64 -> first of them
+    x[:, 2] = -np.inf                          # nothing beats the start value: index 0, max -FLT_MAX
+    a = cm.CUDAMatrix(x)
+    assert a.argmax(axis=0).asarray().tolist() == [[33.0, 0.0, 0.0]]
+    assert orc.argmax_by_axis(x, 0).tolist() == [[33.0, 0.0, 0.0]]
+    m = a.max(axis=0).asarray()
+    assert m[0, 0] == 5.0 and m[0, 2] == -np.finfo(np.float32).max
+    # axis 1: first occurrence
+    y = np.zeros((3, 70), dtype=np.float32, order='F'); y[1, 40] = y[1, 7] = 2.0
+    assert cm.CUDAMatrix(y).argmax(axis=1).asarray().ravel().tolist() == [0.0, 7.0, 0.0]
+
+
+@pytest.mark.parametrize("shape", [(256, 128), (37, 53), (5000, 2)])
+@pytest.mark.parametrize("axis", [0, 1])
+def test_sqsum_and_norm_limit_and_choose_max(cm, rng, shape, axis):
+    x = _rand(rng, shape)
+    a = cm.CUDAMatrix(x)
+    got = a.sqsum(axis=axis).asarray()
+    assert _rel(got, orc.sqsum_by_axis(x, None, axis, 1.0, 0.0)) < REL
+    t0 = _rand(rng, got.shape); t = cm.CUDAMatrix(t0)
+    t.add_sqsums(a, axis=axis, mult=0.25)
+    assert _rel(t.asarray(), orc.sqsum_by_axis(x, t0, axis, 0.25, 1.0)) < 2e-5
+    norm = float(np.median(np.sqrt((x.astype(np.float64) ** 2).sum(axis=axis))))
+    lim = cm.empty(shape)
+    a.norm_limit(norm, axis, target=lim)
+    want = orc.normlimit_by_axis(x, axis, norm)
+    assert np.allclose(lim.asarray(), want, rtol=1e-5, atol=1e-7)
+    ch = cm.empty(shape)
+    a.choose_max(axis, target=ch)
+    assert np.array_equal(ch.asarray(), orc.choose_max_by_axis(x, axis).astype(np.float32))
+    a.choose_max(axis)          # in place
+    assert np.array_equal(a.asarray(), orc.choose_max_by_axis(x, axis).astype(np.float32))
+
+
+def test_choose_max_and_accumulate(cm, rng):
+    x = _rand(rng, (10, 40))
+    acc0 = np.ones((10, 40), dtype=np.float32, order='F')
+    a, acc = cm.CUDAMatrix(x), cm.CUDAMatrix(acc0)
+    a.choose_max_and_accumulate(acc)
+    assert np.array_equal(acc.asarray(), acc0 + orc.choose_max_by_axis(x, 0).astype(np.float32))
+
+
+@pytest.mark.parametrize("shape", [(100, 10), (10, 128), (4096, 64), (1000, 33), (37, 53), (5, 1), (20000, 3)])
+def test_softmax(cm, rng, shape):
+    x = _rand(rng, shape, -8, 8)
+    a, t = cm.CUDAMatrix(x), cm.empty(shape)
+    a.apply_softmax(target=t)
+    got = t.asarray()
+    assert _rel(got, orc.softmax(x)) < REL
+    assert np.max(np.abs(got.astype(np.float64).sum(axis=0) - 1.0)) < 1e-5
+    # shift invariance: softmax(x + c) == softmax(x)
+    b = cm.CUDAMatrix(x + np.float32(3.0))
+    b.apply_softmax()
+    assert np.allclose(b.asarray(), got, rtol=2e-5, atol=1e-9)
+    a.apply_softmax()            # overwrite variant
+    assert np.array_equal(a.asarray(), got)
+
+
+def test_softmax_loss_helpers(cm, rng):
+    x = _rand(rng, (10, 128), -3, 3)
+    labels = np.asarray(rng.integers(0, 10, (1, 128)), dtype=np.float32, order='F')
+    p = cm.CUDAMatrix(x); p.apply_softmax()
+    pn = p.asarray().copy()
+    lab = cm.CUDAMatrix(labels)
+    t = cm.empty((1, 128))
+    p.get_softmax_correct(lab, t)
+    assert np.array_equal(t.asarray(), orc.get_softmax_correct(pn, labels).astype(np.float32))
+    p.get_softmax_cross_entropy(lab, t, tiny=1e-10)
+    assert _rel(t.asarray(), orc.get_softmax_cross_entropy(pn, labels, 1e-10)) < REL
+    g = cm.empty((10, 128))
+    p.apply_softmax_grad(lab, target=g)
+    assert np.array_equal(g.asarray(), orc.apply_softmax_grad(pn, labels).astype(np.float32))
+
+
+def test_vdot_and_euclid_norm(cm, rng):
+    for shape in [(1, 1), (37, 53), (1000, 999)]:
+        x, y = _rand(rng, shape), _rand(rng, shape)
+        a, b = cm.CUDAMatrix(x), cm.CUDAMatrix(y)
+        scale = np.abs(x.astype(np.float64) * y).sum()
+        assert abs(cm.vdot(a, b) - orc.vdot(x, y)) / scale < REL
+        assert abs(a.euclid_norm() - orc.euclid_norm(x)) / orc.euclid_norm(x) < REL
+    with pytest.raises(cm.CUDAMatException, match="Incompatible matrix dimensions"):
+        cm.vdot(a, cm.CUDAMatrix(_rand(rng, (3, 3))))
+
+
+def test_axis_error_codes(cm, rng):
+    a = cm.CUDAMatrix(_rand(rng, (8, 6)))
+    with pytest.raises(cm.CUDAMatException, match="Incompatible matrix dimensions"):
+        a.max(axis=0, target=cm.empty((6, 1)))
+    with pytest.raises(cm.CUDAMatException, match="transposed"):
+        cm._check(cm._cudamat.max_by_axis(a.T.p_mat, cm.empty((1, 6)).p_mat, 0))
+    with pytest.raises(cm.CUDAMatException, match="not supported"):
+        cm._check(cm._cudamat.max_by_axis(a.p_mat, cm.empty((1, 6)).p_mat, 2))
+
+
+@pytest.mark.parametrize("axis", [0, 1])
+def test_full_size_4096_sum_max_softmax(cm, rng, axis):
+    n = 4096
+    x = np.asarray(rng.uniform(-1, 1, (n, n)), dtype=np.float32, order='F')
+    a = cm.CUDAMatrix(x)
+    x64 = x.astype(np.float64)
+    got = a.sum(axis=axis).asarray()
+    assert _rel(got, x64.sum(axis=axis, keepdims=True), np.abs(x64).sum(axis=axis, keepdims=True)) < REL
+    assert np.array_equal(a.max(axis=axis).asarray(), x.max(axis=axis, keepdims=True))
+    if axis == 0:
+        a.apply_softmax()
+        got = a.asarray()
+        assert np.max(np.abs(got.astype(np.float64).sum(axis=0) - 1.0)) < 1e-5
+        cols = np.arange(0, n, 97)
+        assert _rel(got[:, cols], orc.softmax(x[:, cols])) < REL
+    a.free_device_memory()
