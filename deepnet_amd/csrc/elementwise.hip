@@ -7,6 +7,7 @@
 // aligned (column views) are peeled to alignment when they share the same
 // offset and fall back to 4-byte accesses otherwise.
 #include "common.h"
+#include "wide_math.h"
 #include <math.h>
 
 // ------------------------------------------------------------------ functors
@@ -30,20 +31,18 @@
 
 // unary (cudamat_kernels.cu:386-506)
 DN_FUNCTOR0(FSign, a ? copysignf(1.f, a) : 0.f)
-DN_FUNCTOR0(FCos, cosf(a))
-DN_FUNCTOR0(FSin, sinf(a))
-DN_FUNCTOR0(FSigmoid, 1.f / (1.f + expf(-a)))
-// 1 - 2/(exp(2x)+1) is tanh(x); evaluated as tanhf so the result carries the accuracy of
-// the formula itself rather than the cancellation of its fp32 steps near 0.
-DN_FUNCTOR0(FTanh, tanhf(a))
+DN_FUNCTOR0(FCos, (float)dn_cos_wide(a))
+DN_FUNCTOR0(FSin, (float)dn_sin_wide(a))
+DN_FUNCTOR0(FSigmoid, dn_sigmoid(a))
+DN_FUNCTOR0(FTanh, dn_tanh(a))
 DN_FUNCTOR0(FAbs, a * (float)((a > 0.f) - (a < 0.f)))
-DN_FUNCTOR0(FLog1pExp, a > 0.f ? (log1pf(expf(-a)) + a) : log1pf(expf(a)))
-DN_FUNCTOR1(FLog, logf(a + s))
-DN_FUNCTOR0(FExp, expf(a))
+DN_FUNCTOR0(FLog1pExp, dn_softplus(a))
+DN_FUNCTOR1(FLog, dn_log(a + s))
+DN_FUNCTOR0(FExp, dn_exp(a))
 DN_FUNCTOR0(FCeil, ceilf(a))
 DN_FUNCTOR0(FFloor, floorf(a))
 DN_FUNCTOR0(FSqrt, sqrtf(a))
-DN_FUNCTOR1(FPow, powf(a, s))
+DN_FUNCTOR1(FPow, dn_pow(a, s))
 DN_FUNCTOR0(FRecip, (float)(1.0 / (double)a))
 // binary (cudamat_kernels.cu:298-364, 476-500, 600-685)
 DN_FUNCTOR0(FLt, a < b ? 1.f : 0.f)
@@ -56,17 +55,18 @@ DN_FUNCTOR0(FAdd, a + b)
 DN_FUNCTOR0(FSub, a - b)
 DN_FUNCTOR0(FDiv, a / b)
 DN_FUNCTOR0(FMul, a * b)
-DN_FUNCTOR0(FPowMat, powf(a, b))
-DN_FUNCTOR0(FCosDeriv, -a * sinf(b))
-DN_FUNCTOR0(FSinDeriv, a * cosf(b))
+DN_FUNCTOR0(FPowMat, dn_pow(a, b))
+DN_FUNCTOR0(FCosDeriv, (float)(-(double)a * dn_sin_wide(b)))
+DN_FUNCTOR0(FSinDeriv, (float)((double)a * dn_cos_wide(b)))
 DN_FUNCTOR0(FLogisticDeriv, (float)((double)(a * b) * (1.0 - (double)b)))
 DN_FUNCTOR0(FTanhDeriv, (float)((double)a * (1.0 + (double)b) * (1.0 - (double)b) * 0.5))
 DN_FUNCTOR0(FReluDeriv, a * (b > 0.f ? 1.f : 0.f))
-DN_FUNCTOR0(FReluSmoothDeriv, a * -expm1f(-b))
+DN_FUNCTOR0(FReluSmoothDeriv, (float)((double)a * -dn_expm1_wide(-(double)b)))
 DN_FUNCTOR1(FAxpy, a + s * b)
 DN_FUNCTOR1(FAddMultSign, a + ((b > 0.f) ? s : ((b < 0.f) ? -s : 0.f)))
-DN_FUNCTOR1(FCrossEntropy, -a * logf(b + s))
-DN_FUNCTOR1(FCrossEntropyBernoulli, -a * logf(b + s) - (1.f - a) * logf(1.f - b + s))
+DN_FUNCTOR1(FCrossEntropy, (float)(-(double)a * dn_log_wide(b + s)))
+DN_FUNCTOR1(FCrossEntropyBernoulli,
+            (float)(-(double)a * dn_log_wide(b + s) - (double)(1.f - a) * dn_log_wide(1.f - b + s)))
 DN_FUNCTOR1(FCorrectPreds, a * (float)(b >= s) + (1.f - a) * (float)(b < s))
 // matrix (op) scalar (cudamat_kernels.cu:310-364, 687-716)
 DN_FUNCTOR1(FLtS, a < s ? 1.f : 0.f)

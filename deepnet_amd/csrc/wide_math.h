@@ -1,0 +1,152 @@
+// Transcendentals for fp32 inputs evaluated with fp64 internals to a relative
+// error of about 2^-33, so that a whole formula (exp -> add -> divide, log of a
+// sum, a * cos(b) ...) is rounded to fp32 once, at its end.  The fp32 library
+// routines are each allowed a few ulp and a chain of them drifts past the
+// 2-ulp parity bar; fp64 FMAs issue at the fp32 rate on this part, so these cost
+// about as many issue slots as the fp32 versions.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <math.h>
+
+// 1/d for finite non-zero d: hardware estimate plus one Newton step.
+__device__ __forceinline__ double dn_rcp_wide(double d) {
+  double r = __builtin_amdgcn_rcp(d);
+  return r * fma(-d, r, 2.0);
+}
+
+// e^t and e^t - 1.  t*log2(e) is split into an integer n and a fraction; with
+// g = fraction*ln2, |g| <= 0.347, q(g) = e^g - 1 is a degree-8 Taylor sum
+// (remainder g^9/9! < 2.1e-10 of e^g).  e^t = 2^n (1 + q); e^t - 1 is q itself
+// when n == 0, which keeps full relative accuracy for small t.  Arguments beyond
+// +-800 saturate (0 or inf in fp64 either way).
+__device__ __forceinline__ double dn_exp_parts(double t, double* n_out) {
+  t = fmin(fmax(t, -800.0), 800.0) * 1.4426950408889634;
+  const double n = rint(t);
+  const double g = (t - n) * 0.6931471805599453;
+  double p = 2.48015873015873e-05;       // 1/8!
+  p = fma(p, g, 1.984126984126984e-04);  // 1/7!
+  p = fma(p, g, 1.388888888888889e-03);  // 1/6!
+  p = fma(p, g, 8.333333333333333e-03);  // 1/5!
+  p = fma(p, g, 4.166666666666666e-02);  // 1/4!
+  p = fma(p, g, 1.666666666666667e-01);  // 1/3!
+  p = fma(p, g, 0.5);
+  p = fma(p, g, 1.0);
+  *n_out = n;
+  return p * g;  // q(g)
+}
+__device__ __forceinline__ double dn_exp_wide(double t) {
+  double n;
+  const double q = dn_exp_parts(t, &n);
+  return ldexp(1.0 + q, (int)n);
+}
+__device__ __forceinline__ double dn_expm1_wide(double t) {
+  double n;
+  const double q = dn_exp_parts(t, &n);
+  return n == 0.0 ? q : ldexp(1.0 + q, (int)n) - 1.0;
+}
+
+// ln(x) for finite x > 0 (callers handle 0, negatives, inf, NaN).
+// x = m * 2^e with m in [sqrt(1/2), sqrt(2)); ln m = 2*atanh(s), s = (m-1)/(m+1),
+// |s| <= 0.1716, series through s^12/13 (remainder below 2^-39 of the result).
+__device__ __forceinline__ double dn_log_wide_pos(double x) {
+  int e;
+  double m = frexp(x, &e);  // m in [0.5, 1)
+  if (m < 0.7071067811865476) { m *= 2.0; e -= 1; }
+  const double s = (m - 1.0) * dn_rcp_wide(m + 1.0);
+  const double z = s * s;
+  double p = 1.0 / 13.0;
+  p = fma(p, z, 1.0 / 11.0);
+  p = fma(p, z, 1.0 / 9.0);
+  p = fma(p, z, 1.0 / 7.0);
+  p = fma(p, z, 1.0 / 5.0);
+  p = fma(p, z, 1.0 / 3.0);
+  p = fma(p, z, 1.0);
+  return fma((double)e, 0.6931471805599453, 2.0 * s * p);
+}
+
+// ln(x) with logf's special values, still in fp64.
+__device__ __forceinline__ double dn_log_wide(float x) {
+  if (x > 0.f && x < INFINITY) return dn_log_wide_pos((double)x);
+  if (x == 0.f) return -(double)INFINITY;
+  if (x < 0.f) return (double)NAN;
+  return (double)x;  // +inf or NaN
+}
+__device__ __forceinline__ float dn_log(float x) { return (float)dn_log_wide(x); }
+
+// ln(1 + e^x): x + ln(1 + e^-x) for x > 0, ln(1 + e^x) otherwise; ln(1 + u) for a
+// tiny u is u - u^2/2 + u^3/3 (1 + u itself would round u away).
+__device__ __forceinline__ float dn_softplus(float x) {
+  if (x != x) return x;
+  const double u = dn_exp_wide(-(double)fabsf(x));  // in (0, 1]
+  const double l = u < 1e-5 ? u * fma(u, fma(u, 1.0 / 3.0, -0.5), 1.0) : dn_log_wide_pos(1.0 + u);
+  return (float)(x > 0.f ? l + (double)x : l);
+}
+
+// tanh(x) = (e^2x - 1) / (e^2x + 1), the value of the formula 1 - 2/(e^2x + 1).
+__device__ __forceinline__ float dn_tanh(float x) {
+  if (x != x) return x;
+  const double em = dn_expm1_wide(2.0 * (double)fminf(fmaxf(x, -20.f), 20.f));
+  return (float)(em * dn_rcp_wide(em + 2.0));
+}
+
+__device__ __forceinline__ float dn_exp(float x) { return x != x ? x : (float)dn_exp_wide((double)x); }
+
+// 1/(1+exp(-x))
+__device__ __forceinline__ float dn_sigmoid(float x) {
+  const double s = 1.0 + dn_exp_wide(-(double)x);   // in [1, inf]
+  const float r = (s < 1e300) ? (float)dn_rcp_wide(s) : 0.f;
+  return x != x ? x : r;
+}
+
+// sin and cos of x.  Cody-Waite reduction by pi/2 in fp64 (exact through the FMA
+// for |x| < 2^30), then Taylor sums on [-pi/4, pi/4] (remainders < 1e-11).
+// Larger arguments take the library's fp64 routines.
+__device__ __forceinline__ void dn_sincos_wide(float x, double* sn, double* cs) {
+  const double xd = (double)x;
+  if (!(fabsf(x) < 1.0e9f)) {  // huge, inf or NaN
+    *sn = sin(xd);
+    *cs = cos(xd);
+    return;
+  }
+  const double k = rint(xd * 0.6366197723675814);
+  double r = fma(-k, 1.5707963267948966, xd);
+  r = fma(-k, 6.123233995736766e-17, r);
+  const double z = r * r;
+  double ps = -2.505210838544172e-08;      // -1/11!
+  ps = fma(ps, z, 2.755731922398589e-06);  //  1/9!
+  ps = fma(ps, z, -1.984126984126984e-04); // -1/7!
+  ps = fma(ps, z, 8.333333333333333e-03);  //  1/5!
+  ps = fma(ps, z, -1.666666666666667e-01); // -1/3!
+  const double s = fma(r * z, ps, r);
+  double pc = 2.08767569878681e-09;        //  1/12!
+  pc = fma(pc, z, -2.755731922398589e-07); // -1/10!
+  pc = fma(pc, z, 2.48015873015873e-05);   //  1/8!
+  pc = fma(pc, z, -1.388888888888889e-03); // -1/6!
+  pc = fma(pc, z, 4.166666666666666e-02);  //  1/4!
+  pc = fma(pc, z, -0.5);
+  const double c = fma(pc, z, 1.0);
+  const int q = (int)k & 3;
+  const double s_out = (q & 1) ? c : s;
+  const double c_out = (q & 1) ? s : c;
+  *sn = (q & 2) ? -s_out : s_out;
+  *cs = ((q + 1) & 2) ? -c_out : c_out;
+}
+__device__ __forceinline__ double dn_sin_wide(float x) { double s, c; dn_sincos_wide(x, &s, &c); return s; }
+__device__ __forceinline__ double dn_cos_wide(float x) { double s, c; dn_sincos_wide(x, &s, &c); return c; }
+
+// powf(x, p) as exp(p * ln x) in fp64 for the ordinary cases (finite x != 0 with a
+// finite p, negative x only with an integer p); everything else is an exact
+// special value and is left to the library.
+__device__ __forceinline__ float dn_pow(float x, float p) {
+  const float ax = fabsf(x);
+  const bool p_finite = fabsf(p) < INFINITY;
+  if (ax > 0.f && ax < INFINITY && p_finite) {
+    if (x > 0.f) return (float)dn_exp_wide((double)p * dn_log_wide_pos((double)ax));
+    if (rintf(p) == p) {
+      const float r = (float)dn_exp_wide((double)p * dn_log_wide_pos((double)ax));
+      const bool odd = fabsf(p) < 16777216.f && (((long long)p) & 1);
+      return odd ? -r : r;
+    }
+  }
+  return powf(x, p);
+}

@@ -58,9 +58,11 @@ def apply_abs(x):
 
 
 def apply_log_1_plus_exp(x):
+    # log(1 + exp(x)), branches as in cudamat_kernels.cu:427-438; log1p keeps the
+    # float64 evaluation faithful to the formula when exp(.) is far below 1
     x = _a(x)
     with np.errstate(over='ignore'):
-        return np.where(x > 0, np.log(1.0 + np.exp(-x)) + x, np.log(1.0 + np.exp(x)))
+        return np.where(x > 0, np.log1p(np.exp(-x)) + x, np.log1p(np.exp(x)))
 
 
 def apply_log(x, tiny=0.0):
@@ -121,7 +123,7 @@ def apply_sin_deriv(a, b): return _a(a) * np.cos(_a(b))
 def apply_logistic_deriv(a, b): return _a(a) * _a(b) * (1.0 - _a(b))
 def apply_tanh_deriv(a, b): return _a(a) * (1.0 + _a(b)) * (1.0 - _a(b)) * 0.5
 def apply_rectified_linear_deriv(a, b): return _a(a) * (_a(b) > 0)
-def apply_rectified_linear_smooth_deriv(a, b): return _a(a) * (1.0 - np.exp(-_a(b)))
+def apply_rectified_linear_smooth_deriv(a, b): return _a(a) * -np.expm1(-_a(b))  # a*(1 - exp(-b))
 def add_mult(a, b, alpha): return _a(a) + F64(np.float32(alpha)) * _a(b)
 
 

@@ -111,7 +111,7 @@ BINARY = [
     ('less_than', orc.less_than, 0), ('less_than_eq', orc.less_than_eq, 0),
     ('greater_than', orc.greater_than, 0), ('greater_than_eq', orc.greater_than_eq, 0),
     ('upper_bound', orc.upper_bound, 0), ('lower_bound', orc.lower_bound, 0),
-    ('apply_logistic_deriv', orc.apply_logistic_deriv, 1), ('apply_tanh_deriv', orc.apply_tanh_deriv, 1),
+    ('apply_logistic_deriv', orc.apply_logistic_deriv, ULP), ('apply_tanh_deriv', orc.apply_tanh_deriv, 1),
     ('apply_rectified_linear_deriv', orc.apply_rectified_linear_deriv, 0),
     ('apply_rectified_linear_smooth_deriv', orc.apply_rectified_linear_smooth_deriv, ULP),
     ('apply_cos_deriv', orc.apply_cos_deriv, ULP), ('apply_sin_deriv', orc.apply_sin_deriv, ULP),
@@ -302,3 +302,60 @@ def test_full_size_4096(cm, rng, name):
         a.add_row_vec(cm.CUDAMatrix(v))
         assert np.array_equal(a.asarray(), x + v)
     a.free_device_memory()
+
+
+def _log_uniform(rng, n, lo_exp, hi_exp, signed=True):
+    x = np.exp2(rng.uniform(lo_exp, hi_exp, n))
+    if signed:
+        x *= rng.choice([-1.0, 1.0], n)
+    return np.asarray(x, dtype=np.float32).reshape(-1, 1)
+
+
+def test_transcendentals_over_their_whole_range(cm, rng):
+    """2 ulp against the float64 value of each formula from denormal to overflow
+    magnitudes, including the special values."""
+    n = 200000
+    specials = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1.0, -1.0, 1e-45, -1e-45, 3.4e38, -3.4e38,
+                         88.72284, -87.33655, -103.97, 16.635532, -16.635532], dtype=np.float32).reshape(-1, 1)
+    wide = np.vstack([_log_uniform(rng, n, -149, 128), specials])
+    moderate = np.vstack([_log_uniform(rng, n, -30, 7), specials])          # up to +-128
+    positive = np.vstack([_log_uniform(rng, n, -149, 128, signed=False), specials])
+    trig = np.vstack([_log_uniform(rng, n, -30, 29), _log_uniform(rng, 1000, 29, 128), specials])
+    cases = [('exp', orc.apply_exp, moderate), ('sigmoid', orc.apply_sigmoid, moderate),
+             ('tanh', np.tanh, wide), ('log_1_plus_exp', lambda v: np.logaddexp(0.0, v.astype(np.float64)), moderate),
+             ('sqrt', orc.apply_sqrt, positive), ('cos', orc.apply_cos, trig), ('sin', orc.apply_sin, trig)]
+    for name, ofn, x in cases:
+        a = cm.CUDAMatrix(x)
+        getattr(cm, name)(a)
+        with np.errstate(all='ignore'):
+            want = ofn(x.astype(np.float64))
+        d = orc.ulp_diff(a.asarray(), want)
+        k = int(np.argmax(d))
+        assert d.max() <= ULP, "%s: %.2f ulp at x=%r (got %r want %r)" % (name, d.max(), x.ravel()[k],
+                                                                       a.asarray().ravel()[k], want.ravel()[k])
+        a.free_device_memory()
+    a = cm.CUDAMatrix(positive)
+    cm.log(a)
+    with np.errstate(all='ignore'):
+        want = np.log(positive.astype(np.float64))
+    d = orc.ulp_diff(a.asarray(), want)
+    assert d.max() <= ULP, "log: %.2f ulp at %r" % (d.max(), positive.ravel()[int(np.argmax(d))])
+    # pow: positive bases with any exponent, negative bases with integer exponents
+    base = _log_uniform(rng, n, -40, 40, signed=False)
+    expo = np.asarray(rng.uniform(-3, 3, (n, 1)), dtype=np.float32)
+    a, p = cm.CUDAMatrix(base), cm.CUDAMatrix(expo)
+    cm.pow(a, p)
+    with np.errstate(all='ignore'):
+        want = np.power(base.astype(np.float64), expo.astype(np.float64))
+    d = orc.ulp_diff(a.asarray(), want)
+    assert d.max() <= ULP, "pow: %.2f ulp" % d.max()
+    nb = -_log_uniform(rng, 1000, -10, 10, signed=False)
+    for e in (-3.0, -2.0, 0.0, 1.0, 2.0, 5.0):
+        a = cm.CUDAMatrix(nb)
+        cm.pow(a, e)
+        d = orc.ulp_diff(a.asarray(), np.power(nb.astype(np.float64), e))
+        assert d.max() <= ULP, "pow(neg, %g): %.2f ulp" % (e, d.max())
+    a = cm.CUDAMatrix(np.array([[0.0, -2.0, 2.0, np.inf, np.nan]], dtype=np.float32))
+    cm.pow(a, 0.5)
+    got = a.asarray().ravel()
+    assert got[0] == 0 and np.isnan(got[1]) and abs(got[2] - np.sqrt(2)) < 1e-7 and np.isinf(got[3]) and np.isnan(got[4])

@@ -83,7 +83,8 @@ def test_sqsum_and_norm_limit_and_choose_max(cm, rng, shape, axis):
     assert _rel(got, orc.sqsum_by_axis(x, None, axis, 1.0, 0.0)) < REL
     t0 = _rand(rng, got.shape); t = cm.CUDAMatrix(t0)
     t.add_sqsums(a, axis=axis, mult=0.25)
-    assert _rel(t.asarray(), orc.sqsum_by_axis(x, t0, axis, 0.25, 1.0)) < 2e-5
+    want = orc.sqsum_by_axis(x, t0, axis, 0.25, 1.0)
+    assert _rel(t.asarray(), want, np.abs(t0) + np.abs(want - t0)) < REL
     norm = float(np.median(np.sqrt((x.astype(np.float64) ** 2).sum(axis=axis))))
     lim = cm.empty(shape)
     a.norm_limit(norm, axis, target=lim)

@@ -25,7 +25,7 @@ def _device_words(cm):
     view.on_device, view.on_host, view.is_trans, view.owns_data = 1, 0, 0, 0
     view.size[0], view.size[1] = 2 * N, 1
     m = cm.CUDAMatrix(view)
-    return m.asarray().view(np.uint64).ravel().copy()
+    return m.asarray().ravel(order='F').view(np.uint64).copy()
 
 
 @pytest.mark.parametrize("seed", [0, 1, 42, 2**31 - 1])
