@@ -1,0 +1,404 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X matrix backend on synthetic data (one GPU).
+
+A "step" is one pass over the elementwise / reduction / RNG op list of the
+4096 x 4096 fp32 microbench, each op issued once on each of NSETS distinct
+operand sets (so consecutive launches stream from HBM, not from the 256 MB
+last-level cache).  `value` is the algorithmic bytes of a step divided by its
+wall time (inputs resident in HBM, device synchronised on both sides).
+
+Next to it, in the same JSON line:
+  roofline      the axpy kernel (add_mult): algorithmic bytes per launch over the
+                launch duration measured with HIP events on the NULL stream
+  ops           per-op GB/s and fraction of the 8 TB/s HBM peak
+  secondary     RBM CD-1 steps/s (784 x 500, batch 100), MLP steps/s, fp32 GEMM and
+                conv TFLOP/s with their fraction of the 157.3 TFLOP/s MFMA peak
+  cpu_baseline  the same op list timed through the C host restatement
+                (oracle/host_backend.c) on this machine's cores
+"""
+import argparse
+import ctypes as ct
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+MFMA_FP32_PEAK_TFLOPS = 157.3
+N = 4096
+NSETS = 8
+
+
+# ---------------------------------------------------------------- HIP events
+
+class HipEvents(object):
+    """hipEvent timing on the NULL stream (the stream the library launches on)."""
+
+    def __init__(self):
+        self.hip = ct.CDLL('libamdhip64.so')
+        self.hip.hipEventCreate.argtypes = [ct.POINTER(ct.c_void_p)]
+        self.hip.hipEventRecord.argtypes = [ct.c_void_p, ct.c_void_p]
+        self.hip.hipEventSynchronize.argtypes = [ct.c_void_p]
+        self.hip.hipEventElapsedTime.argtypes = [ct.POINTER(ct.c_float), ct.c_void_p, ct.c_void_p]
+        self.pool = []
+
+    def new(self):
+        ev = ct.c_void_p()
+        assert self.hip.hipEventCreate(ct.byref(ev)) == 0
+        self.pool.append(ev)
+        return ev
+
+    def record(self, ev):
+        assert self.hip.hipEventRecord(ev, None) == 0
+
+    def elapsed_ms(self, a, b):
+        assert self.hip.hipEventSynchronize(b) == 0
+        ms = ct.c_float()
+        assert self.hip.hipEventElapsedTime(ct.byref(ms), a, b) == 0
+        return ms.value
+
+
+# ---------------------------------------------------------------- workload
+
+def build_c2(cm, seed=2):
+    """Operand sets of the 4096^2 microbench (seeded, U(-1,1); probabilities U(0,1))."""
+    rng = np.random.default_rng(seed)
+    sets = []
+    for _ in range(NSETS):
+        s = {}
+        s['A'] = cm.CUDAMatrix(np.asarray(rng.uniform(-1, 1, (N, N)), dtype=np.float32, order='F'))
+        s['B'] = cm.CUDAMatrix(np.asarray(rng.uniform(-1, 1, (N, N)), dtype=np.float32, order='F'))
+        s['P'] = cm.CUDAMatrix(np.asarray(rng.random((N, N)), dtype=np.float32, order='F'))
+        s['T'] = cm.empty((N, N))
+        s['col'] = cm.CUDAMatrix(np.asarray(rng.uniform(-1, 1, (N, 1)), dtype=np.float32, order='F'))
+        s['row'] = cm.CUDAMatrix(np.asarray(rng.uniform(-1, 1, (1, N)), dtype=np.float32, order='F'))
+        s['r0'] = cm.empty((1, N))
+        s['r1'] = cm.empty((N, 1))
+        sets.append(s)
+    return sets
+
+
+E = N * N
+VEC = N * 4
+# name -> (algorithmic bytes per launch, callable(set))
+C2_OPS = [
+    ('add_mult', 12 * E, lambda cm, s: s['A'].add_mult(s['B'], 0.5)),
+    ('mult', 12 * E, lambda cm, s: s['A'].mult(s['B'], target=s['T'])),
+    ('apply_sigmoid', 8 * E, lambda cm, s: s['A'].apply_sigmoid(target=s['T'])),
+    ('apply_exp', 8 * E, lambda cm, s: cm.exp(s['A'], target=s['T'])),
+    ('mult_by_col', 8 * E + VEC, lambda cm, s: s['A'].mult_by_col(s['col'], target=s['T'])),
+    ('add_row_vec', 8 * E + VEC, lambda cm, s: s['A'].add_row_vec(s['row'], target=s['T'])),
+    ('sum_axis0', 4 * E + VEC, lambda cm, s: s['A'].sum(axis=0, target=s['r0'])),
+    ('sum_axis1', 4 * E + VEC, lambda cm, s: s['A'].sum(axis=1, target=s['r1'])),
+    ('max_axis0', 4 * E + VEC, lambda cm, s: s['A'].max(axis=0, target=s['r0'])),
+    ('max_axis1', 4 * E + VEC, lambda cm, s: s['A'].max(axis=1, target=s['r1'])),
+    ('softmax', 8 * E, lambda cm, s: s['A'].apply_softmax(target=s['T'])),
+    ('fill_with_rand', 4 * E, lambda cm, s: s['T'].fill_with_rand()),
+    ('sample_bernoulli', 8 * E, lambda cm, s: s['P'].sample_bernoulli(target=s['T'])),
+]
+STEP_BYTES = NSETS * sum(b for _, b, _ in C2_OPS)
+
+
+def run_c2_step(cm, sets, ev=None, marks=None):
+    """One step.  With ev/marks, brackets each op's NSETS launches with events."""
+    for name, _, fn in C2_OPS:
+        if ev is not None:
+            a, b = marks[name]
+            ev.record(a)
+        for s in sets:
+            fn(cm, s)
+        if ev is not None:
+            ev.record(b)
+
+
+# ---------------------------------------------------------------- secondary workloads
+
+class RBM(object):
+    """CD-1 step, 784 visible x 500 hidden, batch 100 (seed 1): dot -> sigmoid ->
+    sample_bernoulli -> dot -> sigmoid -> dot -> sigmoid -> add_dot updates."""
+
+    def __init__(self, cm, nv=784, nh=500, B=100, lr=0.01, seed=1):
+        rng = np.random.default_rng(seed)
+        self.cm, self.B, self.lr = cm, B, lr
+        self.v = cm.CUDAMatrix(np.asarray(rng.random((nv, B)) < 0.13, dtype=np.float32, order='F'))
+        self.W = cm.CUDAMatrix(np.asarray(0.01 * rng.standard_normal((nv, nh)), dtype=np.float32, order='F'))
+        self.bv = cm.CUDAMatrix(np.zeros((nv, 1), dtype=np.float32))
+        self.bh = cm.CUDAMatrix(np.zeros((nh, 1), dtype=np.float32))
+        self.h, self.hs, self.h2 = cm.empty((nh, B)), cm.empty((nh, B)), cm.empty((nh, B))
+        self.v2 = cm.empty((nv, B))
+        self.flops = 5 * 2 * nv * nh * B
+
+    def step(self):
+        cm, eps = self.cm, self.lr / self.B
+        W, v, h, hs, v2, h2 = self.W, self.v, self.h, self.hs, self.v2, self.h2
+        cm.dot(W.T, v, target=h); h.add_col_vec(self.bh); h.apply_sigmoid()
+        h.sample_bernoulli(target=hs)
+        cm.dot(W, hs, target=v2); v2.add_col_vec(self.bv); v2.apply_sigmoid()
+        cm.dot(W.T, v2, target=h2); h2.add_col_vec(self.bh); h2.apply_sigmoid()
+        W.add_dot(v, h.T, mult=eps); W.add_dot(v2, h2.T, mult=-eps)
+        self.bv.add_sums(v, axis=1, mult=eps); self.bv.add_sums(v2, axis=1, mult=-eps)
+        self.bh.add_sums(h, axis=1, mult=eps); self.bh.add_sums(h2, axis=1, mult=-eps)
+
+
+class MLP(object):
+    """784-1024-1024-10 ReLU net, softmax cross-entropy, dropout 0.5 on the hidden
+    layers (fill_with_rand -> greater_than -> mult), momentum SGD; batch 128, seed 3.
+    Op sequence of deepnet/neuralnet.py:138-291 and parameter.py:80-106."""
+
+    def __init__(self, cm, sizes=(784, 1024, 1024, 10), B=128, lr=0.01, mom=0.9, seed=3):
+        rng = np.random.default_rng(seed)
+        self.cm, self.B, self.lr, self.mom, self.sizes = cm, B, lr, mom, sizes
+        f = lambda a: cm.CUDAMatrix(np.asarray(a, dtype=np.float32, order='F'))
+        self.x = f(rng.random((sizes[0], B)))
+        self.labels = f(rng.integers(0, sizes[-1], (1, B)))
+        self.W = [f(0.01 * rng.standard_normal((sizes[i], sizes[i + 1]))) for i in range(3)]
+        self.b = [f(np.zeros((sizes[i + 1], 1))) for i in range(3)]
+        self.dW = [f(np.zeros((sizes[i], sizes[i + 1]))) for i in range(3)]
+        self.db = [f(np.zeros((sizes[i + 1], 1))) for i in range(3)]
+        self.gW = [cm.empty((sizes[i], sizes[i + 1])) for i in range(3)]
+        self.gb = [cm.empty((sizes[i + 1], 1)) for i in range(3)]
+        self.act = [self.x] + [cm.empty((sizes[i + 1], B)) for i in range(3)]
+        self.mask = [cm.empty((sizes[i + 1], B)) for i in range(2)]
+        self.delta = [cm.empty((sizes[i + 1], B)) for i in range(3)]
+        self.loss = cm.empty((1, B))
+        self.flops = 3 * 2 * B * (sizes[0] * sizes[1] + sizes[1] * sizes[2] + sizes[2] * sizes[3])
+
+    def step(self):
+        cm, B = self.cm, self.B
+        act, W, b = self.act, self.W, self.b
+        for i in range(3):
+            cm.dot(W[i].T, act[i], target=act[i + 1])
+            act[i + 1].add_col_vec(b[i])
+            if i < 2:
+                act[i + 1].lower_bound(0)
+                self.mask[i].fill_with_rand(); self.mask[i].greater_than(0.5); act[i + 1].mult(self.mask[i])
+            else:
+                act[i + 1].apply_softmax()
+        act[3].get_softmax_cross_entropy(self.labels, self.loss)
+        act[3].apply_softmax_grad(self.labels, target=self.delta[2])
+        for i in (2, 1, 0):
+            self.gW[i].assign(0); self.gW[i].add_dot(act[i], self.delta[i].T, mult=1.0 / B)
+            self.gb[i].assign(0); self.gb[i].add_sums(self.delta[i], axis=1, mult=1.0 / B)
+            if i > 0:
+                cm.dot(W[i], self.delta[i], target=self.delta[i - 1])
+                self.delta[i - 1].apply_rectified_linear_deriv(act[i])
+        for i in range(3):
+            for p, d, g in ((W[i], self.dW[i], self.gW[i]), (b[i], self.db[i], self.gb[i])):
+                d.mult(self.mom); d.add_mult(g); p.add_mult(d, -self.lr)
+
+
+def time_loop(cm, fn, iters, warmup):
+    for _ in range(warmup):
+        fn()
+    cm.cuda_sync_threads()
+    t0 = time.perf_counter()
+    for _ in range(iters):
+        fn()
+    cm.cuda_sync_threads()
+    return (time.perf_counter() - t0) / iters
+
+
+def gemm_probe(cm, ev, n=4096, iters=10):
+    rng = np.random.default_rng(6)
+    a = cm.CUDAMatrix(np.asarray(rng.uniform(-1, 1, (n, n)), dtype=np.float32, order='F'))
+    b = cm.CUDAMatrix(np.asarray(rng.uniform(-1, 1, (n, n)), dtype=np.float32, order='F'))
+    c = cm.empty((n, n))
+    out = {}
+    for label, x, y in (('nn', a, b), ('tn', a.T, b), ('nt', a, b.T)):
+        cm.dot(x, y, target=c)
+        e0, e1 = ev.new(), ev.new()
+        ev.record(e0)
+        for _ in range(iters):
+            cm.dot(x, y, target=c)
+        ev.record(e1)
+        ms = ev.elapsed_ms(e0, e1) / iters
+        tf = 2.0 * n ** 3 / (ms * 1e-3) / 1e12
+        out[label] = {'ms': round(ms, 4), 'tflops': round(tf, 2), 'frac_mfma_fp32': round(tf / MFMA_FP32_PEAK_TFLOPS, 4)}
+    for m in (a, b, c):
+        m.free_device_memory()
+    return out
+
+
+# ---------------------------------------------------------------- CPU baseline
+
+def cpu_baseline_c2():
+    """The same op list through the C host restatement, single thread, one pass over
+    ONE operand set (4096^2) per op; RNG through the host MWC."""
+    from oracle import mwc
+    lib = ct.CDLL(os.path.join(ROOT, 'oracle', 'liboracle_host.so'))
+    fp = ct.POINTER(ct.c_float)
+    rng = np.random.default_rng(2)
+    A = np.asarray(rng.uniform(-1, 1, (N, N)), dtype=np.float32, order='F')
+    B = np.asarray(rng.uniform(-1, 1, (N, N)), dtype=np.float32, order='F')
+    P = np.asarray(rng.random((N, N)), dtype=np.float32, order='F')
+    T = np.empty((N, N), dtype=np.float32, order='F')
+    col = np.asarray(rng.uniform(-1, 1, N), dtype=np.float32)
+    r = np.empty(N, dtype=np.float32)
+    mults = mwc.load_multipliers(os.path.join(ROOT, 'deepnet_amd', 'rnd_multipliers_32bit.txt'))
+    words = np.empty(mwc.NUM_RND_STREAMS, dtype=np.uint64)
+    p = lambda a: a.ctypes.data_as(fp)
+    u32 = mults.ctypes.data_as(ct.POINTER(ct.c_uint32))
+    u64 = words.ctypes.data_as(ct.POINTER(ct.c_uint64))
+    lib.mwc_seed(u32, u64, ct.c_uint32(2))
+    sz = ct.c_size_t(E)
+    lib.hb_set_threads(1)
+    ops = [
+        ('add_mult', lambda: lib.hb_add_mult(p(A), p(B), ct.c_float(0.5), sz)),
+        ('mult', lambda: lib.hb_mult(p(A), p(B), p(T), sz)),
+        ('apply_sigmoid', lambda: lib.hb_sigmoid(p(A), p(T), sz)),
+        ('apply_exp', lambda: lib.hb_exp(p(A), p(T), sz)),
+        ('mult_by_col', lambda: lib.hb_mult_by_col(p(A), p(col), p(T), N, N)),
+        ('add_row_vec', lambda: lib.hb_add_row_vec(p(A), p(col), p(T), N, N)),
+        ('sum_axis0', lambda: lib.hb_add_sums(p(A), p(r), N, N, 0, ct.c_float(0), ct.c_float(1))),
+        ('sum_axis1', lambda: lib.hb_add_sums(p(A), p(r), N, N, 1, ct.c_float(0), ct.c_float(1))),
+        ('max_axis0', lambda: lib.hb_max(p(A), p(r), N, N, 0)),
+        ('max_axis1', lambda: lib.hb_max(p(A), p(r), N, N, 1)),
+        ('softmax', lambda: lib.hb_softmax(p(A), p(T), N, N)),
+        ('fill_with_rand', lambda: lib.mwc_uniform(u32, u64, p(T), sz)),
+        ('sample_bernoulli', lambda: lib.mwc_bernoulli(u32, u64, p(P), p(T), sz)),
+    ]
+    assert [o[0] for o in ops] == [o[0] for o in C2_OPS]
+    for _, fn in ops:      # touch everything once
+        fn()
+    t0 = time.perf_counter()
+    per_op = {}
+    for name, fn in ops:
+        t1 = time.perf_counter()
+        fn()
+        per_op[name] = time.perf_counter() - t1
+    total = time.perf_counter() - t0
+    nbytes = sum(b for _, b, _ in C2_OPS)
+    return {'value': round(nbytes / total / 1e9, 3), 'unit': 'GB/s', 'cores': 1, 'kind': 'port',
+            'sample': 'one pass of the 13-op list over one 4096x4096 operand set (1/%d of a GPU step), '
+                      'oracle/host_backend.c, gcc -O3 x86-64-v3, 1 thread; host has %d cpus' % (NSETS, os.cpu_count()),
+            'seconds': round(total, 3),
+            'per_op_gbs': {n: round(b / per_op[n] / 1e9, 2) for n, b, _ in C2_OPS}}
+
+
+def cpu_baseline_rbm(steps=10):
+    from oracle import mwc
+    lib = ct.CDLL(os.path.join(ROOT, 'oracle', 'liboracle_host.so'))
+    fp = ct.POINTER(ct.c_float)
+    nv, nh, B = 784, 500, 100
+    rng = np.random.default_rng(1)
+    v = np.asarray(rng.random((nv, B)) < 0.13, dtype=np.float32, order='F')
+    W = np.asarray(0.01 * rng.standard_normal((nv, nh)), dtype=np.float32, order='F')
+    bv, bh = np.zeros(nv, np.float32), np.zeros(nh, np.float32)
+    h, hs, h2 = (np.empty((nh, B), np.float32, order='F') for _ in range(3))
+    v2 = np.empty((nv, B), np.float32, order='F')
+    mults = mwc.load_multipliers(os.path.join(ROOT, 'deepnet_amd', 'rnd_multipliers_32bit.txt'))
+    words = np.empty(mwc.NUM_RND_STREAMS, dtype=np.uint64)
+    u32 = mults.ctypes.data_as(ct.POINTER(ct.c_uint32))
+    u64 = words.ctypes.data_as(ct.POINTER(ct.c_uint64))
+    lib.mwc_seed(u32, u64, ct.c_uint32(1))
+    p = lambda a: a.ctypes.data_as(fp)
+    out = {}
+    for threads in (1, os.cpu_count() or 1):
+        lib.hb_set_threads(threads)
+        call = lambda: lib.hb_rbm_cd1_step(p(W), p(bv), p(bh), p(v), nv, nh, B, ct.c_float(0.01), u32, u64,
+                                           p(h), p(hs), p(v2), p(h2))
+        call()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            call()
+        out[threads] = steps / (time.perf_counter() - t0)
+    lib.hb_set_threads(1)
+    return out
+
+
+# ---------------------------------------------------------------- main
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument('--gpus', type=int, default=1)
+    ap.add_argument('--steps', type=int, default=10)
+    ap.add_argument('--warmup', type=int, default=2)
+    ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
+    ap.add_argument('--only-c2', action='store_true', help='skip the secondary workloads')
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this backend has no multi-GPU path (run with --gpus 1).")
+
+    from deepnet_amd import cudamat as cm
+    cm.cublas_init()
+    cm.CUDAMatrix.init_random(2)
+    ev = HipEvents()
+
+    sets = build_c2(cm)
+    marks = {name: (ev.new(), ev.new()) for name, _, _ in C2_OPS}
+    for _ in range(args.warmup):
+        run_c2_step(cm, sets)
+    cm.cuda_sync_threads()
+    per_op_ms = {name: [] for name, _, _ in C2_OPS}
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        run_c2_step(cm, sets, ev, marks)
+        # reading the events back waits for the step, which the next step would do anyway
+        for name, _, _ in C2_OPS:
+            per_op_ms[name].append(ev.elapsed_ms(*marks[name]) / NSETS)
+    cm.cuda_sync_threads()
+    step_s = (time.perf_counter() - t0) / args.steps
+
+    ops = {}
+    for name, nbytes, _ in C2_OPS:
+        ms = float(np.median(per_op_ms[name]))
+        gbs = nbytes / (ms * 1e-3) / 1e9
+        ops[name] = {'us': round(ms * 1e3, 2), 'gbs': round(gbs, 1), 'frac_hbm': round(gbs / HBM_PEAK_GBS, 4)}
+    value = STEP_BYTES / step_s / 1e9
+
+    roof_op = 'add_mult'
+    roofline = {'kernel': 'k_ew<2, FAxpy> (add_mult, 4096x4096)', 'bound': 'hbm',
+                'achieved': ops[roof_op]['gbs'], 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
+                'frac': round(ops[roof_op]['gbs'] / HBM_PEAK_GBS, 4), 'traffic': None,
+                'algorithmic_bytes_per_launch': 12 * E, 'avg_launch_us': ops[roof_op]['us']}
+
+    secondary = {}
+    if not args.only_c2:
+        for s in sets:
+            for m in s.values():
+                m.free_device_memory()
+        cm.CUDAMatrix.init_random(1)
+        rbm = RBM(cm)
+        t = time_loop(cm, rbm.step, 200, 20)
+        secondary['rbm_cd1'] = {'steps_per_sec': round(1.0 / t, 1), 'us_per_step': round(t * 1e6, 1),
+                                'gemm_tflops': round(rbm.flops / t / 1e12, 3),
+                                'config': '784 visible x 500 hidden, batch 100, fp32'}
+        cm.CUDAMatrix.init_random(3)
+        mlp = MLP(cm)
+        t = time_loop(cm, mlp.step, 100, 10)
+        secondary['mlp_784_1024_1024_10'] = {'steps_per_sec': round(1.0 / t, 1), 'us_per_step': round(t * 1e6, 1),
+                                              'gemm_tflops': round(mlp.flops / t / 1e12, 3), 'batch': 128}
+        secondary['gemm_fp32_4096'] = gemm_probe(cm, ev)
+        try:
+            import bench_conv
+            secondary.update(bench_conv.run(cm, ev))
+        except ImportError:
+            pass
+
+    line = {
+        'metric': 'RBM CD-1 steps/sec; elementwise HBM GB/s; conv fp32 TFLOP/s vs roofline',
+        'value': round(value, 1), 'unit': 'GB/s (elementwise/reduction/RNG microbench, algorithmic bytes)',
+        'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup, 'ms_per_step': round(step_s * 1e3, 3),
+        'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None, 'dtype': 'f32', 'data': 'synthetic',
+        'config': {'workload': 'elementwise+reduction+RNG microbench, 4096x4096 fp32 column-major, 13 ops x %d '
+                               'operand sets per step' % NSETS, 'step_bytes': STEP_BYTES},
+        'roofline': roofline, 'ops': ops, 'secondary': secondary,
+    }
+    if not args.no_cpu:
+        cb = cpu_baseline_c2()
+        if not args.only_c2:
+            r = cpu_baseline_rbm()
+            cb['rbm_cd1_steps_per_sec'] = {'threads_%d' % k: round(v, 2) for k, v in r.items()}
+            if 'rbm_cd1' in secondary:
+                secondary['rbm_cd1']['vs_cpu_1thread'] = round(secondary['rbm_cd1']['steps_per_sec'] / r[1], 1)
+        line['cpu_baseline'] = cb
+    print(json.dumps(line))
+
+
+if __name__ == '__main__':
+    main()
