@@ -9,6 +9,9 @@
 // One CU count for launch sizing; MI355X has 256 CUs in 8 XCDs.  Queried once.
 int dn_num_cus();
 
+// Grow-only device workspace shared by the two-stage kernels (partials + results).
+void* dn_scratch(size_t bytes);
+
 // Records the launch status of the kernel just queued; returns CUDA_ERROR or 0.
 static inline int dn_launch_status() {
   return hipPeekAtLastError() == hipSuccess ? 0 : CUDA_ERROR;

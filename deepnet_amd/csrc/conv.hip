@@ -1,0 +1,643 @@
+// Shared-filter convolution in cuda-convnet's (channels, rows, cols, batch)
+// layout: forward (convUp), gradient w.r.t. the images (convDown) and w.r.t. the
+// filters (convOutp).  Replaces cudamat/cudamat_conv.cu:15-1015 and the kernel
+// templates cudamat_conv_kernels.cuh:82-1235.
+//
+// All three passes are one implicit GEMM  C(r, c) = sum_kk A(r, kk) * B(kk, c)  on
+// the fp32 matrix cores (v_mfma_f32_32x32x2_f32), with 16-deep operand slabs
+// gathered straight from the tensors into LDS (double buffered):
+//
+//   pass   rows r                 cols c            kk                 A                 B
+//   Up     (module, image)        filter of group   (colour, ky, kx)   image patch       filters
+//   Down   (pixel of phase, img)  colour of group   (tap, filter)      hidden acts       filters
+//   Outp   filter of group        (colour, ky, kx)  (module, image)    hidden acts       image patch
+//
+// The batch index is the fastest-varying one everywhere, so rows of Up/Down and
+// the kk of Outp are contiguous runs of images: every gather is a 16-byte load of
+// four neighbouring images.  Down with stride s runs as s*s "phases" (pixels with
+// equal (y - pad) mod s share their set of filter taps), which turns the strided
+// transpose convolution into stride-1 problems without multiplying by zeros.
+// Outp reduces over modules x images with few outputs, so K is split across
+// workgroups and summed by a second kernel.
+//
+// The matrix-core path needs numImages % 16 == 0, filters-per-group % 16 == 0 and
+// 16-byte aligned buffers; anything else takes the one-thread-per-output kernels
+// below, which are also the cross-check of the fast path in the tests.
+#include "common.h"
+#include "../../include/cudamat_conv_amd.h"
+#include <math.h>
+#include <stdio.h>
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+enum { CONV_UP = 0, CONV_DOWN = 1, CONV_OUTP = 2 };
+
+struct ConvArgs {
+  const float* img;   // images: input of Up/Outp
+  const float* flt;   // filters: input of Up/Down
+  const float* hid;   // hidden activations / their gradients: input of Down/Outp
+  float* out;         // Up: hidden acts, Down: images, Outp: filter gradients
+  float* partial;     // Outp split-K workspace
+  int N, C, Cg, H, F, Fg, k, Mx, s, pad0, G;
+  int M, HH, kk2;     // Mx*Mx, H*H, k*k
+  int m_begin, m_count;  // Outp: module chunk [m_begin, m_begin + m_count)
+  int splits, slabs_per_split;
+  float scale_t, scale_o;
+  FastDiv dN, dMx, dk, dkk2;
+};
+
+// ------------------------------------------------------------------ direct kernels
+// One lane per output element; images are the fastest index, so neighbouring
+// lanes read neighbouring addresses.
+
+__global__ void k_conv_up_direct(ConvArgs p) {
+  const long long total = (long long)p.N * p.M * p.F;
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += stride) {
+    const int n = (int)(e % p.N);
+    const int m = (int)((e / p.N) % p.M);
+    const int f = (int)(e / ((long long)p.N * p.M));
+    const int g = f / p.Fg;
+    const int y0 = (m / p.Mx) * p.s + p.pad0, x0 = (m % p.Mx) * p.s + p.pad0;
+    float acc = 0.f;
+    for (int c = 0; c < p.Cg; ++c)
+      for (int ky = 0; ky < p.k; ++ky) {
+        const int y = y0 + ky;
+        if (y < 0 || y >= p.H) continue;
+        for (int kx = 0; kx < p.k; ++kx) {
+          const int x = x0 + kx;
+          if (x < 0 || x >= p.H) continue;
+          acc += p.img[(size_t)p.N * ((size_t)(g * p.Cg + c) * p.HH + y * p.H + x) + n] *
+                 p.flt[(size_t)p.F * ((c * p.k + ky) * p.k + kx) + f];
+        }
+      }
+    p.out[e] = (p.scale_t == 0.f ? 0.f : p.scale_t * p.out[e]) + p.scale_o * acc;
+  }
+}
+
+__global__ void k_conv_down_direct(ConvArgs p) {
+  const long long total = (long long)p.N * p.HH * p.C;
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += stride) {
+    const int n = (int)(e % p.N);
+    const int pix = (int)((e / p.N) % p.HH);
+    const int c = (int)(e / ((long long)p.N * p.HH));
+    const int g = c / p.Cg, cl = c % p.Cg;
+    const int y = pix / p.H - p.pad0, x = pix % p.H - p.pad0;  // coordinates in the padded frame
+    float acc = 0.f;
+    for (int my = 0; my < p.Mx; ++my) {
+      const int ky = y - my * p.s;
+      if (ky < 0 || ky >= p.k) continue;
+      for (int mx = 0; mx < p.Mx; ++mx) {
+        const int kx = x - mx * p.s;
+        if (kx < 0 || kx >= p.k) continue;
+        const size_t wbase = (size_t)p.F * ((cl * p.k + ky) * p.k + kx);
+        for (int fl = 0; fl < p.Fg; ++fl) {
+          const int f = g * p.Fg + fl;
+          acc += p.hid[(size_t)p.N * ((size_t)f * p.M + my * p.Mx + mx) + n] * p.flt[wbase + f];
+        }
+      }
+    }
+    p.out[e] = (p.scale_t == 0.f ? 0.f : p.scale_t * p.out[e]) + p.scale_o * acc;
+  }
+}
+
+// One workgroup per output (f, c, ky, kx): 256 lanes stride over (module, image)
+// of the chunk and meet in LDS.
+__global__ void __launch_bounds__(256) k_conv_outp_direct(ConvArgs p) {
+  __shared__ float red[4];
+  const int q = blockIdx.x % (p.Cg * p.kk2);
+  const int f = blockIdx.x / (p.Cg * p.kk2);
+  const int g = f / p.Fg;
+  const int c = q / p.kk2, ky = (q % p.kk2) / p.k, kx = q % p.k;
+  const long long total = (long long)p.m_count * p.N;
+  float acc = 0.f;
+  for (long long e = threadIdx.x; e < total; e += 256) {
+    const int n = (int)(e % p.N);
+    const int m = p.m_begin + (int)(e / p.N);
+    const int y = (m / p.Mx) * p.s + p.pad0 + ky, x = (m % p.Mx) * p.s + p.pad0 + kx;
+    if (y < 0 || y >= p.H || x < 0 || x >= p.H) continue;
+    acc += p.img[(size_t)p.N * ((size_t)(g * p.Cg + c) * p.HH + y * p.H + x) + n] *
+           p.hid[(size_t)p.N * ((size_t)f * p.M + m) + n];
+  }
+  acc = wave_sum(acc);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = acc;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const float s = (red[0] + red[1]) + (red[2] + red[3]);
+    float* t = p.out + (size_t)p.F * q + f;
+    *t = (p.scale_t == 0.f ? 0.f : p.scale_t * *t) + p.scale_o * s;
+  }
+}
+
+// ------------------------------------------------------------------ matrix-core kernel
+
+#define CV_BK 16
+#define CV_PAD 4
+
+// Geometry of one Down phase (py, px): the pixels y = y_first + s*i, i < QY, whose
+// taps are ky = py + s*t, t < TY, reaching module my = qy_first + i - t.
+struct DownPhase {
+  int py, px, y_first, x_first, QY, QX, qy_first, qx_first, TY, TX;
+};
+__device__ __forceinline__ void down_axis(int ph, int s, int pad0, int H, int k, int* first, int* Q, int* qfirst,
+                                          int* T) {
+  // smallest y >= 0 with (y - pad0) % s == ph   (pad0 <= 0)
+  int y = ph + pad0;            // (y - pad0) == ph
+  if (y < 0) y += ((-y + s - 1) / s) * s;
+  *first = y;
+  *Q = y < H ? (H - 1 - y) / s + 1 : 0;
+  *qfirst = (y - pad0 - ph) / s;
+  *T = ph < k ? (k - ph + s - 1) / s : 0;
+}
+
+template <int MODE, int WAVES_M, int WM, int WN>
+__global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
+  constexpr int WAVES_N = 4 / WAVES_M;
+  constexpr int BM = 32 * WM * WAVES_M, BN = 32 * WN * WAVES_N;
+  constexpr int LA = BM + CV_PAD, LB = BN + CV_PAD;
+  constexpr int TA = BM * CV_BK / 4, TB = BN * CV_BK / 4;  // 16-byte groups per slab
+  constexpr int NA = (TA + 255) / 256, NB = (TB + 255) / 256;
+  __shared__ __attribute__((aligned(16))) float As[2][CV_BK][LA];
+  __shared__ __attribute__((aligned(16))) float Bs[2][CV_BK][LB];
+
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int wm = wv % WAVES_M, wn = wv / WAVES_M;
+  const int lk = lane >> 5, li = lane & 31;
+  const int N = p.N, H = p.H, HH = p.HH, Mx = p.Mx, M = p.M, F = p.F, Fg = p.Fg, Cg = p.Cg, k = p.k, s = p.s;
+
+  // ---- what this workgroup computes
+  int g, rows, cols, nslabs, slab_beg, slab_end, zsplit = 0;
+  DownPhase ph;
+  if (MODE == CONV_UP) {
+    g = blockIdx.z;
+    rows = M * N; cols = Fg;
+    nslabs = (Cg * p.kk2 + CV_BK - 1) / CV_BK;
+    slab_beg = 0; slab_end = nslabs;
+  } else if (MODE == CONV_DOWN) {
+    const int nph = s * s;
+    g = blockIdx.z / nph;
+    const int phase = blockIdx.z % nph;
+    ph.py = phase / s; ph.px = phase % s;
+    down_axis(ph.py, s, p.pad0, H, k, &ph.y_first, &ph.QY, &ph.qy_first, &ph.TY);
+    down_axis(ph.px, s, p.pad0, H, k, &ph.x_first, &ph.QX, &ph.qx_first, &ph.TX);
+    rows = ph.QY * ph.QX * N; cols = Cg;
+    nslabs = ph.TY * ph.TX * (Fg / CV_BK);
+    slab_beg = 0; slab_end = nslabs;
+  } else {
+    g = blockIdx.z / p.splits;
+    zsplit = blockIdx.z % p.splits;
+    rows = Fg; cols = Cg * p.kk2;
+    nslabs = p.m_count * (N / CV_BK);
+    slab_beg = zsplit * p.slabs_per_split;
+    slab_end = slab_beg + p.slabs_per_split < nslabs ? slab_beg + p.slabs_per_split : nslabs;
+  }
+  const int row0 = blockIdx.x * BM, col0 = blockIdx.y * BN;
+  if (row0 >= rows || col0 >= cols) return;  // uniform for the workgroup
+
+  // ---- loop-invariant part of each lane's gathers
+  // A groups: Up/Down are row-contiguous (4 rows of one kk); Outp is kk-contiguous (4 kk of one row).
+  int a_k[NA], a_r[NA], a_y[NA], a_x[NA];
+  long long a_off[NA];
+  bool a_ok[NA];
+#pragma unroll
+  for (int u = 0; u < NA; ++u) {
+    const int f = tid + u * 256;
+    a_ok[u] = f < TA;
+    if (MODE == CONV_OUTP) {
+      a_r[u] = f >> 2; a_k[u] = (f & 3) << 2;
+      const int r = row0 + a_r[u];
+      a_ok[u] = a_ok[u] && r < rows;
+      a_off[u] = (long long)N * M * (g * Fg + r) + (long long)N * p.m_begin;
+      a_y[u] = a_x[u] = 0;
+    } else {
+      a_k[u] = f / (BM / 4); a_r[u] = (f % (BM / 4)) << 2;
+      const int r = row0 + a_r[u];
+      a_ok[u] = a_ok[u] && r < rows;
+      const int pos = (int)fd_div((uint32_t)r, p.dN);  // module (Up) or pixel-of-phase (Down)
+      const int n = r - pos * N;
+      if (MODE == CONV_UP) {
+        const int my = (int)fd_div((uint32_t)pos, p.dMx), mx = pos - my * Mx;
+        a_y[u] = my * s + p.pad0; a_x[u] = mx * s + p.pad0;
+        a_off[u] = (long long)N * ((long long)g * Cg * HH) + n;
+      } else {
+        const int qyi = ph.QX > 0 ? pos / ph.QX : 0, qxi = pos - qyi * ph.QX;
+        a_y[u] = ph.qy_first + qyi; a_x[u] = ph.qx_first + qxi;  // module coordinate before the tap shift
+        a_off[u] = (long long)N * ((long long)g * Fg * M) + n;
+      }
+    }
+  }
+  // B groups: Up is column-contiguous (4 filters of one kk); Down/Outp are kk-contiguous.
+  int b_k[NB], b_c[NB], b_y[NB], b_x[NB];
+  long long b_off[NB];
+  bool b_ok[NB];
+#pragma unroll
+  for (int u = 0; u < NB; ++u) {
+    const int f = tid + u * 256;
+    b_ok[u] = f < TB;
+    if (MODE == CONV_UP) {
+      b_k[u] = f / (BN / 4); b_c[u] = (f % (BN / 4)) << 2;
+      const int c = col0 + b_c[u];
+      b_ok[u] = b_ok[u] && c < cols;
+      b_off[u] = (long long)g * Fg + c;
+      b_y[u] = b_x[u] = 0;
+    } else {
+      b_c[u] = f >> 2; b_k[u] = (f & 3) << 2;
+      const int c = col0 + b_c[u];
+      b_ok[u] = b_ok[u] && c < cols;
+      if (MODE == CONV_DOWN) {
+        b_off[u] = (long long)g * Fg + (long long)F * c * p.kk2;  // + F*(ky*k + kx) + f per slab
+        b_y[u] = b_x[u] = 0;
+      } else {
+        const int cc = (int)fd_div((uint32_t)c, p.dkk2);
+        const int pp = c - cc * p.kk2;
+        const int ky = (int)fd_div((uint32_t)pp, p.dk), kx = pp - ky * k;
+        b_y[u] = p.pad0 + ky; b_x[u] = p.pad0 + kx;
+        b_off[u] = (long long)N * ((long long)(g * Cg + cc) * HH);
+      }
+    }
+  }
+
+  // ---- slab state (uniform across the workgroup)
+  // Down: slab -> (t, u, f0); Outp: slab -> (my, mx, n0).
+  int st_a = 0, st_b = 0, st_c = 0;
+  if (MODE == CONV_DOWN) {
+    const int per_tap = Fg / CV_BK;
+    const int tap = slab_beg / per_tap;
+    st_c = (slab_beg - tap * per_tap) * CV_BK;            // f0
+    st_a = ph.TX > 0 ? tap / ph.TX : 0; st_b = tap - st_a * ph.TX;  // t, u
+  } else if (MODE == CONV_OUTP) {
+    const int per_mod = N / CV_BK;
+    const int m = p.m_begin + slab_beg / per_mod;
+    st_c = (slab_beg % per_mod) * CV_BK;                  // n0
+    st_a = m / Mx; st_b = m - st_a * Mx;                  // my, mx
+  }
+
+  float4 ra[NA], rb[NB];
+  const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
+
+  auto fetch = [&](int slab) {
+    const int kk0 = slab * CV_BK;
+#pragma unroll
+    for (int u = 0; u < NA; ++u) {
+      ra[u] = zero4;
+      if (!a_ok[u]) continue;
+      if (MODE == CONV_UP) {
+        const int kk = kk0 + a_k[u];
+        if (kk < Cg * p.kk2) {
+          const int c = (int)fd_div((uint32_t)kk, p.dkk2);
+          const int pp = kk - c * p.kk2;
+          const int ky = (int)fd_div((uint32_t)pp, p.dk), kx = pp - ky * k;
+          const int y = a_y[u] + ky, x = a_x[u] + kx;
+          if (y >= 0 && y < H && x >= 0 && x < H)
+            ra[u] = *reinterpret_cast<const float4*>(p.img + a_off[u] + (long long)N * (c * HH + y * H + x));
+        }
+      } else if (MODE == CONV_DOWN) {
+        const int my = a_y[u] - st_a, mx = a_x[u] - st_b;
+        if (my >= 0 && my < Mx && mx >= 0 && mx < Mx)
+          ra[u] = *reinterpret_cast<const float4*>(
+              p.hid + a_off[u] + (long long)N * ((long long)(st_c + a_k[u]) * M + my * Mx + mx));
+      } else {
+        ra[u] = *reinterpret_cast<const float4*>(p.hid + a_off[u] + (long long)(slab * CV_BK + a_k[u]));
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < NB; ++u) {
+      rb[u] = zero4;
+      if (!b_ok[u]) continue;
+      if (MODE == CONV_UP) {
+        const int kk = kk0 + b_k[u];
+        if (kk < Cg * p.kk2) rb[u] = *reinterpret_cast<const float4*>(p.flt + b_off[u] + (long long)F * kk);
+      } else if (MODE == CONV_DOWN) {
+        const int ky = ph.py + s * st_a, kx = ph.px + s * st_b;
+        rb[u] = *reinterpret_cast<const float4*>(p.flt + b_off[u] + (long long)F * (ky * k + kx) + st_c + b_k[u]);
+      } else {
+        const int y = st_a * s + b_y[u], x = st_b * s + b_x[u];
+        if (y >= 0 && y < H && x >= 0 && x < H)
+          rb[u] = *reinterpret_cast<const float4*>(p.img + b_off[u] + (long long)N * (y * H + x) + st_c + b_k[u]);
+      }
+    }
+    // advance the uniform slab state
+    if (MODE == CONV_DOWN) {
+      st_c += CV_BK;
+      if (st_c == Fg) { st_c = 0; if (++st_b == ph.TX) { st_b = 0; ++st_a; } }
+    } else if (MODE == CONV_OUTP) {
+      st_c += CV_BK;
+      if (st_c == N) { st_c = 0; if (++st_b == Mx) { st_b = 0; ++st_a; } }
+    }
+  };
+  auto stash = [&](int buf) {
+#pragma unroll
+    for (int u = 0; u < NA; ++u) {
+      if (tid + u * 256 >= TA) continue;
+      if (MODE == CONV_OUTP) {
+        As[buf][a_k[u]][a_r[u]] = ra[u].x; As[buf][a_k[u] + 1][a_r[u]] = ra[u].y;
+        As[buf][a_k[u] + 2][a_r[u]] = ra[u].z; As[buf][a_k[u] + 3][a_r[u]] = ra[u].w;
+      } else {
+        *reinterpret_cast<float4*>(&As[buf][a_k[u]][a_r[u]]) = ra[u];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < NB; ++u) {
+      if (tid + u * 256 >= TB) continue;
+      if (MODE == CONV_UP) {
+        *reinterpret_cast<float4*>(&Bs[buf][b_k[u]][b_c[u]]) = rb[u];
+      } else {
+        Bs[buf][b_k[u]][b_c[u]] = rb[u].x; Bs[buf][b_k[u] + 1][b_c[u]] = rb[u].y;
+        Bs[buf][b_k[u] + 2][b_c[u]] = rb[u].z; Bs[buf][b_k[u] + 3][b_c[u]] = rb[u].w;
+      }
+    }
+  };
+
+  f32x16 acc[WN][WM];
+#pragma unroll
+  for (int j = 0; j < WN; ++j)
+#pragma unroll
+    for (int i = 0; i < WM; ++i)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[j][i][v] = 0.f;
+
+  int buf = 0;
+  if (slab_beg < slab_end) {
+    fetch(slab_beg);
+    stash(0);
+  }
+  __syncthreads();
+  for (int slab = slab_beg; slab < slab_end; ++slab) {
+    const bool more = slab + 1 < slab_end;
+    if (more) fetch(slab + 1);
+#pragma unroll
+    for (int kk = 0; kk < CV_BK; kk += 2) {
+      float av[WM], bv[WN];
+#pragma unroll
+      for (int i = 0; i < WM; ++i) av[i] = As[buf][kk + lk][(wm * WM + i) * 32 + li];
+#pragma unroll
+      for (int j = 0; j < WN; ++j) bv[j] = Bs[buf][kk + lk][(wn * WN + j) * 32 + li];
+#pragma unroll
+      for (int j = 0; j < WN; ++j)
+#pragma unroll
+        for (int i = 0; i < WM; ++i)
+          acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[j], av[i], acc[j][i], 0, 0, 0);
+    }
+    if (more) stash(buf ^ 1);
+    __syncthreads();
+    buf ^= 1;
+  }
+
+  // ---- epilogue: acc[j][i][v] is C(row, col) with row = ... + li, col = ... + 8*(v/4) + 4*lk + v%4
+#pragma unroll
+  for (int i = 0; i < WM; ++i) {
+    const int r = row0 + (wm * WM + i) * 32 + li;
+    if (r >= rows) continue;
+    long long rbase;
+    long long cstride;
+    if (MODE == CONV_UP) {
+      rbase = (long long)g * Fg * M * N + r;            // + c * M*N
+      cstride = (long long)M * N;
+    } else if (MODE == CONV_DOWN) {
+      const int pos = (int)fd_div((uint32_t)r, p.dN);
+      const int n = r - pos * N;
+      const int qyi = pos / ph.QX, qxi = pos - qyi * ph.QX;
+      const int y = ph.y_first + s * qyi, x = ph.x_first + s * qxi;
+      rbase = (long long)N * ((long long)g * Cg * HH + y * H + x) + n;  // + c * N*HH
+      cstride = (long long)N * HH;
+    } else {
+      rbase = (long long)zsplit * ((long long)p.G * Fg * Cg * p.kk2) + ((long long)g * Cg * p.kk2) * Fg + r;
+      cstride = Fg;                                     // partial[zsplit][g][q][f]
+    }
+#pragma unroll
+    for (int j = 0; j < WN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int c = col0 + (wn * WN + j) * 32 + 8 * (v >> 2) + 4 * lk + (v & 3);
+        if (c >= cols) continue;
+        if (MODE == CONV_OUTP) {
+          p.partial[rbase + cstride * c] = acc[j][i][v];
+        } else {
+          float* t = p.out + rbase + cstride * c;
+          *t = (p.scale_t == 0.f ? 0.f : p.scale_t * *t) + p.scale_o * acc[j][i][v];
+        }
+      }
+  }
+}
+
+// dW(f, q) = scale_t*dW + scale_o * sum over splits of partial[z][g][q][fl]
+__global__ void k_conv_outp_finish(ConvArgs p) {
+  const int per_group = p.Fg * p.Cg * p.kk2;
+  const int total = p.G * per_group;
+  for (int e = blockIdx.x * blockDim.x + threadIdx.x; e < total; e += gridDim.x * blockDim.x) {
+    float sum = 0.f;
+    for (int z = 0; z < p.splits; ++z) sum += p.partial[(size_t)z * total + e];
+    const int g = e / per_group, rem = e - g * per_group;
+    const int q = rem / p.Fg, fl = rem - q * p.Fg;
+    float* t = p.out + (size_t)p.F * q + g * p.Fg + fl;
+    *t = (p.scale_t == 0.f ? 0.f : p.scale_t * *t) + p.scale_o * sum;
+  }
+}
+
+// ------------------------------------------------------------------ host side
+
+static char g_conv_err[256];
+static bool g_conv_failed = false;
+
+void conv_set_error(const char* where, const char* what) {
+  snprintf(g_conv_err, sizeof(g_conv_err), "%s: %s", where, what);
+  g_conv_failed = true;
+}
+void conv_clear_error() { g_conv_failed = false; }
+
+#define CONV_REQUIRE(cond, where)        \
+  do {                                   \
+    if (!(cond)) {                       \
+      conv_set_error(where, #cond);      \
+      return;                            \
+    }                                    \
+  } while (0)
+
+static int isqrt_exact(int v) {
+  if (v < 0) return -1;
+  int r = (int)(sqrt((double)v) + 0.5);
+  return r * r == v ? r : -1;
+}
+
+static bool fast_ok(const ConvArgs& a) {
+  return a.N % 16 == 0 && a.Fg % 16 == 0 && dn_aligned16(a.img) && dn_aligned16(a.flt) && dn_aligned16(a.hid) &&
+         (long long)a.N * a.M * a.F < (1ll << 31) && (long long)a.N * a.HH * a.C < (1ll << 31);
+}
+
+static void fill_common(ConvArgs& a, int N, int C, int G, int H, int F, int k, int Mx, int s, int pad0) {
+  a.N = N; a.C = C; a.G = G; a.Cg = C / G; a.H = H; a.F = F; a.Fg = F / G; a.k = k; a.Mx = Mx; a.s = s; a.pad0 = pad0;
+  a.M = Mx * Mx; a.HH = H * H; a.kk2 = k * k;
+  a.m_begin = 0; a.m_count = a.M; a.splits = 1; a.slabs_per_split = 0;
+  a.scale_t = 0.f; a.scale_o = 1.f; a.partial = nullptr;
+  a.dN = make_fastdiv((uint32_t)N); a.dMx = make_fastdiv((uint32_t)Mx);
+  a.dk = make_fastdiv((uint32_t)k); a.dkk2 = make_fastdiv((uint32_t)(k * k));
+}
+
+template <int MODE>
+static void launch_rowmajor(const ConvArgs& a, long long rows, int cols, int gz) {
+  // Up / Down: rows are plentiful, columns few: 4 wavefronts down the rows, WN blocks across.
+  const unsigned gx = (unsigned)((rows + 127) / 128);
+  if (cols <= 32) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 1>), dim3(gx, (cols + 31) / 32, gz), dim3(256), 0, 0, a);
+  else if (cols <= 64) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 2>), dim3(gx, (cols + 63) / 64, gz), dim3(256), 0, 0, a);
+  else if (cols <= 96) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 3>), dim3(gx, (cols + 95) / 96, gz), dim3(256), 0, 0, a);
+  else hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 4>), dim3(gx, (cols + 127) / 128, gz), dim3(256), 0, 0, a);
+}
+
+static void conv_up_impl(cudamat* images, cudamat* filters, cudamat* targets, int numModulesX, int paddingStart,
+                         int moduleStride, int numImgColors, int numGroups, const char* where) {
+  conv_clear_error();
+  CONV_REQUIRE(images->on_device && filters->on_device && targets->on_device, where);
+  CONV_REQUIRE(numGroups >= 1 && numImgColors > 0 && numImgColors % numGroups == 0, where);
+  CONV_REQUIRE(moduleStride >= 1 && numModulesX >= 1, where);
+  const int N = images->size[0], F = filters->size[0];
+  CONV_REQUIRE(N > 0 && F > 0 && F % numGroups == 0, where);
+  CONV_REQUIRE(images->size[1] % numImgColors == 0, where);
+  const int H = isqrt_exact(images->size[1] / numImgColors);
+  CONV_REQUIRE(H > 0, where);
+  const int Cg = numImgColors / numGroups;
+  CONV_REQUIRE(filters->size[1] % Cg == 0, where);
+  const int k = isqrt_exact(filters->size[1] / Cg);
+  CONV_REQUIRE(k > 0, where);
+  const int M = numModulesX * numModulesX;
+  CONV_REQUIRE(paddingStart <= 0, where);
+  CONV_REQUIRE(moduleStride <= k, where);
+  CONV_REQUIRE(targets->size[0] == N && targets->size[1] == F * M, where);
+  ConvArgs a;
+  fill_common(a, N, numImgColors, numGroups, H, F, k, numModulesX, moduleStride, paddingStart);
+  a.img = images->data_device; a.flt = filters->data_device; a.hid = nullptr; a.out = targets->data_device;
+  if (fast_ok(a)) {
+    launch_rowmajor<CONV_UP>(a, (long long)M * N, a.Fg, numGroups);
+  } else {
+    const long long total = (long long)N * M * F;
+    long long blocks = (total + 255) / 256;
+    if (blocks > dn_num_cus() * 16ll) blocks = dn_num_cus() * 16ll;
+    hipLaunchKernelGGL(k_conv_up_direct, dim3((unsigned)blocks), dim3(256), 0, 0, a);
+  }
+  if (dn_launch_status()) conv_set_error(where, hipGetErrorString(hipGetLastError()));
+}
+
+static void conv_down_impl(cudamat* hidActs, cudamat* filters, cudamat* targets, int imgSize, int paddingStart,
+                           int moduleStride, int numImgColors, int numGroups, const char* where) {
+  conv_clear_error();
+  CONV_REQUIRE(hidActs->on_device && filters->on_device && targets->on_device, where);
+  CONV_REQUIRE(numGroups >= 1 && numImgColors > 0 && numImgColors % numGroups == 0, where);
+  CONV_REQUIRE(moduleStride >= 1 && imgSize >= 1, where);
+  const int N = hidActs->size[0], F = filters->size[0];
+  CONV_REQUIRE(N > 0 && F > 0 && F % numGroups == 0, where);
+  CONV_REQUIRE(hidActs->size[1] % F == 0, where);
+  const int M = hidActs->size[1] / F;
+  const int Mx = isqrt_exact(M);
+  CONV_REQUIRE(Mx > 0, where);
+  const int Cg = numImgColors / numGroups;
+  CONV_REQUIRE(filters->size[1] % Cg == 0, where);
+  const int k = isqrt_exact(filters->size[1] / Cg);
+  CONV_REQUIRE(k > 0, where);
+  CONV_REQUIRE(paddingStart <= 0 && moduleStride <= k, where);
+  CONV_REQUIRE(targets->size[0] == N && targets->size[1] == numImgColors * imgSize * imgSize, where);
+  ConvArgs a;
+  fill_common(a, N, numImgColors, numGroups, imgSize, F, k, Mx, moduleStride, paddingStart);
+  a.img = nullptr; a.flt = filters->data_device; a.hid = hidActs->data_device; a.out = targets->data_device;
+  a.img = a.hid;  // alignment test only
+  if (fast_ok(a) && dn_aligned16(a.out)) {
+    const int q = (imgSize + moduleStride - 1) / moduleStride;
+    launch_rowmajor<CONV_DOWN>(a, (long long)q * q * N, a.Cg, numGroups * moduleStride * moduleStride);
+  } else {
+    const long long total = (long long)N * a.HH * numImgColors;
+    long long blocks = (total + 255) / 256;
+    if (blocks > dn_num_cus() * 16ll) blocks = dn_num_cus() * 16ll;
+    hipLaunchKernelGGL(k_conv_down_direct, dim3((unsigned)blocks), dim3(256), 0, 0, a);
+  }
+  if (dn_launch_status()) conv_set_error(where, hipGetErrorString(hipGetLastError()));
+}
+
+static void conv_outp_impl(cudamat* images, cudamat* hidActs, cudamat* targets, int numModulesX, int filterSize,
+                           int paddingStart, int moduleStride, int numImgColors, int numGroups, int partialSum,
+                           const char* where) {
+  conv_clear_error();
+  CONV_REQUIRE(images->on_device && hidActs->on_device && targets->on_device, where);
+  CONV_REQUIRE(numGroups >= 1 && numImgColors > 0 && numImgColors % numGroups == 0, where);
+  CONV_REQUIRE(moduleStride >= 1 && numModulesX >= 1 && filterSize >= 1, where);
+  const int N = images->size[0];
+  CONV_REQUIRE(N > 0 && hidActs->size[0] == N, where);
+  CONV_REQUIRE(images->size[1] % numImgColors == 0, where);
+  const int H = isqrt_exact(images->size[1] / numImgColors);
+  CONV_REQUIRE(H > 0, where);
+  const int M = numModulesX * numModulesX;
+  CONV_REQUIRE(hidActs->size[1] % M == 0, where);
+  const int F = hidActs->size[1] / M;
+  CONV_REQUIRE(F > 0 && F % numGroups == 0, where);
+  if (partialSum == 0) partialSum = M;
+  CONV_REQUIRE(partialSum > 0 && M % partialSum == 0, where);
+  CONV_REQUIRE(paddingStart <= 0 && moduleStride <= filterSize, where);
+  const int Cg = numImgColors / numGroups;
+  const int chunks = M / partialSum;
+  CONV_REQUIRE(targets->size[0] == F && targets->size[1] == chunks * Cg * filterSize * filterSize, where);
+  ConvArgs a;
+  fill_common(a, N, numImgColors, numGroups, H, F, filterSize, numModulesX, moduleStride, paddingStart);
+  a.img = images->data_device; a.hid = hidActs->data_device; a.flt = a.img;
+  const int cols = Cg * a.kk2;
+  const bool fast = fast_ok(a);
+  for (int ch = 0; ch < chunks; ++ch) {
+    a.m_begin = ch * partialSum; a.m_count = partialSum;
+    a.out = targets->data_device + (size_t)ch * cols * F;
+    if (fast) {
+      // rows = filters of a group: pick the tile height that wastes least.
+      const int Fg = a.Fg;
+      const int BMs = Fg <= 32 ? 32 : Fg <= 64 ? 64 : Fg <= 96 ? 96 : 128;
+      const int gx = (Fg + BMs - 1) / BMs, gy = (cols + 127) / 128;
+      const int nslabs = a.m_count * (N / CV_BK);
+      long long want = (4ll * dn_num_cus()) / ((long long)gx * gy * numGroups);
+      if (want < 1) want = 1;
+      if (want > nslabs / 8) want = nslabs / 8 > 0 ? nslabs / 8 : 1;
+      if (want > 1024) want = 1024;
+      a.slabs_per_split = (int)((nslabs + want - 1) / want);
+      a.splits = (nslabs + a.slabs_per_split - 1) / a.slabs_per_split;
+      a.partial = (float*)dn_scratch((size_t)a.splits * F * cols * sizeof(float));
+      if (!a.partial) { conv_set_error(where, "out of device memory for the split-K workspace"); return; }
+      dim3 grid(gx, gy, numGroups * a.splits);
+      if (BMs == 32) hipLaunchKernelGGL((k_conv_mfma<CONV_OUTP, 1, 1, 1>), grid, dim3(256), 0, 0, a);
+      else if (BMs == 64) hipLaunchKernelGGL((k_conv_mfma<CONV_OUTP, 1, 2, 1>), grid, dim3(256), 0, 0, a);
+      else if (BMs == 96) hipLaunchKernelGGL((k_conv_mfma<CONV_OUTP, 1, 3, 1>), grid, dim3(256), 0, 0, a);
+      else hipLaunchKernelGGL((k_conv_mfma<CONV_OUTP, 2, 2, 2>), grid, dim3(256), 0, 0, a);
+      const int total = F * cols;
+      hipLaunchKernelGGL(k_conv_outp_finish, dim3((total + 255) / 256), dim3(256), 0, 0, a);
+    } else {
+      hipLaunchKernelGGL(k_conv_outp_direct, dim3((unsigned)(F * cols)), dim3(256), 0, 0, a);
+    }
+  }
+  if (dn_launch_status()) conv_set_error(where, hipGetErrorString(hipGetLastError()));
+}
+
+extern "C" {
+
+const char* conv_last_error(void) { return g_conv_failed ? g_conv_err : nullptr; }
+
+void convUp(cudamat* images, cudamat* filters, cudamat* targets, int numModulesX, int paddingStart, int moduleStride,
+            int numImgColors, int numGroups) {
+  conv_up_impl(images, filters, targets, numModulesX, paddingStart, moduleStride, numImgColors, numGroups, "convUp");
+}
+
+void convDown(cudamat* hidActs, cudamat* filters, cudamat* targets, int imgSize, int paddingStart, int moduleStride,
+              int numImgColors, int numGroups) {
+  conv_down_impl(hidActs, filters, targets, imgSize, paddingStart, moduleStride, numImgColors, numGroups, "convDown");
+}
+
+void convOutp(cudamat* images, cudamat* hidActs, cudamat* targets, int numModulesX, int filterSize, int paddingStart,
+              int moduleStride, int numImgColors, int numGroups, int partialSum) {
+  conv_outp_impl(images, hidActs, targets, numModulesX, filterSize, paddingStart, moduleStride, numImgColors,
+                 numGroups, partialSum, "convOutp");
+}
+
+// Locally connected layers (one filter bank per module) are not built yet.
+void localUp(cudamat*, cudamat*, cudamat*, int, int, int, int, int) {
+  conv_set_error("localUp", "locally connected layers are not implemented");
+}
+void localDown(cudamat*, cudamat*, cudamat*, int, int, int, int, int) {
+  conv_set_error("localDown", "locally connected layers are not implemented");
+}
+void localOutp(cudamat*, cudamat*, cudamat*, int, int, int, int, int, int, int) {
+  conv_set_error("localOutp", "locally connected layers are not implemented");
+}
+
+}  // extern "C"

@@ -19,6 +19,29 @@ int dn_num_cus() {
   return g_num_cus;
 }
 
+// ------------------------------------------------------------------ scratch
+// Grow-only device workspace for two-stage reductions (partials + result).
+static void* g_scratch = nullptr;
+static size_t g_scratch_bytes = 0;
+
+void* dn_scratch(size_t bytes) {
+  if (bytes > g_scratch_bytes) {
+    if (g_scratch) {
+      hipDeviceSynchronize();
+      hipFree(g_scratch);
+    }
+    size_t want = bytes < (1u << 20) ? (1u << 20) : bytes;
+    if (hipMalloc(&g_scratch, want) != hipSuccess) {
+      g_scratch = nullptr;
+      g_scratch_bytes = 0;
+      hipGetLastError();
+      return nullptr;
+    }
+    g_scratch_bytes = want;
+  }
+  return g_scratch;
+}
+
 // ------------------------------------------------------------------ kernels
 
 // Column-major row-band copy: dst(r, c) = src(r + row0, c) for a band of `rows`

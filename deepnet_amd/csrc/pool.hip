@@ -1,0 +1,392 @@
+// Local max pooling, its gradient, and within-channel response / contrast
+// normalisation with their gradient, in the (channels, rows, cols, batch) layout.
+// Replaces cudamat/cudamat_conv.cu:1021-1387, cudamat_conv_kernels.cuh:1238-2023
+// and cudamat_conv_kernels.cu:30-441.
+//
+// These are HBM-bound.  The batch index is the fastest one, so a lane owns VW
+// neighbouring images (one 16-byte access when VW == 4) of one (channel, output)
+// and walks the window; every lane of a wavefront walks the same window, and the
+// overlap between neighbouring windows is served from cache.
+#include "common.h"
+#include "wide_math.h"
+#include "../../include/cudamat_conv_amd.h"
+#include <math.h>
+
+void conv_set_error(const char* where, const char* what);
+void conv_clear_error();
+
+#define POOL_REQUIRE(cond, where)        \
+  do {                                   \
+    if (!(cond)) {                       \
+      conv_set_error(where, #cond);      \
+      return;                            \
+    }                                    \
+  } while (0)
+
+template <int VW> struct Vec;
+template <> struct Vec<1> {
+  float v[1];
+  __device__ __forceinline__ static Vec load(const float* p) { Vec r; r.v[0] = *p; return r; }
+  __device__ __forceinline__ void store(float* p) const { *p = v[0]; }
+};
+template <> struct Vec<4> {
+  float v[4];
+  __device__ __forceinline__ static Vec load(const float* p) {
+    const float4 t = *reinterpret_cast<const float4*>(p);
+    Vec r; r.v[0] = t.x; r.v[1] = t.y; r.v[2] = t.z; r.v[3] = t.w; return r;
+  }
+  __device__ __forceinline__ void store(float* p) const { *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]); }
+};
+
+struct PoolGeom {
+  int N, NV;        // images, images / VW
+  int F, S, O;      // channels, input size, output size (per side)
+  int subs, start, stride;
+  FastDiv dNV, dO, dS;
+};
+
+// e -> (image group, x, y, channel) for a (NV, X, X, F) index space
+__device__ __forceinline__ void decode4(uint32_t e, const FastDiv& dNV, const FastDiv& dX, int X, int* nv, int* x, int* y,
+                                        int* f) {
+  uint32_t q = fd_div(e, dNV);
+  *nv = (int)(e - q * dNV.d);
+  uint32_t q2 = fd_div(q, dX);
+  *x = (int)(q - q2 * (uint32_t)X);
+  uint32_t q3 = fd_div(q2, dX);
+  *y = (int)(q2 - q3 * (uint32_t)X);
+  *f = (int)q3;
+}
+
+// mode 0: max over the clipped window (start value -2e38, cudamat_conv_kernels.cuh:31-42).
+// mode 1: the reference's "probabilistic max" scan (:44-55, :1550-1623): the candidate
+//         replaces the running value unless running*r_running > candidate*r_candidate.
+template <int VW, int MODE>
+__global__ void __launch_bounds__(256) k_pool(const float* imgs, const float* rnd, float* target, PoolGeom g) {
+  const uint32_t total = (uint32_t)g.NV * g.O * g.O * g.F;
+  for (uint32_t e = blockIdx.x * 256u + threadIdx.x; e < total; e += gridDim.x * 256u) {
+    int nv, ox, oy, f;
+    decode4(e, g.dNV, g.dO, g.O, &nv, &ox, &oy, &f);
+    const int sx = g.start + ox * g.stride, sy = g.start + oy * g.stride;
+    const int x0 = sx > 0 ? sx : 0, y0 = sy > 0 ? sy : 0;
+    const int x1 = sx + g.subs < g.S ? sx + g.subs : g.S, y1 = sy + g.subs < g.S ? sy + g.subs : g.S;
+    const float* base = imgs + (size_t)g.N * ((size_t)f * g.S * g.S) + nv * VW;
+    const float* rbase = MODE == 1 ? rnd + (size_t)g.N * ((size_t)f * g.S * g.S) + nv * VW : nullptr;
+    Vec<VW> acc, racc;
+#pragma unroll
+    for (int i = 0; i < VW; ++i) { acc.v[i] = -2e38f; racc.v[i] = -2e38f; }
+    for (int y = y0; y < y1; ++y)
+      for (int x = x0; x < x1; ++x) {
+        const size_t off = (size_t)g.N * (y * g.S + x);
+        const Vec<VW> v = Vec<VW>::load(base + off);
+        if (MODE == 0) {
+#pragma unroll
+          for (int i = 0; i < VW; ++i) acc.v[i] = acc.v[i] > v.v[i] ? acc.v[i] : v.v[i];
+        } else {
+          const Vec<VW> r = Vec<VW>::load(rbase + off);
+#pragma unroll
+          for (int i = 0; i < VW; ++i) {
+            const bool keep = acc.v[i] * racc.v[i] > v.v[i] * r.v[i];
+            acc.v[i] = keep ? acc.v[i] : v.v[i];
+            racc.v[i] = keep ? racc.v[i] : r.v[i];
+          }
+        }
+      }
+    acc.store(target + (size_t)g.N * ((size_t)(f * g.O + oy) * g.O + ox) + nv * VW);
+  }
+}
+
+// Gradient of max pooling (cudamat_conv_kernels.cuh:1439-1530): each pixel collects
+// maxGrad from every output whose window holds it and whose max equals the pixel.
+template <int VW>
+__global__ void __launch_bounds__(256)
+k_pool_undo(const float* imgs, const float* maxGrads, const float* maxActs, float* target, PoolGeom g) {
+  const uint32_t total = (uint32_t)g.NV * g.S * g.S * g.F;
+  for (uint32_t e = blockIdx.x * 256u + threadIdx.x; e < total; e += gridDim.x * 256u) {
+    int nv, px, py, f;
+    decode4(e, g.dNV, g.dS, g.S, &nv, &px, &py, &f);
+    Vec<VW> acc;
+#pragma unroll
+    for (int i = 0; i < VW; ++i) acc.v[i] = 0.f;
+    const size_t poff = (size_t)g.N * ((size_t)(f * g.S + py) * g.S + px) + nv * VW;
+    const int span = g.start + g.stride * (g.O - 1) + g.subs;
+    if (px >= g.start && px < span && py >= g.start && py < span) {
+      const int oy0 = py - g.start < g.subs ? 0 : 1 + (py - g.start - g.subs) / g.stride;
+      const int oy1 = 1 + (py - g.start) / g.stride < g.O ? 1 + (py - g.start) / g.stride : g.O;
+      const int ox0 = px - g.start < g.subs ? 0 : 1 + (px - g.start - g.subs) / g.stride;
+      const int ox1 = 1 + (px - g.start) / g.stride < g.O ? 1 + (px - g.start) / g.stride : g.O;
+      const Vec<VW> img = Vec<VW>::load(imgs + poff);
+      for (int oy = oy0; oy < oy1; ++oy)
+        for (int ox = ox0; ox < ox1; ++ox) {
+          const size_t ooff = (size_t)g.N * ((size_t)(f * g.O + oy) * g.O + ox) + nv * VW;
+          const Vec<VW> ma = Vec<VW>::load(maxActs + ooff);
+          const Vec<VW> mg = Vec<VW>::load(maxGrads + ooff);
+#pragma unroll
+          for (int i = 0; i < VW; ++i) acc.v[i] += (img.v[i] == ma.v[i] ? 1.f : 0.f) * mg.v[i];
+        }
+    }
+    acc.store(target + poff);
+  }
+}
+
+// denoms = 1 + addScale * sum over the clipped sizeX x sizeX window (origin -sizeX/2)
+// of meanDiffs^2;  target = imgs * denoms^-powScale   (cudamat_conv_kernels.cu:112-176).
+template <int VW>
+__global__ void __launch_bounds__(256)
+k_cnorm(const float* imgs, const float* meanDiffs, float* denoms, float* target, PoolGeom g, int sizeX, float addScale,
+        float powScale) {
+  const uint32_t total = (uint32_t)g.NV * g.S * g.S * g.F;
+  for (uint32_t e = blockIdx.x * 256u + threadIdx.x; e < total; e += gridDim.x * 256u) {
+    int nv, px, py, f;
+    decode4(e, g.dNV, g.dS, g.S, &nv, &px, &py, &f);
+    const int sx = px - sizeX / 2, sy = py - sizeX / 2;
+    const int x0 = sx > 0 ? sx : 0, y0 = sy > 0 ? sy : 0;
+    const int x1 = sx + sizeX < g.S ? sx + sizeX : g.S, y1 = sy + sizeX < g.S ? sy + sizeX : g.S;
+    const float* base = meanDiffs + (size_t)g.N * ((size_t)f * g.S * g.S) + nv * VW;
+    Vec<VW> acc;
+#pragma unroll
+    for (int i = 0; i < VW; ++i) acc.v[i] = 0.f;
+    for (int y = y0; y < y1; ++y)
+      for (int x = x0; x < x1; ++x) {
+        const Vec<VW> v = Vec<VW>::load(base + (size_t)g.N * (y * g.S + x));
+#pragma unroll
+        for (int i = 0; i < VW; ++i) acc.v[i] += v.v[i] * v.v[i];
+      }
+    const size_t poff = (size_t)g.N * ((size_t)(f * g.S + py) * g.S + px) + nv * VW;
+    const Vec<VW> in = Vec<VW>::load(imgs + poff);
+    Vec<VW> d, t;
+#pragma unroll
+    for (int i = 0; i < VW; ++i) {
+      d.v[i] = 1.f + addScale * acc.v[i];
+      t.v[i] = in.v[i] * dn_pow(d.v[i], -powScale);
+    }
+    d.store(denoms + poff);
+    t.store(target + poff);
+  }
+}
+
+// acts := scale * outGrads * acts / denoms   (cudamat_conv_kernels.cuh:2010-2023)
+__global__ void __launch_bounds__(256)
+k_rnorm_undo_prelim(float* acts, const float* denoms, const float* outGrads, size_t n, float scale) {
+  const size_t stride = (size_t)gridDim.x * 256;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride)
+    acts[i] = (scale * outGrads[i] * acts[i]) / denoms[i];
+}
+
+// target = inputs * (sum of the prepared acts over the mirrored window) + outGrads * denoms^-powScale
+// (cudamat_conv_kernels.cuh:1920-2004); the window of pixel p is [p + sizeX/2 - sizeX + 1, p + sizeX/2].
+template <int VW>
+__global__ void __launch_bounds__(256)
+k_rnorm_undo(const float* outGrads, const float* denoms, const float* inputs, const float* acts, float* target,
+             PoolGeom g, int sizeX, float powScale) {
+  const uint32_t total = (uint32_t)g.NV * g.S * g.S * g.F;
+  for (uint32_t e = blockIdx.x * 256u + threadIdx.x; e < total; e += gridDim.x * 256u) {
+    int nv, px, py, f;
+    decode4(e, g.dNV, g.dS, g.S, &nv, &px, &py, &f);
+    const int sy = py + sizeX / 2 - sizeX + 1, sx = px + sizeX / 2 - sizeX + 1;
+    const int y0 = sy > 0 ? sy : 0, x0 = sx > 0 ? sx : 0;
+    const int y1 = py + sizeX / 2 + 1 < g.S ? py + sizeX / 2 + 1 : g.S;
+    const int x1 = px + sizeX / 2 + 1 < g.S ? px + sizeX / 2 + 1 : g.S;
+    const float* base = acts + (size_t)g.N * ((size_t)f * g.S * g.S) + nv * VW;
+    Vec<VW> acc;
+#pragma unroll
+    for (int i = 0; i < VW; ++i) acc.v[i] = 0.f;
+    for (int y = y0; y < y1; ++y)
+      for (int x = x0; x < x1; ++x) {
+        const Vec<VW> v = Vec<VW>::load(base + (size_t)g.N * (y * g.S + x));
+#pragma unroll
+        for (int i = 0; i < VW; ++i) acc.v[i] += v.v[i];
+      }
+    const size_t poff = (size_t)g.N * ((size_t)(f * g.S + py) * g.S + px) + nv * VW;
+    const Vec<VW> inp = Vec<VW>::load(inputs + poff), og = Vec<VW>::load(outGrads + poff),
+                  den = Vec<VW>::load(denoms + poff);
+    Vec<VW> t;
+#pragma unroll
+    for (int i = 0; i < VW; ++i) t.v[i] = inp.v[i] * acc.v[i] + og.v[i] * dn_pow(den.v[i], -powScale);
+    t.store(target + poff);
+  }
+}
+
+// ------------------------------------------------------------------ host side
+
+static int isqrt_exact_p(int v) {
+  if (v < 0) return -1;
+  int r = (int)(sqrt((double)v) + 0.5);
+  return r * r == v ? r : -1;
+}
+
+static bool make_geom(PoolGeom& g, int N, int F, int S, int O, int subs, int start, int stride, int vw) {
+  g.N = N; g.NV = N / vw; g.F = F; g.S = S; g.O = O; g.subs = subs; g.start = start; g.stride = stride;
+  g.dNV = make_fastdiv((uint32_t)g.NV); g.dO = make_fastdiv((uint32_t)(O > 0 ? O : 1));
+  g.dS = make_fastdiv((uint32_t)S);
+  return true;
+}
+
+static unsigned grid_for(long long total) {
+  long long b = (total + 255) / 256;
+  const long long cap = (long long)dn_num_cus() * 32;
+  if (b > cap) b = cap;
+  return (unsigned)(b > 0 ? b : 1);
+}
+
+static bool all_aligned16(std::initializer_list<const void*> ps) {
+  for (const void* p : ps)
+    if (!dn_aligned16(p)) return false;
+  return true;
+}
+
+static void pool_impl(cudamat* images, cudamat* rnd, cudamat* targets, int numFilters, int subsX, int startX,
+                      int strideX, int outputsX, const char* where) {
+  conv_clear_error();
+  POOL_REQUIRE(images->on_device && targets->on_device && (!rnd || rnd->on_device), where);
+  POOL_REQUIRE(numFilters > 0 && subsX > 0 && strideX > 0 && outputsX > 0, where);
+  const int N = images->size[0];
+  POOL_REQUIRE(N > 0 && images->size[1] % numFilters == 0, where);
+  const int S = isqrt_exact_p(images->size[1] / numFilters);
+  POOL_REQUIRE(S > 0, where);
+  POOL_REQUIRE(targets->size[0] == N && targets->size[1] == numFilters * outputsX * outputsX, where);
+  POOL_REQUIRE(!rnd || (rnd->size[0] == N && rnd->size[1] == images->size[1]), where);
+  const long long outs = (long long)N * outputsX * outputsX * numFilters;
+  POOL_REQUIRE(outs < (1ll << 32) && (long long)N * images->size[1] < (1ll << 32), where);
+  const bool v4 = N % 4 == 0 && all_aligned16({images->data_device, targets->data_device, rnd ? rnd->data_device : nullptr});
+  PoolGeom g;
+  make_geom(g, N, numFilters, S, outputsX, subsX, startX, strideX, v4 ? 4 : 1);
+  const unsigned grid = grid_for(outs / (v4 ? 4 : 1));
+  const float* r = rnd ? rnd->data_device : nullptr;
+  if (!rnd) {
+    if (v4) hipLaunchKernelGGL((k_pool<4, 0>), dim3(grid), dim3(256), 0, 0, images->data_device, r, targets->data_device, g);
+    else hipLaunchKernelGGL((k_pool<1, 0>), dim3(grid), dim3(256), 0, 0, images->data_device, r, targets->data_device, g);
+  } else {
+    if (v4) hipLaunchKernelGGL((k_pool<4, 1>), dim3(grid), dim3(256), 0, 0, images->data_device, r, targets->data_device, g);
+    else hipLaunchKernelGGL((k_pool<1, 1>), dim3(grid), dim3(256), 0, 0, images->data_device, r, targets->data_device, g);
+  }
+  if (dn_launch_status()) conv_set_error(where, hipGetErrorString(hipGetLastError()));
+}
+
+static void cnorm_impl(cudamat* images, cudamat* meanDiffs, cudamat* denoms, cudamat* targets, int numFilters,
+                       int sizeX, float addScale, float powScale, const char* where) {
+  conv_clear_error();
+  POOL_REQUIRE(images->on_device && meanDiffs->on_device && denoms->on_device && targets->on_device, where);
+  POOL_REQUIRE(numFilters > 0 && sizeX > 0, where);
+  const int N = images->size[0];
+  POOL_REQUIRE(N > 0 && images->size[1] % numFilters == 0, where);
+  const int S = isqrt_exact_p(images->size[1] / numFilters);
+  POOL_REQUIRE(S > 0, where);
+  for (cudamat* m : {meanDiffs, denoms, targets})
+    POOL_REQUIRE(m->size[0] == N && m->size[1] == images->size[1], where);
+  const long long total = (long long)N * images->size[1];
+  POOL_REQUIRE(total < (1ll << 32), where);
+  const bool v4 = N % 4 == 0 && all_aligned16({images->data_device, meanDiffs->data_device, denoms->data_device,
+                                               targets->data_device});
+  PoolGeom g;
+  make_geom(g, N, numFilters, S, S, 0, 0, 1, v4 ? 4 : 1);
+  const unsigned grid = grid_for(total / (v4 ? 4 : 1));
+  if (v4)
+    hipLaunchKernelGGL((k_cnorm<4>), dim3(grid), dim3(256), 0, 0, (const float*)images->data_device,
+                       (const float*)meanDiffs->data_device, denoms->data_device, targets->data_device, g, sizeX,
+                       addScale, powScale);
+  else
+    hipLaunchKernelGGL((k_cnorm<1>), dim3(grid), dim3(256), 0, 0, (const float*)images->data_device,
+                       (const float*)meanDiffs->data_device, denoms->data_device, targets->data_device, g, sizeX,
+                       addScale, powScale);
+  if (dn_launch_status()) conv_set_error(where, hipGetErrorString(hipGetLastError()));
+}
+
+static void rnorm_undo_impl(cudamat* outGrads, cudamat* denoms, cudamat* inputs, cudamat* acts, cudamat* targets,
+                            int numFilters, int sizeX, float addScale, float powScale, const char* where) {
+  conv_clear_error();
+  POOL_REQUIRE(outGrads->on_device && denoms->on_device && inputs->on_device && acts->on_device && targets->on_device,
+               where);
+  POOL_REQUIRE(numFilters > 0 && sizeX > 0, where);
+  const int N = outGrads->size[0];
+  POOL_REQUIRE(N > 0 && outGrads->size[1] % numFilters == 0, where);
+  const int S = isqrt_exact_p(outGrads->size[1] / numFilters);
+  POOL_REQUIRE(S > 0, where);
+  for (cudamat* m : {denoms, inputs, acts, targets})
+    POOL_REQUIRE(m->size[0] == N && m->size[1] == outGrads->size[1], where);
+  const long long total = (long long)N * outGrads->size[1];
+  POOL_REQUIRE(total < (1ll << 32), where);
+  hipLaunchKernelGGL(k_rnorm_undo_prelim, dim3(grid_for(total)), dim3(256), 0, 0, acts->data_device,
+                     (const float*)denoms->data_device, (const float*)outGrads->data_device, (size_t)total,
+                     -2.f * addScale * powScale);
+  const bool v4 = N % 4 == 0 && all_aligned16({outGrads->data_device, denoms->data_device, inputs->data_device,
+                                               acts->data_device, targets->data_device});
+  PoolGeom g;
+  make_geom(g, N, numFilters, S, S, 0, 0, 1, v4 ? 4 : 1);
+  const unsigned grid = grid_for(total / (v4 ? 4 : 1));
+  if (v4)
+    hipLaunchKernelGGL((k_rnorm_undo<4>), dim3(grid), dim3(256), 0, 0, (const float*)outGrads->data_device,
+                       (const float*)denoms->data_device, (const float*)inputs->data_device,
+                       (const float*)acts->data_device, targets->data_device, g, sizeX, powScale);
+  else
+    hipLaunchKernelGGL((k_rnorm_undo<1>), dim3(grid), dim3(256), 0, 0, (const float*)outGrads->data_device,
+                       (const float*)denoms->data_device, (const float*)inputs->data_device,
+                       (const float*)acts->data_device, targets->data_device, g, sizeX, powScale);
+  if (dn_launch_status()) conv_set_error(where, hipGetErrorString(hipGetLastError()));
+}
+
+extern "C" {
+
+void MaxPool(cudamat* images, cudamat* targets, int numFilters, int subsX, int startX, int strideX, int outputsX) {
+  pool_impl(images, nullptr, targets, numFilters, subsX, startX, strideX, outputsX, "MaxPool");
+}
+
+void ProbMaxPool(cudamat* images, cudamat* rnd, cudamat* targets, int numFilters, int subsX, int startX, int strideX,
+                 int outputsX) {
+  conv_clear_error();
+  POOL_REQUIRE(rnd != nullptr, "ProbMaxPool");
+  pool_impl(images, rnd, targets, numFilters, subsX, startX, strideX, outputsX, "ProbMaxPool");
+}
+
+void MaxPoolUndo(cudamat* images, cudamat* maxGrads, cudamat* maxActs, cudamat* targets, int subsX, int startX,
+                 int strideX, int outputsX) {
+  const char* where = "MaxPoolUndo";
+  conv_clear_error();
+  POOL_REQUIRE(images->on_device && maxGrads->on_device && maxActs->on_device && targets->on_device, where);
+  POOL_REQUIRE(subsX > 0 && strideX > 0 && outputsX > 0, where);
+  const int N = images->size[0];
+  const int outputs = outputsX * outputsX;
+  POOL_REQUIRE(N > 0 && maxGrads->size[1] % outputs == 0, where);
+  const int F = maxGrads->size[1] / outputs;
+  POOL_REQUIRE(F > 0 && images->size[1] % F == 0, where);
+  const int S = isqrt_exact_p(images->size[1] / F);
+  POOL_REQUIRE(S > 0, where);
+  POOL_REQUIRE(maxGrads->size[0] == N && maxActs->size[0] == N && maxActs->size[1] == maxGrads->size[1], where);
+  POOL_REQUIRE(targets->size[0] == N && targets->size[1] == images->size[1], where);
+  const long long total = (long long)N * images->size[1];
+  POOL_REQUIRE(total < (1ll << 32), where);
+  const bool v4 = N % 4 == 0 && all_aligned16({images->data_device, maxGrads->data_device, maxActs->data_device,
+                                               targets->data_device});
+  PoolGeom g;
+  make_geom(g, N, F, S, outputsX, subsX, startX, strideX, v4 ? 4 : 1);
+  const unsigned grid = grid_for(total / (v4 ? 4 : 1));
+  if (v4)
+    hipLaunchKernelGGL((k_pool_undo<4>), dim3(grid), dim3(256), 0, 0, (const float*)images->data_device,
+                       (const float*)maxGrads->data_device, (const float*)maxActs->data_device, targets->data_device, g);
+  else
+    hipLaunchKernelGGL((k_pool_undo<1>), dim3(grid), dim3(256), 0, 0, (const float*)images->data_device,
+                       (const float*)maxGrads->data_device, (const float*)maxActs->data_device, targets->data_device, g);
+  if (dn_launch_status()) conv_set_error(where, hipGetErrorString(hipGetLastError()));
+}
+
+void ResponseNorm(cudamat* images, cudamat* denoms, cudamat* targets, int numFilters, int sizeX, float addScale,
+                  float powScale) {
+  cnorm_impl(images, images, denoms, targets, numFilters, sizeX, addScale, powScale, "ResponseNorm");
+}
+
+void ContrastNorm(cudamat* images, cudamat* meanDiffs, cudamat* denoms, cudamat* targets, int numFilters, int sizeX,
+                  float addScale, float powScale) {
+  cnorm_impl(images, meanDiffs, denoms, targets, numFilters, sizeX, addScale, powScale, "ContrastNorm");
+}
+
+void ResponseNormUndo(cudamat* outGrads, cudamat* denoms, cudamat* inputs, cudamat* acts, cudamat* targets,
+                      int numFilters, int sizeX, float addScale, float powScale) {
+  rnorm_undo_impl(outGrads, denoms, inputs, acts, targets, numFilters, sizeX, addScale, powScale, "ResponseNormUndo");
+}
+
+void ContrastNormUndo(cudamat* outGrads, cudamat* denoms, cudamat* meanDiffs, cudamat* acts, cudamat* targets,
+                      int numFilters, int sizeX, float addScale, float powScale) {
+  rnorm_undo_impl(outGrads, denoms, meanDiffs, acts, targets, numFilters, sizeX, addScale, powScale,
+                  "ContrastNormUndo");
+}
+
+}  // extern "C"

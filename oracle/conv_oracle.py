@@ -1,0 +1,292 @@
+"""TEST INFRASTRUCTURE ONLY - numpy restatement of cudamat_conv's convolution,
+pooling and normalisation.  Only tests/, __graft_entry__.smoke() and bench.py's
+cpu_baseline leg may import this; the product (deepnet_amd/) never does.
+
+Tensors are given in the device layout: 2-D arrays of shape (numImages, C*S*S)
+whose column index is (c*S + y)*S + x  (cudamat/cudamat_conv.cu:9-13); filters are
+(numFilters, Cg*k*k) with column (c*k + ky)*k + kx.  All arithmetic is float64.
+
+Two codings of each convolution pass are kept: `*_loops`, a literal nest of Python
+loops over the definition (tiny shapes only), and the vectorised one used on real
+sizes.  The reference has no tests for these entry points (nothing under
+/root/reference references convUp ... outside convolutions.py), so parity is
+pinned here by: loops == vectorised; == torch.nn.functional.conv2d / max_pool2d /
+avg_pool2d after layout permutes where those define the same thing; the adjoint
+identities <convUp(x,w),y> = <x,convDown(y,w)> = <w,convOutp(x,y)>; and float64
+finite differences for the normalisation gradient (tests/test_oracle_conv.py).
+The tie rule of MaxPoolUndo (every tied position receives the gradient,
+cudamat_conv_kernels.cuh:1502) is pinned by a hand-made case only.
+"""
+import numpy as np
+
+F64 = np.float64
+
+
+def to_nchw(mat, C, S):
+    """(N, C*S*S) device layout -> (N, C, S, S)."""
+    mat = np.asarray(mat, dtype=F64)
+    return mat.reshape(mat.shape[0], C, S, S)
+
+
+def from_nchw(t):
+    return np.asarray(t, dtype=F64).reshape(t.shape[0], -1)
+
+
+def filters_to_fckk(flt, Cg, k):
+    """(F, Cg*k*k) -> (F, Cg, k, k)."""
+    flt = np.asarray(flt, dtype=F64)
+    return flt.reshape(flt.shape[0], Cg, k, k)
+
+
+def n_modules(H, k, stride, padding):
+    """deepnet/convolutions.py:35: n_locs = (x + 2p - size) / stride + 1 (floor)."""
+    return (H + 2 * padding - k) // stride + 1
+
+
+# ---- filterActs: cudamat_conv.cu:15-257, cudamat_conv_kernels.cuh:82-394 ----------
+
+def conv_up_loops(images, filters, C, Mx, padding, stride, groups=1):
+    """out[n, f, my, mx] = sum_{c,ky,kx} img[n, g*Cg+c, my*s+ky-p, mx*s+kx-p] * w[f, c, ky, kx]; zero outside."""
+    images = np.asarray(images, dtype=F64)
+    filters = np.asarray(filters, dtype=F64)
+    N = images.shape[0]
+    H = int(round(np.sqrt(images.shape[1] // C)))
+    F = filters.shape[0]
+    Cg = C // groups
+    k = int(round(np.sqrt(filters.shape[1] // Cg)))
+    Fg = F // groups
+    out = np.zeros((N, F * Mx * Mx))
+    for n in range(N):
+        for f in range(F):
+            g = f // Fg
+            for my in range(Mx):
+                for mx in range(Mx):
+                    acc = 0.0
+                    for c in range(Cg):
+                        for ky in range(k):
+                            for kx in range(k):
+                                y, x = my * stride + ky - padding, mx * stride + kx - padding
+                                if 0 <= y < H and 0 <= x < H:
+                                    acc += images[n, ((g * Cg + c) * H + y) * H + x] * filters[f, (c * k + ky) * k + kx]
+                    out[n, (f * Mx + my) * Mx + mx] = acc
+    return out
+
+
+def _geom(images, filters, C, groups):
+    N = images.shape[0]
+    H = int(round(np.sqrt(images.shape[1] // C)))
+    F = filters.shape[0]
+    Cg = C // groups
+    k = int(round(np.sqrt(filters.shape[1] // Cg)))
+    return N, H, F, Cg, k, F // groups
+
+
+def _patch_view(xp, ky, kx, Mx, stride):
+    """xp: padded (N, C, Hp, Hp) -> (N, C, Mx, Mx) samples at module origin + (ky, kx)."""
+    return xp[:, :, ky:ky + (Mx - 1) * stride + 1:stride, kx:kx + (Mx - 1) * stride + 1:stride]
+
+
+def _pad_for(H, k, Mx, padding, stride):
+    """Zero border wide enough for every module, including ones reaching past the far edge."""
+    far = max(0, (Mx - 1) * stride + k - padding - H)
+    return padding, far
+
+
+def conv_up(images, filters, C, Mx, padding, stride, groups=1):
+    images = np.asarray(images, dtype=F64)
+    filters = np.asarray(filters, dtype=F64)
+    N, H, F, Cg, k, Fg = _geom(images, filters, C, groups)
+    x = to_nchw(images, C, H)
+    w = filters_to_fckk(filters, Cg, k)
+    lo, hi = _pad_for(H, k, Mx, padding, stride)
+    xp = np.pad(x, ((0, 0), (0, 0), (lo, hi), (lo, hi)))
+    out = np.zeros((N, F, Mx, Mx))
+    for g in range(groups):
+        xs = xp[:, g * Cg:(g + 1) * Cg]
+        ws = w[g * Fg:(g + 1) * Fg]
+        for ky in range(k):
+            for kx in range(k):
+                out[:, g * Fg:(g + 1) * Fg] += np.einsum('ncyx,fc->nfyx', _patch_view(xs, ky, kx, Mx, stride), ws[:, :, ky, kx])
+    return from_nchw(out)
+
+
+# ---- imgActs: cudamat_conv.cu:265-640 ------------------------------------------------
+
+def conv_down(hid, filters, C, H, padding, stride, groups=1):
+    """Adjoint of conv_up w.r.t. the images."""
+    hid = np.asarray(hid, dtype=F64)
+    filters = np.asarray(filters, dtype=F64)
+    N, F = hid.shape[0], filters.shape[0]
+    Cg = C // groups
+    k = int(round(np.sqrt(filters.shape[1] // Cg)))
+    Fg = F // groups
+    Mx = int(round(np.sqrt(hid.shape[1] // F)))
+    h = hid.reshape(N, F, Mx, Mx)
+    w = filters_to_fckk(filters, Cg, k)
+    lo, hi = _pad_for(H, k, Mx, padding, stride)
+    gp = np.zeros((N, C, H + lo + hi, H + lo + hi))
+    for g in range(groups):
+        hs = h[:, g * Fg:(g + 1) * Fg]
+        ws = w[g * Fg:(g + 1) * Fg]
+        for ky in range(k):
+            for kx in range(k):
+                _patch_view(gp[:, g * Cg:(g + 1) * Cg], ky, kx, Mx, stride)[...] += np.einsum('nfyx,fc->ncyx', hs, ws[:, :, ky, kx])
+    return from_nchw(gp[:, :, lo:lo + H, lo:lo + H])
+
+
+def conv_down_loops(hid, filters, C, H, padding, stride, groups=1):
+    hid = np.asarray(hid, dtype=F64)
+    filters = np.asarray(filters, dtype=F64)
+    N, F = hid.shape[0], filters.shape[0]
+    Cg = C // groups
+    k = int(round(np.sqrt(filters.shape[1] // Cg)))
+    Fg = F // groups
+    Mx = int(round(np.sqrt(hid.shape[1] // F)))
+    out = np.zeros((N, C * H * H))
+    for n in range(N):
+        for f in range(F):
+            g = f // Fg
+            for my in range(Mx):
+                for mx in range(Mx):
+                    hv = hid[n, (f * Mx + my) * Mx + mx]
+                    for c in range(Cg):
+                        for ky in range(k):
+                            for kx in range(k):
+                                y, x = my * stride + ky - padding, mx * stride + kx - padding
+                                if 0 <= y < H and 0 <= x < H:
+                                    out[n, ((g * Cg + c) * H + y) * H + x] += hv * filters[f, (c * k + ky) * k + kx]
+    return out
+
+
+# ---- weightActs: cudamat_conv.cu:642-1015 ----------------------------------------------
+
+def conv_outp(images, hid, C, Mx, k, padding, stride, groups=1, partial_sum=0):
+    """dw[f, c, ky, kx] = sum_{n, my, mx} img[n, g*Cg+c, my*s+ky-p, mx*s+kx-p] * hid[n, f, my, mx].
+    With partial_sum the modules are summed in consecutive chunks of that many and the
+    result is (F, chunks*Cg*k*k), chunk-major."""
+    images = np.asarray(images, dtype=F64)
+    hid = np.asarray(hid, dtype=F64)
+    N = images.shape[0]
+    H = int(round(np.sqrt(images.shape[1] // C)))
+    F = hid.shape[1] // (Mx * Mx)
+    Cg, Fg = C // groups, F // groups
+    x = to_nchw(images, C, H)
+    h = hid.reshape(N, F, Mx, Mx)
+    lo, hi = _pad_for(H, k, Mx, padding, stride)
+    xp = np.pad(x, ((0, 0), (0, 0), (lo, hi), (lo, hi)))
+    M = Mx * Mx
+    ps = M if partial_sum == 0 else partial_sum
+    chunks = M // ps
+    out = np.zeros((chunks, F, Cg, k, k))
+    for g in range(groups):
+        xs = xp[:, g * Cg:(g + 1) * Cg]
+        hs = h[:, g * Fg:(g + 1) * Fg].reshape(N, Fg, M)
+        for ky in range(k):
+            for kx in range(k):
+                pv = _patch_view(xs, ky, kx, Mx, stride).reshape(N, Cg, M)
+                for ch in range(chunks):
+                    sl = slice(ch * ps, (ch + 1) * ps)
+                    out[ch, g * Fg:(g + 1) * Fg, :, ky, kx] = np.einsum('ncm,nfm->fc', pv[:, :, sl], hs[:, :, sl])
+    return np.concatenate([out[ch].reshape(F, -1) for ch in range(chunks)], axis=1)
+
+
+# ---- pooling: cudamat_conv.cu:1021-1182, cudamat_conv_kernels.cuh:1355-1530 -------------
+
+def max_pool(images, F, subs, start, stride, O):
+    images = np.asarray(images, dtype=F64)
+    N = images.shape[0]
+    S = int(round(np.sqrt(images.shape[1] // F)))
+    x = to_nchw(images, F, S)
+    out = np.full((N, F, O, O), -2e38)
+    for oy in range(O):
+        for ox in range(O):
+            y0, x0 = max(0, start + oy * stride), max(0, start + ox * stride)
+            y1, x1 = min(S, start + oy * stride + subs), min(S, start + ox * stride + subs)
+            if y1 > y0 and x1 > x0:
+                out[:, :, oy, ox] = np.maximum(x[:, :, y0:y1, x0:x1].max(axis=(2, 3)), -2e38)
+    return from_nchw(out)
+
+
+def max_pool_undo(images, max_grads, max_acts, subs, start, stride, O):
+    """target[px] = sum over outputs whose window holds px of (img[px] == maxAct[o]) * maxGrad[o]."""
+    images = np.asarray(images, dtype=F64)
+    N = images.shape[0]
+    F = max_grads.shape[1] // (O * O)
+    S = int(round(np.sqrt(images.shape[1] // F)))
+    x = to_nchw(images, F, S)
+    mg = np.asarray(max_grads, dtype=F64).reshape(N, F, O, O)
+    ma = np.asarray(max_acts, dtype=F64).reshape(N, F, O, O)
+    out = np.zeros((N, F, S, S))
+    for oy in range(O):
+        for ox in range(O):
+            y0, x0 = max(0, start + oy * stride), max(0, start + ox * stride)
+            y1, x1 = min(S, start + oy * stride + subs), min(S, start + ox * stride + subs)
+            if y1 > y0 and x1 > x0:
+                hit = x[:, :, y0:y1, x0:x1] == ma[:, :, oy, ox][:, :, None, None]
+                out[:, :, y0:y1, x0:x1] += hit * mg[:, :, oy, ox][:, :, None, None]
+    return from_nchw(out)
+
+
+def prob_max_pool(images, rnd, F, subs, start, stride, O):
+    """The reference's scan (cudamat_conv_kernels.cuh:44-55, 1594-1608) in float32: the
+    candidate replaces the running value unless running*r_running > candidate*r_candidate,
+    starting from (-2e38, -2e38), whose product overflows to +inf."""
+    images = np.asarray(images, dtype=np.float32)
+    rnd = np.asarray(rnd, dtype=np.float32)
+    N = images.shape[0]
+    S = int(round(np.sqrt(images.shape[1] // F)))
+    x = images.reshape(N, F, S, S)
+    r = rnd.reshape(N, F, S, S)
+    out = np.empty((N, F, O, O), dtype=np.float32)
+    with np.errstate(over='ignore', invalid='ignore'):
+        for oy in range(O):
+            for ox in range(O):
+                acc = np.full((N, F), -2e38, dtype=np.float32)
+                racc = np.full((N, F), -2e38, dtype=np.float32)
+                for y in range(max(0, start + oy * stride), min(S, start + oy * stride + subs)):
+                    for xx in range(max(0, start + ox * stride), min(S, start + ox * stride + subs)):
+                        keep = acc * racc > x[:, :, y, xx] * r[:, :, y, xx]
+                        acc = np.where(keep, acc, x[:, :, y, xx])
+                        racc = np.where(keep, racc, r[:, :, y, xx])
+                out[:, :, oy, ox] = acc
+    return out.reshape(N, -1).astype(F64)
+
+
+# ---- normalisation: cudamat_conv_kernels.cu:112-176, cudamat_conv_kernels.cuh:1920-2023 ----
+
+def _window_sum(t, size, lo_off):
+    """Sum over the clipped window [p + lo_off, p + lo_off + size) along the last two axes."""
+    S = t.shape[-1]
+    out = np.zeros_like(t)
+    for dy in range(lo_off, lo_off + size):
+        for dx in range(lo_off, lo_off + size):
+            ys, xs = slice(max(0, -dy), min(S, S - dy)), slice(max(0, -dx), min(S, S - dx))
+            yd, xd = slice(max(0, dy), min(S, S + dy)), slice(max(0, dx), min(S, S + dx))
+            out[..., ys, xs] += t[..., yd, xd]
+    return out
+
+
+def contrast_norm(images, mean_diffs, F, size, add_scale, pow_scale):
+    """denoms = 1 + addScale * sum_{window at -size/2} meanDiffs^2; target = images * denoms^-powScale."""
+    images = np.asarray(images, dtype=F64)
+    S = int(round(np.sqrt(images.shape[1] // F)))
+    x = to_nchw(images, F, S)
+    md = to_nchw(mean_diffs, F, S)
+    den = 1.0 + F64(np.float32(add_scale)) * _window_sum(md * md, size, -(size // 2))
+    return from_nchw(x * den ** (-F64(np.float32(pow_scale)))), from_nchw(den)
+
+
+def response_norm(images, F, size, add_scale, pow_scale):
+    return contrast_norm(images, images, F, size, add_scale, pow_scale)
+
+
+def response_norm_undo(out_grads, denoms, inputs, acts, F, size, add_scale, pow_scale):
+    """Returns (target, acts_after): acts' = -2*addScale*powScale*outGrads*acts/denoms;
+    target = inputs * sum_{mirrored window} acts' + outGrads * denoms^-powScale."""
+    og = np.asarray(out_grads, dtype=F64)
+    S = int(round(np.sqrt(og.shape[1] // F)))
+    a, p = F64(np.float32(add_scale)), F64(np.float32(pow_scale))
+    og4, den4, in4, act4 = (to_nchw(t, F, S) for t in (out_grads, denoms, inputs, acts))
+    act2 = F64(np.float32(-2.0) * np.float32(add_scale) * np.float32(pow_scale)) * og4 * act4 / den4
+    win = _window_sum(act2, size, size // 2 - size + 1)
+    return from_nchw(in4 * win + og4 * den4 ** (-p)), from_nchw(act2)

@@ -1,0 +1,184 @@
+"""GPU parity of convUp / convDown / convOutp, MaxPool(+Undo), ResponseNorm(+Undo)
+against the float64 restatement: 1e-4 relative for the convolutions (error measured
+against the sum of magnitudes, as for dot), exact for pooling, 2e-6 relative for the
+normalisation.  Shapes with a batch that is not a multiple of 16 run the
+one-lane-per-output kernels; the others the matrix-core kernel."""
+import numpy as np
+import pytest
+
+from oracle import conv_oracle as co
+
+pytestmark = pytest.mark.gpu
+
+REL = 1e-4
+
+CASES = [  # N, C, H, F, k, stride, padding, groups
+    (2, 3, 6, 16, 3, 1, 1, 1),       # direct kernels (batch 2)
+    (3, 4, 7, 8, 3, 2, 1, 2),
+    (16, 3, 6, 16, 3, 1, 1, 1),      # matrix-core kernels from here on
+    (16, 3, 8, 16, 5, 1, 2, 1),
+    (32, 1, 9, 32, 3, 1, 0, 1),
+    (16, 3, 12, 16, 5, 4, 0, 1),     # strided; last module stops short of the edge
+    (16, 3, 13, 48, 4, 3, 2, 1),     # stride 3, 48 filters (3 column blocks)
+    (32, 8, 7, 32, 3, 1, 1, 2),      # 2 groups of 4 colours / 16 filters
+    (16, 32, 6, 64, 3, 2, 1, 2),
+    (128, 3, 32, 64, 5, 1, 2, 1),    # the CIFAR layer of the benchmark
+    (16, 48, 9, 160, 3, 1, 1, 1),    # more than 128 filters: two column tiles
+]
+
+
+def _f(a):
+    return np.asarray(a, dtype=np.float32, order='F')
+
+
+def _relerr(got, want, bound):
+    return np.max(np.abs(np.asarray(got, np.float64) - want) / (bound + 1e-30))
+
+
+@pytest.mark.parametrize("N,C,H,F,k,s,p,G", CASES)
+def test_three_conv_passes(cm, cc, rng, N, C, H, F, k, s, p, G):
+    Mx = co.n_modules(H, k, s, p)
+    x = _f(rng.standard_normal((N, C * H * H)))
+    w = _f(0.1 * rng.standard_normal((F, (C // G) * k * k)))
+    y = _f(rng.standard_normal((N, F * Mx * Mx)))
+    X, W, Y = cm.CUDAMatrix(x), cm.CUDAMatrix(w), cm.CUDAMatrix(y)
+    up = cm.CUDAMatrix(np.full((N, F * Mx * Mx), np.nan, dtype=np.float32))     # must be overwritten, not accumulated
+    cc.convUp(X, W, up, Mx, p, s, C, G)
+    assert _relerr(up.asarray(), co.conv_up(x, w, C, Mx, p, s, G), co.conv_up(np.abs(x), np.abs(w), C, Mx, p, s, G)) < REL
+    down = cm.CUDAMatrix(np.full((N, C * H * H), np.nan, dtype=np.float32))
+    cc.convDown(Y, W, down, Mx, p, s, k, H, C, numGroups=G)
+    assert _relerr(down.asarray(), co.conv_down(y, w, C, H, p, s, G),
+                   co.conv_down(np.abs(y), np.abs(w), C, H, p, s, G) + 1e-6) < REL
+    outp = cm.CUDAMatrix(np.full((F, (C // G) * k * k), np.nan, dtype=np.float32))
+    cc.convOutp(X, Y, outp, Mx, p, k, s, C, numGroups=G)
+    assert _relerr(outp.asarray(), co.conv_outp(x, y, C, Mx, k, p, s, G),
+                   co.conv_outp(np.abs(x), np.abs(y), C, Mx, k, p, s, G)) < REL
+    # adjoint identities on the device results themselves
+    a = float((up.asarray().astype(np.float64) * y).sum())
+    b = float((down.asarray().astype(np.float64) * x).sum())
+    c = float((outp.asarray().astype(np.float64) * w).sum())
+    scale = float((np.abs(up.asarray()).astype(np.float64) * np.abs(y)).sum())
+    assert abs(a - b) / scale < 1e-5 and abs(a - c) / scale < 1e-5
+    for m in (X, W, Y, up, down, outp):
+        m.free_device_memory()
+
+
+def test_outp_with_partial_sums(cm, cc, rng):
+    N, C, H, F, k, s, p = 16, 3, 8, 16, 3, 1, 1
+    Mx = co.n_modules(H, k, s, p)
+    x, y = _f(rng.standard_normal((N, C * H * H))), _f(rng.standard_normal((N, F * Mx * Mx)))
+    t = cm.empty((F, Mx * C * k * k))
+    cc.convOutp(cm.CUDAMatrix(x), cm.CUDAMatrix(y), t, Mx, p, k, s, C, partialSum=Mx)
+    want = co.conv_outp(x, y, C, Mx, k, p, s, partial_sum=Mx)
+    assert np.max(np.abs(t.asarray() - want)) < 1e-3
+
+
+def test_fast_and_direct_kernels_agree(cm, cc, rng):
+    """The same problem through both code paths: batch 16 (matrix cores) and the same 16
+    images split as 2 batches of 8 (one lane per output)."""
+    C, H, F, k, s, p = 3, 10, 16, 5, 2, 2
+    Mx = co.n_modules(H, k, s, p)
+    x = _f(rng.standard_normal((16, C * H * H)))
+    w = _f(0.1 * rng.standard_normal((F, C * k * k)))
+    W = cm.CUDAMatrix(w)
+    full = cm.empty((16, F * Mx * Mx))
+    cc.convUp(cm.CUDAMatrix(x), W, full, Mx, p, s, C)
+    halves = []
+    for part in (x[:8], x[8:]):
+        t = cm.empty((8, F * Mx * Mx))
+        cc.convUp(cm.CUDAMatrix(_f(part)), W, t, Mx, p, s, C)
+        halves.append(t.asarray())
+    assert np.allclose(full.asarray(), np.vstack(halves), rtol=1e-5, atol=1e-5)
+
+
+def test_bad_shapes_raise_instead_of_aborting(cm, cc, rng):
+    X = cm.CUDAMatrix(_f(rng.standard_normal((16, 3 * 36))))
+    W = cm.CUDAMatrix(_f(rng.standard_normal((16, 27))))
+    with pytest.raises(AssertionError):
+        cc.convUp(X, W, cm.empty((16, 5)), 6, 1, 1, 3)
+    with pytest.raises(cm.CUDAMatException, match="convUp"):
+        cc._call('convUp', X.p_mat, W.p_mat, cm.empty((16, 16 * 36)).p_mat, 6, -1, 1, 4, 1)   # 108 % 4 colours
+    with pytest.raises(cm.CUDAMatException, match="not implemented"):
+        cc.localUp(X, W, cm.empty((16, 16 * 36)), 6, 1, 1, 3)
+    host_only = cm.CUDAMatrix(_f(rng.standard_normal((16, 108))), copy_to_device=False)
+    with pytest.raises(cm.CUDAMatException, match="on_device"):
+        cc.MaxPool(host_only, cm.empty((16, 3 * 9)), 3, 2, 0, 2, 3)
+
+
+POOLS = [  # N, F, S, subs, start, stride
+    (2, 3, 8, 2, 0, 2), (5, 4, 9, 3, 0, 2), (16, 16, 32, 3, 0, 2), (16, 8, 7, 3, -1, 2), (128, 64, 32, 3, 0, 2),
+    (4, 2, 6, 2, 0, 1),
+]
+
+
+@pytest.mark.parametrize("N,F,S,subs,start,stride", POOLS)
+def test_max_pool_and_undo(cm, cc, rng, N, F, S, subs, start, stride):
+    O = (S - start - subs + stride - 1) // stride + 1
+    x = _f(rng.standard_normal((N, F * S * S)))
+    X, T = cm.CUDAMatrix(x), cm.empty((N, F * O * O))
+    cc.MaxPool(X, T, F, subs, start, stride, O)
+    want = co.max_pool(x, F, subs, start, stride, O)
+    assert np.array_equal(T.asarray(), want.astype(np.float32))
+    g = _f(rng.standard_normal((N, F * O * O)))
+    U = cm.empty((N, F * S * S))
+    cc.MaxPoolUndo(X, U, cm.CUDAMatrix(g), T, subs, start, stride, O)
+    assert np.allclose(U.asarray(), co.max_pool_undo(x, g, want, subs, start, stride, O), rtol=1e-6, atol=1e-6)
+    # ties: a constant image routes every output's gradient to all pixels of its window
+    ones = cm.CUDAMatrix(np.ones((N, F * S * S), dtype=np.float32))
+    cc.MaxPool(ones, T, F, subs, start, stride, O)
+    cc.MaxPoolUndo(ones, U, cm.CUDAMatrix(g), T, subs, start, stride, O)
+    one_np = np.ones((N, F * S * S))
+    assert np.allclose(U.asarray(), co.max_pool_undo(one_np, g, co.max_pool(one_np, F, subs, start, stride, O), subs, start,
+                                                     stride, O), rtol=1e-5, atol=1e-5)
+
+
+def test_prob_max_pool_follows_the_reference_scan(cm, cc, rng):
+    N, F, S = 16, 4, 6
+    x, r = _f(rng.standard_normal((N, F * S * S))), _f(rng.random((N, F * S * S)))
+    T = cm.empty((N, F * 9))
+    cc.ProbMaxPool(cm.CUDAMatrix(x), cm.CUDAMatrix(r), T, F, 2, 0, 2, 3)
+    assert np.array_equal(T.asarray(), co.prob_max_pool(x, r, F, 2, 0, 2, 3).astype(np.float32))
+
+
+@pytest.mark.parametrize("N,F,S,size", [(2, 3, 7, 3), (16, 16, 15, 5), (5, 4, 6, 4), (128, 64, 15, 5)])
+def test_response_norm_and_undo(cm, cc, rng, N, F, S, size):
+    a, p = 0.001, 0.75
+    x = _f(rng.standard_normal((N, F * S * S)) * 3)
+    X, D, T = cm.CUDAMatrix(x), cm.empty(x.shape), cm.empty(x.shape)
+    cc.ResponseNorm(X, D, T, F, size, a, p)
+    t_want, d_want = co.response_norm(x, F, size, a, p)
+    assert np.allclose(D.asarray(), d_want, rtol=2e-6)
+    assert np.allclose(T.asarray(), t_want, rtol=2e-6, atol=1e-7)
+    g = _f(rng.standard_normal(x.shape))
+    acts = cm.CUDAMatrix(T.asarray().copy(order='F'))
+    U = cm.empty(x.shape)
+    cc.ResponseNormUndo(cm.CUDAMatrix(g), D, X, acts, U, F, size, a, p)
+    u_want, acts_want = co.response_norm_undo(g, D.asarray(), x, T.asarray(), F, size, a, p)
+    assert np.allclose(acts.asarray(), acts_want, rtol=1e-5, atol=1e-9)      # acts is overwritten, as in the reference
+    assert np.allclose(U.asarray(), u_want, rtol=1e-5, atol=1e-6)
+    # contrast norm with separate mean differences
+    md = _f(rng.standard_normal(x.shape))
+    cc.ContrastNorm(X, cm.CUDAMatrix(md), D, T, F, size, a, p)
+    t2, d2 = co.contrast_norm(x, md, F, size, a, p)
+    assert np.allclose(D.asarray(), d2, rtol=2e-6) and np.allclose(T.asarray(), t2, rtol=2e-6, atol=1e-7)
+
+
+def test_conv_layer_chain_like_deepnet(cm, cc, rng):
+    """convolutions.py:5-67 order: transpose -> convUp -> MaxPool -> ResponseNorm -> transpose."""
+    N, C, H, F, k, p = 128, 3, 32, 64, 5, 2
+    Mx = co.n_modules(H, k, 1, p)
+    inputs = _f(rng.standard_normal((C * H * H, N)))            # deepnet keeps (dims, batch)
+    w = _f(0.01 * rng.standard_normal((F, C * k * k)))
+    inp = cm.CUDAMatrix(inputs)
+    xt = cm.empty((N, C * H * H))
+    inp.transpose(xt)
+    conv = cm.empty((N, F * Mx * Mx)); cc.convUp(xt, cm.CUDAMatrix(w), conv, Mx, p, 1, C)
+    O = 15
+    pooled = cm.empty((N, F * O * O)); cc.MaxPool(conv, pooled, F, 3, 0, 2, O)
+    den, normed = cm.empty((N, F * O * O)), cm.empty((N, F * O * O))
+    cc.ResponseNorm(pooled, den, normed, F, 5, 0.001, 0.75)
+    out = cm.empty((F * O * O, N)); normed.transpose(out)
+    want = co.conv_up(inputs.T, w, C, Mx, p, 1)
+    want = co.max_pool(want, F, 3, 0, 2, O)
+    want, _ = co.response_norm(want, F, 5, 0.001, 0.75)
+    assert np.allclose(out.asarray(), want.T, rtol=2e-4, atol=2e-5)
