@@ -352,7 +352,7 @@ def main():
     value = STEP_BYTES / step_s / 1e9
 
     roof_op = 'add_mult'
-    roofline = {'kernel': 'k_ew<2, FAxpy> (add_mult, 4096x4096)', 'bound': 'hbm',
+    roofline = {'kernel': 'k_ew<2, true, FAxpy> (add_mult, 4096x4096)', 'bound': 'hbm',
                 'achieved': ops[roof_op]['gbs'], 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
                 'frac': round(ops[roof_op]['gbs'] / HBM_PEAK_GBS, 4), 'traffic': None,
                 'algorithmic_bytes_per_launch': 12 * E, 'avg_launch_us': ops[roof_op]['us']}

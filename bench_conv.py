@@ -1,0 +1,71 @@
+"""Convolution leg of bench.py: the three conv passes, local max-pool and response
+norm at the benchmark's layer shapes, timed with HIP events on the NULL stream.
+
+  C4   3x32x32 -> 64 @ 5x5, stride 1, padding 2, batch 128; pool 3x3/2 -> 15x15; rnorm 5
+  C5a  3x224x224 -> 96 @ 11x11, stride 4, no padding, batch 128
+  C5b  96x27x27 -> 256 @ 5x5, padding 2, 2 groups, batch 128
+"""
+import numpy as np
+
+MFMA_FP32_PEAK_TFLOPS = 157.3
+HBM_PEAK_GBS = 8000.0
+
+LAYERS = {
+    'c4_3x32x32_64f5': dict(N=128, C=3, H=32, F=64, k=5, s=1, p=2, G=1),
+    'c5a_3x224x224_96f11s4': dict(N=128, C=3, H=224, F=96, k=11, s=4, p=0, G=1),
+    'c5b_96x27x27_256f5g2': dict(N=128, C=96, H=27, F=256, k=5, s=1, p=2, G=2),
+}
+
+
+def _time(ev, fn, iters):
+    fn()
+    e0, e1 = ev.new(), ev.new()
+    ev.record(e0)
+    for _ in range(iters):
+        fn()
+    ev.record(e1)
+    return ev.elapsed_ms(e0, e1) / iters
+
+
+def run(cm, ev, iters=10):
+    from deepnet_amd import cudamat_conv as cc
+    rng = np.random.default_rng(5)
+    f = lambda a: cm.CUDAMatrix(np.asarray(a, dtype=np.float32, order='F'))
+    out = {}
+    for name, L in LAYERS.items():
+        N, C, H, F, k, s, p, G = (L[x] for x in ('N', 'C', 'H', 'F', 'k', 's', 'p', 'G'))
+        Mx = (H + 2 * p - k) // s + 1
+        X = f(rng.standard_normal((N, C * H * H)))
+        W = f(0.01 * rng.standard_normal((F, (C // G) * k * k)))
+        Y = f(rng.standard_normal((N, F * Mx * Mx)))
+        up, down, dw = cm.empty((N, F * Mx * Mx)), cm.empty((N, C * H * H)), cm.empty((F, (C // G) * k * k))
+        flops = 2.0 * N * F * Mx * Mx * (C // G) * k * k
+        res = {'gflop_per_pass': round(flops / 1e9, 3)}
+        for label, fn in (('convUp', lambda: cc.convUp(X, W, up, Mx, p, s, C, G)),
+                          ('convDown', lambda: cc.convDown(Y, W, down, Mx, p, s, k, H, C, numGroups=G)),
+                          ('convOutp', lambda: cc.convOutp(X, Y, dw, Mx, p, k, s, C, numGroups=G))):
+            ms = _time(ev, fn, iters)
+            tf = flops / (ms * 1e-3) / 1e12
+            res[label] = {'ms': round(ms, 4), 'tflops': round(tf, 2),
+                          'frac_mfma_fp32': round(tf / MFMA_FP32_PEAK_TFLOPS, 4)}
+        if name.startswith('c4'):
+            O = 15
+            pooled, grad = cm.empty((N, F * O * O)), f(rng.standard_normal((N, F * O * O)))
+            undo = cm.empty((N, F * Mx * Mx))
+            den, normed, nundo = cm.empty((N, F * O * O)), cm.empty((N, F * O * O)), cm.empty((N, F * O * O))
+            acts = cm.empty((N, F * O * O))
+            e_in, e_out = 4.0 * N * F * Mx * Mx, 4.0 * N * F * O * O
+            for label, fn, nbytes in (
+                    ('MaxPool', lambda: cc.MaxPool(up, pooled, F, 3, 0, 2, O), e_in + e_out),
+                    ('MaxPoolUndo', lambda: cc.MaxPoolUndo(up, undo, grad, pooled, 3, 0, 2, O), 2 * e_in + 2 * e_out),
+                    ('ResponseNorm', lambda: cc.ResponseNorm(pooled, den, normed, F, 5, 0.001, 0.75), 3 * e_out),
+                    ('ResponseNormUndo', lambda: (acts.assign(normed),
+                                                  cc.ResponseNormUndo(grad, den, pooled, acts, nundo, F, 5, 0.001, 0.75)),
+                     (2 + 7) * e_out)):
+                ms = _time(ev, fn, iters)
+                gbs = nbytes / (ms * 1e-3) / 1e9
+                res[label] = {'us': round(ms * 1e3, 2), 'gbs': round(gbs, 1), 'frac_hbm': round(gbs / HBM_PEAK_GBS, 4)}
+        out[name] = res
+        for m in (X, W, Y, up, down, dw):
+            m.free_device_memory()
+    return {'conv': out}

@@ -2,10 +2,10 @@
 // Replaces the grid-stride kernels of cudamat/cudamat_kernels.cu:298-716 and
 // their wrappers cudamat/cudamat.cu:592-1146, 1318-1669, 1763-2102.
 //
-// All of these are HBM-bound.  One templated kernel moves 16-byte vectors with
-// four independent loads in flight per lane; operands that are not 16-byte
-// aligned (column views) are peeled to alignment when they share the same
-// offset and fall back to 4-byte accesses otherwise.
+// All of these are HBM-bound.  One templated kernel moves one 16-byte vector per
+// lane (non-temporal for large operands); operands that are not 16-byte aligned
+// (column views) are peeled to alignment when they share the same offset and
+// fall back to 4-byte accesses otherwise.
 #include "common.h"
 #include "wide_math.h"
 #include <math.h>
@@ -83,40 +83,26 @@ DN_FUNCTOR1(FAssignS, s)
 // ------------------------------------------------------------------ kernels
 
 #define EW_THREADS 256
-#define EW_UNROLL 4
 
-// NIN inputs (0, 1 or 2) -> one output.  [head, head + 4*n4) is moved as
-// 16-byte vectors; the up-to-3 leading and trailing elements by single lanes.
-template <int NIN, class F>
+// NIN inputs (0, 1 or 2) -> one output, one 16-byte vector per lane (the shape
+// that measures fastest on this part: every lane issues its loads at once and
+// the grid is large enough to cover the latency).  [head, head + 4*n4) is moved
+// as vectors; the up-to-3 leading and trailing elements by single lanes.
+template <int NIN, bool STREAM, class F>
 __global__ void __launch_bounds__(EW_THREADS)
 k_ew(const float* a, const float* b, float* t, long long n, int head, long long n4, F f) {
   const long long tid = (long long)blockIdx.x * EW_THREADS + threadIdx.x;
-  const long long stride = (long long)gridDim.x * EW_THREADS;
-  const float4* a4 = reinterpret_cast<const float4*>(a + head);
-  const float4* b4 = reinterpret_cast<const float4*>(b + head);
-  float4* t4 = reinterpret_cast<float4*>(t + head);
-  for (long long i = tid; i < n4; i += stride * EW_UNROLL) {
-    float4 va[EW_UNROLL], vb[EW_UNROLL];
-#pragma unroll
-    for (int u = 0; u < EW_UNROLL; ++u) {
-      const long long j = i + u * stride;
-      if (j < n4) {
-        if (NIN >= 1) va[u] = a4[j];
-        if (NIN >= 2) vb[u] = b4[j];
-      }
-    }
-#pragma unroll
-    for (int u = 0; u < EW_UNROLL; ++u) {
-      const long long j = i + u * stride;
-      if (j < n4) {
-        float4 r;
-        r.x = f(va[u].x, vb[u].x);
-        r.y = f(va[u].y, vb[u].y);
-        r.z = f(va[u].z, vb[u].z);
-        r.w = f(va[u].w, vb[u].w);
-        t4[j] = r;
-      }
-    }
+  if (tid < n4) {
+    const long long e = head + 4 * tid;
+    float4 va = make_float4(0.f, 0.f, 0.f, 0.f), vb = va;
+    if (NIN >= 1) va = dn_ld4<STREAM>(a + e);
+    if (NIN >= 2) vb = dn_ld4<STREAM>(b + e);
+    float4 r;
+    r.x = f(va.x, vb.x);
+    r.y = f(va.y, vb.y);
+    r.z = f(va.z, vb.z);
+    r.w = f(va.w, vb.w);
+    dn_st4<STREAM>(t + e, r);
   }
   // ragged ends
   const long long tail0 = head + 4 * n4;
@@ -150,11 +136,13 @@ static int launch_ew(const float* a, const float* b, float* t, long long n, F f)
   if (same_phase) {
     const int head = (int)(ht < n ? ht : n);
     const long long n4 = (n - head) / 4;
-    long long blocks = (n4 + (long long)EW_THREADS * EW_UNROLL - 1) / ((long long)EW_THREADS * EW_UNROLL);
-    const long long cap = (long long)cus * 16;
-    if (blocks > cap) blocks = cap;
+    long long blocks = (n4 + EW_THREADS - 1) / EW_THREADS;
     if (blocks < 1) blocks = 1;
-    hipLaunchKernelGGL((k_ew<NIN, F>), dim3((unsigned)blocks), dim3(EW_THREADS), 0, 0, a, b, t, n, head, n4, f);
+    if (blocks > 0x7fffffffll) return ERROR_UNSUPPORTED;
+    if (n >= DN_STREAM_MIN_ELEMS)
+      hipLaunchKernelGGL((k_ew<NIN, true, F>), dim3((unsigned)blocks), dim3(EW_THREADS), 0, 0, a, b, t, n, head, n4, f);
+    else
+      hipLaunchKernelGGL((k_ew<NIN, false, F>), dim3((unsigned)blocks), dim3(EW_THREADS), 0, 0, a, b, t, n, head, n4, f);
   } else {
     long long blocks = (n + EW_THREADS - 1) / EW_THREADS;
     const long long cap = (long long)cus * 32;
@@ -168,40 +156,24 @@ static int launch_ew(const float* a, const float* b, float* t, long long n, F f)
 // columns (vec[i / h], a row vector) into a flat pass over the matrix.  The
 // row / column of the first element of each 16-byte group comes from one
 // multiply-high; the other three follow by increment-and-wrap.
-template <bool COLVEC, class F>
+template <bool COLVEC, bool STREAM, class F>
 __global__ void __launch_bounds__(EW_THREADS)
 k_bcast(const float* a, const float* vec, float* t, long long n, int head, long long n4, FastDiv fd, F f) {
   const long long tid = (long long)blockIdx.x * EW_THREADS + threadIdx.x;
-  const long long stride = (long long)gridDim.x * EW_THREADS;
   const uint32_t h = fd.d;
-  if (n4 > 0) {
-    const float4* a4 = reinterpret_cast<const float4*>(a + head);
-    float4* t4 = reinterpret_cast<float4*>(t + head);
-    for (long long i = tid; i < n4; i += stride * EW_UNROLL) {
-      float4 va[EW_UNROLL];
+  if (tid < n4) {
+    const uint32_t e = (uint32_t)(head + 4 * tid);
+    const float4 va = dn_ld4<STREAM>(a + e);
+    uint32_t q = fd_div(e, fd);
+    uint32_t r = e - q * h;
+    float v[4];
+    const float x[4] = {va.x, va.y, va.z, va.w};
 #pragma unroll
-      for (int u = 0; u < EW_UNROLL; ++u) {
-        const long long j = i + u * stride;
-        if (j < n4) va[u] = a4[j];
-      }
-#pragma unroll
-      for (int u = 0; u < EW_UNROLL; ++u) {
-        const long long j = i + u * stride;
-        if (j < n4) {
-          const uint32_t e = (uint32_t)(head + 4 * j);
-          uint32_t q = fd_div(e, fd);
-          uint32_t r = e - q * h;
-          float v[4];
-          const float x[4] = {va[u].x, va[u].y, va[u].z, va[u].w};
-#pragma unroll
-          for (int k = 0; k < 4; ++k) {
-            v[k] = f(x[k], vec[COLVEC ? r : q]);
-            if (++r == h) { r = 0; ++q; }
-          }
-          t4[j] = make_float4(v[0], v[1], v[2], v[3]);
-        }
-      }
+    for (int k = 0; k < 4; ++k) {
+      v[k] = f(x[k], vec[COLVEC ? r : q]);
+      if (++r == h) { r = 0; ++q; }
     }
+    dn_st4<STREAM>(t + e, make_float4(v[0], v[1], v[2], v[3]));
   }
   const long long tail0 = head + 4 * n4;
   long long j = -1;
@@ -236,12 +208,14 @@ static int launch_bcast(const float* a, const float* vec, float* t, int h, int w
   if (head_of(a) == ht) {
     const int head = (int)(ht < n ? ht : n);
     const long long n4 = (n - head) / 4;
-    long long blocks = (n4 + (long long)EW_THREADS * EW_UNROLL - 1) / ((long long)EW_THREADS * EW_UNROLL);
-    const long long cap = (long long)cus * 16;
-    if (blocks > cap) blocks = cap;
+    long long blocks = (n4 + EW_THREADS - 1) / EW_THREADS;
     if (blocks < 1) blocks = 1;
-    hipLaunchKernelGGL((k_bcast<COLVEC, F>), dim3((unsigned)blocks), dim3(EW_THREADS), 0, 0, a, vec, t, n, head, n4,
-                       fd, f);
+    if (n >= DN_STREAM_MIN_ELEMS)
+      hipLaunchKernelGGL((k_bcast<COLVEC, true, F>), dim3((unsigned)blocks), dim3(EW_THREADS), 0, 0, a, vec, t, n,
+                         head, n4, fd, f);
+    else
+      hipLaunchKernelGGL((k_bcast<COLVEC, false, F>), dim3((unsigned)blocks), dim3(EW_THREADS), 0, 0, a, vec, t, n,
+                         head, n4, fd, f);
   } else {
     long long blocks = (n + EW_THREADS - 1) / EW_THREADS;
     const long long cap = (long long)cus * 32;

@@ -17,6 +17,7 @@ void* dn_scratch(size_t bytes);
 // ------------------------------------------------------------------ column walkers
 
 // Visit every element of one column with TPC cooperating lanes: fn(row, value).
+// Four 16-byte loads are issued before any of them is consumed.
 template <int TPC, class Fn>
 __device__ __forceinline__ void for_each_in_col(const float* c, int h, int lane, Fn fn) {
   int head = (int)(((16u - (unsigned)(reinterpret_cast<uintptr_t>(c) & 15u)) & 15u) >> 2);
@@ -24,13 +25,21 @@ __device__ __forceinline__ void for_each_in_col(const float* c, int h, int lane,
   if (lane < head) fn(lane, c[lane]);
   const float4* c4 = reinterpret_cast<const float4*>(c + head);
   const int n4 = (h - head) >> 2;
-  for (int j = lane; j < n4; j += TPC) {
+  int j = lane;
+  for (; j + 3 * TPC < n4; j += 4 * TPC) {
+    float4 v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) v[u] = c4[j + u * TPC];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int b = head + 4 * (j + u * TPC);
+      fn(b, v[u].x); fn(b + 1, v[u].y); fn(b + 2, v[u].z); fn(b + 3, v[u].w);
+    }
+  }
+  for (; j < n4; j += TPC) {
     const float4 v = c4[j];
     const int b = head + 4 * j;
-    fn(b, v.x);
-    fn(b + 1, v.y);
-    fn(b + 2, v.z);
-    fn(b + 3, v.w);
+    fn(b, v.x); fn(b + 1, v.y); fn(b + 2, v.z); fn(b + 3, v.w);
   }
   const int t0 = head + 4 * n4;
   if (lane < h - t0) fn(t0 + lane, c[t0 + lane]);
@@ -300,54 +309,143 @@ k_gemv_cols(const float* M, int ld, int h, int w, const float* x, float* y, floa
   if (active && lane == 0) y[col] = (beta == 0.f ? 0.f : beta * y[col]) + alpha * s;
 }
 
-// Stage 1 of y[i] = beta*y[i] + alpha * sum_j M[i + j*ld] * x[j]: workgroup (bx, by)
-// reduces columns [by*cps, (by+1)*cps) for rows 256*bx .. 256*bx+255 (4 rows per
-// lane as one 16-byte load when vec, else 64 rows per workgroup).  With one
-// split the result goes straight to y.
-template <bool VEC>
+// Two-stage reduction along rows (over the columns j of M[i + j*ld]), for
+//   ROW_DOT:   sum_j M(i,j) * x[j]      ROW_SQSUM: sum_j M(i,j)^2      ROW_MAX: max_j M(i,j)
+// Stage 1: workgroup (bx, by) reduces columns [by*cps, (by+1)*cps) for rows
+// 256*bx .. 256*bx+255 when VEC (4 rows per lane, one 16-byte load per column)
+// or 64*bx .. 64*bx+63 otherwise; its 4 wavefronts take every 4th column, four
+// loads in flight each, and meet in LDS.  With one split the result is final.
+enum { ROW_DOT = 0, ROW_SQSUM = 1, ROW_MAX = 2 };
+
+template <int OP>
+__device__ __forceinline__ float row_combine(float a, float b) { return OP == ROW_MAX ? fmaxf(a, b) : a + b; }
+
+// y = finish(y_old, s): DOT: beta*y + alpha*s; SQSUM: beta*y + alpha*s; MAX: s.
+template <int OP>
+__device__ __forceinline__ float row_finish(float yold, float s, float alpha, float beta) {
+  if (OP == ROW_MAX) return s;
+  return (beta == 0.f ? 0.f : beta * yold) + alpha * s;
+}
+
+template <bool VEC, int OP>
 __global__ void __launch_bounds__(256)
-k_gemv_rows(const float* M, int ld, int h, int w, int cps, const float* x, float* y, float* partial, float alpha,
-            float beta) {
+k_rows_stage1(const float* M, int ld, int h, int w, int cps, const float* x, float* y, float* partial, float alpha,
+              float beta) {
   constexpr int RPL = VEC ? 4 : 1;
   __shared__ float sv[4][64 * RPL];
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int row0 = (blockIdx.x * 64 + lane) * RPL;
   const int j0 = blockIdx.y * cps;
   const int j1 = (j0 + cps < w) ? j0 + cps : w;
+  const float init = OP == ROW_MAX ? -INFINITY : 0.f;
   float acc[RPL];
 #pragma unroll
-  for (int k = 0; k < RPL; ++k) acc[k] = 0.f;
+  for (int k = 0; k < RPL; ++k) acc[k] = init;
+  auto take = [&](int k, float v, float xj) {
+    if (OP == ROW_DOT) acc[k] += v * xj;
+    else if (OP == ROW_SQSUM) acc[k] += v * v;
+    else acc[k] = v > acc[k] ? v : acc[k];
+  };
   if (row0 < h) {
+    int j = j0 + wv;
     if constexpr (VEC) {
-      for (int j = j0 + wv; j < j1; j += 4) {
+      for (; j + 12 < j1; j += 16) {
+        float4 v[4];
+        float xs[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          v[u] = *reinterpret_cast<const float4*>(M + (size_t)(j + 4 * u) * ld + row0);
+          xs[u] = OP == ROW_DOT ? x[j + 4 * u] : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) { take(0, v[u].x, xs[u]); take(1, v[u].y, xs[u]); take(2, v[u].z, xs[u]); take(3, v[u].w, xs[u]); }
+      }
+      for (; j < j1; j += 4) {
         const float4 v = *reinterpret_cast<const float4*>(M + (size_t)j * ld + row0);
-        const float xj = x[j];
-        acc[0] += v.x * xj; acc[1] += v.y * xj; acc[2] += v.z * xj; acc[3] += v.w * xj;
+        const float xj = OP == ROW_DOT ? x[j] : 0.f;
+        take(0, v.x, xj); take(1, v.y, xj); take(2, v.z, xj); take(3, v.w, xj);
       }
     } else {
-      for (int j = j0 + wv; j < j1; j += 4) acc[0] += M[(size_t)j * ld + row0] * x[j];
+      for (; j + 12 < j1; j += 16) {
+        float v[4], xs[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          v[u] = M[(size_t)(j + 4 * u) * ld + row0];
+          xs[u] = OP == ROW_DOT ? x[j + 4 * u] : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) take(0, v[u], xs[u]);
+      }
+      for (; j < j1; j += 4) take(0, M[(size_t)j * ld + row0], OP == ROW_DOT ? x[j] : 0.f);
     }
   }
 #pragma unroll
   for (int k = 0; k < RPL; ++k) sv[wv][lane * RPL + k] = acc[k];
   __syncthreads();
-  // 256 lanes finish 64*RPL rows.
   for (int r = threadIdx.x; r < 64 * RPL; r += 256) {
     const int row = blockIdx.x * 64 * RPL + r;
     if (row < h) {
-      const float s = (sv[0][r] + sv[1][r]) + (sv[2][r] + sv[3][r]);
+      const float s = row_combine<OP>(row_combine<OP>(sv[0][r], sv[1][r]), row_combine<OP>(sv[2][r], sv[3][r]));
       if (partial) partial[(size_t)blockIdx.y * h + row] = s;
-      else y[row] = (beta == 0.f ? 0.f : beta * y[row]) + alpha * s;
+      else y[row] = row_finish<OP>(y[row], s, alpha, beta);
     }
   }
 }
 
-__global__ void k_gemv_rows_finish(const float* partial, int splits, int h, float* y, float alpha, float beta) {
-  const int row = blockIdx.x * blockDim.x + threadIdx.x;
-  if (row >= h) return;
-  float s = 0.f;
-  for (int k = 0; k < splits; ++k) s += partial[(size_t)k * h + row];
-  y[row] = (beta == 0.f ? 0.f : beta * y[row]) + alpha * s;
+// Stage 2: 64 rows per workgroup; its 4 wavefronts take every 4th split, four
+// loads in flight each, and meet in LDS (the order of the additions is fixed).
+template <int OP>
+__global__ void __launch_bounds__(256)
+k_rows_stage2(const float* partial, int splits, int h, float* y, float alpha, float beta) {
+  __shared__ float sv[4][64];
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int row = blockIdx.x * 64 + lane;
+  float acc = OP == ROW_MAX ? -INFINITY : 0.f;
+  if (row < h) {
+    int k = wv;
+    for (; k + 12 < splits; k += 16) {
+      float v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) v[u] = partial[(size_t)(k + 4 * u) * h + row];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) acc = row_combine<OP>(acc, v[u]);
+    }
+    for (; k < splits; k += 4) acc = row_combine<OP>(acc, partial[(size_t)k * h + row]);
+  }
+  sv[wv][lane] = acc;
+  __syncthreads();
+  if (wv == 0 && row < h) {
+    const float s = row_combine<OP>(row_combine<OP>(sv[0][lane], sv[1][lane]), row_combine<OP>(sv[2][lane], sv[3][lane]));
+    y[row] = row_finish<OP>(y[row], s, alpha, beta);
+  }
+}
+
+template <int OP>
+static int rows_reduce(const float* M, int ld, int h, int w, const float* x, float* y, float alpha, float beta) {
+  if (h <= 0) return 0;
+  const bool vec = dn_aligned16(M) && (ld % 4 == 0) && (h % 4 == 0) && h >= 1024;
+  const int rows_per_block = vec ? 256 : 64;
+  const int bx = (h + rows_per_block - 1) / rows_per_block;
+  int splits = (8 * dn_num_cus()) / bx;
+  if (splits > (w + 63) / 64) splits = (w + 63) / 64;
+  if (splits < 1) splits = 1;
+  int cps = (w + splits - 1) / splits;
+  if (cps < 1) cps = 1;
+  splits = w > 0 ? (w + cps - 1) / cps : 1;
+  float* partial = nullptr;
+  if (splits > 1) {
+    partial = (float*)dn_scratch((size_t)splits * h * sizeof(float));
+    if (!partial) return CUDA_ERROR;
+  }
+  dim3 grid(bx, splits);
+  if (vec)
+    hipLaunchKernelGGL((k_rows_stage1<true, OP>), grid, dim3(256), 0, 0, M, ld, h, w, cps, x, y, partial, alpha, beta);
+  else
+    hipLaunchKernelGGL((k_rows_stage1<false, OP>), grid, dim3(256), 0, 0, M, ld, h, w, cps, x, y, partial, alpha, beta);
+  if (splits > 1)
+    hipLaunchKernelGGL((k_rows_stage2<OP>), dim3((h + 63) / 64), dim3(256), 0, 0, (const float*)partial, splits, h, y,
+                       alpha, beta);
+  return dn_launch_status();
 }
 
 // Host entry points used by dot() for vector-shaped products.
@@ -363,29 +461,7 @@ int dn_gemv_cols(const float* M, int ld, int h, int w, const float* x, float* y,
 }
 
 int dn_gemv_rows(const float* M, int ld, int h, int w, const float* x, float* y, float alpha, float beta) {
-  if (h <= 0) return 0;
-  const bool vec = dn_aligned16(M) && (ld % 4 == 0) && (h % 4 == 0) && h >= 1024;
-  const int rows_per_block = vec ? 256 : 64;
-  const int bx = (h + rows_per_block - 1) / rows_per_block;
-  int splits = (4 * dn_num_cus()) / bx;
-  if (splits > (w + 31) / 32) splits = (w + 31) / 32;
-  if (splits < 1) splits = 1;
-  int cps = (w + splits - 1) / splits;
-  if (cps < 1) cps = 1;
-  splits = w > 0 ? (w + cps - 1) / cps : 1;
-  float* partial = nullptr;
-  if (splits > 1) {
-    partial = (float*)dn_scratch((size_t)splits * h * sizeof(float));
-    if (!partial) return CUDA_ERROR;
-  }
-  dim3 grid(bx, splits);
-  if (vec)
-    hipLaunchKernelGGL((k_gemv_rows<true>), grid, dim3(256), 0, 0, M, ld, h, w, cps, x, y, partial, alpha, beta);
-  else
-    hipLaunchKernelGGL((k_gemv_rows<false>), grid, dim3(256), 0, 0, M, ld, h, w, cps, x, y, partial, alpha, beta);
-  if (splits > 1)
-    hipLaunchKernelGGL(k_gemv_rows_finish, dim3((h + 255) / 256), dim3(256), 0, 0, partial, splits, h, y, alpha, beta);
-  return dn_launch_status();
+  return rows_reduce<ROW_DOT>(M, ld, h, w, x, y, alpha, beta);
 }
 
 // ------------------------------------------------------------------ flat dot / norm
@@ -465,10 +541,8 @@ int max_by_axis(cudamat* mat, cudamat* target, int axis) {
     return launch_cols(k_col_max<64>, k_col_max<256>, w, h, (const float*)mat->data_device, target->data_device, w, h);
   } else if (axis == 1) {
     if (target->size[0] != h || target->size[1] != 1) return ERROR_INCOMPATIBLE_DIMENSIONS;
-    if (h <= 0) return 0;
-    hipLaunchKernelGGL(k_row_reduce, dim3((h + 63) / 64), dim3(256), 0, 0, (const float*)mat->data_device,
-                       target->data_device, w, h, 0, 0.f, 0.f);
-    return dn_launch_status();
+    if (w <= 0) return 0;
+    return rows_reduce<ROW_MAX>(mat->data_device, h, h, w, nullptr, target->data_device, 1.f, 0.f);
   }
   return ERROR_UNSUPPORTED;
 }
@@ -526,10 +600,7 @@ int sqsum_by_axis(cudamat* mat, cudamat* target, int axis, float mult, float p) 
                        w, h, mult, p);
   } else if (axis == 1) {
     if (target->size[0] != h || target->size[1] != 1) return ERROR_INCOMPATIBLE_DIMENSIONS;
-    if (h <= 0) return 0;
-    hipLaunchKernelGGL(k_row_reduce, dim3((h + 63) / 64), dim3(256), 0, 0, (const float*)mat->data_device,
-                       target->data_device, w, h, 3, mult, p);
-    return dn_launch_status();
+    return rows_reduce<ROW_SQSUM>(mat->data_device, h, h, w, nullptr, target->data_device, mult, p);
   }
   return ERROR_UNSUPPORTED;
 }

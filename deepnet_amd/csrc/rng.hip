@@ -9,11 +9,11 @@
 //
 // Two schedules produce that same sequence:
 //   serial  - one lane per stream walks its draws in order (short calls);
-//   split   - a stream's draws are cut into fixed chunks of RNG_CHUNK draws
-//             dealt round-robin to RNG_SPLIT lanes; a lane reaches its next
-//             chunk with one modular multiplication by a per-stream constant,
-//             because one step is a multiplication by (2^32)^-1 modulo
-//             m = mult * 2^32 - 1 (word' * 2^32 = m * lo + word).
+//   split   - a stream's draws are cut into parts of 2^c consecutive draws, one
+//             lane per part.  One step is a multiplication by (2^32)^-1 modulo
+//             m = mult * 2^32 - 1 (word' * 2^32 = m * lo + word), so a lane reaches
+//             its first draw by multiplying the stream's word with per-stream
+//             constants (2^32)^-(2^j) mod m, one per set bit of its part number.
 #include "common.h"
 #include <math.h>
 #include <stdio.h>
@@ -30,53 +30,129 @@ __device__ __forceinline__ float mwc_uniform(unsigned long long w) {
   return ((float)(unsigned int)(w & 0xffffffffull) + 1.0f) * 2.3283064365386963e-10f;
 }
 
-__global__ void k_seed(const unsigned int* mults, unsigned long long* words, unsigned int seed) {
+// Layout of the allocation behind rnd_struct::dev_words (N = 12288 words of 8 bytes):
+// a region aligned to 256 KiB holds two word buffers A (offset 0) and B (offset
+// 128 KiB) and, from offset 256 KiB, the jump table: entry j of stream t multiplies
+// a word by (2^32)^-(2^j) modulo m_t, i.e. jumps 2^j draws ahead.  dev_words points
+// at whichever of A / B holds the current words; the split schedule reads one
+// buffer, writes the other and flips the pointer, so no lane can overwrite a word
+// another lane still has to read.  Bit 17 of the pointer tells the two apart.
+#define RNG_JUMP_BITS 21
+#define RNG_BUF_BYTES (128u << 10)
+#define RNG_REGION_BYTES ((size_t)2 * RNG_BUF_BYTES + (size_t)RNG_JUMP_BITS * NUM_RND_STREAMS * 8)
+
+static inline unsigned long long* rng_other(unsigned long long* w) {
+  return reinterpret_cast<unsigned long long*>(reinterpret_cast<uintptr_t>(w) ^ (uintptr_t)RNG_BUF_BYTES);
+}
+static inline const unsigned long long* rng_table(const unsigned long long* w) {
+  return reinterpret_cast<const unsigned long long*>((reinterpret_cast<uintptr_t>(w) & ~(uintptr_t)(2 * RNG_BUF_BYTES - 1)) +
+                                                     2 * RNG_BUF_BYTES);
+}
+
+// x * y * 2^-64 modulo m = mult * 2^32 - 1, in [0, m).  Dividing by 2^32 modulo m is
+// the generator's own step (v -> mult * lo32(v) + (v >> 32)), applied twice to the
+// 128-bit product; the result is below 2m + 2^32, so two subtractions suffice.
+__device__ __forceinline__ unsigned long long mwc_montmul(unsigned long long x, unsigned long long y,
+                                                          unsigned int mult) {
+  const unsigned long long m = ((unsigned long long)mult << 32) - 1ull;
+  unsigned __int128 v = (unsigned __int128)x * y;
+  v = (v >> 32) + (unsigned __int128)mult * (unsigned int)v;
+  v = (v >> 32) + (unsigned __int128)mult * (unsigned int)v;
+  if (v >= m) v -= m;
+  if (v >= m) v -= m;
+  return (unsigned long long)v;
+}
+
+__global__ void k_seed(const unsigned int* mults, unsigned long long* words, unsigned long long* table,
+                       unsigned int seed) {
   const unsigned int idx = blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= NUM_RND_STREAMS) return;
   unsigned long long w = ((unsigned long long)seed << 32) + 1ull;
   const unsigned int mult = mults[idx];
   for (int i = 0; i < NUM_RND_BURNIN; ++i) w = mwc_step(w, mult);
   words[idx] = w;
+  // Jump table in the form t_j = (2^32)^(2 - 2^j) mod m, so that mwc_montmul(w, t_j)
+  // = w * (2^32)^-(2^j): t_0 = 2^32, t_1 = 1, t_{j+1} = mwc_montmul(t_j, t_j).
+  unsigned long long t = 1ull;
+  table[idx] = 1ull << 32;
+  for (int j = 1; j < RNG_JUMP_BITS; ++j) {
+    table[(size_t)j * NUM_RND_STREAMS + idx] = t;
+    t = mwc_montmul(t, t, mult);
+  }
 }
 
 // ------------------------------------------------------------------ consumers
-// One uniform per element.
+// One uniform per element.  load(i) fetches whatever the element needs from memory
+// and does not depend on the draw, so a lane issues a batch of loads before it
+// walks the serial chain of its stream; store(i, u, x) finishes the element.
 struct OpUniform {
   float* out;
-  __device__ __forceinline__ void operator()(size_t i, float u) const { out[i] = u; }
+  __device__ __forceinline__ float load(size_t) const { return 0.f; }
+  __device__ __forceinline__ void store(size_t i, float u, float) const { out[i] = u; }
 };
 struct OpDropout {
   float* data;
   float p, val;
-  __device__ __forceinline__ void operator()(size_t i, float u) const { data[i] = u > p ? data[i] : val; }
+  __device__ __forceinline__ float load(size_t i) const { return data[i]; }
+  __device__ __forceinline__ void store(size_t i, float u, float x) const { data[i] = u > p ? x : val; }
 };
 struct OpBernoulli {
   const float* in;
   float* out;
-  __device__ __forceinline__ void operator()(size_t i, float u) const { out[i] = u < in[i] ? 1.f : 0.f; }
+  __device__ __forceinline__ float load(size_t i) const { return in[i]; }
+  __device__ __forceinline__ void store(size_t i, float u, float x) const { out[i] = u < x ? 1.f : 0.f; }
 };
 struct OpBernoulliTanh {
   const float* in;
   float* out;
-  __device__ __forceinline__ void operator()(size_t i, float u) const {
-    out[i] = (double)u < (1.0 + (double)in[i]) / 2.0 ? 1.f : 0.f;
+  __device__ __forceinline__ float load(size_t i) const { return in[i]; }
+  __device__ __forceinline__ void store(size_t i, float u, float x) const {
+    out[i] = (double)u < (1.0 + (double)x) / 2.0 ? 1.f : 0.f;
   }
 };
 struct OpCopy {  // sample_poisson of the reference: draws are consumed, data copied
   const float* in;
   float* out;
-  __device__ __forceinline__ void operator()(size_t i, float u) const { (void)u; out[i] = in[i]; }
+  __device__ __forceinline__ float load(size_t i) const { return in[i]; }
+  __device__ __forceinline__ void store(size_t i, float u, float x) const { (void)u; out[i] = x; }
 };
 struct OpPerturbEnergy {
   const float* in;
   float* out;
-  __device__ __forceinline__ void operator()(size_t i, float u) const { out[i] = in[i] - logf(-logf(u)); }
+  __device__ __forceinline__ float load(size_t i) const { return in[i]; }
+  __device__ __forceinline__ void store(size_t i, float u, float x) const { out[i] = x - logf(-logf(u)); }
 };
 struct OpPerturbProb {
   const float* in;
   float* out;
-  __device__ __forceinline__ void operator()(size_t i, float u) const { out[i] = -in[i] / logf(u); }
+  __device__ __forceinline__ float load(size_t i) const { return in[i]; }
+  __device__ __forceinline__ void store(size_t i, float u, float x) const { out[i] = -x / logf(u); }
 };
+
+// Draws [d0, d1) of one stream: element index of draw d is d * 12288 + idx.
+#define RNG_BATCH 8
+template <class Op>
+__device__ __forceinline__ unsigned long long rng_walk(unsigned long long w, unsigned int mult, unsigned int idx,
+                                                       unsigned long long d0, unsigned long long d1, const Op& op) {
+  size_t i = (size_t)d0 * NUM_RND_STREAMS + idx;
+  unsigned long long d = d0;
+  for (; d + RNG_BATCH <= d1; d += RNG_BATCH, i += (size_t)RNG_BATCH * NUM_RND_STREAMS) {
+    float x[RNG_BATCH];
+#pragma unroll
+    for (int k = 0; k < RNG_BATCH; ++k) x[k] = op.load(i + (size_t)k * NUM_RND_STREAMS);
+#pragma unroll
+    for (int k = 0; k < RNG_BATCH; ++k) {
+      w = mwc_step(w, mult);
+      op.store(i + (size_t)k * NUM_RND_STREAMS, mwc_uniform(w), x[k]);
+    }
+  }
+  for (; d < d1; ++d, i += NUM_RND_STREAMS) {
+    const float x = op.load(i);
+    w = mwc_step(w, mult);
+    op.store(i, mwc_uniform(w), x);
+  }
+  return w;
+}
 
 #define RNG_BLOCK 64
 #define RNG_BLOCKS (NUM_RND_STREAMS / RNG_BLOCK)
@@ -85,13 +161,36 @@ template <class Op>
 __global__ void __launch_bounds__(RNG_BLOCK)
 k_rng_serial(const unsigned int* mults, unsigned long long* words, size_t n, Op op) {
   const unsigned int idx = blockIdx.x * RNG_BLOCK + threadIdx.x;
-  unsigned long long w = words[idx];
   const unsigned int mult = mults[idx];
-  for (size_t i = idx; i < n; i += NUM_RND_STREAMS) {
-    w = mwc_step(w, mult);
-    op(i, mwc_uniform(w));
+  const unsigned long long draws = n > idx ? (n - idx + NUM_RND_STREAMS - 1) / NUM_RND_STREAMS : 0;
+  words[idx] = rng_walk(words[idx], mult, idx, 0, draws, op);
+}
+
+// Split schedule: lane (stream s, part p) produces draws [p << chbits, (p+1) << chbits)
+// of its stream, reaching its first draw with one jump per set bit of p.  The lane
+// that produces a stream's last draw writes the new word into the other buffer.
+#define RNG_SPLIT_BLOCK 256
+template <class Op>
+__global__ void __launch_bounds__(RNG_SPLIT_BLOCK)
+k_rng_split(const unsigned int* mults, const unsigned long long* words, unsigned long long* next,
+            const unsigned long long* table, size_t n, int chbits, Op op) {
+  constexpr int blocks_per_part = NUM_RND_STREAMS / RNG_SPLIT_BLOCK;
+  const unsigned int part = blockIdx.x / blocks_per_part;
+  const unsigned int idx = (blockIdx.x % blocks_per_part) * RNG_SPLIT_BLOCK + threadIdx.x;
+  if (idx >= n) {  // a stream without draws keeps its word
+    if (part == 0) next[idx] = words[idx];
+    return;
   }
-  words[idx] = w;
+  const unsigned long long draws = (n - idx + NUM_RND_STREAMS - 1) / NUM_RND_STREAMS;  // of this stream
+  const unsigned long long d0 = (unsigned long long)part << chbits;
+  if (d0 >= draws) return;
+  const unsigned long long d1 = d0 + (1ull << chbits) < draws ? d0 + (1ull << chbits) : draws;
+  const unsigned int mult = mults[idx];
+  unsigned long long w = words[idx];
+  for (unsigned int b = 0, pp = part; pp; ++b, pp >>= 1)
+    if (pp & 1u) w = mwc_montmul(w, table[(size_t)(chbits + b) * NUM_RND_STREAMS + idx], mult);
+  w = rng_walk(w, mult, idx, d0, d1, op);
+  if (d1 == draws) next[idx] = w;
 }
 
 // Box-Muller pairs: two draws give elements i and i + 12288 (cudamat_kernels.cu:125-143, 192-211).
@@ -115,9 +214,36 @@ k_rng_gauss(const unsigned int* mults, unsigned long long* words, const float* i
   words[idx] = w;
 }
 
+// Calls with at least RNG_SPLIT_MIN_DRAWS draws per stream are cut into about
+// RNG_SPLIT_PARTS parts per stream (chunk length a power of two, at least 16).
+#define RNG_SPLIT_MIN_DRAWS 32
+#define RNG_SPLIT_PARTS 24
+
 template <class Op>
 static int launch_rng(rnd_struct* st, size_t n, Op op) {
-  hipLaunchKernelGGL((k_rng_serial<Op>), dim3(RNG_BLOCKS), dim3(RNG_BLOCK), 0, 0, st->dev_mults, st->dev_words, n, op);
+  if (n == 0) return 0;
+  const size_t draws = (n + NUM_RND_STREAMS - 1) / NUM_RND_STREAMS;
+  if (draws < RNG_SPLIT_MIN_DRAWS) {
+    hipLaunchKernelGGL((k_rng_serial<Op>), dim3(RNG_BLOCKS), dim3(RNG_BLOCK), 0, 0, st->dev_mults, st->dev_words, n,
+                       op);
+    return dn_launch_status();
+  }
+  int chbits = 4;
+  while (((draws + (1ull << chbits) - 1) >> chbits) > RNG_SPLIT_PARTS) ++chbits;
+  const size_t parts = (draws + (1ull << chbits) - 1) >> chbits;
+  // every jump exponent (chbits + bit of part) must be inside the table
+  int top = 0;
+  while ((parts - 1) >> top) ++top;
+  if (chbits + top > RNG_JUMP_BITS) {
+    hipLaunchKernelGGL((k_rng_serial<Op>), dim3(RNG_BLOCKS), dim3(RNG_BLOCK), 0, 0, st->dev_mults, st->dev_words, n,
+                       op);
+    return dn_launch_status();
+  }
+  const unsigned grid = (unsigned)(parts * (NUM_RND_STREAMS / RNG_SPLIT_BLOCK));
+  unsigned long long* next = rng_other(st->dev_words);
+  hipLaunchKernelGGL((k_rng_split<Op>), dim3(grid), dim3(RNG_SPLIT_BLOCK), 0, 0, st->dev_mults,
+                     (const unsigned long long*)st->dev_words, next, rng_table(st->dev_words), n, chbits, op);
+  st->dev_words = next;
   return dn_launch_status();
 }
 
@@ -137,16 +263,18 @@ int init_random(rnd_struct* rnd_state, int seed, char* cudamatpath) {
   }
   void *dm = nullptr, *dw = nullptr;
   if (hipMalloc(&dm, NUM_RND_STREAMS * sizeof(unsigned int)) != hipSuccess ||
-      hipMalloc(&dw, NUM_RND_STREAMS * sizeof(unsigned long long)) != hipSuccess ||
+      hipMalloc(&dw, RNG_REGION_BYTES + 2 * RNG_BUF_BYTES) != hipSuccess ||
       hipMemcpy(dm, host_mults, NUM_RND_STREAMS * sizeof(unsigned int), hipMemcpyHostToDevice) != hipSuccess) {
     free(host_mults);
     return CUDA_ERROR;
   }
   free(host_mults);
   rnd_state->dev_mults = (unsigned int*)dm;
-  rnd_state->dev_words = (unsigned long long*)dw;
+  // align the region to 256 KiB inside the (never freed, as in the reference) allocation
+  const uintptr_t base = (reinterpret_cast<uintptr_t>(dw) + 2 * RNG_BUF_BYTES - 1) & ~(uintptr_t)(2 * RNG_BUF_BYTES - 1);
+  rnd_state->dev_words = reinterpret_cast<unsigned long long*>(base);
   hipLaunchKernelGGL(k_seed, dim3(RNG_BLOCKS), dim3(RNG_BLOCK), 0, 0, rnd_state->dev_mults, rnd_state->dev_words,
-                     (unsigned int)seed);
+                     const_cast<unsigned long long*>(rng_table(rnd_state->dev_words)), (unsigned int)seed);
   return dn_launch_status();
 }
 

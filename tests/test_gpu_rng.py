@@ -35,7 +35,8 @@ def test_seed_state_matches_host(cm, mults, seed):
     assert np.array_equal(_device_words(cm), host.words)
 
 
-@pytest.mark.parametrize("shape", [(1, 1), (100, 5), (96, 128), (500, 100), (3 * N + 5, 1), (1031, 257)])
+@pytest.mark.parametrize("shape", [(1, 1), (100, 5), (96, 128), (500, 100), (3 * N + 5, 1), (1031, 257),
+                                   (33 * N + 7, 1), (31 * N + 12287, 1), (32 * N, 1), (200 * N + 4097, 1), (2049, 1537)])
 def test_fill_with_rand_bit_exact_and_state_carries_over(cm, mults, shape):
     cm.CUDAMatrix.init_random(42)
     host = mwc.MWC(mults, 42)
