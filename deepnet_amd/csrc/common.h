@@ -9,8 +9,8 @@
 // One CU count for launch sizing; MI355X has 256 CUs in 8 XCDs.  Queried once.
 int dn_num_cus();
 
-// Grow-only device workspace shared by the two-stage kernels (partials + results).
-void* dn_scratch(size_t bytes);
+// Grow-only device workspaces (slot 0: partials and scalar results; slot 1: conv patch matrix).
+void* dn_scratch(size_t bytes, int slot = 0);
 
 // Records the launch status of the kernel just queued; returns CUDA_ERROR or 0.
 static inline int dn_launch_status() {
@@ -85,6 +85,19 @@ __device__ __forceinline__ void dn_st4(float* p, float4 r) {
   } else {
     *reinterpret_cast<float4*>(p) = r;
   }
+}
+// Run-time selected variants (the flag is uniform across the launch).
+__device__ __forceinline__ float4 dn_ld4_rt(const float* p, bool stream) {
+  return stream ? dn_ld4<true>(p) : dn_ld4<false>(p);
+}
+__device__ __forceinline__ void dn_st4_rt(float* p, float4 r, bool stream) {
+  if (stream) dn_st4<true>(p, r); else dn_st4<false>(p, r);
+}
+__device__ __forceinline__ float dn_ld1_rt(const float* p, bool stream) {
+  return stream ? __builtin_nontemporal_load(p) : *p;
+}
+__device__ __forceinline__ void dn_st1_rt(float* p, float v, bool stream) {
+  if (stream) __builtin_nontemporal_store(v, p); else *p = v;
 }
 // Operands of at least this many elements are streamed.
 #define DN_STREAM_MIN_ELEMS (1ll << 22)

@@ -42,6 +42,7 @@ struct ConvArgs {
   int M, HH, kk2;     // Mx*Mx, H*H, k*k
   int m_begin, m_count;  // Outp: module chunk [m_begin, m_begin + m_count)
   int splits, slabs_per_split;
+  int local;          // 1: one filter bank per module (locally connected layers); direct kernels only
   float scale_t, scale_o;
   FastDiv dN, dMx, dk, dkk2;
 };
@@ -59,6 +60,7 @@ __global__ void k_conv_up_direct(ConvArgs p) {
     const int f = (int)(e / ((long long)p.N * p.M));
     const int g = f / p.Fg;
     const int y0 = (m / p.Mx) * p.s + p.pad0, x0 = (m % p.Mx) * p.s + p.pad0;
+    const float* flt = p.flt + (p.local ? (size_t)m * p.Cg * p.kk2 * p.F : 0);
     float acc = 0.f;
     for (int c = 0; c < p.Cg; ++c)
       for (int ky = 0; ky < p.k; ++ky) {
@@ -68,7 +70,7 @@ __global__ void k_conv_up_direct(ConvArgs p) {
           const int x = x0 + kx;
           if (x < 0 || x >= p.H) continue;
           acc += p.img[(size_t)p.N * ((size_t)(g * p.Cg + c) * p.HH + y * p.H + x) + n] *
-                 p.flt[(size_t)p.F * ((c * p.k + ky) * p.k + kx) + f];
+                 flt[(size_t)p.F * ((c * p.k + ky) * p.k + kx) + f];
         }
       }
     p.out[e] = (p.scale_t == 0.f ? 0.f : p.scale_t * p.out[e]) + p.scale_o * acc;
@@ -91,7 +93,8 @@ __global__ void k_conv_down_direct(ConvArgs p) {
       for (int mx = 0; mx < p.Mx; ++mx) {
         const int kx = x - mx * p.s;
         if (kx < 0 || kx >= p.k) continue;
-        const size_t wbase = (size_t)p.F * ((cl * p.k + ky) * p.k + kx);
+        const size_t wbase = (size_t)p.F * ((cl * p.k + ky) * p.k + kx) +
+                             (p.local ? (size_t)(my * p.Mx + mx) * p.Cg * p.kk2 * p.F : 0);
         for (int fl = 0; fl < p.Fg; ++fl) {
           const int f = g * p.Fg + fl;
           acc += p.hid[(size_t)p.N * ((size_t)f * p.M + my * p.Mx + mx) + n] * p.flt[wbase + f];
@@ -421,17 +424,79 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
   }
 }
 
-// dW(f, q) = scale_t*dW + scale_o * sum over splits of partial[z][g][q][fl]
-__global__ void k_conv_outp_finish(ConvArgs p) {
+// dW(f, q) = scale_t*dW + scale_o * sum over splits of partial[z][g][q][fl].
+// 64 outputs per workgroup; its 4 wavefronts take every 4th split, four loads in
+// flight each, and meet in LDS (fixed order of additions).
+__global__ void __launch_bounds__(256) k_conv_outp_finish(ConvArgs p) {
+  __shared__ float sv[4][64];
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int per_group = p.Fg * p.Cg * p.kk2;
   const int total = p.G * per_group;
-  for (int e = blockIdx.x * blockDim.x + threadIdx.x; e < total; e += gridDim.x * blockDim.x) {
-    float sum = 0.f;
-    for (int z = 0; z < p.splits; ++z) sum += p.partial[(size_t)z * total + e];
+  const int e = blockIdx.x * 64 + lane;
+  float acc = 0.f;
+  if (e < total) {
+    int z = wv;
+    for (; z + 12 < p.splits; z += 16) {
+      float v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) v[u] = p.partial[(size_t)(z + 4 * u) * total + e];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) acc += v[u];
+    }
+    for (; z < p.splits; z += 4) acc += p.partial[(size_t)z * total + e];
+  }
+  sv[wv][lane] = acc;
+  __syncthreads();
+  if (wv == 0 && e < total) {
+    const float sum = (sv[0][lane] + sv[1][lane]) + (sv[2][lane] + sv[3][lane]);
     const int g = e / per_group, rem = e - g * per_group;
     const int q = rem / p.Fg, fl = rem - q * p.Fg;
     float* t = p.out + (size_t)p.F * q + g * p.Fg + fl;
     *t = (p.scale_t == 0.f ? 0.f : p.scale_t * *t) + p.scale_o * sum;
+  }
+}
+
+// ------------------------------------------------------------------ convDown through a patch matrix
+// With few colours per group the implicit GEMM above has only Cg useful columns
+// in a 32-wide matrix-core block and re-reads the hidden activations once per
+// filter tap.  Instead: P = hid (M*N x Fg, read once) * W (Fg x Cg*k*k) is a plain
+// product on the buffers as they are (hid is column-major with leading dimension
+// M*N), and every image pixel then gathers the <= ceil(k/s)^2 entries of P that
+// land on it.  P(r, q) with r = module*N + image, q = (c*k + ky)*k + kx.
+int dn_gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, const float* A, int lda, const float* B,
+            int ldb, float beta, float* C, int ldc);
+
+__global__ void __launch_bounds__(256) k_conv_down_gather(ConvArgs p, const float* P, int g) {
+  // one lane: 4 neighbouring images of one (colour of the group, y, x)
+  const int NV = p.N >> 2;
+  const uint32_t total = (uint32_t)NV * p.HH * p.Cg;
+  const long long ldp = (long long)p.M * p.N;
+  for (uint32_t e = blockIdx.x * 256u + threadIdx.x; e < total; e += gridDim.x * 256u) {
+    const uint32_t nv = e % NV;
+    const uint32_t pix = (e / NV) % p.HH;
+    const int c = (int)(e / ((uint32_t)NV * p.HH));
+    const int y = (int)(pix / p.H) - p.pad0, x = (int)(pix % p.H) - p.pad0;  // padded-frame coordinates
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    // modules my with 0 <= y - my*s < k
+    const int my_hi = y / p.s < p.Mx - 1 ? y / p.s : p.Mx - 1;
+    const int mx_hi = x / p.s < p.Mx - 1 ? x / p.s : p.Mx - 1;
+    for (int my = my_hi; my >= 0 && y - my * p.s < p.k; --my) {
+      const int ky = y - my * p.s;
+      for (int mx = mx_hi; mx >= 0 && x - mx * p.s < p.k; --mx) {
+        const int kx = x - mx * p.s;
+        const long long q = (long long)(c * p.k + ky) * p.k + kx;
+        const float4 v = *reinterpret_cast<const float4*>(P + q * ldp + (long long)(my * p.Mx + mx) * p.N + 4 * nv);
+        acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+      }
+    }
+    float* t = p.out + (size_t)p.N * ((size_t)(g * p.Cg + c) * p.HH + pix) + 4 * nv;
+    float4 r = acc;
+    if (p.scale_t != 0.f || p.scale_o != 1.f) {
+      const float4 o = p.scale_t == 0.f ? make_float4(0.f, 0.f, 0.f, 0.f) : *reinterpret_cast<const float4*>(t);
+      r = make_float4(p.scale_t * o.x + p.scale_o * acc.x, p.scale_t * o.y + p.scale_o * acc.y,
+                      p.scale_t * o.z + p.scale_o * acc.z, p.scale_t * o.w + p.scale_o * acc.w);
+    }
+    *reinterpret_cast<float4*>(t) = r;
   }
 }
 
@@ -468,7 +533,7 @@ static bool fast_ok(const ConvArgs& a) {
 static void fill_common(ConvArgs& a, int N, int C, int G, int H, int F, int k, int Mx, int s, int pad0) {
   a.N = N; a.C = C; a.G = G; a.Cg = C / G; a.H = H; a.F = F; a.Fg = F / G; a.k = k; a.Mx = Mx; a.s = s; a.pad0 = pad0;
   a.M = Mx * Mx; a.HH = H * H; a.kk2 = k * k;
-  a.m_begin = 0; a.m_count = a.M; a.splits = 1; a.slabs_per_split = 0;
+  a.m_begin = 0; a.m_count = a.M; a.splits = 1; a.slabs_per_split = 0; a.local = 0;
   a.scale_t = 0.f; a.scale_o = 1.f; a.partial = nullptr;
   a.dN = make_fastdiv((uint32_t)N); a.dMx = make_fastdiv((uint32_t)Mx);
   a.dk = make_fastdiv((uint32_t)k); a.dkk2 = make_fastdiv((uint32_t)(k * k));
@@ -485,7 +550,7 @@ static void launch_rowmajor(const ConvArgs& a, long long rows, int cols, int gz)
 }
 
 static void conv_up_impl(cudamat* images, cudamat* filters, cudamat* targets, int numModulesX, int paddingStart,
-                         int moduleStride, int numImgColors, int numGroups, const char* where) {
+                         int moduleStride, int numImgColors, int numGroups, const char* where, bool local = false) {
   conv_clear_error();
   CONV_REQUIRE(images->on_device && filters->on_device && targets->on_device, where);
   CONV_REQUIRE(numGroups >= 1 && numImgColors > 0 && numImgColors % numGroups == 0, where);
@@ -496,17 +561,19 @@ static void conv_up_impl(cudamat* images, cudamat* filters, cudamat* targets, in
   const int H = isqrt_exact(images->size[1] / numImgColors);
   CONV_REQUIRE(H > 0, where);
   const int Cg = numImgColors / numGroups;
-  CONV_REQUIRE(filters->size[1] % Cg == 0, where);
-  const int k = isqrt_exact(filters->size[1] / Cg);
-  CONV_REQUIRE(k > 0, where);
   const int M = numModulesX * numModulesX;
+  const int fmm = local ? M : 1;  // filter banks
+  CONV_REQUIRE(filters->size[1] % (Cg * fmm) == 0, where);
+  const int k = isqrt_exact(filters->size[1] / (Cg * fmm));
+  CONV_REQUIRE(k > 0, where);
   CONV_REQUIRE(paddingStart <= 0, where);
   CONV_REQUIRE(moduleStride <= k, where);
   CONV_REQUIRE(targets->size[0] == N && targets->size[1] == F * M, where);
   ConvArgs a;
   fill_common(a, N, numImgColors, numGroups, H, F, k, numModulesX, moduleStride, paddingStart);
   a.img = images->data_device; a.flt = filters->data_device; a.hid = nullptr; a.out = targets->data_device;
-  if (fast_ok(a)) {
+  a.local = local ? 1 : 0;
+  if (!local && fast_ok(a)) {
     launch_rowmajor<CONV_UP>(a, (long long)M * N, a.Fg, numGroups);
   } else {
     const long long total = (long long)N * M * F;
@@ -518,7 +585,7 @@ static void conv_up_impl(cudamat* images, cudamat* filters, cudamat* targets, in
 }
 
 static void conv_down_impl(cudamat* hidActs, cudamat* filters, cudamat* targets, int imgSize, int paddingStart,
-                           int moduleStride, int numImgColors, int numGroups, const char* where) {
+                           int moduleStride, int numImgColors, int numGroups, const char* where, bool local = false) {
   conv_clear_error();
   CONV_REQUIRE(hidActs->on_device && filters->on_device && targets->on_device, where);
   CONV_REQUIRE(numGroups >= 1 && numImgColors > 0 && numImgColors % numGroups == 0, where);
@@ -530,8 +597,9 @@ static void conv_down_impl(cudamat* hidActs, cudamat* filters, cudamat* targets,
   const int Mx = isqrt_exact(M);
   CONV_REQUIRE(Mx > 0, where);
   const int Cg = numImgColors / numGroups;
-  CONV_REQUIRE(filters->size[1] % Cg == 0, where);
-  const int k = isqrt_exact(filters->size[1] / Cg);
+  const int fmm = local ? M : 1;
+  CONV_REQUIRE(filters->size[1] % (Cg * fmm) == 0, where);
+  const int k = isqrt_exact(filters->size[1] / (Cg * fmm));
   CONV_REQUIRE(k > 0, where);
   CONV_REQUIRE(paddingStart <= 0 && moduleStride <= k, where);
   CONV_REQUIRE(targets->size[0] == N && targets->size[1] == numImgColors * imgSize * imgSize, where);
@@ -539,7 +607,25 @@ static void conv_down_impl(cudamat* hidActs, cudamat* filters, cudamat* targets,
   fill_common(a, N, numImgColors, numGroups, imgSize, F, k, Mx, moduleStride, paddingStart);
   a.img = nullptr; a.flt = filters->data_device; a.hid = hidActs->data_device; a.out = targets->data_device;
   a.img = a.hid;  // alignment test only
-  if (fast_ok(a) && dn_aligned16(a.out)) {
+  a.local = local ? 1 : 0;
+  if (!local && fast_ok(a) && dn_aligned16(a.out) && a.Cg <= 16) {
+    // few colours: patch-matrix form
+    const long long prow = (long long)a.M * N;
+    const int pcols = a.Cg * a.kk2;
+    float* P = (float*)dn_scratch((size_t)prow * pcols * sizeof(float), 1);
+    if (!P) { conv_set_error(where, "out of device memory for the patch matrix"); return; }
+    for (int g = 0; g < numGroups; ++g) {
+      if (dn_gemm(false, false, (int)prow, pcols, a.Fg, 1.f, a.hid + (size_t)g * a.Fg * prow, (int)prow,
+                  a.flt + (size_t)g * a.Fg, F, 0.f, P, (int)prow)) {
+        conv_set_error(where, "patch product failed");
+        return;
+      }
+      const long long lanes = (long long)(N / 4) * a.HH * a.Cg;
+      long long blocks = (lanes + 255) / 256;
+      if (blocks > dn_num_cus() * 64ll) blocks = dn_num_cus() * 64ll;
+      hipLaunchKernelGGL(k_conv_down_gather, dim3((unsigned)blocks), dim3(256), 0, 0, a, (const float*)P, g);
+    }
+  } else if (!local && fast_ok(a) && dn_aligned16(a.out)) {
     const int q = (imgSize + moduleStride - 1) / moduleStride;
     launch_rowmajor<CONV_DOWN>(a, (long long)q * q * N, a.Cg, numGroups * moduleStride * moduleStride);
   } else {
@@ -587,10 +673,11 @@ static void conv_outp_impl(cudamat* images, cudamat* hidActs, cudamat* targets, 
       const int BMs = Fg <= 32 ? 32 : Fg <= 64 ? 64 : Fg <= 96 ? 96 : 128;
       const int gx = (Fg + BMs - 1) / BMs, gy = (cols + 127) / 128;
       const int nslabs = a.m_count * (N / CV_BK);
-      long long want = (4ll * dn_num_cus()) / ((long long)gx * gy * numGroups);
+      // about two workgroups per CU, at least 16 slabs (256 of the reduction) per split
+      long long want = (2ll * dn_num_cus()) / ((long long)gx * gy * numGroups);
       if (want < 1) want = 1;
-      if (want > nslabs / 8) want = nslabs / 8 > 0 ? nslabs / 8 : 1;
-      if (want > 1024) want = 1024;
+      if (want > nslabs / 16) want = nslabs / 16 > 0 ? nslabs / 16 : 1;
+      if (want > 512) want = 512;
       a.slabs_per_split = (int)((nslabs + want - 1) / want);
       a.splits = (nslabs + a.slabs_per_split - 1) / a.slabs_per_split;
       a.partial = (float*)dn_scratch((size_t)a.splits * F * cols * sizeof(float));
@@ -601,7 +688,7 @@ static void conv_outp_impl(cudamat* images, cudamat* hidActs, cudamat* targets, 
       else if (BMs == 96) hipLaunchKernelGGL((k_conv_mfma<CONV_OUTP, 1, 3, 1>), grid, dim3(256), 0, 0, a);
       else hipLaunchKernelGGL((k_conv_mfma<CONV_OUTP, 2, 2, 2>), grid, dim3(256), 0, 0, a);
       const int total = F * cols;
-      hipLaunchKernelGGL(k_conv_outp_finish, dim3((total + 255) / 256), dim3(256), 0, 0, a);
+      hipLaunchKernelGGL(k_conv_outp_finish, dim3((total + 63) / 64), dim3(256), 0, 0, a);
     } else {
       hipLaunchKernelGGL(k_conv_outp_direct, dim3((unsigned)(F * cols)), dim3(256), 0, 0, a);
     }
@@ -629,15 +716,25 @@ void convOutp(cudamat* images, cudamat* hidActs, cudamat* targets, int numModule
                  numGroups, partialSum, "convOutp");
 }
 
-// Locally connected layers (one filter bank per module) are not built yet.
-void localUp(cudamat*, cudamat*, cudamat*, int, int, int, int, int) {
-  conv_set_error("localUp", "locally connected layers are not implemented");
+// Locally connected layers: one filter bank per module, filters laid out
+// (module, colour, ky, kx, filter) (cudamat_conv_kernels.cuh:66-67).  They run on the
+// one-lane-per-output kernels; the weight gradient is convOutp with one module per
+// chunk, which is how the reference computes it too (cudamat_conv.cu:1421-1423).
+void localUp(cudamat* images, cudamat* filters, cudamat* targets, int numModulesX, int paddingStart, int moduleStride,
+             int numImgColors, int numGroups) {
+  conv_up_impl(images, filters, targets, numModulesX, paddingStart, moduleStride, numImgColors, numGroups, "localUp",
+               true);
 }
-void localDown(cudamat*, cudamat*, cudamat*, int, int, int, int, int) {
-  conv_set_error("localDown", "locally connected layers are not implemented");
+void localDown(cudamat* hidActs, cudamat* filters, cudamat* targets, int imgSize, int paddingStart, int moduleStride,
+               int numImgColors, int numGroups) {
+  conv_down_impl(hidActs, filters, targets, imgSize, paddingStart, moduleStride, numImgColors, numGroups, "localDown",
+                 true);
 }
-void localOutp(cudamat*, cudamat*, cudamat*, int, int, int, int, int, int, int) {
-  conv_set_error("localOutp", "locally connected layers are not implemented");
+void localOutp(cudamat* images, cudamat* hidActs, cudamat* targets, int numModulesX, int filterSize, int paddingStart,
+               int moduleStride, int numImgColors, int numGroups, int partialSum) {
+  (void)partialSum;
+  conv_outp_impl(images, hidActs, targets, numModulesX, filterSize, paddingStart, moduleStride, numImgColors,
+                 numGroups, 1, "localOutp");
 }
 
 }  // extern "C"

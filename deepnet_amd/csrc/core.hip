@@ -20,26 +20,28 @@ int dn_num_cus() {
 }
 
 // ------------------------------------------------------------------ scratch
-// Grow-only device workspace for two-stage reductions (partials + result).
-static void* g_scratch = nullptr;
-static size_t g_scratch_bytes = 0;
+// Grow-only device workspaces.  Slot 0: partials of two-stage reductions and
+// split-K products, scalar results.  Slot 1: the patch matrix of the col2im
+// form of convDown (it is live while a product that may use slot 0 runs).
+static void* g_scratch[2] = {nullptr, nullptr};
+static size_t g_scratch_bytes[2] = {0, 0};
 
-void* dn_scratch(size_t bytes) {
-  if (bytes > g_scratch_bytes) {
-    if (g_scratch) {
+void* dn_scratch(size_t bytes, int slot) {
+  if (bytes > g_scratch_bytes[slot]) {
+    if (g_scratch[slot]) {
       hipDeviceSynchronize();
-      hipFree(g_scratch);
+      hipFree(g_scratch[slot]);
     }
     size_t want = bytes < (1u << 20) ? (1u << 20) : bytes;
-    if (hipMalloc(&g_scratch, want) != hipSuccess) {
-      g_scratch = nullptr;
-      g_scratch_bytes = 0;
+    if (hipMalloc(&g_scratch[slot], want) != hipSuccess) {
+      g_scratch[slot] = nullptr;
+      g_scratch_bytes[slot] = 0;
       hipGetLastError();
       return nullptr;
     }
-    g_scratch_bytes = want;
+    g_scratch_bytes[slot] = want;
   }
-  return g_scratch;
+  return g_scratch[slot];
 }
 
 // ------------------------------------------------------------------ kernels

@@ -12,7 +12,6 @@
 
 int dn_gemv_cols(const float* M, int ld, int h, int w, const float* x, float* y, float alpha, float beta);
 int dn_gemv_rows(const float* M, int ld, int h, int w, const float* x, float* y, float alpha, float beta);
-void* dn_scratch(size_t bytes);
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
@@ -253,6 +252,12 @@ static int gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, co
     hipLaunchKernelGGL(k_gemm_splitk_finish, dim3(blocks), dim3(256), 0, 0, partial, splits, C, ldc, M, N, alpha, beta);
   }
   return dn_launch_status();
+}
+
+// C = beta*C + alpha*op(A)*op(B) on raw column-major buffers, for the other kernels of the library.
+int dn_gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, const float* A, int lda, const float* B,
+            int ldb, float beta, float* C, int ldc) {
+  return gemm(a_trans, b_trans, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc);
 }
 
 extern "C" {

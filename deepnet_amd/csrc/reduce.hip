@@ -12,14 +12,13 @@
 #include <float.h>
 #include <math.h>
 
-void* dn_scratch(size_t bytes);
 
 // ------------------------------------------------------------------ column walkers
 
 // Visit every element of one column with TPC cooperating lanes: fn(row, value).
 // Four 16-byte loads are issued before any of them is consumed.
 template <int TPC, class Fn>
-__device__ __forceinline__ void for_each_in_col(const float* c, int h, int lane, Fn fn) {
+__device__ __forceinline__ void for_each_in_col(const float* c, int h, int lane, Fn fn, bool stream = false) {
   int head = (int)(((16u - (unsigned)(reinterpret_cast<uintptr_t>(c) & 15u)) & 15u) >> 2);
   if (head > h) head = h;
   if (lane < head) fn(lane, c[lane]);
@@ -29,7 +28,7 @@ __device__ __forceinline__ void for_each_in_col(const float* c, int h, int lane,
   for (; j + 3 * TPC < n4; j += 4 * TPC) {
     float4 v[4];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) v[u] = c4[j + u * TPC];
+    for (int u = 0; u < 4; ++u) v[u] = dn_ld4_rt(reinterpret_cast<const float*>(c4 + j + u * TPC), stream);
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int b = head + 4 * (j + u * TPC);
@@ -37,7 +36,7 @@ __device__ __forceinline__ void for_each_in_col(const float* c, int h, int lane,
     }
   }
   for (; j < n4; j += TPC) {
-    const float4 v = c4[j];
+    const float4 v = dn_ld4_rt(reinterpret_cast<const float*>(c4 + j), stream);
     const int b = head + 4 * j;
     fn(b, v.x); fn(b + 1, v.y); fn(b + 2, v.z); fn(b + 3, v.w);
   }
@@ -109,8 +108,9 @@ template <int TPC>
 __global__ void __launch_bounds__(256) k_col_max(const float* mat, float* target, int w, int h) {
   __shared__ float lds4[4];
   COL_SETUP(TPC)
+  const bool stream = (long long)w * h >= DN_STREAM_MIN_ELEMS;
   float m = -FLT_MAX;
-  if (active) for_each_in_col<TPC>(mat + (size_t)col * h, h, lane, [&](int, float v) { if (v > m) m = v; });
+  if (active) for_each_in_col<TPC>(mat + (size_t)col * h, h, lane, [&](int, float v) { if (v > m) m = v; }, stream);
   m = col_combine<TPC, true>(m, lds4);
   if (active && lane == 0) target[col] = m;
 }
@@ -143,8 +143,9 @@ template <int TPC>
 __global__ void __launch_bounds__(256) k_col_sqsum(const float* mat, float* target, int w, int h, float mult, float p) {
   __shared__ float lds4[4];
   COL_SETUP(TPC)
+  const bool stream = (long long)w * h >= DN_STREAM_MIN_ELEMS;
   float s = 0.f;
-  if (active) for_each_in_col<TPC>(mat + (size_t)col * h, h, lane, [&](int, float v) { s += v * v; });
+  if (active) for_each_in_col<TPC>(mat + (size_t)col * h, h, lane, [&](int, float v) { s += v * v; }, stream);
   s = col_combine<TPC, false>(s, lds4);
   // p == 0 overwrites: the previous contents (possibly uninitialised) are not read.
   if (active && lane == 0) target[col] = (p == 0.f ? 0.f : p * target[col]) + mult * s;
@@ -190,16 +191,17 @@ __global__ void __launch_bounds__(256) k_col_softmax_reg(const float* mat, float
   const int col = blockIdx.x * 4 + (int)(threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   if (col >= w) return;
-  const float4* c4 = reinterpret_cast<const float4*>(mat + (size_t)col * h);
-  float4* t4 = reinterpret_cast<float4*>(target + (size_t)col * h);
+  const float* c4 = mat + (size_t)col * h;
+  float* t4 = target + (size_t)col * h;
   const int n4 = h >> 2;
+  const bool stream = (long long)w * h >= DN_STREAM_MIN_ELEMS;
   float4 v[NV];
   float m = -FLT_MAX;
 #pragma unroll
   for (int k = 0; k < NV; ++k) {
     const int j = lane + k * 64;
     if (j < n4) {
-      v[k] = c4[j];
+      v[k] = dn_ld4_rt(c4 + 4 * j, stream);
       m = fmaxf(m, fmaxf(fmaxf(v[k].x, v[k].y), fmaxf(v[k].z, v[k].w)));
     }
   }
@@ -218,7 +220,7 @@ __global__ void __launch_bounds__(256) k_col_softmax_reg(const float* mat, float
 #pragma unroll
   for (int k = 0; k < NV; ++k) {
     const int j = lane + k * 64;
-    if (j < n4) t4[j] = make_float4(v[k].x / s, v[k].y / s, v[k].z / s, v[k].w / s);
+    if (j < n4) dn_st4_rt(t4 + 4 * j, make_float4(v[k].x / s, v[k].y / s, v[k].z / s, v[k].w / s), stream);
   }
 }
 
@@ -303,8 +305,9 @@ __global__ void __launch_bounds__(256)
 k_gemv_cols(const float* M, int ld, int h, int w, const float* x, float* y, float alpha, float beta) {
   __shared__ float lds4[4];
   COL_SETUP(TPC)
+  const bool stream = (long long)w * h >= DN_STREAM_MIN_ELEMS;
   float s = 0.f;
-  if (active) for_each_in_col<TPC>(M + (size_t)col * ld, h, lane, [&](int r, float v) { s += v * x[r]; });
+  if (active) for_each_in_col<TPC>(M + (size_t)col * ld, h, lane, [&](int r, float v) { s += v * x[r]; }, stream);
   s = col_combine<TPC, false>(s, lds4);
   if (active && lane == 0) y[col] = (beta == 0.f ? 0.f : beta * y[col]) + alpha * s;
 }
@@ -316,6 +319,7 @@ k_gemv_cols(const float* M, int ld, int h, int w, const float* x, float* y, floa
 // or 64*bx .. 64*bx+63 otherwise; its 4 wavefronts take every 4th column, four
 // loads in flight each, and meet in LDS.  With one split the result is final.
 enum { ROW_DOT = 0, ROW_SQSUM = 1, ROW_MAX = 2 };
+
 
 template <int OP>
 __device__ __forceinline__ float row_combine(float a, float b) { return OP == ROW_MAX ? fmaxf(a, b) : a + b; }
@@ -338,6 +342,7 @@ k_rows_stage1(const float* M, int ld, int h, int w, int cps, const float* x, flo
   const int j0 = blockIdx.y * cps;
   const int j1 = (j0 + cps < w) ? j0 + cps : w;
   const float init = OP == ROW_MAX ? -INFINITY : 0.f;
+  const bool stream = (long long)w * h >= DN_STREAM_MIN_ELEMS;
   float acc[RPL];
 #pragma unroll
   for (int k = 0; k < RPL; ++k) acc[k] = init;
@@ -354,14 +359,14 @@ k_rows_stage1(const float* M, int ld, int h, int w, int cps, const float* x, flo
         float xs[4];
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-          v[u] = *reinterpret_cast<const float4*>(M + (size_t)(j + 4 * u) * ld + row0);
+          v[u] = dn_ld4_rt(M + (size_t)(j + 4 * u) * ld + row0, stream);
           xs[u] = OP == ROW_DOT ? x[j + 4 * u] : 0.f;
         }
 #pragma unroll
         for (int u = 0; u < 4; ++u) { take(0, v[u].x, xs[u]); take(1, v[u].y, xs[u]); take(2, v[u].z, xs[u]); take(3, v[u].w, xs[u]); }
       }
       for (; j < j1; j += 4) {
-        const float4 v = *reinterpret_cast<const float4*>(M + (size_t)j * ld + row0);
+        const float4 v = dn_ld4_rt(M + (size_t)j * ld + row0, stream);
         const float xj = OP == ROW_DOT ? x[j] : 0.f;
         take(0, v.x, xj); take(1, v.y, xj); take(2, v.z, xj); take(3, v.w, xj);
       }
@@ -438,6 +443,8 @@ static int rows_reduce(const float* M, int ld, int h, int w, const float* x, flo
     if (!partial) return CUDA_ERROR;
   }
   dim3 grid(bx, splits);
+  // (Finishing inside stage 1 by the last-arriving workgroup was measured 8x slower:
+  // the device-scope release fence each workgroup then needs writes back its L2.)
   if (vec)
     hipLaunchKernelGGL((k_rows_stage1<true, OP>), grid, dim3(256), 0, 0, M, ld, h, w, cps, x, y, partial, alpha, beta);
   else

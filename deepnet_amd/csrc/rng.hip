@@ -82,56 +82,46 @@ __global__ void k_seed(const unsigned int* mults, unsigned long long* words, uns
 }
 
 // ------------------------------------------------------------------ consumers
-// One uniform per element.  load(i) fetches whatever the element needs from memory
-// and does not depend on the draw, so a lane issues a batch of loads before it
-// walks the serial chain of its stream; store(i, u, x) finishes the element.
+// One uniform per element.  An op names the array it reads (src, may be null), the
+// array it writes (dst) and the pure function value(u, x) of the uniform u and the
+// loaded x.  The loads do not depend on the draws, so a lane issues a batch of them
+// before it walks the serial chain of its stream.
 struct OpUniform {
-  float* out;
-  __device__ __forceinline__ float load(size_t) const { return 0.f; }
-  __device__ __forceinline__ void store(size_t i, float u, float) const { out[i] = u; }
+  const float* src; float* dst;
+  __device__ __forceinline__ float value(float u, float) const { return u; }
 };
 struct OpDropout {
-  float* data;
+  const float* src; float* dst;
   float p, val;
-  __device__ __forceinline__ float load(size_t i) const { return data[i]; }
-  __device__ __forceinline__ void store(size_t i, float u, float x) const { data[i] = u > p ? x : val; }
+  __device__ __forceinline__ float value(float u, float x) const { return u > p ? x : val; }
 };
 struct OpBernoulli {
-  const float* in;
-  float* out;
-  __device__ __forceinline__ float load(size_t i) const { return in[i]; }
-  __device__ __forceinline__ void store(size_t i, float u, float x) const { out[i] = u < x ? 1.f : 0.f; }
+  const float* src; float* dst;
+  __device__ __forceinline__ float value(float u, float x) const { return u < x ? 1.f : 0.f; }
 };
 struct OpBernoulliTanh {
-  const float* in;
-  float* out;
-  __device__ __forceinline__ float load(size_t i) const { return in[i]; }
-  __device__ __forceinline__ void store(size_t i, float u, float x) const {
-    out[i] = (double)u < (1.0 + (double)x) / 2.0 ? 1.f : 0.f;
+  const float* src; float* dst;
+  __device__ __forceinline__ float value(float u, float x) const {
+    return (double)u < (1.0 + (double)x) / 2.0 ? 1.f : 0.f;
   }
 };
 struct OpCopy {  // sample_poisson of the reference: draws are consumed, data copied
-  const float* in;
-  float* out;
-  __device__ __forceinline__ float load(size_t i) const { return in[i]; }
-  __device__ __forceinline__ void store(size_t i, float u, float x) const { (void)u; out[i] = x; }
+  const float* src; float* dst;
+  __device__ __forceinline__ float value(float, float x) const { return x; }
 };
 struct OpPerturbEnergy {
-  const float* in;
-  float* out;
-  __device__ __forceinline__ float load(size_t i) const { return in[i]; }
-  __device__ __forceinline__ void store(size_t i, float u, float x) const { out[i] = x - logf(-logf(u)); }
+  const float* src; float* dst;
+  __device__ __forceinline__ float value(float u, float x) const { return x - logf(-logf(u)); }
 };
 struct OpPerturbProb {
-  const float* in;
-  float* out;
-  __device__ __forceinline__ float load(size_t i) const { return in[i]; }
-  __device__ __forceinline__ void store(size_t i, float u, float x) const { out[i] = -x / logf(u); }
+  const float* src; float* dst;
+  __device__ __forceinline__ float value(float u, float x) const { return -x / logf(u); }
 };
 
 // Draws [d0, d1) of one stream: element index of draw d is d * 12288 + idx.
+// STREAM: the call is large, use non-temporal accesses.
 #define RNG_BATCH 8
-template <class Op>
+template <bool STREAM, class Op>
 __device__ __forceinline__ unsigned long long rng_walk(unsigned long long w, unsigned int mult, unsigned int idx,
                                                        unsigned long long d0, unsigned long long d1, const Op& op) {
   size_t i = (size_t)d0 * NUM_RND_STREAMS + idx;
@@ -139,17 +129,18 @@ __device__ __forceinline__ unsigned long long rng_walk(unsigned long long w, uns
   for (; d + RNG_BATCH <= d1; d += RNG_BATCH, i += (size_t)RNG_BATCH * NUM_RND_STREAMS) {
     float x[RNG_BATCH];
 #pragma unroll
-    for (int k = 0; k < RNG_BATCH; ++k) x[k] = op.load(i + (size_t)k * NUM_RND_STREAMS);
+    for (int k = 0; k < RNG_BATCH; ++k)
+      x[k] = op.src ? dn_ld1_rt(op.src + i + (size_t)k * NUM_RND_STREAMS, STREAM) : 0.f;
 #pragma unroll
     for (int k = 0; k < RNG_BATCH; ++k) {
       w = mwc_step(w, mult);
-      op.store(i + (size_t)k * NUM_RND_STREAMS, mwc_uniform(w), x[k]);
+      dn_st1_rt(op.dst + i + (size_t)k * NUM_RND_STREAMS, op.value(mwc_uniform(w), x[k]), STREAM);
     }
   }
   for (; d < d1; ++d, i += NUM_RND_STREAMS) {
-    const float x = op.load(i);
+    const float x = op.src ? op.src[i] : 0.f;
     w = mwc_step(w, mult);
-    op.store(i, mwc_uniform(w), x);
+    op.dst[i] = op.value(mwc_uniform(w), x);
   }
   return w;
 }
@@ -163,7 +154,7 @@ k_rng_serial(const unsigned int* mults, unsigned long long* words, size_t n, Op 
   const unsigned int idx = blockIdx.x * RNG_BLOCK + threadIdx.x;
   const unsigned int mult = mults[idx];
   const unsigned long long draws = n > idx ? (n - idx + NUM_RND_STREAMS - 1) / NUM_RND_STREAMS : 0;
-  words[idx] = rng_walk(words[idx], mult, idx, 0, draws, op);
+  words[idx] = rng_walk<false>(words[idx], mult, idx, 0, draws, op);
 }
 
 // Split schedule: lane (stream s, part p) produces draws [p << chbits, (p+1) << chbits)
@@ -189,7 +180,7 @@ k_rng_split(const unsigned int* mults, const unsigned long long* words, unsigned
   unsigned long long w = words[idx];
   for (unsigned int b = 0, pp = part; pp; ++b, pp >>= 1)
     if (pp & 1u) w = mwc_montmul(w, table[(size_t)(chbits + b) * NUM_RND_STREAMS + idx], mult);
-  w = rng_walk(w, mult, idx, d0, d1, op);
+  w = rng_walk<true>(w, mult, idx, d0, d1, op);
   if (d1 == draws) next[idx] = w;
 }
 
@@ -280,7 +271,7 @@ int init_random(rnd_struct* rnd_state, int seed, char* cudamatpath) {
 
 int fill_with_rand(rnd_struct* rnd_state, cudamat* mat) {
   if (!mat->on_device) return ERROR_NOT_ON_DEVICE;
-  return launch_rng(rnd_state, (size_t)dn_len(mat), OpUniform{mat->data_device});
+  return launch_rng(rnd_state, (size_t)dn_len(mat), OpUniform{nullptr, mat->data_device});
 }
 
 int fill_with_randn(rnd_struct* rnd_state, cudamat* mat) {
@@ -315,7 +306,7 @@ int sample_gaussian(rnd_struct* rnd_state, cudamat* mat, cudamat* target, float 
 
 int dropout(rnd_struct* rnd_state, cudamat* mat, float dropprob, float val) {
   if (!mat->on_device) return ERROR_NOT_ON_DEVICE;
-  return launch_rng(rnd_state, (size_t)dn_len(mat), OpDropout{mat->data_device, dropprob, val});
+  return launch_rng(rnd_state, (size_t)dn_len(mat), OpDropout{mat->data_device, mat->data_device, dropprob, val});
 }
 
 }  // extern "C"

@@ -190,6 +190,52 @@ def conv_outp(images, hid, C, Mx, k, padding, stride, groups=1, partial_sum=0):
     return np.concatenate([out[ch].reshape(F, -1) for ch in range(chunks)], axis=1)
 
 
+# ---- locally connected layers: cudamat_conv.cu:1415-1423, filters (module, colour, ky, kx, filter) ----
+
+def local_up(images, filters, C, Mx, padding, stride):
+    """Like conv_up with a separate filter bank per module: filters is (F, M*C*k*k) with
+    column ((m*C + c)*k + ky)*k + kx."""
+    images = np.asarray(images, dtype=F64)
+    filters = np.asarray(filters, dtype=F64)
+    N = images.shape[0]
+    H = int(round(np.sqrt(images.shape[1] // C)))
+    F = filters.shape[0]
+    M = Mx * Mx
+    k = int(round(np.sqrt(filters.shape[1] // (M * C))))
+    w = filters.reshape(F, M, C, k, k)
+    lo, hi = _pad_for(H, k, Mx, padding, stride)
+    xp = np.pad(to_nchw(images, C, H), ((0, 0), (0, 0), (lo, hi), (lo, hi)))
+    out = np.zeros((N, F, Mx, Mx))
+    for my in range(Mx):
+        for mx in range(Mx):
+            patch = xp[:, :, my * stride:my * stride + k, mx * stride:mx * stride + k]
+            out[:, :, my, mx] = np.einsum('ncyx,fcyx->nf', patch, w[:, my * Mx + mx])
+    return from_nchw(out)
+
+
+def local_down(hid, filters, C, H, padding, stride):
+    hid = np.asarray(hid, dtype=F64)
+    filters = np.asarray(filters, dtype=F64)
+    N, F = hid.shape[0], filters.shape[0]
+    Mx = int(round(np.sqrt(hid.shape[1] // F)))
+    M = Mx * Mx
+    k = int(round(np.sqrt(filters.shape[1] // (M * C))))
+    w = filters.reshape(F, M, C, k, k)
+    h = hid.reshape(N, F, Mx, Mx)
+    lo, hi = _pad_for(H, k, Mx, padding, stride)
+    gp = np.zeros((N, C, H + lo + hi, H + lo + hi))
+    for my in range(Mx):
+        for mx in range(Mx):
+            gp[:, :, my * stride:my * stride + k, mx * stride:mx * stride + k] += np.einsum(
+                'nf,fcyx->ncyx', h[:, :, my, mx], w[:, my * Mx + mx])
+    return from_nchw(gp[:, :, lo:lo + H, lo:lo + H])
+
+
+def local_outp(images, hid, C, Mx, k, padding, stride):
+    """(F, M*C*k*k): per-module weight gradient == conv_outp with one module per chunk."""
+    return conv_outp(images, hid, C, Mx, k, padding, stride, partial_sum=1)
+
+
 # ---- pooling: cudamat_conv.cu:1021-1182, cudamat_conv_kernels.cuh:1355-1530 -------------
 
 def max_pool(images, F, subs, start, stride, O):

@@ -98,8 +98,6 @@ def test_bad_shapes_raise_instead_of_aborting(cm, cc, rng):
         cc.convUp(X, W, cm.empty((16, 5)), 6, 1, 1, 3)
     with pytest.raises(cm.CUDAMatException, match="convUp"):
         cc._call('convUp', X.p_mat, W.p_mat, cm.empty((16, 16 * 36)).p_mat, 6, -1, 1, 4, 1)   # 108 % 4 colours
-    with pytest.raises(cm.CUDAMatException, match="not implemented"):
-        cc.localUp(X, W, cm.empty((16, 16 * 36)), 6, 1, 1, 3)
     host_only = cm.CUDAMatrix(_f(rng.standard_normal((16, 108))), copy_to_device=False)
     with pytest.raises(cm.CUDAMatException, match="on_device"):
         cc.MaxPool(host_only, cm.empty((16, 3 * 9)), 3, 2, 0, 2, 3)
@@ -182,3 +180,20 @@ def test_conv_layer_chain_like_deepnet(cm, cc, rng):
     want = co.max_pool(want, F, 3, 0, 2, O)
     want, _ = co.response_norm(want, F, 5, 0.001, 0.75)
     assert np.allclose(out.asarray(), want.T, rtol=2e-4, atol=2e-5)
+
+
+@pytest.mark.parametrize("N,C,H,F,k,s,p", [(4, 2, 6, 16, 3, 1, 1), (16, 3, 8, 16, 3, 2, 0)])
+def test_locally_connected_layers(cm, cc, rng, N, C, H, F, k, s, p):
+    Mx = co.n_modules(H, k, s, p)
+    M = Mx * Mx
+    x = _f(rng.standard_normal((N, C * H * H)))
+    w = _f(0.1 * rng.standard_normal((F, M * C * k * k)))
+    y = _f(rng.standard_normal((N, F * M)))
+    X, W, Y = cm.CUDAMatrix(x), cm.CUDAMatrix(w), cm.CUDAMatrix(y)
+    up, down, outp = cm.empty((N, F * M)), cm.empty((N, C * H * H)), cm.empty((F, M * C * k * k))
+    cc.localUp(X, W, up, Mx, p, s, C)
+    assert np.allclose(up.asarray(), co.local_up(x, w, C, Mx, p, s), rtol=1e-4, atol=1e-5)
+    cc.localDown(Y, W, down, Mx, p, s, k, H, C)
+    assert np.allclose(down.asarray(), co.local_down(y, w, C, H, p, s), rtol=1e-4, atol=1e-5)
+    cc.localOutp(X, Y, outp, Mx, p, k, s, C)
+    assert np.allclose(outp.asarray(), co.local_outp(x, y, C, Mx, k, p, s), rtol=1e-4, atol=1e-4)

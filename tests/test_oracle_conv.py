@@ -140,3 +140,17 @@ def test_response_norm_closed_form_and_gradient(rng, size):
     e = np.zeros_like(x); e[0, 5] = 1e-6
     fd = ((co.response_norm(x + e, F, size, a, p)[0] - co.response_norm(x - e, F, size, a, p)[0]) / 2e-6 * g).sum()
     assert np.isclose(fd, undo[0, 5], rtol=1e-5)
+
+
+def test_local_layers_reduce_to_conv_with_shared_filters_and_are_adjoint(rng):
+    N, C, H, F, k, s, p = 2, 2, 6, 4, 3, 1, 1
+    Mx = co.n_modules(H, k, s, p)
+    M = Mx * Mx
+    x = rng.standard_normal((N, C * H * H))
+    w = rng.standard_normal((F, C * k * k))
+    w_local = np.tile(w.reshape(F, 1, C * k * k), (1, M, 1)).reshape(F, -1)     # the same bank at every module
+    assert np.allclose(co.local_up(x, w_local, C, Mx, p, s), co.conv_up(x, w, C, Mx, p, s))
+    wl = rng.standard_normal((F, M * C * k * k))
+    y = rng.standard_normal((N, F * M))
+    up, down, outp = co.local_up(x, wl, C, Mx, p, s), co.local_down(y, wl, C, H, p, s), co.local_outp(x, y, C, Mx, k, p, s)
+    assert np.isclose((up * y).sum(), (x * down).sum()) and np.isclose((up * y).sum(), (wl * outp).sum())
