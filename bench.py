@@ -320,6 +320,9 @@ def main():
     ap.add_argument('--warmup', type=int, default=2)
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
     ap.add_argument('--only-c2', action='store_true', help='skip the secondary workloads')
+    ap.add_argument('--probe', action='store_true',
+                    help='run only the roofline kernel (add_mult) and a copy-shaped calibration kernel '
+                         '(mult by a scalar into a second matrix), for rocprofv3 --pmc runs')
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this backend has no multi-GPU path (run with --gpus 1).")
@@ -328,6 +331,17 @@ def main():
     cm.cublas_init()
     cm.CUDAMatrix.init_random(2)
     ev = HipEvents()
+
+    if args.probe:
+        sets = build_c2(cm)
+        for _ in range(3):
+            for s in sets:
+                s['A'].add_mult(s['B'], 0.5)          # k_ew<2, true, FAxpy>: reads 2 x 64 MiB, writes 64 MiB
+            for s in sets:
+                s['A'].mult(1.0, target=s['T'])       # k_ew<1, true, FMulS>: reads 64 MiB, writes 64 MiB
+        cm.cuda_sync_threads()
+        print(json.dumps({'probe': 'done', 'elements': E}))
+        return
 
     sets = build_c2(cm)
     marks = {name: (ev.new(), ev.new()) for name, _, _ in C2_OPS}
@@ -352,9 +366,16 @@ def main():
     value = STEP_BYTES / step_s / 1e9
 
     roof_op = 'add_mult'
+    traffic = None
+    try:    # HBM bytes per launch from the committed rocprofv3 --pmc summary (FETCH_SIZE + WRITE_SIZE, calibrated)
+        for ln in open(os.path.join(ROOT, 'profiles', 'k_ew_axpy_hbm_traffic.md')):
+            if ln.startswith('traffic_bytes_per_launch:'):
+                traffic = int(ln.split(':')[1])
+    except OSError:
+        pass
     roofline = {'kernel': 'k_ew<2, true, FAxpy> (add_mult, 4096x4096)', 'bound': 'hbm',
                 'achieved': ops[roof_op]['gbs'], 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
-                'frac': round(ops[roof_op]['gbs'] / HBM_PEAK_GBS, 4), 'traffic': None,
+                'frac': round(ops[roof_op]['gbs'] / HBM_PEAK_GBS, 4), 'traffic': traffic,
                 'algorithmic_bytes_per_launch': 12 * E, 'avg_launch_us': ops[roof_op]['us']}
 
     secondary = {}
