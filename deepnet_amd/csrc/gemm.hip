@@ -169,6 +169,125 @@ k_gemm(const float* __restrict__ A, int lda, const float* __restrict__ B, int ld
     }
 }
 
+// Products too small to fill the chip with 64 x 64 tiles (the RBM / MLP layer shapes):
+// a workgroup owns one 32 x 32 block of C; its NW wavefronts each take every NW-th
+// 32-deep chunk of K, loading their operands straight from global memory in the
+// matrix-core operand layout (no LDS staging, nothing to synchronise while
+// accumulating, two chunks in flight per wavefront), and add their accumulators up
+// through LDS in a fixed order.  One launch, no second kernel.  Within a chunk, lane
+// (row i, half h) supplies k0 + 16h + 4u + v to the (4u+v)-th of 16 successive MFMAs:
+// any order of the k terms is fine as long as both operands use the same one, and
+// this one gives a k-contiguous operand four 16-byte loads per lane that together
+// cover whole 128-byte lines.
+__device__ __forceinline__ float small_ldg(const float* base, unsigned byte_off) {
+  return *reinterpret_cast<const float*>(reinterpret_cast<const char*>(base) + byte_off);
+}
+
+// r[q] = op(P)(row, k0 + 16*lk + q) for q < 16, zero where k >= K.  `row` is already
+// clamped into the matrix, k0 is wave-uniform, and all offsets fit 32 bits (the
+// dispatcher checks), so every load is an SGPR base plus one 32-bit lane offset and
+// none of them sits behind a lane-dependent branch.
+template <bool KC>
+__device__ __forceinline__ void small_load(const float* __restrict__ P, unsigned ld, unsigned row, int k0, int lk, int K,
+                                           bool vec, float (&r)[16]) {
+  if (k0 >= K) {
+#pragma unroll
+    for (int q = 0; q < 16; ++q) r[q] = 0.f;
+    return;
+  }
+  const int kl = k0 + 16 * lk;
+  if (k0 + 32 <= K) {
+    if (KC) {
+      const unsigned off = (row * ld + (unsigned)kl) * 4u;
+      if (vec) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const float4 t =
+              *reinterpret_cast<const float4*>(reinterpret_cast<const char*>(P) + (off + 16u * u));
+          r[4 * u] = t.x; r[4 * u + 1] = t.y; r[4 * u + 2] = t.z; r[4 * u + 3] = t.w;
+        }
+      } else {
+#pragma unroll
+        for (int q = 0; q < 16; ++q) r[q] = small_ldg(P, off + 4u * q);
+      }
+    } else {
+      const float* pu = P + (size_t)k0 * ld;                 // wave-uniform
+      const unsigned off = (16u * lk * ld + row) * 4u;
+#pragma unroll
+      for (int q = 0; q < 16; ++q) r[q] = small_ldg(pu, off + 4u * q * ld);
+    }
+  } else {                                                   // the chunk that crosses K
+#pragma unroll
+    for (int q = 0; q < 16; ++q) {
+      const unsigned kk = (unsigned)min(kl + q, K - 1);
+      r[q] = small_ldg(P, (KC ? row * ld + kk : kk * ld + row) * 4u);
+    }
+#pragma unroll
+    for (int q = 0; q < 16; ++q) r[q] = kl + q < K ? r[q] : 0.f;
+  }
+}
+
+template <bool A_KC, bool B_KC, int NW>
+__global__ void __launch_bounds__(NW * 64)
+k_gemm_small(const float* __restrict__ A, int lda, const float* __restrict__ B, int ldb, float* C, int ldc, int M, int N,
+             int K, float alpha, float beta, bool a_vec, bool b_vec) {
+  constexpr int RED = NW / 2 > 4 ? NW / 2 : 4;
+  __shared__ float red[RED][16 * 64];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);   // tell the compiler it is wave-uniform
+  const int li = lane & 31, lk = lane >> 5;
+  const int m = blockIdx.x * 32 + li, n = blockIdx.y * 32 + li;
+  const bool m_ok = m < M;
+  const unsigned mc = min(m, M - 1), nc = min(n, N - 1);    // rows past the edge repeat the last one; never stored
+
+  f32x16 acc;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+  float a0[16], b0[16], a1[16], b1[16];
+  constexpr int STEP = 32 * NW;
+  int k0 = wv * 32;
+  small_load<A_KC>(A, lda, mc, k0, lk, K, a_vec, a0);
+  small_load<B_KC>(B, ldb, nc, k0, lk, K, b_vec, b0);
+  for (; k0 < K; k0 += STEP) {
+    small_load<A_KC>(A, lda, mc, k0 + STEP, lk, K, a_vec, a1);   // next chunk in flight behind the MFMAs
+    small_load<B_KC>(B, ldb, nc, k0 + STEP, lk, K, b_vec, b1);
+#pragma unroll
+    for (int q = 0; q < 16; ++q) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(b0[q], a0[q], acc, 0, 0, 0);
+#pragma unroll
+    for (int q = 0; q < 16; ++q) { a0[q] = a1[q]; b0[q] = b1[q]; }
+  }
+  // Halve the number of live accumulators until four are left ...
+#pragma unroll
+  for (int half = NW / 2; half >= 4; half >>= 1) {
+    if (wv >= half && wv < 2 * half) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) red[wv - half][v * 64 + lane] = acc[v];
+    }
+    __syncthreads();
+    if (wv < half) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[v] += red[wv][v * 64 + lane];
+    }
+    __syncthreads();
+  }
+  if (wv < 4) {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) red[wv][v * 64 + lane] = acc[v];
+  }
+  __syncthreads();
+  // ... and let every lane finish its share of the 1024 outputs: element e = v*64 + lane
+  // is C(m, n) with m = tile + lane%32, n = tile + 8*(v/4) + 4*(lane/32) + v%4.
+  for (int e = tid; e < 1024; e += NW * 64) {
+    const int v = e >> 6;
+    const float sum = (red[0][e] + red[1][e]) + (red[2][e] + red[3][e]);
+    const int nn = blockIdx.y * 32 + 8 * (v >> 2) + 4 * lk + (v & 3);
+    if (m_ok && nn < N) {
+      float* p = C + (size_t)nn * ldc + m;
+      *p = (beta == 0.f ? 0.f : beta * *p) + alpha * sum;
+    }
+  }
+}
+
 __global__ void k_gemm_splitk_finish(const float* partial, int splits, float* C, int ldc, int M, int N, float alpha,
                                      float beta) {
   const size_t total = (size_t)M * N;
@@ -221,8 +340,29 @@ static int gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, co
   const bool a_vec = dn_aligned16(A) && (lda % 4 == 0);
   const bool b_vec = dn_aligned16(B) && (ldb % 4 == 0);
 
-  // Tile choice: big tiles when they already fill the chip, else 64x64 tiles,
-  // and split K when even those leave most CUs idle.
+  // Tile choice: big tiles when they already fill the chip, else 64x64 tiles; when
+  // even those cannot fill it, the 32x32-per-workgroup kernel that splits K over
+  // its own wavefronts.
+  const long long tiles64 = (long long)((M + 63) / 64) * ((N + 63) / 64);
+  const bool off32 = (size_t)lda * (a_kc ? M : K) < (1u << 30) && (size_t)ldb * (b_kc ? N : K) < (1u << 30);
+  if (tiles64 < cus && off32) {
+    dim3 grid((M + 31) / 32, (N + 31) / 32);
+#define GEMM_SMALL(AK, BK_)                                                                                  \
+  do {                                                                                                       \
+    if (K <= 128)                                                                                            \
+      hipLaunchKernelGGL((k_gemm_small<AK, BK_, 4>), grid, dim3(256), 0, 0, A, lda, B, ldb, C, ldc, M, N, K,  \
+                         alpha, beta, a_vec, b_vec);                                                         \
+    else                                                                                                     \
+      hipLaunchKernelGGL((k_gemm_small<AK, BK_, 8>), grid, dim3(512), 0, 0, A, lda, B, ldb, C, ldc, M, N, K,  \
+                         alpha, beta, a_vec, b_vec);                                                         \
+  } while (0)
+    if (a_kc && b_kc) GEMM_SMALL(true, true);
+    else if (a_kc) GEMM_SMALL(true, false);
+    else if (b_kc) GEMM_SMALL(false, true);
+    else GEMM_SMALL(false, false);
+#undef GEMM_SMALL
+    return dn_launch_status();
+  }
   const long long tiles_big = (long long)((M + 127) / 128) * ((N + 127) / 128);
   const bool big = tiles_big >= cus;
   const int BM = big ? 128 : 64, BN = big ? 128 : 64;

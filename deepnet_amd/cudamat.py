@@ -367,8 +367,7 @@ class CUDAMatrix(object):
         m = _cudamat.get_leading_dimension(mat.p_mat)
         n = _cudamat.get_nonleading_dimension(mat.p_mat)
         if axis == 0:
-            left = _ones(m)
-            left.set_trans(True)
+            left = _ones(m, trans=True)
             right = mat
         elif axis == 1:
             left = mat
@@ -714,13 +713,29 @@ def empty(shape):
     return CUDAMatrix(mat)
 
 
-def _ones(n):
-    """View of the first n entries of the device vector of ones, grown on demand."""
+_ones_views = {}
+
+
+def _ones(n, trans=False):
+    """View of the first n entries of the device vector of ones (grown on demand), as a
+    column or, with trans, as a row.  Views are kept per (n, trans): the sums call this
+    on every step with the same few sizes."""
     if not isinstance(CUDAMatrix.ones, CUDAMatrix):
         raise CUDAMatException("cublas_init() has not been called.")
     if n > CUDAMatrix.ones.shape[0]:
         CUDAMatrix.ones = CUDAMatrix(np.ones((n, 1), dtype=np.float32, order='F'))
-    return CUDAMatrix.ones.slice(0, n)
+        _ones_views.clear()
+    key = (n, trans)
+    view = _ones_views.get(key)
+    if view is None or view._ones_parent is not CUDAMatrix.ones:
+        view = CUDAMatrix.ones.slice(0, n)
+        if trans:
+            view.set_trans(True)
+        view._ones_parent = CUDAMatrix.ones
+        if len(_ones_views) > 256:
+            _ones_views.clear()
+        _ones_views[key] = view
+    return view
 
 
 def sum(mat, axis, target=None):
@@ -729,8 +744,7 @@ def sum(mat, axis, target=None):
     m = _cudamat.get_leading_dimension(mat.p_mat)
     n = _cudamat.get_nonleading_dimension(mat.p_mat)
     if axis == 0:
-        left = _ones(m)
-        left.set_trans(True)
+        left = _ones(m, trans=True)
         right = mat
         if target is None:
             target = empty((1, n))
@@ -874,6 +888,7 @@ init = cublas_init
 
 def cublas_shutdown():
     CUDAMatrix.ones = 0
+    _ones_views.clear()
     _cudamat.cublas_shutdown()
 
 
