@@ -370,12 +370,12 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
     const bool more = slab + 1 < slab_end;
     if (more) fetch(slab + 1);
 #pragma unroll
-    for (int kk = 0; kk < CV_BK; kk += 2) {
+    for (int kk = 0; kk < CV_BK / 2; ++kk) {  // rows kk and kk + BK/2: 32 banks apart, no conflict
       float av[WM], bv[WN];
 #pragma unroll
-      for (int i = 0; i < WM; ++i) av[i] = As[buf][kk + lk][(wm * WM + i) * 32 + li];
+      for (int i = 0; i < WM; ++i) av[i] = As[buf][kk + (CV_BK / 2) * lk][(wm * WM + i) * 32 + li];
 #pragma unroll
-      for (int j = 0; j < WN; ++j) bv[j] = Bs[buf][kk + lk][(wn * WN + j) * 32 + li];
+      for (int j = 0; j < WN; ++j) bv[j] = Bs[buf][kk + (CV_BK / 2) * lk][(wn * WN + j) * 32 + li];
 #pragma unroll
       for (int j = 0; j < WN; ++j)
 #pragma unroll

@@ -68,7 +68,39 @@ k_gemm(const float* __restrict__ A, int lda, const float* __restrict__ B, int ld
 
   float4 ra[A4], rb[B4];
 
-  auto fetch = [&](int k0) {
+  // Tiles that lie wholly inside both operands, on 16-byte aligned data, fetch through
+  // per-lane pointers that advance one slab at a time: no index arithmetic and no
+  // branch around any load.  Edge tiles and the last partial slab take the checked path.
+  const bool a_fast = a_vec && m0 + BM <= M, b_fast = b_vec && n0 + BN <= N;
+  const float* pa[A4];
+  const float* pb[B4];
+#pragma unroll
+  for (int u = 0; u < A4; ++u) {
+    const int f = tid + u * 256;
+    if (A_KC) pa[u] = A + (size_t)(m0 + (f >> 2)) * lda + kbeg + ((f & 3) << 2);
+    else pa[u] = A + (size_t)(kbeg + f / (BM / 4)) * lda + m0 + ((f % (BM / 4)) << 2);
+  }
+#pragma unroll
+  for (int u = 0; u < B4; ++u) {
+    const int f = tid + u * 256;
+    if (B_KC) pb[u] = B + (size_t)(n0 + (f >> 2)) * ldb + kbeg + ((f & 3) << 2);
+    else pb[u] = B + (size_t)(kbeg + f / (BN / 4)) * ldb + n0 + ((f % (BN / 4)) << 2);
+  }
+  const size_t a_step = A_KC ? GEMM_BK : (size_t)GEMM_BK * lda, b_step = B_KC ? GEMM_BK : (size_t)GEMM_BK * ldb;
+
+  auto fetch_fast = [&]() {
+#pragma unroll
+    for (int u = 0; u < A4; ++u) {
+      ra[u] = *reinterpret_cast<const float4*>(pa[u]);
+      pa[u] += a_step;
+    }
+#pragma unroll
+    for (int u = 0; u < B4; ++u) {
+      rb[u] = *reinterpret_cast<const float4*>(pb[u]);
+      pb[u] += b_step;
+    }
+  };
+  auto fetch_checked = [&](int k0) {
 #pragma unroll
     for (int u = 0; u < A4; ++u) {
       const int f = tid + u * 256;
@@ -120,28 +152,53 @@ k_gemm(const float* __restrict__ A, int lda, const float* __restrict__ B, int ld
   };
 
   const int lk = lane >> 5, li = lane & 31;
-  int buf = 0;
-  if (kbeg < kend) {
-    fetch(kbeg);
-    stash(0);
-  }
-  __syncthreads();
-  for (int k0 = kbeg; k0 < kend; k0 += GEMM_BK) {
-    const bool more = k0 + GEMM_BK < kend;
-    if (more) fetch(k0 + GEMM_BK);
+  // One slab: all of its fragments are asked of LDS first (the scheduling fence keeps
+  // the compiler from sinking the reads back to their uses), so the MFMAs of one k
+  // pair run while the reads of the following pairs are still in flight.
+  auto multiply = [&](int buf) {
+    float av[GEMM_BK / 2][WM], bv[GEMM_BK / 2][WN];
 #pragma unroll
-    for (int kk = 0; kk < GEMM_BK; kk += 2) {
-      float av[WM], bv[WN];
+    for (int kk = 0; kk < GEMM_BK / 2; ++kk) {  // rows kk and kk + BK/2: 32 banks apart, no conflict
 #pragma unroll
-      for (int i = 0; i < WM; ++i) av[i] = As[buf][kk + lk][wm * 32 * WM + i * 32 + li];
+      for (int i = 0; i < WM; ++i) av[kk][i] = As[buf][kk + (GEMM_BK / 2) * lk][wm * 32 * WM + i * 32 + li];
 #pragma unroll
-      for (int j = 0; j < WN; ++j) bv[j] = Bs[buf][kk + lk][wn * 32 * WN + j * 32 + li];
+      for (int j = 0; j < WN; ++j) bv[kk][j] = Bs[buf][kk + (GEMM_BK / 2) * lk][wn * 32 * WN + j * 32 + li];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int kk = 0; kk < GEMM_BK / 2; ++kk)
 #pragma unroll
       for (int j = 0; j < WN; ++j)
 #pragma unroll
         for (int i = 0; i < WM; ++i)
-          acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[j], av[i], acc[j][i], 0, 0, 0);
+          acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[kk][j], av[kk][i], acc[j][i], 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);  // the wait for the next slab's global loads stays behind the MFMAs
+  };
+
+  // Tiles wholly inside both operands run their full slabs through a loop whose loads
+  // are unconditional; what is left (edge tiles, the last partial slab) goes through
+  // the checked loop.
+  const bool fast = a_fast && b_fast;
+  int buf = 0, k0 = kbeg;
+  if (kbeg < kend) {
+    if (fast && kbeg + GEMM_BK <= kend) fetch_fast();
+    else fetch_checked(kbeg);
+    stash(0);
+  }
+  __syncthreads();
+  if (fast) {
+    for (; k0 + 2 * GEMM_BK <= kend; k0 += GEMM_BK) {
+      fetch_fast();
+      multiply(buf);
+      stash(buf ^ 1);
+      __syncthreads();
+      buf ^= 1;
     }
+  }
+  for (; k0 < kend; k0 += GEMM_BK) {
+    const bool more = k0 + GEMM_BK < kend;
+    if (more) fetch_checked(k0 + GEMM_BK);
+    multiply(buf);
     if (more) stash(buf ^ 1);
     __syncthreads();
     buf ^= 1;
