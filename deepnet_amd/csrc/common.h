@@ -25,27 +25,28 @@ static inline long long dn_len(const cudamat* m) { return (long long)m->size[0] 
 // integer divide: q = (n * magic) >> 32 >> shift for n < 2^31.
 struct FastDiv {
   uint32_t magic;
-  uint32_t shift;
+  uint32_t sh1, sh2;   // min(ceil(log2 d), 1) and max(ceil(log2 d) - 1, 0)
   uint32_t d;
 };
 
 static inline FastDiv make_fastdiv(uint32_t d) {
   FastDiv f;
   f.d = d;
-  if (d <= 1) { f.magic = 0; f.shift = 0; return f; }
+  if (d == 0) d = 1;
   uint32_t s = 0;
   while ((1ull << s) < d) ++s;            // s = ceil(log2 d)
   uint64_t m = ((1ull << 32) * ((1ull << s) - d)) / d + 1;
   f.magic = (uint32_t)m;
-  f.shift = s;
+  f.sh1 = s < 1 ? s : 1;
+  f.sh2 = s > 1 ? s - 1 : 0;
   return f;
 }
 
-// Exact for every 32-bit n (round-up method: q = (hi + ((n - hi) >> 1)) >> (s-1)).
+// Exact for every 32-bit n and every divisor, without a branch
+// (round-up method: q = (hi + ((n - hi) >> sh1)) >> sh2; d = 1 gives magic 1, no shifts).
 __device__ __forceinline__ uint32_t fd_div(uint32_t n, const FastDiv& f) {
-  if (f.d <= 1) return n;
-  uint32_t hi = __umulhi(n, f.magic);
-  return (hi + ((n - hi) >> 1)) >> (f.shift - 1);
+  const uint32_t hi = __umulhi(n, f.magic);
+  return (hi + ((n - hi) >> f.sh1)) >> f.sh2;
 }
 
 // Wave-wide reductions through cross-lane shuffles (wave64).

@@ -158,7 +158,9 @@ template <int MODE, int WAVES_M, int WM, int WN>
 __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
   constexpr int WAVES_N = 4 / WAVES_M;
   constexpr int BM = 32 * WM * WAVES_M, BN = 32 * WN * WAVES_N;
-  constexpr int LA = BM + CV_PAD, LB = BN + CV_PAD;
+  // Row pitch in LDS: operands written transposed one float per lane want pitch % 8 == 2
+  // (no bank conflicts), those written 16 bytes at a time need pitch % 4 == 0.
+  constexpr int LA = BM + (MODE == CONV_OUTP ? 2 : CV_PAD), LB = BN + (MODE == CONV_UP ? CV_PAD : 2);
   constexpr int TA = BM * CV_BK / 4, TB = BN * CV_BK / 4;  // 16-byte groups per slab
   constexpr int NA = (TA + 255) / 256, NB = (TB + 255) / 256;
   __shared__ __attribute__((aligned(16))) float As[2][CV_BK][LA];
@@ -199,14 +201,38 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
   if (row0 >= rows || col0 >= cols) return;  // uniform for the workgroup
 
   // ---- loop-invariant part of each lane's gathers
+  // The gathers that can fall into the padding (images for Up and Outp, hidden
+  // activations for Down) are addressed as  base + 32-bit lane offset, where
+  //   lane offset = (what depends on the lane, fixed for the whole kernel)
+  //               + (what depends on the slab: wave-uniform, computed on the scalar unit).
+  // base sits `bias` elements below the array so that no lane offset is negative, and a
+  // group outside the image reads the first element of the array (offset = bias) and is
+  // zeroed when it is written to LDS.  Per slab and group this costs a handful of
+  // vector instructions; the index decomposition runs on the scalar unit.
+  const int wvu = __builtin_amdgcn_readfirstlane(wv);
+  constexpr int A_ROWLANES = BM / 4;                               // lanes per kk row of the A tile
+  constexpr bool A_TWO = MODE != CONV_OUTP && A_ROWLANES == 32;    // a wavefront spans two kk rows
+  static_assert(MODE == CONV_OUTP || A_ROWLANES == 32 || A_ROWLANES == 64, "Up/Down tiles are 128 or 256 rows");
+  const int padw = p.pad0 < 0 ? -p.pad0 : 0;
+  const unsigned img_bias = (unsigned)N * (unsigned)(padw * H + padw);
+  unsigned hid_bias = 0;
+  if (MODE == CONV_DOWN) hid_bias = (unsigned)N * (unsigned)(ph.TY * Mx + ph.TX);
+  const char* a_base = nullptr;
+  const char* b_base = nullptr;
+  if (MODE == CONV_UP) a_base = reinterpret_cast<const char*>(p.img) - 4ll * img_bias;
+  if (MODE == CONV_DOWN) a_base = reinterpret_cast<const char*>(p.hid) - 4ll * hid_bias;
+  if (MODE == CONV_OUTP) b_base = reinterpret_cast<const char*>(p.img) - 4ll * img_bias;
+
   // A groups: Up/Down are row-contiguous (4 rows of one kk); Outp is kk-contiguous (4 kk of one row).
-  int a_k[NA], a_r[NA], a_y[NA], a_x[NA];
+  int a_k[NA], a_r[NA], a_y[NA], a_x[NA], a_ks[NA];
+  unsigned a_voff[NA];
   long long a_off[NA];
   bool a_ok[NA];
 #pragma unroll
   for (int u = 0; u < NA; ++u) {
     const int f = tid + u * 256;
     a_ok[u] = f < TA;
+    a_ks[u] = 0; a_voff[u] = 0; a_off[u] = 0;
     if (MODE == CONV_OUTP) {
       a_r[u] = f >> 2; a_k[u] = (f & 3) << 2;
       const int r = row0 + a_r[u];
@@ -214,7 +240,8 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
       a_off[u] = (long long)N * M * (g * Fg + r) + (long long)N * p.m_begin;
       a_y[u] = a_x[u] = 0;
     } else {
-      a_k[u] = f / (BM / 4); a_r[u] = (f % (BM / 4)) << 2;
+      a_k[u] = f / A_ROWLANES; a_r[u] = (f % A_ROWLANES) << 2;
+      a_ks[u] = (wvu * 64 + u * 256) / A_ROWLANES;                 // kk row of lanes 0-31 (scalar)
       const int r = row0 + a_r[u];
       a_ok[u] = a_ok[u] && r < rows;
       const int pos = (int)fd_div((uint32_t)r, p.dN);  // module (Up) or pixel-of-phase (Down)
@@ -222,22 +249,24 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
       if (MODE == CONV_UP) {
         const int my = (int)fd_div((uint32_t)pos, p.dMx), mx = pos - my * Mx;
         a_y[u] = my * s + p.pad0; a_x[u] = mx * s + p.pad0;
-        a_off[u] = (long long)N * ((long long)g * Cg * HH) + n;
+        a_voff[u] = 4u * (unsigned)(n + N * (a_y[u] * H + a_x[u]) + (int)img_bias);
       } else {
         const int qyi = ph.QX > 0 ? pos / ph.QX : 0, qxi = pos - qyi * ph.QX;
         a_y[u] = ph.qy_first + qyi; a_x[u] = ph.qx_first + qxi;  // module coordinate before the tap shift
-        a_off[u] = (long long)N * ((long long)g * Fg * M) + n;
+        a_voff[u] = 4u * (unsigned)(n + N * (a_y[u] * Mx + a_x[u]) + (A_TWO && lk ? N * M : 0));
       }
     }
   }
   // B groups: Up is column-contiguous (4 filters of one kk); Down/Outp are kk-contiguous.
   int b_k[NB], b_c[NB], b_y[NB], b_x[NB];
+  unsigned b_voff[NB];
   long long b_off[NB];
   bool b_ok[NB];
 #pragma unroll
   for (int u = 0; u < NB; ++u) {
     const int f = tid + u * 256;
     b_ok[u] = f < TB;
+    b_voff[u] = 0; b_off[u] = 0;
     if (MODE == CONV_UP) {
       b_k[u] = f / (BN / 4); b_c[u] = (f % (BN / 4)) << 2;
       const int c = col0 + b_c[u];
@@ -256,7 +285,7 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
         const int pp = c - cc * p.kk2;
         const int ky = (int)fd_div((uint32_t)pp, p.dk), kx = pp - ky * k;
         b_y[u] = p.pad0 + ky; b_x[u] = p.pad0 + kx;
-        b_off[u] = (long long)N * ((long long)(g * Cg + cc) * HH);
+        b_voff[u] = 4u * (unsigned)(N * ((g * Cg + cc) * HH + b_y[u] * H + b_x[u]) + b_k[u] + (int)img_bias);
       }
     }
   }
@@ -277,48 +306,71 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
   }
 
   float4 ra[NA], rb[NB];
+  bool ra_ok[NA], rb_ok[NB];
   const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
+  const int Kup = Cg * p.kk2;
 
+  // Every gather is an unconditional 16-byte load (see above); no load sits behind a
+  // branch, so all of a slab's loads are in flight together.
   auto fetch = [&](int slab) {
     const int kk0 = slab * CV_BK;
 #pragma unroll
     for (int u = 0; u < NA; ++u) {
-      ra[u] = zero4;
-      if (!a_ok[u]) continue;
+      bool ok = a_ok[u];
       if (MODE == CONV_UP) {
-        const int kk = kk0 + a_k[u];
-        if (kk < Cg * p.kk2) {
+        // scalar: where tap kk of this wavefront's row(s) lies relative to the module origin
+        int sy[2], sx[2];
+        unsigned so[2];
+        bool sv[2];
+#pragma unroll
+        for (int h = 0; h < (A_TWO ? 2 : 1); ++h) {
+          const int kk = kk0 + a_ks[u] + h;
           const int c = (int)fd_div((uint32_t)kk, p.dkk2);
           const int pp = kk - c * p.kk2;
-          const int ky = (int)fd_div((uint32_t)pp, p.dk), kx = pp - ky * k;
-          const int y = a_y[u] + ky, x = a_x[u] + kx;
-          if (y >= 0 && y < H && x >= 0 && x < H)
-            ra[u] = *reinterpret_cast<const float4*>(p.img + a_off[u] + (long long)N * (c * HH + y * H + x));
+          sy[h] = (int)fd_div((uint32_t)pp, p.dk); sx[h] = pp - sy[h] * k;
+          sv[h] = kk < Kup;
+          so[h] = 4u * (unsigned)N * (unsigned)((g * Cg + c) * HH + sy[h] * H + sx[h]);   // unused when !sv[h]
         }
+        const bool hi = A_TWO && lk;
+        const int y = a_y[u] + (hi ? sy[1] : sy[0]), x = a_x[u] + (hi ? sx[1] : sx[0]);
+        ok = ok & (hi ? sv[1] : sv[0]) & ((unsigned)y < (unsigned)H) & ((unsigned)x < (unsigned)H);
+        const unsigned voff = ok ? a_voff[u] + (hi ? so[1] : so[0]) : 4u * img_bias;
+        ra[u] = *reinterpret_cast<const float4*>(a_base + voff);
       } else if (MODE == CONV_DOWN) {
         const int my = a_y[u] - st_a, mx = a_x[u] - st_b;
-        if (my >= 0 && my < Mx && mx >= 0 && mx < Mx)
-          ra[u] = *reinterpret_cast<const float4*>(
-              p.hid + a_off[u] + (long long)N * ((long long)(st_c + a_k[u]) * M + my * Mx + mx));
+        ok = ok & ((unsigned)my < (unsigned)Mx) & ((unsigned)mx < (unsigned)Mx);
+        const unsigned so = 4u * ((unsigned)N * (unsigned)((g * Fg + st_c + a_ks[u]) * M - st_a * Mx - st_b) + hid_bias);  // scalar
+        const unsigned voff = ok ? a_voff[u] + so : 4u * hid_bias;
+        ra[u] = *reinterpret_cast<const float4*>(a_base + voff);
       } else {
-        ra[u] = *reinterpret_cast<const float4*>(p.hid + a_off[u] + (long long)(slab * CV_BK + a_k[u]));
+        const float* src = p.hid + a_off[u] + (long long)(slab * CV_BK + a_k[u]);
+        if (!ok) src = p.hid;
+        ra[u] = *reinterpret_cast<const float4*>(src);
       }
+      ra_ok[u] = ok;
     }
 #pragma unroll
     for (int u = 0; u < NB; ++u) {
-      rb[u] = zero4;
-      if (!b_ok[u]) continue;
+      bool ok = b_ok[u];
       if (MODE == CONV_UP) {
         const int kk = kk0 + b_k[u];
-        if (kk < Cg * p.kk2) rb[u] = *reinterpret_cast<const float4*>(p.flt + b_off[u] + (long long)F * kk);
+        ok = ok && kk < Kup;
+        const float* src = p.flt + b_off[u] + (long long)F * kk;
+        if (!ok) src = p.flt;
+        rb[u] = *reinterpret_cast<const float4*>(src);
       } else if (MODE == CONV_DOWN) {
         const int ky = ph.py + s * st_a, kx = ph.px + s * st_b;
-        rb[u] = *reinterpret_cast<const float4*>(p.flt + b_off[u] + (long long)F * (ky * k + kx) + st_c + b_k[u]);
+        const float* src = p.flt + b_off[u] + (long long)F * (ky * k + kx) + st_c + b_k[u];
+        if (!ok) src = p.flt;
+        rb[u] = *reinterpret_cast<const float4*>(src);
       } else {
         const int y = st_a * s + b_y[u], x = st_b * s + b_x[u];
-        if (y >= 0 && y < H && x >= 0 && x < H)
-          rb[u] = *reinterpret_cast<const float4*>(p.img + b_off[u] + (long long)N * (y * H + x) + st_c + b_k[u]);
+        ok = ok & ((unsigned)y < (unsigned)H) & ((unsigned)x < (unsigned)H);
+        const unsigned so = 4u * ((unsigned)N * (unsigned)(st_a * s * H + st_b * s) + (unsigned)st_c);  // scalar
+        const unsigned voff = ok ? b_voff[u] + so : 4u * img_bias;
+        rb[u] = *reinterpret_cast<const float4*>(b_base + voff);
       }
+      rb_ok[u] = ok;
     }
     // advance the uniform slab state
     if (MODE == CONV_DOWN) {
@@ -333,6 +385,7 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
 #pragma unroll
     for (int u = 0; u < NA; ++u) {
       if (tid + u * 256 >= TA) continue;
+      if (!ra_ok[u]) ra[u] = zero4;
       if (MODE == CONV_OUTP) {
         As[buf][a_k[u]][a_r[u]] = ra[u].x; As[buf][a_k[u] + 1][a_r[u]] = ra[u].y;
         As[buf][a_k[u] + 2][a_r[u]] = ra[u].z; As[buf][a_k[u] + 3][a_r[u]] = ra[u].w;
@@ -343,6 +396,7 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
 #pragma unroll
     for (int u = 0; u < NB; ++u) {
       if (tid + u * 256 >= TB) continue;
+      if (!rb_ok[u]) rb[u] = zero4;
       if (MODE == CONV_UP) {
         *reinterpret_cast<float4*>(&Bs[buf][b_k[u]][b_c[u]]) = rb[u];
       } else {
@@ -369,19 +423,26 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
   for (int slab = slab_beg; slab < slab_end; ++slab) {
     const bool more = slab + 1 < slab_end;
     if (more) fetch(slab + 1);
+    // All of the slab's fragments are asked of LDS first (the scheduling fences keep
+    // the compiler from sinking the reads back to their uses and from hoisting the
+    // wait for the next slab's gathers above the MFMAs).
+    float av[CV_BK / 2][WM], bv[CV_BK / 2][WN];
 #pragma unroll
     for (int kk = 0; kk < CV_BK / 2; ++kk) {  // rows kk and kk + BK/2: 32 banks apart, no conflict
-      float av[WM], bv[WN];
 #pragma unroll
-      for (int i = 0; i < WM; ++i) av[i] = As[buf][kk + (CV_BK / 2) * lk][(wm * WM + i) * 32 + li];
+      for (int i = 0; i < WM; ++i) av[kk][i] = As[buf][kk + (CV_BK / 2) * lk][(wm * WM + i) * 32 + li];
 #pragma unroll
-      for (int j = 0; j < WN; ++j) bv[j] = Bs[buf][kk + (CV_BK / 2) * lk][(wn * WN + j) * 32 + li];
+      for (int j = 0; j < WN; ++j) bv[kk][j] = Bs[buf][kk + (CV_BK / 2) * lk][(wn * WN + j) * 32 + li];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int kk = 0; kk < CV_BK / 2; ++kk)
 #pragma unroll
       for (int j = 0; j < WN; ++j)
 #pragma unroll
         for (int i = 0; i < WM; ++i)
-          acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[j], av[i], acc[j][i], 0, 0, 0);
-    }
+          acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[kk][j], av[kk][i], acc[j][i], 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
     if (more) stash(buf ^ 1);
     __syncthreads();
     buf ^= 1;
@@ -526,8 +587,10 @@ static int isqrt_exact(int v) {
 }
 
 static bool fast_ok(const ConvArgs& a) {
+  // (the gathers use 32-bit byte offsets that include a margin for the padding / tap shift)
+  const long long margin = (long long)a.N * ((long long)(a.k + (a.pad0 < 0 ? -a.pad0 : 0)) * (a.H + a.Mx) + a.k + a.H);
   return a.N % 16 == 0 && a.Fg % 16 == 0 && dn_aligned16(a.img) && dn_aligned16(a.flt) && dn_aligned16(a.hid) &&
-         (long long)a.N * a.M * a.F < (1ll << 31) && (long long)a.N * a.HH * a.C < (1ll << 31);
+         (long long)a.N * a.M * a.F + margin < (1ll << 30) && (long long)a.N * a.HH * a.C + margin < (1ll << 30);
 }
 
 static void fill_common(ConvArgs& a, int N, int C, int G, int H, int F, int k, int Mx, int s, int pad0) {
@@ -542,11 +605,21 @@ static void fill_common(ConvArgs& a, int N, int C, int G, int H, int F, int k, i
 template <int MODE>
 static void launch_rowmajor(const ConvArgs& a, long long rows, int cols, int gz) {
   // Up / Down: rows are plentiful, columns few: 4 wavefronts down the rows, WN blocks across.
+  // With enough rows to keep every CU busy twice over, each wavefront takes two row
+  // blocks (256-row tiles): twice the MFMAs per LDS read and per barrier.
+  const long long tiles256 = (rows + 255) / 256 * ((cols + 127) / 128) * gz;
+  if (tiles256 >= 2 * dn_num_cus() && cols <= 96) {  // (2 x 4 blocks per wavefront would leave one wavefront per SIMD)
+    const unsigned gx = (unsigned)((rows + 255) / 256);
+    if (cols <= 32) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 2, 1>), dim3(gx, (cols + 31) / 32, gz), dim3(256), 0, 0, a);
+    else if (cols <= 64) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 2, 2>), dim3(gx, (cols + 63) / 64, gz), dim3(256), 0, 0, a);
+    else hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 2, 3>), dim3(gx, (cols + 95) / 96, gz), dim3(256), 0, 0, a);
+    return;
+  }
   const unsigned gx = (unsigned)((rows + 127) / 128);
   if (cols <= 32) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 1>), dim3(gx, (cols + 31) / 32, gz), dim3(256), 0, 0, a);
   else if (cols <= 64) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 2>), dim3(gx, (cols + 63) / 64, gz), dim3(256), 0, 0, a);
   else if (cols <= 96) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 3>), dim3(gx, (cols + 95) / 96, gz), dim3(256), 0, 0, a);
-  else hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 4>), dim3(gx, (cols + 127) / 128, gz), dim3(256), 0, 0, a);
+  else hipLaunchKernelGGL((k_conv_mfma<MODE, 2, 2, 2>), dim3(gx, (cols + 127) / 128, gz), dim3(256), 0, 0, a);  // 64 x 64 per wavefront
 }
 
 static void conv_up_impl(cudamat* images, cudamat* filters, cudamat* targets, int numModulesX, int paddingStart,

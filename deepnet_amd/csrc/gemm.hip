@@ -14,6 +14,7 @@ int dn_gemv_cols(const float* M, int ld, int h, int w, const float* x, float* y,
 int dn_gemv_rows(const float* M, int ld, int h, int w, const float* x, float* y, float alpha, float beta);
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 #define GEMM_BK 16
 #define GEMM_PAD 4
@@ -21,13 +22,13 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 // Four consecutive floats along the contiguous index c (limit c_lim) at the
 // strided index o (limit o_lim); zero outside.  vec_ok: base and ld allow a
 // 16-byte load whenever the four are all inside.
-__device__ __forceinline__ float4 gemm_load4(const float* base, int c, int c_lim, int o, int o_lim, int ld,
+__device__ __forceinline__ f32x4 gemm_load4(const float* base, int c, int c_lim, int o, int o_lim, int ld,
                                              bool vec_ok) {
-  float4 r = make_float4(0.f, 0.f, 0.f, 0.f);
+  f32x4 r = {0.f, 0.f, 0.f, 0.f};
   if (o < o_lim) {
     const float* p = base + (size_t)o * ld + c;
     if (vec_ok && c + 3 < c_lim) {
-      r = *reinterpret_cast<const float4*>(p);
+      r = *reinterpret_cast<const f32x4*>(p);
     } else {
       if (c < c_lim) r.x = p[0];
       if (c + 1 < c_lim) r.y = p[1];
@@ -47,7 +48,10 @@ __global__ void __launch_bounds__(256)
 k_gemm(const float* __restrict__ A, int lda, const float* __restrict__ B, int ldb, float* C, int ldc, int M, int N,
        int K, int k_per_split, float alpha, float beta, float* partial, bool a_vec, bool b_vec) {
   constexpr int BM = 64 * WM, BN = 64 * WN;
-  constexpr int LA = BM + GEMM_PAD, LB = BN + GEMM_PAD;
+  // Row pitch in LDS: a k-contiguous operand is written transposed, one float per lane
+  // (lane = 4 k-quads x rows), which is free of bank conflicts when pitch % 8 == 2; the
+  // other kind is written 16 bytes at a time and needs pitch % 4 == 0.
+  constexpr int LA = BM + (A_KC ? 2 : GEMM_PAD), LB = BN + (B_KC ? 2 : GEMM_PAD);
   constexpr int A4 = BM * GEMM_BK / 4 / 256, B4 = BN * GEMM_BK / 4 / 256;  // float4 per lane per slab
   __shared__ __attribute__((aligned(16))) float As[2][GEMM_BK][LA];
   __shared__ __attribute__((aligned(16))) float Bs[2][GEMM_BK][LB];
@@ -66,40 +70,44 @@ k_gemm(const float* __restrict__ A, int lda, const float* __restrict__ B, int ld
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[j][i][v] = 0.f;
 
-  float4 ra[A4], rb[B4];
+  f32x4 ra[A4], rb[B4];    // slab on its way from global memory to LDS ...
+  f32x4 sa[A4], sb[B4];    // ... and, in the loop for interior tiles, the one after it
 
   // Tiles that lie wholly inside both operands, on 16-byte aligned data, fetch through
   // per-lane pointers that advance one slab at a time: no index arithmetic and no
   // branch around any load.  Edge tiles and the last partial slab take the checked path.
   const bool a_fast = a_vec && m0 + BM <= M, b_fast = b_vec && n0 + BN <= N;
-  const float* pa[A4];
-  const float* pb[B4];
+  typedef const __attribute__((address_space(1))) f32x4* gptr4;   // keeps the loads global_load, never flat
+  gptr4 pa[A4];
+  gptr4 pb[B4];
 #pragma unroll
   for (int u = 0; u < A4; ++u) {
     const int f = tid + u * 256;
-    if (A_KC) pa[u] = A + (size_t)(m0 + (f >> 2)) * lda + kbeg + ((f & 3) << 2);
-    else pa[u] = A + (size_t)(kbeg + f / (BM / 4)) * lda + m0 + ((f % (BM / 4)) << 2);
+    if (A_KC) pa[u] = (gptr4)(A + (size_t)(m0 + (f >> 2)) * lda + kbeg + ((f & 3) << 2));
+    else pa[u] = (gptr4)(A + (size_t)(kbeg + f / (BM / 4)) * lda + m0 + ((f % (BM / 4)) << 2));
   }
 #pragma unroll
   for (int u = 0; u < B4; ++u) {
     const int f = tid + u * 256;
-    if (B_KC) pb[u] = B + (size_t)(n0 + (f >> 2)) * ldb + kbeg + ((f & 3) << 2);
-    else pb[u] = B + (size_t)(kbeg + f / (BN / 4)) * ldb + n0 + ((f % (BN / 4)) << 2);
+    if (B_KC) pb[u] = (gptr4)(B + (size_t)(n0 + (f >> 2)) * ldb + kbeg + ((f & 3) << 2));
+    else pb[u] = (gptr4)(B + (size_t)(kbeg + f / (BN / 4)) * ldb + n0 + ((f % (BN / 4)) << 2));
   }
-  const size_t a_step = A_KC ? GEMM_BK : (size_t)GEMM_BK * lda, b_step = B_KC ? GEMM_BK : (size_t)GEMM_BK * ldb;
+  // steps in 16-byte units (the fast path has lda, ldb multiples of 4)
+  const size_t a_step = A_KC ? GEMM_BK / 4 : (size_t)(GEMM_BK / 4) * lda, b_step = B_KC ? GEMM_BK / 4 : (size_t)(GEMM_BK / 4) * ldb;
 
-  auto fetch_fast = [&]() {
-#pragma unroll
-    for (int u = 0; u < A4; ++u) {
-      ra[u] = *reinterpret_cast<const float4*>(pa[u]);
-      pa[u] += a_step;
-    }
-#pragma unroll
-    for (int u = 0; u < B4; ++u) {
-      rb[u] = *reinterpret_cast<const float4*>(pb[u]);
-      pb[u] += b_step;
-    }
-  };
+  // (macros rather than lambdas taking the register sets by reference: those made the
+  // compiler keep the sets in scratch memory)
+#define GEMM_FETCH_FAST(XA, XB)                                      \
+  do {                                                               \
+    _Pragma("unroll") for (int u = 0; u < A4; ++u) {                 \
+      XA[u] = *pa[u];                                                \
+      pa[u] += a_step;                                               \
+    }                                                                \
+    _Pragma("unroll") for (int u = 0; u < B4; ++u) {                 \
+      XB[u] = *pb[u];                                                \
+      pb[u] += b_step;                                               \
+    }                                                                \
+  } while (0)
   auto fetch_checked = [&](int k0) {
 #pragma unroll
     for (int u = 0; u < A4; ++u) {
@@ -124,32 +132,31 @@ k_gemm(const float* __restrict__ A, int lda, const float* __restrict__ B, int ld
       }
     }
   };
-  auto stash = [&](int buf) {
-#pragma unroll
-    for (int u = 0; u < A4; ++u) {
-      const int f = tid + u * 256;
-      if (A_KC) {
-        const int m = f >> 2, k = (f & 3) << 2;
-        As[buf][k][m] = ra[u].x; As[buf][k + 1][m] = ra[u].y;
-        As[buf][k + 2][m] = ra[u].z; As[buf][k + 3][m] = ra[u].w;
-      } else {
-        const int k = f / (BM / 4), m = (f % (BM / 4)) << 2;
-        *reinterpret_cast<float4*>(&As[buf][k][m]) = ra[u];
-      }
-    }
-#pragma unroll
-    for (int u = 0; u < B4; ++u) {
-      const int f = tid + u * 256;
-      if (B_KC) {
-        const int n = f >> 2, k = (f & 3) << 2;
-        Bs[buf][k][n] = rb[u].x; Bs[buf][k + 1][n] = rb[u].y;
-        Bs[buf][k + 2][n] = rb[u].z; Bs[buf][k + 3][n] = rb[u].w;
-      } else {
-        const int k = f / (BN / 4), n = (f % (BN / 4)) << 2;
-        *reinterpret_cast<float4*>(&Bs[buf][k][n]) = rb[u];
-      }
-    }
-  };
+#define GEMM_STASH(BUF, XA, XB)                                                     \
+  do {                                                                              \
+    _Pragma("unroll") for (int u = 0; u < A4; ++u) {                                \
+      const int f = tid + u * 256;                                                  \
+      if (A_KC) {                                                                   \
+        const int m = f >> 2, k = (f & 3) << 2;                                     \
+        As[BUF][k][m] = XA[u].x; As[BUF][k + 1][m] = XA[u].y;                       \
+        As[BUF][k + 2][m] = XA[u].z; As[BUF][k + 3][m] = XA[u].w;                   \
+      } else {                                                                      \
+        const int k = f / (BM / 4), m = (f % (BM / 4)) << 2;                        \
+        *reinterpret_cast<f32x4*>(&As[BUF][k][m]) = XA[u];                          \
+      }                                                                             \
+    }                                                                               \
+    _Pragma("unroll") for (int u = 0; u < B4; ++u) {                                \
+      const int f = tid + u * 256;                                                  \
+      if (B_KC) {                                                                   \
+        const int n = f >> 2, k = (f & 3) << 2;                                     \
+        Bs[BUF][k][n] = XB[u].x; Bs[BUF][k + 1][n] = XB[u].y;                       \
+        Bs[BUF][k + 2][n] = XB[u].z; Bs[BUF][k + 3][n] = XB[u].w;                   \
+      } else {                                                                      \
+        const int k = f / (BN / 4), n = (f % (BN / 4)) << 2;                        \
+        *reinterpret_cast<f32x4*>(&Bs[BUF][k][n]) = XB[u];                          \
+      }                                                                             \
+    }                                                                               \
+  } while (0)
 
   const int lk = lane >> 5, li = lane & 31;
   // One slab: all of its fragments are asked of LDS first (the scheduling fence keeps
@@ -180,26 +187,41 @@ k_gemm(const float* __restrict__ A, int lda, const float* __restrict__ B, int ld
   // the checked loop.
   const bool fast = a_fast && b_fast;
   int buf = 0, k0 = kbeg;
-  if (kbeg < kend) {
-    if (fast && kbeg + GEMM_BK <= kend) fetch_fast();
-    else fetch_checked(kbeg);
-    stash(0);
-  }
-  __syncthreads();
-  if (fast) {
-    for (; k0 + 2 * GEMM_BK <= kend; k0 += GEMM_BK) {
-      fetch_fast();
+  if (fast && kbeg + 2 * GEMM_BK <= kend) {
+    // Global loads run two slabs ahead of the MFMAs: while slab i is multiplied, slab
+    // i+1 (asked for one iteration ago) is written to LDS and slab i+2 is requested.
+    GEMM_FETCH_FAST(ra, rb);
+    GEMM_STASH(0, ra, rb);
+    GEMM_FETCH_FAST(ra, rb);
+    __syncthreads();
+    while (k0 + 4 * GEMM_BK <= kend) {   // two slabs per trip, so the two register sets swap roles statically
+      GEMM_FETCH_FAST(sa, sb);
       multiply(buf);
-      stash(buf ^ 1);
+      GEMM_STASH(buf ^ 1, ra, rb);
       __syncthreads();
-      buf ^= 1;
+      buf ^= 1; k0 += GEMM_BK;
+      GEMM_FETCH_FAST(ra, rb);
+      multiply(buf);
+      GEMM_STASH(buf ^ 1, sa, sb);
+      __syncthreads();
+      buf ^= 1; k0 += GEMM_BK;
     }
+    multiply(buf);
+    GEMM_STASH(buf ^ 1, ra, rb);
+    __syncthreads();
+    buf ^= 1; k0 += GEMM_BK;         // LDS now holds the full slab at k0, nothing is in flight
+  } else {
+    if (kbeg < kend) {
+      fetch_checked(kbeg);
+      GEMM_STASH(0, ra, rb);
+    }
+    __syncthreads();
   }
   for (; k0 < kend; k0 += GEMM_BK) {
     const bool more = k0 + GEMM_BK < kend;
     if (more) fetch_checked(k0 + GEMM_BK);
     multiply(buf);
-    if (more) stash(buf ^ 1);
+    if (more) GEMM_STASH(buf ^ 1, ra, rb);
     __syncthreads();
     buf ^= 1;
   }
@@ -225,6 +247,9 @@ k_gemm(const float* __restrict__ A, int lda, const float* __restrict__ B, int ld
       }
     }
 }
+
+#undef GEMM_FETCH_FAST
+#undef GEMM_STASH
 
 // Products too small to fill the chip with 64 x 64 tiles (the RBM / MLP layer shapes):
 // a workgroup owns one 32 x 32 block of C; its NW wavefronts each take every NW-th

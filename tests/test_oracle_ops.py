@@ -127,17 +127,13 @@ def test_fastdiv_magic_numbers_used_by_the_device_kernels():
     """The multiply-high division of deepnet_amd/csrc/common.h, restated, against // for
     awkward divisors and dividends up to 2^32 - 1."""
     def make(d):
-        if d <= 1:
-            return (0, 0, d)
         s = (d - 1).bit_length()
-        return ((((1 << 32) * ((1 << s) - d)) // d + 1) & 0xFFFFFFFF, s, d)
+        return ((((1 << 32) * ((1 << s) - d)) // d + 1) & 0xFFFFFFFF, min(s, 1), max(s - 1, 0), d)
 
     def div(n, f):
-        magic, s, d = f
-        if d <= 1:
-            return n
+        magic, sh1, sh2, d = f
         hi = (n * magic) >> 32
-        return ((hi + ((n - hi) >> 1)) & 0xFFFFFFFF) >> (s - 1)
+        return ((hi + ((n - hi) >> sh1)) & 0xFFFFFFFF) >> sh2
 
     rng = np.random.default_rng(0)
     for d in [1, 2, 3, 5, 7, 10, 37, 64, 100, 500, 784, 1023, 1024, 1025, 4096, 12288, 65537, 2 ** 31 - 1, 2 ** 31 + 3]:
