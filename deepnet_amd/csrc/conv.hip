@@ -24,11 +24,13 @@
 // 16-byte aligned buffers; anything else takes the one-thread-per-output kernels
 // below, which are also the cross-check of the fast path in the tests.
 #include "common.h"
+#include <type_traits>
 #include "../../include/cudamat_conv_amd.h"
 #include <math.h>
 #include <stdio.h>
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 enum { CONV_UP = 0, CONV_DOWN = 1, CONV_OUTP = 2 };
 
@@ -305,14 +307,19 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
     st_a = m / Mx; st_b = m - st_a * Mx;                  // my, mx
   }
 
-  float4 ra[NA], rb[NB];
-  bool ra_ok[NA], rb_ok[NB];
-  const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
+  // Two register sets: the gathers run two slabs ahead of the MFMAs.  SET is a
+  // compile-time constant so that every index into them is one too.
+  f32x4 ra[2][NA], rb[2][NB];
+  bool ra_ok[2][NA], rb_ok[2][NB];
+  const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+  typedef std::integral_constant<int, 0> Set0;
+  typedef std::integral_constant<int, 1> Set1;
   const int Kup = Cg * p.kk2;
 
   // Every gather is an unconditional 16-byte load (see above); no load sits behind a
   // branch, so all of a slab's loads are in flight together.
-  auto fetch = [&](int slab) {
+  auto fetch = [&](auto set_tag, int slab) {
+    constexpr int SET = decltype(set_tag)::value;
     const int kk0 = slab * CV_BK;
 #pragma unroll
     for (int u = 0; u < NA; ++u) {
@@ -335,19 +342,19 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
         const int y = a_y[u] + (hi ? sy[1] : sy[0]), x = a_x[u] + (hi ? sx[1] : sx[0]);
         ok = ok & (hi ? sv[1] : sv[0]) & ((unsigned)y < (unsigned)H) & ((unsigned)x < (unsigned)H);
         const unsigned voff = ok ? a_voff[u] + (hi ? so[1] : so[0]) : 4u * img_bias;
-        ra[u] = *reinterpret_cast<const float4*>(a_base + voff);
+        ra[SET][u] = *reinterpret_cast<const f32x4*>(a_base + voff);
       } else if (MODE == CONV_DOWN) {
         const int my = a_y[u] - st_a, mx = a_x[u] - st_b;
         ok = ok & ((unsigned)my < (unsigned)Mx) & ((unsigned)mx < (unsigned)Mx);
         const unsigned so = 4u * ((unsigned)N * (unsigned)((g * Fg + st_c + a_ks[u]) * M - st_a * Mx - st_b) + hid_bias);  // scalar
         const unsigned voff = ok ? a_voff[u] + so : 4u * hid_bias;
-        ra[u] = *reinterpret_cast<const float4*>(a_base + voff);
+        ra[SET][u] = *reinterpret_cast<const f32x4*>(a_base + voff);
       } else {
         const float* src = p.hid + a_off[u] + (long long)(slab * CV_BK + a_k[u]);
         if (!ok) src = p.hid;
-        ra[u] = *reinterpret_cast<const float4*>(src);
+        ra[SET][u] = *reinterpret_cast<const f32x4*>(src);
       }
-      ra_ok[u] = ok;
+      ra_ok[SET][u] = ok;
     }
 #pragma unroll
     for (int u = 0; u < NB; ++u) {
@@ -357,20 +364,20 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
         ok = ok && kk < Kup;
         const float* src = p.flt + b_off[u] + (long long)F * kk;
         if (!ok) src = p.flt;
-        rb[u] = *reinterpret_cast<const float4*>(src);
+        rb[SET][u] = *reinterpret_cast<const f32x4*>(src);
       } else if (MODE == CONV_DOWN) {
         const int ky = ph.py + s * st_a, kx = ph.px + s * st_b;
         const float* src = p.flt + b_off[u] + (long long)F * (ky * k + kx) + st_c + b_k[u];
         if (!ok) src = p.flt;
-        rb[u] = *reinterpret_cast<const float4*>(src);
+        rb[SET][u] = *reinterpret_cast<const f32x4*>(src);
       } else {
         const int y = st_a * s + b_y[u], x = st_b * s + b_x[u];
         ok = ok & ((unsigned)y < (unsigned)H) & ((unsigned)x < (unsigned)H);
         const unsigned so = 4u * ((unsigned)N * (unsigned)(st_a * s * H + st_b * s) + (unsigned)st_c);  // scalar
         const unsigned voff = ok ? b_voff[u] + so : 4u * img_bias;
-        rb[u] = *reinterpret_cast<const float4*>(b_base + voff);
+        rb[SET][u] = *reinterpret_cast<const f32x4*>(b_base + voff);
       }
-      rb_ok[u] = ok;
+      rb_ok[SET][u] = ok;
     }
     // advance the uniform slab state
     if (MODE == CONV_DOWN) {
@@ -381,27 +388,28 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
       if (st_c == N) { st_c = 0; if (++st_b == Mx) { st_b = 0; ++st_a; } }
     }
   };
-  auto stash = [&](int buf) {
+  auto stash = [&](auto set_tag, int buf) {
+    constexpr int SET = decltype(set_tag)::value;
 #pragma unroll
     for (int u = 0; u < NA; ++u) {
       if (tid + u * 256 >= TA) continue;
-      if (!ra_ok[u]) ra[u] = zero4;
+      if (!ra_ok[SET][u]) ra[SET][u] = zero4;
       if (MODE == CONV_OUTP) {
-        As[buf][a_k[u]][a_r[u]] = ra[u].x; As[buf][a_k[u] + 1][a_r[u]] = ra[u].y;
-        As[buf][a_k[u] + 2][a_r[u]] = ra[u].z; As[buf][a_k[u] + 3][a_r[u]] = ra[u].w;
+        As[buf][a_k[u]][a_r[u]] = ra[SET][u].x; As[buf][a_k[u] + 1][a_r[u]] = ra[SET][u].y;
+        As[buf][a_k[u] + 2][a_r[u]] = ra[SET][u].z; As[buf][a_k[u] + 3][a_r[u]] = ra[SET][u].w;
       } else {
-        *reinterpret_cast<float4*>(&As[buf][a_k[u]][a_r[u]]) = ra[u];
+        *reinterpret_cast<f32x4*>(&As[buf][a_k[u]][a_r[u]]) = ra[SET][u];
       }
     }
 #pragma unroll
     for (int u = 0; u < NB; ++u) {
       if (tid + u * 256 >= TB) continue;
-      if (!rb_ok[u]) rb[u] = zero4;
+      if (!rb_ok[SET][u]) rb[SET][u] = zero4;
       if (MODE == CONV_UP) {
-        *reinterpret_cast<float4*>(&Bs[buf][b_k[u]][b_c[u]]) = rb[u];
+        *reinterpret_cast<f32x4*>(&Bs[buf][b_k[u]][b_c[u]]) = rb[SET][u];
       } else {
-        Bs[buf][b_k[u]][b_c[u]] = rb[u].x; Bs[buf][b_k[u] + 1][b_c[u]] = rb[u].y;
-        Bs[buf][b_k[u] + 2][b_c[u]] = rb[u].z; Bs[buf][b_k[u] + 3][b_c[u]] = rb[u].w;
+        Bs[buf][b_k[u]][b_c[u]] = rb[SET][u].x; Bs[buf][b_k[u] + 1][b_c[u]] = rb[SET][u].y;
+        Bs[buf][b_k[u] + 2][b_c[u]] = rb[SET][u].z; Bs[buf][b_k[u] + 3][b_c[u]] = rb[SET][u].w;
       }
     }
   };
@@ -414,21 +422,13 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[j][i][v] = 0.f;
 
-  int buf = 0;
-  if (slab_beg < slab_end) {
-    fetch(slab_beg);
-    stash(0);
-  }
-  __syncthreads();
-  for (int slab = slab_beg; slab < slab_end; ++slab) {
-    const bool more = slab + 1 < slab_end;
-    if (more) fetch(slab + 1);
-    // All of the slab's fragments are asked of LDS first (the scheduling fences keep
-    // the compiler from sinking the reads back to their uses and from hoisting the
-    // wait for the next slab's gathers above the MFMAs).
+  // One slab: all of its fragments are asked of LDS first (the scheduling fences keep
+  // the compiler from sinking the reads back to their uses and from hoisting the wait
+  // for the gathers in flight above the MFMAs).
+  auto multiply = [&](int buf) {
     float av[CV_BK / 2][WM], bv[CV_BK / 2][WN];
 #pragma unroll
-    for (int kk = 0; kk < CV_BK / 2; ++kk) {  // rows kk and kk + BK/2: 32 banks apart, no conflict
+    for (int kk = 0; kk < CV_BK / 2; ++kk) {
 #pragma unroll
       for (int i = 0; i < WM; ++i) av[kk][i] = As[buf][kk + (CV_BK / 2) * lk][(wm * WM + i) * 32 + li];
 #pragma unroll
@@ -443,7 +443,48 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
         for (int i = 0; i < WM; ++i)
           acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[kk][j], av[kk][i], acc[j][i], 0, 0, 0);
     __builtin_amdgcn_sched_barrier(0);
-    if (more) stash(buf ^ 1);
+  };
+
+  // While slab i is multiplied, slab i+1 (asked for one iteration ago) is written to
+  // LDS and slab i+2 is requested; two slabs per trip so the register sets swap roles
+  // statically.  fetch() is always called with consecutive slabs.
+  // (Measured: the deeper prefetch pays for Outp, whose K runs over modules and images;
+  // for Up and Down its extra registers cost more than it hides.)
+  constexpr bool TWO_AHEAD = MODE == CONV_OUTP;
+  int buf = 0, slab = slab_beg;
+  if (TWO_AHEAD && slab_end - slab_beg >= 2) {
+    fetch(Set0(), slab);
+    stash(Set0(), 0);
+    fetch(Set0(), slab + 1);
+    __syncthreads();
+    while (slab + 4 <= slab_end) {
+      fetch(Set1(), slab + 2);
+      multiply(buf);
+      stash(Set0(), buf ^ 1);
+      __syncthreads();
+      buf ^= 1; ++slab;
+      fetch(Set0(), slab + 2);
+      multiply(buf);
+      stash(Set1(), buf ^ 1);
+      __syncthreads();
+      buf ^= 1; ++slab;
+    }
+    multiply(buf);
+    stash(Set0(), buf ^ 1);
+    __syncthreads();
+    buf ^= 1; ++slab;                // LDS holds slab `slab`, nothing is in flight
+  } else {
+    if (slab_beg < slab_end) {
+      fetch(Set0(), slab_beg);
+      stash(Set0(), 0);
+    }
+    __syncthreads();
+  }
+  for (; slab < slab_end; ++slab) {
+    const bool more = slab + 1 < slab_end;
+    if (more) fetch(Set0(), slab + 1);
+    multiply(buf);
+    if (more) stash(Set0(), buf ^ 1);
     __syncthreads();
     buf ^= 1;
   }

@@ -128,9 +128,61 @@ k_pool_undo(const float* imgs, const float* maxGrads, const float* maxActs, floa
   }
 }
 
+// x^y for the normalisation layers through the hardware log2 / exp2 (the reference uses
+// __powf there, cudamat_conv_kernels.cu:112-176); relative error below 1e-6 for the
+// denominators these layers see (1 <= x < ~1e3).
+__device__ __forceinline__ float norm_pow(float x, float y) {
+  return __builtin_amdgcn_exp2f(y * __builtin_amdgcn_logf(x));
+}
+
+// Sum of v (or v*v) over the part of the size x size window with origin (oy, ox) that
+// lies inside the S x S map.  For the usual window sizes (SIZE > 0, compile time) every
+// load is unconditional, from coordinates clamped into the map, and a row of loads is
+// in flight at once; what fell outside is dropped by a select.  SIZE == 0: any size.
+template <int VW, int SIZE, bool SQUARE>
+__device__ __forceinline__ Vec<VW> window_sum(const float* base, int N, int S, int oy, int ox, int size) {
+  Vec<VW> acc;
+#pragma unroll
+  for (int i = 0; i < VW; ++i) acc.v[i] = 0.f;
+  if (SIZE > 0) {
+#pragma unroll
+    for (int dy = 0; dy < SIZE; ++dy) {
+      const int y = oy + dy;
+      const bool vy = (unsigned)y < (unsigned)S;
+      const int yc = y < 0 ? 0 : (y >= S ? S - 1 : y);
+      Vec<VW> v[SIZE > 0 ? SIZE : 1];
+#pragma unroll
+      for (int dx = 0; dx < SIZE; ++dx) {
+        const int x = ox + dx;
+        const int xc = x < 0 ? 0 : (x >= S ? S - 1 : x);
+        v[dx] = Vec<VW>::load(base + (size_t)N * (yc * S + xc));
+      }
+#pragma unroll
+      for (int dx = 0; dx < SIZE; ++dx) {
+        const bool ok = vy & ((unsigned)(ox + dx) < (unsigned)S);
+#pragma unroll
+        for (int i = 0; i < VW; ++i) {
+          const float t = SQUARE ? v[dx].v[i] * v[dx].v[i] : v[dx].v[i];
+          acc.v[i] += ok ? t : 0.f;
+        }
+      }
+    }
+  } else {
+    const int y0 = oy > 0 ? oy : 0, x0 = ox > 0 ? ox : 0;
+    const int y1 = oy + size < S ? oy + size : S, x1 = ox + size < S ? ox + size : S;
+    for (int y = y0; y < y1; ++y)
+      for (int x = x0; x < x1; ++x) {
+        const Vec<VW> v = Vec<VW>::load(base + (size_t)N * (y * S + x));
+#pragma unroll
+        for (int i = 0; i < VW; ++i) acc.v[i] += SQUARE ? v.v[i] * v.v[i] : v.v[i];
+      }
+  }
+  return acc;
+}
+
 // denoms = 1 + addScale * sum over the clipped sizeX x sizeX window (origin -sizeX/2)
 // of meanDiffs^2;  target = imgs * denoms^-powScale   (cudamat_conv_kernels.cu:112-176).
-template <int VW>
+template <int VW, int SIZE>
 __global__ void __launch_bounds__(256)
 k_cnorm(const float* imgs, const float* meanDiffs, float* denoms, float* target, PoolGeom g, int sizeX, float addScale,
         float powScale) {
@@ -138,29 +190,104 @@ k_cnorm(const float* imgs, const float* meanDiffs, float* denoms, float* target,
   for (uint32_t e = blockIdx.x * 256u + threadIdx.x; e < total; e += gridDim.x * 256u) {
     int nv, px, py, f;
     decode4(e, g.dNV, g.dS, g.S, &nv, &px, &py, &f);
-    const int sx = px - sizeX / 2, sy = py - sizeX / 2;
-    const int x0 = sx > 0 ? sx : 0, y0 = sy > 0 ? sy : 0;
-    const int x1 = sx + sizeX < g.S ? sx + sizeX : g.S, y1 = sy + sizeX < g.S ? sy + sizeX : g.S;
     const float* base = meanDiffs + (size_t)g.N * ((size_t)f * g.S * g.S) + nv * VW;
-    Vec<VW> acc;
-#pragma unroll
-    for (int i = 0; i < VW; ++i) acc.v[i] = 0.f;
-    for (int y = y0; y < y1; ++y)
-      for (int x = x0; x < x1; ++x) {
-        const Vec<VW> v = Vec<VW>::load(base + (size_t)g.N * (y * g.S + x));
-#pragma unroll
-        for (int i = 0; i < VW; ++i) acc.v[i] += v.v[i] * v.v[i];
-      }
+    const Vec<VW> acc = window_sum<VW, SIZE, true>(base, g.N, g.S, py - sizeX / 2, px - sizeX / 2, sizeX);
     const size_t poff = (size_t)g.N * ((size_t)(f * g.S + py) * g.S + px) + nv * VW;
     const Vec<VW> in = Vec<VW>::load(imgs + poff);
     Vec<VW> d, t;
 #pragma unroll
     for (int i = 0; i < VW; ++i) {
       d.v[i] = 1.f + addScale * acc.v[i];
-      t.v[i] = in.v[i] * dn_pow(d.v[i], -powScale);
+      t.v[i] = in.v[i] * norm_pow(d.v[i], -powScale);
     }
     d.store(denoms + poff);
     t.store(target + poff);
+  }
+}
+
+// The same two layers for the usual window sizes, with a sliding window in registers: a
+// lane owns SEG consecutive rows of one column of one map (for VW images), sums each
+// window row once (SIZE loads) and adds up the SIZE most recent row sums per output, so
+// an output costs (SEG + SIZE - 1) * SIZE / SEG loads instead of SIZE * SIZE.
+// UNDO == false: denoms / target of the forward pass (window origin -SIZE/2, squares);
+// UNDO == true: the backward pass over the prepared acts (mirrored window, plain sums).
+template <int VW, int SIZE, int SEG, bool UNDO>
+__global__ void __launch_bounds__(256)
+k_norm_rows(const float* a0, const float* a1, const float* a2, const float* win, float* out0, float* out1, PoolGeom g,
+            int nseg, FastDiv dseg, float addScale, float powScale) {
+  // forward: a0 = imgs, win = meanDiffs, out0 = denoms, out1 = target
+  // backward: a0 = outGrads, a1 = denoms, a2 = inputs, win = acts, out1 = target
+  constexpr int ORG = UNDO ? SIZE / 2 - SIZE + 1 : -(SIZE / 2);
+  const int S = g.S, N = g.N;
+  const uint32_t total = (uint32_t)g.NV * S * nseg * g.F;
+  for (uint32_t e = blockIdx.x * 256u + threadIdx.x; e < total; e += gridDim.x * 256u) {
+    uint32_t q = fd_div(e, g.dNV);
+    const int nv = (int)(e - q * g.dNV.d);
+    uint32_t q2 = fd_div(q, g.dS);
+    const int px = (int)(q - q2 * (uint32_t)S);
+    const uint32_t f = fd_div(q2, dseg);
+    const int y0 = (int)(q2 - f * (uint32_t)nseg) * SEG;
+    const float* base = win + (size_t)N * ((size_t)f * S * S) + nv * VW;
+    // clamped column offsets and their validity, shared by all rows
+    int xoff[SIZE];
+    bool xok[SIZE];
+#pragma unroll
+    for (int dx = 0; dx < SIZE; ++dx) {
+      const int x = px + ORG + dx;
+      xok[dx] = (unsigned)x < (unsigned)S;
+      xoff[dx] = N * (x < 0 ? 0 : (x >= S ? S - 1 : x));
+    }
+    Vec<VW> ring[SIZE];
+#pragma unroll
+    for (int j = 0; j < SEG + SIZE - 1; ++j) {
+      const int y = y0 + ORG + j;
+      const bool yok = (unsigned)y < (unsigned)S;
+      const float* row = base + (size_t)N * S * (y < 0 ? 0 : (y >= S ? S - 1 : y));
+      Vec<VW> v[SIZE];
+#pragma unroll
+      for (int dx = 0; dx < SIZE; ++dx) v[dx] = Vec<VW>::load(row + xoff[dx]);
+      Vec<VW> rs;
+#pragma unroll
+      for (int i = 0; i < VW; ++i) rs.v[i] = 0.f;
+#pragma unroll
+      for (int dx = 0; dx < SIZE; ++dx) {
+        const bool ok = yok & xok[dx];
+#pragma unroll
+        for (int i = 0; i < VW; ++i) {
+          const float t = UNDO ? v[dx].v[i] : v[dx].v[i] * v[dx].v[i];
+          rs.v[i] += ok ? t : 0.f;
+        }
+      }
+      ring[j % SIZE] = rs;
+      if (j >= SIZE - 1) {
+        const int py = y0 + j - (SIZE - 1);
+        if (py < S) {
+          Vec<VW> acc = ring[0];
+#pragma unroll
+          for (int r = 1; r < SIZE; ++r)
+#pragma unroll
+            for (int i = 0; i < VW; ++i) acc.v[i] += ring[r].v[i];
+          const size_t poff = (size_t)N * ((size_t)(f * S + py) * S + px) + nv * VW;
+          if (!UNDO) {
+            const Vec<VW> in = Vec<VW>::load(a0 + poff);
+            Vec<VW> d, t;
+#pragma unroll
+            for (int i = 0; i < VW; ++i) {
+              d.v[i] = 1.f + addScale * acc.v[i];
+              t.v[i] = in.v[i] * norm_pow(d.v[i], -powScale);
+            }
+            d.store(out0 + poff);
+            t.store(out1 + poff);
+          } else {
+            const Vec<VW> og = Vec<VW>::load(a0 + poff), den = Vec<VW>::load(a1 + poff), inp = Vec<VW>::load(a2 + poff);
+            Vec<VW> t;
+#pragma unroll
+            for (int i = 0; i < VW; ++i) t.v[i] = inp.v[i] * acc.v[i] + og.v[i] * norm_pow(den.v[i], -powScale);
+            t.store(out1 + poff);
+          }
+        }
+      }
+    }
   }
 }
 
@@ -174,7 +301,7 @@ k_rnorm_undo_prelim(float* acts, const float* denoms, const float* outGrads, siz
 
 // target = inputs * (sum of the prepared acts over the mirrored window) + outGrads * denoms^-powScale
 // (cudamat_conv_kernels.cuh:1920-2004); the window of pixel p is [p + sizeX/2 - sizeX + 1, p + sizeX/2].
-template <int VW>
+template <int VW, int SIZE>
 __global__ void __launch_bounds__(256)
 k_rnorm_undo(const float* outGrads, const float* denoms, const float* inputs, const float* acts, float* target,
              PoolGeom g, int sizeX, float powScale) {
@@ -182,31 +309,22 @@ k_rnorm_undo(const float* outGrads, const float* denoms, const float* inputs, co
   for (uint32_t e = blockIdx.x * 256u + threadIdx.x; e < total; e += gridDim.x * 256u) {
     int nv, px, py, f;
     decode4(e, g.dNV, g.dS, g.S, &nv, &px, &py, &f);
-    const int sy = py + sizeX / 2 - sizeX + 1, sx = px + sizeX / 2 - sizeX + 1;
-    const int y0 = sy > 0 ? sy : 0, x0 = sx > 0 ? sx : 0;
-    const int y1 = py + sizeX / 2 + 1 < g.S ? py + sizeX / 2 + 1 : g.S;
-    const int x1 = px + sizeX / 2 + 1 < g.S ? px + sizeX / 2 + 1 : g.S;
     const float* base = acts + (size_t)g.N * ((size_t)f * g.S * g.S) + nv * VW;
-    Vec<VW> acc;
-#pragma unroll
-    for (int i = 0; i < VW; ++i) acc.v[i] = 0.f;
-    for (int y = y0; y < y1; ++y)
-      for (int x = x0; x < x1; ++x) {
-        const Vec<VW> v = Vec<VW>::load(base + (size_t)g.N * (y * g.S + x));
-#pragma unroll
-        for (int i = 0; i < VW; ++i) acc.v[i] += v.v[i];
-      }
+    const Vec<VW> acc =
+        window_sum<VW, SIZE, false>(base, g.N, g.S, py + sizeX / 2 - sizeX + 1, px + sizeX / 2 - sizeX + 1, sizeX);
     const size_t poff = (size_t)g.N * ((size_t)(f * g.S + py) * g.S + px) + nv * VW;
     const Vec<VW> inp = Vec<VW>::load(inputs + poff), og = Vec<VW>::load(outGrads + poff),
                   den = Vec<VW>::load(denoms + poff);
     Vec<VW> t;
 #pragma unroll
-    for (int i = 0; i < VW; ++i) t.v[i] = inp.v[i] * acc.v[i] + og.v[i] * dn_pow(den.v[i], -powScale);
+    for (int i = 0; i < VW; ++i) t.v[i] = inp.v[i] * acc.v[i] + og.v[i] * norm_pow(den.v[i], -powScale);
     t.store(target + poff);
   }
 }
 
 // ------------------------------------------------------------------ host side
+
+#define NORM_SEG 5   // rows per lane in k_norm_rows
 
 static int isqrt_exact_p(int v) {
   if (v < 0) return -1;
@@ -280,14 +398,26 @@ static void cnorm_impl(cudamat* images, cudamat* meanDiffs, cudamat* denoms, cud
   PoolGeom g;
   make_geom(g, N, numFilters, S, S, 0, 0, 1, v4 ? 4 : 1);
   const unsigned grid = grid_for(total / (v4 ? 4 : 1));
-  if (v4)
-    hipLaunchKernelGGL((k_cnorm<4>), dim3(grid), dim3(256), 0, 0, (const float*)images->data_device,
-                       (const float*)meanDiffs->data_device, denoms->data_device, targets->data_device, g, sizeX,
-                       addScale, powScale);
-  else
-    hipLaunchKernelGGL((k_cnorm<1>), dim3(grid), dim3(256), 0, 0, (const float*)images->data_device,
-                       (const float*)meanDiffs->data_device, denoms->data_device, targets->data_device, g, sizeX,
-                       addScale, powScale);
+#define CNORM_GO(VW, SZ)                                                                                       \
+  hipLaunchKernelGGL((k_cnorm<VW, SZ>), dim3(grid), dim3(256), 0, 0, (const float*)images->data_device,         \
+                     (const float*)meanDiffs->data_device, denoms->data_device, targets->data_device, g, sizeX, \
+                     addScale, powScale)
+#define CNORM_ROWS(SZ)                                                                                          \
+  hipLaunchKernelGGL((k_norm_rows<4, SZ, NORM_SEG, false>), dim3(grid_for((long long)g.NV * S * nseg * numFilters)), \
+                     dim3(256), 0, 0, (const float*)images->data_device, (const float*)nullptr,                  \
+                     (const float*)nullptr, (const float*)meanDiffs->data_device, denoms->data_device,           \
+                     targets->data_device, g, nseg, make_fastdiv((uint32_t)nseg), addScale, powScale)
+  const int nseg = (S + NORM_SEG - 1) / NORM_SEG;
+  if (v4) {
+    if (sizeX == 3) CNORM_ROWS(3);
+    else if (sizeX == 5) CNORM_ROWS(5);
+    else if (sizeX == 7) CNORM_ROWS(7);
+    else CNORM_GO(4, 0);
+  } else {
+    CNORM_GO(1, 0);
+  }
+#undef CNORM_GO
+#undef CNORM_ROWS
   if (dn_launch_status()) conv_set_error(where, hipGetErrorString(hipGetLastError()));
 }
 
@@ -313,14 +443,26 @@ static void rnorm_undo_impl(cudamat* outGrads, cudamat* denoms, cudamat* inputs,
   PoolGeom g;
   make_geom(g, N, numFilters, S, S, 0, 0, 1, v4 ? 4 : 1);
   const unsigned grid = grid_for(total / (v4 ? 4 : 1));
-  if (v4)
-    hipLaunchKernelGGL((k_rnorm_undo<4>), dim3(grid), dim3(256), 0, 0, (const float*)outGrads->data_device,
-                       (const float*)denoms->data_device, (const float*)inputs->data_device,
-                       (const float*)acts->data_device, targets->data_device, g, sizeX, powScale);
-  else
-    hipLaunchKernelGGL((k_rnorm_undo<1>), dim3(grid), dim3(256), 0, 0, (const float*)outGrads->data_device,
-                       (const float*)denoms->data_device, (const float*)inputs->data_device,
-                       (const float*)acts->data_device, targets->data_device, g, sizeX, powScale);
+#define RUNDO_GO(VW, SZ)                                                                                      \
+  hipLaunchKernelGGL((k_rnorm_undo<VW, SZ>), dim3(grid), dim3(256), 0, 0, (const float*)outGrads->data_device, \
+                     (const float*)denoms->data_device, (const float*)inputs->data_device,                     \
+                     (const float*)acts->data_device, targets->data_device, g, sizeX, powScale)
+#define RUNDO_ROWS(SZ)                                                                                         \
+  hipLaunchKernelGGL((k_norm_rows<4, SZ, NORM_SEG, true>), dim3(grid_for((long long)g.NV * S * nseg * numFilters)), \
+                     dim3(256), 0, 0, (const float*)outGrads->data_device, (const float*)denoms->data_device,   \
+                     (const float*)inputs->data_device, (const float*)acts->data_device, (float*)nullptr,       \
+                     targets->data_device, g, nseg, make_fastdiv((uint32_t)nseg), 0.f, powScale)
+  const int nseg = (S + NORM_SEG - 1) / NORM_SEG;
+  if (v4) {
+    if (sizeX == 3) RUNDO_ROWS(3);
+    else if (sizeX == 5) RUNDO_ROWS(5);
+    else if (sizeX == 7) RUNDO_ROWS(7);
+    else RUNDO_GO(4, 0);
+  } else {
+    RUNDO_GO(1, 0);
+  }
+#undef RUNDO_GO
+#undef RUNDO_ROWS
   if (dn_launch_status()) conv_set_error(where, hipGetErrorString(hipGetLastError()));
 }
 

@@ -306,6 +306,8 @@ def _window_sum(t, size, lo_off):
     out = np.zeros_like(t)
     for dy in range(lo_off, lo_off + size):
         for dx in range(lo_off, lo_off + size):
+            if abs(dy) >= S or abs(dx) >= S:
+                continue            # this shift moves the whole map out of the window
             ys, xs = slice(max(0, -dy), min(S, S - dy)), slice(max(0, -dx), min(S, S - dx))
             yd, xd = slice(max(0, dy), min(S, S + dy)), slice(max(0, dx), min(S, S + dx))
             out[..., ys, xs] += t[..., yd, xd]

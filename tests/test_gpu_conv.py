@@ -138,7 +138,8 @@ def test_prob_max_pool_follows_the_reference_scan(cm, cc, rng):
     assert np.array_equal(T.asarray(), co.prob_max_pool(x, r, F, 2, 0, 2, 3).astype(np.float32))
 
 
-@pytest.mark.parametrize("N,F,S,size", [(2, 3, 7, 3), (16, 16, 15, 5), (5, 4, 6, 4), (128, 64, 15, 5)])
+@pytest.mark.parametrize("N,F,S,size", [(2, 3, 7, 3), (16, 16, 15, 5), (5, 4, 6, 4), (128, 64, 15, 5),
+                                      (8, 4, 9, 3), (8, 2, 5, 7), (12, 3, 8, 4), (4, 2, 3, 9)])
 def test_response_norm_and_undo(cm, cc, rng, N, F, S, size):
     a, p = 0.001, 0.75
     x = _f(rng.standard_normal((N, F * S * S)) * 3)
@@ -146,7 +147,7 @@ def test_response_norm_and_undo(cm, cc, rng, N, F, S, size):
     cc.ResponseNorm(X, D, T, F, size, a, p)
     t_want, d_want = co.response_norm(x, F, size, a, p)
     assert np.allclose(D.asarray(), d_want, rtol=2e-6)
-    assert np.allclose(T.asarray(), t_want, rtol=2e-6, atol=1e-7)
+    assert np.allclose(T.asarray(), t_want, rtol=1e-5, atol=1e-7)    # hardware log2/exp2 pow, like the reference's __powf
     g = _f(rng.standard_normal(x.shape))
     acts = cm.CUDAMatrix(T.asarray().copy(order='F'))
     U = cm.empty(x.shape)
@@ -158,7 +159,7 @@ def test_response_norm_and_undo(cm, cc, rng, N, F, S, size):
     md = _f(rng.standard_normal(x.shape))
     cc.ContrastNorm(X, cm.CUDAMatrix(md), D, T, F, size, a, p)
     t2, d2 = co.contrast_norm(x, md, F, size, a, p)
-    assert np.allclose(D.asarray(), d2, rtol=2e-6) and np.allclose(T.asarray(), t2, rtol=2e-6, atol=1e-7)
+    assert np.allclose(D.asarray(), d2, rtol=2e-6) and np.allclose(T.asarray(), t2, rtol=1e-5, atol=1e-7)
 
 
 def test_conv_layer_chain_like_deepnet(cm, cc, rng):
