@@ -397,30 +397,33 @@ k_rows_stage1(const float* M, int ld, int h, int w, int cps, const float* x, flo
   }
 }
 
-// Stage 2: 64 rows per workgroup; its 4 wavefronts take every 4th split, four
-// loads in flight each, and meet in LDS (the order of the additions is fixed).
+// Stage 2: 16 rows per workgroup, 16 lane groups take every 16th split (all of a lane's
+// loads in flight at once for up to 64 splits) and meet in LDS; the order of the
+// additions is fixed.
 template <int OP>
 __global__ void __launch_bounds__(256)
 k_rows_stage2(const float* partial, int splits, int h, float* y, float alpha, float beta) {
-  __shared__ float sv[4][64];
-  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-  const int row = blockIdx.x * 64 + lane;
+  __shared__ float sv[16][17];
+  const int r = threadIdx.x & 15, grp = threadIdx.x >> 4;
+  const int row = blockIdx.x * 16 + r;
   float acc = OP == ROW_MAX ? -INFINITY : 0.f;
   if (row < h) {
-    int k = wv;
-    for (; k + 12 < splits; k += 16) {
+    int k = grp;
+    for (; k + 48 < splits; k += 64) {
       float v[4];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) v[u] = partial[(size_t)(k + 4 * u) * h + row];
+      for (int u = 0; u < 4; ++u) v[u] = partial[(size_t)(k + 16 * u) * h + row];
 #pragma unroll
       for (int u = 0; u < 4; ++u) acc = row_combine<OP>(acc, v[u]);
     }
-    for (; k < splits; k += 4) acc = row_combine<OP>(acc, partial[(size_t)k * h + row]);
+    for (; k < splits; k += 16) acc = row_combine<OP>(acc, partial[(size_t)k * h + row]);
   }
-  sv[wv][lane] = acc;
+  sv[grp][r] = acc;
   __syncthreads();
-  if (wv == 0 && row < h) {
-    const float s = row_combine<OP>(row_combine<OP>(sv[0][lane], sv[1][lane]), row_combine<OP>(sv[2][lane], sv[3][lane]));
+  if (grp == 0 && row < h) {
+    float s = sv[0][r];
+#pragma unroll
+    for (int g2 = 1; g2 < 16; ++g2) s = row_combine<OP>(s, sv[g2][r]);
     y[row] = row_finish<OP>(y[row], s, alpha, beta);
   }
 }
@@ -450,7 +453,7 @@ static int rows_reduce(const float* M, int ld, int h, int w, const float* x, flo
   else
     hipLaunchKernelGGL((k_rows_stage1<false, OP>), grid, dim3(256), 0, 0, M, ld, h, w, cps, x, y, partial, alpha, beta);
   if (splits > 1)
-    hipLaunchKernelGGL((k_rows_stage2<OP>), dim3((h + 63) / 64), dim3(256), 0, 0, (const float*)partial, splits, h, y,
+    hipLaunchKernelGGL((k_rows_stage2<OP>), dim3((h + 15) / 16), dim3(256), 0, 0, (const float*)partial, splits, h, y,
                        alpha, beta);
   return dn_launch_status();
 }
