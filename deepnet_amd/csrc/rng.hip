@@ -184,6 +184,64 @@ k_rng_split(const unsigned int* mults, const unsigned long long* words, unsigned
   if (d1 == draws) next[idx] = w;
 }
 
+// The same schedule with four neighbouring streams per lane, for calls whose element
+// count is a multiple of 4 on 16-byte aligned arrays: then the four streams 4q..4q+3
+// have equally many draws, their elements of one draw are one aligned 16-byte vector,
+// and a lane runs four independent recurrences against one vector load and one vector
+// store per draw (four draws' loads in flight).
+#define RNG_SPLIT4_BLOCK 256
+template <class Op>
+__global__ void __launch_bounds__(RNG_SPLIT4_BLOCK)
+k_rng_split4(const unsigned int* mults, const unsigned long long* words, unsigned long long* next,
+             const unsigned long long* table, size_t n, int chbits, Op op) {
+  constexpr int blocks_per_part = NUM_RND_STREAMS / (4 * RNG_SPLIT4_BLOCK);
+  const unsigned int part = blockIdx.x / blocks_per_part;
+  const unsigned int idx = 4 * ((blockIdx.x % blocks_per_part) * RNG_SPLIT4_BLOCK + threadIdx.x);   // first of 4 streams
+  if (idx >= n) {  // streams without draws keep their words
+    if (part == 0) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) next[idx + j] = words[idx + j];
+    }
+    return;
+  }
+  const unsigned long long draws = (n - idx + NUM_RND_STREAMS - 1) / NUM_RND_STREAMS;  // of each of the four
+  const unsigned long long d0 = (unsigned long long)part << chbits;
+  if (d0 >= draws) return;
+  const unsigned long long d1 = d0 + (1ull << chbits) < draws ? d0 + (1ull << chbits) : draws;
+  unsigned int mult[4];
+  unsigned long long w[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) { mult[j] = mults[idx + j]; w[j] = words[idx + j]; }
+  for (unsigned int b = 0, pp = part; pp; ++b, pp >>= 1)
+    if (pp & 1u) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) w[j] = mwc_montmul(w[j], table[(size_t)(chbits + b) * NUM_RND_STREAMS + idx + j], mult[j]);
+    }
+  size_t i = (size_t)d0 * NUM_RND_STREAMS + idx;
+  unsigned long long d = d0;
+  auto emit = [&](size_t at, const float4& x) {
+    float4 o;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) w[j] = mwc_step(w[j], mult[j]);
+    o.x = op.value(mwc_uniform(w[0]), x.x); o.y = op.value(mwc_uniform(w[1]), x.y);
+    o.z = op.value(mwc_uniform(w[2]), x.z); o.w = op.value(mwc_uniform(w[3]), x.w);
+    dn_st4<true>(op.dst + at, o);
+  };
+  const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (; d + 4 <= d1; d += 4, i += (size_t)4 * NUM_RND_STREAMS) {
+    float4 x[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) x[k] = op.src ? dn_ld4<true>(op.src + i + (size_t)k * NUM_RND_STREAMS) : zero4;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) emit(i + (size_t)k * NUM_RND_STREAMS, x[k]);
+  }
+  for (; d < d1; ++d, i += NUM_RND_STREAMS) emit(i, op.src ? dn_ld4<true>(op.src + i) : zero4);
+  if (d1 == draws) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) next[idx + j] = w[j];
+  }
+}
+
 // Box-Muller pairs: two draws give elements i and i + 12288 (cudamat_kernels.cu:125-143, 192-211).
 __global__ void __launch_bounds__(RNG_BLOCK)
 k_rng_gauss(const unsigned int* mults, unsigned long long* words, const float* in, float* out, size_t n, float mult_by) {
@@ -209,6 +267,7 @@ k_rng_gauss(const unsigned int* mults, unsigned long long* words, const float* i
 // RNG_SPLIT_PARTS parts per stream (chunk length a power of two, at least 16).
 #define RNG_SPLIT_MIN_DRAWS 32
 #define RNG_SPLIT_PARTS 24
+#define RNG_SPLIT4_PARTS 96    // four streams per lane: more parts for as many wavefronts
 
 template <class Op>
 static int launch_rng(rnd_struct* st, size_t n, Op op) {
@@ -219,8 +278,10 @@ static int launch_rng(rnd_struct* st, size_t n, Op op) {
                        op);
     return dn_launch_status();
   }
+  // (measured: pays for the ops that also read an array; a pure fill is faster one stream per lane)
+  const bool vec4 = op.src && n % 4 == 0 && dn_aligned16(op.dst) && dn_aligned16(op.src);
   int chbits = 4;
-  while (((draws + (1ull << chbits) - 1) >> chbits) > RNG_SPLIT_PARTS) ++chbits;
+  while (((draws + (1ull << chbits) - 1) >> chbits) > (vec4 ? RNG_SPLIT4_PARTS : RNG_SPLIT_PARTS)) ++chbits;
   const size_t parts = (draws + (1ull << chbits) - 1) >> chbits;
   // every jump exponent (chbits + bit of part) must be inside the table
   int top = 0;
@@ -230,10 +291,16 @@ static int launch_rng(rnd_struct* st, size_t n, Op op) {
                        op);
     return dn_launch_status();
   }
-  const unsigned grid = (unsigned)(parts * (NUM_RND_STREAMS / RNG_SPLIT_BLOCK));
   unsigned long long* next = rng_other(st->dev_words);
-  hipLaunchKernelGGL((k_rng_split<Op>), dim3(grid), dim3(RNG_SPLIT_BLOCK), 0, 0, st->dev_mults,
-                     (const unsigned long long*)st->dev_words, next, rng_table(st->dev_words), n, chbits, op);
+  if (vec4) {
+    const unsigned grid = (unsigned)(parts * (NUM_RND_STREAMS / (4 * RNG_SPLIT4_BLOCK)));
+    hipLaunchKernelGGL((k_rng_split4<Op>), dim3(grid), dim3(RNG_SPLIT4_BLOCK), 0, 0, st->dev_mults,
+                       (const unsigned long long*)st->dev_words, next, rng_table(st->dev_words), n, chbits, op);
+  } else {
+    const unsigned grid = (unsigned)(parts * (NUM_RND_STREAMS / RNG_SPLIT_BLOCK));
+    hipLaunchKernelGGL((k_rng_split<Op>), dim3(grid), dim3(RNG_SPLIT_BLOCK), 0, 0, st->dev_mults,
+                       (const unsigned long long*)st->dev_words, next, rng_table(st->dev_words), n, chbits, op);
+  }
   st->dev_words = next;
   return dn_launch_status();
 }

@@ -167,6 +167,28 @@ def test_full_size_4096_uniform_and_bernoulli(cm, mults, rng):
     a.free_device_memory(); b.free_device_memory()
 
 
+@pytest.mark.parametrize("n,offset", [(40 * N + 4 * 777, 0), (33 * N + 8, 0), (64 * N, 0), (40 * N + 4 * 777, 1),
+                                      (35 * N + 6, 0)])
+def test_bernoulli_and_dropout_on_the_four_streams_per_lane_schedule(cm, mults, rng, n, offset):
+    """Calls with a source array, a multiple of 4 elements and 16-byte alignment take the
+    schedule with four streams per lane; element counts that leave the last draw ragged,
+    a view that starts one float off alignment, and a count that is not a multiple of 4
+    must all give the host's stream and state, call after call."""
+    cm.CUDAMatrix.init_random(5)
+    host = mwc.MWC(mults, 5)
+    p = np.asarray(rng.random((n + offset, 1)), dtype=np.float32, order='F')
+    P, T = cm.CUDAMatrix(p), cm.empty((n + offset, 1))
+    src, dst = P.slice(offset, n + offset), T.slice(offset, n + offset)
+    for _ in range(2):
+        src.sample_bernoulli(target=dst)
+        assert np.array_equal(dst.asarray().ravel(), host.bernoulli(p[offset:, 0]))
+        assert np.array_equal(_device_words(cm), host.words)
+    src.dropout(0.3, val=2.5)
+    assert np.array_equal(src.asarray().ravel(), host.dropout(p[offset:, 0], 0.3, 2.5))
+    assert np.array_equal(_device_words(cm), host.words)
+    P.free_device_memory(); T.free_device_memory()
+
+
 def test_sampler_error_codes(cm, rng):
     a = cm.CUDAMatrix(np.zeros((4, 4), dtype=np.float32))
     with pytest.raises(cm.CUDAMatException, match="Incompatible matrix dimensions"):
