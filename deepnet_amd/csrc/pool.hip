@@ -136,53 +136,26 @@ __device__ __forceinline__ float norm_pow(float x, float y) {
 }
 
 // Sum of v (or v*v) over the part of the size x size window with origin (oy, ox) that
-// lies inside the S x S map.  For the usual window sizes (SIZE > 0, compile time) every
-// load is unconditional, from coordinates clamped into the map, and a row of loads is
-// in flight at once; what fell outside is dropped by a select.  SIZE == 0: any size.
-template <int VW, int SIZE, bool SQUARE>
+// lies inside the S x S map (any window size; the usual sizes take k_norm_rows below).
+template <int VW, bool SQUARE>
 __device__ __forceinline__ Vec<VW> window_sum(const float* base, int N, int S, int oy, int ox, int size) {
   Vec<VW> acc;
 #pragma unroll
   for (int i = 0; i < VW; ++i) acc.v[i] = 0.f;
-  if (SIZE > 0) {
+  const int y0 = oy > 0 ? oy : 0, x0 = ox > 0 ? ox : 0;
+  const int y1 = oy + size < S ? oy + size : S, x1 = ox + size < S ? ox + size : S;
+  for (int y = y0; y < y1; ++y)
+    for (int x = x0; x < x1; ++x) {
+      const Vec<VW> v = Vec<VW>::load(base + (size_t)N * (y * S + x));
 #pragma unroll
-    for (int dy = 0; dy < SIZE; ++dy) {
-      const int y = oy + dy;
-      const bool vy = (unsigned)y < (unsigned)S;
-      const int yc = y < 0 ? 0 : (y >= S ? S - 1 : y);
-      Vec<VW> v[SIZE > 0 ? SIZE : 1];
-#pragma unroll
-      for (int dx = 0; dx < SIZE; ++dx) {
-        const int x = ox + dx;
-        const int xc = x < 0 ? 0 : (x >= S ? S - 1 : x);
-        v[dx] = Vec<VW>::load(base + (size_t)N * (yc * S + xc));
-      }
-#pragma unroll
-      for (int dx = 0; dx < SIZE; ++dx) {
-        const bool ok = vy & ((unsigned)(ox + dx) < (unsigned)S);
-#pragma unroll
-        for (int i = 0; i < VW; ++i) {
-          const float t = SQUARE ? v[dx].v[i] * v[dx].v[i] : v[dx].v[i];
-          acc.v[i] += ok ? t : 0.f;
-        }
-      }
+      for (int i = 0; i < VW; ++i) acc.v[i] += SQUARE ? v.v[i] * v.v[i] : v.v[i];
     }
-  } else {
-    const int y0 = oy > 0 ? oy : 0, x0 = ox > 0 ? ox : 0;
-    const int y1 = oy + size < S ? oy + size : S, x1 = ox + size < S ? ox + size : S;
-    for (int y = y0; y < y1; ++y)
-      for (int x = x0; x < x1; ++x) {
-        const Vec<VW> v = Vec<VW>::load(base + (size_t)N * (y * S + x));
-#pragma unroll
-        for (int i = 0; i < VW; ++i) acc.v[i] += SQUARE ? v.v[i] * v.v[i] : v.v[i];
-      }
-  }
   return acc;
 }
 
 // denoms = 1 + addScale * sum over the clipped sizeX x sizeX window (origin -sizeX/2)
 // of meanDiffs^2;  target = imgs * denoms^-powScale   (cudamat_conv_kernels.cu:112-176).
-template <int VW, int SIZE>
+template <int VW>
 __global__ void __launch_bounds__(256)
 k_cnorm(const float* imgs, const float* meanDiffs, float* denoms, float* target, PoolGeom g, int sizeX, float addScale,
         float powScale) {
@@ -191,7 +164,7 @@ k_cnorm(const float* imgs, const float* meanDiffs, float* denoms, float* target,
     int nv, px, py, f;
     decode4(e, g.dNV, g.dS, g.S, &nv, &px, &py, &f);
     const float* base = meanDiffs + (size_t)g.N * ((size_t)f * g.S * g.S) + nv * VW;
-    const Vec<VW> acc = window_sum<VW, SIZE, true>(base, g.N, g.S, py - sizeX / 2, px - sizeX / 2, sizeX);
+    const Vec<VW> acc = window_sum<VW, true>(base, g.N, g.S, py - sizeX / 2, px - sizeX / 2, sizeX);
     const size_t poff = (size_t)g.N * ((size_t)(f * g.S + py) * g.S + px) + nv * VW;
     const Vec<VW> in = Vec<VW>::load(imgs + poff);
     Vec<VW> d, t;
@@ -292,16 +265,22 @@ k_norm_rows(const float* a0, const float* a1, const float* a2, const float* win,
 }
 
 // acts := scale * outGrads * acts / denoms   (cudamat_conv_kernels.cuh:2010-2023)
+template <int VW>
 __global__ void __launch_bounds__(256)
-k_rnorm_undo_prelim(float* acts, const float* denoms, const float* outGrads, size_t n, float scale) {
+k_rnorm_undo_prelim(float* acts, const float* denoms, const float* outGrads, size_t nv, float scale) {
   const size_t stride = (size_t)gridDim.x * 256;
-  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride)
-    acts[i] = (scale * outGrads[i] * acts[i]) / denoms[i];
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < nv; i += stride) {
+    const Vec<VW> a = Vec<VW>::load(acts + i * VW), d = Vec<VW>::load(denoms + i * VW), o = Vec<VW>::load(outGrads + i * VW);
+    Vec<VW> t;
+#pragma unroll
+    for (int k = 0; k < VW; ++k) t.v[k] = (scale * o.v[k] * a.v[k]) / d.v[k];
+    t.store(acts + i * VW);
+  }
 }
 
 // target = inputs * (sum of the prepared acts over the mirrored window) + outGrads * denoms^-powScale
 // (cudamat_conv_kernels.cuh:1920-2004); the window of pixel p is [p + sizeX/2 - sizeX + 1, p + sizeX/2].
-template <int VW, int SIZE>
+template <int VW>
 __global__ void __launch_bounds__(256)
 k_rnorm_undo(const float* outGrads, const float* denoms, const float* inputs, const float* acts, float* target,
              PoolGeom g, int sizeX, float powScale) {
@@ -311,7 +290,7 @@ k_rnorm_undo(const float* outGrads, const float* denoms, const float* inputs, co
     decode4(e, g.dNV, g.dS, g.S, &nv, &px, &py, &f);
     const float* base = acts + (size_t)g.N * ((size_t)f * g.S * g.S) + nv * VW;
     const Vec<VW> acc =
-        window_sum<VW, SIZE, false>(base, g.N, g.S, py + sizeX / 2 - sizeX + 1, px + sizeX / 2 - sizeX + 1, sizeX);
+        window_sum<VW, false>(base, g.N, g.S, py + sizeX / 2 - sizeX + 1, px + sizeX / 2 - sizeX + 1, sizeX);
     const size_t poff = (size_t)g.N * ((size_t)(f * g.S + py) * g.S + px) + nv * VW;
     const Vec<VW> inp = Vec<VW>::load(inputs + poff), og = Vec<VW>::load(outGrads + poff),
                   den = Vec<VW>::load(denoms + poff);
@@ -398,8 +377,8 @@ static void cnorm_impl(cudamat* images, cudamat* meanDiffs, cudamat* denoms, cud
   PoolGeom g;
   make_geom(g, N, numFilters, S, S, 0, 0, 1, v4 ? 4 : 1);
   const unsigned grid = grid_for(total / (v4 ? 4 : 1));
-#define CNORM_GO(VW, SZ)                                                                                       \
-  hipLaunchKernelGGL((k_cnorm<VW, SZ>), dim3(grid), dim3(256), 0, 0, (const float*)images->data_device,         \
+#define CNORM_GO(VW)                                                                                           \
+  hipLaunchKernelGGL((k_cnorm<VW>)    , dim3(grid), dim3(256), 0, 0, (const float*)images->data_device,         \
                      (const float*)meanDiffs->data_device, denoms->data_device, targets->data_device, g, sizeX, \
                      addScale, powScale)
 #define CNORM_ROWS(SZ)                                                                                          \
@@ -412,9 +391,9 @@ static void cnorm_impl(cudamat* images, cudamat* meanDiffs, cudamat* denoms, cud
     if (sizeX == 3) CNORM_ROWS(3);
     else if (sizeX == 5) CNORM_ROWS(5);
     else if (sizeX == 7) CNORM_ROWS(7);
-    else CNORM_GO(4, 0);
+    else CNORM_GO(4);
   } else {
-    CNORM_GO(1, 0);
+    CNORM_GO(1);
   }
 #undef CNORM_GO
 #undef CNORM_ROWS
@@ -435,16 +414,21 @@ static void rnorm_undo_impl(cudamat* outGrads, cudamat* denoms, cudamat* inputs,
     POOL_REQUIRE(m->size[0] == N && m->size[1] == outGrads->size[1], where);
   const long long total = (long long)N * outGrads->size[1];
   POOL_REQUIRE(total < (1ll << 32), where);
-  hipLaunchKernelGGL(k_rnorm_undo_prelim, dim3(grid_for(total)), dim3(256), 0, 0, acts->data_device,
-                     (const float*)denoms->data_device, (const float*)outGrads->data_device, (size_t)total,
-                     -2.f * addScale * powScale);
+  if (total % 4 == 0 && all_aligned16({acts->data_device, denoms->data_device, outGrads->data_device}))
+    hipLaunchKernelGGL((k_rnorm_undo_prelim<4>), dim3(grid_for(total / 4)), dim3(256), 0, 0, acts->data_device,
+                       (const float*)denoms->data_device, (const float*)outGrads->data_device, (size_t)(total / 4),
+                       -2.f * addScale * powScale);
+  else
+    hipLaunchKernelGGL((k_rnorm_undo_prelim<1>), dim3(grid_for(total)), dim3(256), 0, 0, acts->data_device,
+                       (const float*)denoms->data_device, (const float*)outGrads->data_device, (size_t)total,
+                       -2.f * addScale * powScale);
   const bool v4 = N % 4 == 0 && all_aligned16({outGrads->data_device, denoms->data_device, inputs->data_device,
                                                acts->data_device, targets->data_device});
   PoolGeom g;
   make_geom(g, N, numFilters, S, S, 0, 0, 1, v4 ? 4 : 1);
   const unsigned grid = grid_for(total / (v4 ? 4 : 1));
-#define RUNDO_GO(VW, SZ)                                                                                      \
-  hipLaunchKernelGGL((k_rnorm_undo<VW, SZ>), dim3(grid), dim3(256), 0, 0, (const float*)outGrads->data_device, \
+#define RUNDO_GO(VW)                                                                                          \
+  hipLaunchKernelGGL((k_rnorm_undo<VW>)    , dim3(grid), dim3(256), 0, 0, (const float*)outGrads->data_device, \
                      (const float*)denoms->data_device, (const float*)inputs->data_device,                     \
                      (const float*)acts->data_device, targets->data_device, g, sizeX, powScale)
 #define RUNDO_ROWS(SZ)                                                                                         \
@@ -457,9 +441,9 @@ static void rnorm_undo_impl(cudamat* outGrads, cudamat* denoms, cudamat* inputs,
     if (sizeX == 3) RUNDO_ROWS(3);
     else if (sizeX == 5) RUNDO_ROWS(5);
     else if (sizeX == 7) RUNDO_ROWS(7);
-    else RUNDO_GO(4, 0);
+    else RUNDO_GO(4);
   } else {
-    RUNDO_GO(1, 0);
+    RUNDO_GO(1);
   }
 #undef RUNDO_GO
 #undef RUNDO_ROWS
