@@ -46,6 +46,7 @@ struct ConvArgs {
   int splits, slabs_per_split;
   int local;          // 1: one filter bank per module (locally connected layers); direct kernels only
   float scale_t, scale_o;
+  unsigned a_bytes, b_bytes;  // sizes of the two gathered arrays (uniform-row kernels: buffer ranges)
   FastDiv dN, dMx, dk, dkk2;
 };
 
@@ -156,7 +157,13 @@ __device__ __forceinline__ void down_axis(int ph, int s, int pad0, int H, int k,
   *T = ph < k ? (k - ph + s - 1) / s : 0;
 }
 
-template <int MODE, int WAVES_M, int WM, int WN>
+// UNI (Up / Down, 128-row tiles, batch a multiple of 128): all rows of a tile belong to
+// one module (Up) or one pixel (Down), so whether a tap falls into the padding is a
+// scalar question.  The gathers then are buffer loads -- lane offset fixed for the whole
+// kernel, slab offset in an SGPR, an out-of-range offset for a tap in the padding, which
+// the hardware answers with zeros -- and cost no vector instructions, which matters
+// because fp32 MFMA and the vector ALU share lanes.  Both operands run two slabs ahead.
+template <int MODE, int WAVES_M, int WM, int WN, bool UNI = false>
 __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
   constexpr int WAVES_N = 4 / WAVES_M;
   constexpr int BM = 32 * WM * WAVES_M, BN = 32 * WN * WAVES_N;
@@ -292,6 +299,37 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
     }
   }
 
+  // ---- uniform-row variant: buffer resources, fixed lane offsets, the tile's module / pixel
+  __amdgpu_buffer_rsrc_t u_ra = __builtin_amdgcn_make_buffer_rsrc((void*)(MODE == CONV_UP ? p.img : p.hid), 0,
+                                                                    (int)p.a_bytes, 0x00020000);
+  __amdgpu_buffer_rsrc_t u_rb = __builtin_amdgcn_make_buffer_rsrc((void*)p.flt, 0, (int)p.b_bytes, 0x00020000);
+  // The two halves of a wavefront (lanes 0-31, 32-63) gather the tile's 128 rows at two
+  // consecutive kk.
+  unsigned u_avo[NA], u_bvo[NB];
+  int u_bks[NB];
+  int u_y = 0, u_x = 0;
+  unsigned u_n0 = 0;
+  if constexpr (UNI) {
+    static_assert(MODE != CONV_OUTP && BM == 128, "uniform rows: Up / Down with 128-row tiles");
+    const int pos = (int)fd_div((uint32_t)row0, p.dN);       // scalar: module (Up) or pixel of the phase (Down)
+    u_n0 = 4u * (unsigned)(row0 - pos * N);
+    if (MODE == CONV_UP) {
+      const int my = (int)fd_div((uint32_t)pos, p.dMx), mx = pos - my * Mx;
+      u_y = my * s + p.pad0; u_x = mx * s + p.pad0;
+    } else {
+      const int qyi = ph.QX > 0 ? pos / ph.QX : 0, qxi = pos - qyi * ph.QX;
+      u_y = ph.qy_first + qyi; u_x = ph.qx_first + qxi;
+    }
+#pragma unroll
+    for (int u = 0; u < NA; ++u) u_avo[u] = 4u * (unsigned)(a_r[u] + (MODE == CONV_DOWN && lk ? M * N : 0));
+#pragma unroll
+    for (int u = 0; u < NB; ++u) {
+      u_bks[u] = __builtin_amdgcn_readfirstlane(b_k[u]);
+      if (MODE == CONV_UP) u_bvo[u] = 4u * (unsigned)(g * Fg + col0 + b_c[u] + F * (b_k[u] - u_bks[u]));
+      else u_bvo[u] = 4u * (unsigned)(g * Fg + b_k[u] + F * (col0 + b_c[u]) * p.kk2);
+    }
+  }
+
   // ---- slab state (uniform across the workgroup)
   // Down: slab -> (t, u, f0); Outp: slab -> (my, mx, n0).
   int st_a = 0, st_b = 0, st_c = 0;
@@ -321,6 +359,51 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
   auto fetch = [&](auto set_tag, int slab) {
     constexpr int SET = decltype(set_tag)::value;
     const int kk0 = slab * CV_BK;
+    if constexpr (UNI) {
+#pragma unroll
+      for (int u = 0; u < NA; ++u) {
+        unsigned voff = u_avo[u], so;
+        if (MODE == CONV_UP) {
+          // per half (kk row): byte offset of its 128 images, or "in the padding"; all scalar
+          // and free of branches (a branch here would split up the slab's loads)
+          unsigned off[2];
+          bool ok[2];
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            const int kk = kk0 + a_ks[u] + h;
+            const int c = (int)fd_div((uint32_t)kk, p.dkk2);
+            const int pp = kk - c * p.kk2;
+            const int ky = (int)fd_div((uint32_t)pp, p.dk), kx = pp - ky * k;
+            const int y = u_y + ky, x = u_x + kx;
+            ok[h] = (kk < Kup) & ((unsigned)y < (unsigned)H) & ((unsigned)x < (unsigned)H);
+            off[h] = 4u * (unsigned)N * (unsigned)((g * Cg + c) * HH + y * H + x) + u_n0;
+          }
+          const unsigned lo = ok[0] ? off[0] : 0xffffffffu, hi = ok[1] ? off[1] : 0xffffffffu;
+          so = lo < hi ? lo : hi;                              // the smaller valid offset ...
+          if (!(ok[0] | ok[1])) so = 0u;
+          const unsigned dlo = ok[0] ? off[0] - so : p.a_bytes, dhi = ok[1] ? off[1] - so : p.a_bytes;   // ... plus a non-negative rest
+          voff += lk ? dhi : dlo;
+        } else {
+          // both halves read the same module, one filter apart (a constant in the lane offset)
+          const int my = u_y - st_a, mx = u_x - st_b;
+          const bool ok = ((unsigned)my < (unsigned)Mx) & ((unsigned)mx < (unsigned)Mx);
+          so = ok ? 4u * (unsigned)N * (unsigned)((g * Fg + st_c + a_ks[u]) * M + my * Mx + mx) + u_n0 : p.a_bytes;
+        }
+        ra[SET][u] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(u_ra, (int)voff, (int)so, 0));
+      }
+#pragma unroll
+      for (int u = 0; u < NB; ++u) {
+        unsigned so;
+        if (MODE == CONV_UP) so = 4u * (unsigned)F * (unsigned)(kk0 + u_bks[u]);
+        else so = 4u * (unsigned)(F * ((ph.py + s * st_a) * k + ph.px + s * st_b) + st_c);
+        rb[SET][u] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(u_rb, (int)u_bvo[u], (int)so, 0));
+      }
+      if (MODE == CONV_DOWN) {
+        st_c += CV_BK;
+        if (st_c == Fg) { st_c = 0; if (++st_b == ph.TX) { st_b = 0; ++st_a; } }
+      }
+      return;
+    }
 #pragma unroll
     for (int u = 0; u < NA; ++u) {
       bool ok = a_ok[u];
@@ -393,7 +476,7 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
 #pragma unroll
     for (int u = 0; u < NA; ++u) {
       if (tid + u * 256 >= TA) continue;
-      if (!ra_ok[SET][u]) ra[SET][u] = zero4;
+      if (!UNI && !ra_ok[SET][u]) ra[SET][u] = zero4;
       if (MODE == CONV_OUTP) {
         As[buf][a_k[u]][a_r[u]] = ra[SET][u].x; As[buf][a_k[u] + 1][a_r[u]] = ra[SET][u].y;
         As[buf][a_k[u] + 2][a_r[u]] = ra[SET][u].z; As[buf][a_k[u] + 3][a_r[u]] = ra[SET][u].w;
@@ -404,7 +487,7 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
 #pragma unroll
     for (int u = 0; u < NB; ++u) {
       if (tid + u * 256 >= TB) continue;
-      if (!rb_ok[SET][u]) rb[SET][u] = zero4;
+      if (!UNI && !rb_ok[SET][u]) rb[SET][u] = zero4;
       if (MODE == CONV_UP) {
         *reinterpret_cast<f32x4*>(&Bs[buf][b_k[u]][b_c[u]]) = rb[SET][u];
       } else {
@@ -450,7 +533,7 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
   // statically.  fetch() is always called with consecutive slabs.
   // (Measured: the deeper prefetch pays for Outp, whose K runs over modules and images;
   // for Up and Down its extra registers cost more than it hides.)
-  constexpr bool TWO_AHEAD = MODE == CONV_OUTP;
+  constexpr bool TWO_AHEAD = MODE == CONV_OUTP || UNI;
   int buf = 0, slab = slab_beg;
   if (TWO_AHEAD && slab_end - slab_beg >= 2) {
     fetch(Set0(), slab);
@@ -638,13 +721,33 @@ static void fill_common(ConvArgs& a, int N, int C, int G, int H, int F, int k, i
   a.N = N; a.C = C; a.G = G; a.Cg = C / G; a.H = H; a.F = F; a.Fg = F / G; a.k = k; a.Mx = Mx; a.s = s; a.pad0 = pad0;
   a.M = Mx * Mx; a.HH = H * H; a.kk2 = k * k;
   a.m_begin = 0; a.m_count = a.M; a.splits = 1; a.slabs_per_split = 0; a.local = 0;
-  a.scale_t = 0.f; a.scale_o = 1.f; a.partial = nullptr;
+  a.scale_t = 0.f; a.scale_o = 1.f; a.partial = nullptr; a.a_bytes = 0; a.b_bytes = 0;
   a.dN = make_fastdiv((uint32_t)N); a.dMx = make_fastdiv((uint32_t)Mx);
   a.dk = make_fastdiv((uint32_t)k); a.dkk2 = make_fastdiv((uint32_t)(k * k));
 }
 
+// Byte sizes of the two gathered arrays for the buffer-load kernels; 0 when one of them
+// is too large for 32-bit buffer offsets (twice the size must not wrap).
+static void set_buffer_ranges(ConvArgs& a, long long a_elems, long long b_elems) {
+  const bool fits = a_elems * 4 < (1ll << 31) && b_elems * 4 < (1ll << 31);
+  a.a_bytes = fits ? (unsigned)(a_elems * 4) : 0u;
+  a.b_bytes = fits ? (unsigned)(b_elems * 4) : 0u;
+}
+
 template <int MODE>
 static void launch_rowmajor(const ConvArgs& a, long long rows, int cols, int gz) {
+  // Batches that are multiples of 128: tiles of 128 rows never straddle a module / pixel.
+  // Measured on the benchmark layers: the buffer-load kernels win for long reductions
+  // with up to 64 or more than 96 columns; 65-96 columns and short reductions are
+  // faster on the 256-row tiles below.
+  const int nslabs = MODE == CONV_UP ? (a.Cg * a.kk2 + CV_BK - 1) / CV_BK : a.kk2 * (a.Fg / CV_BK) / (a.s * a.s);
+  if (a.N % 128 == 0 && a.a_bytes != 0 && a.b_bytes != 0 && nslabs >= 16 && (cols <= 64 || cols > 96)) {
+    const unsigned gx = (unsigned)(rows / 128);
+    if (cols <= 32) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 1, true>), dim3(gx, (cols + 31) / 32, gz), dim3(256), 0, 0, a);
+    else if (cols <= 64) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 2, true>), dim3(gx, (cols + 63) / 64, gz), dim3(256), 0, 0, a);
+    else hipLaunchKernelGGL((k_conv_mfma<MODE, 2, 2, 2, true>), dim3(gx, (cols + 127) / 128, gz), dim3(256), 0, 0, a);
+    return;
+  }
   // Up / Down: rows are plentiful, columns few: 4 wavefronts down the rows, WN blocks across.
   // With enough rows to keep every CU busy twice over, each wavefront takes two row
   // blocks (256-row tiles): twice the MFMAs per LDS read and per barrier.
@@ -687,6 +790,7 @@ static void conv_up_impl(cudamat* images, cudamat* filters, cudamat* targets, in
   fill_common(a, N, numImgColors, numGroups, H, F, k, numModulesX, moduleStride, paddingStart);
   a.img = images->data_device; a.flt = filters->data_device; a.hid = nullptr; a.out = targets->data_device;
   a.local = local ? 1 : 0;
+  set_buffer_ranges(a, (long long)N * numImgColors * H * H, (long long)F * filters->size[1]);
   if (!local && fast_ok(a)) {
     launch_rowmajor<CONV_UP>(a, (long long)M * N, a.Fg, numGroups);
   } else {
@@ -722,6 +826,7 @@ static void conv_down_impl(cudamat* hidActs, cudamat* filters, cudamat* targets,
   a.img = nullptr; a.flt = filters->data_device; a.hid = hidActs->data_device; a.out = targets->data_device;
   a.img = a.hid;  // alignment test only
   a.local = local ? 1 : 0;
+  set_buffer_ranges(a, (long long)N * M * F, (long long)F * filters->size[1]);
   if (!local && fast_ok(a) && dn_aligned16(a.out) && a.Cg <= 16) {
     // few colours: patch-matrix form
     const long long prow = (long long)a.M * N;

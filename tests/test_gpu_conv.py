@@ -24,6 +24,9 @@ CASES = [  # N, C, H, F, k, stride, padding, groups
     (16, 32, 6, 64, 3, 2, 1, 2),
     (128, 3, 32, 64, 5, 1, 2, 1),    # the CIFAR layer of the benchmark
     (16, 48, 9, 160, 3, 1, 1, 1),    # more than 128 filters: two column tiles
+    (128, 48, 6, 32, 3, 1, 1, 2),    # batch 128: the uniform-row (buffer load) kernels, 24 colours per group
+    (128, 40, 7, 48, 3, 2, 1, 1),    # the same with stride 2 (four phases in convDown), 40 colours
+    (256, 20, 5, 144, 4, 1, 2, 1),   # batch 256, 144 filters (two column tiles), padding 2 > k/2
 ]
 
 
