@@ -325,18 +325,30 @@ k_gemm_small(const float* __restrict__ A, int lda, const float* __restrict__ B, 
   f32x16 acc;
 #pragma unroll
   for (int v = 0; v < 16; ++v) acc[v] = 0.f;
-  float a0[16], b0[16], a1[16], b1[16];
+  // Three chunks per wavefront are requested before the first MFMA (for the RBM / MLP
+  // products that is all, or nearly all, of a wavefront's share of K): these kernels live
+  // on memory latency, not on throughput.
+  constexpr int DEPTH = 3;
   constexpr int STEP = 32 * NW;
+  float a[DEPTH][16], b[DEPTH][16];
   int k0 = wv * 32;
-  small_load<A_KC>(A, lda, mc, k0, lk, K, a_vec, a0);
-  small_load<B_KC>(B, ldb, nc, k0, lk, K, b_vec, b0);
-  for (; k0 < K; k0 += STEP) {
-    small_load<A_KC>(A, lda, mc, k0 + STEP, lk, K, a_vec, a1);   // next chunk in flight behind the MFMAs
-    small_load<B_KC>(B, ldb, nc, k0 + STEP, lk, K, b_vec, b1);
 #pragma unroll
-    for (int q = 0; q < 16; ++q) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(b0[q], a0[q], acc, 0, 0, 0);
+  for (int d = 0; d < DEPTH; ++d) {
+    small_load<A_KC>(A, lda, mc, k0 + d * STEP, lk, K, a_vec, a[d]);
+    small_load<B_KC>(B, ldb, nc, k0 + d * STEP, lk, K, b_vec, b[d]);
+  }
+  for (; k0 < K; k0 += DEPTH * STEP) {
 #pragma unroll
-    for (int q = 0; q < 16; ++q) { a0[q] = a1[q]; b0[q] = b1[q]; }
+    for (int d = 0; d < DEPTH; ++d) {
+      if (k0 + d * STEP < K) {                               // wave-uniform
+#pragma unroll
+        for (int q = 0; q < 16; ++q) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(b[d][q], a[d][q], acc, 0, 0, 0);
+        if (k0 + (d + DEPTH) * STEP < K) {                   // refill the set with the chunk DEPTH further on
+          small_load<A_KC>(A, lda, mc, k0 + (d + DEPTH) * STEP, lk, K, a_vec, a[d]);
+          small_load<B_KC>(B, ldb, nc, k0 + (d + DEPTH) * STEP, lk, K, b_vec, b[d]);
+        }
+      }
+    }
   }
   // Halve the number of live accumulators until four are left ...
 #pragma unroll
