@@ -32,7 +32,9 @@
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-enum { CONV_UP = 0, CONV_DOWN = 1, CONV_OUTP = 2 };
+// CONV_DOWNM: convDown for strided layers with few colours, all stride*stride pixel
+// phases merged into the columns of one product (uniform-row kernels only).
+enum { CONV_UP = 0, CONV_DOWN = 1, CONV_OUTP = 2, CONV_DOWNM = 3 };
 
 struct ConvArgs {
   const float* img;   // images: input of Up/Outp
@@ -47,7 +49,8 @@ struct ConvArgs {
   int local;          // 1: one filter bank per module (locally connected layers); direct kernels only
   float scale_t, scale_o;
   unsigned a_bytes, b_bytes;  // sizes of the two gathered arrays (uniform-row kernels: buffer ranges)
-  FastDiv dN, dMx, dk, dkk2;
+  int yq;             // CONV_DOWNM: stride x stride pixel blocks per image side
+  FastDiv dN, dMx, dk, dkk2, dS, dSS;
 };
 
 // ------------------------------------------------------------------ direct kernels
@@ -188,6 +191,17 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
     rows = M * N; cols = Fg;
     nslabs = (Cg * p.kk2 + CV_BK - 1) / CV_BK;
     slab_beg = 0; slab_end = nslabs;
+  } else if (MODE == CONV_DOWNM) {
+    // Rows: (Y, X, image) over blocks of s x s pixels in padded coordinates, pixel
+    // y = Y*s + py + pad0.  Columns: (colour, py, px).  K: (t, u, filter) with the tap
+    // ky = t*s + py of module Y - t (zero weight where ky >= k).
+    g = blockIdx.z;
+    const int T = (k + s - 1) / s;
+    ph.py = ph.px = 0; ph.y_first = ph.x_first = p.pad0;
+    ph.QY = ph.QX = p.yq; ph.qy_first = ph.qx_first = 0; ph.TY = ph.TX = T;
+    rows = p.yq * p.yq * N; cols = Cg * s * s;
+    nslabs = T * T * (Fg / CV_BK);
+    slab_beg = 0; slab_end = nslabs;
   } else if (MODE == CONV_DOWN) {
     const int nph = s * s;
     g = blockIdx.z / nph;
@@ -220,6 +234,7 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
   // vector instructions; the index decomposition runs on the scalar unit.
   const int wvu = __builtin_amdgcn_readfirstlane(wv);
   constexpr int A_ROWLANES = BM / 4;                               // lanes per kk row of the A tile
+  constexpr bool DOWNISH = MODE == CONV_DOWN || MODE == CONV_DOWNM;
   constexpr bool A_TWO = MODE != CONV_OUTP && A_ROWLANES == 32;    // a wavefront spans two kk rows
   static_assert(MODE == CONV_OUTP || A_ROWLANES == 32 || A_ROWLANES == 64, "Up/Down tiles are 128 or 256 rows");
   const int padw = p.pad0 < 0 ? -p.pad0 : 0;
@@ -306,7 +321,7 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
   // The two halves of a wavefront (lanes 0-31, 32-63) gather the tile's 128 rows at two
   // consecutive kk.
   unsigned u_avo[NA], u_bvo[NB];
-  int u_bks[NB];
+  int u_bks[NB], m_py[NB], m_px[NB];
   int u_y = 0, u_x = 0;
   unsigned u_n0 = 0;
   if constexpr (UNI) {
@@ -321,19 +336,28 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
       u_y = ph.qy_first + qyi; u_x = ph.qx_first + qxi;
     }
 #pragma unroll
-    for (int u = 0; u < NA; ++u) u_avo[u] = 4u * (unsigned)(a_r[u] + (MODE == CONV_DOWN && lk ? M * N : 0));
+    for (int u = 0; u < NA; ++u) u_avo[u] = 4u * (unsigned)(a_r[u] + (DOWNISH && lk ? M * N : 0));
 #pragma unroll
     for (int u = 0; u < NB; ++u) {
       u_bks[u] = __builtin_amdgcn_readfirstlane(b_k[u]);
-      if (MODE == CONV_UP) u_bvo[u] = 4u * (unsigned)(g * Fg + col0 + b_c[u] + F * (b_k[u] - u_bks[u]));
-      else u_bvo[u] = 4u * (unsigned)(g * Fg + b_k[u] + F * (col0 + b_c[u]) * p.kk2);
+      if (MODE == CONV_UP) {
+        u_bvo[u] = 4u * (unsigned)(g * Fg + col0 + b_c[u] + F * (b_k[u] - u_bks[u]));
+      } else if (MODE == CONV_DOWNM) {
+        const int j = col0 + b_c[u];                           // column -> (colour, py, px)
+        const int c = (int)fd_div((uint32_t)j, p.dSS), q = j - c * s * s;
+        m_py[u] = (int)fd_div((uint32_t)q, p.dS); m_px[u] = q - m_py[u] * s;
+        if (j >= cols) m_py[u] = k;                            // never a valid tap
+        u_bvo[u] = 4u * (unsigned)(g * Fg + b_k[u] + F * (c * p.kk2 + m_py[u] * k + m_px[u]));
+      } else {
+        u_bvo[u] = 4u * (unsigned)(g * Fg + b_k[u] + F * (col0 + b_c[u]) * p.kk2);
+      }
     }
   }
 
   // ---- slab state (uniform across the workgroup)
   // Down: slab -> (t, u, f0); Outp: slab -> (my, mx, n0).
   int st_a = 0, st_b = 0, st_c = 0;
-  if (MODE == CONV_DOWN) {
+  if (DOWNISH) {
     const int per_tap = Fg / CV_BK;
     const int tap = slab_beg / per_tap;
     st_c = (slab_beg - tap * per_tap) * CV_BK;            // f0
@@ -394,11 +418,16 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
 #pragma unroll
       for (int u = 0; u < NB; ++u) {
         unsigned so;
+        unsigned voff = u_bvo[u];
         if (MODE == CONV_UP) so = 4u * (unsigned)F * (unsigned)(kk0 + u_bks[u]);
         else so = 4u * (unsigned)(F * ((ph.py + s * st_a) * k + ph.px + s * st_b) + st_c);
-        rb[SET][u] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(u_rb, (int)u_bvo[u], (int)so, 0));
+        if (MODE == CONV_DOWNM) {                              // this column's tap of module (Y - t, X - u), if it has one
+          const bool ok = (m_py[u] + s * st_a < k) & (m_px[u] + s * st_b < k);
+          voff = ok ? voff : p.b_bytes;
+        }
+        rb[SET][u] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(u_rb, (int)voff, (int)so, 0));
       }
-      if (MODE == CONV_DOWN) {
+      if (DOWNISH) {
         st_c += CV_BK;
         if (st_c == Fg) { st_c = 0; if (++st_b == ph.TX) { st_b = 0; ++st_a; } }
       }
@@ -582,6 +611,25 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
     if (MODE == CONV_UP) {
       rbase = (long long)g * Fg * M * N + r;            // + c * M*N
       cstride = (long long)M * N;
+    } else if (MODE == CONV_DOWNM) {
+      const int pos = (int)fd_div((uint32_t)r, p.dN);
+      const int n = r - pos * N;
+      const int Y = pos / p.yq, X = pos - Y * p.yq;
+#pragma unroll
+      for (int j = 0; j < WN; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int cc = col0 + (wn * WN + j) * 32 + 8 * (v >> 2) + 4 * lk + (v & 3);
+          if (cc >= cols) continue;
+          const int c = (int)fd_div((uint32_t)cc, p.dSS), q = cc - c * s * s;
+          const int py = (int)fd_div((uint32_t)q, p.dS), px = q - py * s;
+          const int y = Y * s + py + p.pad0, x = X * s + px + p.pad0;
+          if ((unsigned)y < (unsigned)H && (unsigned)x < (unsigned)H) {
+            float* t = p.out + (long long)N * ((long long)(g * Cg + c) * HH + y * H + x) + n;
+            *t = (p.scale_t == 0.f ? 0.f : p.scale_t * *t) + p.scale_o * acc[j][i][v];
+          }
+        }
+      continue;
     } else if (MODE == CONV_DOWN) {
       const int pos = (int)fd_div((uint32_t)r, p.dN);
       const int n = r - pos * N;
@@ -724,6 +772,7 @@ static void fill_common(ConvArgs& a, int N, int C, int G, int H, int F, int k, i
   a.scale_t = 0.f; a.scale_o = 1.f; a.partial = nullptr; a.a_bytes = 0; a.b_bytes = 0;
   a.dN = make_fastdiv((uint32_t)N); a.dMx = make_fastdiv((uint32_t)Mx);
   a.dk = make_fastdiv((uint32_t)k); a.dkk2 = make_fastdiv((uint32_t)(k * k));
+  a.dS = make_fastdiv((uint32_t)s); a.dSS = make_fastdiv((uint32_t)(s * s)); a.yq = 0;
 }
 
 // Byte sizes of the two gathered arrays for the buffer-load kernels; 0 when one of them
@@ -827,7 +876,17 @@ static void conv_down_impl(cudamat* hidActs, cudamat* filters, cudamat* targets,
   a.img = a.hid;  // alignment test only
   a.local = local ? 1 : 0;
   set_buffer_ranges(a, (long long)N * M * F, (long long)F * filters->size[1]);
-  if (!local && fast_ok(a) && dn_aligned16(a.out) && a.Cg <= 16) {
+  if (!local && fast_ok(a) && dn_aligned16(a.out) && a.Cg <= 16 && moduleStride > 1 && N % 128 == 0 && a.a_bytes != 0) {
+    // few colours, strided: the stride^2 pixel phases become columns of one implicit GEMM
+    const int padw = paddingStart < 0 ? -paddingStart : 0;
+    a.yq = (imgSize - 1 + padw) / moduleStride + 1;
+    const int cols = a.Cg * moduleStride * moduleStride;
+    const unsigned gx = (unsigned)((long long)a.yq * a.yq * N / 128);
+    if (cols <= 32) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 1, true>), dim3(gx, 1, numGroups), dim3(256), 0, 0, a);
+    else if (cols <= 64) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 2, true>), dim3(gx, 1, numGroups), dim3(256), 0, 0, a);
+    else if (cols <= 96) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 3, true>), dim3(gx, 1, numGroups), dim3(256), 0, 0, a);
+    else hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 2, 2, 2, true>), dim3(gx, (cols + 127) / 128, numGroups), dim3(256), 0, 0, a);
+  } else if (!local && fast_ok(a) && dn_aligned16(a.out) && a.Cg <= 16) {
     // few colours: patch-matrix form
     const long long prow = (long long)a.M * N;
     const int pcols = a.Cg * a.kk2;

@@ -27,6 +27,11 @@ CASES = [  # N, C, H, F, k, stride, padding, groups
     (128, 48, 6, 32, 3, 1, 1, 2),    # batch 128: the uniform-row (buffer load) kernels, 24 colours per group
     (128, 40, 7, 48, 3, 2, 1, 1),    # the same with stride 2 (four phases in convDown), 40 colours
     (256, 20, 5, 144, 4, 1, 2, 1),   # batch 256, 144 filters (two column tiles), padding 2 > k/2
+    (128, 3, 12, 16, 5, 4, 0, 1),    # few colours, strided, batch 128: convDown with the phases merged into columns
+    (128, 3, 13, 32, 4, 3, 2, 1),    # the same: stride 3 does not divide k = 4, padding 2
+    (128, 4, 9, 32, 3, 2, 1, 2),     # the same: 2 groups of 2 colours
+    (256, 8, 8, 16, 5, 2, 2, 1),     # the same: 8 colours x 4 phases = 32 columns, batch 256
+    (128, 16, 7, 16, 3, 3, 0, 1),    # the same: 16 colours x 9 phases = 144 columns (two column tiles), stride == k
 ]
 
 
