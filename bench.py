@@ -133,6 +133,19 @@ class RBM(object):
         self.v2 = cm.empty((nv, B))
         self.flops = 5 * 2 * nv * nh * B
 
+    def step_fused(self):
+        """The same step through this backend's dot_bias_act extension (10 launches instead
+        of 16; results bit-identical to step())."""
+        cm, eps = self.cm, self.lr / self.B
+        W, v, h, hs, v2, h2 = self.W, self.v, self.h, self.hs, self.v2, self.h2
+        cm.dot_bias_act(W.T, v, self.bh, target=h, act='sigmoid')
+        h.sample_bernoulli(target=hs)
+        cm.dot_bias_act(W, hs, self.bv, target=v2, act='sigmoid')
+        cm.dot_bias_act(W.T, v2, self.bh, target=h2, act='sigmoid')
+        W.add_dot(v, h.T, mult=eps); W.add_dot(v2, h2.T, mult=-eps)
+        self.bv.add_sums(v, axis=1, mult=eps); self.bv.add_sums(v2, axis=1, mult=-eps)
+        self.bh.add_sums(h, axis=1, mult=eps); self.bh.add_sums(h2, axis=1, mult=-eps)
+
     def step(self):
         cm, eps = self.cm, self.lr / self.B
         W, v, h, hs, v2, h2 = self.W, self.v, self.h, self.hs, self.v2, self.h2
@@ -389,6 +402,10 @@ def main():
         secondary['rbm_cd1'] = {'steps_per_sec': round(1.0 / t, 1), 'us_per_step': round(t * 1e6, 1),
                                 'gemm_tflops': round(rbm.flops / t / 1e12, 3),
                                 'config': '784 visible x 500 hidden, batch 100, fp32'}
+        t = time_loop(cm, rbm.step_fused, 200, 20)
+        secondary['rbm_cd1_fused_extension'] = {
+            'steps_per_sec': round(1.0 / t, 1), 'us_per_step': round(t * 1e6, 1),
+            'note': 'same step with dot_bias_act (an extension of this backend, not in the reference API): 10 launches instead of 16'}
         cm.CUDAMatrix.init_random(3)
         mlp = MLP(cm)
         t = time_loop(cm, mlp.step, 100, 10)

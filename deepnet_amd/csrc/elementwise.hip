@@ -454,3 +454,43 @@ int add_diagonal(cudamat* mat, cudamat* vec, cudamat* target) {
 }
 
 }  // extern "C"
+
+int dn_gemm_fused(bool a_trans, bool b_trans, int M, int N, int K, const float* A, int lda, const float* B, int ldb,
+                  float* C, int ldc, const float* bias, int act, bool* fused);
+
+extern "C" {
+
+// Extension (no counterpart in cudamat.cu): target = act(op(mat1) * op(mat2) + bias), the
+// sequence dot -> add_col_vec -> apply_sigmoid / lower_bound(0) / apply_tanh that every
+// layer of deepnet issues (deepnet/dbm.py:95-105, deepnet/neuralnet.py:138-160), in one
+// launch where the product runs as a single kernel, bit-identical to the three calls.
+// bias: rows(target) x 1 or null.  act: 0 none, 1 sigmoid, 2 max(x, 0), 3 tanh.
+int dot_bias_act(cudamat* mat1, cudamat* mat2, cudamat* bias, cudamat* target, int act) {
+  if (!mat1->on_device || !mat2->on_device || !target->on_device || (bias && !bias->on_device)) return ERROR_NOT_ON_DEVICE;
+  if (target->is_trans || (bias && bias->is_trans)) return ERROR_TRANSPOSED;
+  if (act < 0 || act > 3) return ERROR_UNSUPPORTED;
+  if (get_leading_dimension(mat1) != target->size[0] || get_nonleading_dimension(mat2) != target->size[1] ||
+      get_nonleading_dimension(mat1) != get_leading_dimension(mat2))
+    return ERROR_INCOMPATIBLE_DIMENSIONS;
+  if (bias && (bias->size[0] != target->size[0] || bias->size[1] != 1)) return ERROR_INCOMPATIBLE_DIMENSIONS;
+  const int m = target->size[0], n = target->size[1], k = get_leading_dimension(mat2);
+  if (m <= 0 || n <= 0) return 0;
+  bool fused = false;
+  int err;
+  if (n == 1 || k <= 0) {
+    err = dot(mat1, mat2, target, 0.f, 1.f);                 // vector-shaped: the streaming kernels
+  } else {
+    err = dn_gemm_fused(mat1->is_trans != 0, mat2->is_trans != 0, m, n, k, mat1->data_device, mat1->size[0],
+                        mat2->data_device, mat2->size[0], target->data_device, m, bias ? bias->data_device : nullptr,
+                        act, &fused);
+  }
+  if (err || fused) return err;
+  if (bias && (err = add_col_vec(target, bias, target))) return err;
+  if (act == 1) return apply_sigmoid(target, target);
+  if (act == 2) return lower_bound_scalar(target, 0.f, target);
+  if (act == 3) return apply_tanh(target, target);
+  return 0;
+}
+
+
+}  // extern "C"

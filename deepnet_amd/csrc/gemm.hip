@@ -9,12 +9,29 @@
 // products (a single row or column on either side, which is how sum(axis) and
 // add_sums arrive) go to the streaming matrix-vector kernels instead.
 #include "common.h"
+#include "wide_math.h"
 
 int dn_gemv_cols(const float* M, int ld, int h, int w, const float* x, float* y, float alpha, float beta);
 int dn_gemv_rows(const float* M, int ld, int h, int w, const float* x, float* y, float alpha, float beta);
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// What dot_bias_act() appends to the product, element by element and in the order of
+// the separate calls it replaces (add_col_vec, then the activation), so that the fused
+// result is bit-identical to theirs: bias is a column vector over the rows of C or null.
+enum { GEMM_ACT_NONE = 0, GEMM_ACT_SIGMOID = 1, GEMM_ACT_RELU = 2, GEMM_ACT_TANH = 3 };
+struct GemmEpilogue {
+  const float* bias;
+  int act;
+};
+__device__ __forceinline__ float gemm_finish(float v, int m, const GemmEpilogue& e) {
+  if (e.bias) v = v + e.bias[m];
+  if (e.act == GEMM_ACT_SIGMOID) v = dn_sigmoid(v);
+  else if (e.act == GEMM_ACT_RELU) v = v < 0.f ? 0.f : v;
+  else if (e.act == GEMM_ACT_TANH) v = dn_tanh(v);
+  return v;
+}
 
 #define GEMM_BK 16
 #define GEMM_PAD 4
@@ -46,7 +63,7 @@ __device__ __forceinline__ f32x4 gemm_load4(const float* base, int c, int c_lim,
 template <int WM, int WN, bool A_KC, bool B_KC>
 __global__ void __launch_bounds__(256)
 k_gemm(const float* __restrict__ A, int lda, const float* __restrict__ B, int ldb, float* C, int ldc, int M, int N,
-       int K, int k_per_split, float alpha, float beta, float* partial, bool a_vec, bool b_vec) {
+       int K, int k_per_split, float alpha, float beta, float* partial, bool a_vec, bool b_vec, GemmEpilogue epi) {
   constexpr int BM = 64 * WM, BN = 64 * WN;
   // Row pitch in LDS: a k-contiguous operand is written transposed, one float per lane
   // (lane = 4 k-quads x rows), which is free of bank conflicts when pitch % 8 == 2; the
@@ -242,7 +259,7 @@ k_gemm(const float* __restrict__ A, int lda, const float* __restrict__ B, int ld
         if (n < N) {
           float* p = out + (size_t)n * ldo + m;
           if (split) *p = acc[j][i][v];
-          else *p = (beta == 0.f ? 0.f : beta * *p) + alpha * acc[j][i][v];
+          else *p = gemm_finish((beta == 0.f ? 0.f : beta * *p) + alpha * acc[j][i][v], m, epi);
         }
       }
     }
@@ -312,7 +329,7 @@ __device__ __forceinline__ void small_load(const float* __restrict__ P, unsigned
 template <bool A_KC, bool B_KC, int NW>
 __global__ void __launch_bounds__(NW * 64)
 k_gemm_small(const float* __restrict__ A, int lda, const float* __restrict__ B, int ldb, float* C, int ldc, int M, int N,
-             int K, float alpha, float beta, bool a_vec, bool b_vec) {
+             int K, float alpha, float beta, bool a_vec, bool b_vec, GemmEpilogue epi) {
   constexpr int RED = NW / 2 > 4 ? NW / 2 : 4;
   __shared__ float red[RED][16 * 64];
   const int tid = threadIdx.x, lane = tid & 63;
@@ -377,7 +394,7 @@ k_gemm_small(const float* __restrict__ A, int lda, const float* __restrict__ B, 
     const int nn = blockIdx.y * 32 + 8 * (v >> 2) + 4 * lk + (v & 3);
     if (m_ok && nn < N) {
       float* p = C + (size_t)nn * ldc + m;
-      *p = (beta == 0.f ? 0.f : beta * *p) + alpha * sum;
+      *p = gemm_finish((beta == 0.f ? 0.f : beta * *p) + alpha * sum, m, epi);
     }
   }
 }
@@ -408,10 +425,10 @@ __global__ void k_scale(float* C, int ldc, int M, int N, float beta) {
 template <int WM, int WN>
 static void launch_gemm(bool a_kc, bool b_kc, dim3 grid, const float* A, int lda, const float* B, int ldb, float* C,
                         int ldc, int M, int N, int K, int kps, float alpha, float beta, float* partial, bool a_vec,
-                        bool b_vec) {
+                        bool b_vec, GemmEpilogue epi) {
 #define GEMM_GO(AK, BK_)                                                                                         \
   hipLaunchKernelGGL((k_gemm<WM, WN, AK, BK_>), grid, dim3(256), 0, 0, A, lda, B, ldb, C, ldc, M, N, K, kps, alpha, \
-                     beta, partial, a_vec, b_vec)
+                     beta, partial, a_vec, b_vec, epi)
   if (a_kc && b_kc) GEMM_GO(true, true);
   else if (a_kc) GEMM_GO(true, false);
   else if (b_kc) GEMM_GO(false, true);
@@ -420,8 +437,12 @@ static void launch_gemm(bool a_kc, bool b_kc, dim3 grid, const float* A, int lda
 }
 
 // Host-side dispatch shared with tests through dot().
+// epi: what to append to each output (bias / activation); *fused tells the caller whether
+// the launch could carry it (the split-K and empty-K paths cannot).
 static int gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, const float* A, int lda, const float* B,
-                int ldb, float beta, float* C, int ldc) {
+                int ldb, float beta, float* C, int ldc, GemmEpilogue epi = GemmEpilogue{nullptr, GEMM_ACT_NONE},
+                bool* fused = nullptr) {
+  if (fused) *fused = false;
   if (M <= 0 || N <= 0) return 0;
   const int cus = dn_num_cus();
   if (K <= 0) {
@@ -445,16 +466,17 @@ static int gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, co
   do {                                                                                                       \
     if (K <= 128)                                                                                            \
       hipLaunchKernelGGL((k_gemm_small<AK, BK_, 4>), grid, dim3(256), 0, 0, A, lda, B, ldb, C, ldc, M, N, K,  \
-                         alpha, beta, a_vec, b_vec);                                                         \
+                         alpha, beta, a_vec, b_vec, epi);                                                    \
     else                                                                                                     \
       hipLaunchKernelGGL((k_gemm_small<AK, BK_, 8>), grid, dim3(512), 0, 0, A, lda, B, ldb, C, ldc, M, N, K,  \
-                         alpha, beta, a_vec, b_vec);                                                         \
+                         alpha, beta, a_vec, b_vec, epi);                                                    \
   } while (0)
     if (a_kc && b_kc) GEMM_SMALL(true, true);
     else if (a_kc) GEMM_SMALL(true, false);
     else if (b_kc) GEMM_SMALL(false, true);
     else GEMM_SMALL(false, false);
 #undef GEMM_SMALL
+    if (fused) *fused = true;
     return dn_launch_status();
   }
   const long long tiles_big = (long long)((M + 127) / 128) * ((N + 127) / 128);
@@ -478,8 +500,10 @@ static int gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, co
     if (!partial) return CUDA_ERROR;
   }
   dim3 grid(gx, gy, splits);
-  if (big) launch_gemm<2, 2>(a_kc, b_kc, grid, A, lda, B, ldb, C, ldc, M, N, K, kps, alpha, beta, partial, a_vec, b_vec);
-  else launch_gemm<1, 1>(a_kc, b_kc, grid, A, lda, B, ldb, C, ldc, M, N, K, kps, alpha, beta, partial, a_vec, b_vec);
+  const GemmEpilogue none = {nullptr, GEMM_ACT_NONE};
+  if (big) launch_gemm<2, 2>(a_kc, b_kc, grid, A, lda, B, ldb, C, ldc, M, N, K, kps, alpha, beta, partial, a_vec, b_vec, splits > 1 ? none : epi);
+  else launch_gemm<1, 1>(a_kc, b_kc, grid, A, lda, B, ldb, C, ldc, M, N, K, kps, alpha, beta, partial, a_vec, b_vec, splits > 1 ? none : epi);
+  if (fused) *fused = splits == 1;
   if (splits > 1) {
     size_t total = (size_t)M * N;
     unsigned blocks = (unsigned)((total + 255) / 256 < (size_t)cus * 8 ? (total + 255) / 256 : (size_t)cus * 8);
@@ -492,6 +516,13 @@ static int gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, co
 int dn_gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, const float* A, int lda, const float* B,
             int ldb, float beta, float* C, int ldc) {
   return gemm(a_trans, b_trans, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc);
+}
+
+// C = act(op(A)*op(B) + bias) for dot_bias_act(); *fused: whether the launch carried bias and act.
+int dn_gemm_fused(bool a_trans, bool b_trans, int M, int N, int K, const float* A, int lda, const float* B, int ldb,
+                  float* C, int ldc, const float* bias, int act, bool* fused) {
+  const GemmEpilogue epi = {bias, act};
+  return gemm(a_trans, b_trans, M, N, K, 1.f, A, lda, B, ldb, 0.f, C, ldc, epi, fused);
 }
 
 extern "C" {

@@ -89,6 +89,7 @@ _SIGNATURES = {
     'compute_cross_entropy_bernoulli': (_i, [_M, _M, _M, _f]),
     'correct_preds': (_i, [_M, _M, _M, _f]),
     'dot': (_i, [_M, _M, _M, _f, _f]),
+    'dot_bias_act': (_i, [_M, _M, _M, _M, ct.c_int]),
     'vdot': (_f, [_M, _M, ct.POINTER(_i)]), 'euclid_norm': (_f, [_M, ct.POINTER(_i)]),
     'add_mult': (_i, [_M, _M, _f]), 'add_mult_sign': (_i, [_M, _M, _f]),
     'assign_scalar': (_i, [_M, _f]),
@@ -766,6 +767,25 @@ def dot(m1, m2, mult=1.0, target=None):
         n = _cudamat.get_nonleading_dimension(m2.p_mat)
         target = empty((m, n))
     _check(_cudamat.dot(m1.p_mat, m2.p_mat, target.p_mat, 0., float(mult)))
+    return target
+
+
+_ACTS = {None: 0, 'none': 0, 'linear': 0, 'sigmoid': 1, 'logistic': 1, 'relu': 2, 'rectified_linear': 2, 'tanh': 3}
+
+
+def dot_bias_act(m1, m2, bias=None, target=None, act='sigmoid'):
+    """Extension of this backend (not in the reference): target = act(m1 . m2 + bias) in
+    one launch, bit-identical to
+        cm.dot(m1, m2, target=target); target.add_col_vec(bias); target.apply_sigmoid()
+    (act: None, 'sigmoid', 'relu' = lower_bound(0), 'tanh'; bias: rows x 1 or None)."""
+    if act not in _ACTS:
+        raise ValueError("act must be one of %s" % sorted(k for k in _ACTS if k))
+    if target is None:
+        m = _cudamat.get_leading_dimension(m1.p_mat)
+        n = _cudamat.get_nonleading_dimension(m2.p_mat)
+        target = empty((m, n))
+    _check(_cudamat.dot_bias_act(m1.p_mat, m2.p_mat, bias.p_mat if bias is not None else None, target.p_mat,
+                                 _ACTS[act]))
     return target
 
 

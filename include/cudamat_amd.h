@@ -156,6 +156,11 @@ int dot(cudamat* mat1, cudamat* mat2, cudamat* target, float beta, float alpha);
 float vdot(cudamat* mat1, cudamat* mat2, int* err_code);
 int add_mult(cudamat* mat1, cudamat* mat2, float alpha);
 float euclid_norm(cudamat* mat, int* err_code);
+/* Extension, no counterpart in cudamat.cu: target = act(op(mat1)*op(mat2) + bias) in one
+ * launch, bit-identical to dot -> add_col_vec -> apply_sigmoid / lower_bound_scalar(0) /
+ * apply_tanh (the sequence of deepnet/dbm.py:95-105, deepnet/neuralnet.py:138-160).
+ * bias: rows(target) x 1 or NULL; act: 0 none, 1 sigmoid, 2 max(x,0), 3 tanh. */
+int dot_bias_act(cudamat* mat1, cudamat* mat2, cudamat* bias, cudamat* target, int act);
 
 /* ---- binary elementwise and activation derivatives: cudamat.cu:1782-2030 ---- */
 int add_mult_sign(cudamat* mat1, cudamat* mat2, float mult);

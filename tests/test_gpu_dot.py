@@ -115,3 +115,63 @@ def test_large_square_products(cm, rng, n):
     assert np.max(np.abs(ct_.asarray()[np.ix_(rows, cols)] - want_t) / bound_t) < REL
     for h in (a, b, c, ct_):
         h.free_device_memory()
+
+
+# ---- the fused extension: dot -> add_col_vec -> activation in one call
+
+@pytest.mark.parametrize("m,n,k,ta,tb", [
+    (500, 100, 784, True, False),      # RBM up pass (single-launch kernel)
+    (784, 100, 500, False, False),     # RBM down pass
+    (1024, 128, 784, True, False),     # MLP layer
+    (10, 128, 1024, True, False),      # MLP output layer (fewer rows than a tile)
+    (300, 700, 96, False, True),       # mid-sized: split-K path, falls back to separate launches
+    (2048, 2048, 64, False, False),    # big tiles, fused epilogue
+    (37, 1, 50, False, False),         # one output column: matrix-vector kernel
+])
+@pytest.mark.parametrize("act", [None, 'sigmoid', 'relu', 'tanh'])
+def test_dot_bias_act_is_bit_identical_to_the_three_calls(cm, rng, m, n, k, ta, tb, act):
+    a = np.asarray(rng.standard_normal((k, m) if ta else (m, k)), dtype=np.float32, order='F')
+    b = np.asarray(rng.standard_normal((n, k) if tb else (k, n)), dtype=np.float32, order='F')
+    bias = np.asarray(rng.standard_normal((m, 1)), dtype=np.float32, order='F')
+    A, B, V = cm.CUDAMatrix(a), cm.CUDAMatrix(b), cm.CUDAMatrix(bias)
+    opa, opb = (A.T if ta else A), (B.T if tb else B)
+    want = cm.empty((m, n))
+    cm.dot(opa, opb, target=want)
+    want.add_col_vec(V)
+    if act == 'sigmoid':
+        want.apply_sigmoid()
+    elif act == 'relu':
+        want.lower_bound(0)
+    elif act == 'tanh':
+        cm.tanh(want)
+    got = cm.CUDAMatrix(np.full((m, n), np.nan, dtype=np.float32))
+    r = cm.dot_bias_act(opa, opb, V, target=got, act=act)
+    assert r is got
+    assert np.array_equal(got.asarray().view(np.uint32), want.asarray().view(np.uint32))
+    # without a bias, and allocating its own target
+    got2 = cm.dot_bias_act(opa, opb, None, act=act)
+    want2 = cm.dot(opa, opb)
+    if act == 'sigmoid':
+        want2.apply_sigmoid()
+    elif act == 'relu':
+        want2.lower_bound(0)
+    elif act == 'tanh':
+        cm.tanh(want2)
+    assert np.array_equal(got2.asarray().view(np.uint32), want2.asarray().view(np.uint32))
+    for x in (A, B, V, want, got, got2, want2):
+        x.free_device_memory()
+
+
+def test_dot_bias_act_errors(cm, rng):
+    A = cm.CUDAMatrix(np.zeros((8, 5), dtype=np.float32))
+    B = cm.CUDAMatrix(np.zeros((5, 3), dtype=np.float32))
+    T = cm.empty((8, 3))
+    with pytest.raises(cm.CUDAMatException):
+        cm.dot_bias_act(A, B, cm.CUDAMatrix(np.zeros((3, 1), dtype=np.float32)), target=T)     # bias of the wrong length
+    with pytest.raises(cm.CUDAMatException):
+        cm.dot_bias_act(A, B, None, target=cm.empty((8, 4)))
+    with pytest.raises(ValueError):
+        cm.dot_bias_act(A, B, None, target=T, act='softsign')
+    host_only = cm.CUDAMatrix(np.zeros((8, 1), dtype=np.float32), copy_to_device=False)
+    with pytest.raises(cm.CUDAMatException):
+        cm.dot_bias_act(A, B, host_only, target=T)
