@@ -206,3 +206,29 @@ def test_locally_connected_layers(cm, cc, rng, N, C, H, F, k, s, p):
     assert np.allclose(down.asarray(), co.local_down(y, w, C, H, p, s), rtol=1e-4, atol=1e-5)
     cc.localOutp(X, Y, outp, Mx, p, k, s, C)
     assert np.allclose(outp.asarray(), co.local_outp(x, y, C, Mx, k, p, s), rtol=1e-4, atol=1e-4)
+
+
+def _random_conv_cases(seed, count):
+    """Seeded layer geometries that reach every convolution code path: batch 128/256 for the
+    buffer-load kernels (few or many colours, strided or not), batch 16/48 for the general
+    matrix-core kernels, odd batches for the one-lane-per-output kernels."""
+    r = np.random.default_rng(seed)
+    out = []
+    while len(out) < count:
+        N = int(r.choice([128, 128, 256, 16, 48, 6]))
+        G = int(r.choice([1, 1, 2]))
+        Cg = int(r.choice([1, 2, 3, 4, 16, 20, 24]))
+        Fg = int(r.choice([16, 32, 48]))
+        k = int(r.integers(2, 6))
+        s = int(r.integers(1, k + 1))
+        p = int(r.integers(0, k))
+        H = int(r.integers(k, 12))
+        if co.n_modules(H, k, s, p) < 1 or N * Cg * G * H * H > 3_000_000:
+            continue
+        out.append((N, Cg * G, H, Fg * G, k, s, p, G))
+    return out
+
+
+@pytest.mark.parametrize("N,C,H,F,k,s,p,G", _random_conv_cases(20240607, 24))
+def test_three_conv_passes_on_random_geometries(cm, cc, rng, N, C, H, F, k, s, p, G):
+    test_three_conv_passes(cm, cc, rng, N, C, H, F, k, s, p, G)
