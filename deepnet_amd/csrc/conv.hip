@@ -658,30 +658,32 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
 }
 
 // dW(f, q) = scale_t*dW + scale_o * sum over splits of partial[z][g][q][fl].
-// 64 outputs per workgroup; its 4 wavefronts take every 4th split, four loads in
-// flight each, and meet in LDS (fixed order of additions).
+// 16 outputs per workgroup; 16 lane groups take every 16th split, eight loads in flight
+// each, and meet in LDS (fixed order of additions).
 __global__ void __launch_bounds__(256) k_conv_outp_finish(ConvArgs p) {
-  __shared__ float sv[4][64];
-  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  __shared__ float sv[16][17];
+  const int r = threadIdx.x & 15, grp = threadIdx.x >> 4;
   const int per_group = p.Fg * p.Cg * p.kk2;
   const int total = p.G * per_group;
-  const int e = blockIdx.x * 64 + lane;
+  const int e = blockIdx.x * 16 + r;
   float acc = 0.f;
   if (e < total) {
-    int z = wv;
-    for (; z + 12 < p.splits; z += 16) {
-      float v[4];
+    int z = grp;
+    for (; z + 112 < p.splits; z += 128) {
+      float v[8];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) v[u] = p.partial[(size_t)(z + 4 * u) * total + e];
+      for (int u = 0; u < 8; ++u) v[u] = p.partial[(size_t)(z + 16 * u) * total + e];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) acc += v[u];
+      for (int u = 0; u < 8; ++u) acc += v[u];
     }
-    for (; z < p.splits; z += 4) acc += p.partial[(size_t)z * total + e];
+    for (; z < p.splits; z += 16) acc += p.partial[(size_t)z * total + e];
   }
-  sv[wv][lane] = acc;
+  sv[grp][r] = acc;
   __syncthreads();
-  if (wv == 0 && e < total) {
-    const float sum = (sv[0][lane] + sv[1][lane]) + (sv[2][lane] + sv[3][lane]);
+  if (grp == 0 && e < total) {
+    float sum = sv[0][r];
+#pragma unroll
+    for (int g2 = 1; g2 < 16; ++g2) sum += sv[g2][r];
     const int g = e / per_group, rem = e - g * per_group;
     const int q = rem / p.Fg, fl = rem - q * p.Fg;
     float* t = p.out + (size_t)p.F * q + g * p.Fg + fl;
@@ -951,7 +953,7 @@ static void conv_outp_impl(cudamat* images, cudamat* hidActs, cudamat* targets, 
       const int BMs = Fg <= 32 ? 32 : Fg <= 64 ? 64 : Fg <= 96 ? 96 : 128;
       const int gx = (Fg + BMs - 1) / BMs, gy = (cols + 127) / 128;
       const int nslabs = a.m_count * (N / CV_BK);
-      // about two workgroups per CU, at least 16 slabs (256 of the reduction) per split
+      // about two workgroups per CU (measured against one and three), at least 16 slabs (256 of the reduction) per split
       long long want = (2ll * dn_num_cus()) / ((long long)gx * gy * numGroups);
       if (want < 1) want = 1;
       if (want > nslabs / 16) want = nslabs / 16 > 0 ? nslabs / 16 : 1;
@@ -966,7 +968,7 @@ static void conv_outp_impl(cudamat* images, cudamat* hidActs, cudamat* targets, 
       else if (BMs == 96) hipLaunchKernelGGL((k_conv_mfma<CONV_OUTP, 1, 3, 1>), grid, dim3(256), 0, 0, a);
       else hipLaunchKernelGGL((k_conv_mfma<CONV_OUTP, 2, 2, 2>), grid, dim3(256), 0, 0, a);
       const int total = F * cols;
-      hipLaunchKernelGGL(k_conv_outp_finish, dim3((total + 63) / 64), dim3(256), 0, 0, a);
+      hipLaunchKernelGGL(k_conv_outp_finish, dim3((total + 15) / 16), dim3(256), 0, 0, a);
     } else {
       hipLaunchKernelGGL(k_conv_outp_direct, dim3((unsigned)(F * cols)), dim3(256), 0, 0, a);
     }
