@@ -128,6 +128,56 @@ k_pool_undo(const float* imgs, const float* maxGrads, const float* maxActs, floa
   }
 }
 
+// Gradient of max pooling for the usual shapes (window and stride known at compile time,
+// 4 images per lane): a pixel is covered by at most NC x NC windows; every load is
+// unconditional, from window coordinates clamped into the map, so that all of a lane's
+// loads are in flight together, and what fell outside is dropped by a select.  (The same
+// treatment of the forward pass measured slower than its loop and is not used.)
+template <int SUBS, int STRIDE>
+__global__ void __launch_bounds__(256)
+k_pool_undo_fixed(const float* imgs, const float* maxGrads, const float* maxActs, float* target, PoolGeom g) {
+  constexpr int NC = (SUBS + STRIDE - 1) / STRIDE;
+  const uint32_t total = (uint32_t)g.NV * g.S * g.S * g.F;
+  for (uint32_t e = blockIdx.x * 256u + threadIdx.x; e < total; e += gridDim.x * 256u) {
+    int nv, px, py, f;
+    decode4(e, g.dNV, g.dS, g.S, &nv, &px, &py, &f);
+    const size_t poff = (size_t)g.N * ((size_t)(f * g.S + py) * g.S + px) + nv * 4;
+    const int ty = py - g.start, tx = px - g.start;
+    const int oy_hi = ty >= 0 ? ty / STRIDE : 0, ox_hi = tx >= 0 ? tx / STRIDE : 0;
+    const Vec<4> img = Vec<4>::load(imgs + poff);
+    Vec<4> ma[NC][NC], mg[NC][NC];
+    bool ok[NC][NC];
+#pragma unroll
+    for (int jy = 0; jy < NC; ++jy) {
+      const int oy = oy_hi - (NC - 1 - jy);                  // ascending, as the reference scans
+      const bool vy = (ty >= 0) & (oy >= 0) & (oy < g.O) & (ty - oy * STRIDE < SUBS);
+      const int oyc = oy < 0 ? 0 : (oy >= g.O ? g.O - 1 : oy);
+#pragma unroll
+      for (int jx = 0; jx < NC; ++jx) {
+        const int ox = ox_hi - (NC - 1 - jx);
+        ok[jy][jx] = vy & (tx >= 0) & (ox >= 0) & (ox < g.O) & (tx - ox * STRIDE < SUBS);
+        const int oxc = ox < 0 ? 0 : (ox >= g.O ? g.O - 1 : ox);
+        const size_t ooff = (size_t)g.N * ((size_t)(f * g.O + oyc) * g.O + oxc) + nv * 4;
+        ma[jy][jx] = Vec<4>::load(maxActs + ooff);
+        mg[jy][jx] = Vec<4>::load(maxGrads + ooff);
+      }
+    }
+    Vec<4> acc;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc.v[i] = 0.f;
+#pragma unroll
+    for (int jy = 0; jy < NC; ++jy)
+#pragma unroll
+      for (int jx = 0; jx < NC; ++jx)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float t = (img.v[i] == ma[jy][jx].v[i] ? 1.f : 0.f) * mg[jy][jx].v[i];
+          acc.v[i] += ok[jy][jx] ? t : 0.f;
+        }
+    acc.store(target + poff);
+  }
+}
+
 // x^y for the normalisation layers through the hardware log2 / exp2 (the reference uses
 // __powf there, cudamat_conv_kernels.cu:112-176); relative error below 1e-6 for the
 // denominators these layers see (1 <= x < ~1e3).
@@ -485,7 +535,13 @@ void MaxPoolUndo(cudamat* images, cudamat* maxGrads, cudamat* maxActs, cudamat* 
   PoolGeom g;
   make_geom(g, N, F, S, outputsX, subsX, startX, strideX, v4 ? 4 : 1);
   const unsigned grid = grid_for(total / (v4 ? 4 : 1));
-  if (v4)
+  if (v4 && g.subs == 3 && g.stride == 2)
+    hipLaunchKernelGGL((k_pool_undo_fixed<3, 2>), dim3(grid), dim3(256), 0, 0, (const float*)images->data_device,
+                       (const float*)maxGrads->data_device, (const float*)maxActs->data_device, targets->data_device, g);
+  else if (v4 && g.subs == 2 && g.stride == 2)
+    hipLaunchKernelGGL((k_pool_undo_fixed<2, 2>), dim3(grid), dim3(256), 0, 0, (const float*)images->data_device,
+                       (const float*)maxGrads->data_device, (const float*)maxActs->data_device, targets->data_device, g);
+  else if (v4)
     hipLaunchKernelGGL((k_pool_undo<4>), dim3(grid), dim3(256), 0, 0, (const float*)images->data_device,
                        (const float*)maxGrads->data_device, (const float*)maxActs->data_device, targets->data_device, g);
   else

@@ -114,6 +114,8 @@ def test_bad_shapes_raise_instead_of_aborting(cm, cc, rng):
 POOLS = [  # N, F, S, subs, start, stride
     (2, 3, 8, 2, 0, 2), (5, 4, 9, 3, 0, 2), (16, 16, 32, 3, 0, 2), (16, 8, 7, 3, -1, 2), (128, 64, 32, 3, 0, 2),
     (4, 2, 6, 2, 0, 1),
+    (8, 3, 9, 2, 0, 2), (12, 2, 10, 2, -1, 2), (8, 4, 11, 3, -2, 2), (4, 3, 5, 3, 0, 2), (16, 2, 8, 3, 1, 2),   # vector kernels with fixed window shapes
+    (8, 2, 9, 3, 0, 3), (4, 2, 12, 4, -1, 3),    # other shapes: the general kernels
 ]
 
 
