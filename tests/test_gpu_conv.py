@@ -1,7 +1,8 @@
 """GPU parity of convUp / convDown / convOutp, MaxPool(+Undo), ResponseNorm(+Undo)
 against the float64 restatement: 1e-4 relative for the convolutions (error measured
 against the sum of magnitudes, as for dot), exact for pooling, 2e-6 relative for the
-normalisation.  Shapes with a batch that is not a multiple of 16 run the
+normalisation's denominators and 1e-5 for its outputs (x^-p through the hardware log2 / exp2,
+as the reference's __powf).  Shapes with a batch that is not a multiple of 16 run the
 one-lane-per-output kernels; the others the matrix-core kernel."""
 import numpy as np
 import pytest
