@@ -760,6 +760,181 @@ static int isqrt_exact(int v) {
   return r * r == v ? r : -1;
 }
 
+// ------------------------------------------------------------------ convUp, short reductions
+// Layers whose reduction (colours x k x k) has at most 2*KS terms and whose groups
+// have at most 32*CT filters (a first layer over RGB is the usual case) do not need
+// LDS tiles: the whole filter bank of a group lives in registers as MFMA operands
+// and a wavefront walks over tiles of (one module, 32 images).  An image operand is
+// used by this wavefront only, so it goes from global memory straight into the
+// operand register: lane (image n, half h) loads tap k = 2*ks + h for step ks, a
+// 128-byte run per half wavefront.  Interior modules need no vector ALU work at all
+// (fixed lane offsets, module origin in a scalar register); modules that touch the
+// padding mask taps by a bit test and send them out of the buffer's range, where
+// loads return zero.  Output: 128-byte runs per filter.
+// Schedule of a wavefront: while tile i is multiplied, the loads of tile i+1 and the
+// stores of tile i-1 are issued between its MFMAs, so the matrix pipe is never idle
+// behind memory instructions, and the arrival of tile i+1 is awaited at one place
+// (the hand-over), where only the stores of tile i-1 are younger and may stay in flight.
+template <int KS, int CT>
+__global__ void __launch_bounds__(256, 1) k_conv_up_regs(ConvArgs p) {
+  constexpr unsigned FAR = 0x80000000u;  // beyond any buffer here: sizes are below 2^31 bytes
+  __shared__ unsigned yx_tab[2 * KS], tap_tab[2 * KS];
+  const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5, ln = lane & 31;
+  const int g = blockIdx.z;
+  const int K = p.Cg * p.kk2;
+  for (int k = tid; k < 2 * KS; k += 256) {
+    const unsigned c = fd_div((unsigned)k, p.dkk2), r = (unsigned)k - c * (unsigned)p.kk2;
+    const unsigned ky = fd_div(r, p.dk), kx = r - ky * (unsigned)p.k;
+    yx_tab[k] = k < K ? (1u << ky) | (1u << (16 + kx)) : 0xffffffffu;
+    tap_tab[k] = k < K ? ((((unsigned)(g * p.Cg) + c) * p.H + ky) * p.H + kx) * (unsigned)p.N * 4u : FAR;
+  }
+  __amdgpu_buffer_rsrc_t r_img = __builtin_amdgcn_make_buffer_rsrc((void*)p.img, 0, (int)p.a_bytes, 0x00020000);
+  __amdgpu_buffer_rsrc_t r_flt = __builtin_amdgcn_make_buffer_rsrc((void*)p.flt, 0, (int)p.b_bytes, 0x00020000);
+  __amdgpu_buffer_rsrc_t r_out =
+      __builtin_amdgcn_make_buffer_rsrc((void*)p.out, 0, (int)((unsigned)p.N * (unsigned)p.M * (unsigned)p.F * 4u), 0x00020000);
+
+  // Filter operands of this lane: element (filter, tap k) sits at filter + F*k, so a
+  // tap beyond the reduction is beyond the buffer and reads as zero.
+  float b[KS][CT];
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    const int fl = ct * 32 + ln;
+    const unsigned voff = fl < p.Fg ? ((unsigned)(g * p.Fg + fl) + (unsigned)(half * p.F)) * 4u : FAR;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+      b[ks][ct] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r_flt, (int)voff, ks * 8 * p.F, 0));
+  }
+  __syncthreads();
+  unsigned tap[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) tap[ks] = tap_tab[2 * ks + half] + ln * 4u;
+
+  const int NB = p.N >> 5;
+  const int T = p.M * NB;
+  const int nwaves = gridDim.x * 4;
+  const unsigned fstride = (unsigned)p.N * (unsigned)p.M * 4u;        // bytes between filters in the output
+  const unsigned out_lane = ln * 4u + (unsigned)(4 * half) * fstride;
+
+  // One tile step.  MULT: multiply tile `a` into `cur`.  Always: gather tile tn into
+  // `an` and store `prev` (products of the tile whose output offset is out_prev; FAR
+  // drops them).  acc[ct][v] of lane (n, half) is filter ct*32 + 8*(v/4) + 4*half + v%4.
+  auto step = [&](auto mult_tag, const float (&a)[KS], float (&an)[KS], f32x16 (&cur)[CT], const f32x16 (&prev)[CT],
+                  int tn, unsigned out_prev) __attribute__((always_inline)) {
+    constexpr bool MULT = decltype(mult_tag)::value;
+    const int m = (int)fd_div((unsigned)tn, p.dS), nb = tn - m * NB;  // (dS: divisor N/32 for this kernel)
+    const int my = (int)fd_div((unsigned)m, p.dMx), mx = m - my * p.Mx;
+    const int y0 = my * p.s + p.pad0, x0 = mx * p.s + p.pad0;
+    const int base = ((y0 * p.H + x0) * p.N + nb * 32) * 4;
+    const bool interior = y0 >= 0 && x0 >= 0 && y0 + p.k <= p.H && x0 + p.k <= p.H;
+    // bit ky (kx) set: row y0 + ky (column x0 + kx) lies inside the image
+    const int ylo = y0 < 0 ? -y0 : 0, yhi = p.H - y0 < p.k ? p.H - y0 : p.k;
+    const int xlo = x0 < 0 ? -x0 : 0, xhi = p.H - x0 < p.k ? p.H - x0 : p.k;
+    const unsigned ym = yhi > ylo ? ((1u << yhi) - 1u) & ~((1u << ylo) - 1u) : 0u;
+    const unsigned xm = xhi > xlo ? ((1u << xhi) - 1u) & ~((1u << xlo) - 1u) : 0u;
+    const unsigned bad = ~(ym | (xm << 16));
+    unsigned octet[CT][4];  // filters per group are a multiple of 8: an octet is stored whole or dropped
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        octet[ct][q] = out_prev != FAR && ct * 32 + 8 * q < p.Fg ? out_prev + (unsigned)(ct * 32 + 8 * q) * fstride : FAR;
+    if (MULT) {
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) cur[ct][v] = 0.f;
+    }
+    // Loads in the first half of the steps (two per step: the last one still has half a
+    // tile of MFMAs to arrive behind), stores in the second half.
+    constexpr int SPS = (16 * CT + (KS - KS / 2) - 1) / (KS - KS / 2);  // stores per step
+    auto rest = [&](int ks) __attribute__((always_inline)) {
+      if (ks >= KS / 2) {
+#pragma unroll
+        for (int u = 0; u < SPS; ++u) {
+          const int si = (ks - KS / 2) * SPS + u;
+          if (si < 16 * CT) {
+            const float val = prev[si >> 4][si & 15];  // (a bit cast applied to the vector element itself reads element 0)
+            __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(val), r_out, (int)out_lane,
+                                                  (int)(octet[si >> 4][(si >> 2) & 3] + (si & 3) * fstride), 0);
+          }
+        }
+      }
+      if (MULT) {
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct)
+          cur[ct] = __builtin_amdgcn_mfma_f32_32x32x2f32(b[ks][ct], a[ks], cur[ct], 0, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    if (interior) {
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        if (ks < KS / 2) {
+#pragma unroll
+          for (int u = 0; u < 2; ++u)
+            an[2 * ks + u] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r_img, (int)tap[2 * ks + u], base, 0));
+        }
+        rest(ks);
+      }
+    } else {
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        if (ks < KS / 2) {
+#pragma unroll
+          for (int u = 0; u < 2; ++u) {
+            const unsigned yx = yx_tab[2 * (2 * ks + u) + half];
+            const unsigned voff = (yx & bad) ? FAR : tap[2 * ks + u] + (unsigned)base;
+            an[2 * ks + u] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r_img, (int)voff, 0, 0));
+          }
+        }
+        rest(ks);
+      }
+    }
+  };
+  auto out_of = [&](int t) {
+    const int m = (int)fd_div((unsigned)t, p.dS), nb = t - m * NB;
+    return ((unsigned)(nb * 32) + (unsigned)p.N * (unsigned)m) * 4u + (unsigned)(g * p.Fg) * fstride;
+  };
+  // Round i hands tile i*nwaves + (wave + 12*i) mod nwaves to a wavefront: the shift keeps
+  // a wavefront from meeting the same image column in every round (rounds are often a
+  // whole number of module rows apart), which would give some all the tiles that touch
+  // the padding and need the masked gather.
+  const int wave = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(tid >> 6);
+  auto tile_of = [&](int round) {
+    int w = wave + 12 * round;
+    w -= (int)fd_div((unsigned)w, p.dSS) * nwaves;  // (dSS: divisor nwaves for this kernel)
+    return round * nwaves + w;
+  };
+  int round = 0;
+  int t = tile_of(0);
+  if (t >= T) return;
+  float a0[KS], a1[KS];
+  f32x16 acc0[CT], acc1[CT];
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) { acc0[ct][v] = 0.f; acc1[ct][v] = 0.f; }
+  step(std::false_type(), a1, a0, acc0, acc1, t, FAR);
+  // Nothing is in flight when the loop is entered: the waits inside it are then those of
+  // its own steady state (the compiler sizes a wait for the path with the fewest
+  // operations behind the awaited one; a first trip with loads still in flight and no
+  // stores behind them would make every later trip wait for its stores).
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+  unsigned out_prev = FAR;
+  while (true) {
+    int tn = tile_of(++round);
+    step(std::true_type(), a0, a1, acc0, acc1, tn < T ? tn : t, out_prev);
+    out_prev = out_of(t);
+    if (tn >= T) { step(std::false_type(), a0, a0, acc1, acc0, t, out_prev); break; }
+    t = tn;
+    tn = tile_of(++round);
+    step(std::true_type(), a1, a0, acc1, acc0, tn < T ? tn : t, out_prev);
+    out_prev = out_of(t);
+    if (tn >= T) { step(std::false_type(), a1, a1, acc0, acc1, t, out_prev); break; }
+    t = tn;
+  }
+}
+
 static bool fast_ok(const ConvArgs& a) {
   // (the gathers use 32-bit byte offsets that include a margin for the padding / tap shift)
   const long long margin = (long long)a.N * ((long long)(a.k + (a.pad0 < 0 ? -a.pad0 : 0)) * (a.H + a.Mx) + a.k + a.H);
@@ -842,7 +1017,23 @@ static void conv_up_impl(cudamat* images, cudamat* filters, cudamat* targets, in
   a.img = images->data_device; a.flt = filters->data_device; a.hid = nullptr; a.out = targets->data_device;
   a.local = local ? 1 : 0;
   set_buffer_ranges(a, (long long)N * numImgColors * H * H, (long long)F * filters->size[1]);
-  if (!local && fast_ok(a)) {
+  const int K = a.Cg * a.kk2;
+  if (!local && fast_ok(a) && K <= 80 && a.Fg <= 64 && N % 32 == 0 && a.a_bytes != 0 && a.b_bytes != 0) {
+    // short reduction, few filters per group: filter bank in registers
+    const long long tiles = (long long)M * (N / 32);
+    long long blocks = (tiles + 3) / 4;
+    if (blocks > dn_num_cus()) blocks = dn_num_cus();  // one wavefront per SIMD, looping over tiles
+    const dim3 grid((unsigned)blocks, 1, numGroups);
+    a.dS = make_fastdiv((uint32_t)(N / 32));  // tile -> (module, image block)
+    a.dSS = make_fastdiv((uint32_t)(blocks * 4)); // wavefronts of a group
+    if (K <= 32) {
+      if (a.Fg <= 32) hipLaunchKernelGGL((k_conv_up_regs<16, 1>), grid, dim3(256), 0, 0, a);
+      else hipLaunchKernelGGL((k_conv_up_regs<16, 2>), grid, dim3(256), 0, 0, a);
+    } else {
+      if (a.Fg <= 32) hipLaunchKernelGGL((k_conv_up_regs<40, 1>), grid, dim3(256), 0, 0, a);
+      else hipLaunchKernelGGL((k_conv_up_regs<40, 2>), grid, dim3(256), 0, 0, a);
+    }
+  } else if (!local && fast_ok(a)) {
     launch_rowmajor<CONV_UP>(a, (long long)M * N, a.Fg, numGroups);
   } else {
     const long long total = (long long)N * M * F;

@@ -33,6 +33,10 @@ CASES = [  # N, C, H, F, k, stride, padding, groups
     (128, 4, 9, 32, 3, 2, 1, 2),     # the same: 2 groups of 2 colours
     (256, 8, 8, 16, 5, 2, 2, 1),     # the same: 8 colours x 4 phases = 32 columns, batch 256
     (128, 16, 7, 16, 3, 3, 0, 1),    # the same: 16 colours x 9 phases = 144 columns (two column tiles), stride == k
+    (64, 3, 10, 48, 5, 1, 2, 1),     # convUp with the filter bank in registers: 48 filters (a half-used column block)
+    (96, 1, 11, 64, 5, 2, 1, 1),     # the same: 3 image blocks per module, 25 taps, stride 2
+    (32, 5, 6, 16, 4, 1, 3, 1),      # the same: exactly 80 taps, padding 3 (every module touches the padding)
+    (32, 2, 9, 128, 3, 1, 1, 2),     # the same: 2 groups of 64 filters
 ]
 
 
