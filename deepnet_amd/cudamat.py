@@ -53,7 +53,27 @@ class rnd_struct(ct.Structure):
                 ('dev_rnd_words', ct.POINTER(ct.c_longlong))]
 
 
+class sparse_data(ct.Structure):
+    """Mirror of struct sparse_data (cudamat/cudamat.cuh:36-39)."""
+    _fields_ = [('indices', ct.POINTER(ct.c_int)),
+                ('indptr', ct.POINTER(ct.c_int)),
+                ('data', ct.POINTER(ct.c_float))]
+
+
+class cudamat_sparse(ct.Structure):
+    """Mirror of struct cudamat_sparse (cudamat/cudamat.cuh:41-50)."""
+    _fields_ = [('data_host', sparse_data),
+                ('data_device', sparse_data),
+                ('on_device', ct.c_int),
+                ('on_host', ct.c_int),
+                ('size', ct.c_int * 2),
+                ('is_trans', ct.c_int),
+                ('owns_data', ct.c_int),
+                ('nnz', ct.c_int)]
+
+
 _M = ct.POINTER(cudamat)
+_S = ct.POINTER(cudamat_sparse)
 _R = ct.POINTER(rnd_struct)
 _f, _i, _u = ct.c_float, ct.c_int, ct.c_uint
 
@@ -90,6 +110,11 @@ _SIGNATURES = {
     'correct_preds': (_i, [_M, _M, _M, _f]),
     'dot': (_i, [_M, _M, _M, _f, _f]),
     'dot_bias_act': (_i, [_M, _M, _M, _M, ct.c_int]),
+    'init_from_sparse_array': (None, [_S, ct.POINTER(ct.c_float), ct.POINTER(ct.c_int), ct.POINTER(ct.c_int),
+                                      _i, _i, _i]),
+    'allocate_device_memory_sparse': (_i, [_S]), 'copy_sparse_to_device': (_i, [_S]),
+    'free_device_memory_sparse': (_i, [_S]),
+    'sparse_dot': (_i, [_S, _M, _M, _f, _f]),
     'vdot': (_f, [_M, _M, ct.POINTER(_i)]), 'euclid_norm': (_f, [_M, ct.POINTER(_i)]),
     'add_mult': (_i, [_M, _M, _f]), 'add_mult_sign': (_i, [_M, _M, _f]),
     'assign_scalar': (_i, [_M, _f]),
@@ -786,6 +811,44 @@ def dot_bias_act(m1, m2, bias=None, target=None, act='sigmoid'):
         target = empty((m, n))
     _check(_cudamat.dot_bias_act(m1.p_mat, m2.p_mat, bias.p_mat if bias is not None else None, target.p_mat,
                                  _ACTS[act]))
+    return target
+
+
+class SparseCUDAMatrix(object):
+    """A compressed-sparse-row matrix on the device.  The reference exports the C entry
+    points (cudamat.cu:125-213, 407-418, 1698-1727) but has no Python class for them; this
+    one only packs the three CSR arrays (data, indices, indptr as scipy.sparse.csr_matrix
+    holds them) into the C handle and uploads them."""
+
+    def __init__(self, data, indices, indptr, shape, copy_to_device=True):
+        self.data = np.ascontiguousarray(data, dtype=np.float32)
+        self.indices = np.ascontiguousarray(indices, dtype=np.int32)
+        self.indptr = np.ascontiguousarray(indptr, dtype=np.int32)
+        m, n = int(shape[0]), int(shape[1])
+        if self.indptr.size != m + 1 or self.data.size != self.indices.size:
+            raise ValueError("CSR arrays do not fit the shape")
+        self.shape = (m, n)
+        self.mat = cudamat_sparse()
+        self.p_mat = ct.pointer(self.mat)
+        _cudamat.init_from_sparse_array(self.p_mat, self.data.ctypes.data_as(ct.POINTER(ct.c_float)),
+                                        self.indices.ctypes.data_as(ct.POINTER(ct.c_int)),
+                                        self.indptr.ctypes.data_as(ct.POINTER(ct.c_int)), m, n, int(self.data.size))
+        if copy_to_device:
+            self.copy_to_device()
+
+    def copy_to_device(self):
+        _check(_cudamat.copy_sparse_to_device(self.p_mat))
+
+    def free_device_memory(self):
+        _check(_cudamat.free_device_memory_sparse(self.p_mat))
+
+
+def sparse_dot(sparse, dense, target=None, beta=0.0, alpha=1.0):
+    """target = beta * target + alpha * sparse . dense (cudamat.cu:1698-1727; dense and
+    target are taken as plain column-major arrays)."""
+    if target is None:
+        target = empty((sparse.shape[0], dense.mat.size[1]))
+    _check(_cudamat.sparse_dot(sparse.p_mat, dense.p_mat, target.p_mat, ct.c_float(beta), ct.c_float(alpha)))
     return target
 
 

@@ -44,6 +44,25 @@ typedef struct rnd_struct {
   unsigned long long* dev_words;
 } rnd_struct;
 
+/* Compressed-sparse-row matrix handle: cudamat/cudamat.cuh:36-50.  indptr has
+ * size[0] + 1 entries, indices and data nnz entries each. */
+typedef struct sparse_data {
+  int* indices;
+  int* indptr;
+  float* data;
+} sparse_data;
+
+typedef struct cudamat_sparse {
+  sparse_data data_host;
+  sparse_data data_device;
+  int on_device;
+  int on_host;
+  int size[2];
+  int is_trans; /* 0 or 1 */
+  int owns_data;
+  int nnz;
+} cudamat_sparse;
+
 #define NUM_RND_STREAMS 12288 /* cudamat_kernels.cuh:4-6 */
 #define NUM_RND_BURNIN 100    /* cudamat_kernels.cuh:18 */
 
@@ -161,6 +180,17 @@ float euclid_norm(cudamat* mat, int* err_code);
  * apply_tanh (the sequence of deepnet/dbm.py:95-105, deepnet/neuralnet.py:138-160).
  * bias: rows(target) x 1 or NULL; act: 0 none, 1 sigmoid, 2 max(x,0), 3 tanh. */
 int dot_bias_act(cudamat* mat1, cudamat* mat2, cudamat* bias, cudamat* target, int act);
+
+/* ---- sparse (CSR) x dense: cudamat.cu:125-153, 188-213, 407-418, 1698-1727.
+ * sparse_dot: target = beta*target + alpha * mat1 * mat2 with mat2 (k x n) and target
+ * (m x n) read as plain column-major arrays (their is_trans flags are ignored, as in the
+ * reference).  Unlike the reference, a target that is not m x n is refused (-1). ---- */
+void init_from_sparse_array(cudamat_sparse* mat, float* data, int* indices, int* indptr, int m, int n, int nnz);
+int allocate_device_memory_sparse(cudamat_sparse* mat);
+int copy_sparse_to_device(cudamat_sparse* mat);
+int sparse_dot(cudamat_sparse* mat1, cudamat* mat2, cudamat* target, float beta, float alpha);
+/* Extension, no counterpart in cudamat.cu (which never frees a sparse matrix). */
+int free_device_memory_sparse(cudamat_sparse* mat);
 
 /* ---- binary elementwise and activation derivatives: cudamat.cu:1782-2030 ---- */
 int add_mult_sign(cudamat* mat1, cudamat* mat2, float mult);

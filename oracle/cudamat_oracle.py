@@ -203,6 +203,23 @@ def dot(a, b, c=None, beta=0.0, alpha=1.0, trans_a=False, trans_b=False):
     return out
 
 
+def sparse_dot(data, indices, indptr, dense, target=None, beta=0.0, alpha=1.0):
+    """CSR (m x k) times dense (k x n): the loop of kSparseDot (cudamat_kernels.cu:370-384),
+    target[row, col] = alpha * sum_i data[i] * dense[indices[i], col] + beta * target[row, col]
+    over i in [indptr[row], indptr[row+1]), summed in float64 here.  The launcher
+    (cudamat.cu:1698-1727) reads dense and target as plain column-major arrays."""
+    dense = _a(dense)
+    m, n = len(indptr) - 1, dense.shape[1]
+    out = np.zeros((m, n), dtype=F64)
+    for row in range(m):
+        for i in range(int(indptr[row]), int(indptr[row + 1])):
+            out[row, :] += F64(np.float32(data[i])) * dense[int(indices[i]), :]
+    out = F64(np.float32(alpha)) * out
+    if beta != 0.0:
+        out = out + F64(np.float32(beta)) * _a(target)
+    return out
+
+
 # ---- reductions: cudamat.cu:1148-1315, cudamat_kernels.cu:936-1088 ----------
 
 FLT_MAX = float(np.finfo(np.float32).max)

@@ -94,3 +94,16 @@ def test_missing_library_is_loud(tmp_path, monkeypatch):
     mod = importlib.util.module_from_spec(spec)
     with pytest.raises(ImportError, match="no CPU fallback"):
         spec.loader.exec_module(mod)
+
+
+def test_sparse_struct_layout_and_host_side_init():
+    from deepnet_amd import cudamat as cm
+    # three pointers; two of them + 7 ints, padded to pointer alignment (cudamat.cuh:36-50)
+    assert ct.sizeof(cm.sparse_data) == 24 and ct.sizeof(cm.cudamat_sparse) == 80
+    assert cm.cudamat_sparse.size.offset == 56 and cm.cudamat_sparse.nnz.offset == 72
+    sp = cm.SparseCUDAMatrix([1.0, 2.0, 3.0], [0, 2, 1], [0, 2, 3], (2, 3), copy_to_device=False)
+    assert (sp.mat.size[0], sp.mat.size[1], sp.mat.nnz) == (2, 3, 3)
+    assert sp.mat.on_host == 1 and sp.mat.on_device == 0 and sp.mat.owns_data == 1 and sp.mat.is_trans == 0
+    assert sp.mat.data_host.indptr[2] == 3 and sp.mat.data_host.data[1] == 2.0
+    with pytest.raises(ValueError):
+        cm.SparseCUDAMatrix([1.0], [0], [0, 1], (2, 3), copy_to_device=False)

@@ -175,3 +175,50 @@ def test_dot_bias_act_errors(cm, rng):
     host_only = cm.CUDAMatrix(np.zeros((8, 1), dtype=np.float32), copy_to_device=False)
     with pytest.raises(cm.CUDAMatException):
         cm.dot_bias_act(A, B, host_only, target=T)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("m,k,n,density", [(37, 29, 11, 0.2), (64, 64, 16, 0.1), (1000, 4096, 128, 0.01),
+                                           (5, 7, 1, 0.5), (300, 50, 19, 0.0)])
+def test_sparse_dot(cm, rng, m, k, n, density):
+    # CSR x dense against the loop restatement (itself pinned against scipy); rows are
+    # summed in fp32 in index order on the device: tolerance 1e-5 of sum |terms|
+    import scipy.sparse as sps
+    S = sps.random(m, k, density=density, format='csr', random_state=7, dtype=np.float32)
+    S.sort_indices()
+    D = np.asarray(rng.standard_normal((k, n)), dtype=np.float32, order='F')
+    T = np.asarray(rng.standard_normal((m, n)), dtype=np.float32, order='F')
+    sp_ = cm.SparseCUDAMatrix(S.data, S.indices, S.indptr, (m, k))
+    d, t = cm.CUDAMatrix(D), cm.CUDAMatrix(T)
+    bound = np.abs(S).astype(np.float64) @ np.abs(D).astype(np.float64)
+    for beta, alpha in ((0.0, 1.0), (-0.5, 2.0)):
+        t2 = cm.CUDAMatrix(T)
+        cm.sparse_dot(sp_, d, target=t2, beta=beta, alpha=alpha)
+        want = orc.sparse_dot(S.data, S.indices, S.indptr, D, T, beta=beta, alpha=alpha)
+        assert np.max(np.abs(t2.asarray() - want) / (abs(alpha) * bound + abs(beta) * np.abs(T) + 1e-6)) < 1e-5
+        t2.free_device_memory()
+    # beta = 0 must overwrite, not scale, what the target held (NaN * 0 would stay NaN)
+    t3 = cm.CUDAMatrix(np.full((m, n), np.nan, dtype=np.float32))
+    cm.sparse_dot(sp_, d, target=t3)
+    assert np.all(np.isfinite(t3.asarray()))
+    out = cm.sparse_dot(sp_, d)                      # allocates its own m x n target
+    assert out.shape == (m, n) and np.array_equal(out.asarray(), t3.asarray())
+    sp_.free_device_memory()
+    for x in (d, t, t3, out):
+        x.free_device_memory()
+
+
+@pytest.mark.gpu
+def test_sparse_dot_errors(cm, rng):
+    import scipy.sparse as sps
+    S = sps.random(8, 6, density=0.5, format='csr', random_state=1, dtype=np.float32)
+    sp_ = cm.SparseCUDAMatrix(S.data, S.indices, S.indptr, (8, 6))
+    host_only = cm.SparseCUDAMatrix(S.data, S.indices, S.indptr, (8, 6), copy_to_device=False)
+    d = cm.CUDAMatrix(np.zeros((6, 3), dtype=np.float32))
+    with pytest.raises(cm.CUDAMatException):         # not on the device (-8)
+        cm.sparse_dot(host_only, d)
+    with pytest.raises(cm.CUDAMatException):         # inner dimensions differ (-1)
+        cm.sparse_dot(sp_, cm.CUDAMatrix(np.zeros((5, 3), dtype=np.float32)))
+    with pytest.raises(cm.CUDAMatException):         # target of the wrong shape (-1; the reference would overrun it)
+        cm.sparse_dot(sp_, d, target=cm.empty((8, 2)))
+    assert cm._cudamat.sparse_dot(host_only.p_mat, d.p_mat, d.p_mat, 0.0, 1.0) == -8

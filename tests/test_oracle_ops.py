@@ -141,3 +141,26 @@ def test_fastdiv_magic_numbers_used_by_the_device_kernels():
         for n in [0, 1, d - 1, d, d + 1, 2 * d - 1, 2 ** 32 - 1, 2 ** 31, 123456789] + list(rng.integers(0, 2 ** 32, 200)):
             n = int(n)
             assert div(n, f) == n // d, (n, d)
+
+
+def test_sparse_dot_against_scipy_and_a_dense_product(rng):
+    # the loop restatement against two independent routines: scipy's CSR product and the
+    # dense product of the densified matrix; a wrong index array (indices vs indptr), a
+    # transposed dense operand or beta/alpha swapped would fail
+    import scipy.sparse as sps
+    m, k, n = 37, 29, 11
+    S = sps.random(m, k, density=0.2, format='csr', random_state=3, dtype=np.float32)
+    S = S.tolil()
+    S[5, :] = 0          # an empty row
+    S = S.tocsr()
+    S.sort_indices()
+    D = np.asarray(rng.standard_normal((k, n)), dtype=np.float32)
+    T = np.asarray(rng.standard_normal((m, n)), dtype=np.float32)
+    got = orc.sparse_dot(S.data, S.indices, S.indptr, D, T, beta=-0.5, alpha=2.0)
+    want = 2.0 * (S.astype(np.float64) @ D.astype(np.float64)) - 0.5 * T.astype(np.float64)
+    assert np.allclose(got, want, rtol=1e-12, atol=1e-12)
+    dense = np.asarray(S.todense(), dtype=np.float64)
+    assert np.allclose(orc.sparse_dot(S.data, S.indices, S.indptr, D), dense @ D.astype(np.float64), rtol=1e-12, atol=1e-12)
+    # a hand-checked 2 x 3 case: rows [1 0 2], [0 3 0]
+    got = orc.sparse_dot([1, 2, 3], [0, 2, 1], [0, 2, 3], np.array([[1., 10.], [2., 20.], [3., 30.]]))
+    assert np.array_equal(got, np.array([[7., 70.], [6., 60.]]))
