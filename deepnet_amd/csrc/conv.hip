@@ -701,6 +701,116 @@ __global__ void __launch_bounds__(256) k_conv_outp_finish(ConvArgs p) {
 int dn_gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, const float* A, int lda, const float* B,
             int ldb, float beta, float* C, int ldc);
 
+// The patch product for layers with at most 2*KS filters per group and at most 32*CT
+// patch columns, without LDS tiles: W of the group sits in registers as MFMA operands
+// and a wavefront walks over tiles of 32 rows of hid (one module, 32 images), whose
+// operands go from global memory straight into the operand registers (lane (image n,
+// half h) loads filter 2*ks + h for step ks: 128-byte runs).  While tile i is
+// multiplied, the loads of tile i+1 and the stores of tile i-1 are issued between its
+// MFMAs.  Every path issues the same number of memory operations and nothing is in
+// flight when the loop is entered, so that the compiler's wait counts (sized for the
+// path with the fewest operations behind the awaited one) are those of the steady
+// state.  P has pcols rounded up to 8 columns; the extra ones are written as zeros.
+template <int KS, int CT>
+__global__ void __launch_bounds__(256, 1)
+k_conv_patch_regs(const float* hid, const float* flt, float* P, int prow, int Fg, int F, int pcols, int pcols8) {
+  constexpr unsigned FAR = 0x80000000u;  // beyond any buffer here: sizes are below 2^31 bytes
+  const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5, ln = lane & 31;
+  __amdgpu_buffer_rsrc_t r_hid =
+      __builtin_amdgcn_make_buffer_rsrc((void*)hid, 0, (int)((unsigned)prow * (unsigned)Fg * 4u), 0x00020000);
+  __amdgpu_buffer_rsrc_t r_flt =
+      __builtin_amdgcn_make_buffer_rsrc((void*)flt, 0, (int)((unsigned)F * (unsigned)pcols * 4u), 0x00020000);
+  __amdgpu_buffer_rsrc_t r_out =
+      __builtin_amdgcn_make_buffer_rsrc((void*)P, 0, (int)((unsigned)prow * (unsigned)pcols8 * 4u), 0x00020000);
+  // W(f, q) of the group at f + F*q (flt already points at the group's first filter)
+  float b[KS][CT];
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    const int q = ct * 32 + ln;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int f = 2 * ks + half;
+      const unsigned off = q < pcols && f < Fg ? ((unsigned)f + (unsigned)F * (unsigned)q) * 4u : FAR;
+      b[ks][ct] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r_flt, (int)off, 0, 0));
+    }
+  }
+  const int T = prow >> 5;
+  const int nwaves = gridDim.x * 4;
+  const unsigned cstride = (unsigned)prow * 4u;                      // bytes between columns of hid and of P
+  const unsigned in_lane = ln * 4u + (unsigned)half * cstride;       // a filter beyond the group is beyond the buffer
+  const unsigned out_lane = ln * 4u + (unsigned)(4 * half) * cstride;
+
+  // One tile step.  MULT: multiply tile `a` into `cur`.  Always: load tile tn into `an`
+  // and store `prev` at row offset out_prev (FAR drops it).  acc[ct][v] of lane (n, half)
+  // is patch column ct*32 + 8*(v/4) + 4*half + v%4.
+  auto step = [&](auto mult_tag, const float (&a)[KS], float (&an)[KS], f32x16 (&cur)[CT], const f32x16 (&prev)[CT],
+                  int tn, unsigned out_prev) __attribute__((always_inline)) {
+    constexpr bool MULT = decltype(mult_tag)::value;
+    const unsigned base = (unsigned)tn * 128u;
+    unsigned octet[CT][4];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        octet[ct][q] = out_prev != FAR && ct * 32 + 8 * q < pcols8 ? out_prev + (unsigned)(ct * 32 + 8 * q) * cstride : FAR;
+    if (MULT) {
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) cur[ct][v] = 0.f;
+    }
+    constexpr int SPS = (16 * CT + (KS - KS / 2) - 1) / (KS - KS / 2);  // stores per step
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      if (ks < KS / 2) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+          an[2 * ks + u] = __builtin_bit_cast(
+              float, __builtin_amdgcn_raw_buffer_load_b32(r_hid, (int)in_lane, (int)(base + (unsigned)(4 * ks + 2 * u) * cstride), 0));
+      } else {
+#pragma unroll
+        for (int u = 0; u < SPS; ++u) {
+          const int si = (ks - KS / 2) * SPS + u;
+          if (si < 16 * CT) {
+            const float val = prev[si >> 4][si & 15];  // (a bit cast applied to the vector element itself reads element 0)
+            __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(val), r_out, (int)out_lane,
+                                                  (int)(octet[si >> 4][(si >> 2) & 3] + (si & 3) * cstride), 0);
+          }
+        }
+      }
+      if (MULT) {
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct)
+          cur[ct] = __builtin_amdgcn_mfma_f32_32x32x2f32(b[ks][ct], a[ks], cur[ct], 0, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  int t = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(tid >> 6);
+  if (t >= T) return;
+  float a0[KS], a1[KS];
+  f32x16 acc0[CT], acc1[CT];
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) { acc0[ct][v] = 0.f; acc1[ct][v] = 0.f; }
+  step(std::false_type(), a1, a0, acc0, acc1, t, FAR);
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): nothing in flight when the loop is entered
+  unsigned out_prev = FAR;
+  while (true) {
+    int tn = t + nwaves;
+    step(std::true_type(), a0, a1, acc0, acc1, tn < T ? tn : t, out_prev);
+    out_prev = (unsigned)t * 128u;
+    if (tn >= T) { step(std::false_type(), a0, a0, acc1, acc0, t, out_prev); break; }
+    t = tn;
+    tn = t + nwaves;
+    step(std::true_type(), a1, a0, acc1, acc0, tn < T ? tn : t, out_prev);
+    out_prev = (unsigned)t * 128u;
+    if (tn >= T) { step(std::false_type(), a1, a1, acc0, acc1, t, out_prev); break; }
+    t = tn;
+  }
+}
+
 __global__ void __launch_bounds__(256) k_conv_down_gather(ConvArgs p, const float* P, int g) {
   // one lane: 4 neighbouring images of one (colour of the group, y, x)
   const int NV = p.N >> 2;
@@ -1082,12 +1192,24 @@ static void conv_down_impl(cudamat* hidActs, cudamat* filters, cudamat* targets,
   } else if (!local && fast_ok(a) && dn_aligned16(a.out) && a.Cg <= 16) {
     // few colours: patch-matrix form
     const long long prow = (long long)a.M * N;
-    const int pcols = a.Cg * a.kk2;
-    float* P = (float*)dn_scratch((size_t)prow * pcols * sizeof(float), 1);
+    const int pcols = a.Cg * a.kk2, pcols8 = (pcols + 7) & ~7;
+    float* P = (float*)dn_scratch((size_t)prow * pcols8 * sizeof(float), 1);
     if (!P) { conv_set_error(where, "out of device memory for the patch matrix"); return; }
+    // short reductions over the filters: the register-resident product
+    const bool regs = a.Fg <= 64 && pcols <= 96 && prow % 32 == 0 && prow * pcols8 * 4 < (1ll << 31) &&
+                      prow * a.Fg * 4 < (1ll << 31) && (long long)F * pcols * 4 < (1ll << 31);
     for (int g = 0; g < numGroups; ++g) {
-      if (dn_gemm(false, false, (int)prow, pcols, a.Fg, 1.f, a.hid + (size_t)g * a.Fg * prow, (int)prow,
-                  a.flt + (size_t)g * a.Fg, F, 0.f, P, (int)prow)) {
+      const float* hid_g = a.hid + (size_t)g * a.Fg * prow;
+      const float* flt_g = a.flt + (size_t)g * a.Fg;
+      if (regs) {
+        long long blocks = (prow / 32 + 3) / 4;
+        if (blocks > dn_num_cus()) blocks = dn_num_cus();  // one wavefront per SIMD, looping over tiles
+        const dim3 grid((unsigned)blocks);
+#define PATCH_REGS(KS, CT) hipLaunchKernelGGL((k_conv_patch_regs<KS, CT>), grid, dim3(256), 0, 0, hid_g, flt_g, P, (int)prow, a.Fg, F, pcols, pcols8)
+        if (a.Fg <= 32) { if (pcols <= 32) PATCH_REGS(16, 1); else if (pcols <= 64) PATCH_REGS(16, 2); else PATCH_REGS(16, 3); }
+        else { if (pcols <= 32) PATCH_REGS(32, 1); else if (pcols <= 64) PATCH_REGS(32, 2); else PATCH_REGS(32, 3); }
+#undef PATCH_REGS
+      } else if (dn_gemm(false, false, (int)prow, pcols, a.Fg, 1.f, hid_g, (int)prow, flt_g, F, 0.f, P, (int)prow)) {
         conv_set_error(where, "patch product failed");
         return;
       }
