@@ -494,3 +494,71 @@ int dot_bias_act(cudamat* mat1, cudamat* mat2, cudamat* bias, cudamat* target, i
 
 
 }  // extern "C"
+
+
+// ------------------------------------------------------------------ fused parameter update
+// The update of deepnet/parameter.py:80-106 in one pass over the parameter:
+//   w_delta = momentum*w_delta [+ l2*w] [+ l1*sign(w)] + gradient;  w -= epsilon*w_delta;
+//   [gradient = 0]
+// Each step rounds as the separate calls do (mult by a scalar: one multiply; add_mult: one
+// fused multiply-add; add_mult_sign: one add), so the results are the same bits.
+template <bool VEC>
+__global__ void __launch_bounds__(EW_THREADS)
+k_momentum_update(float* w, float* wd, float* g, long long n, float momentum, float l2, float l1, float eps,
+                  int use_l2, int use_l1, int reset) {
+  auto one = [&](float wv, float dv, float gv, float& w_out, float& d_out) {
+    float d = __fmul_rn(momentum, dv);
+    if (use_l2) d = __fmaf_rn(l2, wv, d);
+    if (use_l1) d = __fadd_rn(d, (wv > 0.f) ? l1 : ((wv < 0.f) ? -l1 : 0.f));
+    d = __fmaf_rn(1.f, gv, d);
+    d_out = d;
+    w_out = __fmaf_rn(-eps, d, wv);
+  };
+  const long long tid = (long long)blockIdx.x * EW_THREADS + threadIdx.x;
+  if (VEC) {
+    if (tid * 4 >= n) return;
+    const float4 wv = *reinterpret_cast<const float4*>(w + 4 * tid);
+    const float4 dv = *reinterpret_cast<const float4*>(wd + 4 * tid);
+    const float4 gv = *reinterpret_cast<const float4*>(g + 4 * tid);
+    float4 wo, dox;
+    one(wv.x, dv.x, gv.x, wo.x, dox.x);
+    one(wv.y, dv.y, gv.y, wo.y, dox.y);
+    one(wv.z, dv.z, gv.z, wo.z, dox.z);
+    one(wv.w, dv.w, gv.w, wo.w, dox.w);
+    *reinterpret_cast<float4*>(wd + 4 * tid) = dox;
+    *reinterpret_cast<float4*>(w + 4 * tid) = wo;
+    if (reset) *reinterpret_cast<float4*>(g + 4 * tid) = make_float4(0.f, 0.f, 0.f, 0.f);
+  } else {
+    if (tid >= n) return;
+    float wo, dox;
+    one(w[tid], wd[tid], g[tid], wo, dox);
+    wd[tid] = dox;
+    w[tid] = wo;
+    if (reset) g[tid] = 0.f;
+  }
+}
+
+// Extension (no counterpart in cudamat.cu).  Checks as add_mult: device, transposedness, dims.
+extern "C" int momentum_update(cudamat* w, cudamat* w_delta, cudamat* gradient, float momentum, float l2_decay,
+                               float l1_decay, float epsilon, int flags) {
+  if (!w->on_device || !w_delta->on_device || !gradient->on_device) return ERROR_NOT_ON_DEVICE;
+  if (w->is_trans != w_delta->is_trans || w->is_trans != gradient->is_trans) return ERROR_TRANSPOSEDNESS;
+  if (!same_dims(w, w_delta) || !same_dims(w, gradient)) return ERROR_INCOMPATIBLE_DIMENSIONS;
+  const long long n = dn_len(w);
+  if (n <= 0) return 0;
+  const int use_l2 = flags & 1, use_l1 = (flags >> 1) & 1, reset = (flags >> 2) & 1;
+  const bool vec = n % 4 == 0 && dn_aligned16(w->data_device) && dn_aligned16(w_delta->data_device) &&
+                   dn_aligned16(gradient->data_device);
+  const long long lanes = vec ? n / 4 : n;
+  const long long blocks = (lanes + EW_THREADS - 1) / EW_THREADS;
+  if (blocks > 0x7fffffffll) return ERROR_UNSUPPORTED;
+  if (vec)
+    hipLaunchKernelGGL((k_momentum_update<true>), dim3((unsigned)blocks), dim3(EW_THREADS), 0, 0, w->data_device,
+                       w_delta->data_device, gradient->data_device, n, momentum, l2_decay, l1_decay, epsilon, use_l2,
+                       use_l1, reset);
+  else
+    hipLaunchKernelGGL((k_momentum_update<false>), dim3((unsigned)blocks), dim3(EW_THREADS), 0, 0, w->data_device,
+                       w_delta->data_device, gradient->data_device, n, momentum, l2_decay, l1_decay, epsilon, use_l2,
+                       use_l1, reset);
+  return dn_launch_status();
+}

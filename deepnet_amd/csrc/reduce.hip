@@ -168,8 +168,18 @@ __global__ void __launch_bounds__(256) k_col_normlimit(const float* mat, float* 
 
 // Column softmax: max, sum of exp(x - max), divide (cudamat_kernels.cu:868-934).
 // The column is re-read from cache for the second and third pass.
+// Optional extras of the fused loss step (all three null for plain softmax): with
+// labels, loss[col] = -log(p[label] + tiny) and grad = p - onehot(label), each value
+// computed from the stored p exactly as get_softmax_cross_entropy / apply_softmax_grad do.
+struct SoftmaxExtras {
+  const float* labels;
+  float* loss;
+  float* grad;
+  float tiny;
+};
+
 template <int TPC>
-__global__ void __launch_bounds__(256) k_col_softmax(const float* mat, float* target, int w, int h) {
+__global__ void __launch_bounds__(256) k_col_softmax(const float* mat, float* target, int w, int h, SoftmaxExtras x) {
   __shared__ float lds4[4];
   COL_SETUP(TPC)
   const float* c = mat + (size_t)col * h;
@@ -180,14 +190,26 @@ __global__ void __launch_bounds__(256) k_col_softmax(const float* mat, float* ta
   float s = 0.f;
   if (active) for_each_in_col<TPC>(c, h, lane, [&](int, float v) { s += expf(v - m); });
   s = col_combine<TPC, false>(s, lds4);
-  if (active) for_each_in_col<TPC>(c, h, lane, [&](int r, float v) { t[r] = expf(v - m) / s; });
+  if (!active) return;
+  if (!x.labels) {
+    for_each_in_col<TPC>(c, h, lane, [&](int r, float v) { t[r] = expf(v - m) / s; });
+  } else {
+    const int label = (int)x.labels[col];
+    float* gcol = x.grad ? x.grad + (size_t)col * h : nullptr;
+    for_each_in_col<TPC>(c, h, lane, [&](int r, float v) {
+      const float pr = expf(v - m) / s;
+      t[r] = pr;
+      if (gcol) gcol[r] = pr - ((label == r) ? 1.f : 0.f);
+      if (x.loss && r == label) x.loss[col] = -logf(pr + x.tiny);
+    });
+  }
 }
 
 // Columns of at most 64 * 4 * NV floats stay in registers between the passes:
 // one read and one write of HBM per element.  Requires h % 4 == 0 and 16-byte
 // aligned columns.
 template <int NV>
-__global__ void __launch_bounds__(256) k_col_softmax_reg(const float* mat, float* target, int w, int h) {
+__global__ void __launch_bounds__(256) k_col_softmax_reg(const float* mat, float* target, int w, int h, SoftmaxExtras x) {
   const int col = blockIdx.x * 4 + (int)(threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   if (col >= w) return;
@@ -220,7 +242,22 @@ __global__ void __launch_bounds__(256) k_col_softmax_reg(const float* mat, float
 #pragma unroll
   for (int k = 0; k < NV; ++k) {
     const int j = lane + k * 64;
-    if (j < n4) dn_st4_rt(t4 + 4 * j, make_float4(v[k].x / s, v[k].y / s, v[k].z / s, v[k].w / s), stream);
+    if (j < n4) {
+      const float4 pr = make_float4(v[k].x / s, v[k].y / s, v[k].z / s, v[k].w / s);
+      dn_st4_rt(t4 + 4 * j, pr, stream);
+      if (x.labels) {
+        const int label = (int)x.labels[col], r0 = 4 * j;
+        if (x.grad)
+          dn_st4_rt(x.grad + (size_t)col * h + r0,
+                    make_float4(pr.x - ((label == r0) ? 1.f : 0.f), pr.y - ((label == r0 + 1) ? 1.f : 0.f),
+                                pr.z - ((label == r0 + 2) ? 1.f : 0.f), pr.w - ((label == r0 + 3) ? 1.f : 0.f)),
+                    stream);
+        if (x.loss && label >= r0 && label < r0 + 4) {
+          const float pl = label == r0 ? pr.x : (label == r0 + 1 ? pr.y : (label == r0 + 2 ? pr.z : pr.w));
+          x.loss[col] = -logf(pl + x.tiny);
+        }
+      }
+    }
   }
 }
 
@@ -631,20 +668,21 @@ int normlimit_by_axis(cudamat* mat, cudamat* target, int axis, float norm) {
   return ERROR_UNSUPPORTED;
 }
 
-static int softmax_impl(const float* in, float* out, int w, int h) {
+static int softmax_impl(const float* in, float* out, int w, int h, SoftmaxExtras x = SoftmaxExtras{nullptr, nullptr, nullptr, 0.f}) {
   if (w <= 0 || h <= 0) return 0;
-  const bool reg_ok = (h % 4 == 0) && dn_aligned16(in) && dn_aligned16(out) && h <= 64 * 4 * 16;
+  const bool reg_ok = (h % 4 == 0) && dn_aligned16(in) && dn_aligned16(out) && h <= 64 * 4 * 16 &&
+                      (!x.grad || dn_aligned16(x.grad));
   if (reg_ok) {
     const int n4 = h / 4;
     dim3 grid((w + 3) / 4), block(256);
-    if (n4 <= 64) hipLaunchKernelGGL((k_col_softmax_reg<1>), grid, block, 0, 0, in, out, w, h);
-    else if (n4 <= 128) hipLaunchKernelGGL((k_col_softmax_reg<2>), grid, block, 0, 0, in, out, w, h);
-    else if (n4 <= 256) hipLaunchKernelGGL((k_col_softmax_reg<4>), grid, block, 0, 0, in, out, w, h);
-    else if (n4 <= 512) hipLaunchKernelGGL((k_col_softmax_reg<8>), grid, block, 0, 0, in, out, w, h);
-    else hipLaunchKernelGGL((k_col_softmax_reg<16>), grid, block, 0, 0, in, out, w, h);
+    if (n4 <= 64) hipLaunchKernelGGL((k_col_softmax_reg<1>), grid, block, 0, 0, in, out, w, h, x);
+    else if (n4 <= 128) hipLaunchKernelGGL((k_col_softmax_reg<2>), grid, block, 0, 0, in, out, w, h, x);
+    else if (n4 <= 256) hipLaunchKernelGGL((k_col_softmax_reg<4>), grid, block, 0, 0, in, out, w, h, x);
+    else if (n4 <= 512) hipLaunchKernelGGL((k_col_softmax_reg<8>), grid, block, 0, 0, in, out, w, h, x);
+    else hipLaunchKernelGGL((k_col_softmax_reg<16>), grid, block, 0, 0, in, out, w, h, x);
     return dn_launch_status();
   }
-  return launch_cols(k_col_softmax<64>, k_col_softmax<256>, w, h, in, out, w, h);
+  return launch_cols(k_col_softmax<64>, k_col_softmax<256>, w, h, in, out, w, h, x);
 }
 
 int softmax(cudamat* mat, cudamat* target) {
@@ -652,6 +690,21 @@ int softmax(cudamat* mat, cudamat* target) {
   if (int e = check_axis_common(mat, target)) return e;
   if (target->size[0] != h || target->size[1] != w) return ERROR_INCOMPATIBLE_DIMENSIONS;
   return softmax_impl(mat->data_device, target->data_device, w, h);
+}
+
+// Extension (no counterpart in cudamat.cu): softmax -> get_softmax_cross_entropy ->
+// apply_softmax_grad in one launch; loss and grad may each be NULL.
+int softmax_ce_grad(cudamat* mat, cudamat* labels, cudamat* probs, cudamat* loss, cudamat* grad, float tiny) {
+  const int h = mat->size[0], w = mat->size[1];
+  if (int e = check_axis_common(mat, probs)) return e;
+  if (!labels->on_device || (loss && !loss->on_device) || (grad && !grad->on_device)) return ERROR_NOT_ON_DEVICE;
+  if (probs->size[0] != h || probs->size[1] != w) return ERROR_INCOMPATIBLE_DIMENSIONS;
+  if (labels->size[0] != 1 || labels->size[1] != w) return ERROR_INCOMPATIBLE_DIMENSIONS;
+  if (loss && (loss->size[0] != 1 || loss->size[1] != w)) return ERROR_INCOMPATIBLE_DIMENSIONS;
+  if (grad && (grad->size[0] != h || grad->size[1] != w)) return ERROR_INCOMPATIBLE_DIMENSIONS;
+  return softmax_impl(mat->data_device, probs->data_device, w, h,
+                      SoftmaxExtras{labels->data_device, loss ? loss->data_device : nullptr,
+                                    grad ? grad->data_device : nullptr, tiny});
 }
 
 int softmax_overwrite(cudamat* mat) {

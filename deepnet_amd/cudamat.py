@@ -110,6 +110,8 @@ _SIGNATURES = {
     'correct_preds': (_i, [_M, _M, _M, _f]),
     'dot': (_i, [_M, _M, _M, _f, _f]),
     'dot_bias_act': (_i, [_M, _M, _M, _M, ct.c_int]),
+    'momentum_update': (_i, [_M, _M, _M, _f, _f, _f, _f, ct.c_int]),
+    'softmax_ce_grad': (_i, [_M, _M, _M, _M, _M, _f]),
     'init_from_sparse_array': (None, [_S, ct.POINTER(ct.c_float), ct.POINTER(ct.c_int), ct.POINTER(ct.c_int),
                                       _i, _i, _i]),
     'allocate_device_memory_sparse': (_i, [_S]), 'copy_sparse_to_device': (_i, [_S]),
@@ -812,6 +814,30 @@ def dot_bias_act(m1, m2, bias=None, target=None, act='sigmoid'):
     _check(_cudamat.dot_bias_act(m1.p_mat, m2.p_mat, bias.p_mat if bias is not None else None, target.p_mat,
                                  _ACTS[act]))
     return target
+
+
+def softmax_ce_grad(mat, labels, probs=None, loss=None, grad=None, tiny=1e-10):
+    """Extension of this backend (not in the reference): one launch for
+        mat.apply_softmax(target=probs); probs.get_softmax_cross_entropy(labels, target=loss, tiny=tiny)
+        probs.apply_softmax_grad(labels, target=grad)
+    with the same bits; probs defaults to mat (in place), loss and grad are skipped when None."""
+    if probs is None:
+        probs = mat
+    _check(_cudamat.softmax_ce_grad(mat.p_mat, labels.p_mat, probs.p_mat, loss.p_mat if loss is not None else None,
+                                    grad.p_mat if grad is not None else None, ct.c_float(tiny)))
+    return probs
+
+
+def momentum_update(w, w_delta, gradient, momentum, epsilon, l2_decay=None, l1_decay=None, reset_gradient=True):
+    """Extension of this backend (not in the reference): the update of
+    deepnet/parameter.py:80-106 in one pass over the parameter, the same bits as
+        w_delta.mult(momentum); w_delta.add_mult(w, l2_decay); w_delta.add_mult_sign(w, l1_decay)
+        w_delta.add_mult(gradient); w.add_mult(w_delta, -epsilon); gradient.assign(0)
+    (the l2 / l1 terms only when a decay is given, the last call only with reset_gradient)."""
+    flags = (1 if l2_decay is not None else 0) | (2 if l1_decay is not None else 0) | (4 if reset_gradient else 0)
+    _check(_cudamat.momentum_update(w.p_mat, w_delta.p_mat, gradient.p_mat, ct.c_float(momentum),
+                                    ct.c_float(l2_decay or 0.0), ct.c_float(l1_decay or 0.0), ct.c_float(epsilon), flags))
+    return w
 
 
 class SparseCUDAMatrix(object):

@@ -181,6 +181,20 @@ float euclid_norm(cudamat* mat, int* err_code);
  * bias: rows(target) x 1 or NULL; act: 0 none, 1 sigmoid, 2 max(x,0), 3 tanh. */
 int dot_bias_act(cudamat* mat1, cudamat* mat2, cudamat* bias, cudamat* target, int act);
 
+/* Extension, no counterpart in cudamat.cu: the parameter update of deepnet/parameter.py:80-106
+ * in one pass, the same bits as the calls it replaces:
+ *   w_delta.mult(momentum); [w_delta.add_mult(w, l2_decay);] [w_delta.add_mult_sign(w, l1_decay);]
+ *   w_delta.add_mult(gradient); w.add_mult(w_delta, -epsilon); [gradient.assign(0)]
+ * flags: bit 0 apply l2_decay, bit 1 apply l1_decay, bit 2 clear the gradient. */
+int momentum_update(cudamat* w, cudamat* w_delta, cudamat* gradient, float momentum, float l2_decay, float l1_decay,
+                    float epsilon, int flags);
+
+/* Extension, no counterpart in cudamat.cu: softmax(mat) -> probs, and from the stored probs
+ * loss = -log(probs[label] + tiny) (1 x cols, may be NULL) and grad = probs - onehot(label)
+ * (may be NULL) in the same launch: the bits of softmax -> get_softmax_cross_entropy ->
+ * apply_softmax_grad (deepnet/softmax_layer.py:11-86).  probs may be mat itself. */
+int softmax_ce_grad(cudamat* mat, cudamat* labels, cudamat* probs, cudamat* loss, cudamat* grad, float tiny);
+
 /* ---- sparse (CSR) x dense: cudamat.cu:125-153, 188-213, 407-418, 1698-1727.
  * sparse_dot: target = beta*target + alpha * mat1 * mat2 with mat2 (k x n) and target
  * (m x n) read as plain column-major arrays (their is_trans flags are ignored, as in the

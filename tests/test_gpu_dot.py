@@ -222,3 +222,22 @@ def test_sparse_dot_errors(cm, rng):
     with pytest.raises(cm.CUDAMatException):         # target of the wrong shape (-1; the reference would overrun it)
         cm.sparse_dot(sp_, d, target=cm.empty((8, 2)))
     assert cm._cudamat.sparse_dot(host_only.p_mat, d.p_mat, d.p_mat, 0.0, 1.0) == -8
+
+
+@pytest.mark.gpu
+def test_fused_training_steps_of_the_bench_match_the_reference_sequences(cm):
+    # bench.py's RBM and MLP steps through the extensions leave the same bits in every
+    # parameter as the reference call sequences (same seeds, three steps each)
+    import bench
+    def run(cls, seed, fused, params):
+        cm.CUDAMatrix.init_random(seed)
+        model = cls(cm)
+        for _ in range(3):
+            (model.step_fused if fused else model.step)()
+        return [p.asarray().copy() for p in params(model)]
+    for cls, seed, params in ((bench.RBM, 1, lambda m: [m.W, m.bv, m.bh]),
+                              (bench.MLP, 3, lambda m: m.W + m.b + m.dW + [m.loss])):
+        plain, fused = run(cls, seed, False, params), run(cls, seed, True, params)
+        for a, b in zip(plain, fused):
+            assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+    cm.CUDAMatrix.init_random(1)

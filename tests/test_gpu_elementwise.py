@@ -359,3 +359,50 @@ def test_transcendentals_over_their_whole_range(cm, rng):
     cm.pow(a, 0.5)
     got = a.asarray().ravel()
     assert got[0] == 0 and np.isnan(got[1]) and abs(got[2] - np.sqrt(2)) < 1e-7 and np.isinf(got[3]) and np.isnan(got[4])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(784, 500), (1024, 1), (37, 13), (4096, 1024)])
+@pytest.mark.parametrize("l2,l1,reset", [(None, None, True), (0.0005, None, True), (0.0005, 0.001, False), (None, 0.001, True)])
+def test_momentum_update_is_bit_identical_to_the_calls_it_replaces(cm, rng, shape, l2, l1, reset):
+    # the sequence of deepnet/parameter.py:80-106 against the one-pass extension; the oracle
+    # pins the sequence's formula (float64, 2 ulp per step is too loose a bar for equality of
+    # the two device paths, which is asserted bit for bit)
+    w0 = np.asarray(rng.standard_normal(shape), dtype=np.float32, order='F')
+    w0.flat[::7] = 0.0                                   # sign(0) = 0 in the l1 term
+    d0 = np.asarray(0.1 * rng.standard_normal(shape), dtype=np.float32, order='F')
+    g0 = np.asarray(rng.standard_normal(shape), dtype=np.float32, order='F')
+    mom, eps = 0.9, 0.01
+    w, d, g = cm.CUDAMatrix(w0), cm.CUDAMatrix(d0), cm.CUDAMatrix(g0)
+    d.mult(mom)
+    if l2 is not None:
+        d.add_mult(w, l2)
+    if l1 is not None:
+        d.add_mult_sign(w, l1)
+    d.add_mult(g)
+    w.add_mult(d, -eps)
+    if reset:
+        g.assign(0)
+    w2, d2, g2 = cm.CUDAMatrix(w0), cm.CUDAMatrix(d0), cm.CUDAMatrix(g0)
+    cm.momentum_update(w2, d2, g2, mom, eps, l2_decay=l2, l1_decay=l1, reset_gradient=reset)
+    assert np.array_equal(w.asarray().view(np.uint32), w2.asarray().view(np.uint32))
+    assert np.array_equal(d.asarray().view(np.uint32), d2.asarray().view(np.uint32))
+    assert np.array_equal(g.asarray(), g2.asarray())
+    # and the formula itself, in float64
+    want_d = np.float32(mom) * d0.astype(np.float64) + (np.float32(l2) * w0.astype(np.float64) if l2 is not None else 0) \
+        + (np.float32(l1) * np.sign(w0).astype(np.float64) if l1 is not None else 0) + g0
+    want_w = w0 - np.float32(eps) * want_d
+    assert np.max(np.abs(d2.asarray() - want_d)) < 1e-5 and np.max(np.abs(w2.asarray() - want_w)) < 1e-5
+    for x in (w, d, g, w2, d2, g2):
+        x.free_device_memory()
+
+
+@pytest.mark.gpu
+def test_momentum_update_errors(cm, rng):
+    a = cm.CUDAMatrix(np.zeros((4, 3), dtype=np.float32))
+    b = cm.CUDAMatrix(np.zeros((3, 4), dtype=np.float32))
+    host = cm.CUDAMatrix(np.zeros((4, 3), dtype=np.float32), copy_to_device=False)
+    lib = cm._cudamat
+    assert lib.momentum_update(a.p_mat, a.p_mat, host.p_mat, 0.9, 0.0, 0.0, 0.01, 0) == -8
+    assert lib.momentum_update(a.p_mat, b.T.p_mat, a.p_mat, 0.9, 0.0, 0.0, 0.01, 0) == -7
+    assert lib.momentum_update(a.p_mat, b.p_mat, a.p_mat, 0.9, 0.0, 0.0, 0.01, 0) == -1

@@ -174,3 +174,45 @@ def test_full_size_4096_sum_max_softmax(cm, rng, axis):
         cols = np.arange(0, n, 97)
         assert _rel(got[:, cols], orc.softmax(x[:, cols])) < REL
     a.free_device_memory()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("h,w", [(10, 128), (1000, 64), (4096, 33), (7, 5), (256, 256)])
+def test_softmax_ce_grad_is_bit_identical_to_the_three_calls(cm, rng, h, w):
+    # both softmax kernels (columns held in registers: h % 4 == 0; generic otherwise)
+    x = np.asarray(3.0 * rng.standard_normal((h, w)), dtype=np.float32, order='F')
+    lab = np.asarray(rng.integers(0, h, (1, w)), dtype=np.float32, order='F')
+    X, L = cm.CUDAMatrix(x), cm.CUDAMatrix(lab)
+    p1, l1, g1 = cm.empty((h, w)), cm.empty((1, w)), cm.empty((h, w))
+    X.apply_softmax(target=p1)
+    p1.get_softmax_cross_entropy(L, l1, tiny=1e-10)
+    p1.apply_softmax_grad(L, target=g1)
+    p2, l2, g2 = cm.empty((h, w)), cm.empty((1, w)), cm.empty((h, w))
+    cm.softmax_ce_grad(X, L, probs=p2, loss=l2, grad=g2, tiny=1e-10)
+    for a, b in ((p1, p2), (l1, l2), (g1, g2)):
+        assert np.array_equal(a.asarray().view(np.uint32), b.asarray().view(np.uint32))
+    # in place, without loss or gradient: plain softmax
+    X2 = cm.CUDAMatrix(x)
+    cm.softmax_ce_grad(X2, L)
+    assert np.array_equal(X2.asarray().view(np.uint32), p1.asarray().view(np.uint32))
+    # and against the float64 definitions
+    e = np.exp(x.astype(np.float64) - x.max(axis=0, keepdims=True))
+    p = e / e.sum(axis=0, keepdims=True)
+    idx = lab.astype(int)[0]
+    assert np.max(np.abs(p2.asarray() - p)) < 1e-6
+    assert np.max(np.abs(l2.asarray()[0] + np.log(p[idx, np.arange(w)] + 1e-10)) / (1 + np.abs(np.log(p[idx, np.arange(w)] + 1e-10)))) < 1e-5
+    onehot = np.zeros((h, w)); onehot[idx, np.arange(w)] = 1
+    assert np.max(np.abs(g2.asarray() - (p - onehot))) < 1e-6
+
+
+@pytest.mark.gpu
+def test_softmax_ce_grad_errors(cm, rng):
+    X = cm.CUDAMatrix(np.zeros((5, 4), dtype=np.float32))
+    L = cm.CUDAMatrix(np.zeros((1, 4), dtype=np.float32))
+    lib = cm._cudamat
+    assert lib.softmax_ce_grad(X.p_mat, L.p_mat, cm.empty((4, 5)).p_mat, None, None, 0.0) == -1
+    assert lib.softmax_ce_grad(X.p_mat, cm.empty((1, 3)).p_mat, X.p_mat, None, None, 0.0) == -1
+    assert lib.softmax_ce_grad(X.p_mat, L.p_mat, X.p_mat, cm.empty((1, 3)).p_mat, None, 0.0) == -1
+    assert lib.softmax_ce_grad(X.T.p_mat, L.p_mat, X.p_mat, None, None, 0.0) == -5
+    host = cm.CUDAMatrix(np.zeros((1, 4), dtype=np.float32), copy_to_device=False)
+    assert lib.softmax_ce_grad(X.p_mat, host.p_mat, X.p_mat, None, None, 0.0) == -8
