@@ -722,18 +722,22 @@ k_conv_patch_regs(const float* hid, const float* flt, float* P, int prow, int Fg
       __builtin_amdgcn_make_buffer_rsrc((void*)flt, 0, (int)((unsigned)F * (unsigned)pcols * 4u), 0x00020000);
   __amdgpu_buffer_rsrc_t r_out =
       __builtin_amdgcn_make_buffer_rsrc((void*)P, 0, (int)((unsigned)prow * (unsigned)pcols8 * 4u), 0x00020000);
-  // W(f, q) of the group at f + F*q (flt already points at the group's first filter)
+  // W(f, q) of the group sits at f + F*q (flt already points at the group's first filter):
+  // lanes of an operand run along q, so it is read along f (whole cache lines) into LDS
+  // and picked up from there; rows of 32*CT + 1 floats keep both sides off bank conflicts.
+  constexpr int QP = 32 * CT + 1;
+  __shared__ float w_lds[2 * KS * QP];
+  for (int e = tid; e < 2 * KS * 32 * CT; e += 256) {
+    const int f = e % (2 * KS), q = e / (2 * KS);
+    const unsigned off = q < pcols && f < Fg ? ((unsigned)f + (unsigned)F * (unsigned)q) * 4u : FAR;
+    w_lds[f * QP + q] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r_flt, (int)off, 0, 0));
+  }
+  __syncthreads();
   float b[KS][CT];
 #pragma unroll
-  for (int ct = 0; ct < CT; ++ct) {
-    const int q = ct * 32 + ln;
+  for (int ct = 0; ct < CT; ++ct)
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      const int f = 2 * ks + half;
-      const unsigned off = q < pcols && f < Fg ? ((unsigned)f + (unsigned)F * (unsigned)q) * 4u : FAR;
-      b[ks][ct] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r_flt, (int)off, 0, 0));
-    }
-  }
+    for (int ks = 0; ks < KS; ++ks) b[ks][ct] = w_lds[(2 * ks + half) * QP + ct * 32 + ln];
   const int T = prow >> 5;
   const int nwaves = gridDim.x * 4;
   const unsigned cstride = (unsigned)prow * 4u;                      // bytes between columns of hid and of P
@@ -808,6 +812,53 @@ k_conv_patch_regs(const float* hid, const float* flt, float* P, int prow, int Fg
     out_prev = (unsigned)t * 128u;
     if (tn >= T) { step(std::false_type(), a1, a1, acc0, acc1, t, out_prev); break; }
     t = tn;
+  }
+}
+
+// Stride 1 with a compile-time filter size: every pixel has exactly K x K candidate
+// modules, the loops unroll and all K*K loads of a lane are in flight together (a tap
+// whose module lies outside the grid re-reads module 0 and is weighted by zero).
+template <int K>
+__global__ void __launch_bounds__(256) k_conv_down_gather_s1(ConvArgs p, const float* P, int g) {
+  const int NV = p.N >> 2;
+  const uint32_t total = (uint32_t)NV * p.HH * p.Cg;
+  const long long ldp = (long long)p.M * p.N;
+  for (uint32_t e = blockIdx.x * 256u + threadIdx.x; e < total; e += gridDim.x * 256u) {
+    const uint32_t nv = e % NV;
+    const uint32_t pix = (e / NV) % p.HH;
+    const int c = (int)(e / ((uint32_t)NV * p.HH));
+    const int y = (int)(pix / p.H) - p.pad0, x = (int)(pix % p.H) - p.pad0;  // padded-frame coordinates
+    const float* base = P + (long long)c * K * K * ldp + 4 * nv;
+    float4 v[K * K];
+    bool ok[K * K];
+#pragma unroll
+    for (int ky = 0; ky < K; ++ky)
+#pragma unroll
+      for (int kx = 0; kx < K; ++kx) {
+        const int my = y - ky, mx = x - kx;
+        const bool in = my >= 0 && my < p.Mx && mx >= 0 && mx < p.Mx;
+        ok[ky * K + kx] = in;
+        v[ky * K + kx] = *reinterpret_cast<const float4*>(base + (long long)(ky * K + kx) * ldp +
+                                                          (long long)(in ? my * p.Mx + mx : 0) * p.N);
+      }
+    // same order of additions as the general kernel: my (and within it mx) descending
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int ky = 0; ky < K; ++ky)
+#pragma unroll
+      for (int kx = 0; kx < K; ++kx)
+        if (ok[ky * K + kx]) {
+          const float4 t = v[ky * K + kx];
+          acc.x += t.x; acc.y += t.y; acc.z += t.z; acc.w += t.w;
+        }
+    float* t = p.out + (size_t)p.N * ((size_t)(g * p.Cg + c) * p.HH + pix) + 4 * nv;
+    float4 r = acc;
+    if (p.scale_t != 0.f || p.scale_o != 1.f) {
+      const float4 o = p.scale_t == 0.f ? make_float4(0.f, 0.f, 0.f, 0.f) : *reinterpret_cast<const float4*>(t);
+      r = make_float4(p.scale_t * o.x + p.scale_o * acc.x, p.scale_t * o.y + p.scale_o * acc.y,
+                      p.scale_t * o.z + p.scale_o * acc.z, p.scale_t * o.w + p.scale_o * acc.w);
+    }
+    *reinterpret_cast<float4*>(t) = r;
   }
 }
 
@@ -1216,7 +1267,10 @@ static void conv_down_impl(cudamat* hidActs, cudamat* filters, cudamat* targets,
       const long long lanes = (long long)(N / 4) * a.HH * a.Cg;
       long long blocks = (lanes + 255) / 256;
       if (blocks > dn_num_cus() * 64ll) blocks = dn_num_cus() * 64ll;
-      hipLaunchKernelGGL(k_conv_down_gather, dim3((unsigned)blocks), dim3(256), 0, 0, a, (const float*)P, g);
+      if (a.s == 1 && a.k == 3) hipLaunchKernelGGL((k_conv_down_gather_s1<3>), dim3((unsigned)blocks), dim3(256), 0, 0, a, (const float*)P, g);
+      else if (a.s == 1 && a.k == 5) hipLaunchKernelGGL((k_conv_down_gather_s1<5>), dim3((unsigned)blocks), dim3(256), 0, 0, a, (const float*)P, g);
+      else if (a.s == 1 && a.k == 7) hipLaunchKernelGGL((k_conv_down_gather_s1<7>), dim3((unsigned)blocks), dim3(256), 0, 0, a, (const float*)P, g);
+      else hipLaunchKernelGGL(k_conv_down_gather, dim3((unsigned)blocks), dim3(256), 0, 0, a, (const float*)P, g);
     }
   } else if (!local && fast_ok(a) && dn_aligned16(a.out)) {
     const int q = (imgSize + moduleStride - 1) / moduleStride;
