@@ -342,10 +342,19 @@ k_gemm_small(const float* __restrict__ A, int lda, const float* __restrict__ B, 
   f32x16 acc;
 #pragma unroll
   for (int v = 0; v < 16; ++v) acc[v] = 0.f;
-  // Three chunks per wavefront are requested before the first MFMA (for the RBM / MLP
-  // products that is all, or nearly all, of a wavefront's share of K): these kernels live
-  // on memory latency, not on throughput.
-  constexpr int DEPTH = 3;
+  // beta != 0: the outputs this lane will finish are read now, under the operand loads
+  constexpr int EPL = 1024 / (NW * 64);
+  float cprev[EPL];
+#pragma unroll
+  for (int u = 0; u < EPL; ++u) {
+    const int v = (tid + u * NW * 64) >> 6;
+    const int nn = blockIdx.y * 32 + 8 * (v >> 2) + 4 * lk + (v & 3);
+    cprev[u] = (beta != 0.f && m_ok && nn < N) ? C[(size_t)nn * ldc + m] : 0.f;
+  }
+  // Four chunks per wavefront are requested before the first MFMA (for the RBM / MLP
+  // products that is all of a wavefront's share of K, the ragged last chunk included):
+  // these kernels live on memory latency, not on throughput.
+  constexpr int DEPTH = 4;
   constexpr int STEP = 32 * NW;
   float a[DEPTH][16], b[DEPTH][16];
   int k0 = wv * 32;
@@ -388,14 +397,14 @@ k_gemm_small(const float* __restrict__ A, int lda, const float* __restrict__ B, 
   __syncthreads();
   // ... and let every lane finish its share of the 1024 outputs: element e = v*64 + lane
   // is C(m, n) with m = tile + lane%32, n = tile + 8*(v/4) + 4*(lane/32) + v%4.
-  for (int e = tid; e < 1024; e += NW * 64) {
+#pragma unroll
+  for (int u = 0; u < EPL; ++u) {
+    const int e = tid + u * NW * 64;
     const int v = e >> 6;
     const float sum = (red[0][e] + red[1][e]) + (red[2][e] + red[3][e]);
     const int nn = blockIdx.y * 32 + 8 * (v >> 2) + 4 * lk + (v & 3);
-    if (m_ok && nn < N) {
-      float* p = C + (size_t)nn * ldc + m;
-      *p = gemm_finish((beta == 0.f ? 0.f : beta * *p) + alpha * sum, m, epi);
-    }
+    if (m_ok && nn < N)
+      C[(size_t)nn * ldc + m] = gemm_finish((beta == 0.f ? 0.f : beta * cprev[u]) + alpha * sum, m, epi);
   }
 }
 
