@@ -1247,8 +1247,9 @@ static void conv_down_impl(cudamat* hidActs, cudamat* filters, cudamat* targets,
     float* P = (float*)dn_scratch((size_t)prow * pcols8 * sizeof(float), 1);
     if (!P) { conv_set_error(where, "out of device memory for the patch matrix"); return; }
     // short reductions over the filters: the register-resident product
-    const bool regs = a.Fg <= 64 && pcols <= 96 && prow % 32 == 0 && prow * pcols8 * 4 < (1ll << 31) &&
-                      prow * a.Fg * 4 < (1ll << 31) && (long long)F * pcols * 4 < (1ll << 31);
+    // (offsets are 32-bit: 96 columns of P, and the up to 64 filter rows the kernel asks for, must fit)
+    const bool regs = a.Fg <= 64 && pcols <= 96 && prow % 32 == 0 && prow * 96 * 4 < (1ll << 31) &&
+                      (long long)F * pcols * 4 < (1ll << 31);
     for (int g = 0; g < numGroups; ++g) {
       const float* hid_g = a.hid + (size_t)g * a.Fg * prow;
       const float* flt_g = a.flt + (size_t)g * a.Fg;

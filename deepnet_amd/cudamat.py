@@ -392,8 +392,8 @@ class CUDAMatrix(object):
 
     def add_sums(self, mat, axis, mult=1.):
         """self += mult * (sums of mat along axis)."""
-        m = _cudamat.get_leading_dimension(mat.p_mat)
-        n = _cudamat.get_nonleading_dimension(mat.p_mat)
+        sz = mat.mat.size                      # (what get_leading / get_nonleading_dimension return)
+        m, n = (sz[1], sz[0]) if mat.mat.is_trans else (sz[0], sz[1])
         if axis == 0:
             left = _ones(m, trans=True)
             right = mat
