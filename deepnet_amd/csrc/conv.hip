@@ -657,6 +657,203 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
   }
 }
 
+// ------------------------------------------------------------------ convOutp, small outputs
+// Weight gradients of a layer with at most 32*RT filters per group and at most 32*CT
+// patch columns (a first layer over RGB: 64 x 75).  Both operands are contiguous along
+// the images, which is the reduction index here, so a chunk of (one module, 64 images)
+// is read row by row in whole 256-byte runs and kept in LDS as [row][image] with an odd
+// pitch: an MFMA operand (lane = row, two neighbouring images) is then one conflict-free
+// LDS read.  The four wavefronts each hold the whole RT x CT block of accumulators and
+// split the 32 steps of a chunk between them (no columns are padded to a wavefront
+// grid, one barrier per chunk); they are summed through LDS once, at the end, and every
+// workgroup writes one partial block for k_conv_outp_finish.
+template <int RT, int CT>
+__global__ void __launch_bounds__(256, 1) k_conv_outp_small(ConvArgs p) {
+  constexpr unsigned FAR = 0x80000000u;  // beyond any buffer here: sizes are below 2^31 bytes
+  constexpr int PITCH = 65;              // 64 images + 1: rows land on different banks
+  constexpr int NAV = RT * 2, NBV = CT * 2;   // 16-byte loads per lane and chunk (32 rows x 16 = 512 = 2 x 256)
+  // one LDS arena: the two operand tiles (double buffered) while chunks are multiplied,
+  // the four wavefronts' accumulators when they are summed at the end
+  constexpr int TILES = 2 * 32 * (RT + CT) * PITCH, SUMS = 4 * 16 * RT * CT * 64;
+  __shared__ float arena[TILES > SUMS ? TILES : SUMS];
+  float (*As)[32 * RT][PITCH] = reinterpret_cast<float (*)[32 * RT][PITCH]>(arena);
+  float (*Bs)[32 * CT][PITCH] = reinterpret_cast<float (*)[32 * CT][PITCH]>(arena + 2 * 32 * RT * PITCH);
+  const int tid = threadIdx.x, lane = tid & 63, li = lane & 31, lk = lane >> 5;
+  const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int g = blockIdx.z;
+  const int N = p.N, H = p.H, Fg = p.Fg, cols = p.Cg * p.kk2;
+  __amdgpu_buffer_rsrc_t r_img = __builtin_amdgcn_make_buffer_rsrc((void*)p.img, 0, (int)p.a_bytes, 0x00020000);
+  __amdgpu_buffer_rsrc_t r_hid = __builtin_amdgcn_make_buffer_rsrc((void*)p.hid, 0, (int)p.b_bytes, 0x00020000);
+  // lane's rows of the two tiles: row = tid/16 + 16*u, images 4*(tid%16) .. +3 of the chunk
+  const int r16 = tid >> 4, n4 = (tid & 15) * 4;
+  unsigned a_voff[NAV];      // hid(f, module, image) at image + N*(module + M*f)
+#pragma unroll
+  for (int u = 0; u < NAV; ++u) {
+    const int f = r16 + 16 * u;
+    a_voff[u] = f < Fg ? ((unsigned)(g * Fg + f) * (unsigned)p.M * (unsigned)N + (unsigned)n4) * 4u : FAR;
+  }
+  unsigned b_voff[NBV], b_yx[NBV];   // img(colour, y0 + ky, x0 + kx, image); bit ky | bit 16 + kx of the tap
+#pragma unroll
+  for (int u = 0; u < NBV; ++u) {
+    const unsigned q = r16 + 16 * u;
+    const unsigned c = fd_div(q, p.dkk2), r = q - c * (unsigned)p.kk2;
+    const unsigned ky = fd_div(r, p.dk), kx = r - ky * (unsigned)p.k;
+    const bool live = (int)q < cols;
+    b_voff[u] = live ? ((((unsigned)(g * p.Cg) + c) * H + ky) * H + kx) * (unsigned)N * 4u + (unsigned)n4 * 4u : FAR;
+    b_yx[u] = live ? (1u << ky) | (1u << (16 + kx)) : 0xffffffffu;
+  }
+  f32x16 acc[CT][RT];
+#pragma unroll
+  for (int j = 0; j < CT; ++j)
+#pragma unroll
+    for (int i = 0; i < RT; ++i)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[j][i][v] = 0.f;
+
+  const int halves = N >> 6;                         // chunks of 64 images per module
+  f32x4 ra[2][NAV], rb[2][NBV];   // two register sets: chunks are requested two ahead
+  typedef std::integral_constant<int, 0> Set0;
+  typedef std::integral_constant<int, 1> Set1;
+  // chunk ci of this workgroup: module m_begin + (blockIdx.x + gridDim.x * (ci / halves)), images 64 * (ci % halves)
+  auto fetch = [&](auto set_tag, int ci) __attribute__((always_inline)) {
+    constexpr int SET = decltype(set_tag)::value;
+    const int mi = blockIdx.x + gridDim.x * (ci / halves);
+    const int m = p.m_begin + mi, n0 = (ci % halves) * 64;
+    const int my = (int)fd_div((unsigned)m, p.dMx), mx = m - my * p.Mx;
+    const int y0 = my * p.s + p.pad0, x0 = mx * p.s + p.pad0;
+    const unsigned a_so = ((unsigned)m * (unsigned)N + (unsigned)n0) * 4u;
+#pragma unroll
+    for (int u = 0; u < NAV; ++u)
+      ra[SET][u] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r_hid, (int)a_voff[u], (int)a_so, 0));
+    const int ylo = y0 < 0 ? -y0 : 0, yhi = H - y0 < p.k ? H - y0 : p.k;
+    const int xlo = x0 < 0 ? -x0 : 0, xhi = H - x0 < p.k ? H - x0 : p.k;
+    const unsigned ym = yhi > ylo ? ((1u << yhi) - 1u) & ~((1u << ylo) - 1u) : 0u;
+    const unsigned xm = xhi > xlo ? ((1u << xhi) - 1u) & ~((1u << xlo) - 1u) : 0u;
+    const unsigned bad = ~(ym | (xm << 16));
+    const unsigned b_add = (unsigned)(((y0 * H + x0) * N + n0) * 4);
+#pragma unroll
+    for (int u = 0; u < NBV; ++u) {
+      const unsigned voff = (b_yx[u] & bad) ? FAR : b_voff[u] + b_add;
+      rb[SET][u] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r_img, (int)voff, 0, 0));
+    }
+  };
+  // The chunk held in LDS buffer `buf` is multiplied (steps 8*wv .. 8*wv + 7 of its 32)
+  // while register set SET, if STASH, goes to the other buffer: its LDS writes are
+  // issued between the MFMAs, and the second half of the operand reads under the
+  // first half of the MFMAs.
+  // `next`: chunk to request (into the other register set) once the first MFMAs are under
+  // way, so that its scalar address arithmetic runs beside them; -1: none.
+  auto multiply = [&](auto set_tag, auto stash_tag, int buf, int next) __attribute__((always_inline)) {
+    constexpr int SET = decltype(set_tag)::value;
+    constexpr bool STASH = decltype(stash_tag)::value;
+    constexpr int NW = 4 * (NAV + NBV);                 // LDS writes of a lane per chunk
+    constexpr int WPS = (NW + 7) / 8;                   // ... per step
+    float av[8][RT], bv[8][CT];
+    auto read = [&](int t) __attribute__((always_inline)) {
+      const int kk = 2 * (8 * wv + t) + lk;
+#pragma unroll
+      for (int i = 0; i < RT; ++i) av[t][i] = As[buf][i * 32 + li][kk];
+#pragma unroll
+      for (int j = 0; j < CT; ++j) bv[t][j] = Bs[buf][j * 32 + li][kk];
+    };
+#pragma unroll
+    for (int t = 0; t < 4; ++t) read(t);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int t = 4; t < 8; ++t) read(t);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+#pragma unroll
+      for (int j = 0; j < CT; ++j)
+#pragma unroll
+        for (int i = 0; i < RT; ++i)
+          acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[t][j], av[t][i], acc[j][i], 0, 0, 0);
+      if (t == 0 && next >= 0) fetch(std::integral_constant<int, SET ^ 1>(), next);
+      if (STASH) {
+#pragma unroll
+        for (int w = t * WPS; w < (t + 1) * WPS && w < NW; ++w) {
+          const int u = w >> 2, jj = w & 3;
+          if (u < NAV) As[buf ^ 1][r16 + 16 * u][n4 + jj] = ra[SET][u][jj];
+          else Bs[buf ^ 1][r16 + 16 * (u - NAV)][n4 + jj] = rb[SET][u - NAV][jj];
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  auto stash = [&](auto set_tag, int buf) __attribute__((always_inline)) {
+    constexpr int SET = decltype(set_tag)::value;
+#pragma unroll
+    for (int u = 0; u < NAV; ++u)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) As[buf][r16 + 16 * u][n4 + j] = ra[SET][u][j];
+#pragma unroll
+    for (int u = 0; u < NBV; ++u)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) Bs[buf][r16 + 16 * u][n4 + j] = rb[SET][u][j];
+  };
+  const int my_chunks = (int)blockIdx.x < p.m_count ? ((p.m_count - 1 - (int)blockIdx.x) / (int)gridDim.x + 1) * halves : 0;
+  // While chunk i is multiplied, chunk i+1 (asked for one trip ago) is written to LDS and
+  // chunk i+2 is requested; two chunks per trip so that the register sets swap statically.
+  typedef std::true_type Yes;
+  typedef std::false_type No;
+  int ci = 0, buf = 0;
+  if (my_chunks >= 2) {
+    fetch(Set0(), 0);
+    stash(Set0(), 0);
+    fetch(Set0(), 1);
+    __syncthreads();
+    while (ci + 4 <= my_chunks) {
+      multiply(Set0(), Yes(), buf, ci + 2);
+      __syncthreads();
+      buf ^= 1; ++ci;
+      multiply(Set1(), Yes(), buf, ci + 2);
+      __syncthreads();
+      buf ^= 1; ++ci;
+    }
+    multiply(Set0(), Yes(), buf, -1);
+    __syncthreads();
+    buf ^= 1; ++ci;                  // LDS holds chunk ci, nothing is in flight
+  } else {
+    if (my_chunks > 0) {
+      fetch(Set0(), 0);
+      stash(Set0(), 0);
+    }
+    __syncthreads();
+  }
+  for (; ci < my_chunks; ++ci) {
+    if (ci + 1 < my_chunks) {
+      fetch(Set0(), ci + 1);
+      multiply(Set0(), Yes(), buf, -1);
+    } else {
+      multiply(Set0(), No(), buf, -1);
+    }
+    __syncthreads();
+    buf ^= 1;
+  }
+  // Sum the four wavefronts' accumulators in a fixed order: every wavefront leaves its
+  // 16*RT*CT values per lane in LDS and then finishes a quarter of them.
+  constexpr int NACC = 16 * RT * CT;
+  float (*sums)[NACC][64] = reinterpret_cast<float (*)[NACC][64]>(arena);
+#pragma unroll
+  for (int j = 0; j < CT; ++j)
+#pragma unroll
+    for (int i = 0; i < RT; ++i)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) sums[wv][(j * RT + i) * 16 + v][lane] = acc[j][i][v];
+  __syncthreads();
+  // value e = (j*RT + i)*16 + v of lane (li, lk): column q = j*32 + 8*(v/4) + 4*lk + v%4, filter f = i*32 + li
+  float* part = p.partial + (size_t)blockIdx.x * ((size_t)p.G * Fg * cols) + (size_t)g * Fg * cols;
+#pragma unroll
+  for (int x = 0; x < NACC / 4; ++x) {
+    const int e = wv * (NACC / 4) + x;
+    const float sum = (sums[0][e][lane] + sums[1][e][lane]) + (sums[2][e][lane] + sums[3][e][lane]);
+    const int v = e & 15, ji = e >> 4, jt = ji / RT, it = ji - jt * RT;
+    const int q = jt * 32 + 8 * (v >> 2) + 4 * lk + (v & 3), f = it * 32 + li;
+    if (q < cols && f < Fg) part[(size_t)q * Fg + f] = sum;
+  }
+}
+
 // dW(f, q) = scale_t*dW + scale_o * sum over splits of partial[z][g][q][fl].
 // 16 outputs per workgroup; 16 lane groups take every 16th split, eight loads in flight
 // each, and meet in LDS (fixed order of additions).
@@ -1315,7 +1512,25 @@ static void conv_outp_impl(cudamat* images, cudamat* hidActs, cudamat* targets, 
   for (int ch = 0; ch < chunks; ++ch) {
     a.m_begin = ch * partialSum; a.m_count = partialSum;
     a.out = targets->data_device + (size_t)ch * cols * F;
-    if (fast) {
+    const bool small = fast && a.Fg <= 64 && cols <= 96 && N % 64 == 0 &&
+                       (long long)N * numImgColors * H * H * 4 < (1ll << 31) && (long long)N * M * F * 4 < (1ll << 31);
+    if (small) {
+      // few filters and few patch columns: every wavefront holds the whole output block
+      int nblocks = a.m_count < dn_num_cus() ? a.m_count : dn_num_cus();
+      a.splits = nblocks;
+      a.a_bytes = (unsigned)((long long)N * numImgColors * H * H * 4);
+      a.b_bytes = (unsigned)((long long)N * M * F * 4);
+      a.partial = (float*)dn_scratch((size_t)a.splits * F * cols * sizeof(float));
+      if (!a.partial) { conv_set_error(where, "out of device memory for the split-K workspace"); return; }
+      const dim3 grid((unsigned)nblocks, 1, numGroups);
+      const int rt = a.Fg <= 32 ? 1 : 2, ct = cols <= 32 ? 1 : cols <= 64 ? 2 : 3;
+#define OUTP_SMALL(RT, CT) hipLaunchKernelGGL((k_conv_outp_small<RT, CT>), grid, dim3(256), 0, 0, a)
+      if (rt == 1) { if (ct == 1) OUTP_SMALL(1, 1); else if (ct == 2) OUTP_SMALL(1, 2); else OUTP_SMALL(1, 3); }
+      else { if (ct == 1) OUTP_SMALL(2, 1); else if (ct == 2) OUTP_SMALL(2, 2); else OUTP_SMALL(2, 3); }
+#undef OUTP_SMALL
+      const int total = F * cols;
+      hipLaunchKernelGGL(k_conv_outp_finish, dim3((total + 15) / 16), dim3(256), 0, 0, a);
+    } else if (fast) {
       // rows = filters of a group: pick the tile height that wastes least.
       const int Fg = a.Fg;
       const int BMs = Fg <= 32 ? 32 : Fg <= 64 ? 64 : Fg <= 96 ? 96 : 128;
