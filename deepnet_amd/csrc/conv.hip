@@ -924,10 +924,20 @@ k_conv_patch_regs(const float* hid, const float* flt, float* P, int prow, int Fg
   // and picked up from there; rows of 32*CT + 1 floats keep both sides off bank conflicts.
   constexpr int QP = 32 * CT + 1;
   __shared__ float w_lds[2 * KS * QP];
-  for (int e = tid; e < 2 * KS * 32 * CT; e += 256) {
-    const int f = e % (2 * KS), q = e / (2 * KS);
-    const unsigned off = q < pcols && f < Fg ? ((unsigned)f + (unsigned)F * (unsigned)q) * 4u : FAR;
-    w_lds[f * QP + q] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r_flt, (int)off, 0, 0));
+  {
+    constexpr int PER_LANE = 2 * KS * 32 * CT / 256;   // all requested before the first is written
+    float w[PER_LANE];
+#pragma unroll
+    for (int it = 0; it < PER_LANE; ++it) {
+      const int e = tid + it * 256, f = e % (2 * KS), q = e / (2 * KS);
+      const unsigned off = q < pcols && f < Fg ? ((unsigned)f + (unsigned)F * (unsigned)q) * 4u : FAR;
+      w[it] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r_flt, (int)off, 0, 0));
+    }
+#pragma unroll
+    for (int it = 0; it < PER_LANE; ++it) {
+      const int e = tid + it * 256, f = e % (2 * KS), q = e / (2 * KS);
+      w_lds[f * QP + q] = w[it];
+    }
   }
   __syncthreads();
   float b[KS][CT];
