@@ -326,12 +326,42 @@ __device__ __forceinline__ void small_load(const float* __restrict__ P, unsigned
   }
 }
 
+// K-contiguous operands, whole chunks, 16-byte aligned: the 32 x 32 chunk is read the
+// way it lies in memory (8 lanes per row, 128-byte runs: 8 cache lines per instruction
+// instead of 64) and turned into the MFMA layout through a wavefront-private LDS tile.
+// r[4u + j] = op(P)(row0 + lane/8 + 8u, k0 + 4*(lane%8) + j); rows past the edge repeat the last one.
+__device__ __forceinline__ void small_load_rows(const float* __restrict__ P, unsigned ld, unsigned row0, unsigned last_row,
+                                                int k0, int lane, float (&r)[16]) {
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const unsigned row = min(row0 + (unsigned)(lane >> 3) + 8u * u, last_row);
+    const unsigned off = (row * ld + (unsigned)k0 + 4u * (lane & 7)) * 4u;
+    const float4 t = *reinterpret_cast<const float4*>(reinterpret_cast<const char*>(P) + off);
+    r[4 * u] = t.x; r[4 * u + 1] = t.y; r[4 * u + 2] = t.z; r[4 * u + 3] = t.w;
+  }
+}
+// In: r as small_load_rows left it.  Out: r[q] = chunk(row lane%32, k = 16*(lane/32) + q).
+// The pitch of 33 floats keeps both the writes (4 rows x 8 quads per half wavefront) and
+// the reads (32 rows, one column) on 32 different banks.  Only this wavefront touches `tile`.
+__device__ __forceinline__ void small_restage(float (*tile)[33], int lane, float (&r)[16]) {
+#pragma unroll
+  for (int u = 0; u < 4; ++u)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) tile[(lane >> 3) + 8 * u][4 * (lane & 7) + j] = r[4 * u + j];
+  __builtin_amdgcn_wave_barrier();
+#pragma unroll
+  for (int q = 0; q < 16; ++q) r[q] = tile[lane & 31][16 * (lane >> 5) + q];
+  __builtin_amdgcn_wave_barrier();
+}
+
 template <bool A_KC, bool B_KC, int NW>
 __global__ void __launch_bounds__(NW * 64)
 k_gemm_small(const float* __restrict__ A, int lda, const float* __restrict__ B, int ldb, float* C, int ldc, int M, int N,
              int K, float alpha, float beta, bool a_vec, bool b_vec, GemmEpilogue epi) {
   constexpr int RED = NW / 2 > 4 ? NW / 2 : 4;
   __shared__ float red[RED][16 * 64];
+  constexpr int NSTAGE = (A_KC ? 1 : 0) + (B_KC ? 1 : 0);
+  __shared__ float stage[NW][NSTAGE > 0 ? NSTAGE : 1][32][33];  // wavefront-private restaging tiles
   const int tid = threadIdx.x, lane = tid & 63;
   const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);   // tell the compiler it is wave-uniform
   const int li = lane & 31, lk = lane >> 5;
@@ -358,20 +388,31 @@ k_gemm_small(const float* __restrict__ A, int lda, const float* __restrict__ B, 
   constexpr int STEP = 32 * NW;
   float a[DEPTH][16], b[DEPTH][16];
   int k0 = wv * 32;
+  // (a chunk takes the row-wise path when it is K-contiguous, aligned and whole)
+  auto load_a = [&](int kc, float (&r)[16]) __attribute__((always_inline)) {
+    if (A_KC && a_vec && kc + 32 <= K) small_load_rows(A, lda, blockIdx.x * 32, M - 1, kc, lane, r);
+    else small_load<A_KC>(A, lda, mc, kc, lk, K, a_vec, r);
+  };
+  auto load_b = [&](int kc, float (&r)[16]) __attribute__((always_inline)) {
+    if (B_KC && b_vec && kc + 32 <= K) small_load_rows(B, ldb, blockIdx.y * 32, N - 1, kc, lane, r);
+    else small_load<B_KC>(B, ldb, nc, kc, lk, K, b_vec, r);
+  };
 #pragma unroll
   for (int d = 0; d < DEPTH; ++d) {
-    small_load<A_KC>(A, lda, mc, k0 + d * STEP, lk, K, a_vec, a[d]);
-    small_load<B_KC>(B, ldb, nc, k0 + d * STEP, lk, K, b_vec, b[d]);
+    load_a(k0 + d * STEP, a[d]);
+    load_b(k0 + d * STEP, b[d]);
   }
   for (; k0 < K; k0 += DEPTH * STEP) {
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
       if (k0 + d * STEP < K) {                               // wave-uniform
+        if (A_KC && a_vec && k0 + d * STEP + 32 <= K) small_restage(stage[wv][0], lane, a[d]);
+        if (B_KC && b_vec && k0 + d * STEP + 32 <= K) small_restage(stage[wv][NSTAGE - 1], lane, b[d]);
 #pragma unroll
         for (int q = 0; q < 16; ++q) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(b[d][q], a[d][q], acc, 0, 0, 0);
         if (k0 + (d + DEPTH) * STEP < K) {                   // refill the set with the chunk DEPTH further on
-          small_load<A_KC>(A, lda, mc, k0 + (d + DEPTH) * STEP, lk, K, a_vec, a[d]);
-          small_load<B_KC>(B, ldb, nc, k0 + (d + DEPTH) * STEP, lk, K, b_vec, b[d]);
+          load_a(k0 + (d + DEPTH) * STEP, a[d]);
+          load_b(k0 + (d + DEPTH) * STEP, b[d]);
         }
       }
     }
