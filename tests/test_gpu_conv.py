@@ -239,3 +239,31 @@ def _random_conv_cases(seed, count):
 @pytest.mark.parametrize("N,C,H,F,k,s,p,G", _random_conv_cases(20240607, 24))
 def test_three_conv_passes_on_random_geometries(cm, cc, rng, N, C, H, F, k, s, p, G):
     test_three_conv_passes(cm, cc, rng, N, C, H, F, k, s, p, G)
+
+
+def _random_small_layer_cases(seed, count):
+    """Seeded first-layer-like geometries (few colours, few filters, short reductions) for
+    the register-resident convUp / patch-product convDown kernels and the small-output
+    convOutp kernel: batches of 32..160 (one to five image blocks per module; 64-image
+    chunks with and without a remainder), reductions up to and beyond the 80 / 96 term
+    limits, filter groups that are not a multiple of 32, every stride and padding."""
+    r = np.random.default_rng(seed)
+    out = []
+    while len(out) < count:
+        N = int(r.choice([32, 64, 96, 128, 160]))
+        G = int(r.choice([1, 1, 2]))
+        Cg = int(r.choice([1, 2, 3, 4, 5]))
+        Fg = int(r.choice([16, 32, 48, 64]))
+        k = int(r.integers(2, 7))
+        s = int(r.integers(1, k + 1))
+        p = int(r.integers(0, k))
+        H = int(r.integers(k, 15))
+        if co.n_modules(H, k, s, p) < 1 or Cg * k * k > 110:
+            continue
+        out.append((N, Cg * G, H, Fg * G, k, s, p, G))
+    return out
+
+
+@pytest.mark.parametrize("N,C,H,F,k,s,p,G", _random_small_layer_cases(20240611, 30))
+def test_three_conv_passes_on_random_small_layers(cm, cc, rng, N, C, H, F, k, s, p, G):
+    test_three_conv_passes(cm, cc, rng, N, C, H, F, k, s, p, G)
