@@ -241,3 +241,29 @@ def test_fused_training_steps_of_the_bench_match_the_reference_sequences(cm):
         for a, b in zip(plain, fused):
             assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
     cm.CUDAMatrix.init_random(1)
+
+
+def _random_small_products(seed, count):
+    r = np.random.default_rng(seed)
+    out = []
+    for _ in range(count):
+        m, n = int(r.integers(1, 300)), int(r.integers(1, 300))
+        k = int(r.choice([int(r.integers(1, 40)), int(r.integers(40, 1100)), 4 * int(r.integers(8, 260))]))
+        out.append((m, k, n, bool(r.integers(0, 2)), bool(r.integers(0, 2)), float(r.choice([0.0, 1.0, -0.5]))))
+    return out
+
+
+@pytest.mark.parametrize("m,k,n,ta,tb,beta", _random_small_products(20240612, 40))
+def test_small_products_on_random_shapes(cm, rng, m, k, n, ta, tb, beta):
+    # the one-launch kernel for products that cannot fill the chip: ragged tiles, ragged and
+    # whole chunks of the reduction, leading dimensions that are and are not multiples of 4
+    A, B, C = _rand(rng, (m, k)), _rand(rng, (k, n)), _rand(rng, (m, n))
+    a = cm.CUDAMatrix(np.asfortranarray(A.T)) if ta else cm.CUDAMatrix(A)
+    b = cm.CUDAMatrix(np.asfortranarray(B.T)) if tb else cm.CUDAMatrix(B)
+    c = cm.CUDAMatrix(C) if beta != 0.0 else cm.CUDAMatrix(np.full((m, n), np.nan, dtype=np.float32))
+    cm._check(cm._cudamat.dot((a.T if ta else a).p_mat, (b.T if tb else b).p_mat, c.p_mat, beta, 1.5))
+    want = 1.5 * (A.astype(np.float64) @ B.astype(np.float64)) + (beta * C.astype(np.float64) if beta != 0.0 else 0.0)
+    bound = 1.5 * (np.abs(A).astype(np.float64) @ np.abs(B)) + abs(beta) * np.abs(C) + 1e-30
+    assert np.max(np.abs(c.asarray() - want) / bound) < REL
+    for h in (a, b, c):
+        h.free_device_memory()
