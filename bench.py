@@ -245,7 +245,13 @@ def gemm_probe(cm, ev, n=4096, iters=10):
     c = cm.empty((n, n))
     out = {}
     for label, x, y in (('nn', a, b), ('tn', a.T, b), ('nt', a, b.T)):
-        cm.dot(x, y, target=c)
+        # untimed warm-up: the core clock under matrix-core load needs a few tens of ms to
+        # settle (the first variant timed cold reads 10 % low)
+        t0 = time.perf_counter()
+        while (time.perf_counter() - t0) < 0.03:
+            for _ in range(4):
+                cm.dot(x, y, target=c)
+            cm.cuda_sync_threads()
         e0, e1 = ev.new(), ev.new()
         ev.record(e0)
         for _ in range(iters):

@@ -17,8 +17,18 @@ LAYERS = {
 }
 
 
-def _time(ev, fn, iters):
+WARM_MS = 30.0   # the core clock under matrix-core load needs a few tens of ms to settle
+
+
+def _time(ev, fn, iters, sync):
+    import time
     fn()
+    sync()
+    t0 = time.perf_counter()
+    while (time.perf_counter() - t0) * 1e3 < WARM_MS:
+        for _ in range(5):
+            fn()
+        sync()
     e0, e1 = ev.new(), ev.new()
     ev.record(e0)
     for _ in range(iters):
@@ -44,7 +54,7 @@ def run(cm, ev, iters=10):
         for label, fn in (('convUp', lambda: cc.convUp(X, W, up, Mx, p, s, C, G)),
                           ('convDown', lambda: cc.convDown(Y, W, down, Mx, p, s, k, H, C, numGroups=G)),
                           ('convOutp', lambda: cc.convOutp(X, Y, dw, Mx, p, k, s, C, numGroups=G))):
-            ms = _time(ev, fn, iters)
+            ms = _time(ev, fn, iters, cm.cuda_sync_threads)
             tf = flops / (ms * 1e-3) / 1e12
             res[label] = {'ms': round(ms, 4), 'tflops': round(tf, 2),
                           'frac_mfma_fp32': round(tf / MFMA_FP32_PEAK_TFLOPS, 4)}
@@ -62,7 +72,7 @@ def run(cm, ev, iters=10):
                     ('ResponseNormUndo', lambda: (acts.assign(normed),
                                                   cc.ResponseNormUndo(grad, den, pooled, acts, nundo, F, 5, 0.001, 0.75)),
                      (2 + 7) * e_out)):
-                ms = _time(ev, fn, iters)
+                ms = _time(ev, fn, iters, cm.cuda_sync_threads)
                 gbs = nbytes / (ms * 1e-3) / 1e9
                 res[label] = {'us': round(ms * 1e3, 2), 'gbs': round(gbs, 1), 'frac_hbm': round(gbs / HBM_PEAK_GBS, 4)}
         out[name] = res
