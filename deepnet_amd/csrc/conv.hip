@@ -166,7 +166,7 @@ __device__ __forceinline__ void down_axis(int ph, int s, int pad0, int H, int k,
 // kernel, slab offset in an SGPR, an out-of-range offset for a tap in the padding, which
 // the hardware answers with zeros -- and cost no vector instructions, which matters
 // because fp32 MFMA and the vector ALU share lanes.  Both operands run two slabs ahead.
-template <int MODE, int WAVES_M, int WM, int WN, bool UNI = false>
+template <int MODE, int WAVES_M, int WM, int WN, bool UNI = false, int N16 = 0>
 __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
   constexpr int WAVES_N = 4 / WAVES_M;
   constexpr int BM = 32 * WM * WAVES_M, BN = 32 * WN * WAVES_N;
@@ -533,11 +533,45 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
     for (int i = 0; i < WM; ++i)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[j][i][v] = 0.f;
+  // N16 > 0: the columns are covered by N16 blocks of 16 with v_mfma_f32_16x16x4_f32
+  // (merged-phase convDown, whose column count is colours x stride^2: 48 columns cost
+  // three blocks of 16 instead of two of 32).  A wavefront's 32 rows are two blocks of 16.
+  static_assert(N16 == 0 || (MODE == CONV_DOWNM && WM == 1 && WAVES_M == 4 && N16 * 16 <= BN), "16-wide blocks: merged-phase convDown only");
+  constexpr int N16A = N16 > 0 ? N16 : 1;
+  f32x4 acc16[N16A][2];
+#pragma unroll
+  for (int j = 0; j < N16A; ++j)
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) acc16[j][i][v] = 0.f;
+  const int l16 = lane & 15, k16 = lane >> 4;
 
   // One slab: all of its fragments are asked of LDS first (the scheduling fences keep
   // the compiler from sinking the reads back to their uses and from hoisting the wait
   // for the gathers in flight above the MFMAs).
   auto multiply = [&](int buf) {
+    if constexpr (N16 > 0) {
+      // lane (l16, k16): operand element (row or column l16 of its block, k = 4*step + k16)
+      float av[CV_BK / 4][2], bv[CV_BK / 4][N16A];
+#pragma unroll
+      for (int kk = 0; kk < CV_BK / 4; ++kk) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) av[kk][i] = As[buf][4 * kk + k16][wm * 32 + i * 16 + l16];
+#pragma unroll
+        for (int j = 0; j < N16A; ++j) bv[kk][j] = Bs[buf][4 * kk + k16][j * 16 + l16];
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int kk = 0; kk < CV_BK / 4; ++kk)
+#pragma unroll
+        for (int j = 0; j < N16A; ++j)
+#pragma unroll
+          for (int i = 0; i < 2; ++i)
+            acc16[j][i] = __builtin_amdgcn_mfma_f32_16x16x4f32(bv[kk][j], av[kk][i], acc16[j][i], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      return;
+    }
     float av[CV_BK / 2][WM], bv[CV_BK / 2][WN];
 #pragma unroll
     for (int kk = 0; kk < CV_BK / 2; ++kk) {
@@ -601,6 +635,32 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
     buf ^= 1;
   }
 
+  if constexpr (N16 > 0) {
+    // acc16[j][i][v] is C(row, col) with row = ... + i*16 + l16, col = j*16 + 4*k16 + v
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int r = row0 + wm * 32 + i * 16 + l16;
+      if (r >= rows) continue;
+      const int pos = (int)fd_div((uint32_t)r, p.dN);
+      const int n = r - pos * N;
+      const int Y = pos / p.yq, X = pos - Y * p.yq;
+#pragma unroll
+      for (int j = 0; j < N16A; ++j)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          const int cc = col0 + j * 16 + 4 * k16 + v;
+          if (cc >= cols) continue;
+          const int c = (int)fd_div((uint32_t)cc, p.dSS), q = cc - c * s * s;
+          const int py = (int)fd_div((uint32_t)q, p.dS), px = q - py * s;
+          const int y = Y * s + py + p.pad0, x = X * s + px + p.pad0;
+          if ((unsigned)y < (unsigned)H && (unsigned)x < (unsigned)H) {
+            float* t = p.out + (long long)N * ((long long)(g * Cg + c) * HH + y * H + x) + n;
+            *t = (p.scale_t == 0.f ? 0.f : p.scale_t * *t) + p.scale_o * acc16[j][i][v];
+          }
+        }
+    }
+    return;
+  }
   // ---- epilogue: acc[j][i][v] is C(row, col) with row = ... + li, col = ... + 8*(v/4) + 4*lk + v%4
 #pragma unroll
   for (int i = 0; i < WM; ++i) {
@@ -1443,7 +1503,10 @@ static void conv_down_impl(cudamat* hidActs, cudamat* filters, cudamat* targets,
     a.yq = (imgSize - 1 + padw) / moduleStride + 1;
     const int cols = a.Cg * moduleStride * moduleStride;
     const unsigned gx = (unsigned)((long long)a.yq * a.yq * N / 128);
-    if (cols <= 32) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 1, true>), dim3(gx, 1, numGroups), dim3(256), 0, 0, a);
+    // column counts that leave a 32-wide block half empty take 16-wide blocks
+    if (cols <= 16) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 1, true, 1>), dim3(gx, 1, numGroups), dim3(256), 0, 0, a);
+    else if (cols <= 32) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 1, true>), dim3(gx, 1, numGroups), dim3(256), 0, 0, a);
+    else if (cols <= 48) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 2, true, 3>), dim3(gx, 1, numGroups), dim3(256), 0, 0, a);
     else if (cols <= 64) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 2, true>), dim3(gx, 1, numGroups), dim3(256), 0, 0, a);
     else if (cols <= 96) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 3, true>), dim3(gx, 1, numGroups), dim3(256), 0, 0, a);
     else hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 2, 2, 2, true>), dim3(gx, (cols + 127) / 128, numGroups), dim3(256), 0, 0, a);
