@@ -534,9 +534,10 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[j][i][v] = 0.f;
   // N16 > 0: the columns are covered by N16 blocks of 16 with v_mfma_f32_16x16x4_f32
-  // (merged-phase convDown, whose column count is colours x stride^2: 48 columns cost
-  // three blocks of 16 instead of two of 32).  A wavefront's 32 rows are two blocks of 16.
-  static_assert(N16 == 0 || (MODE == CONV_DOWNM && WM == 1 && WAVES_M == 4 && N16 * 16 <= BN), "16-wide blocks: merged-phase convDown only");
+  // (48 columns, e.g. colours x stride^2 of a merged-phase convDown or 48 colours per
+  // group, cost three blocks of 16 instead of two of 32).  A wavefront's 32 rows are two
+  // blocks of 16.
+  static_assert(N16 == 0 || (MODE != CONV_OUTP && WM == 1 && WAVES_M == 4 && N16 * 16 <= BN), "16-wide blocks: 128-row Up / Down tiles");
   constexpr int N16A = N16 > 0 ? N16 : 1;
   f32x4 acc16[N16A][2];
 #pragma unroll
@@ -643,21 +644,43 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
       if (r >= rows) continue;
       const int pos = (int)fd_div((uint32_t)r, p.dN);
       const int n = r - pos * N;
-      const int Y = pos / p.yq, X = pos - Y * p.yq;
+      if constexpr (MODE == CONV_DOWNM) {
+        const int Y = pos / p.yq, X = pos - Y * p.yq;
 #pragma unroll
-      for (int j = 0; j < N16A; ++j)
+        for (int j = 0; j < N16A; ++j)
 #pragma unroll
-        for (int v = 0; v < 4; ++v) {
-          const int cc = col0 + j * 16 + 4 * k16 + v;
-          if (cc >= cols) continue;
-          const int c = (int)fd_div((uint32_t)cc, p.dSS), q = cc - c * s * s;
-          const int py = (int)fd_div((uint32_t)q, p.dS), px = q - py * s;
-          const int y = Y * s + py + p.pad0, x = X * s + px + p.pad0;
-          if ((unsigned)y < (unsigned)H && (unsigned)x < (unsigned)H) {
-            float* t = p.out + (long long)N * ((long long)(g * Cg + c) * HH + y * H + x) + n;
+          for (int v = 0; v < 4; ++v) {
+            const int cc = col0 + j * 16 + 4 * k16 + v;
+            if (cc >= cols) continue;
+            const int c = (int)fd_div((uint32_t)cc, p.dSS), q = cc - c * s * s;
+            const int py = (int)fd_div((uint32_t)q, p.dS), px = q - py * s;
+            const int y = Y * s + py + p.pad0, x = X * s + px + p.pad0;
+            if ((unsigned)y < (unsigned)H && (unsigned)x < (unsigned)H) {
+              float* t = p.out + (long long)N * ((long long)(g * Cg + c) * HH + y * H + x) + n;
+              *t = (p.scale_t == 0.f ? 0.f : p.scale_t * *t) + p.scale_o * acc16[j][i][v];
+            }
+          }
+      } else {
+        long long rbase, cstride;
+        if (MODE == CONV_UP) {
+          rbase = (long long)g * Fg * M * N + r;
+          cstride = (long long)M * N;
+        } else {
+          const int qyi = pos / ph.QX, qxi = pos - qyi * ph.QX;
+          const int y = ph.y_first + s * qyi, x = ph.x_first + s * qxi;
+          rbase = (long long)N * ((long long)g * Cg * HH + y * H + x) + n;
+          cstride = (long long)N * HH;
+        }
+#pragma unroll
+        for (int j = 0; j < N16A; ++j)
+#pragma unroll
+          for (int v = 0; v < 4; ++v) {
+            const int c = col0 + j * 16 + 4 * k16 + v;
+            if (c >= cols) continue;
+            float* t = p.out + rbase + cstride * c;
             *t = (p.scale_t == 0.f ? 0.f : p.scale_t * *t) + p.scale_o * acc16[j][i][v];
           }
-        }
+      }
     }
     return;
   }
@@ -1397,7 +1420,10 @@ static void launch_rowmajor(const ConvArgs& a, long long rows, int cols, int gz)
   const int nslabs = MODE == CONV_UP ? (a.Cg * a.kk2 + CV_BK - 1) / CV_BK : a.kk2 * (a.Fg / CV_BK) / (a.s * a.s);
   if (a.N % 128 == 0 && a.a_bytes != 0 && a.b_bytes != 0 && nslabs >= 16 && (cols <= 64 || cols > 96)) {
     const unsigned gx = (unsigned)(rows / 128);
-    if (cols <= 32) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 1, true>), dim3(gx, (cols + 31) / 32, gz), dim3(256), 0, 0, a);
+    // (column counts that leave a 32-wide block half empty take 16-wide blocks)
+    if (cols <= 16) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 1, true, 1>), dim3(gx, 1, gz), dim3(256), 0, 0, a);
+    else if (cols <= 32) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 1, true>), dim3(gx, (cols + 31) / 32, gz), dim3(256), 0, 0, a);
+    else if (cols <= 48) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 2, true, 3>), dim3(gx, 1, gz), dim3(256), 0, 0, a);
     else if (cols <= 64) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 2, true>), dim3(gx, (cols + 63) / 64, gz), dim3(256), 0, 0, a);
     else hipLaunchKernelGGL((k_conv_mfma<MODE, 2, 2, 2, true>), dim3(gx, (cols + 127) / 128, gz), dim3(256), 0, 0, a);
     return;

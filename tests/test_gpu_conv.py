@@ -37,6 +37,9 @@ CASES = [  # N, C, H, F, k, stride, padding, groups
     (96, 1, 11, 64, 5, 2, 1, 1),     # the same: 3 image blocks per module, 25 taps, stride 2
     (32, 5, 6, 16, 4, 1, 3, 1),      # the same: exactly 80 taps, padding 3 (every module touches the padding)
     (32, 2, 9, 128, 3, 1, 1, 2),     # the same: 2 groups of 64 filters
+    (128, 48, 7, 32, 5, 1, 2, 1),    # uniform-row kernels with 16-wide column blocks: convDown onto 48 colours
+    (128, 16, 8, 48, 5, 1, 2, 1),    # the same: convUp onto 48 filters, convDown onto 16 colours (one block of 16)
+    (128, 96, 6, 64, 5, 1, 2, 2),    # the same in 2 groups of 48 colours / 32 filters (the shape of config 5b)
 ]
 
 
