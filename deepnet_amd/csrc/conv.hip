@@ -23,6 +23,14 @@
 // The matrix-core path needs numImages % 16 == 0, filters-per-group % 16 == 0 and
 // 16-byte aligned buffers; anything else takes the one-thread-per-output kernels
 // below, which are also the cross-check of the fast path in the tests.
+//
+// First-layer shapes (few colours, few filters) have their own kernels further down,
+// because a 16-deep, 128-column LDS pipeline is mostly prologue and padding for them:
+//   k_conv_up_regs     convUp with colours*k*k <= 80: filter bank in registers
+//   k_conv_patch_regs  convDown, stride 1, <= 16 colours: P = hid * W in registers,
+//                      then k_conv_down_gather(_s1) sums the entries that land on a pixel
+//   k_conv_outp_small  convOutp with <= 64 x 96 outputs: [row][image] LDS tiles, every
+//                      wavefront holds the whole output block
 #include "common.h"
 #include <type_traits>
 #include "../../include/cudamat_conv_amd.h"
