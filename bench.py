@@ -238,7 +238,7 @@ def time_loop(cm, fn, iters, warmup):
     return (time.perf_counter() - t0) / iters
 
 
-def gemm_probe(cm, ev, n=4096, iters=10):
+def gemm_probe(cm, ev, n=4096, iters=10, warm_s=0.03):
     rng = np.random.default_rng(6)
     a = cm.CUDAMatrix(np.asarray(rng.uniform(-1, 1, (n, n)), dtype=np.float32, order='F'))
     b = cm.CUDAMatrix(np.asarray(rng.uniform(-1, 1, (n, n)), dtype=np.float32, order='F'))
@@ -248,7 +248,7 @@ def gemm_probe(cm, ev, n=4096, iters=10):
         # untimed warm-up: the core clock under matrix-core load needs a few tens of ms to
         # settle (the first variant timed cold reads 10 % low)
         t0 = time.perf_counter()
-        while (time.perf_counter() - t0) < 0.03:
+        while (time.perf_counter() - t0) < warm_s:
             for _ in range(4):
                 cm.dot(x, y, target=c)
             cm.cuda_sync_threads()
@@ -364,6 +364,8 @@ def main():
     ap.add_argument('--warmup', type=int, default=2)
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
     ap.add_argument('--only-c2', action='store_true', help='skip the secondary workloads')
+    ap.add_argument('--probe-mfma', action='store_true',
+                    help='launch only the 4096^3 products and the conv layers a few times (for rocprofv3 --pmc runs)')
     ap.add_argument('--probe', action='store_true',
                     help='run only the roofline kernel (add_mult) and a copy-shaped calibration kernel '
                          '(mult by a scalar into a second matrix), for rocprofv3 --pmc runs')
@@ -375,6 +377,15 @@ def main():
     cm.cublas_init()
     cm.CUDAMatrix.init_random(2)
     ev = HipEvents()
+
+    if args.probe_mfma:
+        # the matrix-core kernels only, a few launches each and no clock warm-up: for counter runs
+        import bench_conv
+        bench_conv.WARM_MS = 0.0
+        out = {'gemm_fp32_4096': gemm_probe(cm, ev, iters=3, warm_s=0.0)}
+        out.update(bench_conv.run(cm, ev, iters=3))
+        print(json.dumps({'probe_mfma': out}))
+        return
 
     if args.probe:
         sets = build_c2(cm)

@@ -180,7 +180,8 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
   constexpr int BM = 32 * WM * WAVES_M, BN = 32 * WN * WAVES_N;
   // Row pitch in LDS: operands written transposed one float per lane want pitch % 8 == 2
   // (no bank conflicts), those written 16 bytes at a time need pitch % 4 == 0.
-  constexpr int LA = BM + (MODE == CONV_OUTP ? 2 : CV_PAD), LB = BN + (MODE == CONV_UP ? CV_PAD : 2);
+  // (16-wide blocks read k rows 4 apart per lane group: both pitches are then 4 mod 8, rows 16 banks apart)
+  constexpr int LA = BM + (MODE == CONV_OUTP ? 2 : CV_PAD), LB = BN + (MODE == CONV_UP || N16 > 0 ? CV_PAD : 2);
   constexpr int TA = BM * CV_BK / 4, TB = BN * CV_BK / 4;  // 16-byte groups per slab
   constexpr int NA = (TA + 255) / 256, NB = (TB + 255) / 256;
   __shared__ __attribute__((aligned(16))) float As[2][CV_BK][LA];
@@ -561,14 +562,16 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
   // for the gathers in flight above the MFMAs).
   auto multiply = [&](int buf) {
     if constexpr (N16 > 0) {
-      // lane (l16, k16): operand element (row or column l16 of its block, k = 4*step + k16)
+      // lane (l16, k16): operand element (row or column l16 of its block, k = step + 4*k16:
+      // any assignment of the slab's 16 k to (step, k16) will do as long as both operands
+      // use the same one, and rows 4 apart sit 16 banks apart)
       float av[CV_BK / 4][2], bv[CV_BK / 4][N16A];
 #pragma unroll
       for (int kk = 0; kk < CV_BK / 4; ++kk) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) av[kk][i] = As[buf][4 * kk + k16][wm * 32 + i * 16 + l16];
+        for (int i = 0; i < 2; ++i) av[kk][i] = As[buf][kk + 4 * k16][wm * 32 + i * 16 + l16];
 #pragma unroll
-        for (int j = 0; j < N16A; ++j) bv[kk][j] = Bs[buf][4 * kk + k16][j * 16 + l16];
+        for (int j = 0; j < N16A; ++j) bv[kk][j] = Bs[buf][kk + 4 * k16][j * 16 + l16];
       }
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
