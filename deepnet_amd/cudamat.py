@@ -72,9 +72,12 @@ class cudamat_sparse(ct.Structure):
                 ('nnz', ct.c_int)]
 
 
-_M = ct.POINTER(cudamat)
-_S = ct.POINTER(cudamat_sparse)
-_R = ct.POINTER(rnd_struct)
+# Handles are declared as void*: ctypes converts a pointer object (CUDAMatrix.p_mat) to a
+# void* argument markedly faster than it type-checks a POINTER(cudamat) one, and the steps
+# of small models are bound by exactly this per-call host cost.
+_M = ct.c_void_p
+_S = ct.c_void_p
+_R = ct.c_void_p
 _f, _i, _u = ct.c_float, ct.c_int, ct.c_uint
 
 # name -> (restype, argtypes): the prototypes of include/cudamat_amd.h.

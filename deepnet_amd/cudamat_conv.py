@@ -22,7 +22,7 @@ if not os.path.exists(_LIB_PATH):
                       % (_LIB_PATH, os.path.join(_HERE, 'csrc')))
 _ConvNet = ct.CDLL(_LIB_PATH)
 
-_M = ct.POINTER(cudamat)
+_M = ct.c_void_p   # (see cudamat.py: void* handles convert faster than typed pointers)
 _i, _f = ct.c_int, ct.c_float
 _SIGNATURES = {
     'convUp': [_M, _M, _M, _i, _i, _i, _i, _i],

@@ -67,8 +67,8 @@ def test_host_side_argument_errors_need_no_device():
     assert lib.max_by_axis(a.p_mat, b.p_mat, 0) == -8
     assert lib.copy_to_host(a.p_mat) == -8
     assert lib.fill_with_rand(None, a.p_mat) == -8
-    assert lib.get_slice(a.p_mat, cm.cudamat(), 0, 1) == -8
-    assert lib.get_slice(a.T.p_mat, cm.cudamat(), 0, 1) == -5        # transposed first (cudamat.cu:332-336)
+    assert lib.get_slice(a.p_mat, ct.byref(cm.cudamat()), 0, 1) == -8
+    assert lib.get_slice(a.T.p_mat, ct.byref(cm.cudamat()), 0, 1) == -5        # transposed first (cudamat.cu:332-336)
     assert lib.sample_bernoulli(None, a.p_mat, cm.CUDAMatrix(np.zeros((2, 2), np.float32), False).p_mat) == -1
     with pytest.raises(cm.CUDAMatException, match="not in device memory"):
         a.add(b)

@@ -1,5 +1,7 @@
 """GPU tests of handles, transfers, views, row slices, transpose and the column
 gather / scatter ops (modelled on cudamat/test_cudamat.py:12-290, 596-794)."""
+import ctypes as ct
+
 import numpy as np
 import pytest
 
@@ -72,7 +74,7 @@ def test_column_slices_alias_the_parent(cm, rng):
     with pytest.raises(cm.CUDAMatException):
         a.slice(5, 21)
     with pytest.raises(cm.CUDAMatException, match="transposed"):
-        cm._check(cm._cudamat.get_slice(a.T.p_mat, cm.cudamat(), 0, 1))
+        cm._check(cm._cudamat.get_slice(a.T.p_mat, ct.byref(cm.cudamat()), 0, 1))
     row = cm.CUDAMatrix(_rand(rng, (1, 30)))
     assert np.array_equal(row.slice(4, 9).asarray(), row.asarray()[:, 4:9])
 
