@@ -1483,7 +1483,8 @@ static void conv_up_impl(cudamat* images, cudamat* filters, cudamat* targets, in
   a.local = local ? 1 : 0;
   set_buffer_ranges(a, (long long)N * numImgColors * H * H, (long long)F * filters->size[1]);
   const int K = a.Cg * a.kk2;
-  if (!local && fast_ok(a) && K <= 80 && a.Fg <= 64 && N % 32 == 0 && a.a_bytes != 0 && a.b_bytes != 0) {
+  if (!local && fast_ok(a) && K <= 80 && a.Fg <= 64 && N % 32 == 0 && a.a_bytes != 0 && a.b_bytes != 0 &&
+      (long long)N * M * F * 4 < (1ll << 31)) {  // (32-bit offsets into the output, and an out-of-range offset beyond it)
     // short reduction, few filters per group: filter bank in registers
     const long long tiles = (long long)M * (N / 32);
     long long blocks = (tiles + 3) / 4;
