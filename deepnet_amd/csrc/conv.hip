@@ -174,8 +174,12 @@ __device__ __forceinline__ void down_axis(int ph, int s, int pad0, int H, int k,
 // kernel, slab offset in an SGPR, an out-of-range offset for a tap in the padding, which
 // the hardware answers with zeros -- and cost no vector instructions, which matters
 // because fp32 MFMA and the vector ALU share lanes.  Both operands run two slabs ahead.
-template <int MODE, int WAVES_M, int WM, int WN, bool UNI = false, int N16 = 0>
+// INSIDE (general convUp gather only): no padding, the last module ends inside the image
+// and the rows fill their tiles, so no image group is ever masked: its gather is an add
+// and a load (a tap beyond the reduction re-reads the last one against a zero filter row).
+template <int MODE, int WAVES_M, int WM, int WN, bool UNI = false, int N16 = 0, bool INSIDE = false>
 __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
+  static_assert(!INSIDE || (MODE == CONV_UP && !UNI), "INSIDE: the general convUp gather");
   constexpr int WAVES_N = 4 / WAVES_M;
   constexpr int BM = 32 * WM * WAVES_M, BN = 32 * WN * WAVES_N;
   // Row pitch in LDS: operands written transposed one float per lane want pitch % 8 == 2
@@ -452,18 +456,23 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
         bool sv[2];
 #pragma unroll
         for (int h = 0; h < (A_TWO ? 2 : 1); ++h) {
-          const int kk = kk0 + a_ks[u] + h;
+          int kk = kk0 + a_ks[u] + h;
+          sv[h] = kk < Kup;
+          if (INSIDE && !sv[h]) kk = Kup - 1;
           const int c = (int)fd_div((uint32_t)kk, p.dkk2);
           const int pp = kk - c * p.kk2;
           sy[h] = (int)fd_div((uint32_t)pp, p.dk); sx[h] = pp - sy[h] * k;
-          sv[h] = kk < Kup;
           so[h] = 4u * (unsigned)N * (unsigned)((g * Cg + c) * HH + sy[h] * H + sx[h]);   // unused when !sv[h]
         }
         const bool hi = A_TWO && lk;
-        const int y = a_y[u] + (hi ? sy[1] : sy[0]), x = a_x[u] + (hi ? sx[1] : sx[0]);
-        ok = ok & (hi ? sv[1] : sv[0]) & ((unsigned)y < (unsigned)H) & ((unsigned)x < (unsigned)H);
-        const unsigned voff = ok ? a_voff[u] + (hi ? so[1] : so[0]) : 4u * img_bias;
-        ra[SET][u] = *reinterpret_cast<const f32x4*>(a_base + voff);
+        if constexpr (INSIDE) {
+          ra[SET][u] = *reinterpret_cast<const f32x4*>(a_base + (a_voff[u] + (hi ? so[1] : so[0])));
+        } else {
+          const int y = a_y[u] + (hi ? sy[1] : sy[0]), x = a_x[u] + (hi ? sx[1] : sx[0]);
+          ok = ok & (hi ? sv[1] : sv[0]) & ((unsigned)y < (unsigned)H) & ((unsigned)x < (unsigned)H);
+          const unsigned voff = ok ? a_voff[u] + (hi ? so[1] : so[0]) : 4u * img_bias;
+          ra[SET][u] = *reinterpret_cast<const f32x4*>(a_base + voff);
+        }
       } else if (MODE == CONV_DOWN) {
         const int my = a_y[u] - st_a, mx = a_x[u] - st_b;
         ok = ok & ((unsigned)my < (unsigned)Mx) & ((unsigned)mx < (unsigned)Mx);
@@ -514,7 +523,7 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
 #pragma unroll
     for (int u = 0; u < NA; ++u) {
       if (tid + u * 256 >= TA) continue;
-      if (!UNI && !ra_ok[SET][u]) ra[SET][u] = zero4;
+      if (!UNI && !INSIDE && !ra_ok[SET][u]) ra[SET][u] = zero4;
       if (MODE == CONV_OUTP) {
         As[buf][a_k[u]][a_r[u]] = ra[SET][u].x; As[buf][a_k[u] + 1][a_r[u]] = ra[SET][u].y;
         As[buf][a_k[u] + 2][a_r[u]] = ra[SET][u].z; As[buf][a_k[u] + 3][a_r[u]] = ra[SET][u].w;
@@ -1445,6 +1454,14 @@ static void launch_rowmajor(const ConvArgs& a, long long rows, int cols, int gz)
   const long long tiles256 = (rows + 255) / 256 * ((cols + 127) / 128) * gz;
   if (tiles256 >= 2 * dn_num_cus() && cols <= 96) {  // (2 x 4 blocks per wavefront would leave one wavefront per SIMD)
     const unsigned gx = (unsigned)((rows + 255) / 256);
+    if constexpr (MODE == CONV_UP) {
+      if (a.pad0 == 0 && (a.Mx - 1) * a.s + a.k <= a.H && rows % 256 == 0) {  // nothing to mask in the image gather
+        if (cols <= 32) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 2, 1, false, 0, true>), dim3(gx, (cols + 31) / 32, gz), dim3(256), 0, 0, a);
+        else if (cols <= 64) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 2, 2, false, 0, true>), dim3(gx, (cols + 63) / 64, gz), dim3(256), 0, 0, a);
+        else hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 2, 3, false, 0, true>), dim3(gx, (cols + 95) / 96, gz), dim3(256), 0, 0, a);
+        return;
+      }
+    }
     if (cols <= 32) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 2, 1>), dim3(gx, (cols + 31) / 32, gz), dim3(256), 0, 0, a);
     else if (cols <= 64) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 2, 2>), dim3(gx, (cols + 63) / 64, gz), dim3(256), 0, 0, a);
     else hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 2, 3>), dim3(gx, (cols + 95) / 96, gz), dim3(256), 0, 0, a);

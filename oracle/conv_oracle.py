@@ -192,6 +192,79 @@ def conv_outp(images, hid, C, Mx, k, padding, stride, groups=1, partial_sum=0):
 
 # ---- locally connected layers: cudamat_conv.cu:1415-1423, filters (module, colour, ky, kx, filter) ----
 
+# ---- single outputs of the three passes: for checks at sizes where the full float64
+# ---- convolution would take minutes.  Each returns (value, sum of |terms|).
+
+def conv_up_at(images, filters, C, Mx, padding, stride, groups, n, f, my, mx):
+    """targets[n, (f, my, mx)] of convUp, straight from the definition
+    (cudamat_conv_kernels.cuh:82-257: out = sum_{c,ky,kx} img(g*Cg+c, my*s-pad+ky, mx*s-pad+kx) * w(f, c, ky, kx))."""
+    N, H, F, Cg, k, Fg = _geom(images, filters, C, groups)
+    g = f // Fg
+    w = np.asarray(filters[f], dtype=F64).reshape(Cg, k, k)
+    x = np.asarray(images[n], dtype=F64).reshape(C, H, H)[g * Cg:(g + 1) * Cg]
+    val = mag = 0.0
+    for ky in range(k):
+        y = my * stride - padding + ky
+        if not 0 <= y < H:
+            continue
+        for kx in range(k):
+            xx = mx * stride - padding + kx
+            if 0 <= xx < H:
+                t = x[:, y, xx] * w[:, ky, kx]
+                val += t.sum(); mag += np.abs(t).sum()
+    return val, mag
+
+
+def conv_down_at(hid, filters, C, H, padding, stride, groups, n, c, y, x):
+    """targets[n, (c, y, x)] of convDown: the sum over the group's filters and over the
+    modules (my, mx) whose tap (y + pad - my*s, x + pad - mx*s) exists
+    (cudamat_conv_kernels.cuh:265-640)."""
+    hid = np.asarray(hid)
+    F = filters.shape[0]
+    Cg = C // groups
+    Fg = F // groups
+    k = int(round((filters.shape[1] // Cg) ** 0.5))
+    M = hid.shape[1] // F
+    Mx = int(round(M ** 0.5))
+    g, cl = c // Cg, c % Cg
+    w = np.asarray(filters[g * Fg:(g + 1) * Fg], dtype=F64).reshape(Fg, Cg, k, k)[:, cl]
+    h = np.asarray(hid[n], dtype=F64).reshape(F, Mx, Mx)[g * Fg:(g + 1) * Fg]
+    val = mag = 0.0
+    for my in range(Mx):
+        ky = y + padding - my * stride
+        if not 0 <= ky < k:
+            continue
+        for mx in range(Mx):
+            kx = x + padding - mx * stride
+            if 0 <= kx < k:
+                t = h[:, my, mx] * w[:, ky, kx]
+                val += t.sum(); mag += np.abs(t).sum()
+    return val, mag
+
+
+def conv_outp_at(images, hid, C, Mx, k, padding, stride, groups, f, c, ky, kx):
+    """targets[f, (c, ky, kx)] of convOutp with one module group (c counts colours of
+    f's group): the sum over all modules and images (cudamat_conv_kernels.cuh:642-1015)."""
+    images, hid = np.asarray(images), np.asarray(hid)
+    N = images.shape[0]
+    H = int(round((images.shape[1] // C) ** 0.5))
+    F = hid.shape[1] // (Mx * Mx)
+    Cg, Fg = C // groups, F // groups
+    g = f // Fg
+    x = images.reshape(N, C, H, H)[:, g * Cg + c]
+    h = hid.reshape(N, F, Mx, Mx)[:, f]
+    val = mag = 0.0
+    for my in range(Mx):
+        y = my * stride - padding + ky
+        if not 0 <= y < H:
+            continue
+        xs = np.arange(Mx) * stride - padding + kx
+        ok = (xs >= 0) & (xs < H)
+        t = x[:, y, xs[ok]].astype(F64) * h[:, my, ok].astype(F64)
+        val += t.sum(); mag += np.abs(t).sum()
+    return val, mag
+
+
 def local_up(images, filters, C, Mx, padding, stride):
     """Like conv_up with a separate filter bank per module: filters is (F, M*C*k*k) with
     column ((m*C + c)*k + ky)*k + kx."""

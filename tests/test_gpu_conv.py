@@ -270,3 +270,49 @@ def _random_small_layer_cases(seed, count):
 @pytest.mark.parametrize("N,C,H,F,k,s,p,G", _random_small_layer_cases(20240611, 30))
 def test_three_conv_passes_on_random_small_layers(cm, cc, rng, N, C, H, F, k, s, p, G):
     test_three_conv_passes(cm, cc, rng, N, C, H, F, k, s, p, G)
+
+
+FULL_LAYERS = [  # the conv layers of benchmark config 5 at full size: N, C, H, F, k, stride, padding, groups
+    (128, 3, 224, 96, 11, 4, 0, 1),
+    (128, 96, 27, 256, 5, 1, 2, 2),
+]
+
+
+@pytest.mark.parametrize("N,C,H,F,k,s,p,G", FULL_LAYERS)
+def test_benchmark_layers_at_full_size_on_sampled_outputs(cm, cc, N, C, H, F, k, s, p, G):
+    """The kernels these shapes select (256-row tiles with the unmasked gather, uniform-row
+    tiles, 16-wide column blocks, split-K convOutp) only come into play at sizes where the
+    float64 passes would take minutes: random outputs of each pass are checked against the
+    definition evaluated for that single output, and the three results against each other
+    through the adjoint identities."""
+    r = np.random.default_rng(55)
+    Mx = co.n_modules(H, k, s, p)
+    Cg = C // G
+    x = _f(r.standard_normal((N, C * H * H)))
+    w = _f(0.05 * r.standard_normal((F, Cg * k * k)))
+    y = _f(r.standard_normal((N, F * Mx * Mx)))
+    X, W, Y = cm.CUDAMatrix(x), cm.CUDAMatrix(w), cm.CUDAMatrix(y)
+    up, down, outp = cm.empty((N, F * Mx * Mx)), cm.empty((N, C * H * H)), cm.empty((F, Cg * k * k))
+    cc.convUp(X, W, up, Mx, p, s, C, G)
+    cc.convDown(Y, W, down, Mx, p, s, k, H, C, numGroups=G)
+    cc.convOutp(X, Y, outp, Mx, p, k, s, C, numGroups=G)
+    u, d, o = up.asarray().reshape(N, F, Mx, Mx), down.asarray().reshape(N, C, H, H), outp.asarray().reshape(F, Cg, k, k)
+    edge = lambda size: int(r.choice([0, size - 1, int(r.integers(size))]))      # borders twice as often as the interior
+    for _ in range(300):
+        n, f, my, mx = int(r.integers(N)), int(r.integers(F)), edge(Mx), edge(Mx)
+        val, mag = co.conv_up_at(x, w, C, Mx, p, s, G, n, f, my, mx)
+        assert abs(u[n, f, my, mx] - val) <= REL * mag + 1e-30
+        c, yy, xx = int(r.integers(C)), edge(H), edge(H)
+        val, mag = co.conv_down_at(y, w, C, H, p, s, G, n, c, yy, xx)
+        assert abs(d[n, c, yy, xx] - val) <= REL * mag + 1e-6
+    for _ in range(12):
+        f, cl, ky, kx = int(r.integers(F)), int(r.integers(Cg)), edge(k), edge(k)
+        val, mag = co.conv_outp_at(x, y, C, Mx, k, p, s, G, f, cl, ky, kx)
+        assert abs(o[f, cl, ky, kx] - val) <= REL * mag
+    a = float((up.asarray().astype(np.float64) * y).sum())
+    b = float((down.asarray().astype(np.float64) * x).sum())
+    c_ = float((outp.asarray().astype(np.float64) * w).sum())
+    scale = float((np.abs(up.asarray()).astype(np.float64) * np.abs(y)).sum())
+    assert abs(a - b) / scale < 1e-5 and abs(a - c_) / scale < 1e-5
+    for m in (X, W, Y, up, down, outp):
+        m.free_device_memory()

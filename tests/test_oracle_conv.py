@@ -154,3 +154,23 @@ def test_local_layers_reduce_to_conv_with_shared_filters_and_are_adjoint(rng):
     y = rng.standard_normal((N, F * M))
     up, down, outp = co.local_up(x, wl, C, Mx, p, s), co.local_down(y, wl, C, H, p, s), co.local_outp(x, y, C, Mx, k, p, s)
     assert np.isclose((up * y).sum(), (x * down).sum()) and np.isclose((up * y).sum(), (wl * outp).sum())
+
+
+@pytest.mark.parametrize("N,C,H,F,k,s,p,G", [(3, 4, 7, 6, 3, 2, 1, 2), (2, 3, 9, 4, 4, 3, 2, 1), (4, 2, 6, 2, 5, 1, 4, 1)])
+def test_single_output_evaluators_agree_with_the_full_passes(rng, N, C, H, F, k, s, p, G):
+    # the sampled forms used for full-size device checks, against the vectorised passes
+    # (themselves pinned against the literal loops, torch and the adjoint identities)
+    Mx = co.n_modules(H, k, s, p)
+    x = rng.standard_normal((N, C * H * H))
+    w = rng.standard_normal((F, (C // G) * k * k))
+    y = rng.standard_normal((N, F * Mx * Mx))
+    up = co.conv_up(x, w, C, Mx, p, s, G).reshape(N, F, Mx, Mx)
+    down = co.conv_down(y, w, C, H, p, s, G).reshape(N, C, H, H)
+    outp = co.conv_outp(x, y, C, Mx, k, p, s, G).reshape(F, C // G, k, k)
+    for _ in range(40):
+        n, f, my, mx = rng.integers(N), rng.integers(F), rng.integers(Mx), rng.integers(Mx)
+        assert abs(co.conv_up_at(x, w, C, Mx, p, s, G, n, f, my, mx)[0] - up[n, f, my, mx]) < 1e-10
+        c, yy, xx = rng.integers(C), rng.integers(H), rng.integers(H)
+        assert abs(co.conv_down_at(y, w, C, H, p, s, G, n, c, yy, xx)[0] - down[n, c, yy, xx]) < 1e-10
+        cl, ky, kx = rng.integers(C // G), rng.integers(k), rng.integers(k)
+        assert abs(co.conv_outp_at(x, y, C, Mx, k, p, s, G, f, cl, ky, kx)[0] - outp[f, cl, ky, kx]) < 1e-10
