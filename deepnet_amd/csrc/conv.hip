@@ -174,12 +174,14 @@ __device__ __forceinline__ void down_axis(int ph, int s, int pad0, int H, int k,
 // kernel, slab offset in an SGPR, an out-of-range offset for a tap in the padding, which
 // the hardware answers with zeros -- and cost no vector instructions, which matters
 // because fp32 MFMA and the vector ALU share lanes.  Both operands run two slabs ahead.
-// INSIDE (general convUp gather only): no padding, the last module ends inside the image
-// and the rows fill their tiles, so no image group is ever masked: its gather is an add
-// and a load (a tap beyond the reduction re-reads the last one against a zero filter row).
+// INSIDE (general gathers of the image: convUp rows, convOutp columns): no padding and the
+// last module ends inside the image, so no image group is ever masked and its gather is
+// an add and a load.  convUp: the rows fill their tiles, and a tap beyond the reduction
+// re-reads the last one against a zero filter row.  convOutp: rows and columns beyond
+// the output are computed on whatever valid data was read and never stored.
 template <int MODE, int WAVES_M, int WM, int WN, bool UNI = false, int N16 = 0, bool INSIDE = false>
 __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
-  static_assert(!INSIDE || (MODE == CONV_UP && !UNI), "INSIDE: the general convUp gather");
+  static_assert(!INSIDE || ((MODE == CONV_UP || MODE == CONV_OUTP) && !UNI), "INSIDE: the general gathers of the image");
   constexpr int WAVES_N = 4 / WAVES_M;
   constexpr int BM = 32 * WM * WAVES_M, BN = 32 * WN * WAVES_N;
   // Row pitch in LDS: operands written transposed one float per lane want pitch % 8 == 2
@@ -323,6 +325,7 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
         const int ky = (int)fd_div((uint32_t)pp, p.dk), kx = pp - ky * k;
         b_y[u] = p.pad0 + ky; b_x[u] = p.pad0 + kx;
         b_voff[u] = 4u * (unsigned)(N * ((g * Cg + cc) * HH + b_y[u] * H + b_x[u]) + b_k[u] + (int)img_bias);
+        if (INSIDE && !b_ok[u]) b_voff[u] = 4u * (unsigned)b_k[u];   // a column beyond the output: any valid address
       }
     }
   }
@@ -501,11 +504,15 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
         if (!ok) src = p.flt;
         rb[SET][u] = *reinterpret_cast<const f32x4*>(src);
       } else {
-        const int y = st_a * s + b_y[u], x = st_b * s + b_x[u];
-        ok = ok & ((unsigned)y < (unsigned)H) & ((unsigned)x < (unsigned)H);
         const unsigned so = 4u * ((unsigned)N * (unsigned)(st_a * s * H + st_b * s) + (unsigned)st_c);  // scalar
-        const unsigned voff = ok ? b_voff[u] + so : 4u * img_bias;
-        rb[SET][u] = *reinterpret_cast<const f32x4*>(b_base + voff);
+        if constexpr (INSIDE) {
+          rb[SET][u] = *reinterpret_cast<const f32x4*>(b_base + (b_voff[u] + so));
+        } else {
+          const int y = st_a * s + b_y[u], x = st_b * s + b_x[u];
+          ok = ok & ((unsigned)y < (unsigned)H) & ((unsigned)x < (unsigned)H);
+          const unsigned voff = ok ? b_voff[u] + so : 4u * img_bias;
+          rb[SET][u] = *reinterpret_cast<const f32x4*>(b_base + voff);
+        }
       }
       rb_ok[SET][u] = ok;
     }
@@ -534,7 +541,7 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
 #pragma unroll
     for (int u = 0; u < NB; ++u) {
       if (tid + u * 256 >= TB) continue;
-      if (!UNI && !rb_ok[SET][u]) rb[SET][u] = zero4;
+      if (!UNI && !(INSIDE && MODE == CONV_OUTP) && !rb_ok[SET][u]) rb[SET][u] = zero4;
       if (MODE == CONV_UP) {
         *reinterpret_cast<f32x4*>(&Bs[buf][b_k[u]][b_c[u]]) = rb[SET][u];
       } else {
@@ -1674,7 +1681,13 @@ static void conv_outp_impl(cudamat* images, cudamat* hidActs, cudamat* targets, 
       a.partial = (float*)dn_scratch((size_t)a.splits * F * cols * sizeof(float));
       if (!a.partial) { conv_set_error(where, "out of device memory for the split-K workspace"); return; }
       dim3 grid(gx, gy, numGroups * a.splits);
-      if (BMs == 32) hipLaunchKernelGGL((k_conv_mfma<CONV_OUTP, 1, 1, 1>), grid, dim3(256), 0, 0, a);
+      if (paddingStart == 0 && (numModulesX - 1) * moduleStride + filterSize <= H) {  // nothing to mask in the image gather
+        if (BMs == 32) hipLaunchKernelGGL((k_conv_mfma<CONV_OUTP, 1, 1, 1, false, 0, true>), grid, dim3(256), 0, 0, a);
+        else if (BMs == 64) hipLaunchKernelGGL((k_conv_mfma<CONV_OUTP, 1, 2, 1, false, 0, true>), grid, dim3(256), 0, 0, a);
+        else if (BMs == 96) hipLaunchKernelGGL((k_conv_mfma<CONV_OUTP, 1, 3, 1, false, 0, true>), grid, dim3(256), 0, 0, a);
+        else hipLaunchKernelGGL((k_conv_mfma<CONV_OUTP, 2, 2, 2, false, 0, true>), grid, dim3(256), 0, 0, a);
+      }
+      else if (BMs == 32) hipLaunchKernelGGL((k_conv_mfma<CONV_OUTP, 1, 1, 1>), grid, dim3(256), 0, 0, a);
       else if (BMs == 64) hipLaunchKernelGGL((k_conv_mfma<CONV_OUTP, 1, 2, 1>), grid, dim3(256), 0, 0, a);
       else if (BMs == 96) hipLaunchKernelGGL((k_conv_mfma<CONV_OUTP, 1, 3, 1>), grid, dim3(256), 0, 0, a);
       else hipLaunchKernelGGL((k_conv_mfma<CONV_OUTP, 2, 2, 2>), grid, dim3(256), 0, 0, a);
