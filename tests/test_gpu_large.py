@@ -215,3 +215,48 @@ def test_conv_passes_with_outputs_beyond_32_bit_byte_offsets(cm, cc, N):
         assert abs(o[f, cl, ky, kx] - val) <= 1e-4 * mag
     for m in (X, Wm, Y, up, down, outp):
         m.free_device_memory()
+
+
+def _rows(mat, N):
+    """Host copy of a few images (rows) of a device matrix: first, middle (around the row
+    whose first-filter offset passes 2^31 bytes) and last."""
+    parts = []
+    for lo in (0, N // 2 - 2, N - 4):
+        parts.append(mat.get_row_slice(lo, lo + 4).asarray().copy())
+    return _f(np.concatenate(parts, axis=0))
+
+
+def test_pool_and_norm_on_maps_beyond_32_bit_byte_offsets(cm, cc):
+    N, F, S = 16512, 64, 32                      # 16512 x 65536 floats: 4.33 GB per matrix
+    subs, start, stride = 3, 0, 2
+    O = (S - start - subs + stride - 1) // stride + 1
+    X = cm.empty((N, F * S * S))
+    X.fill_with_randn()
+    x = _rows(X, N)
+    T = cm.empty((N, F * O * O))
+    cc.MaxPool(X, T, F, subs, start, stride, O)
+    want = co.max_pool(x, F, subs, start, stride, O)
+    assert np.array_equal(_rows(T, N), want.astype(np.float32))
+    G = cm.empty((N, F * O * O))
+    G.fill_with_randn()
+    g = _rows(G, N)
+    U = cm.empty((N, F * S * S))
+    cc.MaxPoolUndo(X, U, G, T, subs, start, stride, O)
+    assert np.allclose(_rows(U, N), co.max_pool_undo(x, g, want, subs, start, stride, O), rtol=1e-6, atol=1e-6)
+    G.free_device_memory(); T.free_device_memory()
+    # response normalisation over the same maps, then its gradient
+    a, p, size = 0.001, 0.75, 5
+    D, Tn = cm.empty((N, F * S * S)), cm.empty((N, F * S * S))
+    cc.ResponseNorm(X, D, Tn, F, size, a, p)
+    t_want, d_want = co.response_norm(x, F, size, a, p)
+    assert np.allclose(_rows(D, N), d_want, rtol=2e-6)
+    assert np.allclose(_rows(Tn, N), t_want, rtol=1e-5, atol=1e-7)
+    U.fill_with_randn()                          # U now holds the incoming gradient
+    og, d_got, t_got = _rows(U, N), _rows(D, N), _rows(Tn, N)
+    R = cm.empty((N, F * S * S))
+    cc.ResponseNormUndo(U, D, X, Tn, R, F, size, a, p)
+    u_want, acts_want = co.response_norm_undo(og, d_got, x, t_got, F, size, a, p)
+    assert np.allclose(_rows(Tn, N), acts_want, rtol=1e-5, atol=1e-9)
+    assert np.allclose(_rows(R, N), u_want, rtol=1e-5, atol=1e-6)
+    for m in (X, U, D, Tn, R):
+        m.free_device_memory()
