@@ -75,7 +75,34 @@ def run(cm, ev, iters=10):
                 ms = _time(ev, fn, iters, cm.cuda_sync_threads)
                 gbs = nbytes / (ms * 1e-3) / 1e9
                 res[label] = {'us': round(ms * 1e3, 2), 'gbs': round(gbs, 1), 'frac_hbm': round(gbs / HBM_PEAK_GBS, 4)}
+            res['stage_fwd_bwd'] = _stage(cm, ev, iters, L, W, rng)
         out[name] = res
         for m in (X, W, Y, up, down, dw):
             m.free_device_memory()
     return {'conv': out}
+
+
+def _stage(cm, ev, iters, L, W, rng):
+    """The whole conv stage of a deepnet edge at this layer (transpose, convUp, pool 3x3/2,
+    rnorm 5, transpose; then the backward pass and the weight gradient) through
+    deepnet_amd/convolutions.py: twelve library calls per step."""
+    import types
+    from deepnet_amd import convolutions as cv_mod
+    N, C, H, F, k, s, p = (L[x] for x in ('N', 'C', 'H', 'F', 'k', 's', 'p'))
+    cv = cv_mod.ConvParams(size=k, stride=s, padding=p, num_filters=F, num_colors=C, max_pool=True, pool_size=3,
+                           pool_stride=2, rnorm=True, norm_size=5)
+    O = ((H + 2 * p - k) // s + 1 - 3) // 2 + 1
+    f = lambda a: cm.CUDAMatrix(np.asarray(a, dtype=np.float32, order='F'))
+    inputs, deriv = f(rng.standard_normal((C * H * H, N))), f(rng.standard_normal((F * O * O, N)))
+    edge = cv_mod.ConvEdge(W, cv, inputs.shape, deriv.shape)
+    state, grad = cm.empty(deriv.shape), cm.empty(W.shape)
+    layer = types.SimpleNamespace(dirty=False, is_input=False, deriv=cm.empty(inputs.shape))
+
+    def step():
+        layer.dirty = False
+        cv_mod.ConvolveUp(inputs, edge, state)
+        cv_mod.AccumulateConvDeriv(layer, edge, deriv)
+        cv_mod.ConvOuter(edge, grad)
+    ms = _time(ev, step, iters, cm.cuda_sync_threads)
+    edge.free_device_memory()
+    return {'us': round(ms * 1e3, 1), 'steps_per_sec': round(1e3 / ms, 1)}

@@ -411,3 +411,56 @@ def response_norm_undo(out_grads, denoms, inputs, acts, F, size, add_scale, pow_
     act2 = F64(np.float32(-2.0) * np.float32(add_scale) * np.float32(pow_scale)) * og4 * act4 / den4
     win = _window_sum(act2, size, size // 2 - size + 1)
     return from_nchw(in4 * win + og4 * den4 ** (-p)), from_nchw(act2)
+
+
+# ---- the conv stage of an edge: deepnet/convolutions.py:5-184 -------------------------------
+# cv is any object with the fields of Parameter.Convolution (deepnet.proto:64-78).  Layer
+# states are (dims, batch) as in deepnet; everything in between is in the device layout.
+
+def _stage_sites(cv, numdims):
+    side = int(round(np.sqrt(numdims // cv.num_colors)))
+    n_locs = n_modules(side, cv.size, cv.stride, cv.padding)                       # convolutions.py:35
+    n_pool = (n_locs - cv.pool_size) // cv.pool_stride + 1 if cv.max_pool else n_locs   # :48
+    return side, n_locs, n_pool
+
+
+def stage_forward(inputs, w, cv, local=False):
+    """ConvolveUp (convolutions.py:5-67) without probabilistic pooling.  Returns a dict with
+    the state (dims_out, batch) and every intermediate the backward pass reads."""
+    x_t = np.asarray(inputs, dtype=F64).T
+    side, n_locs, n_pool = _stage_sites(cv, x_t.shape[1])
+    up = local_up if local else conv_up
+    keep = {'input_t': x_t}
+    cur = up(x_t, w, cv.num_colors, n_locs, cv.padding, cv.stride)
+    if cv.max_pool:
+        keep['unpooled'] = cur
+        cur = max_pool(cur, cv.num_filters, cv.pool_size, 0, cv.pool_stride, n_pool)
+    if cv.rnorm:
+        keep['unnormalized'] = cur
+        cur, keep['denoms'] = response_norm(cur, cv.num_filters, cv.norm_size, cv.add_scale, cv.pow_scale)
+    keep['output_t'] = cur
+    keep['state'] = cur.T
+    return keep
+
+
+def stage_backward(fwd, w, cv, deriv, local=False):
+    """AccumulateConvDeriv + ConvOuter (convolutions.py:69-184) on what stage_forward kept:
+    returns (gradient w.r.t. the inputs as (dims_in, batch), gradient w.r.t. the weights).
+    The normalisation step is given the operands in deepnet's order (:120-122): the normalised
+    outputs where the library call names `inputs`, the un-normalised layer where it names `acts`."""
+    grads = np.asarray(deriv, dtype=F64).T
+    acts = fwd['output_t']
+    side, n_locs, n_pool = _stage_sites(cv, fwd['input_t'].shape[1])
+    if cv.rnorm:
+        grads, _ = response_norm_undo(grads, fwd['denoms'], acts, fwd['unnormalized'], cv.num_filters,
+                                      cv.norm_size, cv.add_scale, cv.pow_scale)
+        acts = fwd['unnormalized']
+    if cv.max_pool:
+        grads = max_pool_undo(fwd['unpooled'], grads, acts, cv.pool_size, 0, cv.pool_stride, n_pool)
+    if local:
+        d_in = local_down(grads, w, cv.num_colors, side, cv.padding, cv.stride)
+        d_w = local_outp(fwd['input_t'], grads, cv.num_colors, n_locs, cv.size, cv.padding, cv.stride)
+    else:
+        d_in = conv_down(grads, w, cv.num_colors, side, cv.padding, cv.stride)
+        d_w = conv_outp(fwd['input_t'], grads, cv.num_colors, n_locs, cv.size, cv.padding, cv.stride)
+    return d_in.T, d_w

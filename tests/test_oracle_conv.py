@@ -174,3 +174,60 @@ def test_single_output_evaluators_agree_with_the_full_passes(rng, N, C, H, F, k,
         assert abs(co.conv_down_at(y, w, C, H, p, s, G, n, c, yy, xx)[0] - down[n, c, yy, xx]) < 1e-10
         cl, ky, kx = rng.integers(C // G), rng.integers(k), rng.integers(k)
         assert abs(co.conv_outp_at(x, y, C, Mx, k, p, s, G, f, cl, ky, kx)[0] - outp[f, cl, ky, kx]) < 1e-10
+
+
+class _Cv(object):
+    """Parameter.Convolution with the proto's defaults (deepnet.proto:64-78)."""
+
+    def __init__(self, **kw):
+        self.size = self.stride = self.padding = self.num_filters = self.num_colors = 0
+        self.max_pool, self.pool_size, self.pool_stride, self.prob = False, 0, 0, False
+        self.rnorm, self.norm_size, self.pow_scale, self.add_scale = False, 0, 0.75, 0.001
+        self.__dict__.update(kw)
+
+
+def _torch_stage(x, w, cv, side):
+    """The stage in torch on (N, C, H, W) tensors: conv2d -> max_pool2d -> LRN by avg_pool2d."""
+    t = TF.conv2d(x, w, stride=cv.stride, padding=cv.padding)
+    if cv.max_pool:
+        t = TF.max_pool2d(t, cv.pool_size, cv.pool_stride)
+    unnorm, den = t, None
+    if cv.rnorm:
+        den = 1.0 + cv.add_scale_f * cv.norm_size ** 2 * TF.avg_pool2d(t * t, cv.norm_size, 1, cv.norm_size // 2,
+                                                                      count_include_pad=True)
+        t = t * den ** (-cv.pow_scale_f)
+    return t, unnorm, den
+
+
+@pytest.mark.parametrize("pool,rnorm", [(False, False), (True, False), (False, True), (True, True)])
+def test_conv_stage_forward_and_backward_against_torch(rng, pool, rnorm):
+    """Forward: the chain in torch.  Backward without normalisation: torch.autograd's gradient of
+    that chain (pooling windows that fit the map, no ties).  With normalisation the reference
+    feeds ResponseNormUndo its operands in the other order, which is not the true gradient: its
+    result is pinned against the same expression written with torch's pooling routines."""
+    N, C, H, F, k = 3, 2, 9, 16, 3
+    cv = _Cv(size=k, stride=1, padding=1, num_filters=F, num_colors=C, max_pool=pool, pool_size=3, pool_stride=2,
+             rnorm=rnorm, norm_size=3)
+    cv.add_scale_f, cv.pow_scale_f = float(np.float32(cv.add_scale)), float(np.float32(cv.pow_scale))
+    inputs = rng.standard_normal((C * H * H, N))                       # deepnet's (dims, batch)
+    w = rng.standard_normal((F, C * k * k))
+    fwd = co.stage_forward(inputs, w, cv)
+    xt = torch.from_numpy(co.to_nchw(inputs.T, C, H)).requires_grad_(True)
+    wt = torch.from_numpy(co.filters_to_fckk(w, C, k)).requires_grad_(True)
+    out, unnorm, den = _torch_stage(xt, wt, cv, H)
+    assert np.allclose(fwd['state'].T, out.detach().numpy().reshape(N, -1), atol=1e-12)
+    deriv = rng.standard_normal(fwd['state'].shape)
+    g = torch.from_numpy(deriv.T.reshape(out.shape).copy())
+    if rnorm:
+        # deepnet's operand order: y_k * window_sum(-2ab * g * x / d) + g * d^-b, then the true
+        # gradient of the rest of the chain
+        ab = float(np.float32(-2.0) * np.float32(cv.add_scale) * np.float32(cv.pow_scale))
+        inner = ab * g * unnorm.detach() / den.detach()
+        win = cv.norm_size ** 2 * TF.avg_pool2d(inner, cv.norm_size, 1, cv.norm_size // 2, count_include_pad=True)
+        g = out.detach() * win + g * den.detach() ** (-cv.pow_scale_f)
+        unnorm.backward(g)
+    else:
+        out.backward(g)
+    d_in, d_w = co.stage_backward(fwd, w, cv, deriv)
+    assert np.allclose(d_in.T, xt.grad.numpy().reshape(N, -1), atol=1e-10)
+    assert np.allclose(d_w, wt.grad.numpy().reshape(F, -1), atol=1e-10)
