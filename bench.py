@@ -227,6 +227,29 @@ class MLP(object):
             cm.momentum_update(b[i], self.db[i], self.gb[i], self.mom, self.lr, reset_gradient=False)
 
 
+def net_mlp(cm, sizes=(784, 1024, 1024, 10), B=128, seed=3, fused=False):
+    """The MLP of config 3 as a deepnet net: Layer / Edge / NeuralNet objects of this package
+    driven by TrainOneBatch, i.e. the reference's own control flow (neuralnet.py:138-337) with
+    its per-step loss read-backs (two blocking sums per step in SoftmaxLayer.GetLoss)."""
+    from deepnet_amd import layer as dl, neuralnet as dnn, parameter as dp
+    rng = np.random.default_rng(seed)
+    sgd = dict(base_epsilon=0.01, initial_momentum=0.9, final_momentum=0.9)
+    layers = [dl.LinearLayer('input', sizes[0], B, hyperparams=dp.Hyperparams(), is_input=True)]
+    for i in (1, 2):
+        layers.append(dl.ReluLayer('hidden%d' % i, sizes[i], B,
+                                   hyperparams=dp.Hyperparams(activation=dp.RECTIFIED_LINEAR, dropout=True, **sgd)))
+    layers.append(dl.SoftmaxLayer('output', 1, B, hyperparams=dp.Hyperparams(activation=dp.SOFTMAX, **sgd),
+                                  numlabels=sizes[3], is_output=True, loss_function=dp.CROSS_ENTROPY))
+    edges = [dnn.Edge(layers[i], layers[i + 1], 0.01 * rng.standard_normal((sizes[i], sizes[i + 1])),
+                      hyperparams=dp.Hyperparams(**sgd)) for i in range(3)]
+    for obj in layers + edges:
+        obj.fused = fused
+    net = dnn.NeuralNet(layers, edges)
+    layers[0].data.assign(cm.CUDAMatrix(np.asarray(rng.random((sizes[0], B)), dtype=np.float32, order='F')))
+    layers[-1].data.assign(cm.CUDAMatrix(np.asarray(rng.integers(0, sizes[3], (1, B)), dtype=np.float32, order='F')))
+    return net
+
+
 def time_loop(cm, fn, iters, warmup):
     for _ in range(warmup):
         fn()
@@ -457,6 +480,11 @@ def main():
         secondary['mlp_fused_extensions'] = {
             'steps_per_sec': round(1.0 / t, 1), 'us_per_step': round(t * 1e6, 1),
             'note': 'same step with dot_bias_act, softmax_ce_grad and momentum_update (extensions of this backend, not in the reference API): 32 launches instead of 51'}
+        net = net_mlp(cm)
+        t = time_loop(cm, lambda: net.TrainOneBatch(0), 100, 10)
+        secondary['mlp_through_neuralnet_classes'] = {
+            'steps_per_sec': round(1.0 / t, 1), 'us_per_step': round(t * 1e6, 1),
+            'note': 'same net as Layer / Edge / NeuralNet objects, TrainOneBatch with its two blocking loss read-backs per step'}
         secondary['gemm_fp32_4096'] = gemm_probe(cm, ev)
         try:
             import bench_conv

@@ -1,0 +1,202 @@
+"""Feed-forward nets trained by back-propagation on the MI355X backend: the training-step
+core of the reference's deepnet/neuralnet.py -- ``ComputeUp`` (:138-207), ``ComputeDown``
+(:209-235), ``AccumulateDeriv`` (:237-255), ``UpdateEdgeParams`` (:257-275),
+``UpdateLayerParams`` (:277-290), ``ForwardPropagate`` / ``BackwardPropagate`` /
+``TrainOneBatch`` / ``EvaluateOneBatch`` (:292-337) -- and the part of deepnet/edge.py a
+training step touches, issuing the same matrix and conv calls in the same order.
+
+A net is built from Layer objects and Edge objects (dense or conv / locally connected)
+instead of a protobuf model; data handlers, model files, evaluation loops over data sets,
+tied parameters and replicated-softmax neighbours stay outside.
+"""
+import sys
+
+import numpy as np
+
+from .choose_matrix_library import cm
+from .convolutions import ConvolveUp, AccumulateConvDeriv, ConvOuter, AddConvolveUp, ConvEdge
+from .parameter import Parameter, Hyperparams
+
+
+class Edge(Parameter):
+    """A weight matrix between two layers (deepnet/edge.py:8-35, 83-92).  Dense: ``weight`` is
+    (node1 dims, node2 dims).  With ``conv_params``: (num_filters, colours * size^2) shared
+    filters, or one bank per module when ``local``; the conv buffers are those of ConvEdge."""
+
+    def __init__(self, node1, node2, weight, hyperparams=None, conv_params=None, local=False, up_factor=1.0,
+                 block_gradient=False):
+        super(Edge, self).__init__()
+        self.node1, self.node2 = node1, node2
+        self.name = '%s:%s' % (node1.name, node2.name)
+        self.hyperparams = hyperparams or Hyperparams()
+        self.proto = _EdgeProto(up_factor, block_gradient)
+        self.tied_to = None
+        self.marker = 0
+        self.conv = conv_params is not None and not local
+        self.local = conv_params is not None and local
+        w = cm.CUDAMatrix(np.asarray(weight, dtype=np.float32, order='F'))
+        self.params['weight'] = w
+        if conv_params is not None:
+            self.conv_params = conv_params
+            buffers = ConvEdge(w, conv_params, node1.state.shape, node2.state.shape, conv=not local)
+            for name in ('input_t', 'input_t2', 'output_t', 'output_t2', 'unpooled_layer', 'rnd',
+                         'unrnormalized_layer', 'denoms', 'rnorm_temp1', 'rnorm_temp2'):
+                if hasattr(buffers, name):
+                    setattr(self, name, getattr(buffers, name))
+        else:
+            assert w.shape == (node1.state.shape[0], node2.state.shape[0])
+        self.AllocateMemory()
+        node1.AddOutgoingEdge(self)
+        node2.AddIncomingEdge(self)
+
+    def AllocateMemory(self):
+        shape = self.params['weight'].shape
+        zeros = lambda: cm.CUDAMatrix(np.zeros(shape, dtype=np.float32, order='F'))
+        self.temp, self.gradient, self.gradient_history = zeros(), zeros(), zeros()
+
+
+class _EdgeProto(object):
+    def __init__(self, up_factor, block_gradient):
+        self.up_factor, self.block_gradient = up_factor, block_gradient
+
+
+class NeuralNet(object):
+
+    def __init__(self, layers, edges, verbose=False):
+        self.layer, self.edge, self.verbose = list(layers), list(edges), verbose
+        self.input_datalayer = [n for n in self.layer if n.is_input]
+        self.output_datalayer = [n for n in self.layer if n.is_output]
+        self.train_stop_steps = sys.maxsize
+        self.node_list = self.Sort()
+
+    def Sort(self):
+        """Layers in an order in which every layer comes after all layers feeding it."""
+        for e in self.edge:
+            e.marker = 0
+        order, ready = [], [n for n in self.layer if not n.incoming_neighbour]
+        while ready:
+            n = ready.pop()
+            order.append(n)
+            for e in n.outgoing_edge:
+                if e.marker == 0:
+                    e.marker = 1
+                    if all(x.marker == 1 for x in e.node2.incoming_edge):
+                        ready.append(e.node2)
+        if not all(e.marker == 1 for e in self.edge):
+            raise Exception('Invalid net for backprop. Cycle exists.')
+        return order
+
+    def ComputeUp(self, layer, train=False, step=0, maxsteps=0):
+        """State of ``layer`` from the states of the layers feeding it; then dropout."""
+        layer.dirty = False
+        if layer.is_input or layer.is_initialized:
+            layer.GetData()
+        else:
+            for i, edge in enumerate(layer.incoming_edge):
+                if edge in layer.outgoing_edge:
+                    continue
+                inputs = layer.incoming_neighbour[i].state
+                if edge.conv or edge.local:
+                    if i == 0:
+                        ConvolveUp(inputs, edge, layer.state)
+                    else:
+                        AddConvolveUp(inputs, edge, layer.state)
+                else:
+                    w = edge.params['weight']
+                    factor = edge.proto.up_factor
+                    if i == 0:
+                        cm.dot(w.T, inputs, target=layer.state)
+                        if factor != 1:
+                            layer.state.mult(factor)
+                    else:
+                        layer.state.add_dot(w.T, inputs, mult=factor)
+            layer.state.add_col_vec(layer.params['bias'])
+            layer.ApplyActivation()
+        h = layer.hyperparams
+        if h.dropout:
+            if train and maxsteps - step >= h.stop_dropout_for_last:
+                if h.mult_dropout:
+                    layer.mask.fill_with_randn()
+                    layer.mask.add(1)
+                    layer.state.mult(layer.mask)
+                else:
+                    layer.mask.fill_with_rand()
+                    layer.mask.greater_than(h.dropout_prob)
+                    if h.blocksize > 1:
+                        layer.mask.blockify(h.blocksize)
+                    layer.state.mult(layer.mask)
+            elif not h.mult_dropout:
+                layer.state.mult(1.0 - h.dropout_prob)      # the expected output
+        return None
+
+    def ComputeDown(self, layer, step):
+        """Back-propagate through ``layer``: its deriv holds the gradient w.r.t. its outputs on
+        entry and w.r.t. its inputs afterwards; send it down every incoming edge and update the
+        parameters of those edges and of the layer."""
+        if layer.is_input:
+            return None
+        if layer.is_output:
+            loss = layer.GetLoss(get_deriv=True)
+        else:
+            loss = None
+            layer.ComputeDeriv()
+        for edge in layer.incoming_edge:
+            if edge.conv or edge.local:
+                AccumulateConvDeriv(edge.node1, edge, layer.deriv)
+            else:
+                self.AccumulateDeriv(edge.node1, edge, layer.deriv)
+            self.UpdateEdgeParams(edge, layer.deriv, step)
+        self.UpdateLayerParams(layer, step)
+        return loss
+
+    def AccumulateDeriv(self, layer, edge, deriv):
+        if layer.is_input or edge.proto.block_gradient:
+            return
+        if layer.dirty:
+            layer.deriv.add_dot(edge.params['weight'], deriv)
+        else:
+            cm.dot(edge.params['weight'], deriv, target=layer.deriv)
+            layer.dirty = True
+
+    def UpdateEdgeParams(self, edge, deriv, step):
+        numcases = edge.node1.batchsize
+        if edge.conv or edge.local:
+            ConvOuter(edge, edge.temp)
+            edge.gradient.add_mult(edge.temp, mult=1.0 / numcases)
+        else:
+            edge.gradient.add_dot(edge.node1.state, deriv.T, mult=1.0 / numcases)
+        edge.num_grads_received += 1
+        if edge.num_grads_received == edge.num_shares:
+            edge.Update('weight', step)
+
+    def UpdateLayerParams(self, layer, step):
+        layer.gradient.add_sums(layer.deriv, axis=1, mult=1.0 / layer.batchsize)
+        layer.num_grads_received += 1
+        if layer.num_grads_received == layer.num_shares:
+            layer.Update('bias', step, no_reg=True)     # the bias is not regularised
+
+    def ForwardPropagate(self, train=False, step=0):
+        losses = []
+        for node in self.node_list:
+            loss = self.ComputeUp(node, train, step, self.train_stop_steps)
+            if loss:
+                losses.append(loss)
+        return losses
+
+    def BackwardPropagate(self, step):
+        losses = []
+        for node in reversed(self.node_list):
+            loss = self.ComputeDown(node, step)
+            if loss:
+                losses.append(loss)
+        return losses
+
+    def TrainOneBatch(self, step):
+        losses = self.ForwardPropagate(train=True)
+        losses.extend(self.BackwardPropagate(step))
+        return losses
+
+    def EvaluateOneBatch(self):
+        losses = self.ForwardPropagate()
+        losses.extend([node.GetLoss() for node in self.output_datalayer])
+        return losses

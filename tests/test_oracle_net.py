@@ -1,0 +1,141 @@
+"""CPU-only pins of the training-step restatement (oracle/net_oracle.py): gradients and k
+steps of momentum SGD against torch.autograd / torch.optim.SGD on the same model, the update
+rule's optional terms against explicit formulas, the schedules against closed forms."""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as TF
+
+from oracle import conv_oracle as co
+from oracle import net_oracle as no
+
+
+class _Cv(object):
+    def __init__(self, **kw):
+        self.size = self.stride = self.padding = self.num_filters = self.num_colors = 0
+        self.max_pool, self.pool_size, self.pool_stride, self.prob = False, 0, 0, False
+        self.rnorm, self.norm_size, self.pow_scale, self.add_scale = False, 0, 0.75, 0.001
+        self.__dict__.update(kw)
+
+
+def _half_slope_tanh(x):
+    """tanh whose backward pass has half the slope, like the reference's kTanhDeriv
+    (cudamat_kernels.cu:663-669: a * (1 + b) * (1 - b) * 0.5)."""
+    y = 0.5 * torch.tanh(x)
+    return y + y.detach()
+
+
+def _torch_act(act, x):
+    return {'LOGISTIC': torch.sigmoid, 'TANH': _half_slope_tanh, 'RECTIFIED_LINEAR': torch.relu,
+            'LINEAR': lambda t: t}[act](x)
+
+
+@pytest.mark.parametrize("hidden,loss", [('RECTIFIED_LINEAR', 'softmax'), ('LOGISTIC', 'softmax'), ('TANH', 'logistic_ce'),
+                                         ('RECTIFIED_LINEAR', 'linear_sq')])
+def test_dense_net_steps_equal_torch_sgd(rng, hidden, loss):
+    sizes, B, steps = (12, 9, 7, 5), 6, 4
+    mom, eps, l2 = 0.9, 0.05, 0.01
+    # float32-representable hyper-parameters, so that both sides use the same numbers
+    mom, eps, l2 = (float(np.float32(v)) for v in (mom, eps, l2))
+    he = no.Hyper(base_epsilon=eps, initial_momentum=mom, final_momentum=mom, apply_l2_decay=True, l2_decay=l2)
+    hl = no.Hyper(base_epsilon=eps, initial_momentum=mom, final_momentum=mom)
+    hd = no.Hyper(base_epsilon=eps, initial_momentum=mom, final_momentum=mom, dropout=True, dropout_prob=0.5)
+    out_act = {'softmax': 'SOFTMAX', 'logistic_ce': 'LOGISTIC', 'linear_sq': 'LINEAR'}[loss]
+    Ws = [0.3 * rng.standard_normal((sizes[i], sizes[i + 1])) for i in range(3)]
+    bs = [0.1 * rng.standard_normal((sizes[i + 1], 1)) for i in range(3)]
+    layers = [{'act': 'LINEAR', 'hyper': hl},
+              {'act': hidden, 'hyper': hd, 'bias': bs[0], 'edge': {'w': Ws[0], 'hyper': he}},
+              {'act': hidden, 'hyper': hl, 'bias': bs[1], 'edge': {'w': Ws[1], 'hyper': he}},
+              {'act': out_act, 'hyper': hl, 'bias': bs[2], 'edge': {'w': Ws[2], 'hyper': he},
+               'loss': 'SQUARED_LOSS' if loss == 'linear_sq' else 'CROSS_ENTROPY'}]
+    net = no.Net(layers)
+    tw = [torch.tensor(w, requires_grad=True) for w in Ws]
+    tb = [torch.tensor(b, requires_grad=True) for b in bs]
+    opt = torch.optim.SGD([{'params': tw, 'weight_decay': l2}, {'params': tb, 'weight_decay': 0.0}], lr=eps, momentum=mom)
+    for step in range(steps):
+        x = rng.standard_normal((sizes[0], B))
+        mask = (rng.random((sizes[1], B)) > 0.5).astype(np.float64)
+        if loss == 'softmax':
+            targets = rng.integers(0, sizes[-1], (1, B)).astype(np.float64)
+        elif loss == 'logistic_ce':
+            targets = (rng.random((sizes[-1], B)) < 0.5).astype(np.float64)
+        else:
+            targets = rng.standard_normal((sizes[-1], B))
+        perf = net.train_step(x, targets, step, masks=[None, mask, None, None])
+        # the same step in torch: mean loss over the batch gives deepnet's 1/B gradients
+        opt.zero_grad()
+        h = torch.tensor(x)
+        h = _torch_act(hidden, tw[0].T @ h + tb[0]) * torch.tensor(mask)
+        h = _torch_act(hidden, tw[1].T @ h + tb[1])
+        z = tw[2].T @ h + tb[2]
+        if loss == 'softmax':
+            L = TF.cross_entropy(z.T, torch.tensor(targets.ravel()).long(), reduction='sum')
+            assert abs(perf['cross_entropy'] - float(L.detach())) < 1e-6 * max(1.0, abs(float(L.detach())))
+        elif loss == 'logistic_ce':
+            L = TF.binary_cross_entropy_with_logits(z, torch.tensor(targets), reduction='sum')
+            assert abs(perf['cross_entropy'] - float(L.detach())) < 1e-6 * max(1.0, abs(float(L.detach())))
+        else:
+            L = 0.5 * ((z - torch.tensor(targets)) ** 2).sum()
+            assert abs(perf['error'] - 2 * float(L.detach())) < 1e-9 * max(1.0, float(L.detach()))
+        (L / B).backward()
+        opt.step()
+        for i in range(3):
+            assert np.allclose(net.layers[i + 1]['edge']['w'], tw[i].detach().numpy(), rtol=0, atol=1e-12), (step, i)
+            assert np.allclose(net.layers[i + 1]['bias'], tb[i].detach().numpy(), rtol=0, atol=1e-12), (step, i)
+
+
+def test_conv_net_steps_equal_torch_sgd(rng):
+    """input 2x8x8 -> conv 3x3 pad 1 (8 filters) + pool 2/2 -> ReLU -> dense softmax."""
+    N, C, H, F, k, classes = 5, 2, 8, 16, 3, 4
+    cv = _Cv(size=k, stride=1, padding=1, num_filters=F, num_colors=C, max_pool=True, pool_size=2, pool_stride=2)
+    mom, eps = float(np.float32(0.5)), float(np.float32(0.1))
+    h = no.Hyper(base_epsilon=eps, initial_momentum=mom, final_momentum=mom)
+    wc, bc = 0.3 * rng.standard_normal((F, C * k * k)), 0.1 * rng.standard_normal((F * 16, 1))
+    wd, bd = 0.1 * rng.standard_normal((F * 16, classes)), np.zeros((classes, 1))
+    net = no.Net([{'act': 'LINEAR', 'hyper': h},
+                  {'act': 'RECTIFIED_LINEAR', 'hyper': h, 'bias': bc, 'edge': {'w': wc, 'hyper': h, 'cv': cv}},
+                  {'act': 'SOFTMAX', 'hyper': h, 'bias': bd, 'edge': {'w': wd, 'hyper': h}, 'loss': 'CROSS_ENTROPY'}])
+    t = [torch.tensor(a, requires_grad=True) for a in (wc, bc, wd, bd)]
+    opt = torch.optim.SGD(t, lr=eps, momentum=mom)
+    for step in range(3):
+        x = rng.standard_normal((C * H * H, N))
+        labels = rng.integers(0, classes, (1, N)).astype(np.float64)
+        net.train_step(x, labels, step)
+        opt.zero_grad()
+        xt = torch.tensor(co.to_nchw(x.T, C, H))
+        a = TF.max_pool2d(TF.conv2d(xt, t[0].reshape(F, C, k, k), padding=1), 2, 2)       # (N, F, 4, 4)
+        a = torch.relu(a.reshape(N, -1).T + t[1])                                           # (F*16, N), deepnet's order
+        z = t[2].T @ a + t[3]
+        (TF.cross_entropy(z.T, torch.tensor(labels.ravel()).long(), reduction='sum') / N).backward()
+        opt.step()
+        got = [net.layers[1]['edge']['w'], net.layers[1]['bias'], net.layers[2]['edge']['w'], net.layers[2]['bias']]
+        for g, want in zip(got, t):
+            assert np.allclose(g, want.detach().numpy(), rtol=0, atol=1e-12), step
+
+
+def test_update_rule_optional_terms_and_schedules(rng):
+    w, v, g = rng.standard_normal((6, 4)), rng.standard_normal((6, 4)), rng.standard_normal((6, 4))
+    h = no.Hyper(base_epsilon=0.5, initial_momentum=0.5, final_momentum=0.75, momentum_change_steps=10,
+                 apply_l1_decay=True, l1_decay=0.25, apply_l1decay_after=3, apply_weight_norm=True, weight_norm=1.5,
+                 epsilon_decay='INVERSE_T', epsilon_decay_half_life=8, start_learning_after=2)
+    # schedules: momentum rises from initial to final with time constant momentum_change_steps
+    m0, e0 = no.momentum_and_epsilon(h, 0)
+    assert m0 == 0.5 and e0 == 0.0                              # no learning before start_learning_after
+    m10, e8 = no.momentum_and_epsilon(h, 10)[0], no.momentum_and_epsilon(h, 8)[1]
+    assert abs(m10 - (0.75 - 0.25 * np.exp(-1.0))) < 1e-7 and e8 == 0.25   # half life: epsilon halves at step 8
+    h2 = no.Hyper(base_epsilon=0.5, epsilon_decay='EXPONENTIAL', epsilon_decay_half_life=8)
+    assert no.momentum_and_epsilon(h2, 16)[1] == 0.125
+    # step 3: the L1 term is not yet applied (step > apply_l1decay_after); step 4: it is
+    for step, l1_on in ((3, False), (4, True)):
+        m, e = no.momentum_and_epsilon(h, step)
+        v2 = m * v + (0.25 * np.sign(w) if l1_on else 0.0) + g
+        w2 = w - e * v2
+        n = np.sqrt((w2 ** 2).sum(axis=0))
+        w2 = w2 * np.where(n > 1.5, 1.5 / n, 1.0)
+        gw, gv = no.update(h, w, v, g, step)
+        assert np.allclose(gv, v2, atol=1e-14) and np.allclose(gw, w2, atol=1e-14)
+        assert np.all(np.sqrt((gw ** 2).sum(axis=0)) <= 1.5 + 1e-12)
+    # no_reg (the bias): neither decay nor the norm limit
+    gw, gv = no.update(h, w, v, g, 9, no_reg=True)
+    m, e = no.momentum_and_epsilon(h, 9)
+    assert np.allclose(gv, m * v + g, atol=1e-14) and np.allclose(gw, w - e * (m * v + g), atol=1e-14)
