@@ -63,24 +63,27 @@ __global__ void k_blockify(const float* source, float* target, int numdims, int 
 
 // One column = one image of source_w x source_w pixels with num_channels
 // interleaved channels; crop a target_w x target_w window shifted by
-// (off_x, off_y) from the centred position.
+// (off_x, off_y) from the centred position.  The source pixel is addressed the way
+// the reference does it (cudamat_kernels.cu:795-817): a flat pixel index
+// img*S*S + (pad + off_x + tx)*S + (pad + off_y + ty), so a window that leaves the image
+// on the right continues in the next pixel row, and one that leaves it at the bottom in
+// the next image -- deepnet's data cache relies on nothing else, but its offsets do reach
+// there (datahandler.py:350-352 adds the centring shift that the kernel adds again).
+// Only an index outside the whole source matrix reads 0 instead of foreign memory.
 __global__ void k_translate(const float* source, float* target, const float* off_x_arr, const float* off_y_arr,
-                            int source_w, int target_w, int num_channels) {
+                            int source_w, int target_w, int num_channels, long long total) {
   const int img = blockIdx.x;
   const int pad = (source_w - target_w) / 2;
   const int tts = target_w * target_w, sts = source_w * source_w;
   const int off_x = (int)off_x_arr[img], off_y = (int)off_y_arr[img];
   const long long target_off = (long long)img * tts;
-  const long long source_off = (long long)img * sts;
+  const long long source_off = (long long)img * sts + (long long)(pad + off_x) * source_w + (pad + off_y);
   const int per_img = tts * num_channels;
   for (int e = threadIdx.x; e < per_img; e += blockDim.x) {
     const int pix = e / num_channels, ch = e - pix * num_channels;
     const int tx = pix / target_w, ty = pix - tx * target_w;
-    const int sx = pad + off_x + tx, sy = pad + off_y + ty;
-    // A window pushed past the image edge reads zeros instead of neighbouring memory.
-    const bool inside = sx >= 0 && sx < source_w && sy >= 0 && sy < source_w;
-    target[num_channels * (target_off + pix) + ch] =
-        inside ? source[num_channels * (source_off + (long long)sx * source_w + sy) + ch] : 0.f;
+    const long long src = num_channels * (source_off + (long long)tx * source_w + ty) + ch;
+    target[num_channels * (target_off + pix) + ch] = (src >= 0 && src < total) ? source[src] : 0.f;
   }
 }
 
@@ -178,7 +181,7 @@ int generate_translations_big_var_off(cudamat* source, cudamat* target, cudamat*
   if (imgs == 0) return 0;
   hipLaunchKernelGGL(k_translate, dim3(imgs), dim3(512), 0, 0, (const float*)source->data_device, target->data_device,
                      (const float*)off_x->data_device, (const float*)off_y->data_device, source_w, target_w,
-                     num_channels);
+                     num_channels, (long long)imgs * source->size[0]);
   return dn_launch_status();
 }
 

@@ -386,16 +386,23 @@ def accumulate_columns(mat, indices, target_width, mult, avg):
 
 
 def generate_translations(src, source_w, target_w, off_x, off_y, num_channels):
-    """cudamat_kernels.cu:795-817: column = image, pixels row-major with channels
-    interleaved; crop target_w^2 at (pad+off_x, pad+off_y)."""
+    """cudamat_kernels.cu:795-817: column = image, pixels row-major with channels interleaved;
+    target pixel (tx, ty) of image b comes from the flat pixel index
+    b*S*S + (pad + off_x + tx)*S + (pad + off_y + ty) of the whole source matrix, so a window
+    leaving the image continues in the next pixel row / the next image.  An index outside the
+    matrix (the reference reads foreign memory there) gives 0."""
     src = _a(src)
     n = src.shape[1]
+    flat = src.ravel(order='F')
     pad = (source_w - target_w) // 2
+    tx, ty = np.meshgrid(np.arange(target_w), np.arange(target_w), indexing='ij')
     out = np.zeros((target_w * target_w * num_channels, n))
     for b in range(n):
-        img = src[:, b].reshape(source_w, source_w, num_channels)
         ox, oy = int(np.asarray(off_x).ravel()[b]), int(np.asarray(off_y).ravel()[b])
-        out[:, b] = img[pad + ox:pad + ox + target_w, pad + oy:pad + oy + target_w, :].ravel()
+        pix = b * source_w * source_w + (pad + ox + tx) * source_w + (pad + oy + ty)          # (target_w, target_w)
+        idx = (num_channels * pix[..., None] + np.arange(num_channels)).ravel()
+        ok = (idx >= 0) & (idx < flat.size)
+        out[:, b] = np.where(ok, flat[np.clip(idx, 0, flat.size - 1)], 0.0)
     return out
 
 

@@ -142,3 +142,8 @@ def test_blockify_expand_accumulate_translations(cm, rng):
     ox = np.array([[0, 1, -1, 1, 0]], dtype=np.float32); oy = np.array([[0, -1, 1, 1, -1]], dtype=np.float32)
     tr = cm.CUDAMatrix(imgs).generate_translations(8, 6, cm.CUDAMatrix(ox), cm.CUDAMatrix(oy))
     assert np.array_equal(tr.asarray(), orc.generate_translations(imgs, 8, 6, ox, oy, 3).astype(np.float32))
+    # offsets that push the window out of the image: the next pixel row / next image, 0 past the matrix
+    ox = np.array([[2, 3, -2, 0, 3]], dtype=np.float32); oy = np.array([[3, 0, -3, 2, 3]], dtype=np.float32)
+    tr = cm.CUDAMatrix(imgs).generate_translations(8, 6, cm.CUDAMatrix(ox), cm.CUDAMatrix(oy))
+    want = orc.generate_translations(imgs, 8, 6, ox, oy, 3).astype(np.float32)
+    assert np.array_equal(tr.asarray(), want) and (want[:, 4] == 0).any() and (want[:, 0] != 0).all()

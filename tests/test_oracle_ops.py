@@ -112,6 +112,13 @@ def test_gather_scatter_semantics(rng):
     tr = orc.generate_translations(imgs, 4, 2, np.array([[0, 1]]), np.array([[0, -1]]), 1)
     assert np.array_equal(tr[:, 0], imgs[:, 0].reshape(4, 4)[1:3, 1:3].ravel())
     assert np.array_equal(tr[:, 1], imgs[:, 1].reshape(4, 4)[2:4, 0:2].ravel())
+    # a window leaving the image: flat pixel addressing (cudamat_kernels.cu:807,814).  Image 0 is pixels
+    # 0..15, image 1 pixels 16..31 of the matrix; pad = 1.  Offsets (1, 2): origin row 2, column 3, so the
+    # second column of the window is column 4 = column 0 of the next row.
+    tr = orc.generate_translations(imgs, 4, 2, np.array([[1, 2]]), np.array([[2, 2]]), 1)
+    assert tr[:, 0].tolist() == [11.0, 12.0, 15.0, 16.0]          # pixel 16 already belongs to image 1
+    # image 1, origin row 3: its second window row lies beyond the matrix -> 0 (foreign memory in the reference)
+    assert tr[:, 1].tolist() == [16 + 15.0, 0.0, 0.0, 0.0]
 
 
 def test_ulp_helper():
