@@ -378,6 +378,25 @@ def cpu_baseline_rbm(steps=100):
     return out
 
 
+def cpu_baseline_conv_c4():
+    """One run of each conv pass of config 4 through the float64 numpy restatement (patch
+    views + tensordot; numpy's own threading): the reference's CPU library has no convolution,
+    so this is the only CPU figure there is to put beside the conv kernels."""
+    from oracle import conv_oracle as co
+    rng = np.random.default_rng(4)
+    N, C, H, F, k, p = 128, 3, 32, 64, 5, 2
+    x = rng.standard_normal((N, C * H * H)).astype(np.float32)
+    w = (0.01 * rng.standard_normal((F, C * k * k))).astype(np.float32)
+    y = rng.standard_normal((N, F * H * H)).astype(np.float32)
+    out = {}
+    for name, fn in (('convUp', lambda: co.conv_up(x, w, C, H, p, 1)), ('convDown', lambda: co.conv_down(y, w, C, H, p, 1)),
+                     ('convOutp', lambda: co.conv_outp(x, y, C, H, k, p, 1))):
+        t0 = time.perf_counter()
+        fn()
+        out[name] = round((time.perf_counter() - t0) * 1e3, 1)
+    return out
+
+
 # ---------------------------------------------------------------- main
 
 def main():
@@ -508,6 +527,7 @@ def main():
             cb['rbm_cd1_steps_per_sec'] = {'threads_%d' % k: round(v, 2) for k, v in r.items()}
             if 'rbm_cd1' in secondary:
                 secondary['rbm_cd1']['vs_cpu_1thread'] = round(secondary['rbm_cd1']['steps_per_sec'] / r[1], 1)
+            cb['conv_c4_numpy_f64_ms'] = cpu_baseline_conv_c4()
         line['cpu_baseline'] = cb
     print(json.dumps(line))
 

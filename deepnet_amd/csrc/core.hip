@@ -77,6 +77,38 @@ __global__ void __launch_bounds__(256) k_transpose(const float* in, float* out, 
   }
 }
 
+// The same for 16-byte aligned matrices whose sides are multiples of 4: every lane moves
+// 16 bytes per access on both sides (a quarter of the memory instructions; the transposes
+// of the conv stage are latency-bound), the tile is turned around in LDS one float at a
+// time.  Lane t: 4 consecutive rows 4*(t%16).. of column t/16 + 16*u on the way in,
+// 4 consecutive columns of row t/16 + 16*u of the tile on the way out.
+__global__ void __launch_bounds__(256) k_transpose4(const float* in, float* out, int h, int w) {
+  __shared__ float tile[TR_TILE][TR_TILE + 1];   // [column][row]
+  const int q = (threadIdx.x & 15) * 4, p = threadIdx.x >> 4;
+  const int r0 = blockIdx.x * TR_TILE, c0 = blockIdx.y * TR_TILE;
+  float4 v[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int r = r0 + q, c = c0 + p + 16 * u;
+    v[u] = (r < h && c < w) ? *reinterpret_cast<const float4*>(in + (size_t)c * h + r) : make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    float* t = &tile[p + 16 * u][q];
+    t[0] = v[u].x; t[1] = v[u].y; t[2] = v[u].z; t[3] = v[u].w;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int r = r0 + p + 16 * u, c = c0 + q;     // out(c, r) = in(r, c), contiguous along c
+    if (r < h && c < w) {
+      const int lr = p + 16 * u;
+      *reinterpret_cast<float4*>(out + (size_t)r * w + c) =
+          make_float4(tile[q][lr], tile[q + 1][lr], tile[q + 2][lr], tile[q + 3][lr]);
+    }
+  }
+}
+
 // ------------------------------------------------------------------ C ABI
 
 extern "C" {
@@ -272,7 +304,10 @@ int copy_transpose(cudamat* source, cudamat* target) {
   if (source->size[0] != target->size[1] || source->size[1] != target->size[0]) return ERROR_INCOMPATIBLE_DIMENSIONS;
   if (height == 0 || width == 0) return 0;
   dim3 grid((height + TR_TILE - 1) / TR_TILE, (width + TR_TILE - 1) / TR_TILE);
-  hipLaunchKernelGGL(k_transpose, grid, dim3(256), 0, 0, source->data_device, target->data_device, height, width);
+  if (height % 4 == 0 && width % 4 == 0 && dn_aligned16(source->data_device) && dn_aligned16(target->data_device))
+    hipLaunchKernelGGL(k_transpose4, grid, dim3(256), 0, 0, source->data_device, target->data_device, height, width);
+  else
+    hipLaunchKernelGGL(k_transpose, grid, dim3(256), 0, 0, source->data_device, target->data_device, height, width);
   return dn_launch_status();
 }
 

@@ -41,7 +41,8 @@ def test_empty_matrices_are_harmless(cm):
 
 
 def test_copy_transpose(cm, rng):
-    for shape in [(256, 128), (37, 53), (1, 9), (9, 1), (3072, 128), (65, 64)]:
+    for shape in [(256, 128), (37, 53), (1, 9), (9, 1), (3072, 128), (65, 64), (128, 14400), (14400, 128), (68, 132),
+                  (4, 4), (132, 4), (60, 200)]:        # (multiples of 4 take the 16-byte kernel, ragged tiles included)
         x = _rand(rng, shape)
         a = cm.CUDAMatrix(x)
         t = a.transpose()
@@ -51,6 +52,10 @@ def test_copy_transpose(cm, rng):
         assert np.array_equal(t2.asarray(), x.T)
     with pytest.raises(cm.CUDAMatException):
         a.transpose(target=cm.empty((5, 5)))
+    # a source view that starts off a 16-byte boundary (column 1 of a 3-row parent) takes the scalar kernel
+    x = _rand(rng, (3, 17))
+    view = cm.CUDAMatrix(x).slice(1, 17).reshape((4, 12))
+    assert np.array_equal(view.transpose().asarray(), x[:, 1:].reshape((4, 12), order='F').T)
 
 
 def test_column_slices_alias_the_parent(cm, rng):
