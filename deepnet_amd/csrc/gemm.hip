@@ -540,6 +540,10 @@ static int gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, co
     long long want = (2ll * cus + tiles - 1) / tiles;
     if (want > kslabs / 4) want = kslabs / 4;  // at least 4 slabs (64 deep) per slice
     if (want > 32) want = 32;
+    // The second kernel costs about 5 us and a split slice starts its pipeline anew: measured
+    // on 1024 x 1024 outputs a split only pays from K = 2048 on (K = 128: 13 us split, 7.5 us
+    // whole), and with 1.5 tiles per CU (1280 x 1280) it never does.
+    if (K < 2048 || tiles * 4 >= (long long)cus * 5) want = 1;
     if (want > 1) splits = (int)want;
   }
   int kps = ((K + splits - 1) / splits + GEMM_BK - 1) / GEMM_BK * GEMM_BK;

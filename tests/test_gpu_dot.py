@@ -117,6 +117,24 @@ def test_large_square_products(cm, rng, n):
         h.free_device_memory()
 
 
+@pytest.mark.parametrize("ta,tb", [(False, False), (True, False), (False, True), (True, True)])
+def test_split_k_products(cm, rng, ta, tb):
+    """About one 64 x 64 tile per CU and K >= 2048: the reduction is split over two workgroups
+    per tile and summed by a second kernel, with alpha and beta applied there."""
+    m, n, k = 1024, 1040, 2500
+    A = np.asarray(rng.uniform(-1, 1, (k, m) if ta else (m, k)), dtype=np.float32, order='F')
+    B = np.asarray(rng.uniform(-1, 1, (n, k) if tb else (k, n)), dtype=np.float32, order='F')
+    C = np.asarray(rng.uniform(-1, 1, (m, n)), dtype=np.float32, order='F')
+    a, b, c = cm.CUDAMatrix(A), cm.CUDAMatrix(B), cm.CUDAMatrix(C)
+    c.add_dot(a.T if ta else a, b.T if tb else b, mult=-0.75)
+    opa = (A.T if ta else A).astype(np.float64); opb = (B.T if tb else B).astype(np.float64)
+    want = C.astype(np.float64) - 0.75 * (opa @ opb)
+    bound = np.abs(C).astype(np.float64) + 0.75 * (np.abs(opa) @ np.abs(opb))
+    assert np.max(np.abs(c.asarray() - want) / bound) < REL
+    for h in (a, b, c):
+        h.free_device_memory()
+
+
 # ---- the fused extension: dot -> add_col_vec -> activation in one call
 
 @pytest.mark.parametrize("m,n,k,ta,tb", [
@@ -124,7 +142,8 @@ def test_large_square_products(cm, rng, n):
     (784, 100, 500, False, False),     # RBM down pass
     (1024, 128, 784, True, False),     # MLP layer
     (10, 128, 1024, True, False),      # MLP output layer (fewer rows than a tile)
-    (300, 700, 96, False, True),       # mid-sized: split-K path, falls back to separate launches
+    (300, 700, 96, False, True),       # mid-sized: the single-launch kernel
+    (1024, 1024, 2304, True, False),   # one 64 x 64 tile per CU and a long K: split-K, falls back to separate launches
     (2048, 2048, 64, False, False),    # big tiles, fused epilogue
     (37, 1, 50, False, False),         # one output column: matrix-vector kernel
 ])
