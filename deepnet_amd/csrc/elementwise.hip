@@ -156,7 +156,7 @@ static int launch_ew(const float* a, const float* b, float* t, long long n, F f)
 // columns (vec[i / h], a row vector) into a flat pass over the matrix.  The
 // row / column of the first element of each 16-byte group comes from one
 // multiply-high; the other three follow by increment-and-wrap.
-template <bool COLVEC, bool STREAM, class F>
+template <bool COLVEC, bool STREAM, bool VEC4, class F>
 __global__ void __launch_bounds__(EW_THREADS)
 k_bcast(const float* a, const float* vec, float* t, long long n, int head, long long n4, FastDiv fd, F f) {
   const long long tid = (long long)blockIdx.x * EW_THREADS + threadIdx.x;
@@ -168,10 +168,17 @@ k_bcast(const float* a, const float* vec, float* t, long long n, int head, long 
     uint32_t r = e - q * h;
     float v[4];
     const float x[4] = {va.x, va.y, va.z, va.w};
+    if constexpr (VEC4) {
+      // COLVEC, no head, h a multiple of 4, aligned vector: the four rows are one 16-byte
+      // group of the vector and never wrap into the next column
+      const float4 vv = *reinterpret_cast<const float4*>(vec + r);
+      v[0] = f(x[0], vv.x); v[1] = f(x[1], vv.y); v[2] = f(x[2], vv.z); v[3] = f(x[3], vv.w);
+    } else {
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      v[k] = f(x[k], vec[COLVEC ? r : q]);
-      if (++r == h) { r = 0; ++q; }
+      for (int k = 0; k < 4; ++k) {
+        v[k] = f(x[k], vec[COLVEC ? r : q]);
+        if (++r == h) { r = 0; ++q; }
+      }
     }
     dn_st4<STREAM>(t + e, make_float4(v[0], v[1], v[2], v[3]));
   }
@@ -210,12 +217,16 @@ static int launch_bcast(const float* a, const float* vec, float* t, int h, int w
     const long long n4 = (n - head) / 4;
     long long blocks = (n4 + EW_THREADS - 1) / EW_THREADS;
     if (blocks < 1) blocks = 1;
-    if (n >= DN_STREAM_MIN_ELEMS)
-      hipLaunchKernelGGL((k_bcast<COLVEC, true, F>), dim3((unsigned)blocks), dim3(EW_THREADS), 0, 0, a, vec, t, n,
-                         head, n4, fd, f);
-    else
-      hipLaunchKernelGGL((k_bcast<COLVEC, false, F>), dim3((unsigned)blocks), dim3(EW_THREADS), 0, 0, a, vec, t, n,
-                         head, n4, fd, f);
+    const bool vec4 = COLVEC && head == 0 && h % 4 == 0 && dn_aligned16(vec);
+#define BCAST_LAUNCH(ST, V4)                                                                                  \
+  hipLaunchKernelGGL((k_bcast<COLVEC, ST, V4, F>), dim3((unsigned)blocks), dim3(EW_THREADS), 0, 0, a, vec, t, n, \
+                     head, n4, fd, f)
+    if (n >= DN_STREAM_MIN_ELEMS) {
+      if (vec4) BCAST_LAUNCH(true, COLVEC); else BCAST_LAUNCH(true, false);
+    } else {
+      if (vec4) BCAST_LAUNCH(false, COLVEC); else BCAST_LAUNCH(false, false);
+    }
+#undef BCAST_LAUNCH
   } else {
     long long blocks = (n + EW_THREADS - 1) / EW_THREADS;
     const long long cap = (long long)cus * 32;
