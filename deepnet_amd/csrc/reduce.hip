@@ -166,6 +166,19 @@ __global__ void __launch_bounds__(256) k_col_normlimit(const float* mat, float* 
   for_each_in_col<TPC>(c, h, lane, [&](int r, float v) { t[r] = v * scale; });
 }
 
+// e^t for t <= 0 in softmax: t*log2(e) as a two-term product (the rounding of the first
+// term and the tail of the constant go into a correction factor), then the hardware exp2.
+// Relative error about 1.5 ulp over the whole range, against the 1e-5 these outputs are
+// held to; a result below the normal range may come out as 0.  t = -inf gives 0, NaN stays NaN.
+__device__ __forceinline__ float softmax_exp(float t) {
+  t = t < -128.f ? -128.f : t;      // (e^-128 is 0 in fp32; keeps -inf out of the correction term)
+  const float L2E = 1.44269502162933349609375f, L2E_LO = 1.925963033500011e-08f;
+  const float p = t * L2E;
+  const float lo = __fmaf_rn(t, L2E_LO, __fmaf_rn(t, L2E, -p));
+  const float e = __builtin_amdgcn_exp2f(p);
+  return __fmaf_rn(e, lo * 0.693147182464599609375f, e);
+}
+
 // Column softmax: max, sum of exp(x - max), divide (cudamat_kernels.cu:868-934).
 // The column is re-read from cache for the second and third pass.
 // Optional extras of the fused loss step (all three null for plain softmax): with
@@ -188,16 +201,17 @@ __global__ void __launch_bounds__(256) k_col_softmax(const float* mat, float* ta
   if (active) for_each_in_col<TPC>(c, h, lane, [&](int, float v) { if (v > m) m = v; });
   m = col_combine<TPC, true>(m, lds4);
   float s = 0.f;
-  if (active) for_each_in_col<TPC>(c, h, lane, [&](int, float v) { s += expf(v - m); });
+  if (active) for_each_in_col<TPC>(c, h, lane, [&](int, float v) { s += softmax_exp(v - m); });
   s = col_combine<TPC, false>(s, lds4);
   if (!active) return;
+  const float inv = 1.f / s;
   if (!x.labels) {
-    for_each_in_col<TPC>(c, h, lane, [&](int r, float v) { t[r] = expf(v - m) / s; });
+    for_each_in_col<TPC>(c, h, lane, [&](int r, float v) { t[r] = softmax_exp(v - m) * inv; });
   } else {
     const int label = (int)x.labels[col];
     float* gcol = x.grad ? x.grad + (size_t)col * h : nullptr;
     for_each_in_col<TPC>(c, h, lane, [&](int r, float v) {
-      const float pr = expf(v - m) / s;
+      const float pr = softmax_exp(v - m) * inv;
       t[r] = pr;
       if (gcol) gcol[r] = pr - ((label == r) ? 1.f : 0.f);
       if (x.loss && r == label) x.loss[col] = -logf(pr + x.tiny);
@@ -233,17 +247,18 @@ __global__ void __launch_bounds__(256) k_col_softmax_reg(const float* mat, float
   for (int k = 0; k < NV; ++k) {
     const int j = lane + k * 64;
     if (j < n4) {
-      v[k].x = expf(v[k].x - m); v[k].y = expf(v[k].y - m);
-      v[k].z = expf(v[k].z - m); v[k].w = expf(v[k].w - m);
+      v[k].x = softmax_exp(v[k].x - m); v[k].y = softmax_exp(v[k].y - m);
+      v[k].z = softmax_exp(v[k].z - m); v[k].w = softmax_exp(v[k].w - m);
       s += (v[k].x + v[k].y) + (v[k].z + v[k].w);
     }
   }
   s = wave_sum(s);
+  const float inv = 1.f / s;
 #pragma unroll
   for (int k = 0; k < NV; ++k) {
     const int j = lane + k * 64;
     if (j < n4) {
-      const float4 pr = make_float4(v[k].x / s, v[k].y / s, v[k].z / s, v[k].w / s);
+      const float4 pr = make_float4(v[k].x * inv, v[k].y * inv, v[k].z * inv, v[k].w * inv);
       dn_st4_rt(t4 + 4 * j, pr, stream);
       if (x.labels) {
         const int label = (int)x.labels[col], r0 = 4 * j;

@@ -121,6 +121,23 @@ def test_softmax(cm, rng, shape):
     assert np.array_equal(a.asarray(), got)
 
 
+@pytest.mark.parametrize("h", [64, 37])          # columns held in registers / the generic kernel
+def test_softmax_over_wide_ranges_and_masked_entries(cm, rng, h):
+    x = _rand(rng, (h, 40), -60, 60)
+    x[3, :] = -np.inf                               # a masked logit: probability 0, the rest unaffected
+    x[:, 7] *= 1.4                                  # differences down to -168: underflow to 0
+    t = cm.CUDAMatrix(x).apply_softmax(target=cm.empty(x.shape)).asarray()
+    want = orc.softmax(x)
+    assert np.all(t[3, :] == 0) and np.all(np.isfinite(t))
+    big = want > 1e-30
+    assert np.max(np.abs(t[big] - want[big]) / want[big]) < REL
+    assert np.all(t[~big] < 2e-30)
+    assert np.max(np.abs(t.astype(np.float64).sum(axis=0) - 1.0)) < 1e-5
+    x[5, 2] = np.nan                                # NaN is not swallowed
+    t = cm.CUDAMatrix(x).apply_softmax(target=cm.empty(x.shape)).asarray()
+    assert np.all(np.isnan(t[:, 2])) and np.all(np.isfinite(np.delete(t, 2, axis=1)))
+
+
 def test_softmax_loss_helpers(cm, rng):
     x = _rand(rng, (10, 128), -3, 3)
     labels = np.asarray(rng.integers(0, 10, (1, 128)), dtype=np.float32, order='F')
