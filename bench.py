@@ -250,6 +250,20 @@ def net_mlp(cm, sizes=(784, 1024, 1024, 10), B=128, seed=3, fused=False):
     return net
 
 
+def net_rbm(cm, nv=784, nh=500, B=100, lr=0.01, seed=1):
+    """The RBM of config 1 as a two-layer DBM object trained by CD-1: the reference's own control
+    flow (dbm.py:64-282: sufficient statistics, gradient, momentum update, the reconstruction
+    error read back every step)."""
+    from deepnet_amd import dbm, layer as dl, neuralnet as dnn, parameter as dp
+    rng = np.random.default_rng(seed)
+    hyp = lambda **kw: dp.Hyperparams(base_epsilon=lr, **kw)
+    vis = dl.LogisticLayer('visible', nv, B, hyperparams=hyp(activation=dp.LOGISTIC), is_input=True)
+    hid = dl.LogisticLayer('hidden', nh, B, hyperparams=hyp(activation=dp.LOGISTIC))
+    edge = dnn.Edge(vis, hid, 0.01 * rng.standard_normal((nv, nh)), hyperparams=hyp(), directed=False)
+    vis.data.assign(cm.CUDAMatrix(np.asarray(rng.random((nv, B)) < 0.13, dtype=np.float32, order='F')))
+    return dbm.DBM([vis, hid], [edge], optimizer='CD')
+
+
 def time_loop(cm, fn, iters, warmup):
     for _ in range(warmup):
         fn()
@@ -504,6 +518,11 @@ def main():
         secondary['mlp_through_neuralnet_classes'] = {
             'steps_per_sec': round(1.0 / t, 1), 'us_per_step': round(t * 1e6, 1),
             'note': 'same net as Layer / Edge / NeuralNet objects, TrainOneBatch with its two blocking loss read-backs per step'}
+        rbm_net = net_rbm(cm)
+        t = time_loop(cm, lambda: rbm_net.TrainOneBatch(0), 100, 10)
+        secondary['rbm_through_dbm_class'] = {
+            'steps_per_sec': round(1.0 / t, 1), 'us_per_step': round(t * 1e6, 1),
+            'note': 'same RBM as a two-layer DBM object, TrainOneBatch (CD-1) with sufficient statistics, momentum updates and the blocking reconstruction-error read-back'}
         secondary['gemm_fp32_4096'] = gemm_probe(cm, ev)
         try:
             import bench_conv

@@ -45,9 +45,9 @@ class Layer(Parameter):
         self.dirty = False
         self.data = None
         numdims = dimensions * numlabels
-        if not is_input:
-            self.params['bias'] = _zeros((numdims, 1)) if bias is None else cm.CUDAMatrix(
-                np.asarray(bias, dtype=np.float32, order='F').reshape(numdims, 1))
+        self.params['bias'] = _zeros((numdims, 1)) if bias is None else cm.CUDAMatrix(
+            np.asarray(bias, dtype=np.float32, order='F').reshape(numdims, 1))
+        self.sample_input = self.hyperparams.sample_input
         self.AllocateMemory(batchsize)
 
     # ---- graph bookkeeping (layer.py:102-121)
@@ -81,6 +81,24 @@ class Layer(Parameter):
             self.data = _zeros((self.dimensions, batchsize))
         if self.hyperparams.dropout:
             self.mask = _zeros(self.state.shape)
+
+    def AllocateSamplingMemory(self, persistent):
+        """What a layer of a Boltzmann machine holds besides its state (layer.py:176-186): the
+        sufficient statistics, and with persistent chains separate positive / negative states and
+        samples (``state`` / ``sample`` then point at the pair of the current phase)."""
+        numdims = self.dimensions * self.numlabels
+        self.suff_stats = cm.empty((numdims, 1))
+        if persistent:
+            self.pos_state, self.pos_sample = self.state, self.sample
+            self.neg_state, self.neg_sample = _zeros(self.state.shape), _zeros(self.state.shape)
+
+    def CollectSufficientStatistics(self, neg=False):
+        """layer.py:194-205 without the sparsity term: the row sums of the state, added with
+        sign +1 in the positive and -1 in the negative phase."""
+        if not neg:
+            self.state.sum(axis=1, target=self.suff_stats)
+        else:
+            self.suff_stats.add_sums(self.state, axis=1, mult=-1.0)
 
     def SetData(self, data):
         self.data = data

@@ -21,15 +21,16 @@ from .parameter import Parameter, Hyperparams
 class Edge(Parameter):
     """A weight matrix between two layers (deepnet/edge.py:8-35, 83-92).  Dense: ``weight`` is
     (node1 dims, node2 dims).  With ``conv_params``: (num_filters, colours * size^2) shared
-    filters, or one bank per module when ``local``; the conv buffers are those of ConvEdge."""
+    filters, or one bank per module when ``local``; the conv buffers are those of ConvEdge.
+    ``directed=False`` makes the edge incoming and outgoing at both ends."""
 
     def __init__(self, node1, node2, weight, hyperparams=None, conv_params=None, local=False, up_factor=1.0,
-                 block_gradient=False):
+                 block_gradient=False, down_factor=1.0, directed=True):
         super(Edge, self).__init__()
         self.node1, self.node2 = node1, node2
         self.name = '%s:%s' % (node1.name, node2.name)
         self.hyperparams = hyperparams or Hyperparams()
-        self.proto = _EdgeProto(up_factor, block_gradient)
+        self.proto = _EdgeProto(up_factor, block_gradient, down_factor)
         self.tied_to = None
         self.marker = 0
         self.conv = conv_params is not None and not local
@@ -48,16 +49,29 @@ class Edge(Parameter):
         self.AllocateMemory()
         node1.AddOutgoingEdge(self)
         node2.AddIncomingEdge(self)
+        if not directed:              # Boltzmann machines: either end is computed from the other (edge.py:30-38)
+            node1.AddIncomingEdge(self)
+            node2.AddOutgoingEdge(self)
 
     def AllocateMemory(self):
         shape = self.params['weight'].shape
         zeros = lambda: cm.CUDAMatrix(np.zeros(shape, dtype=np.float32, order='F'))
         self.temp, self.gradient, self.gradient_history = zeros(), zeros(), zeros()
 
+    def CollectSufficientStatistics(self, neg=False):
+        """edge.py:222-242 for ordinary units: node1.state node2.state^T, set in the positive
+        phase and subtracted in the negative one."""
+        if not hasattr(self, 'suff_stats'):
+            self.suff_stats = cm.empty(self.params['weight'].shape)
+        if not neg:
+            cm.dot(self.node1.state, self.node2.state.T, target=self.suff_stats)
+        else:
+            self.suff_stats.add_dot(self.node1.state, self.node2.state.T, mult=-1.0)
+
 
 class _EdgeProto(object):
-    def __init__(self, up_factor, block_gradient):
-        self.up_factor, self.block_gradient = up_factor, block_gradient
+    def __init__(self, up_factor, block_gradient, down_factor=1.0):
+        self.up_factor, self.block_gradient, self.down_factor = up_factor, block_gradient, down_factor
 
 
 class NeuralNet(object):

@@ -24,7 +24,8 @@ class Hyperparams(object):
         final_momentum=0.0, momentum_change_steps=10, dropout=False, dropout_prob=0.5, apply_weight_norm=False,
         weight_norm=10.0, apply_l2_decay=False, l2_decay=0.01, activation=LINEAR, stop_dropout_for_last=0,
         start_learning_after=0, apply_l1_decay=False, l1_decay=0.01, apply_l1decay_after=0, blocksize=1,
-        mult_dropout=False, sparsity=False)
+        mult_dropout=False, sparsity=False, mf_steps=1, gibbs_steps=1, step_up_cd_after=0, start_step_up_cd_after=0,
+        sample_input=False, sample_input_after=0)
 
     def __init__(self, **fields):
         unknown = set(fields) - set(self._DEFAULTS)

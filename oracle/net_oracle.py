@@ -172,3 +172,36 @@ class Net(object):
                                                 d.sum(axis=1, keepdims=True) / B, step, no_reg=True)
             d = d_in
         return perf
+
+
+def rbm_cd_step(p, hyper, v_data, step, hid_samples, vis_act='LOGISTIC', hid_act='LOGISTIC'):
+    """One contrastive-divergence step of a two-layer Boltzmann machine as deepnet/dbm.py runs it
+    (PositivePhase :121-152, NegativePhase :186-236 with unsampled inputs, the updates :246-266,
+    sufficient statistics layer.py:194-205 and edge.py:236-242).  p holds float64 'W' (visible x
+    hidden), 'bv', 'bh' (column vectors) and the previous updates 'dW', 'dbv', 'dbh'; hyper the
+    Hyper objects 'edge', 'vis', 'hid'.  hid_samples[i] is the hidden sample that drives Gibbs sweep
+    i (the caller feeds the ones the device drew), so len(hid_samples) sweeps are made.  Returns
+    the squared reconstruction error of the first sweep.
+
+    Pinned by tests/test_oracle_net.py against the C coding of the CD-1 step in
+    oracle/host_backend.c (hb_rbm_cd1_step, written from cudamat/examples/rbm_cudamat.py:46-89)
+    fed the same samples, and by the fixed point W = 0 where every quantity has a closed form."""
+    v = np.asarray(v_data, dtype=F64)
+    B = v.shape[1]
+    W, bv, bh = p['W'], p['bv'], p['bh']
+    h = activate(hid_act, W.T @ v + bh)
+    stats_W, stats_v, stats_h = v @ h.T, v.sum(axis=1, keepdims=True), h.sum(axis=1, keepdims=True)
+    error = None
+    for i, hs in enumerate(hid_samples):
+        v_neg = activate(vis_act, W @ np.asarray(hs, dtype=F64) + bv)
+        if i == 0:
+            error = float(((v_neg - v) ** 2).sum())
+        h_neg = activate(hid_act, W.T @ v_neg + bh)
+    stats_W = stats_W - v_neg @ h_neg.T
+    stats_v = stats_v - v_neg.sum(axis=1, keepdims=True)
+    stats_h = stats_h - h_neg.sum(axis=1, keepdims=True)
+    scale = F64(np.float32(-1.0 / B))
+    p['W'], p['dW'] = update(hyper['edge'], W, p['dW'], scale * stats_W, step)
+    p['bv'], p['dbv'] = update(hyper['vis'], bv, p['dbv'], scale * stats_v, step, no_reg=True)
+    p['bh'], p['dbh'] = update(hyper['hid'], bh, p['dbh'], scale * stats_h, step, no_reg=True)
+    return error

@@ -139,3 +139,43 @@ def test_update_rule_optional_terms_and_schedules(rng):
     gw, gv = no.update(h, w, v, g, 9, no_reg=True)
     m, e = no.momentum_and_epsilon(h, 9)
     assert np.allclose(gv, m * v + g, atol=1e-14) and np.allclose(gw, w - e * (m * v + g), atol=1e-14)
+
+
+def test_rbm_cd_step_against_the_c_coding_and_a_fixed_point(rng):
+    import ctypes as ct
+    import os
+    from oracle import mwc
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    lib = ct.CDLL(os.path.join(root, 'oracle', 'liboracle_host.so'))
+    nv, nh, B, lr = 60, 40, 20, 0.1
+    v = np.asarray(rng.random((nv, B)) < 0.3, dtype=np.float32, order='F')
+    W = np.asarray(0.1 * rng.standard_normal((nv, nh)), dtype=np.float32, order='F')
+    bv = np.asarray(0.1 * rng.standard_normal(nv), dtype=np.float32)
+    bh = np.asarray(0.1 * rng.standard_normal(nh), dtype=np.float32)
+    p = {'W': W.astype(np.float64), 'bv': bv.astype(np.float64).reshape(-1, 1), 'bh': bh.astype(np.float64).reshape(-1, 1)}
+    p.update(dW=np.zeros((nv, nh)), dbv=np.zeros((nv, 1)), dbh=np.zeros((nh, 1)))
+    mults = mwc.load_multipliers(os.path.join(root, 'deepnet_amd', 'rnd_multipliers_32bit.txt'))
+    words = np.empty(mwc.NUM_RND_STREAMS, dtype=np.uint64)
+    fp = ct.POINTER(ct.c_float)
+    u32, u64 = mults.ctypes.data_as(ct.POINTER(ct.c_uint32)), words.ctypes.data_as(ct.POINTER(ct.c_uint64))
+    lib.mwc_seed(u32, u64, ct.c_uint32(5))
+    h, hs, h2 = (np.empty((nh, B), np.float32, order='F') for _ in range(3))
+    v2 = np.empty((nv, B), np.float32, order='F')
+    q = lambda a: a.ctypes.data_as(fp)
+    lib.hb_set_threads(1)
+    lib.hb_rbm_cd1_step(q(W), q(bv), q(bh), q(v), nv, nh, B, ct.c_float(lr), u32, u64, q(h), q(hs), q(v2), q(h2))
+    hyp = no.Hyper(base_epsilon=lr)                       # no momentum, no decay: the example's plain SGD
+    err = no.rbm_cd_step(p, {'edge': hyp, 'vis': hyp, 'hid': hyp}, v, 0, [hs])
+    assert np.allclose(p['W'], W, rtol=1e-5, atol=1e-7)
+    assert np.allclose(p['bv'].ravel(), bv, rtol=1e-5, atol=1e-7) and np.allclose(p['bh'].ravel(), bh, rtol=1e-5, atol=1e-7)
+    assert abs(err - float(((v2.astype(np.float64) - v) ** 2).sum())) < 1e-4 * err
+    # W = 0, zero biases: h = 1/2 everywhere, the reconstruction is 1/2 whatever the samples, so
+    # dW = eps/B * (v - 1/2) (1/2)^T summed over the batch, dbv = eps * (mean(v) - 1/2), dbh = 0
+    z = {'W': np.zeros((nv, nh)), 'bv': np.zeros((nv, 1)), 'bh': np.zeros((nh, 1)),
+         'dW': np.zeros((nv, nh)), 'dbv': np.zeros((nv, 1)), 'dbh': np.zeros((nh, 1))}
+    err = no.rbm_cd_step(z, {'edge': hyp, 'vis': hyp, 'hid': hyp}, v, 0, [hs, 1 - hs])
+    eps = float(np.float32(lr))
+    rowsum = (v.astype(np.float64) - 0.5).sum(axis=1, keepdims=True)
+    assert np.allclose(z['W'], eps / B * 0.5 * rowsum * np.ones((1, nh)), rtol=1e-6, atol=1e-12)
+    assert np.allclose(z['bv'], eps / B * rowsum, rtol=1e-6, atol=1e-12) and np.allclose(z['bh'], 0.0, atol=1e-12)
+    assert abs(err - 0.25 * nv * B) < 1e-9
