@@ -518,11 +518,19 @@ def main():
         secondary['mlp_through_neuralnet_classes'] = {
             'steps_per_sec': round(1.0 / t, 1), 'us_per_step': round(t * 1e6, 1),
             'note': 'same net as Layer / Edge / NeuralNet objects, TrainOneBatch with its two blocking loss read-backs per step'}
+        for obj in net.layer + net.edge:
+            obj.fused = True
+        t = time_loop(cm, lambda: net.TrainOneBatch(0), 100, 10)
+        secondary['mlp_through_neuralnet_classes']['us_per_step_fused_extensions'] = round(t * 1e6, 1)
         rbm_net = net_rbm(cm)
         t = time_loop(cm, lambda: rbm_net.TrainOneBatch(0), 100, 10)
         secondary['rbm_through_dbm_class'] = {
             'steps_per_sec': round(1.0 / t, 1), 'us_per_step': round(t * 1e6, 1),
             'note': 'same RBM as a two-layer DBM object, TrainOneBatch (CD-1) with sufficient statistics, momentum updates and the blocking reconstruction-error read-back'}
+        for obj in rbm_net.layer + rbm_net.edge:
+            obj.fused = True
+        t = time_loop(cm, lambda: rbm_net.TrainOneBatch(0), 100, 10)
+        secondary['rbm_through_dbm_class']['us_per_step_fused_extensions'] = round(t * 1e6, 1)
         secondary['gemm_fp32_4096'] = gemm_probe(cm, ev)
         try:
             import bench_conv

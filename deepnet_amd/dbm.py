@@ -7,7 +7,7 @@ layers and edges of this package.  An RBM is the two-layer case: one input layer
 layer, one edge.  Initialiser nets, sparsity and replicated softmax are not carried over.
 """
 from .choose_matrix_library import cm
-from .neuralnet import NeuralNet
+from .neuralnet import NeuralNet, fused_up
 
 CD, PCD = 'CD', 'PCD'
 
@@ -48,7 +48,14 @@ class DBM(NeuralNet):
         if layer.is_input and not compute_input:
             layer.GetData()
         else:
-            for i, edge in enumerate(layer.incoming_edge):
+            fused = False
+            if len(layer.incoming_edge) == 1:
+                edge, neighbour = layer.incoming_edge[0], layer.incoming_neighbour[0]
+                up = edge.node2 is layer
+                if (edge.proto.up_factor if up else edge.proto.down_factor) == 1:
+                    w = edge.params['weight']
+                    fused = fused_up(layer, w.T if up else w, neighbour.sample if use_samples else neighbour.state)
+            for i, edge in enumerate([] if fused else layer.incoming_edge):
                 neighbour = layer.incoming_neighbour[i]
                 inputs = neighbour.sample if use_samples else neighbour.state
                 if edge.node2 is layer:
@@ -61,8 +68,9 @@ class DBM(NeuralNet):
                         layer.state.mult(factor)
                 else:
                     layer.state.add_dot(w, inputs, mult=factor)
-            layer.state.add_col_vec(layer.params['bias'])
-            layer.ApplyActivation()
+            if not fused:
+                layer.state.add_col_vec(layer.params['bias'])
+                layer.ApplyActivation()
         h = layer.hyperparams
         if h.dropout:
             if train and maxsteps - step >= h.stop_dropout_for_last:

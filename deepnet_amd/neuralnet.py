@@ -15,6 +15,7 @@ import numpy as np
 
 from .choose_matrix_library import cm
 from .convolutions import ConvolveUp, AccumulateConvDeriv, ConvOuter, AddConvolveUp, ConvEdge
+from . import parameter as P
 from .parameter import Parameter, Hyperparams
 
 
@@ -69,6 +70,22 @@ class Edge(Parameter):
             self.suff_stats.add_dot(self.node1.state, self.node2.state.T, mult=-1.0)
 
 
+# Activations the backend's dot_bias_act can apply in the product's epilogue (None: bias only).
+_EPILOGUE = {P.LINEAR: None, P.LOGISTIC: 'sigmoid', P.RECTIFIED_LINEAR: 'relu', P.TANH: 'tanh', P.SOFTMAX: None}
+
+
+def fused_up(layer, w, inputs):
+    """state = activation(w . inputs + bias) in one launch where the layer asks for it
+    (``layer.fused``) and its activation has an epilogue; the same bits as dot, add_col_vec,
+    ApplyActivation.  Returns False when the three calls have to be made."""
+    if not layer.fused or layer.activation not in _EPILOGUE or layer.replicated_neighbour is not None:
+        return False
+    cm.dot_bias_act(w, inputs, layer.params['bias'], target=layer.state, act=_EPILOGUE[layer.activation])
+    if layer.activation == P.SOFTMAX:
+        layer.ApplyActivation()
+    return True
+
+
 class _EdgeProto(object):
     def __init__(self, up_factor, block_gradient, down_factor=1.0):
         self.up_factor, self.block_gradient, self.down_factor = up_factor, block_gradient, down_factor
@@ -106,26 +123,31 @@ class NeuralNet(object):
         if layer.is_input or layer.is_initialized:
             layer.GetData()
         else:
-            for i, edge in enumerate(layer.incoming_edge):
-                if edge in layer.outgoing_edge:
-                    continue
-                inputs = layer.incoming_neighbour[i].state
-                if edge.conv or edge.local:
-                    if i == 0:
-                        ConvolveUp(inputs, edge, layer.state)
+            only = layer.incoming_edge[0] if len(layer.incoming_edge) == 1 else None
+            done = (only is not None and not (only.conv or only.local) and only not in layer.outgoing_edge
+                    and only.proto.up_factor == 1
+                    and fused_up(layer, only.params['weight'].T, layer.incoming_neighbour[0].state))
+            if not done:
+                for i, edge in enumerate(layer.incoming_edge):
+                    if edge in layer.outgoing_edge:
+                        continue
+                    inputs = layer.incoming_neighbour[i].state
+                    if edge.conv or edge.local:
+                        if i == 0:
+                            ConvolveUp(inputs, edge, layer.state)
+                        else:
+                            AddConvolveUp(inputs, edge, layer.state)
                     else:
-                        AddConvolveUp(inputs, edge, layer.state)
-                else:
-                    w = edge.params['weight']
-                    factor = edge.proto.up_factor
-                    if i == 0:
-                        cm.dot(w.T, inputs, target=layer.state)
-                        if factor != 1:
-                            layer.state.mult(factor)
-                    else:
-                        layer.state.add_dot(w.T, inputs, mult=factor)
-            layer.state.add_col_vec(layer.params['bias'])
-            layer.ApplyActivation()
+                        w = edge.params['weight']
+                        factor = edge.proto.up_factor
+                        if i == 0:
+                            cm.dot(w.T, inputs, target=layer.state)
+                            if factor != 1:
+                                layer.state.mult(factor)
+                        else:
+                            layer.state.add_dot(w.T, inputs, mult=factor)
+                layer.state.add_col_vec(layer.params['bias'])
+                layer.ApplyActivation()
         h = layer.hyperparams
         if h.dropout:
             if train and maxsteps - step >= h.stop_dropout_for_last:

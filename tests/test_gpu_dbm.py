@@ -106,6 +106,25 @@ def test_rbm_with_persistent_chains(cm, rng):
         assert vis.state is vis.pos_state and hid.sample is hid.pos_sample      # back in the positive phase
 
 
+def test_fused_route_leaves_the_same_bits(cm):
+    """`fused = True` on layers and edges sends every up pass through dot_bias_act and every
+    update through momentum_update: the parameters after two CD-1 steps are bit-identical."""
+    results = []
+    for fused in (False, True):
+        r = np.random.default_rng(8)
+        cm.CUDAMatrix.init_random(8)
+        kw = dict(base_epsilon=0.05, initial_momentum=0.7, final_momentum=0.7, apply_l2_decay=True, l2_decay=0.002)
+        net, vis, hid, edge, _, _ = _rbm(cm, 200, 120, 40, r, 'CD', 1, kw)
+        for obj in (vis, hid, edge):
+            obj.fused = fused
+        for step in range(2):
+            vis.data.assign(cm.CUDAMatrix(_f(r.random((200, 40)) < 0.2)))
+            net.TrainOneBatch(step)
+        results.append([m.asarray().copy() for m in (edge.params['weight'], vis.params['bias'], hid.params['bias'])])
+    for a, b in zip(*results):
+        assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+
+
 def test_three_layer_machine_runs_mean_field_and_gibbs_sweeps(cm, rng):
     """A deep Boltzmann machine (visible - hidden1 - hidden2): no closed form to compare with,
     so only what must hold: the middle layer is computed from both neighbours, the updates are
