@@ -247,6 +247,36 @@ k_gemm(const float* __restrict__ A, int lda, const float* __restrict__ B, int ld
   const bool split = gridDim.z > 1;
   float* out = split ? partial + (size_t)blockIdx.z * M * N : C;
   const int ldo = split ? M : ldc;
+  if (!split && beta != 0.f) {
+    // Read-modify-write: the sixteen old values of a block are requested before its first
+    // store.  (A load placed after a store to the same array cannot be moved above it, so
+    // sixteen load -> store pairs would be sixteen round trips one after the other:
+    // 4096 x 4096 x 128 with beta = 1 took 88 us that way, 72 us this way.)
+#pragma unroll
+    for (int j = 0; j < WN; ++j) {
+      const int nb = n0 + wn * 32 * WN + j * 32 + 4 * lk;
+      float cold[WM][16];
+#pragma unroll
+      for (int i = 0; i < WM; ++i) {
+        const int m = m0 + wm * 32 * WM + i * 32 + li;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int n = nb + 8 * (v >> 2) + (v & 3);
+          cold[i][v] = (m < M && n < N) ? out[(size_t)n * ldo + m] : 0.f;
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < WM; ++i) {
+        const int m = m0 + wm * 32 * WM + i * 32 + li;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int n = nb + 8 * (v >> 2) + (v & 3);
+          if (m < M && n < N) out[(size_t)n * ldo + m] = gemm_finish(beta * cold[i][v] + alpha * acc[j][i][v], m, epi);
+        }
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int j = 0; j < WN; ++j)
 #pragma unroll
@@ -259,7 +289,7 @@ k_gemm(const float* __restrict__ A, int lda, const float* __restrict__ B, int ld
         if (n < N) {
           float* p = out + (size_t)n * ldo + m;
           if (split) *p = acc[j][i][v];
-          else *p = gemm_finish((beta == 0.f ? 0.f : beta * *p) + alpha * acc[j][i][v], m, epi);
+          else *p = gemm_finish(alpha * acc[j][i][v], m, epi);
         }
       }
     }
@@ -510,7 +540,11 @@ static int gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, co
   // its own wavefronts.
   const long long tiles64 = (long long)((M + 63) / 64) * ((N + 63) / 64);
   const bool off32 = (size_t)lda * (a_kc ? M : K) < (1u << 30) && (size_t)ldb * (b_kc ? N : K) < (1u << 30);
-  if (tiles64 < cus && off32) {
+  // That kernel re-reads its operands from L2 for every 32 x 32 block ((M/32)(N/32) 64 K floats):
+  // beyond about 1.5e9 multiply-adds that traffic costs more than LDS tiles with a split K
+  // (measured: 4096 x 128 x 4096 66 us against 53 us, 2048 x 128 x 2048 17.7 against 21.4).
+  const bool heavy = (double)M * (double)N * (double)K >= 1.5e9;
+  if (tiles64 < cus && off32 && !heavy) {
     dim3 grid((M + 31) / 32, (N + 31) / 32);
 #define GEMM_SMALL(AK, BK_)                                                                                  \
   do {                                                                                                       \
@@ -543,7 +577,7 @@ static int gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, co
     // The second kernel costs about 5 us and a split slice starts its pipeline anew: measured
     // on 1024 x 1024 outputs a split only pays from K = 2048 on (K = 128: 13 us split, 7.5 us
     // whole), and with 1.5 tiles per CU (1280 x 1280) it never does.
-    if (K < 2048 || tiles * 4 >= (long long)cus * 5) want = 1;
+    if ((K < 2048 && !(heavy && K >= 1024)) || tiles * 4 >= (long long)cus * 5) want = 1;
     if (want > 1) splits = (int)want;
   }
   int kps = ((K + splits - 1) / splits + GEMM_BK - 1) / GEMM_BK * GEMM_BK;
