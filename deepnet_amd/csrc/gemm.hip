@@ -564,7 +564,14 @@ static int gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, co
     return dn_launch_status();
   }
   const long long tiles_big = (long long)((M + 127) / 128) * ((N + 127) / 128);
-  const bool big = tiles_big >= cus;
+  // 128 x 128 tiles (two workgroups per CU) against 64 x 64 tiles (five), as measured:
+  // short reductions are mostly prologue and epilogue, which more resident workgroups hide
+  // (4096 x 4096 x 128, beta = 1: 71 us against 60 us; up to K = 512 when C is also read); and
+  // a tile count that leaves the last round of a CU half empty costs more than the smaller
+  // tile's lower matrix-core rate of about 0.92 (3072 x 3072 x 2048: 404 us against 336 us).
+  const int kmax64 = beta != 0.f ? 512 : 128;
+  auto fill = [&](long long t) { return (double)t / (double)(((t + cus - 1) / cus) * cus); };
+  const bool big = tiles_big >= cus && K > kmax64 && fill(tiles_big) >= 0.92 * fill(tiles64);
   const int BM = big ? 128 : 64, BN = big ? 128 : 64;
   const int gx = (M + BM - 1) / BM, gy = (N + BN - 1) / BN;
   int splits = 1;
