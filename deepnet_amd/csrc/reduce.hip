@@ -488,6 +488,7 @@ static int rows_reduce(const float* M, int ld, int h, int w, const float* x, flo
   const int bx = (h + rows_per_block - 1) / rows_per_block;
   int splits = (8 * dn_num_cus()) / bx;
   if (splits > (w + 63) / 64) splits = (w + 63) / 64;
+  if (w <= 128) splits = 1;   // (layer states of up to 128 cases: the rows alone fill the chip, one launch)
   if (splits < 1 || (size_t)h * w <= (1u << 18)) splits = 1;   // small: one launch beats two
   int cps = (w + splits - 1) / splits;
   if (cps < 1) cps = 1;
