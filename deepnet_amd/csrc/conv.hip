@@ -1452,7 +1452,20 @@ static void launch_rowmajor(const ConvArgs& a, long long rows, int cols, int gz)
     else if (cols <= 32) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 1, true>), dim3(gx, (cols + 31) / 32, gz), dim3(256), 0, 0, a);
     else if (cols <= 48) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 2, true, 3>), dim3(gx, 1, gz), dim3(256), 0, 0, a);
     else if (cols <= 64) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 2, true>), dim3(gx, (cols + 63) / 64, gz), dim3(256), 0, 0, a);
-    else hipLaunchKernelGGL((k_conv_mfma<MODE, 2, 2, 2, true>), dim3(gx, (cols + 127) / 128, gz), dim3(256), 0, 0, a);
+    else {
+      // More than 96 columns: 128-wide tiles (64 x 64 per wavefront) or 64-wide ones (32 x 64).
+      // What decides is how full the column tiles are and how evenly the tiles spread over the
+      // CUs; at equal fill the wide tile is the faster one for convUp (the image gather is
+      // repeated per column tile: measured rate 0.82 of the wide tile's), for convDown neither.
+      // (384 filters in 2 groups on 13 x 13 maps: Up 449 -> 288 us, Down 330 -> 221 us.)
+      const int cus = dn_num_cus();
+      auto spread = [&](long long t) { return (double)t / (double)(((t + cus - 1) / cus) * cus); };
+      const int c128 = (cols + 127) / 128, c64 = (cols + 63) / 64;
+      const double s128 = (double)cols / (128.0 * c128) * spread((long long)gx * c128 * gz);
+      const double s64 = (double)cols / (64.0 * c64) * spread((long long)gx * c64 * gz) * (MODE == CONV_UP ? 0.82 : 1.0);
+      if (s64 > s128) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 2, true>), dim3(gx, c64, gz), dim3(256), 0, 0, a);
+      else hipLaunchKernelGGL((k_conv_mfma<MODE, 2, 2, 2, true>), dim3(gx, c128, gz), dim3(256), 0, 0, a);
+    }
     return;
   }
   // Up / Down: rows are plentiful, columns few: 4 wavefronts down the rows, WN blocks across.

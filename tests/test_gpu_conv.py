@@ -40,6 +40,11 @@ CASES = [  # N, C, H, F, k, stride, padding, groups
     (128, 48, 7, 32, 5, 1, 2, 1),    # uniform-row kernels with 16-wide column blocks: convDown onto 48 colours
     (128, 16, 8, 48, 5, 1, 2, 1),    # the same: convUp onto 48 filters, convDown onto 16 colours (one block of 16)
     (128, 96, 6, 64, 5, 1, 2, 2),    # the same in 2 groups of 48 colours / 32 filters (the shape of config 5b)
+    (128, 32, 6, 160, 3, 1, 1, 1),   # uniform-row kernels, more than 96 columns on few tiles: 64-wide column tiles (convUp: 64 + 64 + 32 filters)
+    (128, 160, 6, 32, 3, 1, 1, 1),   # the same for convDown onto 160 colours
+    (128, 64, 5, 224, 3, 1, 1, 2),   # the same in 2 groups: 112 filters per group (64 + 48)
+    (128, 224, 5, 64, 3, 1, 1, 2),   # ... and 112 colours per group in convDown
+    (128, 32, 14, 256, 3, 1, 1, 1),  # full 128-wide column tiles and enough of them: the wide kernel stays
 ]
 
 
