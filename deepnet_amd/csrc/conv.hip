@@ -1681,7 +1681,8 @@ static void conv_outp_impl(cudamat* images, cudamat* hidActs, cudamat* targets, 
     } else if (fast) {
       // rows = filters of a group: pick the tile height that wastes least.
       const int Fg = a.Fg;
-      const int BMs = Fg <= 32 ? 32 : Fg <= 64 ? 64 : Fg <= 96 ? 96 : 128;
+      int BMs = Fg <= 32 ? 32 : Fg <= 64 ? 64 : Fg <= 96 ? 96 : 128;
+      if (Fg > 128 && (Fg + 95) / 96 * 96 < (Fg + 127) / 128 * 128) BMs = 96;   // e.g. 192 filters: 2 x 96, not 2 x 128
       const int gx = (Fg + BMs - 1) / BMs, gy = (cols + 127) / 128;
       const int nslabs = a.m_count * (N / CV_BK);
       // about two workgroups per CU (measured against one and three), at least 16 slabs (256 of the reduction) per split

@@ -45,6 +45,8 @@ CASES = [  # N, C, H, F, k, stride, padding, groups
     (128, 64, 5, 224, 3, 1, 1, 2),   # the same in 2 groups: 112 filters per group (64 + 48)
     (128, 224, 5, 64, 3, 1, 1, 2),   # ... and 112 colours per group in convDown
     (128, 32, 14, 256, 3, 1, 1, 1),  # full 128-wide column tiles and enough of them: the wide kernel stays
+    (32, 16, 6, 192, 3, 1, 1, 1),    # convOutp with 192 filters: two 96-row tiles instead of two 128-row ones
+    (32, 32, 5, 320, 3, 1, 1, 2),    # the same in 2 groups of 160 filters (96 + 64)
 ]
 
 
