@@ -53,7 +53,8 @@ struct ConvArgs {
   int N, C, Cg, H, F, Fg, k, Mx, s, pad0, G;
   int M, HH, kk2;     // Mx*Mx, H*H, k*k
   int m_begin, m_count;  // Outp: module chunk [m_begin, m_begin + m_count)
-  int splits, slabs_per_split;
+  int splits, slabs_per_split;   // Outp always; Up / Down (stride 1) when the tiles alone cannot fill the chip
+  long long split_stride;        // Up / Down with splits > 1: elements between the partial outputs in `partial`
   int local;          // 1: one filter bank per module (locally connected layers); direct kernels only
   float scale_t, scale_o;
   unsigned a_bytes, b_bytes;  // sizes of the two gathered arrays (uniform-row kernels: buffer ranges)
@@ -202,10 +203,12 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
   int g, rows, cols, nslabs, slab_beg, slab_end, zsplit = 0;
   DownPhase ph;
   if (MODE == CONV_UP) {
-    g = blockIdx.z;
+    g = blockIdx.z / p.splits;
+    zsplit = blockIdx.z % p.splits;
     rows = M * N; cols = Fg;
     nslabs = (Cg * p.kk2 + CV_BK - 1) / CV_BK;
-    slab_beg = 0; slab_end = nslabs;
+    slab_beg = p.splits > 1 ? zsplit * p.slabs_per_split : 0;
+    slab_end = p.splits > 1 && slab_beg + p.slabs_per_split < nslabs ? slab_beg + p.slabs_per_split : nslabs;
   } else if (MODE == CONV_DOWNM) {
     // Rows: (Y, X, image) over blocks of s x s pixels in padded coordinates, pixel
     // y = Y*s + py + pad0.  Columns: (colour, py, px).  K: (t, u, filter) with the tap
@@ -219,14 +222,17 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
     slab_beg = 0; slab_end = nslabs;
   } else if (MODE == CONV_DOWN) {
     const int nph = s * s;
-    g = blockIdx.z / nph;
-    const int phase = blockIdx.z % nph;
+    const int zz = blockIdx.z / p.splits;             // (splits > 1 only with stride 1: one phase)
+    zsplit = blockIdx.z % p.splits;
+    g = zz / nph;
+    const int phase = zz % nph;
     ph.py = phase / s; ph.px = phase % s;
     down_axis(ph.py, s, p.pad0, H, k, &ph.y_first, &ph.QY, &ph.qy_first, &ph.TY);
     down_axis(ph.px, s, p.pad0, H, k, &ph.x_first, &ph.QX, &ph.qx_first, &ph.TX);
     rows = ph.QY * ph.QX * N; cols = Cg;
     nslabs = ph.TY * ph.TX * (Fg / CV_BK);
-    slab_beg = 0; slab_end = nslabs;
+    slab_beg = p.splits > 1 ? zsplit * p.slabs_per_split : 0;
+    slab_end = p.splits > 1 && slab_beg + p.slabs_per_split < nslabs ? slab_beg + p.slabs_per_split : nslabs;
   } else {
     g = blockIdx.z / p.splits;
     zsplit = blockIdx.z % p.splits;
@@ -663,6 +669,8 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
     buf ^= 1;
   }
 
+  // Up / Down with a split reduction: this workgroup's sums go to its own copy of the output.
+  float* const outb = (MODE == CONV_UP || MODE == CONV_DOWN) && p.splits > 1 ? p.partial + zsplit * p.split_stride : p.out;
   if constexpr (N16 > 0) {
     // acc16[j][i][v] is C(row, col) with row = ... + i*16 + l16, col = j*16 + 4*k16 + v
 #pragma unroll
@@ -704,7 +712,7 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
           for (int v = 0; v < 4; ++v) {
             const int c = col0 + j * 16 + 4 * k16 + v;
             if (c >= cols) continue;
-            float* t = p.out + rbase + cstride * c;
+            float* t = outb + rbase + cstride * c;
             *t = (p.scale_t == 0.f ? 0.f : p.scale_t * *t) + p.scale_o * acc16[j][i][v];
           }
       }
@@ -760,7 +768,7 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
         if (MODE == CONV_OUTP) {
           p.partial[rbase + cstride * c] = acc[j][i][v];
         } else {
-          float* t = p.out + rbase + cstride * c;
+          float* t = outb + rbase + cstride * c;
           *t = (p.scale_t == 0.f ? 0.f : p.scale_t * *t) + p.scale_o * acc[j][i][v];
         }
       }
@@ -1423,7 +1431,7 @@ static bool fast_ok(const ConvArgs& a) {
 static void fill_common(ConvArgs& a, int N, int C, int G, int H, int F, int k, int Mx, int s, int pad0) {
   a.N = N; a.C = C; a.G = G; a.Cg = C / G; a.H = H; a.F = F; a.Fg = F / G; a.k = k; a.Mx = Mx; a.s = s; a.pad0 = pad0;
   a.M = Mx * Mx; a.HH = H * H; a.kk2 = k * k;
-  a.m_begin = 0; a.m_count = a.M; a.splits = 1; a.slabs_per_split = 0; a.local = 0;
+  a.m_begin = 0; a.m_count = a.M; a.splits = 1; a.slabs_per_split = 0; a.split_stride = 0; a.local = 0;
   a.scale_t = 0.f; a.scale_o = 1.f; a.partial = nullptr; a.a_bytes = 0; a.b_bytes = 0;
   a.dN = make_fastdiv((uint32_t)N); a.dMx = make_fastdiv((uint32_t)Mx);
   a.dk = make_fastdiv((uint32_t)k); a.dkk2 = make_fastdiv((uint32_t)(k * k));
@@ -1438,8 +1446,62 @@ static void set_buffer_ranges(ConvArgs& a, long long a_elems, long long b_elems)
   a.b_bytes = fits ? (unsigned)(b_elems * 4) : 0u;
 }
 
+// out = sum of the `splits` partial outputs of a convUp / convDown whose reduction was split.
+__global__ void __launch_bounds__(256) k_conv_sum_splits(const float* partial, int splits, long long total4, float* out) {
+  const long long stride = (long long)gridDim.x * 256;
+  for (long long e = (long long)blockIdx.x * 256 + threadIdx.x; e < total4; e += stride) {
+    float4 s = reinterpret_cast<const float4*>(partial)[e];
+    for (int z = 1; z < splits; ++z) {
+      const float4 v = reinterpret_cast<const float4*>(partial)[(long long)z * total4 + e];
+      s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+    }
+    reinterpret_cast<float4*>(out)[e] = s;
+  }
+}
+
 template <int MODE>
-static void launch_rowmajor(const ConvArgs& a, long long rows, int cols, int gz) {
+static void launch_rowmajor_tiles(const ConvArgs& a, long long rows, int cols, int gz);
+
+// Layers on small maps (8 x 8, 16 x 16 modules at batch 128) have fewer tiles than the chip
+// has CUs, and a lone workgroup per CU walks its reduction at the pace of the memory
+// latency: split the reduction over up to 16 workgroups per tile (at least 8 slabs each)
+// and sum the partial outputs with a second kernel.  (32 -> 64 filters of 5 x 5 on 8 x 8
+// maps: convUp 51 -> 17 us.)
+template <int MODE>
+static void launch_rowmajor(const ConvArgs& a0, long long rows, int cols, int gz) {
+  ConvArgs a = a0;
+  const int cus = dn_num_cus();
+  const long long tiles = (rows + 127) / 128 * (cols <= 96 ? 1 : (cols + 127) / 128) * gz;
+  const int nslabs = MODE == CONV_UP ? (a.Cg * a.kk2 + CV_BK - 1) / CV_BK : a.kk2 * (a.Fg / CV_BK);
+  const long long total = MODE == CONV_UP ? (long long)a.N * a.M * a.F : (long long)a.N * a.HH * a.C;
+  long long want = 1;
+  if ((MODE == CONV_UP || (MODE == CONV_DOWN && a.s == 1)) && tiles < cus && a.scale_t == 0.f && a.scale_o == 1.f) {
+    want = (2ll * cus) / tiles;
+    if (want > nslabs / 8) want = nslabs / 8;
+    if (want > 16) want = 16;
+    if (want < 1) want = 1;
+  }
+  if (want > 1) {
+    a.slabs_per_split = (int)((nslabs + want - 1) / want);
+    a.splits = (nslabs + a.slabs_per_split - 1) / a.slabs_per_split;
+  }
+  if (a.splits > 1) {
+    a.partial = (float*)dn_scratch((size_t)a.splits * total * sizeof(float));
+    if (!a.partial) { a.splits = 1; a.slabs_per_split = 0; }
+    else a.split_stride = total;
+  }
+  launch_rowmajor_tiles<MODE>(a, rows, cols, gz * a.splits);
+  if (a.splits > 1) {
+    const long long total4 = total / 4;            // (the batch is a multiple of 16)
+    long long blocks = (total4 + 255) / 256;
+    if (blocks > 8ll * cus) blocks = 8ll * cus;
+    hipLaunchKernelGGL(k_conv_sum_splits, dim3((unsigned)blocks), dim3(256), 0, 0, (const float*)a.partial, a.splits, total4,
+                       a.out);
+  }
+}
+
+template <int MODE>
+static void launch_rowmajor_tiles(const ConvArgs& a, long long rows, int cols, int gz) {
   // Batches that are multiples of 128: tiles of 128 rows never straddle a module / pixel.
   // Measured on the benchmark layers: the buffer-load kernels win for long reductions
   // with up to 64 or more than 96 columns; 65-96 columns and short reductions are

@@ -47,6 +47,8 @@ CASES = [  # N, C, H, F, k, stride, padding, groups
     (128, 32, 14, 256, 3, 1, 1, 1),  # full 128-wide column tiles and enough of them: the wide kernel stays
     (32, 16, 6, 192, 3, 1, 1, 1),    # convOutp with 192 filters: two 96-row tiles instead of two 128-row ones
     (32, 32, 5, 320, 3, 1, 1, 2),    # the same in 2 groups of 160 filters (96 + 64)
+    (128, 32, 8, 64, 5, 1, 2, 1),    # a small map with a long reduction: convUp / convDown split their reduction over workgroups
+    (128, 64, 4, 96, 3, 1, 1, 2),    # the same in 2 groups of 32 colours / 48 filters (three 16-wide column blocks in convUp)
 ]
 
 
