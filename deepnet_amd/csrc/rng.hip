@@ -336,13 +336,19 @@ int init_random(rnd_struct* rnd_state, int seed, char* cudamatpath) {
   return dn_launch_status();
 }
 
+// A generator that init_random() never set up (null handle or null state pointers): the
+// reference would dereference it; here the call is refused.
+static inline bool rng_ready(const rnd_struct* st) { return st && st->dev_mults && st->dev_words; }
+
 int fill_with_rand(rnd_struct* rnd_state, cudamat* mat) {
   if (!mat->on_device) return ERROR_NOT_ON_DEVICE;
+  if (!rng_ready(rnd_state)) return ERROR_GENERIC;
   return launch_rng(rnd_state, (size_t)dn_len(mat), OpUniform{nullptr, mat->data_device});
 }
 
 int fill_with_randn(rnd_struct* rnd_state, cudamat* mat) {
   if (!mat->on_device) return ERROR_NOT_ON_DEVICE;
+  if (!rng_ready(rnd_state)) return ERROR_GENERIC;
   hipLaunchKernelGGL(k_rng_gauss, dim3(RNG_BLOCKS), dim3(RNG_BLOCK), 0, 0, rnd_state->dev_mults, rnd_state->dev_words,
                      (const float*)nullptr, mat->data_device, (size_t)dn_len(mat), 1.f);
   return dn_launch_status();
@@ -354,6 +360,7 @@ int fill_with_randn(rnd_struct* rnd_state, cudamat* mat) {
     if (mat->size[0] != target->size[0] || mat->size[1] != target->size[1])                            \
       return ERROR_INCOMPATIBLE_DIMENSIONS;                                                            \
     if (!mat->on_device || !target->on_device) return ERROR_NOT_ON_DEVICE;                             \
+    if (!rng_ready(rnd_state)) return ERROR_GENERIC;                                                   \
     return launch_rng(rnd_state, (size_t)dn_len(mat), OP{mat->data_device, target->data_device});      \
   }
 
@@ -366,6 +373,7 @@ DN_SAMPLER(perturb_prob, OpPerturbProb)
 int sample_gaussian(rnd_struct* rnd_state, cudamat* mat, cudamat* target, float mult) {
   if (mat->size[0] != target->size[0] || mat->size[1] != target->size[1]) return ERROR_INCOMPATIBLE_DIMENSIONS;
   if (!mat->on_device || !target->on_device) return ERROR_NOT_ON_DEVICE;
+  if (!rng_ready(rnd_state)) return ERROR_GENERIC;
   hipLaunchKernelGGL(k_rng_gauss, dim3(RNG_BLOCKS), dim3(RNG_BLOCK), 0, 0, rnd_state->dev_mults, rnd_state->dev_words,
                      (const float*)mat->data_device, target->data_device, (size_t)dn_len(mat), mult);
   return dn_launch_status();
@@ -373,6 +381,7 @@ int sample_gaussian(rnd_struct* rnd_state, cudamat* mat, cudamat* target, float 
 
 int dropout(rnd_struct* rnd_state, cudamat* mat, float dropprob, float val) {
   if (!mat->on_device) return ERROR_NOT_ON_DEVICE;
+  if (!rng_ready(rnd_state)) return ERROR_GENERIC;
   return launch_rng(rnd_state, (size_t)dn_len(mat), OpDropout{mat->data_device, mat->data_device, dropprob, val});
 }
 

@@ -70,6 +70,15 @@ def test_host_side_argument_errors_need_no_device():
     assert lib.get_slice(a.p_mat, ct.byref(cm.cudamat()), 0, 1) == -8
     assert lib.get_slice(a.T.p_mat, ct.byref(cm.cudamat()), 0, 1) == -5        # transposed first (cudamat.cu:332-336)
     assert lib.sample_bernoulli(None, a.p_mat, cm.CUDAMatrix(np.zeros((2, 2), np.float32), False).p_mat) == -1
+    # a generator that init_random() never set up is refused (-6) instead of dereferenced
+    fake = cm.cudamat()
+    fake.on_device, fake.size[0], fake.size[1] = 1, 2, 2        # claims to be on the device; never touched
+    empty_state = cm.rnd_struct()
+    for st in (None, ct.byref(empty_state)):
+        assert lib.fill_with_rand(st, ct.byref(fake)) == -6 and lib.fill_with_randn(st, ct.byref(fake)) == -6
+        assert lib.sample_bernoulli(st, ct.byref(fake), ct.byref(fake)) == -6
+        assert lib.sample_gaussian(st, ct.byref(fake), ct.byref(fake), ct.c_float(1.0)) == -6
+        assert lib.dropout(st, ct.byref(fake), ct.c_float(0.5), ct.c_float(0.0)) == -6
     with pytest.raises(cm.CUDAMatException, match="not in device memory"):
         a.add(b)
     # reshape is pure bookkeeping
