@@ -21,8 +21,9 @@
 // workgroups and summed by a second kernel.
 //
 // The matrix-core path needs numImages % 16 == 0, filters-per-group % 16 == 0 and
-// 16-byte aligned buffers; anything else takes the one-thread-per-output kernels
-// below, which are also the cross-check of the fast path in the tests.
+// 16-byte aligned buffers; other batches above 16 images are padded into a workspace by
+// the entry points (see padded_batch), and anything else takes the one-thread-per-output
+// kernels below, which are also the cross-check of the fast path in the tests.
 //
 // First-layer shapes (few colours, few filters) have their own kernels further down,
 // because a 16-deep, 128-column LDS pipeline is mostly prologue and padding for them:
@@ -1780,18 +1781,102 @@ extern "C" {
 
 const char* conv_last_error(void) { return g_conv_failed ? g_conv_err : nullptr; }
 
+// Batches that are not a multiple of 16 images (deepnet's own examples train with 100): the
+// matrix-core kernels need whole groups of images, so the batch-indexed operands are copied into
+// a workspace with the batch rounded up (to a multiple of 128 when that costs at most 30 %
+// more images, which also admits the uniform-row and register kernels; else of 32), the pad
+// images zero, the pass runs on the copies, and a batch-indexed result is copied back.  Zero
+// images add nothing to a weight gradient and their outputs are dropped, so results are the
+// padded pass's exactly.  (64 -> 64 filters of 5 x 5 on 13 x 13 maps at batch 100: convUp
+// 977 us on the one-lane-per-output kernel.)
+static int padded_batch(int N) {
+  if (N <= 16 || N % 16 == 0) return N;
+  const int n128 = (N + 127) / 128 * 128;
+  return (n128 - N) * 10 <= 3 * N ? n128 : (N + 31) / 32 * 32;
+}
+
+// dst (Np x cols) = src (N x cols) with zero rows N .. Np-1, or back (rows 0 .. N-1 only).
+__global__ void __launch_bounds__(256) k_pad_batch(const float* src, float* dst, int N, int Np, long long cols, int unpad) {
+  const long long total = (unpad ? (long long)N : (long long)Np) * cols;
+  const long long stride = (long long)gridDim.x * 256;
+  const int rows = unpad ? N : Np;
+  for (long long e = (long long)blockIdx.x * 256 + threadIdx.x; e < total; e += stride) {
+    const long long c = e / rows;
+    const int r = (int)(e - c * rows);
+    if (unpad) dst[c * N + r] = src[c * Np + r];
+    else dst[e] = r < N ? src[c * N + r] : 0.f;
+  }
+}
+
+static void pad_batch(const float* src, float* dst, int N, int Np, long long cols, bool unpad) {
+  const long long total = (unpad ? (long long)N : (long long)Np) * cols;
+  long long blocks = (total + 255) / 256;
+  if (blocks > 16ll * dn_num_cus()) blocks = 16ll * dn_num_cus();
+  if (blocks < 1) blocks = 1;
+  hipLaunchKernelGGL(k_pad_batch, dim3((unsigned)blocks), dim3(256), 0, 0, src, dst, N, Np, cols, unpad ? 1 : 0);
+}
+
+// Padded stand-ins for up to three batch-indexed matrices in one workspace; null where the batch
+// needs no padding or the workspace cannot be had (then the pass runs as it is).
+struct PaddedBatch {
+  cudamat m[3];
+  int N, Np;
+  bool on;
+  PaddedBatch(cudamat* a, cudamat* b, cudamat* c) : N(a->size[0]), Np(padded_batch(a->size[0])), on(false) {
+    cudamat* src[3] = {a, b, c};
+    if (Np == N || !a->on_device || (b && (!b->on_device || b->size[0] != N)) || (c && (!c->on_device || c->size[0] != N))) return;
+    size_t elems = 0;
+    for (cudamat* x : src) if (x) elems += ((size_t)Np * x->size[1] + 3) / 4 * 4;
+    float* ws = (float*)dn_scratch(elems * sizeof(float), 2);
+    if (!ws) return;
+    for (int i = 0; i < 3; ++i) {
+      if (!src[i]) continue;
+      m[i] = *src[i];
+      m[i].data_device = ws;
+      m[i].size[0] = Np;
+      m[i].owns_data = 0;
+      ws += ((size_t)Np * src[i]->size[1] + 3) / 4 * 4;
+    }
+    on = true;
+  }
+  void fill(int i, const cudamat* from) { pad_batch(from->data_device, m[i].data_device, N, Np, from->size[1], false); }
+  void drain(int i, cudamat* to) { pad_batch(m[i].data_device, to->data_device, N, Np, to->size[1], true); }
+};
+
 void convUp(cudamat* images, cudamat* filters, cudamat* targets, int numModulesX, int paddingStart, int moduleStride,
             int numImgColors, int numGroups) {
+  PaddedBatch pb(images, targets, nullptr);
+  if (pb.on) {
+    pb.fill(0, images);
+    conv_up_impl(&pb.m[0], filters, &pb.m[1], numModulesX, paddingStart, moduleStride, numImgColors, numGroups, "convUp");
+    if (!conv_last_error()) pb.drain(1, targets);
+    return;
+  }
   conv_up_impl(images, filters, targets, numModulesX, paddingStart, moduleStride, numImgColors, numGroups, "convUp");
 }
 
 void convDown(cudamat* hidActs, cudamat* filters, cudamat* targets, int imgSize, int paddingStart, int moduleStride,
               int numImgColors, int numGroups) {
+  PaddedBatch pb(hidActs, targets, nullptr);
+  if (pb.on) {
+    pb.fill(0, hidActs);
+    conv_down_impl(&pb.m[0], filters, &pb.m[1], imgSize, paddingStart, moduleStride, numImgColors, numGroups, "convDown");
+    if (!conv_last_error()) pb.drain(1, targets);
+    return;
+  }
   conv_down_impl(hidActs, filters, targets, imgSize, paddingStart, moduleStride, numImgColors, numGroups, "convDown");
 }
 
 void convOutp(cudamat* images, cudamat* hidActs, cudamat* targets, int numModulesX, int filterSize, int paddingStart,
               int moduleStride, int numImgColors, int numGroups, int partialSum) {
+  PaddedBatch pb(images, hidActs, nullptr);
+  if (pb.on) {
+    pb.fill(0, images);
+    pb.fill(1, hidActs);
+    conv_outp_impl(&pb.m[0], &pb.m[1], targets, numModulesX, filterSize, paddingStart, moduleStride, numImgColors,
+                   numGroups, partialSum, "convOutp");
+    return;
+  }
   conv_outp_impl(images, hidActs, targets, numModulesX, filterSize, paddingStart, moduleStride, numImgColors,
                  numGroups, partialSum, "convOutp");
 }

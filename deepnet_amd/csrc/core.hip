@@ -22,9 +22,10 @@ int dn_num_cus() {
 // ------------------------------------------------------------------ scratch
 // Grow-only device workspaces.  Slot 0: partials of two-stage reductions and
 // split-K products, scalar results.  Slot 1: the patch matrix of the col2im
-// form of convDown (it is live while a product that may use slot 0 runs).
-static void* g_scratch[2] = {nullptr, nullptr};
-static size_t g_scratch_bytes[2] = {0, 0};
+// form of convDown (it is live while a product that may use slot 0 runs).  Slot 2:
+// batch-padded copies of conv operands (live across a whole conv call).
+static void* g_scratch[3] = {nullptr, nullptr, nullptr};
+static size_t g_scratch_bytes[3] = {0, 0, 0};
 
 void* dn_scratch(size_t bytes, int slot) {
   if (bytes > g_scratch_bytes[slot]) {

@@ -49,6 +49,12 @@ CASES = [  # N, C, H, F, k, stride, padding, groups
     (32, 32, 5, 320, 3, 1, 1, 2),    # the same in 2 groups of 160 filters (96 + 64)
     (128, 32, 8, 64, 5, 1, 2, 1),    # a small map with a long reduction: convUp / convDown split their reduction over workgroups
     (128, 64, 4, 96, 3, 1, 1, 2),    # the same in 2 groups of 32 colours / 48 filters (three 16-wide column blocks in convUp)
+    (100, 1, 12, 64, 5, 1, 2, 1),    # batch 100 (deepnet's examples): operands padded to 128 images, register / uniform-row kernels
+    (100, 32, 7, 32, 3, 1, 1, 1),    # the same with many colours
+    (50, 4, 7, 32, 3, 2, 1, 2),      # batch 50 -> 64, strided, 2 groups
+    (20, 3, 6, 16, 5, 1, 2, 1),      # batch 20 -> 32
+    (200, 16, 5, 48, 3, 1, 1, 1),    # batch 200 -> 256
+    (36, 2, 6, 16, 3, 1, 0, 1),      # batch 36 -> 64 with a batch-indexed result that must not spill into its neighbours
 ]
 
 

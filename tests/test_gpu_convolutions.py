@@ -38,6 +38,7 @@ STAGES = [  # N, C, H, F, k, stride, padding, pool (size, stride) or None, norm 
     (64, 4, 12, 16, 3, 1, 1, None, 3, True),
     (32, 16, 13, 32, 3, 2, 0, (2, 2), 5, True),      # strided modules, many colours
     (16, 2, 8, 16, 3, 1, 1, (2, 2), 3, False),       # locally connected
+    (100, 1, 28, 64, 5, 1, 2, (3, 2), None, True),   # the first layer of deepnet's example convnet at its batch size of 100
 ]
 
 
