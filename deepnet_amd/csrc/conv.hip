@@ -21,8 +21,9 @@
 // workgroups and summed by a second kernel.
 //
 // The matrix-core path needs numImages % 16 == 0, filters-per-group % 16 == 0 and
-// 16-byte aligned buffers; other batches above 16 images are padded into a workspace by
-// the entry points (see padded_batch), and anything else takes the one-thread-per-output
+// 16-byte aligned buffers; other batches above 16 images and other filter counts (one
+// group) are padded into a workspace by the entry points (see padded_batch,
+// padded_filters), and anything else takes the one-thread-per-output
 // kernels below, which are also the cross-check of the fast path in the tests.
 //
 // First-layer shapes (few colours, few filters) have their own kernels further down,
@@ -1843,16 +1844,124 @@ struct PaddedBatch {
   void drain(int i, cudamat* to) { pad_batch(m[i].data_device, to->data_device, N, Np, to->size[1], true); }
 };
 
+// Filter counts that are not a multiple of 16 (20 or 50 filters of a LeNet-like net), one group:
+// the same remedy along the filter index.  Zero filters are appended to the filter bank, the
+// hidden activations get zero maps for them (their columns come last in the (image, filter *
+// modules) layout, so that is one contiguous copy and a zero tail), and the pass runs on the
+// copies; the extra outputs of convUp and the extra rows of a weight gradient are dropped.
+// (20 -> 50 filters of 5 x 5 at batch 128: convOutp 390 us on the one-lane-per-output kernel.)
+static int padded_filters(int F, int numGroups) {
+  return numGroups == 1 && F > 0 && F % 16 != 0 ? (F + 15) / 16 * 16 : F;
+}
+
+// Filter-major arrays (f + F*q): dst (Fp x Q) = src (F x Q) with zero rows F .. Fp-1, or back.
+__global__ void __launch_bounds__(256) k_pad_filters(const float* src, float* dst, int F, int Fp, long long Q, int unpad) {
+  const int rows = unpad ? F : Fp;
+  const long long total = (long long)rows * Q;
+  const long long stride = (long long)gridDim.x * 256;
+  for (long long e = (long long)blockIdx.x * 256 + threadIdx.x; e < total; e += stride) {
+    const long long q = e / rows;
+    const int f = (int)(e - q * rows);
+    if (unpad) dst[q * F + f] = src[q * Fp + f];
+    else dst[e] = f < F ? src[q * F + f] : 0.f;
+  }
+}
+// dst[0 .. n_total) = src[0 .. n_copy) followed by zeros.
+__global__ void __launch_bounds__(256) k_copy_prefix(const float* src, float* dst, long long n_copy, long long n_total) {
+  const long long stride = (long long)gridDim.x * 256;
+  for (long long e = (long long)blockIdx.x * 256 + threadIdx.x; e < n_total; e += stride) dst[e] = e < n_copy ? src[e] : 0.f;
+}
+static unsigned pad_grid(long long total) {
+  long long blocks = (total + 255) / 256;
+  if (blocks > 16ll * dn_num_cus()) blocks = 16ll * dn_num_cus();
+  return (unsigned)(blocks < 1 ? 1 : blocks);
+}
+// A stand-in of `rows x cols` floats for `like` at `*ws`, which is moved past it (16-byte steps).
+static cudamat pad_standin(const cudamat* like, int rows, long long cols, float** ws) {
+  cudamat m = *like;
+  m.data_device = *ws;
+  m.size[0] = rows; m.size[1] = (int)cols;
+  m.owns_data = 0;
+  *ws += ((size_t)rows * cols + 3) / 4 * 4;
+  return m;
+}
+
+static void conv_up_filters(cudamat* images, cudamat* filters, cudamat* targets, int numModulesX, int paddingStart,
+                            int moduleStride, int numImgColors, int numGroups) {
+  const int F = filters->size[0], Fp = padded_filters(F, numGroups), N = images->size[0];
+  const long long Q = filters->size[1], M = (long long)numModulesX * numModulesX;
+  float* ws = nullptr;
+  if (Fp != F && images->on_device && filters->on_device && targets->on_device && targets->size[0] == N &&
+      targets->size[1] == F * M && (long long)N * Fp * M < (1ll << 31) && Fp * Q < (1ll << 31))
+    ws = (float*)dn_scratch((((size_t)Fp * Q + 3) / 4 * 4 + ((size_t)N * Fp * M + 3) / 4 * 4) * sizeof(float), 3);
+  if (!ws) {
+    conv_up_impl(images, filters, targets, numModulesX, paddingStart, moduleStride, numImgColors, numGroups, "convUp");
+    return;
+  }
+  cudamat fp = pad_standin(filters, Fp, Q, &ws), tp = pad_standin(targets, N, Fp * M, &ws);
+  hipLaunchKernelGGL(k_pad_filters, dim3(pad_grid(Fp * Q)), dim3(256), 0, 0, (const float*)filters->data_device, fp.data_device, F, Fp, Q, 0);
+  conv_up_impl(images, &fp, &tp, numModulesX, paddingStart, moduleStride, numImgColors, numGroups, "convUp");
+  if (!conv_last_error())
+    hipLaunchKernelGGL(k_copy_prefix, dim3(pad_grid((long long)N * F * M)), dim3(256), 0, 0, (const float*)tp.data_device,
+                       targets->data_device, (long long)N * F * M, (long long)N * F * M);
+}
+
+static void conv_down_filters(cudamat* hidActs, cudamat* filters, cudamat* targets, int imgSize, int paddingStart,
+                              int moduleStride, int numImgColors, int numGroups) {
+  const int F = filters->size[0], Fp = padded_filters(F, numGroups), N = hidActs->size[0];
+  const long long Q = filters->size[1];
+  float* ws = nullptr;
+  if (Fp != F && hidActs->on_device && filters->on_device && targets->on_device && hidActs->size[1] % F == 0 &&
+      (long long)N * (hidActs->size[1] / F) * Fp < (1ll << 31) && Fp * Q < (1ll << 31))
+    ws = (float*)dn_scratch((((size_t)Fp * Q + 3) / 4 * 4 + ((size_t)N * (hidActs->size[1] / F) * Fp + 3) / 4 * 4) * sizeof(float), 3);
+  if (!ws) {
+    conv_down_impl(hidActs, filters, targets, imgSize, paddingStart, moduleStride, numImgColors, numGroups, "convDown");
+    return;
+  }
+  const long long M = hidActs->size[1] / F;
+  cudamat fp = pad_standin(filters, Fp, Q, &ws), hp = pad_standin(hidActs, N, Fp * M, &ws);
+  hipLaunchKernelGGL(k_pad_filters, dim3(pad_grid(Fp * Q)), dim3(256), 0, 0, (const float*)filters->data_device, fp.data_device, F, Fp, Q, 0);
+  hipLaunchKernelGGL(k_copy_prefix, dim3(pad_grid((long long)N * Fp * M)), dim3(256), 0, 0, (const float*)hidActs->data_device,
+                     hp.data_device, (long long)N * F * M, (long long)N * Fp * M);
+  conv_down_impl(&hp, &fp, targets, imgSize, paddingStart, moduleStride, numImgColors, numGroups, "convDown");
+}
+
+static void conv_outp_filters(cudamat* images, cudamat* hidActs, cudamat* targets, int numModulesX, int filterSize,
+                              int paddingStart, int moduleStride, int numImgColors, int numGroups, int partialSum) {
+  const long long M = (long long)numModulesX * numModulesX;
+  const int N = images->size[0];
+  const int F = M > 0 && hidActs->size[1] % M == 0 ? (int)(hidActs->size[1] / M) : 0;
+  const int Fp = padded_filters(F, numGroups);
+  const long long Q = targets->size[1];
+  float* ws = nullptr;
+  if (Fp != F && images->on_device && hidActs->on_device && targets->on_device && hidActs->size[0] == N &&
+      targets->size[0] == F && (long long)N * Fp * M < (1ll << 31) && Fp * Q < (1ll << 31))
+    ws = (float*)dn_scratch((((size_t)Fp * Q + 3) / 4 * 4 + ((size_t)N * Fp * M + 3) / 4 * 4) * sizeof(float), 3);
+  if (!ws) {
+    conv_outp_impl(images, hidActs, targets, numModulesX, filterSize, paddingStart, moduleStride, numImgColors, numGroups,
+                   partialSum, "convOutp");
+    return;
+  }
+  cudamat tp = pad_standin(targets, Fp, Q, &ws), hp = pad_standin(hidActs, N, Fp * M, &ws);
+  hipLaunchKernelGGL(k_copy_prefix, dim3(pad_grid((long long)N * Fp * M)), dim3(256), 0, 0, (const float*)hidActs->data_device,
+                     hp.data_device, (long long)N * F * M, (long long)N * Fp * M);
+  conv_outp_impl(images, &hp, &tp, numModulesX, filterSize, paddingStart, moduleStride, numImgColors, numGroups, partialSum,
+                 "convOutp");
+  if (!conv_last_error())
+    hipLaunchKernelGGL(k_pad_filters, dim3(pad_grid((long long)F * Q)), dim3(256), 0, 0, (const float*)tp.data_device,
+                       targets->data_device, F, Fp, Q, 1);
+}
+
 void convUp(cudamat* images, cudamat* filters, cudamat* targets, int numModulesX, int paddingStart, int moduleStride,
             int numImgColors, int numGroups) {
   PaddedBatch pb(images, targets, nullptr);
   if (pb.on) {
     pb.fill(0, images);
-    conv_up_impl(&pb.m[0], filters, &pb.m[1], numModulesX, paddingStart, moduleStride, numImgColors, numGroups, "convUp");
+    conv_up_filters(&pb.m[0], filters, &pb.m[1], numModulesX, paddingStart, moduleStride, numImgColors, numGroups);
     if (!conv_last_error()) pb.drain(1, targets);
     return;
   }
-  conv_up_impl(images, filters, targets, numModulesX, paddingStart, moduleStride, numImgColors, numGroups, "convUp");
+  conv_up_filters(images, filters, targets, numModulesX, paddingStart, moduleStride, numImgColors, numGroups);
 }
 
 void convDown(cudamat* hidActs, cudamat* filters, cudamat* targets, int imgSize, int paddingStart, int moduleStride,
@@ -1860,11 +1969,11 @@ void convDown(cudamat* hidActs, cudamat* filters, cudamat* targets, int imgSize,
   PaddedBatch pb(hidActs, targets, nullptr);
   if (pb.on) {
     pb.fill(0, hidActs);
-    conv_down_impl(&pb.m[0], filters, &pb.m[1], imgSize, paddingStart, moduleStride, numImgColors, numGroups, "convDown");
+    conv_down_filters(&pb.m[0], filters, &pb.m[1], imgSize, paddingStart, moduleStride, numImgColors, numGroups);
     if (!conv_last_error()) pb.drain(1, targets);
     return;
   }
-  conv_down_impl(hidActs, filters, targets, imgSize, paddingStart, moduleStride, numImgColors, numGroups, "convDown");
+  conv_down_filters(hidActs, filters, targets, imgSize, paddingStart, moduleStride, numImgColors, numGroups);
 }
 
 void convOutp(cudamat* images, cudamat* hidActs, cudamat* targets, int numModulesX, int filterSize, int paddingStart,
@@ -1873,12 +1982,12 @@ void convOutp(cudamat* images, cudamat* hidActs, cudamat* targets, int numModule
   if (pb.on) {
     pb.fill(0, images);
     pb.fill(1, hidActs);
-    conv_outp_impl(&pb.m[0], &pb.m[1], targets, numModulesX, filterSize, paddingStart, moduleStride, numImgColors,
-                   numGroups, partialSum, "convOutp");
+    conv_outp_filters(&pb.m[0], &pb.m[1], targets, numModulesX, filterSize, paddingStart, moduleStride, numImgColors,
+                      numGroups, partialSum);
     return;
   }
-  conv_outp_impl(images, hidActs, targets, numModulesX, filterSize, paddingStart, moduleStride, numImgColors,
-                 numGroups, partialSum, "convOutp");
+  conv_outp_filters(images, hidActs, targets, numModulesX, filterSize, paddingStart, moduleStride, numImgColors, numGroups,
+                    partialSum);
 }
 
 // Locally connected layers: one filter bank per module, filters laid out

@@ -23,9 +23,10 @@ int dn_num_cus() {
 // Grow-only device workspaces.  Slot 0: partials of two-stage reductions and
 // split-K products, scalar results.  Slot 1: the patch matrix of the col2im
 // form of convDown (it is live while a product that may use slot 0 runs).  Slot 2:
-// batch-padded copies of conv operands (live across a whole conv call).
-static void* g_scratch[3] = {nullptr, nullptr, nullptr};
-static size_t g_scratch_bytes[3] = {0, 0, 0};
+// batch-padded copies of conv operands (live across a whole conv call).  Slot 3: the same
+// for operands padded to a multiple of 16 filters.
+static void* g_scratch[4] = {nullptr, nullptr, nullptr, nullptr};
+static size_t g_scratch_bytes[4] = {0, 0, 0, 0};
 
 void* dn_scratch(size_t bytes, int slot) {
   if (bytes > g_scratch_bytes[slot]) {

@@ -55,6 +55,10 @@ CASES = [  # N, C, H, F, k, stride, padding, groups
     (20, 3, 6, 16, 5, 1, 2, 1),      # batch 20 -> 32
     (200, 16, 5, 48, 3, 1, 1, 1),    # batch 200 -> 256
     (36, 2, 6, 16, 3, 1, 0, 1),      # batch 36 -> 64 with a batch-indexed result that must not spill into its neighbours
+    (128, 1, 12, 20, 5, 1, 0, 1),    # 20 filters (a LeNet-like first layer): filter bank and hidden maps padded to 32 filters
+    (128, 20, 8, 50, 5, 1, 0, 1),    # 20 colours -> 50 filters (padded to 64)
+    (100, 3, 8, 10, 3, 1, 1, 1),     # batch 100 and 10 filters: both paddings at once
+    (64, 4, 9, 24, 3, 2, 1, 1),      # 24 filters, strided
 ]
 
 
