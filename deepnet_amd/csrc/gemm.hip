@@ -33,6 +33,8 @@ __device__ __forceinline__ float gemm_finish(float v, int m, const GemmEpilogue&
   return v;
 }
 
+struct __attribute__((packed, aligned(4))) gemm_f4u { float x, y, z, w; };   // four floats at any 4-byte boundary
+
 #define GEMM_BK 16
 #define GEMM_PAD 4
 
@@ -46,6 +48,11 @@ __device__ __forceinline__ f32x4 gemm_load4(const float* base, int c, int c_lim,
     const float* p = base + (size_t)o * ld + c;
     if (vec_ok && c + 3 < c_lim) {
       r = *reinterpret_cast<const f32x4*>(p);
+    } else if (c + 3 < c_lim) {
+      // a leading dimension or base that is not a multiple of 16 bytes: still one 16-byte
+      // request (global memory takes it at 4-byte alignment), not four 4-byte ones
+      const gemm_f4u t = *reinterpret_cast<const gemm_f4u*>(p);
+      r.x = t.x; r.y = t.y; r.z = t.z; r.w = t.w;
     } else {
       if (c < c_lim) r.x = p[0];
       if (c + 1 < c_lim) r.y = p[1];
@@ -337,7 +344,10 @@ __device__ __forceinline__ void small_load(const float* __restrict__ P, unsigned
         }
       } else {
 #pragma unroll
-        for (int q = 0; q < 16; ++q) r[q] = small_ldg(P, off + 4u * q);
+        for (int u = 0; u < 4; ++u) {
+          const gemm_f4u t = *reinterpret_cast<const gemm_f4u*>(reinterpret_cast<const char*>(P) + (off + 16u * u));
+          r[4 * u] = t.x; r[4 * u + 1] = t.y; r[4 * u + 2] = t.z; r[4 * u + 3] = t.w;
+        }
       }
     } else {
       const float* pu = P + (size_t)k0 * ld;                 // wave-uniform
@@ -360,14 +370,20 @@ __device__ __forceinline__ void small_load(const float* __restrict__ P, unsigned
 // way it lies in memory (8 lanes per row, 128-byte runs: 8 cache lines per instruction
 // instead of 64) and turned into the MFMA layout through a wavefront-private LDS tile.
 // r[4u + j] = op(P)(row0 + lane/8 + 8u, k0 + 4*(lane%8) + j); rows past the edge repeat the last one.
+// (aligned: rows start on 16-byte boundaries; otherwise the same requests at 4-byte alignment)
 __device__ __forceinline__ void small_load_rows(const float* __restrict__ P, unsigned ld, unsigned row0, unsigned last_row,
-                                                int k0, int lane, float (&r)[16]) {
+                                                int k0, int lane, bool aligned, float (&r)[16]) {
 #pragma unroll
   for (int u = 0; u < 4; ++u) {
     const unsigned row = min(row0 + (unsigned)(lane >> 3) + 8u * u, last_row);
     const unsigned off = (row * ld + (unsigned)k0 + 4u * (lane & 7)) * 4u;
-    const float4 t = *reinterpret_cast<const float4*>(reinterpret_cast<const char*>(P) + off);
-    r[4 * u] = t.x; r[4 * u + 1] = t.y; r[4 * u + 2] = t.z; r[4 * u + 3] = t.w;
+    if (aligned) {
+      const float4 t = *reinterpret_cast<const float4*>(reinterpret_cast<const char*>(P) + off);
+      r[4 * u] = t.x; r[4 * u + 1] = t.y; r[4 * u + 2] = t.z; r[4 * u + 3] = t.w;
+    } else {
+      const gemm_f4u t = *reinterpret_cast<const gemm_f4u*>(reinterpret_cast<const char*>(P) + off);
+      r[4 * u] = t.x; r[4 * u + 1] = t.y; r[4 * u + 2] = t.z; r[4 * u + 3] = t.w;
+    }
   }
 }
 // In: r as small_load_rows left it.  Out: r[q] = chunk(row lane%32, k = 16*(lane/32) + q).
@@ -418,13 +434,13 @@ k_gemm_small(const float* __restrict__ A, int lda, const float* __restrict__ B, 
   constexpr int STEP = 32 * NW;
   float a[DEPTH][16], b[DEPTH][16];
   int k0 = wv * 32;
-  // (a chunk takes the row-wise path when it is K-contiguous, aligned and whole)
+  // (a chunk takes the row-wise path when it is K-contiguous and whole)
   auto load_a = [&](int kc, float (&r)[16]) __attribute__((always_inline)) {
-    if (A_KC && a_vec && kc + 32 <= K) small_load_rows(A, lda, blockIdx.x * 32, M - 1, kc, lane, r);
+    if (A_KC && kc + 32 <= K) small_load_rows(A, lda, blockIdx.x * 32, M - 1, kc, lane, a_vec, r);
     else small_load<A_KC>(A, lda, mc, kc, lk, K, a_vec, r);
   };
   auto load_b = [&](int kc, float (&r)[16]) __attribute__((always_inline)) {
-    if (B_KC && b_vec && kc + 32 <= K) small_load_rows(B, ldb, blockIdx.y * 32, N - 1, kc, lane, r);
+    if (B_KC && kc + 32 <= K) small_load_rows(B, ldb, blockIdx.y * 32, N - 1, kc, lane, b_vec, r);
     else small_load<B_KC>(B, ldb, nc, kc, lk, K, b_vec, r);
   };
 #pragma unroll
@@ -436,8 +452,8 @@ k_gemm_small(const float* __restrict__ A, int lda, const float* __restrict__ B, 
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
       if (k0 + d * STEP < K) {                               // wave-uniform
-        if (A_KC && a_vec && k0 + d * STEP + 32 <= K) small_restage(stage[wv][0], lane, a[d]);
-        if (B_KC && b_vec && k0 + d * STEP + 32 <= K) small_restage(stage[wv][NSTAGE - 1], lane, b[d]);
+        if (A_KC && k0 + d * STEP + 32 <= K) small_restage(stage[wv][0], lane, a[d]);
+        if (B_KC && k0 + d * STEP + 32 <= K) small_restage(stage[wv][NSTAGE - 1], lane, b[d]);
 #pragma unroll
         for (int q = 0; q < 16; ++q) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(b[d][q], a[d][q], acc, 0, 0, 0);
         if (k0 + (d + DEPTH) * STEP < K) {                   // refill the set with the chunk DEPTH further on
