@@ -264,6 +264,33 @@ def net_rbm(cm, nv=784, nh=500, B=100, lr=0.01, seed=1):
     return dbm.DBM([vis, hid], [edge], optimizer='CD')
 
 
+def net_example_convnet(cm, B=100, seed=12):
+    """The model of deepnet/examples/convnet (model_conv.pbtxt, batch 100 as in train.pbtxt):
+    28 x 28 inputs -> conv 5 x 5 (64 filters) + pool 3/2 -> conv 5 x 5 (64 -> 64) + pool 3/2 -> 1024 ReLU
+    -> softmax(10), as Layer / Edge / NeuralNet objects."""
+    from deepnet_amd import layer as dl, neuralnet as dnn, parameter as dp, convolutions as dc
+    rng = np.random.default_rng(seed)
+    net_h = dict(base_epsilon=0.01, initial_momentum=0.5, final_momentum=0.9, momentum_change_steps=10000)
+    conv_h = dict(base_epsilon=0.001, initial_momentum=0.9, final_momentum=0.9, momentum_change_steps=20000)
+    hyp = lambda act, **kw: dp.Hyperparams(activation=act, **kw)
+    L = [dl.LinearLayer('input_layer', 784, B, hyperparams=hyp(dp.LINEAR), is_input=True),
+         dl.ReluLayer('hidden1', 10816, B, hyperparams=hyp(dp.RECTIFIED_LINEAR, **net_h)),
+         dl.ReluLayer('hidden2', 2304, B, hyperparams=hyp(dp.RECTIFIED_LINEAR, **net_h)),
+         dl.ReluLayer('hidden3', 1024, B, hyperparams=hyp(dp.RECTIFIED_LINEAR, **net_h)),
+         dl.SoftmaxLayer('output_layer', 1, B, hyperparams=hyp(dp.SOFTMAX, **net_h), numlabels=10, is_output=True,
+                         loss_function=dp.CROSS_ENTROPY)]
+    cv = lambda colors: dc.ConvParams(size=5, stride=1, padding=2, num_filters=64, num_colors=colors, max_pool=True,
+                                      pool_size=3, pool_stride=2)
+    dense = dp.Hyperparams(apply_l2_decay=True, l2_decay=0.001, **net_h)
+    E = [dnn.Edge(L[0], L[1], 0.1 * rng.standard_normal((64, 25)), hyperparams=dp.Hyperparams(**conv_h), conv_params=cv(1)),
+         dnn.Edge(L[1], L[2], 0.02 * rng.standard_normal((64, 1600)), hyperparams=dp.Hyperparams(**conv_h), conv_params=cv(64)),
+         dnn.Edge(L[2], L[3], 0.02 * rng.standard_normal((2304, 1024)), hyperparams=dense),
+         dnn.Edge(L[3], L[4], 0.05 * rng.standard_normal((1024, 10)), hyperparams=dense)]
+    L[0].data.assign(cm.CUDAMatrix(np.asarray(rng.random((784, B)), dtype=np.float32, order='F')))
+    L[-1].data.assign(cm.CUDAMatrix(np.asarray(rng.integers(0, 10, (1, B)), dtype=np.float32, order='F')))
+    return dnn.NeuralNet(L, E)
+
+
 def time_loop(cm, fn, iters, warmup):
     for _ in range(warmup):
         fn()
@@ -531,6 +558,11 @@ def main():
             obj.fused = True
         t = time_loop(cm, lambda: rbm_net.TrainOneBatch(0), 100, 10)
         secondary['rbm_through_dbm_class']['us_per_step_fused_extensions'] = round(t * 1e6, 1)
+        convnet = net_example_convnet(cm)
+        t = time_loop(cm, lambda: convnet.TrainOneBatch(0), 50, 5)
+        secondary['example_convnet_batch100'] = {
+            'steps_per_sec': round(1.0 / t, 1), 'us_per_step': round(t * 1e6, 1),
+            'note': 'deepnet/examples/convnet (two conv + pool stages, 1024 ReLU, softmax) at its batch size of 100: TrainOneBatch through the layer / edge classes'}
         secondary['gemm_fp32_4096'] = gemm_probe(cm, ev)
         try:
             import bench_conv

@@ -162,3 +162,30 @@ def test_small_convnet_trains_like_the_oracle(cm, dn):
     net, onet = _build_chain(dn, spec, B, rng)
     batches = [(rng.standard_normal((C * H * H, B)), rng.integers(0, 10, (1, B)).astype(np.float64)) for _ in range(3)]
     _train_and_compare(cm, net, onet, batches, rtol=2e-4, atol=2e-6)
+
+
+def test_example_convnet_of_the_reference_at_its_batch_size(cm, dn):
+    """deepnet/examples/convnet/model_conv.pbtxt: 784 -> conv 5x5 pad 2 (64 filters) + pool 3/2 ->
+    10816 ReLU -> conv 5x5 pad 2 (64 -> 64) + pool 3/2 -> 2304 ReLU -> 1024 ReLU -> softmax(10),
+    batch 100 (train.pbtxt), its learning rates, momentum schedules and L2 decay."""
+    rng = np.random.default_rng(12)
+    cm.CUDAMatrix.init_random(12)
+    B = 100
+    net_h = dict(base_epsilon=0.01, initial_momentum=0.5, final_momentum=0.9, momentum_change_steps=10000,
+                 apply_l2_decay=True, l2_decay=0.001)
+    bias_h = dict(net_h, apply_l2_decay=False)
+    conv_h = dict(base_epsilon=0.001, initial_momentum=0.9, final_momentum=0.9, momentum_change_steps=20000)
+    cv1 = dn.cv.ConvParams(size=5, stride=1, padding=2, num_filters=64, num_colors=1, max_pool=True, pool_size=3, pool_stride=2)
+    cv2 = dn.cv.ConvParams(size=5, stride=1, padding=2, num_filters=64, num_colors=64, max_pool=True, pool_size=3, pool_stride=2)
+    w1 = _f(0.1 * rng.standard_normal((64, 25)))
+    w2 = _f(0.02 * rng.standard_normal((64, 64 * 25)))
+    w3 = _f(0.02 * rng.standard_normal((2304, 1024)))
+    w4 = _f(0.05 * rng.standard_normal((1024, 10)))
+    spec = [(dn.P.LINEAR, 784, {}, None),
+            (dn.P.RECTIFIED_LINEAR, 10816, bias_h, {'w': w1, 'hyper': conv_h, 'cv': cv1}),
+            (dn.P.RECTIFIED_LINEAR, 2304, bias_h, {'w': w2, 'hyper': conv_h, 'cv': cv2}),
+            (dn.P.RECTIFIED_LINEAR, 1024, bias_h, {'w': w3, 'hyper': net_h}),
+            (dn.P.SOFTMAX, 10, bias_h, {'w': w4, 'hyper': net_h})]
+    net, onet = _build_chain(dn, spec, B, rng)
+    batches = [(rng.random((784, B)), rng.integers(0, 10, (1, B)).astype(np.float64)) for _ in range(2)]
+    _train_and_compare(cm, net, onet, batches, rtol=2e-4, atol=2e-6)
