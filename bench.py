@@ -563,6 +563,10 @@ def main():
         secondary['example_convnet_batch100'] = {
             'steps_per_sec': round(1.0 / t, 1), 'us_per_step': round(t * 1e6, 1),
             'note': 'deepnet/examples/convnet (two conv + pool stages, 1024 ReLU, softmax) at its batch size of 100: TrainOneBatch through the layer / edge classes'}
+        for obj in convnet.layer + convnet.edge:
+            obj.fused = True
+        t = time_loop(cm, lambda: convnet.TrainOneBatch(0), 50, 5)
+        secondary['example_convnet_batch100']['us_per_step_fused_extensions'] = round(t * 1e6, 1)
         secondary['gemm_fp32_4096'] = gemm_probe(cm, ev)
         try:
             import bench_conv

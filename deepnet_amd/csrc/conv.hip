@@ -1797,24 +1797,36 @@ static int padded_batch(int N) {
 }
 
 // dst (Np x cols) = src (N x cols) with zero rows N .. Np-1, or back (rows 0 .. N-1 only).
-__global__ void __launch_bounds__(256) k_pad_batch(const float* src, float* dst, int N, int Np, long long cols, int unpad) {
-  const long long total = (unpad ? (long long)N : (long long)Np) * cols;
-  const long long stride = (long long)gridDim.x * 256;
-  const int rows = unpad ? N : Np;
-  for (long long e = (long long)blockIdx.x * 256 + threadIdx.x; e < total; e += stride) {
-    const long long c = e / rows;
-    const int r = (int)(e - c * rows);
-    if (unpad) dst[c * N + r] = src[c * Np + r];
-    else dst[e] = r < N ? src[c * N + r] : 0.f;
+// One lane per group of four rows when VEC (both batch sizes are then multiples of 4); the
+// column of a group comes from one multiply-high.
+__global__ void __launch_bounds__(256) k_pad_batch(const float* src, float* dst, int N, int Np, unsigned total, FastDiv drows, int unpad,
+                                                   int VEC) {
+  const int W = VEC ? 4 : 1;
+  const unsigned rows = drows.d;                     // row groups per column of the array being written
+  for (unsigned e = blockIdx.x * 256u + threadIdx.x; e < total; e += gridDim.x * 256u) {
+    const unsigned c = fd_div(e, drows);
+    const unsigned r = (e - c * rows) * W;
+    const float* s = src + (size_t)c * (unpad ? Np : N) + r;
+    float* d = dst + (size_t)c * (unpad ? N : Np) + r;
+    if (VEC) {
+      const float4 v = (unpad || (int)r < N) ? *reinterpret_cast<const float4*>(s) : make_float4(0.f, 0.f, 0.f, 0.f);
+      *reinterpret_cast<float4*>(d) = v;
+    } else {
+      *d = (unpad || (int)r < N) ? *s : 0.f;
+    }
   }
 }
 
 static void pad_batch(const float* src, float* dst, int N, int Np, long long cols, bool unpad) {
-  const long long total = (unpad ? (long long)N : (long long)Np) * cols;
+  const bool vec = N % 4 == 0 && dn_aligned16(src) && dn_aligned16(dst);
+  const int rows = (unpad ? N : Np) / (vec ? 4 : 1);
+  const long long total = (long long)rows * cols;
+  if (total <= 0) return;
   long long blocks = (total + 255) / 256;
   if (blocks > 16ll * dn_num_cus()) blocks = 16ll * dn_num_cus();
-  if (blocks < 1) blocks = 1;
-  hipLaunchKernelGGL(k_pad_batch, dim3((unsigned)blocks), dim3(256), 0, 0, src, dst, N, Np, cols, unpad ? 1 : 0);
+  const FastDiv fd = make_fastdiv((uint32_t)rows);
+  hipLaunchKernelGGL(k_pad_batch, dim3((unsigned)blocks), dim3(256), 0, 0, src, dst, N, Np, (unsigned)total, fd, unpad ? 1 : 0,
+                     vec ? 1 : 0);
 }
 
 // Padded stand-ins for up to three batch-indexed matrices in one workspace; null where the batch
