@@ -4,8 +4,10 @@ the reference's deepnet/dbm.py -- ``ComputeUp`` (:64-118), ``PositivePhase`` (:1
 ``UpdateEdgeParams`` (:246-266), ``TrainOneBatch`` / ``EvaluateOneBatch`` (:273-282) -- with CD
 (one set of states, chains restarted at the data) and PCD (persistent negative states), over the
 layers and edges of this package.  An RBM is the two-layer case: one input layer, one hidden
-layer, one edge.  Initialiser nets, sparsity and replicated softmax are not carried over.
+layer, one edge.  Initialiser nets and replicated softmax are not carried over.
 """
+import types
+
 from .choose_matrix_library import cm
 from .neuralnet import NeuralNet, fused_up
 
@@ -94,7 +96,9 @@ class DBM(NeuralNet):
         losses = []
         if train:
             for node in self.layer:
-                node.CollectSufficientStatistics()
+                r = node.CollectSufficientStatistics()
+                if r is not None:           # a layer with a sparsity target reports its mean activity (dbm.py:147-153)
+                    losses.append(types.SimpleNamespace(count=1, sparsity=r))
             for edge in self.edge:
                 edge.CollectSufficientStatistics()
         # With CD the reconstruction error is measured by the negative phase.

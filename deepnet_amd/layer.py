@@ -3,7 +3,7 @@ reference's deepnet/layer.py and its activation subclasses (logistic_layer.py, t
 relu_layer.py, linear_layer.py, softmax_layer.py) -- ``ApplyActivation``, ``ComputeDeriv``,
 ``Sample``, ``GetLoss``, ``GetData`` and the buffers of ``AllocateMemory`` -- issuing the same
 matrix calls in the same order.  Configuration comes as plain arguments instead of protobuf
-messages; sparsity targets, tied layers, replicated softmax and display are not carried over.
+messages; tied layers, replicated softmax and display are not carried over.
 
 States are (dimensions * numlabels, batchsize) matrices, one column per case.
 """
@@ -66,6 +66,10 @@ class Layer(Parameter):
         self.AllocateBatchsizeDependentMemory(batchsize)
         numdims = self.dimensions * self.numlabels
         self.dimsize = _zeros((numdims, 1))
+        if self.hyperparams.sparsity:
+            self.means = cm.CUDAMatrix(np.full((numdims, 1), self.hyperparams.sparsity_target, dtype=np.float32, order='F'))
+            self.sparsity_gradient = _zeros((numdims, 1))
+            self.means_temp2 = _zeros((numdims, 1))
         self.gradient = _zeros((numdims, 1))
         self.gradient_history = _zeros((numdims, 1))
 
@@ -92,13 +96,35 @@ class Layer(Parameter):
             self.pos_state, self.pos_sample = self.state, self.sample
             self.neg_state, self.neg_sample = _zeros(self.state.shape), _zeros(self.state.shape)
 
+    def GetSparsityGradient(self):
+        """layer.py:138-155: running mean activity of every unit (damped by sparsity_damping),
+        and cost * (mean - target) / divisor as the extra gradient."""
+        h = self.hyperparams
+        self.means.mult(h.sparsity_damping)
+        self.means.add_sums(self.state, axis=1, mult=(1 - h.sparsity_damping) / self.batchsize)
+        self.means.subtract(h.sparsity_target, target=self.sparsity_gradient)
+        self.sparsity_gradient.divide(self.GetSparsityDivisor())
+        self.sparsity_gradient.mult(h.sparsity_cost)
+        return self.sparsity_gradient
+
+    def GetSparsityDivisor(self):
+        """layer.py:256-258 (rectified linear units use it as it stands)."""
+        self.means_temp2.assign(1)
+        return self.means_temp2
+
     def CollectSufficientStatistics(self, neg=False):
-        """layer.py:194-205 without the sparsity term: the row sums of the state, added with
-        sign +1 in the positive and -1 in the negative phase."""
+        """layer.py:194-213: the row sums of the state, added with sign +1 in the positive and
+        -1 in the negative phase; with a sparsity target the positive statistics are moved
+        by -batchsize * sparsity gradient and the mean of the running means is returned."""
+        h = self.hyperparams
         if not neg:
             self.state.sum(axis=1, target=self.suff_stats)
+            if h.sparsity:
+                self.suff_stats.add_mult(self.GetSparsityGradient(), -self.batchsize)
+                return self.means.sum() / self.means.shape[0]
         else:
             self.suff_stats.add_sums(self.state, axis=1, mult=-1.0)
+        return None
 
     def SetData(self, data):
         self.data = data
@@ -144,6 +170,9 @@ class LinearLayer(Layer):
     """deepnet/linear_layer.py (without a learnt precision)."""
     activation = P.LINEAR
 
+    def GetSparsityDivisor(self):
+        raise Exception('Sparsity not implemented for linear units.')
+
     def ComputeDeriv(self):
         if self.hyperparams.dropout:
             self.deriv.mult(self.mask)
@@ -169,6 +198,13 @@ class LogisticLayer(Layer):
 
     def Sample(self):
         self.state.sample_bernoulli(target=self.sample)
+
+    def GetSparsityDivisor(self):
+        """logistic_layer.py:64-68: mean * (1 - mean)."""
+        self.means_temp2.assign(1)
+        self.means_temp2.subtract(self.means)
+        self.means_temp2.mult(self.means)
+        return self.means_temp2
 
     def ComputeDeriv(self):
         self.deriv.apply_logistic_deriv(self.state)
@@ -199,6 +235,9 @@ class TanhLayer(Layer):
 
     def Sample(self):
         self.state.sample_bernoulli_tanh(target=self.sample)
+
+    def GetSparsityDivisor(self):
+        raise Exception('Sparsity not implemented for tanh units.')
 
     def ComputeDeriv(self):
         self.deriv.apply_tanh_deriv(self.state)
@@ -249,6 +288,9 @@ class SoftmaxLayer(Layer):
     def Sample(self):
         self.state.perturb_prob_for_softmax_sampling(target=self.sample)
         self.sample.choose_max(axis=0)
+
+    def GetSparsityDivisor(self):
+        raise Exception('Sparsity not implemented for softmax units.')
 
     def ComputeDeriv(self):
         raise Exception('Back prop through softmax not implemented.')

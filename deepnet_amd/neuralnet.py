@@ -65,7 +65,13 @@ class Edge(Parameter):
         if not hasattr(self, 'suff_stats'):
             self.suff_stats = cm.empty(self.params['weight'].shape)
         if not neg:
+            # with sparsity targets the statistics are taken of state - sparsity gradient (:230-240)
+            sparse = [n for n in (self.node1, self.node2) if n.hyperparams.sparsity]
+            for n in sparse:
+                n.state.add_col_mult(n.sparsity_gradient, -1)
             cm.dot(self.node1.state, self.node2.state.T, target=self.suff_stats)
+            for n in sparse:
+                n.state.add_col_vec(n.sparsity_gradient)
         else:
             self.suff_stats.add_dot(self.node1.state, self.node2.state.T, mult=-1.0)
 
@@ -175,6 +181,8 @@ class NeuralNet(object):
             loss = layer.GetLoss(get_deriv=True)
         else:
             loss = None
+            if layer.hyperparams.sparsity:          # neuralnet.py:221-223
+                layer.deriv.add_col_vec(layer.GetSparsityGradient())
             layer.ComputeDeriv()
         for edge in layer.incoming_edge:
             if edge.conv or edge.local:

@@ -25,7 +25,7 @@ class Hyperparams(object):
         weight_norm=10.0, apply_l2_decay=False, l2_decay=0.01, activation=LINEAR, stop_dropout_for_last=0,
         start_learning_after=0, apply_l1_decay=False, l1_decay=0.01, apply_l1decay_after=0, blocksize=1,
         mult_dropout=False, sparsity=False, mf_steps=1, gibbs_steps=1, step_up_cd_after=0, start_step_up_cd_after=0,
-        sample_input=False, sample_input_after=0)
+        sample_input=False, sample_input_after=0, sparsity_target=0.1, sparsity_cost=0.001, sparsity_damping=0.9)
 
     def __init__(self, **fields):
         unknown = set(fields) - set(self._DEFAULTS)

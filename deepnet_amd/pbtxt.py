@@ -1,0 +1,210 @@
+"""Reader for deepnet's text-format configuration files (model / operation .pbtxt, the files
+deepnet/util.py:55-93 reads with protobuf's text_format.Merge) without generated protobuf
+classes: the text is parsed into a tree of ``Message`` objects that keep which fields were
+written, so that "merge the fields that are set" (the MergeFrom of deepnet/neuralnet.py:78-93)
+can be done on them.  Only the grammar is known here, not the schema: every field holds the
+list of values written for it, ``get`` returns the last one (what a non-repeated field ends
+up with), ``all`` the list (a repeated field).  Enum values stay as their names.
+"""
+import re
+
+_TOKEN = re.compile(r"""
+    \s+ | \#[^\n]*                                   # blanks and comments
+  | (?P<str>"(?:[^"\\\n]|\\.)*" | '(?:[^'\\\n]|\\.)*')
+  | (?P<num>[-+]?(?:\d+\.?\d*(?:[eE][-+]?\d+)?|\.\d+(?:[eE][-+]?\d+)?|inf|nan)f?(?![\w.]))
+  | (?P<name>[A-Za-z_][\w.]*)
+  | (?P<punct>[{}<>:;,\[\]])
+""", re.VERBOSE)
+
+_ESCAPES = {'n': '\n', 't': '\t', 'r': '\r', '\\': '\\', '"': '"', "'": "'", '0': '\0'}
+
+
+class ParseError(ValueError):
+    pass
+
+
+class Message(object):
+    """Fields in the order written.  ``msg.get('dimensions')``, ``msg.all('shape')``,
+    ``'hyperparams' in msg``; attribute access is ``get`` and raises for a field not written."""
+
+    def __init__(self, fields=None):
+        self._fields = list(fields or [])
+
+    def add(self, name, value):
+        self._fields.append((name, value))
+
+    def all(self, name):
+        return [v for n, v in self._fields if n == name]
+
+    def get(self, name, default=None):
+        for n, v in reversed(self._fields):
+            if n == name:
+                return v
+        return default
+
+    def names(self):
+        seen = []
+        for n, _ in self._fields:
+            if n not in seen:
+                seen.append(n)
+        return seen
+
+    def scalars(self):
+        """{name: last value} of the fields that are not sub-messages."""
+        return {n: v for n, v in self._fields if not isinstance(v, Message)}
+
+    def __contains__(self, name):
+        return any(n == name for n, _ in self._fields)
+
+    def __getattr__(self, name):
+        if name.startswith('_'):
+            raise AttributeError(name)
+        for n, v in reversed(self._fields):
+            if n == name:
+                return v
+        raise AttributeError('field %r was not written' % name)
+
+    def __eq__(self, other):
+        return isinstance(other, Message) and self._fields == other._fields
+
+    def __repr__(self):
+        return 'Message(%r)' % (self._fields,)
+
+
+def _tokens(text):
+    pos, line = 0, 1
+    while pos < len(text):
+        m = _TOKEN.match(text, pos)
+        if not m:
+            raise ParseError('line %d: cannot read %r' % (line, text[pos:pos + 20]))
+        line += text.count('\n', pos, m.end())
+        pos = m.end()
+        if m.lastgroup:
+            yield m.lastgroup, m.group(m.lastgroup), line
+    yield 'end', '', line
+
+
+def _unquote(tok):
+    body, out, i = tok[1:-1], [], 0
+    while i < len(body):
+        c = body[i]
+        if c == '\\':
+            i += 1
+            e = body[i]
+            if e == 'x':
+                out.append(chr(int(body[i + 1:i + 3], 16)))
+                i += 2
+            elif e in '01234567' and body[i:i + 3].isdigit():
+                out.append(chr(int(body[i:i + 3], 8)))
+                i += 2
+            else:
+                out.append(_ESCAPES.get(e, e))
+        else:
+            out.append(c)
+        i += 1
+    return ''.join(out)
+
+
+def _number(tok):
+    t = tok[:-1] if tok.endswith('f') and not tok.endswith('inf') else tok
+    try:
+        return int(t)
+    except ValueError:
+        return float(t)
+
+
+class _Parser(object):
+    def __init__(self, text):
+        self.toks = list(_tokens(text))
+        self.i = 0
+
+    def peek(self):
+        return self.toks[self.i]
+
+    def take(self):
+        t = self.toks[self.i]
+        self.i += 1
+        return t
+
+    def fail(self, what):
+        kind, val, line = self.peek()
+        raise ParseError('line %d: %s, found %r' % (line, what, val or kind))
+
+    def message(self, closer):
+        msg = Message()
+        while True:
+            kind, val, _ = self.peek()
+            if kind == 'punct' and val in ',;':
+                self.take()
+                continue
+            if closer is None and kind == 'end':
+                return msg
+            if closer is not None and kind == 'punct' and val == closer:
+                self.take()
+                return msg
+            if kind != 'name':
+                self.fail('expected a field name')
+            name = self.take()[1]
+            kind, val, _ = self.peek()
+            colon = kind == 'punct' and val == ':'
+            if colon:
+                self.take()
+                kind, val, _ = self.peek()
+            if kind == 'punct' and val in '{<':
+                self.take()
+                msg.add(name, self.message('}' if val == '{' else '>'))
+            elif not colon:
+                self.fail("expected ':' or '{' after %s" % name)
+            elif kind == 'punct' and val == '[':
+                self.take()
+                while True:
+                    kind, val, _ = self.peek()
+                    if kind == 'punct' and val == ']':
+                        self.take()
+                        break
+                    if kind == 'punct' and val == ',':
+                        self.take()
+                        continue
+                    msg.add(name, self.scalar())
+            else:
+                msg.add(name, self.scalar())
+
+    def scalar(self):
+        kind, val, _ = self.peek()
+        if kind == 'str':
+            parts = []
+            while self.peek()[0] == 'str':           # adjacent strings concatenate
+                parts.append(_unquote(self.take()[1]))
+            return ''.join(parts)
+        if kind == 'num':
+            return _number(self.take()[1])
+        if kind == 'name':
+            self.take()
+            if val in ('true', 'True', 't'):
+                return True
+            if val in ('false', 'False', 'f'):
+                return False
+            if val in ('inf', 'infinity', 'nan'):
+                return float(val[:3])
+            return val                                # an enum value, by name
+        self.fail('expected a value')
+
+
+def parse(text):
+    """The top-level message of a text-format file."""
+    return _Parser(text).message(None)
+
+
+def merged(base, over):
+    """``base`` with the fields written in ``over`` on top: non-repeated semantics, scalar
+    fields replaced, sub-messages merged recursively (protobuf's MergeFrom for the messages
+    deepnet merges, which hold no repeated fields)."""
+    out = Message()
+    for name in list(base.names() if base else []) + [n for n in (over.names() if over else []) if not base or n not in base]:
+        b = base.get(name) if base and name in base else None
+        o = over.get(name) if over and name in over else None
+        if isinstance(b, Message) or isinstance(o, Message):
+            out.add(name, merged(b if isinstance(b, Message) else None, o if isinstance(o, Message) else None))
+        else:
+            out.add(name, o if o is not None else b)
+    return out

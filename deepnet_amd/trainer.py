@@ -1,0 +1,172 @@
+"""Build a net on the device from deepnet's own model files.
+
+``CreateDeepnet(model, train_op, eval_op)`` has the role of deepnet/trainer.py:34-46 followed
+by ``LoadModelOnGPU`` (deepnet/neuralnet.py:70-109): the model-wide hyper-parameters are merged
+under those of every layer and edge, parameters are initialised as deepnet/parameter.py:43-71
+does (same numpy generator, seeded with the model's seed, same order: layers, then edges, as
+listed), layers and edges are created and sorted.  ``model`` / ``train_op`` are the parsed
+text files (``util.ReadModel`` / ``util.ReadOperation``), paths to them, or their text.
+A field that would change the arithmetic of a step and has no counterpart here (tied
+parameters, pretrained initialisation, sparsity, replicated softmax, ...) raises
+NotImplementedError by name instead of being dropped.
+"""
+import os
+
+import numpy as np
+
+from . import pbtxt
+from .choose_matrix_library import cm
+from .convolutions import ConvParams
+from .dbm import DBM
+from .layer import LAYER_TYPES
+from .neuralnet import Edge, NeuralNet
+from .parameter import Hyperparams
+
+# Hyperparams fields that switch on behaviour this package does not have: refused when set.
+_SWITCHES = ('adapt', 'normalize', 'learn_precision', 'add_noise', 'shift', 'fast_dropout',
+             'shared_prior', 'soft_shared_prior', 'left_window', 'right_window', 'decay_learning_rate_for_last',
+             'additive_prior', 'multiplicative_prior', 'adaptive_prior')
+_OFF = (False, 0, 0.0, 'NO_ADAPT', None)
+
+_CONV_FIELDS = ('size', 'stride', 'padding', 'num_filters', 'num_colors', 'max_pool', 'pool_size', 'pool_stride',
+                'rnorm', 'norm_size', 'pow_scale', 'add_scale', 'prob')
+
+
+def _as_message(x):
+    if x is None or isinstance(x, pbtxt.Message):
+        return x
+    if isinstance(x, str) and '\n' not in x and os.path.exists(x):
+        with open(x) as f:
+            return pbtxt.parse(f.read())
+    return pbtxt.parse(x)
+
+
+def _hyperparams(model_hyp, own_hyp, where):
+    """deepnet/neuralnet.py:80-93: the model's fields, overwritten by the fields written for
+    this layer / edge; everything else at the defaults of the message."""
+    fields = pbtxt.merged(model_hyp, own_hyp).scalars()
+    for name in _SWITCHES:
+        if fields.get(name) not in _OFF:
+            raise NotImplementedError('%s: hyperparams.%s = %r is not supported' % (where, name, fields[name]))
+    known = {k: v for k, v in fields.items() if k in Hyperparams._DEFAULTS}
+    return Hyperparams(**known)
+
+
+def InitializeParameter(param, dims):
+    """deepnet/parameter.py:43-71 on the numpy global generator (seeded by the caller)."""
+    kind = param.get('initialization', 'CONSTANT')
+    sigma = param.get('sigma', 0.001)
+    if kind == 'CONSTANT':
+        return np.zeros(tuple(dims)) + param.get('constant', 0.0)
+    if kind == 'DENSE_GAUSSIAN':
+        return sigma * np.random.randn(*dims)
+    if kind == 'DENSE_UNIFORM':
+        return sigma * (2 * np.random.rand(*dims) - 1)
+    if kind in ('DENSE_GAUSSIAN_SQRT_FAN_IN', 'DENSE_UNIFORM_SQRT_FAN_IN'):
+        assert len(dims) > 1
+        # (the reference takes dimensions[0], the filter count, as the fan-in of conv / local weights)
+        fan_in = dims[0] if (param.get('conv', False) or param.get('local', False)) else dims[1]
+        stddev = sigma / np.sqrt(fan_in)
+        if kind == 'DENSE_GAUSSIAN_SQRT_FAN_IN':
+            return stddev * np.random.randn(*dims)
+        return stddev * (2 * np.random.rand(*dims) - 1)
+    if kind == 'PRETRAINED':
+        raise NotImplementedError('parameter %s: PRETRAINED initialisation is not supported' % param.get('name'))
+    raise Exception('Unknown parameter initialization.')
+
+
+def _refuse(msg, fields, where):
+    for name in fields:
+        if msg.get(name) not in _OFF and msg.get(name) != '':
+            raise NotImplementedError('%s: %s is not supported' % (where, name))
+
+
+def _layer(proto, model_hyp, batchsize):
+    name = proto.name
+    _refuse(proto, ('tied', 'is_initialized'), 'layer ' + name)
+    hyp = _hyperparams(model_hyp, proto.get('hyperparams'), 'layer ' + name)
+    if hyp.activation not in LAYER_TYPES:
+        raise NotImplementedError('layer %s: activation %s is not supported' % (name, hyp.activation))
+    dims, numlabels = proto.dimensions, proto.get('numlabels', 1)
+    bias = None
+    for param in proto.all('param'):
+        if param.name != 'bias':
+            raise NotImplementedError('layer %s: parameter %s is not supported' % (name, param.name))
+        if 'mat' in param:
+            raise NotImplementedError('layer %s: stored parameter values are not read from text files' % name)
+        pdims = param.all('dimensions') or [numlabels * dims, 1]
+        if len(pdims) == 1:
+            pdims = pdims + [1]
+        bias = InitializeParameter(param, pdims)
+    return LAYER_TYPES[hyp.activation](
+        name, dims, batchsize, hyperparams=hyp, numlabels=numlabels, is_input=proto.get('is_input', False),
+        is_output=proto.get('is_output', False), loss_function=proto.get('loss_function', 'SQUARED_LOSS'),
+        loss_weight=proto.get('loss_weight', 1.0), bias=bias)
+
+
+def _edge(proto, model_hyp, layers):
+    where = 'edge %s:%s' % (proto.node1, proto.node2)
+    _refuse(proto, ('tied', 'tied_transpose'), where)
+    hyp = _hyperparams(model_hyp, proto.get('hyperparams'), where)
+    by_name = {l.name: l for l in layers}
+    node1, node2 = by_name[proto.node1], by_name[proto.node2]
+    params = proto.all('param')
+    if len(params) != 1 or params[0].name != 'weight':
+        raise NotImplementedError('%s: exactly one parameter, "weight", is supported' % where)
+    param = params[0]
+    if 'mat' in param:
+        raise NotImplementedError('%s: stored parameter values are not read from text files' % where)
+    conv, local = param.get('conv', False), param.get('local', False)
+    cv = None
+    if conv or local:
+        cvm = param.get('conv_params') or pbtxt.Message()
+        cv = ConvParams(**{k: cvm.get(k) for k in _CONV_FIELDS if k in cvm})
+    dims = param.all('dimensions')
+    if not dims:
+        if conv:
+            dims = [cv.num_filters, cv.size ** 2 * cv.num_colors]
+        elif local:
+            side = int(round((node1.dimensions * node1.numlabels // cv.num_colors) ** 0.5))
+            n_locs = (side + 2 * cv.padding - cv.size) // cv.stride + 1
+            dims = [cv.num_filters, n_locs ** 2 * cv.size ** 2 * cv.num_colors]
+        else:
+            dims = [node1.numlabels * node1.dimensions, node2.numlabels * node2.dimensions]
+    weight = InitializeParameter(param, dims)
+    return Edge(node1, node2, weight, hyperparams=hyp, conv_params=cv, local=bool(local),
+                up_factor=proto.get('up_factor', 1.0), block_gradient=proto.get('block_gradient', False),
+                down_factor=proto.get('down_factor', 1.0), directed=proto.get('directed', True))
+
+
+def CreateDeepnet(model, train_op=None, eval_op=None, batchsize=None):
+    """A NeuralNet (FEED_FORWARD_NET) or DBM (DBM) with its parameters on the device."""
+    model, train_op, eval_op = _as_message(model), _as_message(train_op), _as_message(eval_op)
+    op = train_op or eval_op
+    if batchsize is None:
+        if op is None:
+            raise ValueError('a batch size or an operation that names one is needed')
+        batchsize = op.get('batchsize', 1)
+    seed = model.get('seed', 0)
+    cm.CUDAMatrix.init_random(seed)          # deepnet/neuralnet.py:43-44
+    np.random.seed(seed)
+    model_hyp = model.get('hyperparams')
+    layers = [_layer(p, model_hyp, batchsize) for p in model.all('layer')]
+    edges = [_edge(p, model_hyp, layers) for p in model.all('edge')]
+    by_name = {l.name: l for l in layers}
+    kind = model.model_type
+    if kind == 'FEED_FORWARD_NET':
+        net = NeuralNet(layers, edges, verbose=bool(op and op.get('verbose', False)))
+    elif kind == 'DBM':
+        h = _hyperparams(model_hyp, None, 'model')
+        optimizer = train_op.get('optimizer', 'CD') if train_op else 'CD'
+        if optimizer not in ('CD', 'PCD'):
+            raise NotImplementedError('a DBM is trained with CD or PCD, not %s' % optimizer)
+        net = DBM(layers, edges, optimizer=optimizer, mf_steps=h.mf_steps, gibbs_steps=h.gibbs_steps,
+                  start_step_up_cd_after=h.start_step_up_cd_after, step_up_cd_after=h.step_up_cd_after,
+                  positive_phase_order=[by_name[n] for n in model.all('positive_phase_order')] or None,
+                  negative_phase_order=[by_name[n] for n in model.all('negative_phase_order')] or None)
+    else:
+        raise NotImplementedError('model_type %s is not supported' % kind)
+    net.net, net.t_op, net.e_op, net.batchsize = model, train_op, eval_op, batchsize
+    if train_op and 'stopcondition' in train_op and train_op.stopcondition.get('steps', 0) > 0:
+        net.train_stop_steps = train_op.stopcondition.steps
+    return net

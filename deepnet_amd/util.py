@@ -2,6 +2,8 @@
 reference keeps in ``Parameter.mat`` with the shape in ``Parameter.dimensions``
 (deepnet/util.py:13-21, deepnet/parameter.py:17-19).  Works on any object with ``name``, ``mat``
 and ``dimensions`` attributes, e.g. a message of the reference's deepnet_pb2 or ``ParamRecord``."""
+import os
+
 import numpy as np
 
 
@@ -42,3 +44,22 @@ def LoadParameters(obj, records):
             obj.params[rec.name].overwrite(mat)
         else:
             obj.params[rec.name] = cm.CUDAMatrix(mat)
+
+
+def _read_text_message(path):
+    from . import pbtxt
+    if os.path.splitext(path)[1] != '.pbtxt':
+        raise NotImplementedError('%s: only text-format (.pbtxt) files are read; binary protocol '
+                                  'buffers need the generated message classes' % path)
+    with open(path) as f:
+        return pbtxt.parse(f.read())
+
+
+def ReadModel(proto_file):
+    """deepnet/util.py:67-77 for text-format files: the Model message as a pbtxt.Message tree."""
+    return _read_text_message(proto_file)
+
+
+def ReadOperation(proto_file):
+    """deepnet/util.py:55-65 for text-format files."""
+    return _read_text_message(proto_file)

@@ -32,7 +32,25 @@ class Hyper(object):
         self.apply_l1decay_after, self.apply_weight_norm, self.weight_norm = 0, False, 10.0
         self.start_learning_after = 0
         self.dropout, self.dropout_prob = False, 0.5
+        self.sparsity, self.sparsity_target, self.sparsity_cost, self.sparsity_damping = False, 0.1, 0.001, 0.9
         self.__dict__.update(kw)
+
+
+def sparsity_gradient(h, act, means, state):
+    """layer.py:138-155 with the divisors of logistic_layer.py:64-68 (mean * (1 - mean)) and
+    layer.py:256-258 (1, rectified linear units): the running means after seeing ``state`` and
+    cost * (mean - target) / divisor.  For logistic units this is cost * d/d(mean) of the
+    Kullback-Leibler divergence between Bernoulli(target) and Bernoulli(mean), which is what
+    tests/test_oracle_net.py checks it against by finite differences."""
+    d = F64(np.float32(h.sparsity_damping))
+    means = d * means + F64(np.float32((1 - h.sparsity_damping) / state.shape[1])) * state.sum(axis=1, keepdims=True)
+    if act == 'LOGISTIC':
+        div = means * (1.0 - means)
+    elif act == 'RECTIFIED_LINEAR':
+        div = 1.0
+    else:
+        raise ValueError('sparsity targets exist for logistic and rectified linear units')
+    return means, F64(np.float32(h.sparsity_cost)) * (means - F64(np.float32(h.sparsity_target))) / div
 
 
 def momentum_and_epsilon(h, step):
@@ -161,6 +179,11 @@ class Net(object):
         for i in range(len(self.layers) - 1, 0, -1):
             L, e = self.layers[i], self.layers[i]['edge']
             if i < len(self.layers) - 1:
+                if L['hyper'].sparsity:               # neuralnet.py:221-223
+                    if 'means' not in L:
+                        L['means'] = np.full((d.shape[0], 1), F64(np.float32(L['hyper'].sparsity_target)))
+                    L['means'], grad = sparsity_gradient(L['hyper'], L['act'], L['means'], self.states[i])
+                    d = d + grad
                 d = self._through_activation(i, d)
             below = self.states[i - 1]
             if e.get('cv') is not None:
@@ -181,7 +204,8 @@ def rbm_cd_step(p, hyper, v_data, step, hid_samples, vis_act='LOGISTIC', hid_act
     hidden), 'bv', 'bh' (column vectors) and the previous updates 'dW', 'dbv', 'dbh'; hyper the
     Hyper objects 'edge', 'vis', 'hid'.  hid_samples[i] is the hidden sample that drives Gibbs sweep
     i (the caller feeds the ones the device drew), so len(hid_samples) sweeps are made.  Returns
-    the squared reconstruction error of the first sweep.
+    the squared reconstruction error of the first sweep.  A sparsity target on the hidden layer
+    moves the positive statistics by the sparsity gradient.
 
     Pinned by tests/test_oracle_net.py against the C coding of the CD-1 step in
     oracle/host_backend.c (hb_rbm_cd1_step, written from cudamat/examples/rbm_cudamat.py:46-89)
@@ -191,6 +215,14 @@ def rbm_cd_step(p, hyper, v_data, step, hid_samples, vis_act='LOGISTIC', hid_act
     W, bv, bh = p['W'], p['bv'], p['bh']
     h = activate(hid_act, W.T @ v + bh)
     stats_W, stats_v, stats_h = v @ h.T, v.sum(axis=1, keepdims=True), h.sum(axis=1, keepdims=True)
+    if hyper['hid'].sparsity:
+        # hidden units with a sparsity target (layer.py:206-209, edge.py:230-240): p['means_h'] carries
+        # the running means from step to step
+        if 'means_h' not in p:
+            p['means_h'] = np.full_like(bh, F64(np.float32(hyper['hid'].sparsity_target)))
+        p['means_h'], grad = sparsity_gradient(hyper['hid'], hid_act, p['means_h'], h)
+        stats_h = stats_h - B * grad
+        stats_W = v @ (h - grad).T
     error = None
     for i, hs in enumerate(hid_samples):
         v_neg = activate(vis_act, W @ np.asarray(hs, dtype=F64) + bv)

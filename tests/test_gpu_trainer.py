@@ -1,0 +1,193 @@
+"""Nets built from deepnet's own model files (deepnet_amd/trainer.py: the role of
+deepnet/trainer.py:34-46 + deepnet/neuralnet.py:70-109 + deepnet/parameter.py:21-71): the initial
+parameters against the numpy draws the reference makes (same seed, same order), the merged
+hyper-parameters, and training steps against the float64 restatement in oracle/net_oracle.py
+(parameters within 1e-4 relative + 1e-6, losses within 1e-5 relative).  The model files under
+tests/golden/ were written for these tests in the format of deepnet/examples/*/model*.pbtxt."""
+import os
+import sys
+
+import numpy as np
+import pytest
+
+sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+from oracle import net_oracle as no   # noqa: E402
+
+pytestmark = pytest.mark.gpu
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), 'golden')
+TRAIN_OP = 'optimizer: %s\nstopcondition { steps: 100 }\ntrain: true\nbatchsize: 32\ndata_proto: "unused.pbtxt"\n'
+
+
+def _f(a):
+    return np.asarray(a, dtype=np.float32, order='F')
+
+
+def _ohyper(h):
+    return no.Hyper(**{k: getattr(h, k) for k in vars(no.Hyper()) if hasattr(h, k)})
+
+
+def _oracle_chain(net, order):
+    """The oracle's list-of-dicts form of a chain-shaped device net, from the device's parameters."""
+    by_name = {l.name: l for l in net.layer}
+    out = []
+    for i, name in enumerate(order):
+        L = by_name[name]
+        d = {'act': L.activation, 'hyper': _ohyper(L.hyperparams)}
+        if i:
+            E = next(e for e in net.edge if e.node2 is L)
+            assert E.node1 is by_name[order[i - 1]]
+            d.update(bias=L.params['bias'].asarray().astype(np.float64), loss=L.loss_function,
+                     edge={'w': E.params['weight'].asarray().astype(np.float64), 'hyper': _ohyper(E.hyperparams),
+                           'cv': getattr(E, 'conv_params', None), 'local': E.local})
+        out.append(d)
+    return no.Net(out), [by_name[n] for n in order]
+
+
+def _steps_match(cm, net, onet, chain, batches):
+    for step, (x, t) in enumerate(batches):
+        chain[0].data.assign(cm.CUDAMatrix(_f(x)))
+        chain[-1].data.assign(cm.CUDAMatrix(_f(t)))
+        losses = net.TrainOneBatch(step)
+        masks = [L.mask.asarray().copy() if L.hyperparams.dropout else None for L in chain]
+        perf = onet.train_step(x, t, step, masks=masks)
+        assert len(losses) == 1
+        for key, want in perf.items():
+            assert abs(getattr(losses[0], key) - want) <= 1e-5 * max(1.0, abs(want)), (step, key)
+        for i, L in enumerate(chain[1:], 1):
+            E = next(e for e in net.edge if e.node2 is L)
+            assert np.allclose(E.params['weight'].asarray(), onet.layers[i]['edge']['w'], rtol=1e-4, atol=1e-6), (step, i)
+            assert np.allclose(L.params['bias'].asarray(), onet.layers[i]['bias'], rtol=1e-4, atol=1e-6), (step, i)
+
+
+def test_convnet_from_a_model_file(cm, cc):
+    from deepnet_amd import trainer, util, layer as dl, neuralnet as dnn
+    model = util.ReadModel(os.path.join(GOLDEN, 'small_convnet.pbtxt'))
+    net = trainer.CreateDeepnet(model, TRAIN_OP % 'GRADIENT_DESCENT')
+    assert type(net) is dnn.NeuralNet and net.batchsize == 32 and net.train_stop_steps == 100
+    by_name = {l.name: l for l in net.layer}
+    assert [type(by_name[n]) for n in ('input_layer', 'output_layer', 'hidden1', 'hidden3')] == \
+        [dl.LinearLayer, dl.SoftmaxLayer, dl.ReluLayer, dl.ReluLayer]
+    assert [n.name for n in net.node_list] == ['input_layer', 'hidden1', 'hidden2', 'hidden3', 'output_layer']
+
+    # parameter.py:43-71 on numpy's global generator, seeded with the model's seed: layers, then edges, as listed
+    r = np.random.RandomState(17)
+    want = {'output_layer': np.zeros((10, 1)), 'hidden1': np.zeros((400, 1)) + 0.1,
+            'hidden2': 0.01 * r.randn(144, 1), 'hidden3': np.zeros((64, 1))}
+    want_w = [0.1 * r.randn(16, 18), (1.0 / np.sqrt(16)) * r.randn(16, 9 * 9 * 16),
+              (1.0 / np.sqrt(64)) * (2 * r.rand(144, 64) - 1), 0.1 * (2 * r.rand(64, 10) - 1)]
+    for name, b in want.items():
+        assert np.array_equal(by_name[name].params['bias'].asarray(), b.astype(np.float32)), name
+    for E, w in zip(net.edge, want_w):
+        assert np.array_equal(E.params['weight'].asarray(), w.astype(np.float32)), E.name
+    assert net.edge[0].conv and net.edge[1].local and not (net.edge[2].conv or net.edge[2].local)
+
+    # neuralnet.py:80-93: the model's hyper-parameters under those written for the layer / edge
+    h1, h3, e0, e1 = by_name['hidden1'].hyperparams, by_name['hidden3'].hyperparams, net.edge[0].hyperparams, net.edge[1].hyperparams
+    assert (h1.activation, h1.apply_l2_decay, h1.base_epsilon, h1.final_momentum) == ('RECTIFIED_LINEAR', False, 0.05, 0.9)
+    assert (h3.dropout, h3.dropout_prob, h3.apply_l2_decay) == (True, 0.5, True)
+    assert (e0.base_epsilon, e0.initial_momentum, e0.final_momentum, e0.momentum_change_steps, e0.apply_l2_decay) == \
+        (0.01, 0.9, 0.9, 5, False)
+    assert (e1.base_epsilon, e1.initial_momentum, e1.apply_l2_decay, e1.l2_decay) == (0.05, 0.5, True, 0.001)
+    assert by_name['output_layer'].hyperparams.dropout is False and by_name['output_layer'].loss_function == 'CROSS_ENTROPY'
+
+    order = ['input_layer', 'hidden1', 'hidden2', 'hidden3', 'output_layer']
+    onet, chain = _oracle_chain(net, order)
+    rng = np.random.default_rng(4)
+    batches = [(rng.standard_normal((288, 32)), rng.integers(0, 10, (1, 32)).astype(np.float64)) for _ in range(3)]
+    _steps_match(cm, net, onet, chain, batches)
+
+
+DENSE_SPARSE = '''
+name: "sparse_ff"  model_type: FEED_FORWARD_NET  seed: 3
+hyperparams { base_epsilon: 0.1 initial_momentum: 0.5 final_momentum: 0.5 activation: LOGISTIC }
+layer { name: "in" dimensions: 40 is_input: true hyperparams { activation: LINEAR } }
+layer { name: "h1" dimensions: 48 param { name: "bias" initialization: CONSTANT }
+        hyperparams { sparsity: true sparsity_target: 0.1 sparsity_cost: 0.5 sparsity_damping: 0.5 } }
+layer { name: "h2" dimensions: 24 param { name: "bias" initialization: CONSTANT }
+        hyperparams { activation: RECTIFIED_LINEAR sparsity: true sparsity_target: 0.05 sparsity_cost: 0.25 } }
+layer { name: "out" dimensions: 8 is_output: true loss_function: CROSS_ENTROPY param { name: "bias" initialization: CONSTANT } }
+edge { node1: "in" node2: "h1" param { name: "weight" initialization: DENSE_GAUSSIAN sigma: 0.3 } }
+edge { node1: "h1" node2: "h2" param { name: "weight" initialization: DENSE_GAUSSIAN sigma: 0.3 } }
+edge { node1: "h2" node2: "out" param { name: "weight" initialization: DENSE_GAUSSIAN sigma: 0.3 } }
+'''
+
+
+def test_sparsity_targets_on_hidden_layers_of_a_feed_forward_net(cm):
+    """neuralnet.py:221-223 + layer.py:138-155: logistic units (divisor mean (1 - mean)) and
+    rectified linear units (divisor 1), running means carried from step to step."""
+    from deepnet_amd import trainer
+    net = trainer.CreateDeepnet(DENSE_SPARSE, batchsize=16)
+    onet, chain = _oracle_chain(net, ['in', 'h1', 'h2', 'out'])
+    rng = np.random.default_rng(9)
+    batches = [(rng.standard_normal((40, 16)), (rng.random((8, 16)) < 0.3).astype(np.float64)) for _ in range(4)]
+    _steps_match(cm, net, onet, chain, batches)
+    for i in (1, 2):
+        assert np.allclose(chain[i].means.asarray(), onet.layers[i]['means'], rtol=1e-5)
+    assert abs(float(onet.layers[1]['means'].mean()) - 0.1) > 0.05       # the means did move away from the target
+
+
+def test_rbm_with_a_sparsity_target_from_a_model_file(cm):
+    """layer.py:206-212, edge.py:230-240, dbm.py:147-153 through the two-layer DBM."""
+    from deepnet_amd import trainer, dbm
+    net = trainer.CreateDeepnet(os.path.join(GOLDEN, 'small_rbm.pbtxt'), TRAIN_OP % 'CD')
+    assert type(net) is dbm.DBM and net.cd and net.gibbs_steps == 2 and net.batchsize == 32
+    vis, hid = net.layer
+    edge = net.edge[0]
+    assert edge in vis.incoming_edge and edge in hid.outgoing_edge           # directed: false
+    r = np.random.RandomState(0)                                             # no seed written: 0
+    w0 = ((1.0 / np.sqrt(64)) * r.randn(96, 64)).astype(np.float32)
+    assert np.array_equal(edge.params['weight'].asarray(), w0)
+    assert np.all(hid.params['bias'].asarray() == -1.0)
+    p = {'W': w0.astype(np.float64), 'bv': np.zeros((96, 1)), 'bh': np.full((64, 1), -1.0),
+         'dW': np.zeros((96, 64)), 'dbv': np.zeros((96, 1)), 'dbh': np.zeros((64, 1))}
+    oh = {'edge': _ohyper(edge.hyperparams), 'vis': _ohyper(vis.hyperparams), 'hid': _ohyper(hid.hyperparams)}
+    assert oh['hid'].sparsity and not oh['vis'].sparsity and oh['edge'].apply_l2_decay
+    drawn, original = [], hid.Sample
+
+    def sample():
+        original()
+        drawn.append(hid.sample.asarray().copy())
+    hid.Sample = sample
+    rng = np.random.default_rng(12)
+    for step in range(4):
+        v = (rng.random((96, 32)) < 0.3).astype(np.float64)
+        vis.data.assign(cm.CUDAMatrix(_f(v)))
+        del drawn[:]
+        losses = net.TrainOneBatch(step)
+        err = no.rbm_cd_step(p, oh, v, step, drawn[:2])
+        sparsity = [l.sparsity for l in losses if hasattr(l, 'sparsity')]
+        errors = [l.error for l in losses if hasattr(l, 'error')]
+        assert len(losses) == 2 and len(sparsity) == 1 and len(errors) == 1
+        assert abs(sparsity[0] - float(p['means_h'].mean())) <= 1e-5
+        assert abs(errors[0] - err) <= 1e-5 * err
+        assert np.allclose(hid.means.asarray(), p['means_h'], rtol=1e-5)
+        for got, want in ((edge.params['weight'], p['W']), (vis.params['bias'], p['bv']), (hid.params['bias'], p['bh'])):
+            assert np.allclose(got.asarray(), want, rtol=1e-4, atol=1e-6), step
+        # the hidden state is restored after the statistics were taken of state - gradient
+    assert float(p['means_h'].mean()) > 0.2                                  # activity above the target: the term is live
+
+
+@pytest.mark.parametrize("text,what", [
+    ('name: "m" model_type: DBN', 'model_type'),
+    ('name: "m" model_type: FEED_FORWARD_NET layer { name: "a" dimensions: 4 tied: true tied_to: "b" }', 'tied'),
+    ('name: "m" model_type: FEED_FORWARD_NET layer { name: "a" dimensions: 4 hyperparams { activation: REPLICATED_SOFTMAX } }', 'activation'),
+    ('name: "m" model_type: FEED_FORWARD_NET layer { name: "a" dimensions: 4 hyperparams { adapt: ADAGRAD } }', 'adapt'),
+    ('name: "m" model_type: FEED_FORWARD_NET layer { name: "a" dimensions: 4 param { name: "bias" initialization: PRETRAINED } }', 'PRETRAINED'),
+    ('name: "m" model_type: FEED_FORWARD_NET layer { name: "a" dimensions: 4 hyperparams { activation: TANH sparsity: true } is_input: true }'
+     ' layer { name: "b" dimensions: 4 hyperparams { activation: TANH sparsity: true } }'
+     ' layer { name: "c" dimensions: 2 is_output: true }'
+     ' edge { node1: "a" node2: "b" param { name: "weight" } } edge { node1: "b" node2: "c" param { name: "weight" } }', None),
+])
+def test_what_the_builder_does_not_have_is_refused_by_name(cm, text, what):
+    from deepnet_amd import trainer
+    if what is None:
+        # builds, and fails where the reference fails too: tanh units have no sparsity divisor (tanh_layer.py:45-50
+        # reads a buffer that is never allocated)
+        net = trainer.CreateDeepnet(text, batchsize=4)
+        net.layer[0].data.assign(cm.CUDAMatrix(_f(np.ones((4, 4)))))
+        net.layer[2].data.assign(cm.CUDAMatrix(_f(np.ones((2, 4)))))
+        with pytest.raises(Exception, match='Sparsity not implemented'):
+            net.TrainOneBatch(0)
+        return
+    with pytest.raises(NotImplementedError, match=what):
+        trainer.CreateDeepnet(text, batchsize=4)

@@ -179,3 +179,72 @@ def test_rbm_cd_step_against_the_c_coding_and_a_fixed_point(rng):
     assert np.allclose(z['W'], eps / B * 0.5 * rowsum * np.ones((1, nh)), rtol=1e-6, atol=1e-12)
     assert np.allclose(z['bv'], eps / B * rowsum, rtol=1e-6, atol=1e-12) and np.allclose(z['bh'], 0.0, atol=1e-12)
     assert abs(err - 0.25 * nv * B) < 1e-9
+
+
+def test_sparsity_term_is_the_kl_gradient_and_enters_both_kinds_of_step(rng):
+    """layer.py:138-155.  (1) For logistic units cost * (mean - target) / (mean (1 - mean)) is the
+    derivative of cost * KL(Bernoulli(target) || Bernoulli(mean)): checked by central differences,
+    and the running mean by writing the recursion out.  (2) With damping 0 the mean is the batch
+    mean, so a feed-forward step equals torch SGD on loss + B * cost * sum_i KL(target || mean_i).
+    (3) An RBM at W = 0, b = 0 has every unit at 1/2, which gives the update in closed form."""
+    h = no.Hyper(sparsity=True, sparsity_target=0.25, sparsity_cost=0.125, sparsity_damping=0.5)
+    state1, state2 = rng.random((5, 4)), rng.random((5, 4))
+    m0 = np.full((5, 1), 0.25)
+    m1, g1 = no.sparsity_gradient(h, 'LOGISTIC', m0, state1)
+    m2, g2 = no.sparsity_gradient(h, 'LOGISTIC', m1, state2)
+    assert np.allclose(m2, 0.25 * 0.25 + 0.25 * state1.mean(axis=1, keepdims=True) + 0.5 * state2.mean(axis=1, keepdims=True),
+                       rtol=0, atol=1e-15)
+    kl = lambda m: 0.25 * np.log(0.25 / m) + 0.75 * np.log(0.75 / (1 - m))
+    d = 1e-6
+    assert np.allclose(g2, 0.125 * (kl(m2 + d) - kl(m2 - d)) / (2 * d), rtol=1e-7)
+    _, g_relu = no.sparsity_gradient(h, 'RECTIFIED_LINEAR', m1, state2)
+    assert np.allclose(g_relu, 0.125 * (m2 - 0.25), rtol=0, atol=1e-15)
+    with pytest.raises(ValueError):
+        no.sparsity_gradient(h, 'TANH', m0, state1)
+
+    # (2) feed-forward, batch of 8 so that 1/B is the same number in float32 and float64
+    sizes, B, steps = (12, 9, 7, 5), 8, 3
+    eps, mom = float(np.float32(0.05)), float(np.float32(0.9))
+    he = no.Hyper(base_epsilon=eps, initial_momentum=mom, final_momentum=mom)
+    hs = no.Hyper(base_epsilon=eps, initial_momentum=mom, final_momentum=mom, sparsity=True, sparsity_target=0.25,
+                  sparsity_cost=0.125, sparsity_damping=0.0)
+    Ws = [0.3 * rng.standard_normal((sizes[i], sizes[i + 1])) for i in range(3)]
+    bs = [0.1 * rng.standard_normal((sizes[i + 1], 1)) for i in range(3)]
+    net = no.Net([{'act': 'LINEAR', 'hyper': he},
+                  {'act': 'LOGISTIC', 'hyper': he, 'bias': bs[0], 'edge': {'w': Ws[0], 'hyper': he}},
+                  {'act': 'LOGISTIC', 'hyper': hs, 'bias': bs[1], 'edge': {'w': Ws[1], 'hyper': he}},
+                  {'act': 'SOFTMAX', 'hyper': he, 'bias': bs[2], 'edge': {'w': Ws[2], 'hyper': he}, 'loss': 'CROSS_ENTROPY'}])
+    tw = [torch.tensor(w, requires_grad=True) for w in Ws]
+    tb = [torch.tensor(b, requires_grad=True) for b in bs]
+    opt = torch.optim.SGD(tw + tb, lr=eps, momentum=mom)
+    for step in range(steps):
+        x = rng.standard_normal((sizes[0], B))
+        targets = rng.integers(0, sizes[-1], (1, B)).astype(np.float64)
+        net.train_step(x, targets, step)
+        opt.zero_grad()
+        a1 = torch.sigmoid(tw[0].T @ torch.tensor(x) + tb[0])
+        a2 = torch.sigmoid(tw[1].T @ a1 + tb[1])
+        z = tw[2].T @ a2 + tb[2]
+        m = a2.mean(dim=1)
+        penalty = (0.25 * torch.log(0.25 / m) + 0.75 * torch.log(0.75 / (1 - m))).sum()
+        L = TF.cross_entropy(z.T, torch.tensor(targets.ravel()).long(), reduction='sum') + B * 0.125 * penalty
+        (L / B).backward()
+        opt.step()
+        for i in range(3):
+            assert np.allclose(net.layers[i + 1]['edge']['w'], tw[i].detach().numpy(), rtol=0, atol=1e-12), (step, i)
+            assert np.allclose(net.layers[i + 1]['bias'], tb[i].detach().numpy(), rtol=0, atol=1e-12), (step, i)
+
+    # (3) RBM at the origin: all probabilities 1/2
+    nv, nh = 6, 4
+    hr = no.Hyper(base_epsilon=eps, sparsity=True, sparsity_target=0.25, sparsity_cost=0.125, sparsity_damping=0.5)
+    plain = no.Hyper(base_epsilon=eps)
+    p = {'W': np.zeros((nv, nh)), 'bv': np.zeros((nv, 1)), 'bh': np.zeros((nh, 1)),
+         'dW': np.zeros((nv, nh)), 'dbv': np.zeros((nv, 1)), 'dbh': np.zeros((nh, 1))}
+    v = (rng.random((nv, B)) < 0.5).astype(np.float64)
+    no.rbm_cd_step(p, {'edge': plain, 'vis': plain, 'hid': hr}, v, 0, [np.zeros((nh, B))])
+    mean = 0.5 * 0.25 + 0.5 * 0.5
+    g = 0.125 * (mean - 0.25) / (mean * (1 - mean))
+    assert np.allclose(p['means_h'], mean, rtol=0, atol=1e-15)
+    assert np.allclose(p['bh'], -eps * g, rtol=0, atol=1e-15)
+    assert np.allclose(p['W'], eps * (v.sum(axis=1, keepdims=True) * (0.5 - g) / B - 0.25) * np.ones((1, nh)), rtol=0, atol=1e-15)
+    assert np.allclose(p['bv'], eps * (v.mean(axis=1, keepdims=True) - 0.5), rtol=0, atol=1e-15)
