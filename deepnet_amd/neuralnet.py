@@ -10,6 +10,7 @@ instead of a protobuf model; data handlers, model files, evaluation loops over d
 tied parameters and replicated-softmax neighbours stay outside.
 """
 import sys
+import types
 
 import numpy as np
 
@@ -104,6 +105,7 @@ class NeuralNet(object):
         self.input_datalayer = [n for n in self.layer if n.is_input]
         self.output_datalayer = [n for n in self.layer if n.is_output]
         self.train_stop_steps = sys.maxsize
+        self.batchsize = self.layer[0].batchsize if self.layer else 0
         self.node_list = self.Sort()
 
     def Sort(self):
@@ -244,3 +246,62 @@ class NeuralNet(object):
         losses = self.ForwardPropagate()
         losses.extend([node.GetLoss() for node in self.output_datalayer])
         return losses
+
+    # ---- the loop around the step (neuralnet.py:340-392, 510-530, 589-670)
+    @property
+    def datalayer(self):
+        """Layers that read a data stream, in the order listed: stream i of a handler feeds datalayer[i]."""
+        return [n for n in self.layer if n.is_input or n.is_output]
+
+    def GetBatch(self, handler):
+        """neuralnet.py:510-516: the next batch of every stream becomes the data of its layer
+        (views into the handler's device-resident chunk, no copy)."""
+        data_list = handler.Get(self.batchsize)
+        layers = self.datalayer
+        assert len(data_list) == len(layers), '%d streams for %d data layers' % (len(data_list), len(layers))
+        for layer, data in zip(layers, data_list):
+            assert data.shape[1] == layer.batchsize, 'batch of %d for layers of %d' % (data.shape[1], layer.batchsize)
+            layer.SetData(data)
+
+    def Evaluate(self, handler, steps):
+        """``steps`` batches through EvaluateOneBatch, losses accumulated (neuralnet.py:340-392
+        without collecting predictions)."""
+        stats = []
+        for _ in range(steps):
+            self.GetBatch(handler)
+            stats = Accumulate(stats, self.EvaluateOneBatch())
+        return stats
+
+    def Train(self, train_handler, steps=None, eval_handler=None, eval_steps=1, eval_after=0, start_step=0,
+              report=None):
+        """The training loop of neuralnet.py:589-670 without checkpoints, display and model
+        selection: fetch a batch, TrainOneBatch, accumulate the losses; every ``eval_after``
+        steps evaluate on ``eval_handler`` and start the accumulators afresh.  Returns the
+        list of {'step', 'train', 'eval'} records (also handed to ``report`` as they are made);
+        without ``eval_after`` one record at the end."""
+        stop = self.train_stop_steps if steps is None else steps
+        stats, history = [], []
+        step = start_step
+        while step < stop:
+            self.GetBatch(train_handler)
+            stats = Accumulate(stats, self.TrainOneBatch(step))
+            step += 1
+            if (eval_after and step % eval_after == 0) or step == stop:
+                record = {'step': step, 'train': stats,
+                          'eval': self.Evaluate(eval_handler, eval_steps) if eval_handler is not None else None}
+                history.append(record)
+                if report is not None:
+                    report(record)
+                stats = []
+        return history
+
+
+def Accumulate(stats, losses):
+    """deepnet/util.py:137-142 over whatever counters the losses carry (count, cross_entropy,
+    error, correct_preds, sparsity): the first batch starts the accumulators."""
+    if not stats:
+        return [types.SimpleNamespace(**vars(l)) for l in losses]
+    for acc, loss in zip(stats, losses):
+        for key, value in vars(loss).items():
+            setattr(acc, key, getattr(acc, key, 0) + value)
+    return stats

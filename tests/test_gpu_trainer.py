@@ -191,3 +191,83 @@ def test_what_the_builder_does_not_have_is_refused_by_name(cm, text, what):
         return
     with pytest.raises(NotImplementedError, match=what):
         trainer.CreateDeepnet(text, batchsize=4)
+
+
+BLOBS = '''
+name: "blobs"  model_type: FEED_FORWARD_NET  seed: 5
+hyperparams { base_epsilon: 0.1 initial_momentum: 0.5 final_momentum: 0.9 momentum_change_steps: 50 activation: LOGISTIC }
+layer { name: "in" dimensions: 20 is_input: true hyperparams { activation: LINEAR } }
+layer { name: "h" dimensions: 32 param { name: "bias" initialization: CONSTANT } }
+layer { name: "out" dimensions: 1 numlabels: 3 is_output: true loss_function: CROSS_ENTROPY
+        hyperparams { activation: SOFTMAX } param { name: "bias" initialization: CONSTANT } }
+edge { node1: "in" node2: "h" param { name: "weight" initialization: DENSE_GAUSSIAN_SQRT_FAN_IN sigma: 1.0 } }
+edge { node1: "h" node2: "out" param { name: "weight" initialization: DENSE_GAUSSIAN_SQRT_FAN_IN sigma: 1.0 } }
+'''
+
+
+def test_training_loop_learns_from_a_device_resident_data_set(cm):
+    """Model file -> net, arrays -> GPUCache (shuffled on the device), NeuralNet.Train with periodic
+    evaluation (neuralnet.py:589-670): three Gaussian blobs are told apart after 300 steps, the
+    accumulated counters add up, and the parameters equal those of stepping by hand over the
+    same batches."""
+    from deepnet_amd import trainer, datahandler as dh
+    rng = np.random.default_rng(21)
+    centres = 1.5 * rng.standard_normal((3, 20))
+
+    def blobs(n):
+        labels = rng.integers(0, 3, n)
+        return (centres[labels] + rng.standard_normal((n, 20))).astype(np.float32), labels.reshape(-1, 1).astype(np.float32)
+    train_x, train_y = blobs(600)
+    test_x, test_y = blobs(200)
+    op = 'optimizer: GRADIENT_DESCENT\nstopcondition { steps: 300 }\nbatchsize: 50\ndata_proto: "unused"\n'
+
+    def run(by_hand):
+        np.random.seed(77)                   # the shuffles of the cache
+        net = trainer.CreateDeepnet(BLOBS, op)
+        train = dh.GPUCache(dh.ArraySource([train_x, train_y]), 600, [20, 1], randomize=False)
+        test = dh.GPUCache(dh.ArraySource([test_x, test_y]), 200, [20, 1])
+        if by_hand:
+            for step in range(300):
+                net.GetBatch(train)
+                net.TrainOneBatch(step)
+            return net, None
+        seen = []
+        history = net.Train(train, eval_handler=test, eval_steps=4, eval_after=100, report=seen.append)
+        assert history == seen
+        return net, history
+    net, history = run(False)
+    assert [r['step'] for r in history] == [100, 200, 300]
+    for r in history:
+        assert len(r['train']) == 1 and r['train'][0].count == 100 * 50
+        assert len(r['eval']) == 1 and r['eval'][0].count == 4 * 50
+    first, last = history[0], history[-1]
+    assert last['eval'][0].correct_preds / 200.0 > 0.95
+    assert last['train'][0].cross_entropy < 0.5 * first['train'][0].cross_entropy
+    # before training the net is at chance
+    fresh = trainer.CreateDeepnet(BLOBS, op)
+    chance = fresh.Evaluate(dh.GPUCache(dh.ArraySource([test_x, test_y]), 200, [20, 1]), 4)
+    assert chance[0].correct_preds / 200.0 < 0.7
+    by_hand, _ = run(True)
+    for a, b in zip(net.edge, by_hand.edge):
+        assert np.array_equal(a.params['weight'].asarray(), b.params['weight'].asarray())
+    # a shuffled cache serves the same set in another order: still learns
+    np.random.seed(1)
+    net2 = trainer.CreateDeepnet(BLOBS, op)
+    shuffled = dh.GPUCache(dh.ArraySource([train_x, train_y]), 600, [20, 1], randomize=True)
+    h2 = net2.Train(shuffled, steps=300, eval_handler=dh.GPUCache(dh.ArraySource([test_x, test_y]), 200, [20, 1]), eval_steps=4)
+    assert [r['step'] for r in h2] == [300] and h2[0]['eval'][0].correct_preds / 200.0 > 0.95
+
+
+def test_rbm_training_loop_lowers_the_reconstruction_error(cm):
+    from deepnet_amd import trainer, datahandler as dh
+    rng = np.random.default_rng(2)
+    # bars: every image is 12 x 8 with whole rows on or off
+    rows = rng.random((640, 12, 1)) < 0.3
+    data = np.broadcast_to(rows, (640, 12, 8)).reshape(640, 96).astype(np.float32)
+    net = trainer.CreateDeepnet(os.path.join(GOLDEN, 'small_rbm.pbtxt'), TRAIN_OP % 'CD')
+    cache = dh.GPUCache(dh.ArraySource([data]), 640, [96])
+    history = net.Train(cache, steps=400, eval_after=100)
+    errors = [r['train'][-1].error / r['train'][-1].count for r in history]
+    assert len(history) == 4 and all(r['eval'] is None for r in history)
+    assert errors[-1] < 0.7 * errors[0] and errors[-1] < errors[1]
+    assert history[0]['train'][0].count == 100 and hasattr(history[0]['train'][0], 'sparsity')
