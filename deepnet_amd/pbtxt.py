@@ -23,6 +23,10 @@ class ParseError(ValueError):
     pass
 
 
+class Enum(str):
+    """An enum value, kept by name: compares like the string, written back without quotes."""
+
+
 class Message(object):
     """Fields in the order written.  ``msg.get('dimensions')``, ``msg.all('shape')``,
     ``'hyperparams' in msg``; attribute access is ``get`` and raises for a field not written."""
@@ -41,6 +45,14 @@ class Message(object):
             if n == name:
                 return v
         return default
+
+    def set(self, name, *values):
+        """Replace whatever was written for ``name`` by ``values`` (at the position of the
+        first occurrence, or at the end)."""
+        at = next((i for i, (n, _) in enumerate(self._fields) if n == name), len(self._fields))
+        kept = [(n, v) for n, v in self._fields if n != name]
+        at = min(at, len(kept))
+        self._fields = kept[:at] + [(name, v) for v in values] + kept[at:]
 
     def names(self):
         seen = []
@@ -186,7 +198,7 @@ class _Parser(object):
                 return False
             if val in ('inf', 'infinity', 'nan'):
                 return float(val[:3])
-            return val                                # an enum value, by name
+            return Enum(val)                          # an enum value, by name
         self.fail('expected a value')
 
 
@@ -208,3 +220,39 @@ def merged(base, over):
         else:
             out.add(name, o if o is not None else b)
     return out
+
+
+def _quote(raw):
+    """A bytes or str value as a double-quoted literal in printable ASCII (octal escapes, as
+    protobuf's text_format writes bytes fields)."""
+    data = raw if isinstance(raw, bytes) else raw.encode('utf-8')
+    out = []
+    for b in data:
+        c = chr(b)
+        if c in '"\\':
+            out.append('\\' + c)
+        elif c == '\n':
+            out.append('\\n')
+        elif 32 <= b < 127:
+            out.append(c)
+        else:
+            out.append('\\%03o' % b)
+    return '"' + ''.join(out) + '"'
+
+
+def dumps(msg, indent=0):
+    """The text form of a message tree; ``parse(dumps(m)) == m`` for trees made of Message, Enum,
+    bool, int, float and str values (bytes values come back as str with one character per byte)."""
+    pad, lines = '  ' * indent, []
+    for name, v in msg._fields:
+        if isinstance(v, Message):
+            lines.append('%s%s {\n%s%s}\n' % (pad, name, dumps(v, indent + 1), pad))
+        elif isinstance(v, bool):
+            lines.append('%s%s: %s\n' % (pad, name, 'true' if v else 'false'))
+        elif isinstance(v, Enum):
+            lines.append('%s%s: %s\n' % (pad, name, v))
+        elif isinstance(v, (bytes, str)):
+            lines.append('%s%s: %s\n' % (pad, name, _quote(v)))
+        else:
+            lines.append('%s%s: %r\n' % (pad, name, v))
+    return ''.join(lines)

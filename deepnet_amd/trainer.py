@@ -75,6 +75,16 @@ def InitializeParameter(param, dims):
     raise Exception('Unknown parameter initialization.')
 
 
+def _stored(param, dims):
+    """The array a parameter message carries in ``mat`` (deepnet/util.py:13-15: row-major float32)."""
+    raw = param.mat
+    raw = raw.encode('latin-1') if isinstance(raw, str) else raw
+    a = np.frombuffer(raw, dtype=np.float32)
+    if a.size != int(np.prod(dims)):
+        raise ValueError('parameter %s: %d stored values for dimensions %s' % (param.get('name'), a.size, list(dims)))
+    return a.reshape(tuple(dims)).copy()
+
+
 def _refuse(msg, fields, where):
     for name in fields:
         if msg.get(name) not in _OFF and msg.get(name) != '':
@@ -92,12 +102,11 @@ def _layer(proto, model_hyp, batchsize):
     for param in proto.all('param'):
         if param.name != 'bias':
             raise NotImplementedError('layer %s: parameter %s is not supported' % (name, param.name))
-        if 'mat' in param:
-            raise NotImplementedError('layer %s: stored parameter values are not read from text files' % name)
         pdims = param.all('dimensions') or [numlabels * dims, 1]
         if len(pdims) == 1:
             pdims = pdims + [1]
-        bias = InitializeParameter(param, pdims)
+        # stored values win over the initialisation rule (parameter.py:36-39)
+        bias = _stored(param, pdims) if 'mat' in param else InitializeParameter(param, pdims)
     return LAYER_TYPES[hyp.activation](
         name, dims, batchsize, hyperparams=hyp, numlabels=numlabels, is_input=proto.get('is_input', False),
         is_output=proto.get('is_output', False), loss_function=proto.get('loss_function', 'SQUARED_LOSS'),
@@ -114,8 +123,6 @@ def _edge(proto, model_hyp, layers):
     if len(params) != 1 or params[0].name != 'weight':
         raise NotImplementedError('%s: exactly one parameter, "weight", is supported' % where)
     param = params[0]
-    if 'mat' in param:
-        raise NotImplementedError('%s: stored parameter values are not read from text files' % where)
     conv, local = param.get('conv', False), param.get('local', False)
     cv = None
     if conv or local:
@@ -131,7 +138,7 @@ def _edge(proto, model_hyp, layers):
             dims = [cv.num_filters, n_locs ** 2 * cv.size ** 2 * cv.num_colors]
         else:
             dims = [node1.numlabels * node1.dimensions, node2.numlabels * node2.dimensions]
-    weight = InitializeParameter(param, dims)
+    weight = _stored(param, dims) if 'mat' in param else InitializeParameter(param, dims)
     return Edge(node1, node2, weight, hyperparams=hyp, conv_params=cv, local=bool(local),
                 up_factor=proto.get('up_factor', 1.0), block_gradient=proto.get('block_gradient', False),
                 down_factor=proto.get('down_factor', 1.0), directed=proto.get('directed', True))
@@ -170,3 +177,24 @@ def CreateDeepnet(model, train_op=None, eval_op=None, batchsize=None):
     if train_op and 'stopcondition' in train_op and train_op.stopcondition.get('steps', 0) > 0:
         net.train_stop_steps = train_op.stopcondition.steps
     return net
+
+
+def ModelWithParameters(net):
+    """The net's model message with the current device parameters stored in it (``dimensions``
+    and ``mat`` of every parameter, as deepnet/parameter.py:17-19 stores them before a
+    checkpoint is written): ``util.WritePbtxt(path, ModelWithParameters(net))`` writes a model
+    file that ``CreateDeepnet`` loads back with the same parameters."""
+    model = pbtxt.parse(pbtxt.dumps(net.net))            # a deep copy
+    by_layer = {l.name: l for l in net.layer}
+    by_edge = {(e.node1.name, e.node2.name): e for e in net.edge}
+    for proto in model.all('layer'):
+        for param in proto.all('param'):
+            arr = by_layer[proto.name].params[param.name].asarray()
+            param.set('dimensions', *arr.shape)
+            param.set('mat', np.ascontiguousarray(arr, dtype=np.float32).tobytes())
+    for proto in model.all('edge'):
+        for param in proto.all('param'):
+            arr = by_edge[(proto.node1, proto.node2)].params[param.name].asarray()
+            param.set('dimensions', *arr.shape)
+            param.set('mat', np.ascontiguousarray(arr, dtype=np.float32).tobytes())
+    return model

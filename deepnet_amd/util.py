@@ -63,3 +63,10 @@ def ReadModel(proto_file):
 def ReadOperation(proto_file):
     """deepnet/util.py:55-65 for text-format files."""
     return _read_text_message(proto_file)
+
+
+def WritePbtxt(output_file, pb):
+    """deepnet/util.py:79-81: a message tree as a text-format file."""
+    from . import pbtxt
+    with open(output_file, 'w') as f:
+        f.write(pbtxt.dumps(pb))

@@ -271,3 +271,38 @@ def test_rbm_training_loop_lowers_the_reconstruction_error(cm):
     assert len(history) == 4 and all(r['eval'] is None for r in history)
     assert errors[-1] < 0.7 * errors[0] and errors[-1] < errors[1]
     assert history[0]['train'][0].count == 100 and hasattr(history[0]['train'][0], 'sparsity')
+
+
+def test_model_written_with_its_parameters_loads_back_bit_for_bit(cm, cc, tmp_path):
+    """parameter.py:17-19 / util.py:13-21, 79-81: train a few steps, store the parameters in the
+    model message, write it as text, build a second net from the file: same parameters, same
+    next step."""
+    from deepnet_amd import trainer, util
+    net = trainer.CreateDeepnet(os.path.join(GOLDEN, 'small_convnet.pbtxt'), TRAIN_OP % 'GRADIENT_DESCENT')
+    by_name = {l.name: l for l in net.layer}
+    rng = np.random.default_rng(6)
+    x, t = _f(rng.standard_normal((288, 32))), _f(rng.integers(0, 10, (1, 32)))
+    for step in range(2):
+        by_name['input_layer'].data.assign(cm.CUDAMatrix(x))
+        by_name['output_layer'].data.assign(cm.CUDAMatrix(t))
+        net.TrainOneBatch(step)
+    path = str(tmp_path / 'checkpoint.pbtxt')
+    util.WritePbtxt(path, trainer.ModelWithParameters(net))
+    again = trainer.CreateDeepnet(util.ReadModel(path), TRAIN_OP % 'GRADIENT_DESCENT')
+    for a, b in zip(net.edge, again.edge):
+        assert a.params['weight'].shape == b.params['weight'].shape
+        assert np.array_equal(a.params['weight'].asarray().view(np.uint32), b.params['weight'].asarray().view(np.uint32))
+    for a, b in zip(net.layer, again.layer):
+        assert np.array_equal(a.params['bias'].asarray().view(np.uint32), b.params['bias'].asarray().view(np.uint32))
+    # evaluation (no dropout, no momentum history involved) gives the same loss
+    losses = []
+    for n in (net, again):
+        names = {l.name: l for l in n.layer}
+        names['input_layer'].data.assign(cm.CUDAMatrix(x))
+        names['output_layer'].data.assign(cm.CUDAMatrix(t))
+        losses.append(n.EvaluateOneBatch()[0].cross_entropy)
+    assert losses[0] == losses[1]
+    with pytest.raises(ValueError, match='stored values'):
+        bad = util.ReadModel(path)
+        bad.all('layer')[2].param.set('dimensions', 3, 1)
+        trainer.CreateDeepnet(bad, TRAIN_OP % 'GRADIENT_DESCENT')

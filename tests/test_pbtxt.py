@@ -75,3 +75,22 @@ def test_read_model_takes_text_files_only(tmp_path):
     assert op.optimizer == 'CD' and op.stopcondition.steps == 10 and op.batchsize == 32
     with pytest.raises(NotImplementedError):
         util.ReadModel(str(tmp_path / 'model.gz'))
+
+
+def test_written_text_reads_back_the_same_tree():
+    m = pbtxt.parse(open(os.path.join(HERE, 'golden', 'small_convnet.pbtxt')).read())
+    assert pbtxt.parse(pbtxt.dumps(m)) == m
+    extra = pbtxt.Message()
+    extra.add('mat', bytes(range(256)))
+    extra.add('text', 'a "quoted" \\ back\nslash')
+    extra.add('tiny', 1e-30)
+    extra.add('kind', pbtxt.Enum('PCD'))
+    text = pbtxt.dumps(extra)
+    assert all(32 <= ord(c) < 127 or c == '\n' for c in text)            # printable ASCII: octal escapes for the rest
+    back = pbtxt.parse(text)
+    assert back.mat.encode('latin-1') == bytes(range(256))
+    assert back.text == 'a "quoted" \\ back\nslash' and back.tiny == 1e-30
+    assert back.kind == 'PCD' and isinstance(back.kind, pbtxt.Enum) and 'kind: PCD' in text
+    m.set('seed', 3)
+    m.set('shape', 1, 2)
+    assert m.seed == 3 and m.names().index('seed') == 2 and m.all('shape') == [1, 2]
