@@ -7,7 +7,7 @@ does (same numpy generator, seeded with the model's seed, same order: layers, th
 listed), layers and edges are created and sorted.  ``model`` / ``train_op`` are the parsed
 text files (``util.ReadModel`` / ``util.ReadOperation``), paths to them, or their text.
 A field that would change the arithmetic of a step and has no counterpart here (tied
-parameters, pretrained initialisation, sparsity, replicated softmax, ...) raises
+parameters, replicated softmax, adaptive learning rates, ...) raises
 NotImplementedError by name instead of being dropped.
 """
 import os
@@ -52,7 +52,62 @@ def _hyperparams(model_hyp, own_hyp, where):
     return Hyperparams(**known)
 
 
-def InitializeParameter(param, dims):
+def _pretrained_array(param, model_file, find):
+    """One file named by ``pretrained_model``: an .npy array, or a model file in which
+    ``find(model)`` picks the layer / edge whose parameter of the same name is taken."""
+    ext = os.path.splitext(model_file)[1]
+    if ext == '.npy':
+        return np.load(model_file), None
+    if ext == '.npz':
+        stats = np.load(model_file)
+        if param.name != 'bias':
+            raise NotImplementedError('parameter %s from an .npz file is not supported' % param.name)
+        return np.nan_to_num(stats['mean'] / stats['std']), None
+    from .util import ReadModel
+    holder = find(ReadModel(model_file))
+    stored = next(p for p in holder.all('param') if p.name == param.name)
+    assert 'mat' in stored and stored.mat != '', 'Pretrained param %s of model %s is empty!!' % (stored.name, model_file)
+    return _stored(stored, stored.all('dimensions')), stored.all('dimensions')
+
+
+def LoadPretrained(param, dims, prefix, names):
+    """deepnet/layer.py:66-98 (``names`` = (layer name,)) and deepnet/edge.py:165-215 (``names`` =
+    (node1, node2)): the mean over the files listed in ``pretrained_model`` of the parameter of the
+    same name found there, for edges times ``mult_factor`` and transposed when
+    ``transpose_pretrained``."""
+    files = param.all('pretrained_model')
+    assert files, 'parameter %s: PRETRAINED without pretrained_model' % param.name
+    transpose = param.get('transpose_pretrained', False)
+    if len(names) == 1:
+        want = (param.get('pretrained_model_node1', '') or names[0],)
+        find = lambda model: next(n for n in model.all('layer') if n.name == want[0])
+    else:
+        want = (param.get('pretrained_model_node1', '') or names[0], param.get('pretrained_model_node2', '') or names[1])
+        if transpose:
+            want = want[::-1]
+
+        def find(model):
+            try:
+                return next(e for e in model.all('edge') if (e.node1, e.node2) == want)
+            except StopIteration:
+                raise LookupError('No edge found between %s and %s.' % want)
+    total = None
+    for name in files:
+        this_mat, stored_dims = _pretrained_array(param, os.path.join(prefix, name), find)
+        if len(names) == 2:
+            if stored_dims is not None:
+                expect = list(stored_dims)[::-1] if transpose else list(stored_dims)
+                assert list(dims) == expect, 'Param has shape %s but pretrained param has shape %s' % (list(dims), expect)
+                this_mat = param.get('mult_factor', 1.0) * this_mat
+            if transpose:
+                this_mat = this_mat.T
+        elif this_mat.ndim == 1:
+            this_mat = this_mat.reshape(-1, 1)
+        total = this_mat if total is None else total + this_mat
+    return total / len(files)
+
+
+def InitializeParameter(param, dims, prefix='', names=()):
     """deepnet/parameter.py:43-71 on the numpy global generator (seeded by the caller)."""
     kind = param.get('initialization', 'CONSTANT')
     sigma = param.get('sigma', 0.001)
@@ -71,7 +126,7 @@ def InitializeParameter(param, dims):
             return stddev * np.random.randn(*dims)
         return stddev * (2 * np.random.rand(*dims) - 1)
     if kind == 'PRETRAINED':
-        raise NotImplementedError('parameter %s: PRETRAINED initialisation is not supported' % param.get('name'))
+        return LoadPretrained(param, dims, prefix, names)
     raise Exception('Unknown parameter initialization.')
 
 
@@ -91,8 +146,9 @@ def _refuse(msg, fields, where):
             raise NotImplementedError('%s: %s is not supported' % (where, name))
 
 
-def _layer(proto, model_hyp, batchsize):
+def _layer(proto, model_hyp, batchsize, prefix=''):
     name = proto.name
+    prefix = proto.get('prefix', '') or prefix
     _refuse(proto, ('tied', 'is_initialized'), 'layer ' + name)
     hyp = _hyperparams(model_hyp, proto.get('hyperparams'), 'layer ' + name)
     if hyp.activation not in LAYER_TYPES:
@@ -106,15 +162,16 @@ def _layer(proto, model_hyp, batchsize):
         if len(pdims) == 1:
             pdims = pdims + [1]
         # stored values win over the initialisation rule (parameter.py:36-39)
-        bias = _stored(param, pdims) if 'mat' in param else InitializeParameter(param, pdims)
+        bias = _stored(param, pdims) if 'mat' in param else InitializeParameter(param, pdims, prefix, (name,))
     return LAYER_TYPES[hyp.activation](
         name, dims, batchsize, hyperparams=hyp, numlabels=numlabels, is_input=proto.get('is_input', False),
         is_output=proto.get('is_output', False), loss_function=proto.get('loss_function', 'SQUARED_LOSS'),
         loss_weight=proto.get('loss_weight', 1.0), bias=bias)
 
 
-def _edge(proto, model_hyp, layers):
+def _edge(proto, model_hyp, layers, prefix=''):
     where = 'edge %s:%s' % (proto.node1, proto.node2)
+    prefix = proto.get('prefix', '') or prefix
     _refuse(proto, ('tied', 'tied_transpose'), where)
     hyp = _hyperparams(model_hyp, proto.get('hyperparams'), where)
     by_name = {l.name: l for l in layers}
@@ -138,7 +195,7 @@ def _edge(proto, model_hyp, layers):
             dims = [cv.num_filters, n_locs ** 2 * cv.size ** 2 * cv.num_colors]
         else:
             dims = [node1.numlabels * node1.dimensions, node2.numlabels * node2.dimensions]
-    weight = _stored(param, dims) if 'mat' in param else InitializeParameter(param, dims)
+    weight = _stored(param, dims) if 'mat' in param else InitializeParameter(param, dims, prefix, (proto.node1, proto.node2))
     return Edge(node1, node2, weight, hyperparams=hyp, conv_params=cv, local=bool(local),
                 up_factor=proto.get('up_factor', 1.0), block_gradient=proto.get('block_gradient', False),
                 down_factor=proto.get('down_factor', 1.0), directed=proto.get('directed', True))
@@ -156,8 +213,9 @@ def CreateDeepnet(model, train_op=None, eval_op=None, batchsize=None):
     cm.CUDAMatrix.init_random(seed)          # deepnet/neuralnet.py:43-44
     np.random.seed(seed)
     model_hyp = model.get('hyperparams')
-    layers = [_layer(p, model_hyp, batchsize) for p in model.all('layer')]
-    edges = [_edge(p, model_hyp, layers) for p in model.all('edge')]
+    prefix = model.get('prefix', '')
+    layers = [_layer(p, model_hyp, batchsize, prefix) for p in model.all('layer')]
+    edges = [_edge(p, model_hyp, layers, prefix) for p in model.all('edge')]
     by_name = {l.name: l for l in layers}
     kind = model.model_type
     if kind == 'FEED_FORWARD_NET':
