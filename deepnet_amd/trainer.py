@@ -23,9 +23,12 @@ from .neuralnet import Edge, NeuralNet
 from .parameter import Hyperparams
 
 # Hyperparams fields that switch on behaviour this package does not have: refused when set.
-_SWITCHES = ('adapt', 'normalize', 'learn_precision', 'add_noise', 'shift', 'fast_dropout',
-             'shared_prior', 'soft_shared_prior', 'left_window', 'right_window', 'decay_learning_rate_for_last',
-             'additive_prior', 'multiplicative_prior', 'adaptive_prior')
+# shared_prior / soft_shared_prior select other edge classes (transfer_edge.py:6, soft_transfer_edge.py:6);
+# add_noise / shift / the windows are instructions to the data handler (datahandler.py:505-535), which the
+# caller builds here.  The remaining unknown fields are read only by replicated-softmax layers
+# (normalize, the priors) and fast-dropout nets, refused by activation / model type, or by nothing
+# (adapt, learn_precision, decay_learning_rate_for_last), or concern display and model selection.
+_SWITCHES = ('shared_prior', 'soft_shared_prior', 'add_noise', 'shift', 'left_window', 'right_window')
 _OFF = (False, 0, 0.0, 'NO_ADAPT', None)
 
 _CONV_FIELDS = ('size', 'stride', 'padding', 'num_filters', 'num_colors', 'max_pool', 'pool_size', 'pool_stride',

@@ -171,7 +171,7 @@ def test_rbm_with_a_sparsity_target_from_a_model_file(cm):
     ('name: "m" model_type: DBN', 'model_type'),
     ('name: "m" model_type: FEED_FORWARD_NET layer { name: "a" dimensions: 4 tied: true tied_to: "b" }', 'tied'),
     ('name: "m" model_type: FEED_FORWARD_NET layer { name: "a" dimensions: 4 hyperparams { activation: REPLICATED_SOFTMAX } }', 'activation'),
-    ('name: "m" model_type: FEED_FORWARD_NET layer { name: "a" dimensions: 4 hyperparams { adapt: ADAGRAD } }', 'adapt'),
+    ('name: "m" model_type: FEED_FORWARD_NET layer { name: "a" dimensions: 4 hyperparams { shared_prior: true adapt: ADAGRAD } }', 'shared_prior'),
     ('name: "m" model_type: FEED_FORWARD_NET layer { name: "a" dimensions: 4 param { name: "bias" initialization: PRETRAINED'
      ' pretrained_model: "binary_checkpoint.gz" } }', 'text-format'),
     ('name: "m" model_type: FEED_FORWARD_NET layer { name: "a" dimensions: 4 hyperparams { activation: TANH sparsity: true } is_input: true }'
