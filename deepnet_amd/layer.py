@@ -1,6 +1,6 @@
 """Layers of units for feed-forward nets on the MI355X backend: the step-path part of the
 reference's deepnet/layer.py and its activation subclasses (logistic_layer.py, tanh_layer.py,
-relu_layer.py, linear_layer.py, softmax_layer.py) -- ``ApplyActivation``, ``ComputeDeriv``,
+relu_layer.py, linear_layer.py, softmax_layer.py, sin_layer.py, cos_layer.py) -- ``ApplyActivation``, ``ComputeDeriv``,
 ``Sample``, ``GetLoss``, ``GetData`` and the buffers of ``AllocateMemory`` -- issuing the same
 matrix calls in the same order.  Configuration comes as plain arguments instead of protobuf
 messages; tied layers, replicated softmax and display are not carried over.
@@ -338,7 +338,36 @@ class SoftmaxLayer(Layer):
         return perf
 
 
-LAYER_TYPES = {cls.activation: cls for cls in (LinearLayer, LogisticLayer, TanhLayer, ReluLayer, SoftmaxLayer)}
+class SinLayer(Layer):
+    """deepnet/sin_layer.py: hidden units sin(x); the input is kept for the derivative."""
+    activation = P.SIN
+
+    def AllocateBatchsizeDependentMemory(self, batchsize):
+        super(SinLayer, self).AllocateBatchsizeDependentMemory(batchsize)
+        self.backup_state = _zeros(self.statesize.shape)
+
+    def ApplyActivation(self):
+        self.backup_state.assign(self.state)
+        cm.sin(self.state)
+
+    def ComputeDeriv(self):
+        self.deriv.apply_sin_deriv(self.backup_state)
+
+
+class CosLayer(SinLayer):
+    """deepnet/cos_layer.py."""
+    activation = P.COS
+
+    def ApplyActivation(self):
+        self.backup_state.assign(self.state)
+        cm.cos(self.state)
+
+    def ComputeDeriv(self):
+        self.deriv.apply_cos_deriv(self.backup_state)
+
+
+LAYER_TYPES = {cls.activation: cls for cls in (LinearLayer, LogisticLayer, TanhLayer, ReluLayer, SoftmaxLayer, SinLayer,
+                                               CosLayer)}
 
 
 def CreateLayer(activation, *args, **kwargs):

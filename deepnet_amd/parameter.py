@@ -15,6 +15,7 @@ from .choose_matrix_library import cm
 # Hyperparams.Decay / Hyperparams.Activation / Layer.LossFunction values, by the proto's names
 NONE, INVERSE_T, EXPONENTIAL = 'NONE', 'INVERSE_T', 'EXPONENTIAL'
 LINEAR, LOGISTIC, TANH, RECTIFIED_LINEAR, SOFTMAX = 'LINEAR', 'LOGISTIC', 'TANH', 'RECTIFIED_LINEAR', 'SOFTMAX'
+SIN, COS = 'SIN', 'COS'
 SQUARED_LOSS, CROSS_ENTROPY = 'SQUARED_LOSS', 'CROSS_ENTROPY'
 
 

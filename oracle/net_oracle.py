@@ -92,6 +92,10 @@ def activate(act, x):
     if act == 'SOFTMAX':
         e = np.exp(x - x.max(axis=0, keepdims=True))
         return e / e.sum(axis=0, keepdims=True)
+    if act == 'SIN':
+        return np.sin(x)
+    if act == 'COS':
+        return np.cos(x)
     assert act == 'LINEAR'
     return x
 
@@ -112,7 +116,7 @@ class Net(object):
     def forward(self, x, masks=None, train=False):
         """ComputeUp over the chain; masks[i] multiplies the state of layer i when it has dropout
         and train is set, otherwise such a state is scaled by 1 - dropout_prob."""
-        states, stages = [], []
+        states, stages, pre = [], [], {}
         for i, L in enumerate(self.layers):
             if i == 0:
                 s = np.array(x, dtype=F64)
@@ -126,12 +130,13 @@ class Net(object):
                 else:
                     stages.append(None)
                     s = e['w'].T @ states[-1]
-                s = activate(L['act'], s + L['bias'])
+                pre[i] = s + L['bias']
+                s = activate(L['act'], pre[i])
             h = L['hyper']
             if h.dropout:
                 s = s * np.asarray(masks[i], dtype=F64) if train else s * F64(np.float32(1.0 - h.dropout_prob))
             states.append(s)
-        self.states, self.stages = states, stages
+        self.states, self.stages, self.pre = states, stages, pre
         return states[-1]
 
     def loss_and_deriv(self, targets):
@@ -162,6 +167,10 @@ class Net(object):
             return d * s * (1.0 - s)
         if act == 'RECTIFIED_LINEAR':
             return d * (s > 0)
+        if act == 'SIN':                            # sin_layer.py:15-17, cos_layer.py:15-17: from the kept input
+            return d * np.cos(self.pre[i])
+        if act == 'COS':
+            return d * -np.sin(self.pre[i])
         if act == 'TANH':
             d = d * (1.0 + s) * (1.0 - s) * 0.5     # the reference's kTanhDeriv halves the slope (cudamat_kernels.cu:663-669)
         # tanh and linear units multiply by the mask explicitly (tanh_layer.py:19-21, linear_layer.py:28-30)
