@@ -38,8 +38,8 @@ _CONV_FIELDS = ('size', 'stride', 'padding', 'num_filters', 'num_colors', 'max_p
 def _as_message(x):
     if x is None or isinstance(x, pbtxt.Message):
         return x
-    if isinstance(x, str) and '\n' not in x and os.path.exists(x):
-        with open(x) as f:
+    if isinstance(x, str) and '\n' not in x and (os.path.exists(x) or x.endswith('.pbtxt')):
+        with open(x) as f:              # (a missing .pbtxt path raises FileNotFoundError, not a parse error)
             return pbtxt.parse(f.read())
     return pbtxt.parse(x)
 
