@@ -276,6 +276,82 @@ __global__ void __launch_bounds__(256) k_col_softmax_reg(const float* mat, float
   }
 }
 
+// The same for tall columns (1024 < h <= 4096) when there are enough of them: the
+// 256 lanes of a workgroup run down CB neighbouring columns at once (NVB 16-byte
+// groups per lane and column), so that a load instruction of the workgroup covers
+// 4 KiB of one column; maxima and sums meet through LDS.
+template <int NVB, int CB, bool STREAM>
+__global__ void __launch_bounds__(256) k_col_softmax_blk(const float* mat, float* target, int w, int h, SoftmaxExtras x) {
+  __shared__ float red[2][4][CB];
+  const int col0 = blockIdx.x * CB;
+  const int n4 = h >> 2;
+  const int wv = threadIdx.x >> 6;
+  float4 v[CB][NVB];
+#pragma unroll
+  for (int cb = 0; cb < CB; ++cb) {
+    const float* c4 = mat + (size_t)(col0 + cb < w ? col0 + cb : w - 1) * h;
+#pragma unroll
+    for (int k = 0; k < NVB; ++k) {
+      const int j = threadIdx.x + k * 256;
+      v[cb][k] = j < n4 ? dn_ld4<STREAM>(c4 + 4 * j) : make_float4(-FLT_MAX, -FLT_MAX, -FLT_MAX, -FLT_MAX);
+    }
+  }
+  float m[CB];
+#pragma unroll
+  for (int cb = 0; cb < CB; ++cb) {
+    float t = -FLT_MAX;
+#pragma unroll
+    for (int k = 0; k < NVB; ++k) t = fmaxf(t, fmaxf(fmaxf(v[cb][k].x, v[cb][k].y), fmaxf(v[cb][k].z, v[cb][k].w)));
+    t = wave_max(t);
+    if ((threadIdx.x & 63) == 0) red[0][wv][cb] = t;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int cb = 0; cb < CB; ++cb) m[cb] = fmaxf(fmaxf(red[0][0][cb], red[0][1][cb]), fmaxf(red[0][2][cb], red[0][3][cb]));
+#pragma unroll
+  for (int cb = 0; cb < CB; ++cb) {
+    float s = 0.f;
+#pragma unroll
+    for (int k = 0; k < NVB; ++k) {
+      const int j = threadIdx.x + k * 256;
+      if (j < n4) {
+        v[cb][k].x = softmax_exp(v[cb][k].x - m[cb]); v[cb][k].y = softmax_exp(v[cb][k].y - m[cb]);
+        v[cb][k].z = softmax_exp(v[cb][k].z - m[cb]); v[cb][k].w = softmax_exp(v[cb][k].w - m[cb]);
+        s += (v[cb][k].x + v[cb][k].y) + (v[cb][k].z + v[cb][k].w);
+      }
+    }
+    s = wave_sum(s);
+    if ((threadIdx.x & 63) == 0) red[1][wv][cb] = s;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int cb = 0; cb < CB; ++cb) {
+    const int col = col0 + cb;
+    if (col >= w) break;
+    const float inv = 1.f / ((red[1][0][cb] + red[1][1][cb]) + (red[1][2][cb] + red[1][3][cb]));
+    float* t4 = target + (size_t)col * h;
+#pragma unroll
+    for (int k = 0; k < NVB; ++k) {
+      const int j = threadIdx.x + k * 256;
+      if (j < n4) {
+        const float4 pr = make_float4(v[cb][k].x * inv, v[cb][k].y * inv, v[cb][k].z * inv, v[cb][k].w * inv);
+        dn_st4<STREAM>(t4 + 4 * j, pr);
+        if (x.labels) {
+          const int label = (int)x.labels[col], r0 = 4 * j;
+          if (x.grad)
+            dn_st4<STREAM>(x.grad + (size_t)col * h + r0,
+                           make_float4(pr.x - ((label == r0) ? 1.f : 0.f), pr.y - ((label == r0 + 1) ? 1.f : 0.f),
+                                       pr.z - ((label == r0 + 2) ? 1.f : 0.f), pr.w - ((label == r0 + 3) ? 1.f : 0.f)));
+          if (x.loss && label >= r0 && label < r0 + 4) {
+            const float pl = label == r0 ? pr.x : (label == r0 + 1 ? pr.y : (label == r0 + 2 ? pr.z : pr.w));
+            x.loss[col] = -logf(pl + x.tiny);
+          }
+        }
+      }
+    }
+  }
+}
+
 __global__ void k_softmax_grad(const float* mat, const float* labels, float* target, int w, int h, FastDiv fd) {
   const size_t n = (size_t)w * h;
   const size_t stride = (size_t)gridDim.x * blockDim.x;
@@ -364,6 +440,88 @@ k_gemv_cols(const float* M, int ld, int h, int w, const float* x, float* y, floa
   if (active && lane == 0) y[col] = (beta == 0.f ? 0.f : beta * y[col]) + alpha * s;
 }
 
+// Column reductions of tall matrices with many columns: the 256 lanes of a
+// workgroup run down CB neighbouring columns at once, 4 x CB 16-byte loads in
+// flight per lane (a 4096-row column is one trip), the weights of the weighted
+// sum held in registers across the CB columns.  Requires 16-byte aligned
+// columns (M aligned, ld % 4 == 0) and h % 4 == 0.
+//   COL_DOT: y[j] = beta*y[j] + alpha * sum_i M(i,j) x[i]    COL_SQSUM: the same over M(i,j)^2
+//   COL_MAX: y[j] = max_i M(i,j), starting from -FLT_MAX
+enum { COL_DOT = 0, COL_SQSUM = 1, COL_MAX = 2 };
+
+template <int CB, int OP, bool STREAM>
+__global__ void __launch_bounds__(256)
+k_colblock(const float* M, int ld, int h, int w, const float* x, float* y, float alpha, float beta) {
+  __shared__ float lds[4][CB];
+  const int n4 = h >> 2;
+  const int col0 = blockIdx.x * CB;
+  const float neutral = OP == COL_MAX ? -FLT_MAX : 0.f;
+  const float* cp[CB];
+#pragma unroll
+  for (int cb = 0; cb < CB; ++cb) cp[cb] = M + (size_t)(col0 + cb < w ? col0 + cb : w - 1) * ld;
+  float acc[CB];
+#pragma unroll
+  for (int cb = 0; cb < CB; ++cb) acc[cb] = neutral;
+  for (int j0 = threadIdx.x; j0 < n4; j0 += 1024) {
+    float4 v[4][CB], xv[4];
+    // loads issued column by column, down each column: the workgroup walks its CB
+    // neighbouring columns as one sequential range (measured 8% faster than chunk by chunk)
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int j = j0 + 256 * k;
+      xv[k] = (OP == COL_DOT && j < n4) ? *reinterpret_cast<const float4*>(x + 4 * j) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const int j = j0 + 256 * k;
+        v[k][cb] = j < n4 ? dn_ld4<STREAM>(cp[cb] + 4 * j) : make_float4(neutral, neutral, neutral, neutral);
+      }
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+#pragma unroll
+      for (int cb = 0; cb < CB; ++cb) {
+        const float4 t = v[k][cb];
+        if (OP == COL_DOT) { acc[cb] += t.x * xv[k].x; acc[cb] += t.y * xv[k].y; acc[cb] += t.z * xv[k].z; acc[cb] += t.w * xv[k].w; }
+        else if (OP == COL_SQSUM) { acc[cb] += t.x * t.x; acc[cb] += t.y * t.y; acc[cb] += t.z * t.z; acc[cb] += t.w * t.w; }
+        else acc[cb] = fmaxf(fmaxf(acc[cb], fmaxf(t.x, t.y)), fmaxf(t.z, t.w));
+      }
+  }
+#pragma unroll
+  for (int cb = 0; cb < CB; ++cb) {
+    const float r = OP == COL_MAX ? wave_max(acc[cb]) : wave_sum(acc[cb]);
+    if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6][cb] = r;
+  }
+  __syncthreads();
+  const int cb = threadIdx.x;
+  if (cb < CB && col0 + cb < w) {
+    const float a = lds[0][cb], b = lds[1][cb], c = lds[2][cb], d = lds[3][cb];
+    if (OP == COL_MAX) y[col0 + cb] = fmaxf(fmaxf(a, b), fmaxf(c, d));
+    else y[col0 + cb] = (beta == 0.f ? 0.f : beta * y[col0 + cb]) + alpha * ((a + b) + (c + d));
+  }
+}
+
+// Launches k_colblock when the shape suits it (tall, aligned, enough columns to
+// fill the chip with 256-lane workgroups); returns false otherwise.
+template <int OP>
+static bool colblock_launch(const float* M, int ld, int h, int w, const float* x, float* y, float alpha, float beta) {
+  if (h < 1024 || (h & 3) || (ld & 3) || !dn_aligned16(M) || (OP == COL_DOT && !dn_aligned16(x))) return false;
+  const int cus = dn_num_cus();
+  const bool stream = (long long)w * h >= DN_STREAM_MIN_ELEMS;
+  if (w >= 8 * cus) {
+    if (stream)
+      hipLaunchKernelGGL((k_colblock<4, OP, true>), dim3((w + 3) / 4), dim3(256), 0, 0, M, ld, h, w, x, y, alpha, beta);
+    else
+      hipLaunchKernelGGL((k_colblock<4, OP, false>), dim3((w + 3) / 4), dim3(256), 0, 0, M, ld, h, w, x, y, alpha, beta);
+  } else if (w >= 4 * cus) {
+    hipLaunchKernelGGL((k_colblock<2, OP, false>), dim3((w + 1) / 2), dim3(256), 0, 0, M, ld, h, w, x, y, alpha, beta);
+  } else {
+    return false;
+  }
+  return true;
+}
+
 // Two-stage reduction along rows (over the columns j of M[i + j*ld]), for
 //   ROW_DOT:   sum_j M(i,j) * x[j]      ROW_SQSUM: sum_j M(i,j)^2      ROW_MAX: max_j M(i,j)
 // Stage 1: workgroup (bx, by) reduces columns [by*cps, (by+1)*cps) for rows
@@ -383,18 +541,17 @@ __device__ __forceinline__ float row_finish(float yold, float s, float alpha, fl
   return (beta == 0.f ? 0.f : beta * yold) + alpha * s;
 }
 
-template <bool VEC, int OP>
-__global__ void __launch_bounds__(256)
+template <bool VEC, int OP, int NW, int U, bool STREAM>
+__global__ void __launch_bounds__(NW * 64)
 k_rows_stage1(const float* M, int ld, int h, int w, int cps, const float* x, float* y, float* partial, float alpha,
               float beta) {
   constexpr int RPL = VEC ? 4 : 1;
-  __shared__ float sv[4][64 * RPL];
+  __shared__ float sv[NW][64 * RPL];
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int row0 = (blockIdx.x * 64 + lane) * RPL;
   const int j0 = blockIdx.y * cps;
   const int j1 = (j0 + cps < w) ? j0 + cps : w;
   const float init = OP == ROW_MAX ? -INFINITY : 0.f;
-  const bool stream = (long long)w * h >= DN_STREAM_MIN_ELEMS;
   float acc[RPL];
 #pragma unroll
   for (int k = 0; k < RPL; ++k) acc[k] = init;
@@ -404,36 +561,97 @@ k_rows_stage1(const float* M, int ld, int h, int w, int cps, const float* x, flo
     else acc[k] = v > acc[k] ? v : acc[k];
   };
   if (row0 < h) {
-    int j = j0 + wv;
-    if constexpr (VEC) {
-      for (; j + 12 < j1; j += 16) {
-        float4 v[4];
-        float xs[4];
+    // U columns of this wavefront in flight per trip; a column past the range is
+    // read as the neutral element
+    for (int j = j0 + wv; j < j1; j += NW * U) {
+      float xs[U];
+      if constexpr (VEC) {
+        float4 v[U];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          v[u] = dn_ld4_rt(M + (size_t)(j + 4 * u) * ld + row0, stream);
-          xs[u] = OP == ROW_DOT ? x[j + 4 * u] : 0.f;
+        for (int u = 0; u < U; ++u) {
+          const int jj = j + NW * u;
+          if (jj < j1) {
+            v[u] = dn_ld4<STREAM>(M + (size_t)jj * ld + row0);
+            xs[u] = OP == ROW_DOT ? x[jj] : 0.f;
+          } else {
+            v[u] = make_float4(init, init, init, init);
+            xs[u] = 0.f;
+          }
         }
 #pragma unroll
-        for (int u = 0; u < 4; ++u) { take(0, v[u].x, xs[u]); take(1, v[u].y, xs[u]); take(2, v[u].z, xs[u]); take(3, v[u].w, xs[u]); }
-      }
-      for (; j < j1; j += 4) {
-        const float4 v = dn_ld4_rt(M + (size_t)j * ld + row0, stream);
-        const float xj = OP == ROW_DOT ? x[j] : 0.f;
-        take(0, v.x, xj); take(1, v.y, xj); take(2, v.z, xj); take(3, v.w, xj);
-      }
-    } else {
-      for (; j + 12 < j1; j += 16) {
-        float v[4], xs[4];
+        for (int u = 0; u < U; ++u) { take(0, v[u].x, xs[u]); take(1, v[u].y, xs[u]); take(2, v[u].z, xs[u]); take(3, v[u].w, xs[u]); }
+      } else {
+        float v[U];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          v[u] = M[(size_t)(j + 4 * u) * ld + row0];
-          xs[u] = OP == ROW_DOT ? x[j + 4 * u] : 0.f;
+        for (int u = 0; u < U; ++u) {
+          const int jj = j + NW * u;
+          if (jj < j1) {
+            v[u] = M[(size_t)jj * ld + row0];
+            xs[u] = OP == ROW_DOT ? x[jj] : 0.f;
+          } else {
+            v[u] = init;
+            xs[u] = 0.f;
+          }
         }
 #pragma unroll
-        for (int u = 0; u < 4; ++u) take(0, v[u], xs[u]);
+        for (int u = 0; u < U; ++u) take(0, v[u], xs[u]);
       }
-      for (; j < j1; j += 4) take(0, M[(size_t)j * ld + row0], OP == ROW_DOT ? x[j] : 0.f);
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < RPL; ++k) sv[wv][lane * RPL + k] = acc[k];
+  __syncthreads();
+  for (int r = threadIdx.x; r < 64 * RPL; r += NW * 64) {
+    const int row = blockIdx.x * 64 * RPL + r;
+    if (row < h) {
+      float s = sv[0][r];
+#pragma unroll
+      for (int k = 1; k < NW; ++k) s = row_combine<OP>(s, sv[k][r]);
+      if (partial) partial[(size_t)blockIdx.y * h + row] = s;
+      else y[row] = row_finish<OP>(y[row], s, alpha, beta);
+    }
+  }
+}
+
+// Stage 2: a lane owns RPL neighbouring rows (one 16-byte load per split when
+// VEC), the 4 wavefronts of a workgroup take every 4th split, 8 loads in flight,
+// and meet in LDS; the order of the additions is fixed.
+template <bool VEC, int OP>
+__global__ void __launch_bounds__(256)
+k_rows_stage2(const float* partial, int splits, int h, float* y, float alpha, float beta) {
+  constexpr int RPL = VEC ? 4 : 1;
+  __shared__ float sv[4][64 * RPL];
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int row0 = (blockIdx.x * 64 + lane) * RPL;
+  const float init = OP == ROW_MAX ? -INFINITY : 0.f;
+  float acc[RPL];
+#pragma unroll
+  for (int k = 0; k < RPL; ++k) acc[k] = init;
+  if (row0 < h) {
+    for (int s = wv; s < splits; s += 32) {
+      if constexpr (VEC) {
+        float4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int ss = s + 4 * u;
+          v[u] = ss < splits ? *reinterpret_cast<const float4*>(partial + (size_t)ss * h + row0)
+                             : make_float4(init, init, init, init);
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          acc[0] = row_combine<OP>(acc[0], v[u].x); acc[1] = row_combine<OP>(acc[1], v[u].y);
+          acc[2] = row_combine<OP>(acc[2], v[u].z); acc[3] = row_combine<OP>(acc[3], v[u].w);
+        }
+      } else {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int ss = s + 4 * u;
+          v[u] = ss < splits ? partial[(size_t)ss * h + row0] : init;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) acc[0] = row_combine<OP>(acc[0], v[u]);
+      }
     }
   }
 #pragma unroll
@@ -443,40 +661,8 @@ k_rows_stage1(const float* M, int ld, int h, int w, int cps, const float* x, flo
     const int row = blockIdx.x * 64 * RPL + r;
     if (row < h) {
       const float s = row_combine<OP>(row_combine<OP>(sv[0][r], sv[1][r]), row_combine<OP>(sv[2][r], sv[3][r]));
-      if (partial) partial[(size_t)blockIdx.y * h + row] = s;
-      else y[row] = row_finish<OP>(y[row], s, alpha, beta);
+      y[row] = row_finish<OP>(y[row], s, alpha, beta);
     }
-  }
-}
-
-// Stage 2: 16 rows per workgroup, 16 lane groups take every 16th split (all of a lane's
-// loads in flight at once for up to 64 splits) and meet in LDS; the order of the
-// additions is fixed.
-template <int OP>
-__global__ void __launch_bounds__(256)
-k_rows_stage2(const float* partial, int splits, int h, float* y, float alpha, float beta) {
-  __shared__ float sv[16][17];
-  const int r = threadIdx.x & 15, grp = threadIdx.x >> 4;
-  const int row = blockIdx.x * 16 + r;
-  float acc = OP == ROW_MAX ? -INFINITY : 0.f;
-  if (row < h) {
-    int k = grp;
-    for (; k + 48 < splits; k += 64) {
-      float v[4];
-#pragma unroll
-      for (int u = 0; u < 4; ++u) v[u] = partial[(size_t)(k + 16 * u) * h + row];
-#pragma unroll
-      for (int u = 0; u < 4; ++u) acc = row_combine<OP>(acc, v[u]);
-    }
-    for (; k < splits; k += 16) acc = row_combine<OP>(acc, partial[(size_t)k * h + row]);
-  }
-  sv[grp][r] = acc;
-  __syncthreads();
-  if (grp == 0 && row < h) {
-    float s = sv[0][r];
-#pragma unroll
-    for (int g2 = 1; g2 < 16; ++g2) s = row_combine<OP>(s, sv[g2][r]);
-    y[row] = row_finish<OP>(y[row], s, alpha, beta);
   }
 }
 
@@ -499,21 +685,37 @@ static int rows_reduce(const float* M, int ld, int h, int w, const float* x, flo
     if (!partial) return CUDA_ERROR;
   }
   dim3 grid(bx, splits);
-  // (Finishing inside stage 1 by the last-arriving workgroup was measured 8x slower:
-  // the device-scope release fence each workgroup then needs writes back its L2.)
-  if (vec)
-    hipLaunchKernelGGL((k_rows_stage1<true, OP>), grid, dim3(256), 0, 0, M, ld, h, w, cps, x, y, partial, alpha, beta);
-  else
-    hipLaunchKernelGGL((k_rows_stage1<false, OP>), grid, dim3(256), 0, 0, M, ld, h, w, cps, x, y, partial, alpha, beta);
-  if (splits > 1)
-    hipLaunchKernelGGL((k_rows_stage2<OP>), dim3((h + 15) / 16), dim3(256), 0, 0, (const float*)partial, splits, h, y,
-                       alpha, beta);
+  // One launch with the last-arriving workgroup of a row block adding up the partial
+  // sums was measured and lost: device-scope atomics on one counter are served one
+  // after the other at about 190 ns each (64 arrivals: +12 us), and a release fence
+  // per workgroup costs more still.  A workgroup that owns few rows over all columns
+  // needs no second stage but reads 64-byte runs (18 us against 12 + 2.5 for two stages).
+  if (vec) {
+    // 8 wavefronts x 8 columns in flight: a 64-column slice is one trip
+    if (cps > 16 && (long long)w * h >= DN_STREAM_MIN_ELEMS)
+      hipLaunchKernelGGL((k_rows_stage1<true, OP, 8, 8, true>), grid, dim3(512), 0, 0, M, ld, h, w, cps, x, y, partial, alpha, beta);
+    else if (cps > 16)
+      hipLaunchKernelGGL((k_rows_stage1<true, OP, 8, 8, false>), grid, dim3(512), 0, 0, M, ld, h, w, cps, x, y, partial, alpha, beta);
+    else
+      hipLaunchKernelGGL((k_rows_stage1<true, OP, 4, 4, false>), grid, dim3(256), 0, 0, M, ld, h, w, cps, x, y, partial, alpha, beta);
+  } else {
+    hipLaunchKernelGGL((k_rows_stage1<false, OP, 4, 4, false>), grid, dim3(256), 0, 0, M, ld, h, w, cps, x, y, partial, alpha, beta);
+  }
+  if (splits > 1) {
+    if (h % 4 == 0)
+      hipLaunchKernelGGL((k_rows_stage2<true, OP>), dim3((h + 255) / 256), dim3(256), 0, 0, (const float*)partial, splits,
+                         h, y, alpha, beta);
+    else
+      hipLaunchKernelGGL((k_rows_stage2<false, OP>), dim3((h + 63) / 64), dim3(256), 0, 0, (const float*)partial, splits,
+                         h, y, alpha, beta);
+  }
   return dn_launch_status();
 }
 
 // Host entry points used by dot() for vector-shaped products.
 int dn_gemv_cols(const float* M, int ld, int h, int w, const float* x, float* y, float alpha, float beta) {
   if (w <= 0) return 0;
+  if (colblock_launch<COL_DOT>(M, ld, h, w, x, y, alpha, beta)) return dn_launch_status();
   const int cus = dn_num_cus();
   if (w < cus * 2 && h >= 4096) {
     hipLaunchKernelGGL((k_gemv_cols<256>), dim3(w), dim3(256), 0, 0, M, ld, h, w, x, y, alpha, beta);
@@ -601,6 +803,8 @@ int max_by_axis(cudamat* mat, cudamat* target, int axis) {
   if (int e = check_axis_common(mat, target)) return e;
   if (axis == 0) {
     if (target->size[0] != 1 || target->size[1] != w) return ERROR_INCOMPATIBLE_DIMENSIONS;
+    if (w > 0 && colblock_launch<COL_MAX>(mat->data_device, h, h, w, nullptr, target->data_device, 1.f, 0.f))
+      return dn_launch_status();
     return launch_cols(k_col_max<64>, k_col_max<256>, w, h, (const float*)mat->data_device, target->data_device, w, h);
   } else if (axis == 1) {
     if (target->size[0] != h || target->size[1] != 1) return ERROR_INCOMPATIBLE_DIMENSIONS;
@@ -659,6 +863,8 @@ int sqsum_by_axis(cudamat* mat, cudamat* target, int axis, float mult, float p) 
   if (int e = check_axis_common(mat, target)) return e;
   if (axis == 0) {
     if (target->size[0] != 1 || target->size[1] != w) return ERROR_INCOMPATIBLE_DIMENSIONS;
+    if (w > 0 && colblock_launch<COL_SQSUM>(mat->data_device, h, h, w, nullptr, target->data_device, mult, p))
+      return dn_launch_status();
     return launch_cols(k_col_sqsum<64>, k_col_sqsum<256>, w, h, (const float*)mat->data_device, target->data_device,
                        w, h, mult, p);
   } else if (axis == 1) {
@@ -688,6 +894,16 @@ static int softmax_impl(const float* in, float* out, int w, int h, SoftmaxExtras
   if (w <= 0 || h <= 0) return 0;
   const bool reg_ok = (h % 4 == 0) && dn_aligned16(in) && dn_aligned16(out) && h <= 64 * 4 * 16 &&
                       (!x.grad || dn_aligned16(x.grad));
+  if (reg_ok && h > 1024 && w >= 8 * dn_num_cus()) {
+    const int n4 = h / 4;
+    dim3 grid((w + 3) / 4), block(256);
+    const bool stream = (long long)w * h >= DN_STREAM_MIN_ELEMS;
+    if (n4 <= 512) hipLaunchKernelGGL((k_col_softmax_blk<2, 4, false>), grid, block, 0, 0, in, out, w, h, x);
+    else if (n4 <= 768) hipLaunchKernelGGL((k_col_softmax_blk<3, 4, false>), grid, block, 0, 0, in, out, w, h, x);
+    else if (stream) hipLaunchKernelGGL((k_col_softmax_blk<4, 4, true>), grid, block, 0, 0, in, out, w, h, x);
+    else hipLaunchKernelGGL((k_col_softmax_blk<4, 4, false>), grid, block, 0, 0, in, out, w, h, x);
+    return dn_launch_status();
+  }
   if (reg_ok) {
     const int n4 = h / 4;
     dim3 grid((w + 3) / 4), block(256);
