@@ -161,7 +161,7 @@ k_rng_serial(const unsigned int* mults, unsigned long long* words, size_t n, Op 
 // of its stream, reaching its first draw with one jump per set bit of p.  The lane
 // that produces a stream's last draw writes the new word into the other buffer.
 #define RNG_SPLIT_BLOCK 256
-template <class Op>
+template <class Op, int B>
 __global__ void __launch_bounds__(RNG_SPLIT_BLOCK)
 k_rng_split(const unsigned int* mults, const unsigned long long* words, unsigned long long* next,
             const unsigned long long* table, size_t n, int chbits, Op op) {
@@ -176,70 +176,44 @@ k_rng_split(const unsigned int* mults, const unsigned long long* words, unsigned
   const unsigned long long d0 = (unsigned long long)part << chbits;
   if (d0 >= draws) return;
   const unsigned long long d1 = d0 + (1ull << chbits) < draws ? d0 + (1ull << chbits) : draws;
+  size_t i = (size_t)d0 * NUM_RND_STREAMS + idx;
+  unsigned long long d = d0;
+  // The array reads do not depend on the generator: the first batch is requested
+  // before the jump-ahead arithmetic, which then runs under the memory latency.
+  float x[B];
+  const bool full0 = d + B <= d1;
+  if (full0) {
+#pragma unroll
+    for (int k = 0; k < B; ++k) x[k] = op.src ? __builtin_nontemporal_load(op.src + i + (size_t)k * NUM_RND_STREAMS) : 0.f;
+  }
   const unsigned int mult = mults[idx];
   unsigned long long w = words[idx];
   for (unsigned int b = 0, pp = part; pp; ++b, pp >>= 1)
     if (pp & 1u) w = mwc_montmul(w, table[(size_t)(chbits + b) * NUM_RND_STREAMS + idx], mult);
-  w = rng_walk<true>(w, mult, idx, d0, d1, op);
-  if (d1 == draws) next[idx] = w;
-}
-
-// The same schedule with four neighbouring streams per lane, for calls whose element
-// count is a multiple of 4 on 16-byte aligned arrays: then the four streams 4q..4q+3
-// have equally many draws, their elements of one draw are one aligned 16-byte vector,
-// and a lane runs four independent recurrences against one vector load and one vector
-// store per draw (four draws' loads in flight).
-#define RNG_SPLIT4_BLOCK 256
-template <class Op>
-__global__ void __launch_bounds__(RNG_SPLIT4_BLOCK)
-k_rng_split4(const unsigned int* mults, const unsigned long long* words, unsigned long long* next,
-             const unsigned long long* table, size_t n, int chbits, Op op) {
-  constexpr int blocks_per_part = NUM_RND_STREAMS / (4 * RNG_SPLIT4_BLOCK);
-  const unsigned int part = blockIdx.x / blocks_per_part;
-  const unsigned int idx = 4 * ((blockIdx.x % blocks_per_part) * RNG_SPLIT4_BLOCK + threadIdx.x);   // first of 4 streams
-  if (idx >= n) {  // streams without draws keep their words
-    if (part == 0) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) next[idx + j] = words[idx + j];
-    }
-    return;
-  }
-  const unsigned long long draws = (n - idx + NUM_RND_STREAMS - 1) / NUM_RND_STREAMS;  // of each of the four
-  const unsigned long long d0 = (unsigned long long)part << chbits;
-  if (d0 >= draws) return;
-  const unsigned long long d1 = d0 + (1ull << chbits) < draws ? d0 + (1ull << chbits) : draws;
-  unsigned int mult[4];
-  unsigned long long w[4];
-#pragma unroll
-  for (int j = 0; j < 4; ++j) { mult[j] = mults[idx + j]; w[j] = words[idx + j]; }
-  for (unsigned int b = 0, pp = part; pp; ++b, pp >>= 1)
-    if (pp & 1u) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) w[j] = mwc_montmul(w[j], table[(size_t)(chbits + b) * NUM_RND_STREAMS + idx + j], mult[j]);
-    }
-  size_t i = (size_t)d0 * NUM_RND_STREAMS + idx;
-  unsigned long long d = d0;
-  auto emit = [&](size_t at, const float4& x) {
-    float4 o;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) w[j] = mwc_step(w[j], mult[j]);
-    o.x = op.value(mwc_uniform(w[0]), x.x); o.y = op.value(mwc_uniform(w[1]), x.y);
-    o.z = op.value(mwc_uniform(w[2]), x.z); o.w = op.value(mwc_uniform(w[3]), x.w);
-    dn_st4<true>(op.dst + at, o);
+  auto emit = [&](size_t at, float xv) {
+    w = mwc_step(w, mult);
+    __builtin_nontemporal_store(op.value(mwc_uniform(w), xv), op.dst + at);
   };
-  const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
-  for (; d + 4 <= d1; d += 4, i += (size_t)4 * NUM_RND_STREAMS) {
-    float4 x[4];
+  if (full0) {
+    for (;;) {
+      const size_t inext = i + (size_t)B * NUM_RND_STREAMS;
+      const bool more = d + 2 * B <= d1;
+      float y[B];
 #pragma unroll
-    for (int k = 0; k < 4; ++k) x[k] = op.src ? dn_ld4<true>(op.src + i + (size_t)k * NUM_RND_STREAMS) : zero4;
+      for (int k = 0; k < B; ++k) y[k] = x[k];
+      if (more) {   // the next batch is requested before this one is consumed
 #pragma unroll
-    for (int k = 0; k < 4; ++k) emit(i + (size_t)k * NUM_RND_STREAMS, x[k]);
+        for (int k = 0; k < B; ++k) x[k] = op.src ? __builtin_nontemporal_load(op.src + inext + (size_t)k * NUM_RND_STREAMS) : 0.f;
+      }
+#pragma unroll
+      for (int k = 0; k < B; ++k) emit(i + (size_t)k * NUM_RND_STREAMS, y[k]);
+      d += B;
+      i = inext;
+      if (!more) break;
+    }
   }
-  for (; d < d1; ++d, i += NUM_RND_STREAMS) emit(i, op.src ? dn_ld4<true>(op.src + i) : zero4);
-  if (d1 == draws) {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) next[idx + j] = w[j];
-  }
+  for (; d < d1; ++d, i += NUM_RND_STREAMS) emit(i, op.src ? op.src[i] : 0.f);
+  if (d1 == draws) next[idx] = w;
 }
 
 // Box-Muller pairs: two draws give elements i and i + 12288 (cudamat_kernels.cu:125-143, 192-211).
@@ -263,11 +237,17 @@ k_rng_gauss(const unsigned int* mults, unsigned long long* words, const float* i
   words[idx] = w;
 }
 
-// Calls with at least RNG_SPLIT_MIN_DRAWS draws per stream are cut into about
-// RNG_SPLIT_PARTS parts per stream (chunk length a power of two, at least 16).
+// Calls with at least RNG_SPLIT_MIN_DRAWS draws per stream are cut into parts of 2^c
+// draws.  A pure fill takes about RNG_SPLIT_PARTS parts per stream (c >= 4).  An op
+// that also reads an array takes parts of 16 draws while that gives at most
+// RNG_SPLIT_SRC_PARTS parts, all 16 reads of a lane in flight under its jump
+// arithmetic; measured on 4096 x 4096 (sample_bernoulli): 25.0 us against 27-28 us
+// for 64-draw parts and for four streams per lane with 16-byte accesses.  Part
+// counts whose workgroups fill the chip's resident slots a little more than a whole
+// number of times (43 parts of 32 draws: 2064 workgroups for 2048 slots) cost 2 us.
 #define RNG_SPLIT_MIN_DRAWS 32
 #define RNG_SPLIT_PARTS 24
-#define RNG_SPLIT4_PARTS 96    // four streams per lane: more parts for as many wavefronts
+#define RNG_SPLIT_SRC_PARTS 96
 
 template <class Op>
 static int launch_rng(rnd_struct* st, size_t n, Op op) {
@@ -278,10 +258,8 @@ static int launch_rng(rnd_struct* st, size_t n, Op op) {
                        op);
     return dn_launch_status();
   }
-  // (measured: pays for the ops that also read an array; a pure fill is faster one stream per lane)
-  const bool vec4 = op.src && n % 4 == 0 && dn_aligned16(op.dst) && dn_aligned16(op.src);
   int chbits = 4;
-  while (((draws + (1ull << chbits) - 1) >> chbits) > (vec4 ? RNG_SPLIT4_PARTS : RNG_SPLIT_PARTS)) ++chbits;
+  while (((draws + (1ull << chbits) - 1) >> chbits) > (size_t)(op.src ? RNG_SPLIT_SRC_PARTS : RNG_SPLIT_PARTS)) ++chbits;
   const size_t parts = (draws + (1ull << chbits) - 1) >> chbits;
   // every jump exponent (chbits + bit of part) must be inside the table
   int top = 0;
@@ -292,15 +270,13 @@ static int launch_rng(rnd_struct* st, size_t n, Op op) {
     return dn_launch_status();
   }
   unsigned long long* next = rng_other(st->dev_words);
-  if (vec4) {
-    const unsigned grid = (unsigned)(parts * (NUM_RND_STREAMS / (4 * RNG_SPLIT4_BLOCK)));
-    hipLaunchKernelGGL((k_rng_split4<Op>), dim3(grid), dim3(RNG_SPLIT4_BLOCK), 0, 0, st->dev_mults,
+  const unsigned grid = (unsigned)(parts * (NUM_RND_STREAMS / RNG_SPLIT_BLOCK));
+  if (op.src)
+    hipLaunchKernelGGL((k_rng_split<Op, 16>), dim3(grid), dim3(RNG_SPLIT_BLOCK), 0, 0, st->dev_mults,
                        (const unsigned long long*)st->dev_words, next, rng_table(st->dev_words), n, chbits, op);
-  } else {
-    const unsigned grid = (unsigned)(parts * (NUM_RND_STREAMS / RNG_SPLIT_BLOCK));
-    hipLaunchKernelGGL((k_rng_split<Op>), dim3(grid), dim3(RNG_SPLIT_BLOCK), 0, 0, st->dev_mults,
+  else
+    hipLaunchKernelGGL((k_rng_split<Op, 4>), dim3(grid), dim3(RNG_SPLIT_BLOCK), 0, 0, st->dev_mults,
                        (const unsigned long long*)st->dev_words, next, rng_table(st->dev_words), n, chbits, op);
-  }
   st->dev_words = next;
   return dn_launch_status();
 }
