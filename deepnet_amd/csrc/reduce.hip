@@ -666,10 +666,162 @@ k_rows_stage2(const float* partial, int splits, int h, float* y, float alpha, fl
   }
 }
 
+// One launch for 16-byte aligned operands: a workgroup owns 64 rows (16 lanes x 4 rows,
+// the 4 lane groups of a wavefront on 4 neighbouring columns: 256-byte runs) and the
+// columns [by*cps, (by+1)*cps); NW wavefronts x U loads in flight.  With more than one
+// column slice (at most ROWS_ONE_MAX_SPLITS, chosen so that about one workgroup per CU
+// runs) a workgroup publishes its 64 partial results and counts itself in; the one that
+// arrives last adds the slices up in slice order, so the result does not depend on the
+// order of arrival.  Partials travel as agent-scope atomic stores and loads (they bypass
+// the non-coherent cache levels; a release fence per wavefront was measured 5-10x slower
+// than the whole kernel), the counter returns to zero for the next launch.
+#define ROWS_ONE_MAX_SPLITS 8
+
+template <int OP, int NW, int U, bool STREAM>
+__global__ void __launch_bounds__(NW * 64)
+k_rows_one(const float* M, int ld, int h, int w, int cps, const float* x, float* y, float* partial,
+           unsigned* counters, float alpha, float beta) {
+  __shared__ float sv[NW][64];
+  __shared__ int s_last;
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int r = lane & 15, c = lane >> 4;
+  const int row0 = (blockIdx.x * 16 + r) * 4;
+  const int j0 = blockIdx.y * cps;
+  const int j1 = (j0 + cps < w) ? j0 + cps : w;
+  const float init = OP == ROW_MAX ? -INFINITY : 0.f;
+  float acc[4] = {init, init, init, init};
+  auto take = [&](int k, float v, float xj) {
+    if (OP == ROW_DOT) acc[k] += v * xj;
+    else if (OP == ROW_SQSUM) acc[k] += v * v;
+    else acc[k] = v > acc[k] ? v : acc[k];
+  };
+  if (row0 < h) {
+    for (int j = j0 + wv * 4 + c; j < j1; j += NW * 4 * U) {
+      float4 v[U];
+      float xs[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int jj = j + NW * 4 * u;
+        if (jj < j1) {
+          v[u] = dn_ld4<STREAM>(M + (size_t)jj * ld + row0);
+          xs[u] = OP == ROW_DOT ? x[jj] : 0.f;
+        } else {
+          v[u] = make_float4(init, init, init, init);
+          xs[u] = 0.f;
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) { take(0, v[u].x, xs[u]); take(1, v[u].y, xs[u]); take(2, v[u].z, xs[u]); take(3, v[u].w, xs[u]); }
+    }
+  }
+#pragma unroll
+  for (int o = 16; o < 64; o <<= 1)
+#pragma unroll
+    for (int k = 0; k < 4; ++k) acc[k] = row_combine<OP>(acc[k], __shfl_xor(acc[k], o, WAVE));
+  if (c == 0) *reinterpret_cast<float4*>(&sv[wv][r * 4]) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+  __syncthreads();
+  const int splits = gridDim.y;
+  const int row = blockIdx.x * 64 + (int)threadIdx.x;
+  const bool mine = threadIdx.x < 64 && row < h;
+  if (mine) {
+    float s = sv[0][threadIdx.x];
+#pragma unroll
+    for (int k = 1; k < NW; ++k) s = row_combine<OP>(s, sv[k][threadIdx.x]);
+    if (splits == 1) y[row] = row_finish<OP>(y[row], s, alpha, beta);
+    else __hip_atomic_store(partial + (size_t)blockIdx.y * h + row, s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  if (splits == 1) return;
+  __builtin_amdgcn_s_waitcnt(0);   // the stores of this wavefront have been acknowledged
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const unsigned old = __hip_atomic_fetch_add(counters + blockIdx.x, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    s_last = (old == (unsigned)splits - 1u);
+    if (s_last) __hip_atomic_store(counters + blockIdx.x, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  __syncthreads();
+  if (!s_last || !mine) return;
+  float pv[ROWS_ONE_MAX_SPLITS];
+#pragma unroll
+  for (int k = 0; k < ROWS_ONE_MAX_SPLITS; ++k)
+    pv[k] = k < splits ? __hip_atomic_load(partial + (size_t)k * h + row, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : init;
+  float t = pv[0];
+#pragma unroll
+  for (int k = 1; k < ROWS_ONE_MAX_SPLITS; ++k)
+    if (k < splits) t = row_combine<OP>(t, pv[k]);
+  y[row] = row_finish<OP>(y[row], t, alpha, beta);
+}
+
+// Workspace of k_rows_one: slice partials and one arrival counter per 64-row block.
+struct RowsWorkspace {
+  float* partial;      // room for partial_floats floats
+  size_t partial_floats;
+  unsigned* counters;  // zero between launches
+  int num_counters;
+};
+
+// Number of column slices for the one-launch kernel: about one workgroup per CU, a slice
+// at least 256 columns wide.  0 when that would take more than ROWS_ONE_MAX_SPLITS slices
+// (few rows, very many columns): such shapes keep the two-stage kernels.
+static int rows_one_splits(int h, int w) {
+  const int bx = (h + 63) / 64;
+  int splits = (dn_num_cus() + bx / 2) / bx;
+  if (splits > w / 256) splits = w / 256;
+  if (splits < 1) splits = 1;
+  return splits <= ROWS_ONE_MAX_SPLITS ? splits : 0;
+}
+
+template <int OP>
+static int rows_reduce_one(const float* M, int ld, int h, int w, const float* x, float* y, float alpha, float beta,
+                           const RowsWorkspace& ws) {
+  const int bx = (h + 63) / 64;
+  int splits = rows_one_splits(h, w);
+  if (splits > 1 && (bx > ws.num_counters || (size_t)splits * h > ws.partial_floats)) return ERROR_GENERIC;
+  const int cps = (w + splits - 1) / splits;
+  splits = (w + cps - 1) / cps;
+  dim3 grid(bx, splits);
+  const bool stream = (long long)w * h >= DN_STREAM_MIN_ELEMS;
+  if (cps <= 64)
+    hipLaunchKernelGGL((k_rows_one<OP, 4, 4, false>), grid, dim3(256), 0, 0, M, ld, h, w, cps, x, y, ws.partial, ws.counters, alpha, beta);
+  else if (stream)
+    hipLaunchKernelGGL((k_rows_one<OP, 16, 8, true>), grid, dim3(1024), 0, 0, M, ld, h, w, cps, x, y, ws.partial, ws.counters, alpha, beta);
+  else
+    hipLaunchKernelGGL((k_rows_one<OP, 16, 8, false>), grid, dim3(1024), 0, 0, M, ld, h, w, cps, x, y, ws.partial, ws.counters, alpha, beta);
+  return dn_launch_status();
+}
+
+static inline bool rows_one_ok(const float* M, int ld, int h) {
+  return dn_aligned16(M) && (ld % 4 == 0) && (h % 4 == 0);
+}
+
+// The library's own workspace: counters for 16384 row blocks (zeroed once; matrices with
+// more rows than that have no column slices), partials from the grow-only scratch.
+static int rows_workspace(int h, int w, RowsWorkspace* ws) {
+  static unsigned* counters = nullptr;
+  const int kCounters = 16384;
+  ws->partial = nullptr; ws->partial_floats = 0; ws->counters = nullptr; ws->num_counters = 0;
+  const int splits = rows_one_splits(h, w);
+  if (splits == 1) return 0;
+  if (!counters) {
+    if (hipMalloc(&counters, kCounters * sizeof(unsigned)) != hipSuccess) { counters = nullptr; hipGetLastError(); return CUDA_ERROR; }
+    if (hipMemset(counters, 0, kCounters * sizeof(unsigned)) != hipSuccess) return CUDA_ERROR;
+  }
+  ws->partial = (float*)dn_scratch((size_t)splits * h * sizeof(float));
+  if (!ws->partial) return CUDA_ERROR;
+  ws->partial_floats = (size_t)splits * h;
+  ws->counters = counters;
+  ws->num_counters = kCounters;
+  return 0;
+}
+
 template <int OP>
 static int rows_reduce(const float* M, int ld, int h, int w, const float* x, float* y, float alpha, float beta) {
   if (h <= 0) return 0;
-  const bool vec = dn_aligned16(M) && (ld % 4 == 0) && (h % 4 == 0) && h >= 1024;
+  if (rows_one_ok(M, ld, h) && rows_one_splits(h, w) > 0) {
+    RowsWorkspace ws;
+    if (int e = rows_workspace(h, w, &ws)) return e;
+    return rows_reduce_one<OP>(M, ld, h, w, x, y, alpha, beta, ws);
+  }
+  const bool vec = rows_one_ok(M, ld, h) && h >= 1024;
   const int rows_per_block = vec ? 256 : 64;
   const int bx = (h + rows_per_block - 1) / rows_per_block;
   int splits = (8 * dn_num_cus()) / bx;
@@ -685,11 +837,6 @@ static int rows_reduce(const float* M, int ld, int h, int w, const float* x, flo
     if (!partial) return CUDA_ERROR;
   }
   dim3 grid(bx, splits);
-  // One launch with the last-arriving workgroup of a row block adding up the partial
-  // sums was measured and lost: device-scope atomics on one counter are served one
-  // after the other at about 190 ns each (64 arrivals: +12 us), and a release fence
-  // per workgroup costs more still.  A workgroup that owns few rows over all columns
-  // needs no second stage but reads 64-byte runs (18 us against 12 + 2.5 for two stages).
   if (vec) {
     // 8 wavefronts x 8 columns in flight: a 64-column slice is one trip
     if (cps > 16 && (long long)w * h >= DN_STREAM_MIN_ELEMS)
