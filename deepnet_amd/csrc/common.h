@@ -12,6 +12,9 @@ int dn_num_cus();
 // Grow-only device workspaces (slot 0: partials and scalar results; slot 1: conv patch matrix).
 void* dn_scratch(size_t bytes, int slot = 0);
 
+// Looks up (once per device) the fixed workspace of the entry points that allocate nothing.
+int dn_noalloc_setup();
+
 // Records the launch status of the kernel just queued; returns CUDA_ERROR or 0.
 static inline int dn_launch_status() {
   return hipPeekAtLastError() == hipSuccess ? 0 : CUDA_ERROR;

@@ -122,6 +122,8 @@ int cublas_init(void) {
   // the device so a missing GPU is reported here rather than at the first op.
   int n = 0;
   if (hipGetDeviceCount(&n) != hipSuccess || n <= 0) return CUBLAS_ERROR;
+  // the fixed workspace of the entry points that allocate nothing, for the current device
+  if (dn_noalloc_setup() == CUDA_ERROR) return CUBLAS_ERROR;
   return 0;
 }
 

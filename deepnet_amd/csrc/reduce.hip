@@ -859,6 +859,38 @@ static int rows_reduce(const float* M, int ld, int h, int w, const float* x, flo
   return dn_launch_status();
 }
 
+// ------------------------------------------------------------------ reductions that allocate nothing
+// A fixed workspace for k_rows_one inside the code object, for callers that may not
+// allocate (HIP graph capture, serving loops): room for NOALLOC_PARTIAL_FLOATS slice
+// partials and NOALLOC_COUNTERS arrival counters.  Every GPU holds its own copy of the
+// array at its own address; the address is looked up once per device.
+#define NOALLOC_PARTIAL_FLOATS 65536
+#define NOALLOC_COUNTERS 1024
+#define NOALLOC_MAX_DEVICES 16
+static __device__ __align__(256) unsigned char scratch[(NOALLOC_PARTIAL_FLOATS + NOALLOC_COUNTERS) * 4];
+static unsigned char* g_noalloc_ptr[NOALLOC_MAX_DEVICES] = {nullptr};
+
+__global__ void k_fill_u32(unsigned* p, int n, unsigned v) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+
+// Looks up the current device's copy of the workspace and clears its counters (with a
+// kernel, not a memset: a memset node must not end up in a caller's graph).
+int dn_noalloc_setup() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return CUDA_ERROR;
+  if (dev < 0 || dev >= NOALLOC_MAX_DEVICES) return ERROR_UNSUPPORTED;
+  if (g_noalloc_ptr[dev]) return 0;
+  unsigned char* ptr = nullptr;
+  if (hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return CUDA_ERROR;
+  hipLaunchKernelGGL(k_fill_u32, dim3((NOALLOC_COUNTERS + 255) / 256), dim3(256), 0, 0,
+                     reinterpret_cast<unsigned*>(ptr + (size_t)NOALLOC_PARTIAL_FLOATS * 4), NOALLOC_COUNTERS, 0u);
+  if (dn_launch_status()) return CUDA_ERROR;
+  g_noalloc_ptr[dev] = ptr;
+  return 0;
+}
+
 // Host entry points used by dot() for vector-shaped products.
 int dn_gemv_cols(const float* M, int ld, int h, int w, const float* x, float* y, float alpha, float beta) {
   if (w <= 0) return 0;
@@ -959,6 +991,51 @@ int max_by_axis(cudamat* mat, cudamat* target, int axis) {
     return rows_reduce<ROW_MAX>(mat->data_device, h, h, w, nullptr, target->data_device, 1.f, 0.f);
   }
   return ERROR_UNSUPPORTED;
+}
+
+// max_by_axis without any allocation (no counterpart in cudamat.cu; for callers that cannot
+// allocate device memory).  Same kernels and the same results as max_by_axis; the slice
+// partials and arrival counters of the axis-1 kernel live in this library's fixed workspace
+// instead of the grow-only scratch.  Returns ERROR_UNSUPPORTED when a call would need more
+// than NOALLOC_PARTIAL_FLOATS partials or NOALLOC_COUNTERS row blocks of 64 rows with
+// column slices.  Calls that overlap on one GPU (different streams or threads) race on the
+// workspace; its counters are zero between calls.
+int max_by_axis_noalloc(cudamat* mat, cudamat* target, int axis) {
+  const int h = mat->size[0], w = mat->size[1];
+  if (int e = check_axis_common(mat, target)) return e;
+  if (axis == 0) {
+    if (target->size[0] != 1 || target->size[1] != w) return ERROR_INCOMPATIBLE_DIMENSIONS;
+    if (w > 0 && colblock_launch<COL_MAX>(mat->data_device, h, h, w, nullptr, target->data_device, 1.f, 0.f))
+      return dn_launch_status();
+    return launch_cols(k_col_max<64>, k_col_max<256>, w, h, (const float*)mat->data_device, target->data_device, w, h);
+  }
+  if (axis != 1) return ERROR_UNSUPPORTED;
+  if (target->size[0] != h || target->size[1] != 1) return ERROR_INCOMPATIBLE_DIMENSIONS;
+  if (w <= 0 || h <= 0) return 0;
+  const float* M = mat->data_device;
+  if (!rows_one_ok(M, h, h) || rows_one_splits(h, w) == 0) {
+    // unaligned operand, or few rows and very many columns: the 64-row kernel over all columns,
+    // one launch and no partials
+    hipLaunchKernelGGL((k_rows_stage1<false, ROW_MAX, 4, 4, false>), dim3((h + 63) / 64, 1), dim3(256), 0, 0, M, h, h, w,
+                       w, (const float*)nullptr, target->data_device, (float*)nullptr, 1.f, 0.f);
+    return dn_launch_status();
+  }
+  RowsWorkspace ws = {nullptr, 0, nullptr, 0};
+  const int splits = rows_one_splits(h, w);
+  if (splits > 1) {
+    if ((size_t)splits * h > NOALLOC_PARTIAL_FLOATS || (h + 63) / 64 > NOALLOC_COUNTERS) return ERROR_UNSUPPORTED;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return CUDA_ERROR;
+    if (dev < 0 || dev >= NOALLOC_MAX_DEVICES) return ERROR_UNSUPPORTED;
+    if (!g_noalloc_ptr[dev])
+      if (int e = dn_noalloc_setup()) return e;
+    unsigned char* ptr = g_noalloc_ptr[dev];
+    ws.partial = reinterpret_cast<float*>(ptr);
+    ws.partial_floats = NOALLOC_PARTIAL_FLOATS;
+    ws.counters = reinterpret_cast<unsigned*>(ptr + (size_t)NOALLOC_PARTIAL_FLOATS * 4);
+    ws.num_counters = NOALLOC_COUNTERS;
+  }
+  return rows_reduce_one<ROW_MAX>(M, h, h, w, nullptr, target->data_device, 1.f, 0.f, ws);
 }
 
 int argmax_by_axis(cudamat* mat, cudamat* target, int axis) {

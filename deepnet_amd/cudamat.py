@@ -104,7 +104,7 @@ _SIGNATURES = {
     'dropout': (_i, [_R, _M, _f, _f]),
     'add_col_mult': (_i, [_M, _M, _M, _f]), 'add_row_mult': (_i, [_M, _M, _M, _f]),
     'mult_diagonal_scalar': (_i, [_M, _f, _M]), 'add_diagonal_scalar': (_i, [_M, _f, _M]),
-    'max_by_axis': (_i, [_M, _M, _i]), 'argmax_by_axis': (_i, [_M, _M, _i]),
+    'max_by_axis': (_i, [_M, _M, _i]), 'max_by_axis_noalloc': (_i, [_M, _M, _i]), 'argmax_by_axis': (_i, [_M, _M, _i]),
     'choose_max_by_axis': (_i, [_M, _M, _i]), 'choose_max_and_accumulate': (_i, [_M, _M]),
     'sqsum_by_axis': (_i, [_M, _M, _i, _f, _f]), 'normlimit_by_axis': (_i, [_M, _M, _i, _f]),
     'apply_log': (_i, [_M, _M, _f]), 'apply_pow': (_i, [_M, _f, _M]),
@@ -433,6 +433,12 @@ class CUDAMatrix(object):
     def max(self, axis, target=None):
         target = self._axis_target(axis, target)
         _check(_cudamat.max_by_axis(self.p_mat, target.p_mat, int(axis)))
+        return target
+
+    def max_noalloc(self, axis, target):
+        """max(axis) into an existing target through the entry point that allocates no
+        device memory (an extension of this backend; the target is not optional)."""
+        _check(_cudamat.max_by_axis_noalloc(self.p_mat, target.p_mat, int(axis)))
         return target
 
     def argmax(self, axis, target=None):

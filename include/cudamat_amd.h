@@ -142,6 +142,14 @@ int lower_bound_scalar(cudamat* mat, float val, cudamat* target);
  * which the reference answers with ERROR_UNSUPPORTED, reduces each row here with
  * the semantics of eigenmat/eigenmat.cc:617-731. ---- */
 int max_by_axis(cudamat* mat, cudamat* target, int axis);
+/* No counterpart in the reference.  max_by_axis for callers that cannot allocate device
+ * memory (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc): same kernels, same results, but the slice partials and arrival counters of
+ * the axis-1 kernel sit in a fixed 260 KiB workspace inside the library's code object
+ * (one copy per GPU, held until the process ends) and nothing is allocated or freed.
+ * ERROR_UNSUPPORTED (-9) when the shape would need more than 65536 partial floats or 1024
+ * row blocks with column slices.  Calls that overlap on one GPU race on the workspace. */
+int max_by_axis_noalloc(cudamat* mat, cudamat* target, int axis);
 int argmax_by_axis(cudamat* mat, cudamat* target, int axis);
 int choose_max_by_axis(cudamat* mat, cudamat* target, int axis);
 int choose_max_and_accumulate(cudamat* mat, cudamat* acc);
