@@ -351,6 +351,183 @@ k_rnorm_undo(const float* outGrads, const float* denoms, const float* inputs, co
   }
 }
 
+// The normalisation layers on maps that fit in LDS: a workgroup owns one map of IB
+// neighbouring images (QB = IB/4 groups of 4 images), reads every element once from global
+// memory (a lane of the 1024 holds up to NORM_LDS_SLOTS 16-byte groups of it in registers, all loads in
+// flight together), and forms the window sums in two passes through LDS: sums along x of
+// the squares (forward) or of the prepared acts (backward) into a second tile, then sums
+// along y of those.  Any window size; reads of a workgroup all come before its writes and
+// cover only its own tile, so operands may alias.
+//   forward:  denoms = 1 + addScale * sum(win^2);  target = imgs * denoms^-powScale
+//   backward: acts := scale * outGrads * acts / denoms (stored, as the reference's first
+//             kernel does), target = inputs * sum(acts) + outGrads * denoms^-powScale
+#define NORM_LDS_SLOTS 2
+#define NORM_LDS_THREADS 1024
+#define NORM_LDS_MAX_GROUPS (NORM_LDS_SLOTS * NORM_LDS_THREADS)   // 16-byte groups per tile (32 KiB)
+
+// SIZE > 0: window size known at compile time (all LDS reads of a lane independent and in
+// flight together); SIZE == 0: any size, a loop.
+template <int QB, bool UNDO, bool SAME, int SIZE>
+__global__ void __launch_bounds__(NORM_LDS_THREADS)
+k_norm_lds(const float* a0, const float* a1, const float* a2, const float* win, float* out0, float* out1, int N, int S,
+           FastDiv dS, int nblk, int size_rt, float addScale, float powScale) {
+  const int size = SIZE > 0 ? SIZE : size_rt;
+  // forward: a0 = imgs, win = meanDiffs (SAME: the same array), out0 = denoms, out1 = target
+  // backward: a0 = outGrads, a1 = denoms, a2 = inputs, win = acts (also written), out1 = target
+  extern __shared__ float4 lds[];
+  const int f = blockIdx.x / nblk, b = blockIdx.x - f * nblk;
+  const int n0 = b * (QB * 4);
+  const int qn = (N - n0) / 4 < QB ? (N - n0) / 4 : QB;      // image groups of this block that exist
+  const int SS = S * S;
+  const int groups = SS * QB;
+  float4* tileA = lds;
+  float4* tileB = lds + groups;
+  const size_t map0 = (size_t)N * ((size_t)f * SS) + n0;
+  const int org = UNDO ? size / 2 - size + 1 : -(size / 2);
+  float4 keep0[NORM_LDS_SLOTS], keep1[NORM_LDS_SLOTS];
+  // keep0: forward imgs / backward inputs;  keep1: backward outGrads * denoms^-powScale
+  {
+    float4 w[NORM_LDS_SLOTS], og[NORM_LDS_SLOTS], den[NORM_LDS_SLOTS];
+#pragma unroll
+    for (int k = 0; k < NORM_LDS_SLOTS; ++k) {
+      const int i = (int)threadIdx.x + NORM_LDS_THREADS * k;
+      const int pix = i / QB, q = i - pix * QB;
+      const bool ok = i < groups && q < qn;
+      const size_t off = map0 + (size_t)N * pix + 4 * q;
+      const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
+      w[k] = ok ? *reinterpret_cast<const float4*>(win + off) : z;
+      if (UNDO) {
+        og[k] = ok ? *reinterpret_cast<const float4*>(a0 + off) : z;
+        den[k] = ok ? *reinterpret_cast<const float4*>(a1 + off) : make_float4(1.f, 1.f, 1.f, 1.f);
+        keep0[k] = ok ? *reinterpret_cast<const float4*>(a2 + off) : z;
+      } else if (!SAME) {
+        keep0[k] = ok ? *reinterpret_cast<const float4*>(a0 + off) : z;
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < NORM_LDS_SLOTS; ++k) {
+      const int i = (int)threadIdx.x + NORM_LDS_THREADS * k;
+      if (i >= groups) continue;
+      if (UNDO) {
+        const float sc = addScale;                 // -2 * addScale * powScale, prepared by the host
+        float4 t;
+        t.x = (sc * og[k].x * w[k].x) / den[k].x; t.y = (sc * og[k].y * w[k].y) / den[k].y;
+        t.z = (sc * og[k].z * w[k].z) / den[k].z; t.w = (sc * og[k].w * w[k].w) / den[k].w;
+        tileA[i] = t;
+        const int pix = i / QB, q = i - pix * QB;
+        if (q < qn) *reinterpret_cast<float4*>(const_cast<float*>(win) + map0 + (size_t)N * pix + 4 * q) = t;
+        keep1[k] = make_float4(og[k].x * norm_pow(den[k].x, -powScale), og[k].y * norm_pow(den[k].y, -powScale),
+                               og[k].z * norm_pow(den[k].z, -powScale), og[k].w * norm_pow(den[k].w, -powScale));
+      } else {
+        if (SAME) keep0[k] = w[k];
+        tileA[i] = make_float4(w[k].x * w[k].x, w[k].y * w[k].y, w[k].z * w[k].z, w[k].w * w[k].w);
+      }
+    }
+  }
+  __syncthreads();
+  // sums along x
+#pragma unroll
+  for (int k = 0; k < NORM_LDS_SLOTS; ++k) {
+    const int i = (int)threadIdx.x + NORM_LDS_THREADS * k;
+    if (i >= groups) continue;
+    const int pix = i / QB;
+    const int y = (int)fd_div((uint32_t)pix, dS), x = pix - y * S;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (SIZE > 0) {
+      float4 t[SIZE > 0 ? SIZE : 1];
+#pragma unroll
+      for (int d = 0; d < SIZE; ++d) {
+        const bool ok = (unsigned)(x + org + d) < (unsigned)S;
+        t[d] = tileA[i + (ok ? (org + d) * QB : 0)];
+      }
+#pragma unroll
+      for (int d = 0; d < SIZE; ++d) {
+        const bool ok = (unsigned)(x + org + d) < (unsigned)S;
+        acc.x += ok ? t[d].x : 0.f; acc.y += ok ? t[d].y : 0.f; acc.z += ok ? t[d].z : 0.f; acc.w += ok ? t[d].w : 0.f;
+      }
+    } else {
+      const int x0 = x + org > 0 ? x + org : 0, x1 = x + org + size < S ? x + org + size : S;
+      for (int xx = x0; xx < x1; ++xx) {
+        const float4 t = tileA[i + (xx - x) * QB];
+        acc.x += t.x; acc.y += t.y; acc.z += t.z; acc.w += t.w;
+      }
+    }
+    tileB[i] = acc;
+  }
+  __syncthreads();
+  // sums along y, then the output
+#pragma unroll
+  for (int k = 0; k < NORM_LDS_SLOTS; ++k) {
+    const int i = (int)threadIdx.x + NORM_LDS_THREADS * k;
+    if (i >= groups) continue;
+    const int pix = i / QB, q = i - pix * QB;
+    if (q >= qn) continue;
+    const int y = (int)fd_div((uint32_t)pix, dS);
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (SIZE > 0) {
+      float4 t[SIZE > 0 ? SIZE : 1];
+#pragma unroll
+      for (int d = 0; d < SIZE; ++d) {
+        const bool ok = (unsigned)(y + org + d) < (unsigned)S;
+        t[d] = tileB[i + (ok ? (org + d) * S * QB : 0)];
+      }
+#pragma unroll
+      for (int d = 0; d < SIZE; ++d) {
+        const bool ok = (unsigned)(y + org + d) < (unsigned)S;
+        acc.x += ok ? t[d].x : 0.f; acc.y += ok ? t[d].y : 0.f; acc.z += ok ? t[d].z : 0.f; acc.w += ok ? t[d].w : 0.f;
+      }
+    } else {
+      const int y0 = y + org > 0 ? y + org : 0, y1 = y + org + size < S ? y + org + size : S;
+      for (int yy = y0; yy < y1; ++yy) {
+        const float4 t = tileB[i + (yy - y) * S * QB];
+        acc.x += t.x; acc.y += t.y; acc.z += t.z; acc.w += t.w;
+      }
+    }
+    const size_t off = map0 + (size_t)N * pix + 4 * q;
+    if (!UNDO) {
+      const float4 d = make_float4(1.f + addScale * acc.x, 1.f + addScale * acc.y, 1.f + addScale * acc.z, 1.f + addScale * acc.w);
+      const float4 in = keep0[k];
+      *reinterpret_cast<float4*>(out0 + off) = d;
+      *reinterpret_cast<float4*>(out1 + off) = make_float4(in.x * norm_pow(d.x, -powScale), in.y * norm_pow(d.y, -powScale),
+                                                           in.z * norm_pow(d.z, -powScale), in.w * norm_pow(d.w, -powScale));
+    } else {
+      const float4 in = keep0[k], pw = keep1[k];
+      *reinterpret_cast<float4*>(out1 + off) =
+          make_float4(in.x * acc.x + pw.x, in.y * acc.y + pw.y, in.z * acc.z + pw.z, in.w * acc.w + pw.w);
+    }
+  }
+}
+
+// Largest image block (in groups of 4 images) whose two LDS tiles fit; 0 if none does.
+static int norm_lds_qb(int N, int S) {
+  const long long ss = (long long)S * S;
+  int qb = 8;
+  while (qb >= 1 && ss * qb > NORM_LDS_MAX_GROUPS) qb >>= 1;
+  while (qb > 1 && (qb / 2) * 4 >= N) qb >>= 1;      // no wider than the batch
+  return qb;
+}
+
+template <bool UNDO>
+static void norm_lds_launch(int qb, bool same, const float* a0, const float* a1, const float* a2, const float* win,
+                            float* out0, float* out1, int N, int S, int F, int size, float addScale, float powScale) {
+  const int nblk = (N + qb * 4 - 1) / (qb * 4);
+  const dim3 grid((unsigned)(F * nblk)), block(NORM_LDS_THREADS);
+  const size_t lds = (size_t)2 * S * S * qb * sizeof(float4);
+  const FastDiv dS = make_fastdiv((uint32_t)S);
+#define NORM_LDS_GO(QB, SM, SZ) \
+  hipLaunchKernelGGL((k_norm_lds<QB, UNDO, SM, SZ>), grid, block, lds, 0, a0, a1, a2, win, out0, out1, N, S, dS, nblk, size, addScale, powScale)
+#define NORM_LDS_SZ(QB, SM) do { if (size == 3) NORM_LDS_GO(QB, SM, 3); else if (size == 5) NORM_LDS_GO(QB, SM, 5); \
+                                 else if (size == 7) NORM_LDS_GO(QB, SM, 7); else NORM_LDS_GO(QB, SM, 0); } while (0)
+#define NORM_LDS_QB(QB) do { if (same && !UNDO) NORM_LDS_SZ(QB, true); else NORM_LDS_SZ(QB, false); } while (0)
+  if (qb == 8) NORM_LDS_QB(8);
+  else if (qb == 4) NORM_LDS_QB(4);
+  else if (qb == 2) NORM_LDS_QB(2);
+  else NORM_LDS_QB(1);
+#undef NORM_LDS_QB
+#undef NORM_LDS_SZ
+#undef NORM_LDS_GO
+}
+
 // ------------------------------------------------------------------ host side
 
 #define NORM_SEG 5   // rows per lane in k_norm_rows
@@ -437,7 +614,12 @@ static void cnorm_impl(cudamat* images, cudamat* meanDiffs, cudamat* denoms, cud
                      (const float*)nullptr, (const float*)meanDiffs->data_device, denoms->data_device,           \
                      targets->data_device, g, nseg, make_fastdiv((uint32_t)nseg), addScale, powScale)
   const int nseg = (S + NORM_SEG - 1) / NORM_SEG;
-  if (v4) {
+  const int qb = v4 ? norm_lds_qb(N, S) : 0;
+  if (qb > 0 && (long long)numFilters * ((N + qb * 4 - 1) / (qb * 4)) <= 0x7fffffffll) {
+    norm_lds_launch<false>(qb, images->data_device == meanDiffs->data_device, images->data_device, nullptr, nullptr,
+                           meanDiffs->data_device, denoms->data_device, targets->data_device, N, S, numFilters, sizeX,
+                           addScale, powScale);
+  } else if (v4) {
     if (sizeX == 3) CNORM_ROWS(3);
     else if (sizeX == 5) CNORM_ROWS(5);
     else if (sizeX == 7) CNORM_ROWS(7);
@@ -464,6 +646,17 @@ static void rnorm_undo_impl(cudamat* outGrads, cudamat* denoms, cudamat* inputs,
     POOL_REQUIRE(m->size[0] == N && m->size[1] == outGrads->size[1], where);
   const long long total = (long long)N * outGrads->size[1];
   POOL_REQUIRE(total < (1ll << 32), where);
+  {
+    const bool v4all = N % 4 == 0 && all_aligned16({outGrads->data_device, denoms->data_device, inputs->data_device,
+                                                    acts->data_device, targets->data_device});
+    const int qb = v4all ? norm_lds_qb(N, S) : 0;
+    if (qb > 0) {
+      norm_lds_launch<true>(qb, false, outGrads->data_device, denoms->data_device, inputs->data_device, acts->data_device,
+                            nullptr, targets->data_device, N, S, numFilters, sizeX, -2.f * addScale * powScale, powScale);
+      if (dn_launch_status()) conv_set_error(where, hipGetErrorString(hipGetLastError()));
+      return;
+    }
+  }
   if (total % 4 == 0 && all_aligned16({acts->data_device, denoms->data_device, outGrads->data_device}))
     hipLaunchKernelGGL((k_rnorm_undo_prelim<4>), dim3(grid_for(total / 4)), dim3(256), 0, 0, acts->data_device,
                        (const float*)denoms->data_device, (const float*)outGrads->data_device, (size_t)(total / 4),
