@@ -250,20 +250,6 @@ def net_mlp(cm, sizes=(784, 1024, 1024, 10), B=128, seed=3, fused=False):
     return net
 
 
-def net_rbm(cm, nv=784, nh=500, B=100, lr=0.01, seed=1):
-    """The RBM of config 1 as a two-layer DBM object trained by CD-1: the reference's own control
-    flow (dbm.py:64-282: sufficient statistics, gradient, momentum update, the reconstruction
-    error read back every step)."""
-    from deepnet_amd import dbm, layer as dl, neuralnet as dnn, parameter as dp
-    rng = np.random.default_rng(seed)
-    hyp = lambda **kw: dp.Hyperparams(base_epsilon=lr, **kw)
-    vis = dl.LogisticLayer('visible', nv, B, hyperparams=hyp(activation=dp.LOGISTIC), is_input=True)
-    hid = dl.LogisticLayer('hidden', nh, B, hyperparams=hyp(activation=dp.LOGISTIC))
-    edge = dnn.Edge(vis, hid, 0.01 * rng.standard_normal((nv, nh)), hyperparams=hyp(), directed=False)
-    vis.data.assign(cm.CUDAMatrix(np.asarray(rng.random((nv, B)) < 0.13, dtype=np.float32, order='F')))
-    return dbm.DBM([vis, hid], [edge], optimizer='CD')
-
-
 def net_example_convnet(cm, B=100, seed=12):
     """The model of deepnet/examples/convnet (model_conv.pbtxt, batch 100 as in train.pbtxt):
     28 x 28 inputs -> conv 5 x 5 (64 filters) + pool 3/2 -> conv 5 x 5 (64 -> 64) + pool 3/2 -> 1024 ReLU
@@ -419,22 +405,52 @@ def cpu_baseline_rbm(steps=100):
     return out
 
 
-def cpu_baseline_conv_c4():
-    """One run of each conv pass of config 4 through the float64 numpy restatement (patch
-    views + tensordot; numpy's own threading): the reference's CPU library has no convolution,
-    so this is the only CPU figure there is to put beside the conv kernels."""
+def cpu_baseline_mlp(steps=8):
+    """The MLP step of config 3 (784-1024-1024-10, batch 128) through oracle/host_backend.c
+    (hb_mlp_step: the same op sequence as MLP.step), on 1 thread and on all host threads."""
+    from oracle import host_steps
+    lib = host_steps.load()
+    rng = np.random.default_rng(3)
+    sizes, B = (784, 1024, 1024, 10), 128
+    x = rng.random((sizes[0], B))
+    labels = rng.integers(0, sizes[-1], (1, B))
+    W = [0.01 * rng.standard_normal((sizes[i], sizes[i + 1])) for i in range(3)]
+    b = [np.zeros(sizes[i + 1]) for i in range(3)]
+    m = host_steps.HostMLP(lib, sizes, B, x, labels, W, b, 0.01, 0.9, seed=3)
+    out = {}
+    for threads in (1, os.cpu_count() or 1):
+        lib.hb_set_threads(threads)
+        m.step()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            m.step()
+        out[threads] = steps / (time.perf_counter() - t0)
+    lib.hb_set_threads(1)
+    return out
+
+
+def cpu_baseline_conv():
+    """The conv passes through the float64 numpy restatement (patch views + tensordot; numpy's
+    own threading): the reference's CPU library has no convolution, so this is the only CPU
+    figure there is to put beside the conv kernels.  Config 4 runs whole (one pass each);
+    configs 5a / 5b take minutes per pass at batch 128, so they run on a sample of 8 of the 128
+    images (same layer geometry, 1/16 of the work) and the time is reported for that sample."""
     from oracle import conv_oracle as co
     rng = np.random.default_rng(4)
-    N, C, H, F, k, p = 128, 3, 32, 64, 5, 2
-    x = rng.standard_normal((N, C * H * H)).astype(np.float32)
-    w = (0.01 * rng.standard_normal((F, C * k * k))).astype(np.float32)
-    y = rng.standard_normal((N, F * H * H)).astype(np.float32)
     out = {}
-    for name, fn in (('convUp', lambda: co.conv_up(x, w, C, H, p, 1)), ('convDown', lambda: co.conv_down(y, w, C, H, p, 1)),
-                     ('convOutp', lambda: co.conv_outp(x, y, C, H, k, p, 1))):
-        t0 = time.perf_counter()
-        fn()
-        out[name] = round((time.perf_counter() - t0) * 1e3, 1)
+    for name, (N, C, H, F, k, s, p, G) in (('c4', (128, 3, 32, 64, 5, 1, 2, 1)), ('c5a_8_of_128_images', (8, 3, 224, 96, 11, 4, 0, 1)),
+                                           ('c5b_8_of_128_images', (8, 96, 27, 256, 5, 1, 2, 2))):
+        Mx = (H + 2 * p - k) // s + 1
+        x = rng.standard_normal((N, C * H * H)).astype(np.float32)
+        w = (0.01 * rng.standard_normal((F, (C // G) * k * k))).astype(np.float32)
+        y = rng.standard_normal((N, F * Mx * Mx)).astype(np.float32)
+        res = {}
+        for label, fn in (('convUp', lambda: co.conv_up(x, w, C, Mx, p, s, G)), ('convDown', lambda: co.conv_down(y, w, C, H, p, s, G)),
+                          ('convOutp', lambda: co.conv_outp(x, y, C, Mx, k, p, s, G))):
+            t0 = time.perf_counter()
+            fn()
+            res[label] = round((time.perf_counter() - t0) * 1e3, 1)
+        out[name] = res
     return out
 
 
@@ -514,6 +530,8 @@ def main():
     roofline = {'kernel': 'k_ew<2, true, FAxpy> (add_mult, 4096x4096)', 'bound': 'hbm',
                 'achieved': ops[roof_op]['gbs'], 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
                 'frac': round(ops[roof_op]['gbs'] / HBM_PEAK_GBS, 4), 'traffic': traffic,
+                'traffic_source': 'profiles/k_ew_axpy_hbm_traffic.md (an earlier rocprofv3 --pmc run of bench.py --probe, '
+                                  'not measured by this run)',
                 'algorithmic_bytes_per_launch': 12 * E, 'avg_launch_us': ops[roof_op]['us']}
 
     secondary = {}
@@ -549,15 +567,6 @@ def main():
             obj.fused = True
         t = time_loop(cm, lambda: net.TrainOneBatch(0), 100, 10)
         secondary['mlp_through_neuralnet_classes']['us_per_step_fused_extensions'] = round(t * 1e6, 1)
-        rbm_net = net_rbm(cm)
-        t = time_loop(cm, lambda: rbm_net.TrainOneBatch(0), 100, 10)
-        secondary['rbm_through_dbm_class'] = {
-            'steps_per_sec': round(1.0 / t, 1), 'us_per_step': round(t * 1e6, 1),
-            'note': 'same RBM as a two-layer DBM object, TrainOneBatch (CD-1) with sufficient statistics, momentum updates and the blocking reconstruction-error read-back'}
-        for obj in rbm_net.layer + rbm_net.edge:
-            obj.fused = True
-        t = time_loop(cm, lambda: rbm_net.TrainOneBatch(0), 100, 10)
-        secondary['rbm_through_dbm_class']['us_per_step_fused_extensions'] = round(t * 1e6, 1)
         convnet = net_example_convnet(cm)
         t = time_loop(cm, lambda: convnet.TrainOneBatch(0), 50, 5)
         secondary['example_convnet_batch100'] = {
@@ -582,6 +591,8 @@ def main():
         'config': {'workload': 'elementwise+reduction+RNG microbench, 4096x4096 fp32 column-major, 13 ops x %d '
                                'operand sets per step' % NSETS, 'step_bytes': STEP_BYTES},
         'roofline': roofline, 'ops': ops, 'secondary': secondary,
+        'timing': 'value: wall time of the K steps between two device synchronisations; ops: HIP events around the %d '
+                  'launches of an op in a step, median over the K steps' % NSETS,
     }
     if not args.no_cpu:
         cb = cpu_baseline_c2()
@@ -590,7 +601,12 @@ def main():
             cb['rbm_cd1_steps_per_sec'] = {'threads_%d' % k: round(v, 2) for k, v in r.items()}
             if 'rbm_cd1' in secondary:
                 secondary['rbm_cd1']['vs_cpu_1thread'] = round(secondary['rbm_cd1']['steps_per_sec'] / r[1], 1)
-            cb['conv_c4_numpy_f64_ms'] = cpu_baseline_conv_c4()
+            r = cpu_baseline_mlp()
+            cb['mlp_784_1024_1024_10_steps_per_sec'] = {'threads_%d' % k: round(v, 2) for k, v in r.items()}
+            if 'mlp_784_1024_1024_10' in secondary:
+                secondary['mlp_784_1024_1024_10']['vs_cpu_1thread'] = round(
+                    secondary['mlp_784_1024_1024_10']['steps_per_sec'] / r[1], 1)
+            cb['conv_numpy_f64_ms'] = cpu_baseline_conv()
         line['cpu_baseline'] = cb
     print(json.dumps(line))
 

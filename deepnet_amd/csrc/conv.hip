@@ -1477,7 +1477,9 @@ static void launch_rowmajor(const ConvArgs& a0, long long rows, int cols, int gz
   const int nslabs = MODE == CONV_UP ? (a.Cg * a.kk2 + CV_BK - 1) / CV_BK : a.kk2 * (a.Fg / CV_BK);
   const long long total = MODE == CONV_UP ? (long long)a.N * a.M * a.F : (long long)a.N * a.HH * a.C;
   long long want = 1;
-  if ((MODE == CONV_UP || (MODE == CONV_DOWN && a.s == 1)) && tiles < cus && a.scale_t == 0.f && a.scale_o == 1.f) {
+  // (the sum of the partial outputs writes 16-byte groups)
+  if ((MODE == CONV_UP || (MODE == CONV_DOWN && a.s == 1)) && tiles < cus && a.scale_t == 0.f && a.scale_o == 1.f &&
+      dn_aligned16(a.out)) {
     want = (2ll * cus) / tiles;
     if (want > nslabs / 8) want = nslabs / 8;
     if (want > 16) want = 16;
@@ -1840,6 +1842,8 @@ struct PaddedBatch {
     if (Np == N || !a->on_device || (b && (!b->on_device || b->size[0] != N)) || (c && (!c->on_device || c->size[0] != N))) return;
     size_t elems = 0;
     for (cudamat* x : src) if (x) elems += ((size_t)Np * x->size[1] + 3) / 4 * 4;
+    // the copy kernel indexes with 32 bits: larger operands run unpadded
+    for (cudamat* x : src) if (x && (long long)Np * x->size[1] >= (1ll << 32)) return;
     float* ws = (float*)dn_scratch(elems * sizeof(float), 2);
     if (!ws) return;
     for (int i = 0; i < 3; ++i) {

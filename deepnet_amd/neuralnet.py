@@ -128,6 +128,7 @@ class NeuralNet(object):
     def ComputeUp(self, layer, train=False, step=0, maxsteps=0):
         """State of ``layer`` from the states of the layers feeding it; then dropout."""
         layer.dirty = False
+        perf = None
         if layer.is_input or layer.is_initialized:
             layer.GetData()
         else:
@@ -156,6 +157,10 @@ class NeuralNet(object):
                             layer.state.add_dot(w.T, inputs, mult=factor)
                 layer.state.add_col_vec(layer.params['bias'])
                 layer.ApplyActivation()
+            if layer.hyperparams.sparsity:          # neuralnet.py:176-181: the mean activity, reported as a loss record
+                layer.state.sum(axis=1, target=layer.dimsize)
+                perf = types.SimpleNamespace(count=layer.batchsize,
+                                             sparsity=layer.dimsize.sum() / layer.dimsize.shape[0])
         h = layer.hyperparams
         if h.dropout:
             if train and maxsteps - step >= h.stop_dropout_for_last:
@@ -171,7 +176,7 @@ class NeuralNet(object):
                     layer.state.mult(layer.mask)
             elif not h.mult_dropout:
                 layer.state.mult(1.0 - h.dropout_prob)      # the expected output
-        return None
+        return perf
 
     def ComputeDown(self, layer, step):
         """Back-propagate through ``layer``: its deriv holds the gradient w.r.t. its outputs on

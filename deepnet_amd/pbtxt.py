@@ -106,9 +106,12 @@ def _unquote(tok):
             if e == 'x':
                 out.append(chr(int(body[i + 1:i + 3], 16)))
                 i += 2
-            elif e in '01234567' and body[i:i + 3].isdigit():
-                out.append(chr(int(body[i:i + 3], 8)))
-                i += 2
+            elif e in '01234567':                     # one to three octal digits
+                j = i + 1
+                while j < len(body) and j < i + 3 and body[j] in '01234567':
+                    j += 1
+                out.append(chr(int(body[i:j], 8) & 0xff))
+                i = j - 1
             else:
                 out.append(_ESCAPES.get(e, e))
         else:
@@ -225,7 +228,15 @@ def merged(base, over):
 def _quote(raw):
     """A bytes or str value as a double-quoted literal in printable ASCII (octal escapes, as
     protobuf's text_format writes bytes fields)."""
-    data = raw if isinstance(raw, bytes) else raw.encode('utf-8')
+    # a parsed bytes field is a str with one character per byte: those go back out as the bytes
+    # they stand for (latin-1); only text with characters beyond 0xFF is written as UTF-8
+    if isinstance(raw, bytes):
+        data = raw
+    else:
+        try:
+            data = raw.encode('latin-1')
+        except UnicodeEncodeError:
+            data = raw.encode('utf-8')
     out = []
     for b in data:
         c = chr(b)

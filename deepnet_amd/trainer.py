@@ -17,7 +17,6 @@ import numpy as np
 from . import pbtxt
 from .choose_matrix_library import cm
 from .convolutions import ConvParams
-from .dbm import DBM
 from .layer import LAYER_TYPES
 from .neuralnet import Edge, NeuralNet
 from .parameter import Hyperparams
@@ -27,8 +26,11 @@ from .parameter import Hyperparams
 # add_noise / shift / the windows are instructions to the data handler (datahandler.py:505-535), which the
 # caller builds here.  The remaining unknown fields are read only by replicated-softmax layers
 # (normalize, the priors) and fast-dropout nets, refused by activation / model type, or by nothing
-# (adapt, learn_precision, decay_learning_rate_for_last), or concern display and model selection.
-_SWITCHES = ('shared_prior', 'soft_shared_prior', 'add_noise', 'shift', 'left_window', 'right_window')
+# (decay_learning_rate_for_last), or concern display and model selection.  adapt other than NO_ADAPT
+# raises 'Not implemented.' in the reference too (parameter.py:89-96); learn_precision selects the
+# precision parameters of Gaussian units, which are not carried over.
+_SWITCHES = ('shared_prior', 'soft_shared_prior', 'add_noise', 'shift', 'left_window', 'right_window', 'adapt',
+             'learn_precision')
 _OFF = (False, 0, 0.0, 'NO_ADAPT', None)
 
 _CONV_FIELDS = ('size', 'stride', 'padding', 'num_filters', 'num_colors', 'max_pool', 'pool_size', 'pool_stride',
@@ -205,7 +207,8 @@ def _edge(proto, model_hyp, layers, prefix=''):
 
 
 def CreateDeepnet(model, train_op=None, eval_op=None, batchsize=None):
-    """A NeuralNet (FEED_FORWARD_NET) or DBM (DBM) with its parameters on the device."""
+    """A NeuralNet (FEED_FORWARD_NET) with its parameters on the device; Boltzmann machines and
+    belief nets (model_type DBM / DBN) are refused by name."""
     model, train_op, eval_op = _as_message(model), _as_message(train_op), _as_message(eval_op)
     op = train_op or eval_op
     if batchsize is None:
@@ -223,15 +226,6 @@ def CreateDeepnet(model, train_op=None, eval_op=None, batchsize=None):
     kind = model.model_type
     if kind == 'FEED_FORWARD_NET':
         net = NeuralNet(layers, edges, verbose=bool(op and op.get('verbose', False)))
-    elif kind == 'DBM':
-        h = _hyperparams(model_hyp, None, 'model')
-        optimizer = train_op.get('optimizer', 'CD') if train_op else 'CD'
-        if optimizer not in ('CD', 'PCD'):
-            raise NotImplementedError('a DBM is trained with CD or PCD, not %s' % optimizer)
-        net = DBM(layers, edges, optimizer=optimizer, mf_steps=h.mf_steps, gibbs_steps=h.gibbs_steps,
-                  start_step_up_cd_after=h.start_step_up_cd_after, step_up_cd_after=h.step_up_cd_after,
-                  positive_phase_order=[by_name[n] for n in model.all('positive_phase_order')] or None,
-                  negative_phase_order=[by_name[n] for n in model.all('negative_phase_order')] or None)
     else:
         raise NotImplementedError('model_type %s is not supported' % kind)
     net.net, net.t_op, net.e_op, net.batchsize = model, train_op, eval_op, batchsize

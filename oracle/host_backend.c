@@ -271,3 +271,60 @@ void hb_rbm_cd1_step(float* W, float* bv, float* bh, const float* v, int nv, int
   hb_add_sums(h, bh, nh, B, 1, 1.f, eps);
   hb_add_sums(h2, bh, nh, B, 1, 1.f, -eps);
 }
+
+/* ------------------------------------------------------------------ MLP step
+ * One momentum-SGD step of a ReLU net with dropout 0.5 on the hidden layers and a
+ * softmax output, written against the ops above in the order deepnet issues them
+ * (forward deepnet/neuralnet.py:138-205, loss and its gradient softmax_layer.py:40-66,
+ * backward neuralnet.py:207-291, update parameter.py:80-106 with momentum only):
+ *   a[i+1] = W[i]^T a[i] + b[i];  hidden: max(.,0) * (u > 0.5), u from the MWC streams;
+ *   top: softmax;  loss[j] = -log(p[label_j, j] + 1e-10);  d[nl-1] = p - onehot(label)
+ *   gW[i] = a[i] d[i]^T / B;  gb[i] = rowsum(d[i]) / B;  d[i-1] = (W[i] d[i]) * (a[i] > 0)
+ *   dX = mom * dX + gX;  X -= lr * dX      for X in W[i], b[i]
+ * nl weight layers, sizes[0..nl]; every array column-major with the unit index fastest.
+ * Pinned by tests/test_oracle_host.py against oracle/net_oracle.py fed the masks drawn here.
+ */
+void hb_mlp_step(int nl, const int* sizes, int B, float lr, float mom, float** W, float** b, float** dW, float** db,
+                 float** gW, float** gb, float** act, float** mask, float** delta, const float* labels, float* loss,
+                 const uint32_t* mults, uint64_t* words) {
+  for (int i = 0; i < nl; ++i) {
+    const int in = sizes[i], out = sizes[i + 1];
+    const size_t n = (size_t)out * B;
+    hb_gemm(1, 0, out, B, in, 1.f, W[i], in, act[i], in, 0.f, act[i + 1], out);
+    hb_add_col_vec(act[i + 1], b[i], act[i + 1], out, B);
+    if (i < nl - 1) {
+      hb_lower_bound_scalar(act[i + 1], 0.f, act[i + 1], n);
+      mwc_uniform(mults, words, mask[i], n);
+      hb_greater_than_scalar(mask[i], 0.5f, mask[i], n);
+      hb_mult(act[i + 1], mask[i], act[i + 1], n);
+    } else {
+      hb_softmax(act[i + 1], act[i + 1], out, B);
+    }
+  }
+  {
+    const int out = sizes[nl];
+    const float* p = act[nl];
+    float* d = delta[nl - 1];
+    for (int j = 0; j < B; ++j) {
+      const int label = (int)labels[j];
+      loss[j] = -logf(p[(size_t)j * out + label] + 1e-10f);
+      for (int i = 0; i < out; ++i) d[(size_t)j * out + i] = p[(size_t)j * out + i] - (i == label ? 1.f : 0.f);
+    }
+  }
+  const float invB = 1.f / (float)B;
+  for (int i = nl - 1; i >= 0; --i) {
+    const int in = sizes[i], out = sizes[i + 1];
+    memset(gW[i], 0, sizeof(float) * (size_t)in * out);
+    hb_gemm(0, 1, in, out, B, invB, act[i], in, delta[i], out, 1.f, gW[i], in);
+    hb_add_sums(delta[i], gb[i], out, B, 1, 0.f, invB);
+    if (i > 0) {
+      hb_gemm(0, 0, in, B, out, 1.f, W[i], in, delta[i], out, 0.f, delta[i - 1], in);
+      hb_relu_deriv(delta[i - 1], act[i], delta[i - 1], (size_t)in * B);
+    }
+  }
+  for (int i = 0; i < nl; ++i) {
+    const size_t nw = (size_t)sizes[i] * sizes[i + 1], nb = (size_t)sizes[i + 1];
+    hb_mult_scalar(dW[i], mom, dW[i], nw); hb_add_mult(dW[i], gW[i], 1.f, nw); hb_add_mult(W[i], dW[i], -lr, nw);
+    hb_mult_scalar(db[i], mom, db[i], nb); hb_add_mult(db[i], gb[i], 1.f, nb); hb_add_mult(b[i], db[i], -lr, nb);
+  }
+}

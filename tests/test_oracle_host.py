@@ -86,3 +86,37 @@ def test_rbm_step_matches_a_numpy_evaluation(lib, rng):
     assert np.allclose(W, W0 + eps * (v @ hh.T - vv @ hh2.T), rtol=1e-4, atol=1e-6)
     assert np.allclose(bv, bv0 + eps * (v.sum(axis=1) - vv.sum(axis=1)), rtol=1e-4, atol=1e-6)
     assert np.allclose(bh, bh0 + eps * (hh.sum(axis=1) - hh2.sum(axis=1)), rtol=1e-4, atol=1e-6)
+
+
+def test_mlp_step_matches_the_float64_net_oracle(lib, rng):
+    """hb_mlp_step (the CPU baseline of the MLP benchmark step) against oracle/net_oracle.py,
+    itself pinned by torch SGD, fed the dropout masks the C code drew; and the masks against
+    the host generator."""
+    import sys
+    sys.path.insert(0, ROOT)
+    from oracle import host_steps, mwc, net_oracle as no
+    sizes, B, lr, mom = (20, 16, 12, 5), 8, 0.1, 0.9
+    x = rng.random((sizes[0], B))
+    labels = rng.integers(0, sizes[-1], B)
+    W = [0.3 * rng.standard_normal((sizes[i], sizes[i + 1])) for i in range(3)]
+    b = [0.1 * rng.standard_normal(sizes[i + 1]) for i in range(3)]
+    m = host_steps.HostMLP(lib, sizes, B, x, labels, W, b, lr, mom, seed=5)
+    hyp = lambda **kw: no.Hyper(base_epsilon=lr, initial_momentum=mom, final_momentum=mom, **kw)
+    layers = [{'act': 'LINEAR', 'hyper': hyp()}]
+    for i, act in enumerate(('RECTIFIED_LINEAR', 'RECTIFIED_LINEAR', 'SOFTMAX')):
+        layers.append({'act': act, 'hyper': hyp(dropout=i < 2), 'bias': m.b[i].copy(),
+                       'edge': {'w': m.W[i].copy(), 'hyper': hyp()}, 'loss': 'CROSS_ENTROPY'})
+    onet = no.Net(layers)
+    host = mwc.MWC(m.mults, 5)
+    x32 = m.act[0].astype(np.float64)
+    for step in range(3):
+        m.step()
+        for k in range(2):
+            u = host.uniform(sizes[k + 1] * B).reshape((sizes[k + 1], B), order='F')
+            assert np.array_equal(m.mask[k], (u > np.float32(0.5)).astype(np.float32))
+        perf = onet.train_step(x32, labels.reshape(1, -1), step, masks=[None, m.mask[0], m.mask[1], None])
+        assert abs(float(m.loss.sum()) - perf['cross_entropy']) <= 1e-5 * perf['cross_entropy']
+        for i in range(3):
+            L = onet.layers[i + 1]
+            assert np.allclose(m.W[i], L['edge']['w'], rtol=1e-4, atol=1e-6)
+            assert np.allclose(m.b[i], L['bias'].ravel(), rtol=1e-4, atol=1e-6)

@@ -94,3 +94,37 @@ def test_written_text_reads_back_the_same_tree():
     m.set('seed', 3)
     m.set('shape', 1, 2)
     assert m.seed == 3 and m.names().index('seed') == 2 and m.all('shape') == [1, 2]
+
+
+def test_bytes_fields_survive_parse_and_dumps_more_than_once(tmp_path):
+    """A stored parameter is raw float32 bytes (util.py:13-21); most of them are >= 0x80.  A
+    parsed model holds them as a str with one character per byte, and writing that back must
+    give the same bytes again, however often."""
+    import numpy as np
+    from deepnet_amd import util
+    arr = np.array([[-1.5, 3.25e-7], [1e30, -0.0]], dtype=np.float32)
+    raw = arr.tobytes() + bytes(range(256))
+    m = pbtxt.Message()
+    p = pbtxt.Message()
+    p.add('name', 'weight')
+    p.add('mat', raw)
+    m.add('param', p)
+    text1 = pbtxt.dumps(m)
+    once = pbtxt.parse(text1)
+    text2 = pbtxt.dumps(once)
+    twice = pbtxt.parse(text2)
+    assert text1 == text2 and text1.isascii()
+    for got in (once.param.mat, twice.param.mat):
+        assert len(got) == len(raw) and got.encode('latin-1') == raw
+    # ReadModel -> WritePbtxt -> ReadModel
+    path1, path2 = str(tmp_path / 'a.pbtxt'), str(tmp_path / 'b.pbtxt')
+    util.WritePbtxt(path1, m)
+    util.WritePbtxt(path2, util.ReadModel(path1))
+    assert util.ReadModel(path2).param.mat.encode('latin-1') == raw
+    # text beyond latin-1 is still written (as UTF-8 bytes)
+    assert '\\' in pbtxt.dumps(pbtxt.parse('name: "\u4e2d"'))
+
+
+def test_octal_and_hex_escapes_of_one_to_three_digits():
+    m = pbtxt.parse(r'a: "\0" b: "\18" c: "\101\7z" d: "\x41\377" e: "\1019"')
+    assert m.a == '\x00' and m.b == '\x018' and m.c == 'A\x07z' and m.d == 'A\xff' and m.e == 'A9'
