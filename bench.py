@@ -468,6 +468,9 @@ def main():
     ap.add_argument('--probe', action='store_true',
                     help='run only the roofline kernel (add_mult) and a copy-shaped calibration kernel '
                          '(mult by a scalar into a second matrix), for rocprofv3 --pmc runs')
+    ap.add_argument('--probe-c2', action='store_true',
+                    help='launch every op of the 4096^2 list three times over the 8 operand sets, plus the copy-shaped '
+                         'calibration kernel, and nothing else (for rocprofv3 --pmc runs)')
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this backend has no multi-GPU path (run with --gpus 1).")
@@ -495,6 +498,16 @@ def main():
                 s['A'].mult(1.0, target=s['T'])       # k_ew<1, true, FMulS>: reads 64 MiB, writes 64 MiB
         cm.cuda_sync_threads()
         print(json.dumps({'probe': 'done', 'elements': E}))
+        return
+
+    if args.probe_c2:
+        sets = build_c2(cm)
+        for _ in range(3):
+            for s in sets:
+                s['A'].mult(1.0, target=s['T'])       # k_ew<1, true, FMulS>: reads 64 MiB, writes 64 MiB
+            run_c2_step(cm, sets)
+        cm.cuda_sync_threads()
+        print(json.dumps({'probe_c2': 'done', 'elements': E, 'ops': [n for n, _, _ in C2_OPS]}))
         return
 
     sets = build_c2(cm)

@@ -79,7 +79,30 @@ def run(cm, ev, iters=10):
         out[name] = res
         for m in (X, W, Y, up, down, dw):
             m.free_device_memory()
+    out['local_64x8x8_64f3'] = _local(cm, cc, ev, iters, rng)
     return {'conv': out}
+
+
+def _local(cm, cc, ev, iters, rng):
+    """A locally connected layer (unshared filters: one bank per module) at batch 128:
+    64 colours on 8 x 8 maps, 64 filters of 3 x 3, padding 1 (64 modules)."""
+    N, C, H, F, k, s, p = 128, 64, 8, 64, 3, 1, 1
+    Mx = (H + 2 * p - k) // s + 1
+    M = Mx * Mx
+    f = lambda a: cm.CUDAMatrix(np.asarray(a, dtype=np.float32, order='F'))
+    X, W, Y = f(rng.standard_normal((N, C * H * H))), f(0.01 * rng.standard_normal((F, M * C * k * k))), f(rng.standard_normal((N, F * M)))
+    up, down, dw = cm.empty((N, F * M)), cm.empty((N, C * H * H)), cm.empty((F, M * C * k * k))
+    flops = 2.0 * N * F * M * C * k * k
+    res = {'gflop_per_pass': round(flops / 1e9, 3)}
+    for label, fn in (('localUp', lambda: cc.localUp(X, W, up, Mx, p, s, C)),
+                      ('localDown', lambda: cc.localDown(Y, W, down, Mx, p, s, k, H, C)),
+                      ('localOutp', lambda: cc.localOutp(X, Y, dw, Mx, p, k, s, C))):
+        ms = _time(ev, fn, iters, cm.cuda_sync_threads)
+        tf = flops / (ms * 1e-3) / 1e12
+        res[label] = {'ms': round(ms, 4), 'tflops': round(tf, 2), 'frac_mfma_fp32': round(tf / MFMA_FP32_PEAK_TFLOPS, 4)}
+    for m in (X, W, Y, up, down, dw):
+        m.free_device_memory()
+    return res
 
 
 def _stage(cm, ev, iters, L, W, rng):

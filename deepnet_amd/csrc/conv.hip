@@ -55,9 +55,10 @@ struct ConvArgs {
   int N, C, Cg, H, F, Fg, k, Mx, s, pad0, G;
   int M, HH, kk2;     // Mx*Mx, H*H, k*k
   int m_begin, m_count;  // Outp: module chunk [m_begin, m_begin + m_count)
+  int chunks;            // Outp, general kernel: chunks of m_count modules batched along grid z (1: one chunk)
   int splits, slabs_per_split;   // Outp always; Up / Down (stride 1) when the tiles alone cannot fill the chip
   long long split_stride;        // Up / Down with splits > 1: elements between the partial outputs in `partial`
-  int local;          // 1: one filter bank per module (locally connected layers); direct kernels only
+  int local;          // 1: one filter bank per module (locally connected layers); direct and uniform-row kernels
   float scale_t, scale_o;
   unsigned a_bytes, b_bytes;  // sizes of the two gathered arrays (uniform-row kernels: buffer ranges)
   int yq;             // CONV_DOWNM: stride x stride pixel blocks per image side
@@ -182,8 +183,9 @@ __device__ __forceinline__ void down_axis(int ph, int s, int pad0, int H, int k,
 // an add and a load.  convUp: the rows fill their tiles, and a tap beyond the reduction
 // re-reads the last one against a zero filter row.  convOutp: rows and columns beyond
 // the output are computed on whatever valid data was read and never stored.
-template <int MODE, int WAVES_M, int WM, int WN, bool UNI = false, int N16 = 0, bool INSIDE = false>
+template <int MODE, int WAVES_M, int WM, int WN, bool UNI = false, int N16 = 0, bool INSIDE = false, bool LOCAL = false>
 __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
+  static_assert(!LOCAL || UNI, "one filter bank per module: uniform-row kernels only");
   static_assert(!INSIDE || ((MODE == CONV_UP || MODE == CONV_OUTP) && !UNI), "INSIDE: the general gathers of the image");
   constexpr int WAVES_N = 4 / WAVES_M;
   constexpr int BM = 32 * WM * WAVES_M, BN = 32 * WN * WAVES_N;
@@ -202,7 +204,7 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
   const int N = p.N, H = p.H, HH = p.HH, Mx = p.Mx, M = p.M, F = p.F, Fg = p.Fg, Cg = p.Cg, k = p.k, s = p.s;
 
   // ---- what this workgroup computes
-  int g, rows, cols, nslabs, slab_beg, slab_end, zsplit = 0;
+  int g, rows, cols, nslabs, slab_beg, slab_end, zsplit = 0, out_chunk = 0;
   DownPhase ph;
   if (MODE == CONV_UP) {
     g = blockIdx.z / p.splits;
@@ -236,7 +238,9 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
     slab_beg = p.splits > 1 ? zsplit * p.slabs_per_split : 0;
     slab_end = p.splits > 1 && slab_beg + p.slabs_per_split < nslabs ? slab_beg + p.slabs_per_split : nslabs;
   } else {
-    g = blockIdx.z / p.splits;
+    const int zz = blockIdx.z / p.splits;               // (chunk, group)
+    g = zz % p.G;
+    out_chunk = zz / p.G;
     zsplit = blockIdx.z % p.splits;
     rows = Fg; cols = Cg * p.kk2;
     nslabs = p.m_count * (N / CV_BK);
@@ -284,7 +288,7 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
       a_r[u] = f >> 2; a_k[u] = (f & 3) << 2;
       const int r = row0 + a_r[u];
       a_ok[u] = a_ok[u] && r < rows;
-      a_off[u] = (long long)N * M * (g * Fg + r) + (long long)N * p.m_begin;
+      a_off[u] = (long long)N * M * (g * Fg + r) + (long long)N * (p.m_begin + out_chunk * p.m_count);
       a_y[u] = a_x[u] = 0;
     } else {
       a_k[u] = f / A_ROWLANES; a_r[u] = (f % A_ROWLANES) << 2;
@@ -348,6 +352,10 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
   int u_bks[NB], m_py[NB], m_px[NB];
   int u_y = 0, u_x = 0;
   unsigned u_n0 = 0;
+  // locally connected layers: one filter bank per module, F * Cg * k * k floats apart
+  // (filters laid out (module, colour, ky, kx, filter)); convolution: one bank
+  const unsigned bank_bytes = LOCAL ? 4u * (unsigned)F * (unsigned)(Cg * p.kk2) : 0u;
+  unsigned u_bank = 0;
   if constexpr (UNI) {
     static_assert(MODE != CONV_OUTP && BM == 128, "uniform rows: Up / Down with 128-row tiles");
     const int pos = (int)fd_div((uint32_t)row0, p.dN);       // scalar: module (Up) or pixel of the phase (Down)
@@ -355,6 +363,7 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
     if (MODE == CONV_UP) {
       const int my = (int)fd_div((uint32_t)pos, p.dMx), mx = pos - my * Mx;
       u_y = my * s + p.pad0; u_x = mx * s + p.pad0;
+      u_bank = bank_bytes * (unsigned)pos;                     // this tile's module
     } else {
       const int qyi = ph.QX > 0 ? pos / ph.QX : 0, qxi = pos - qyi * ph.QX;
       u_y = ph.qy_first + qyi; u_x = ph.qx_first + qxi;
@@ -388,7 +397,7 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
     st_a = ph.TX > 0 ? tap / ph.TX : 0; st_b = tap - st_a * ph.TX;  // t, u
   } else if (MODE == CONV_OUTP) {
     const int per_mod = N / CV_BK;
-    const int m = p.m_begin + slab_beg / per_mod;
+    const int m = p.m_begin + out_chunk * p.m_count + slab_beg / per_mod;
     st_c = (slab_beg % per_mod) * CV_BK;                  // n0
     st_a = m / Mx; st_b = m - st_a * Mx;                  // my, mx
   }
@@ -443,8 +452,18 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
       for (int u = 0; u < NB; ++u) {
         unsigned so;
         unsigned voff = u_bvo[u];
-        if (MODE == CONV_UP) so = 4u * (unsigned)F * (unsigned)(kk0 + u_bks[u]);
-        else so = 4u * (unsigned)(F * ((ph.py + s * st_a) * k + ph.px + s * st_b) + st_c);
+        if (MODE == CONV_UP) {
+          so = 4u * (unsigned)F * (unsigned)(kk0 + u_bks[u]) + u_bank;
+        } else {
+          so = 4u * (unsigned)(F * ((ph.py + s * st_a) * k + ph.px + s * st_b) + st_c);
+          if constexpr (LOCAL) {
+            // the bank of the module this slab's tap reaches (a module outside the map has zero
+            // activations: any bank will do)
+            const int my = u_y - st_a, mx = u_x - st_b;
+            const bool in_map = ((unsigned)my < (unsigned)Mx) & ((unsigned)mx < (unsigned)Mx);
+            so += in_map ? bank_bytes * (unsigned)(my * Mx + mx) : 0u;
+          }
+        }
         if (MODE == CONV_DOWNM) {                              // this column's tap of module (Y - t, X - u), if it has one
           const bool ok = (m_py[u] + s * st_a < k) & (m_px[u] + s * st_b < k);
           voff = ok ? voff : p.b_bytes;
@@ -758,7 +777,7 @@ __global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
       rbase = (long long)N * ((long long)g * Cg * HH + y * H + x) + n;  // + c * N*HH
       cstride = (long long)N * HH;
     } else {
-      rbase = (long long)zsplit * ((long long)p.G * Fg * Cg * p.kk2) + ((long long)g * Cg * p.kk2) * Fg + r;
+      rbase = ((long long)out_chunk * p.splits + zsplit) * ((long long)p.G * Fg * Cg * p.kk2) + ((long long)g * Cg * p.kk2) * Fg + r;
       cstride = Fg;                                     // partial[zsplit][g][q][f]
     }
 #pragma unroll
@@ -983,17 +1002,18 @@ __global__ void __launch_bounds__(256) k_conv_outp_finish(ConvArgs p) {
   const int per_group = p.Fg * p.Cg * p.kk2;
   const int total = p.G * per_group;
   const int e = blockIdx.x * 16 + r;
+  const float* part = p.partial + (size_t)blockIdx.y * p.splits * total;   // (grid y: chunk of modules)
   float acc = 0.f;
   if (e < total) {
     int z = grp;
     for (; z + 112 < p.splits; z += 128) {
       float v[8];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) v[u] = p.partial[(size_t)(z + 16 * u) * total + e];
+      for (int u = 0; u < 8; ++u) v[u] = part[(size_t)(z + 16 * u) * total + e];
 #pragma unroll
       for (int u = 0; u < 8; ++u) acc += v[u];
     }
-    for (; z < p.splits; z += 16) acc += p.partial[(size_t)z * total + e];
+    for (; z < p.splits; z += 16) acc += part[(size_t)z * total + e];
   }
   sv[grp][r] = acc;
   __syncthreads();
@@ -1003,7 +1023,7 @@ __global__ void __launch_bounds__(256) k_conv_outp_finish(ConvArgs p) {
     for (int g2 = 1; g2 < 16; ++g2) sum += sv[g2][r];
     const int g = e / per_group, rem = e - g * per_group;
     const int q = rem / p.Fg, fl = rem - q * p.Fg;
-    float* t = p.out + (size_t)p.F * q + g * p.Fg + fl;
+    float* t = p.out + (size_t)blockIdx.y * total + (size_t)p.F * q + g * p.Fg + fl;
     *t = (p.scale_t == 0.f ? 0.f : p.scale_t * *t) + p.scale_o * sum;
   }
 }
@@ -1433,7 +1453,7 @@ static bool fast_ok(const ConvArgs& a) {
 static void fill_common(ConvArgs& a, int N, int C, int G, int H, int F, int k, int Mx, int s, int pad0) {
   a.N = N; a.C = C; a.G = G; a.Cg = C / G; a.H = H; a.F = F; a.Fg = F / G; a.k = k; a.Mx = Mx; a.s = s; a.pad0 = pad0;
   a.M = Mx * Mx; a.HH = H * H; a.kk2 = k * k;
-  a.m_begin = 0; a.m_count = a.M; a.splits = 1; a.slabs_per_split = 0; a.split_stride = 0; a.local = 0;
+  a.m_begin = 0; a.m_count = a.M; a.chunks = 1; a.splits = 1; a.slabs_per_split = 0; a.split_stride = 0; a.local = 0;
   a.scale_t = 0.f; a.scale_o = 1.f; a.partial = nullptr; a.a_bytes = 0; a.b_bytes = 0;
   a.dN = make_fastdiv((uint32_t)N); a.dMx = make_fastdiv((uint32_t)Mx);
   a.dk = make_fastdiv((uint32_t)k); a.dkk2 = make_fastdiv((uint32_t)(k * k));
@@ -1463,6 +1483,10 @@ __global__ void __launch_bounds__(256) k_conv_sum_splits(const float* partial, i
 
 template <int MODE>
 static void launch_rowmajor_tiles(const ConvArgs& a, long long rows, int cols, int gz);
+template <int MODE, bool LOCAL = false>
+static void launch_uniform_rows(const ConvArgs& a, long long rows, int cols, int gz);
+template <int MODE>
+static void launch_general_rows(const ConvArgs& a, long long rows, int cols, int gz);
 
 // Layers on small maps (8 x 8, 16 x 16 modules at batch 128) have fewer tiles than the chip
 // has CUs, and a lone workgroup per CU walks its reduction at the pace of the memory
@@ -1512,12 +1536,22 @@ static void launch_rowmajor_tiles(const ConvArgs& a, long long rows, int cols, i
   // faster on the 256-row tiles below.
   const int nslabs = MODE == CONV_UP ? (a.Cg * a.kk2 + CV_BK - 1) / CV_BK : a.kk2 * (a.Fg / CV_BK) / (a.s * a.s);
   if (a.N % 128 == 0 && a.a_bytes != 0 && a.b_bytes != 0 && nslabs >= 16 && (cols <= 64 || cols > 96)) {
+    launch_uniform_rows<MODE>(a, rows, cols, gz);
+    return;
+  }
+  launch_general_rows<MODE>(a, rows, cols, gz);
+}
+
+// The uniform-row kernels (batch a multiple of 128, both operands within 32-bit buffer ranges).
+template <int MODE, bool LOCAL>
+static void launch_uniform_rows(const ConvArgs& a, long long rows, int cols, int gz) {
+  {
     const unsigned gx = (unsigned)(rows / 128);
     // (column counts that leave a 32-wide block half empty take 16-wide blocks)
-    if (cols <= 16) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 1, true, 1>), dim3(gx, 1, gz), dim3(256), 0, 0, a);
-    else if (cols <= 32) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 1, true>), dim3(gx, (cols + 31) / 32, gz), dim3(256), 0, 0, a);
-    else if (cols <= 48) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 2, true, 3>), dim3(gx, 1, gz), dim3(256), 0, 0, a);
-    else if (cols <= 64) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 2, true>), dim3(gx, (cols + 63) / 64, gz), dim3(256), 0, 0, a);
+    if (cols <= 16) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 1, true, 1, false, LOCAL>), dim3(gx, 1, gz), dim3(256), 0, 0, a);
+    else if (cols <= 32) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 1, true, 0, false, LOCAL>), dim3(gx, (cols + 31) / 32, gz), dim3(256), 0, 0, a);
+    else if (cols <= 48) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 2, true, 3, false, LOCAL>), dim3(gx, 1, gz), dim3(256), 0, 0, a);
+    else if (cols <= 64) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 2, true, 0, false, LOCAL>), dim3(gx, (cols + 63) / 64, gz), dim3(256), 0, 0, a);
     else {
       // More than 96 columns: 128-wide tiles (64 x 64 per wavefront) or 64-wide ones (32 x 64).
       // What decides is how full the column tiles are and how evenly the tiles spread over the
@@ -1529,11 +1563,14 @@ static void launch_rowmajor_tiles(const ConvArgs& a, long long rows, int cols, i
       const int c128 = (cols + 127) / 128, c64 = (cols + 63) / 64;
       const double s128 = (double)cols / (128.0 * c128) * spread((long long)gx * c128 * gz);
       const double s64 = (double)cols / (64.0 * c64) * spread((long long)gx * c64 * gz) * (MODE == CONV_UP ? 0.82 : 1.0);
-      if (s64 > s128) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 2, true>), dim3(gx, c64, gz), dim3(256), 0, 0, a);
-      else hipLaunchKernelGGL((k_conv_mfma<MODE, 2, 2, 2, true>), dim3(gx, c128, gz), dim3(256), 0, 0, a);
+      if (s64 > s128) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 2, true, 0, false, LOCAL>), dim3(gx, c64, gz), dim3(256), 0, 0, a);
+      else hipLaunchKernelGGL((k_conv_mfma<MODE, 2, 2, 2, true, 0, false, LOCAL>), dim3(gx, c128, gz), dim3(256), 0, 0, a);
     }
-    return;
   }
+}
+
+template <int MODE>
+static void launch_general_rows(const ConvArgs& a, long long rows, int cols, int gz) {
   // Up / Down: rows are plentiful, columns few: 4 wavefronts down the rows, WN blocks across.
   // With enough rows to keep every CU busy twice over, each wavefront takes two row
   // blocks (256-row tiles): twice the MFMAs per LDS read and per barrier.
@@ -1604,6 +1641,10 @@ static void conv_up_impl(cudamat* images, cudamat* filters, cudamat* targets, in
     }
   } else if (!local && fast_ok(a)) {
     launch_rowmajor<CONV_UP>(a, (long long)M * N, a.Fg, numGroups);
+  } else if (local && fast_ok(a) && N % 128 == 0 && a.a_bytes != 0 && a.b_bytes != 0) {
+    // locally connected: a 128-row tile is one module, so the uniform-row kernels only add that
+    // module's bank to the filter offset
+    launch_uniform_rows<CONV_UP, true>(a, (long long)M * N, a.Fg, numGroups);
   } else {
     const long long total = (long long)N * M * F;
     long long blocks = (total + 255) / 256;
@@ -1638,19 +1679,30 @@ static void conv_down_impl(cudamat* hidActs, cudamat* filters, cudamat* targets,
   a.img = a.hid;  // alignment test only
   a.local = local ? 1 : 0;
   set_buffer_ranges(a, (long long)N * M * F, (long long)F * filters->size[1]);
-  if (!local && fast_ok(a) && dn_aligned16(a.out) && a.Cg <= 16 && moduleStride > 1 && N % 128 == 0 && a.a_bytes != 0) {
+  const bool local_uni = local && fast_ok(a) && dn_aligned16(a.out) && N % 128 == 0 && a.a_bytes != 0 && a.b_bytes != 0;
+  if ((!local || local_uni) && fast_ok(a) && dn_aligned16(a.out) && a.Cg <= 16 && moduleStride > 1 && N % 128 == 0 &&
+      a.a_bytes != 0 && a.b_bytes != 0) {
     // few colours, strided: the stride^2 pixel phases become columns of one implicit GEMM
     const int padw = paddingStart < 0 ? -paddingStart : 0;
     a.yq = (imgSize - 1 + padw) / moduleStride + 1;
     const int cols = a.Cg * moduleStride * moduleStride;
     const unsigned gx = (unsigned)((long long)a.yq * a.yq * N / 128);
     // column counts that leave a 32-wide block half empty take 16-wide blocks
-    if (cols <= 16) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 1, true, 1>), dim3(gx, 1, numGroups), dim3(256), 0, 0, a);
-    else if (cols <= 32) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 1, true>), dim3(gx, 1, numGroups), dim3(256), 0, 0, a);
-    else if (cols <= 48) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 2, true, 3>), dim3(gx, 1, numGroups), dim3(256), 0, 0, a);
-    else if (cols <= 64) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 2, true>), dim3(gx, 1, numGroups), dim3(256), 0, 0, a);
-    else if (cols <= 96) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 3, true>), dim3(gx, 1, numGroups), dim3(256), 0, 0, a);
-    else hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 2, 2, 2, true>), dim3(gx, (cols + 127) / 128, numGroups), dim3(256), 0, 0, a);
+    if (local) {
+      if (cols <= 16) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 1, true, 1, false, true>), dim3(gx, 1, numGroups), dim3(256), 0, 0, a);
+      else if (cols <= 32) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 1, true, 0, false, true>), dim3(gx, 1, numGroups), dim3(256), 0, 0, a);
+      else if (cols <= 48) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 2, true, 3, false, true>), dim3(gx, 1, numGroups), dim3(256), 0, 0, a);
+      else if (cols <= 64) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 2, true, 0, false, true>), dim3(gx, 1, numGroups), dim3(256), 0, 0, a);
+      else if (cols <= 96) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 3, true, 0, false, true>), dim3(gx, 1, numGroups), dim3(256), 0, 0, a);
+      else hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 2, 2, 2, true, 0, false, true>), dim3(gx, (cols + 127) / 128, numGroups), dim3(256), 0, 0, a);
+    } else {
+      if (cols <= 16) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 1, true, 1>), dim3(gx, 1, numGroups), dim3(256), 0, 0, a);
+      else if (cols <= 32) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 1, true>), dim3(gx, 1, numGroups), dim3(256), 0, 0, a);
+      else if (cols <= 48) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 2, true, 3>), dim3(gx, 1, numGroups), dim3(256), 0, 0, a);
+      else if (cols <= 64) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 2, true>), dim3(gx, 1, numGroups), dim3(256), 0, 0, a);
+      else if (cols <= 96) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 3, true>), dim3(gx, 1, numGroups), dim3(256), 0, 0, a);
+      else hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 2, 2, 2, true>), dim3(gx, (cols + 127) / 128, numGroups), dim3(256), 0, 0, a);
+    }
   } else if (!local && fast_ok(a) && dn_aligned16(a.out) && a.Cg <= 16) {
     // few colours: patch-matrix form
     const long long prow = (long long)a.M * N;
@@ -1687,6 +1739,10 @@ static void conv_down_impl(cudamat* hidActs, cudamat* filters, cudamat* targets,
   } else if (!local && fast_ok(a) && dn_aligned16(a.out)) {
     const int q = (imgSize + moduleStride - 1) / moduleStride;
     launch_rowmajor<CONV_DOWN>(a, (long long)q * q * N, a.Cg, numGroups * moduleStride * moduleStride);
+  } else if (local_uni) {
+    // locally connected: a 128-row tile is one pixel; every slab adds the bank of the module its tap reaches
+    const int q = (imgSize + moduleStride - 1) / moduleStride;
+    launch_uniform_rows<CONV_DOWN, true>(a, (long long)q * q * N, a.Cg, numGroups * moduleStride * moduleStride);
   } else {
     const long long total = (long long)N * a.HH * numImgColors;
     long long blocks = (total + 255) / 256;
@@ -1723,10 +1779,14 @@ static void conv_outp_impl(cudamat* images, cudamat* hidActs, cudamat* targets, 
   a.img = images->data_device; a.hid = hidActs->data_device; a.flt = a.img;
   const int cols = Cg * a.kk2;
   const bool fast = fast_ok(a);
-  for (int ch = 0; ch < chunks; ++ch) {
+  // Several chunks (partial sums over groups of modules; one module each for a locally connected
+  // layer): all of them in one launch of the general kernel, the chunk along grid z
+  const bool batched = fast && chunks > 1;
+  for (int ch = 0; ch < (batched ? 1 : chunks); ++ch) {
     a.m_begin = ch * partialSum; a.m_count = partialSum;
+    a.chunks = batched ? chunks : 1;
     a.out = targets->data_device + (size_t)ch * cols * F;
-    const bool small = fast && a.Fg <= 64 && cols <= 96 && N % 64 == 0 &&
+    const bool small = fast && !batched && a.Fg <= 64 && cols <= 96 && N % 64 == 0 &&
                        (long long)N * numImgColors * H * H * 4 < (1ll << 31) && (long long)N * M * F * 4 < (1ll << 31);
     if (small) {
       // few filters and few patch columns: every wavefront holds the whole output block
@@ -1752,15 +1812,16 @@ static void conv_outp_impl(cudamat* images, cudamat* hidActs, cudamat* targets, 
       const int gx = (Fg + BMs - 1) / BMs, gy = (cols + 127) / 128;
       const int nslabs = a.m_count * (N / CV_BK);
       // about two workgroups per CU (measured against one and three), at least 16 slabs (256 of the reduction) per split
-      long long want = (2ll * dn_num_cus()) / ((long long)gx * gy * numGroups);
+      long long want = (2ll * dn_num_cus()) / ((long long)gx * gy * numGroups * a.chunks);
       if (want < 1) want = 1;
       if (want > nslabs / 16) want = nslabs / 16 > 0 ? nslabs / 16 : 1;
       if (want > 512) want = 512;
       a.slabs_per_split = (int)((nslabs + want - 1) / want);
       a.splits = (nslabs + a.slabs_per_split - 1) / a.slabs_per_split;
-      a.partial = (float*)dn_scratch((size_t)a.splits * F * cols * sizeof(float));
+      CONV_REQUIRE((long long)numGroups * a.splits * a.chunks <= 65535, where);
+      a.partial = (float*)dn_scratch((size_t)a.chunks * a.splits * F * cols * sizeof(float));
       if (!a.partial) { conv_set_error(where, "out of device memory for the split-K workspace"); return; }
-      dim3 grid(gx, gy, numGroups * a.splits);
+      dim3 grid(gx, gy, numGroups * a.splits * a.chunks);
       if (paddingStart == 0 && (numModulesX - 1) * moduleStride + filterSize <= H) {  // nothing to mask in the image gather
         if (BMs == 32) hipLaunchKernelGGL((k_conv_mfma<CONV_OUTP, 1, 1, 1, false, 0, true>), grid, dim3(256), 0, 0, a);
         else if (BMs == 64) hipLaunchKernelGGL((k_conv_mfma<CONV_OUTP, 1, 2, 1, false, 0, true>), grid, dim3(256), 0, 0, a);
@@ -1772,7 +1833,7 @@ static void conv_outp_impl(cudamat* images, cudamat* hidActs, cudamat* targets, 
       else if (BMs == 96) hipLaunchKernelGGL((k_conv_mfma<CONV_OUTP, 1, 3, 1>), grid, dim3(256), 0, 0, a);
       else hipLaunchKernelGGL((k_conv_mfma<CONV_OUTP, 2, 2, 2>), grid, dim3(256), 0, 0, a);
       const int total = F * cols;
-      hipLaunchKernelGGL(k_conv_outp_finish, dim3((total + 15) / 16), dim3(256), 0, 0, a);
+      hipLaunchKernelGGL(k_conv_outp_finish, dim3((total + 15) / 16, a.chunks), dim3(256), 0, 0, a);
     } else {
       hipLaunchKernelGGL(k_conv_outp_direct, dim3((unsigned)(F * cols)), dim3(256), 0, 0, a);
     }
@@ -1837,7 +1898,10 @@ struct PaddedBatch {
   cudamat m[3];
   int N, Np;
   bool on;
-  PaddedBatch(cudamat* a, cudamat* b, cudamat* c) : N(a->size[0]), Np(padded_batch(a->size[0])), on(false) {
+  // to128: round every batch of at least 32 images up to a multiple of 128 (locally connected
+  // layers, whose matrix-core kernels need that)
+  PaddedBatch(cudamat* a, cudamat* b, cudamat* c, bool to128 = false)
+      : N(a->size[0]), Np(to128 && a->size[0] >= 32 ? (a->size[0] + 127) / 128 * 128 : padded_batch(a->size[0])), on(false) {
     cudamat* src[3] = {a, b, c};
     if (Np == N || !a->on_device || (b && (!b->on_device || b->size[0] != N)) || (c && (!c->on_device || c->size[0] != N))) return;
     size_t elems = 0;
@@ -2007,16 +2071,35 @@ void convOutp(cudamat* images, cudamat* hidActs, cudamat* targets, int numModule
 }
 
 // Locally connected layers: one filter bank per module, filters laid out
-// (module, colour, ky, kx, filter) (cudamat_conv_kernels.cuh:66-67).  They run on the
-// one-lane-per-output kernels; the weight gradient is convOutp with one module per
-// chunk, which is how the reference computes it too (cudamat_conv.cu:1421-1423).
+// (module, colour, ky, kx, filter) (cudamat_conv_kernels.cuh:66-67).  Batches that are a
+// multiple of 128 run on the uniform-row matrix-core kernels, which add a module's bank to
+// the filter offset (the reference switches its conv kernels the same way, with a template
+// flag, cudamat_conv.cu:1415-1420); other batches are padded up to one when that is cheap,
+// else take the one-lane-per-output kernels.  The weight gradient is convOutp with one
+// module per chunk, which is how the reference computes it too (cudamat_conv.cu:1421-1423).
 void localUp(cudamat* images, cudamat* filters, cudamat* targets, int numModulesX, int paddingStart, int moduleStride,
              int numImgColors, int numGroups) {
+  PaddedBatch pb(images, targets, nullptr, true);
+  if (pb.on) {
+    pb.fill(0, images);
+    conv_up_impl(&pb.m[0], filters, &pb.m[1], numModulesX, paddingStart, moduleStride, numImgColors, numGroups, "localUp",
+                 true);
+    if (!conv_last_error()) pb.drain(1, targets);
+    return;
+  }
   conv_up_impl(images, filters, targets, numModulesX, paddingStart, moduleStride, numImgColors, numGroups, "localUp",
                true);
 }
 void localDown(cudamat* hidActs, cudamat* filters, cudamat* targets, int imgSize, int paddingStart, int moduleStride,
                int numImgColors, int numGroups) {
+  PaddedBatch pb(hidActs, targets, nullptr, true);
+  if (pb.on) {
+    pb.fill(0, hidActs);
+    conv_down_impl(&pb.m[0], filters, &pb.m[1], imgSize, paddingStart, moduleStride, numImgColors, numGroups, "localDown",
+                   true);
+    if (!conv_last_error()) pb.drain(1, targets);
+    return;
+  }
   conv_down_impl(hidActs, filters, targets, imgSize, paddingStart, moduleStride, numImgColors, numGroups, "localDown",
                  true);
 }

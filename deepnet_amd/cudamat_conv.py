@@ -109,19 +109,21 @@ def localUp(images, filters, targets, numModulesX, paddingStart, moduleStride, n
           numImgColors, numGroups)
 
 
-def localDown(hidSums, filters, targets, numModulesX, paddingStart, moduleStride, filterSizeX, imSizeX, numImgColors):
+def localDown(hidSums, filters, targets, numModulesX, paddingStart, moduleStride, filterSizeX, imSizeX, numImgColors,
+              numGroups=1):
     numImages = hidSums.shape[0]
     assert paddingStart >= 0
     assert targets.shape == (numImages, numImgColors * imSizeX * imSizeX)
     _call('localDown', hidSums.p_mat, filters.p_mat, targets.p_mat, imSizeX, -paddingStart, moduleStride,
-          numImgColors, 1)
+          numImgColors, numGroups)
 
 
-def localOutp(images, hidSums, targets, numModulesX, paddingStart, filterSizeX, moduleStride, numImgColors):
+def localOutp(images, hidSums, targets, numModulesX, paddingStart, filterSizeX, moduleStride, numImgColors,
+              numGroups=1):
     numFilters = hidSums.shape[1] // (numModulesX ** 2)
-    assert targets.shape == (numFilters, numModulesX ** 2 * numImgColors * filterSizeX ** 2)
+    assert targets.shape == (numFilters, numModulesX ** 2 * (numImgColors // numGroups) * filterSizeX ** 2)
     _call('localOutp', images.p_mat, hidSums.p_mat, targets.p_mat, numModulesX, filterSizeX, -paddingStart,
-          moduleStride, numImgColors, 1, 0)
+          moduleStride, numImgColors, numGroups, 0)
 
 
 def MaxPool(images, targets, numChannels, subsX, startX, strideX, outputsX):

@@ -257,7 +257,14 @@ def test_conv_layer_chain_like_deepnet(cm, cc, rng):
     assert np.allclose(out.asarray(), want.T, rtol=2e-4, atol=2e-5)
 
 
-@pytest.mark.parametrize("N,C,H,F,k,s,p", [(4, 2, 6, 16, 3, 1, 1), (16, 3, 8, 16, 3, 2, 0)])
+@pytest.mark.parametrize("N,C,H,F,k,s,p", [
+    (4, 2, 6, 16, 3, 1, 1), (16, 3, 8, 16, 3, 2, 0),           # one lane per output
+    # batches of 128: the matrix-core kernels with one filter bank per module.  Stride 1 and
+    # strided with few colours (phases merged into columns) or many; 16 to 96 filters; padding
+    (128, 3, 8, 32, 3, 1, 1), (128, 3, 9, 16, 3, 2, 0), (128, 20, 6, 48, 3, 1, 0), (256, 4, 7, 64, 5, 1, 2),
+    (128, 32, 6, 96, 3, 2, 1), (128, 1, 10, 16, 4, 2, 0), (128, 3, 12, 64, 5, 1, 2),
+    # batches that are padded up to 128 (100 images, 40 images), and one too small for that
+    (100, 3, 8, 32, 3, 1, 1), (40, 2, 7, 16, 3, 2, 1), (24, 2, 7, 16, 3, 2, 1)])
 def test_locally_connected_layers(cm, cc, rng, N, C, H, F, k, s, p):
     Mx = co.n_modules(H, k, s, p)
     M = Mx * Mx
@@ -272,6 +279,30 @@ def test_locally_connected_layers(cm, cc, rng, N, C, H, F, k, s, p):
     assert np.allclose(down.asarray(), co.local_down(y, w, C, H, p, s), rtol=1e-4, atol=1e-5)
     cc.localOutp(X, Y, outp, Mx, p, k, s, C)
     assert np.allclose(outp.asarray(), co.local_outp(x, y, C, Mx, k, p, s), rtol=1e-4, atol=1e-4)
+
+
+def test_locally_connected_layers_with_groups(cm, cc, rng):
+    """Two groups at batch 128: each group of filters sees its own half of the colours, which is
+    the ungrouped layer applied to the two halves."""
+    N, C, H, F, k, s, p, G = 128, 8, 7, 64, 3, 1, 1, 2
+    Mx = co.n_modules(H, k, s, p)
+    M, Cg, Fg = Mx * Mx, C // G, F // G
+    x = _f(rng.standard_normal((N, C * H * H)))
+    w = _f(0.1 * rng.standard_normal((F, M * Cg * k * k)))
+    y = _f(rng.standard_normal((N, F * M)))
+    X, W, Y = cm.CUDAMatrix(x), cm.CUDAMatrix(w), cm.CUDAMatrix(y)
+    up, down, outp = cm.empty((N, F * M)), cm.empty((N, C * H * H)), cm.empty((F, M * Cg * k * k))
+    cc.localUp(X, W, up, Mx, p, s, C, G)
+    cc.localDown(Y, W, down, Mx, p, s, k, H, C, numGroups=G)
+    cc.localOutp(X, Y, outp, Mx, p, k, s, C, numGroups=G)
+    for g in range(G):
+        xs = x[:, g * Cg * H * H:(g + 1) * Cg * H * H]
+        ws = w[g * Fg:(g + 1) * Fg]
+        ys = y[:, g * Fg * M:(g + 1) * Fg * M]
+        assert np.allclose(up.asarray()[:, g * Fg * M:(g + 1) * Fg * M], co.local_up(xs, ws, Cg, Mx, p, s), rtol=1e-4, atol=1e-5)
+        assert np.allclose(down.asarray()[:, g * Cg * H * H:(g + 1) * Cg * H * H], co.local_down(ys, ws, Cg, H, p, s),
+                           rtol=1e-4, atol=1e-5)
+        assert np.allclose(outp.asarray()[g * Fg:(g + 1) * Fg], co.local_outp(xs, ys, Cg, Mx, k, p, s), rtol=1e-4, atol=1e-4)
 
 
 def _random_conv_cases(seed, count):
