@@ -495,6 +495,107 @@ k_gemm_small(const float* __restrict__ A, int lda, const float* __restrict__ B, 
   }
 }
 
+// The same single-launch scheme on 16 x 16 output blocks (v_mfma_f32_16x16x4_f32), for products
+// whose 32 x 32 blocks would occupy less than half of the CUs (the forward passes of the RBM
+// and MLP configurations: 500 x 100 and 1024 x 128 outputs): four times the workgroups, so
+// the matrix-core time of a block (K/32 chunks of 8 instructions) spreads over the whole chip.
+// Lane (i, kq) of a wavefront holds, for chunk c, row i of an operand at k = 32c + 8kq + j,
+// j < 8: two 16-byte loads when the operand is K-contiguous, 64-byte runs per 16 lanes when
+// it is not; step j of a chunk multiplies the four k values {8kq + j}.  The NW wavefronts take
+// every NW-th chunk, four in flight each, and add up through LDS in wavefront order.
+typedef float f32x4m __attribute__((ext_vector_type(4)));
+
+// One whole chunk: no conditions, so that every load of a wavefront's four chunks is in
+// flight before the first multiplication (16-byte requests are taken at 4-byte alignment).
+template <bool KC>
+__device__ __forceinline__ void tile16_load(const float* __restrict__ P, unsigned ld, unsigned row, int chunk, int kq,
+                                            float (&r)[8]) {
+  const unsigned kl = 32u * (unsigned)chunk + 8u * (unsigned)kq;
+  if (KC) {
+    const char* base = reinterpret_cast<const char*>(P) + ((size_t)row * ld + kl) * 4u;
+    const gemm_f4u t0 = *reinterpret_cast<const gemm_f4u*>(base), t1 = *reinterpret_cast<const gemm_f4u*>(base + 16);
+    r[0] = t0.x; r[1] = t0.y; r[2] = t0.z; r[3] = t0.w; r[4] = t1.x; r[5] = t1.y; r[6] = t1.z; r[7] = t1.w;
+  } else {
+    const float* pu = P + (size_t)kl * ld + row;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) r[j] = pu[(size_t)j * ld];
+  }
+}
+// The chunk that crosses K: element by element, zero beyond K.
+template <bool KC>
+__device__ __forceinline__ void tile16_load_tail(const float* __restrict__ P, unsigned ld, unsigned row, int chunk, int kq,
+                                                 int K, float (&r)[8]) {
+  const int kl = 32 * chunk + 8 * kq;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const unsigned kk = (unsigned)min(kl + j, K - 1);
+    r[j] = KC ? P[(size_t)row * ld + kk] : P[(size_t)kk * ld + row];
+  }
+#pragma unroll
+  for (int j = 0; j < 8; ++j) r[j] = kl + j < K ? r[j] : 0.f;
+}
+
+template <bool A_KC, bool B_KC, int NW>
+__global__ void __launch_bounds__(NW * 64)
+k_gemm_tile16(const float* __restrict__ A, int lda, const float* __restrict__ B, int ldb, float* C, int ldc, int M, int N,
+              int K, float alpha, float beta, GemmEpilogue epi) {
+  __shared__ float red[NW][4 * 64];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int li = lane & 15, kq = lane >> 4;
+  const int m0 = blockIdx.x * 16, n0 = blockIdx.y * 16;
+  const unsigned mc = min(m0 + li, M - 1), nc = min(n0 + li, N - 1);   // rows past the edge repeat the last one; never stored
+  // the output this lane finishes after the wavefronts have met: element e = tid (NW * 64 >= 256)
+  const int ev = tid >> 6;                                   // accumulator register v of element e
+  const int em = m0 + li, en = n0 + 4 * kq + ev;
+  const bool e_ok = tid < 256 && em < M && en < N;
+  const float cprev = (beta != 0.f && e_ok) ? C[(size_t)en * ldc + em] : 0.f;
+
+  constexpr int DEPTH = 4;
+  const int nfull = K >> 5;                                  // whole chunks; wavefront wv takes wv, wv + NW, ...
+  f32x4m acc = {0.f, 0.f, 0.f, 0.f};
+  if (nfull > 0) {
+    float a[DEPTH][8], b[DEPTH][8];
+    int c = wv;
+    // a set beyond the last chunk re-reads the last one and is never multiplied
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+      const int cc = min(c + d * NW, nfull - 1);
+      tile16_load<A_KC>(A, lda, mc, cc, kq, a[d]);
+      tile16_load<B_KC>(B, ldb, nc, cc, kq, b[d]);
+    }
+    for (; c < nfull; c += DEPTH * NW) {
+#pragma unroll
+      for (int d = 0; d < DEPTH; ++d) {
+        if (c + d * NW < nfull) {                            // wave-uniform
+#pragma unroll
+          for (int j = 0; j < 8; ++j) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(b[d][j], a[d][j], acc, 0, 0, 0);
+        }
+        const int cc = min(c + (d + DEPTH) * NW, nfull - 1);
+        tile16_load<A_KC>(A, lda, mc, cc, kq, a[d]);
+        tile16_load<B_KC>(B, ldb, nc, cc, kq, b[d]);
+      }
+    }
+  }
+  if ((K & 31) && wv == nfull % NW) {                        // the ragged end of K, once
+    float ta[8], tb[8];
+    tile16_load_tail<A_KC>(A, lda, mc, nfull, kq, K, ta);
+    tile16_load_tail<B_KC>(B, ldb, nc, nfull, kq, K, tb);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(tb[j], ta[j], acc, 0, 0, 0);
+  }
+  // acc[v] of lane (i, kq) is C(m0 + i, n0 + 4*kq + v)
+#pragma unroll
+  for (int v = 0; v < 4; ++v) red[wv][v * 64 + lane] = acc[v];
+  __syncthreads();
+  if (e_ok) {
+    float sum = red[0][tid];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) sum += red[w][tid];
+    C[(size_t)en * ldc + em] = gemm_finish((beta == 0.f ? 0.f : beta * cprev) + alpha * sum, em, epi);
+  }
+}
+
 __global__ void k_gemm_splitk_finish(const float* partial, int splits, float* C, int ldc, int M, int N, float alpha,
                                      float beta) {
   const size_t total = (size_t)M * N;
@@ -560,6 +661,27 @@ static int gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, co
   // beyond about 1.5e9 multiply-adds that traffic costs more than LDS tiles with a split K
   // (measured: 4096 x 128 x 4096 66 us against 53 us, 2048 x 128 x 2048 17.7 against 21.4).
   const bool heavy = (double)M * (double)N * (double)K >= 1.5e9;
+  const long long tiles32 = (long long)((M + 31) / 32) * ((N + 31) / 32);
+  if (tiles64 < cus && off32 && !heavy && tiles32 * 2 <= cus) {
+    // 32 x 32 blocks would leave more than half of the CUs idle: 16 x 16 blocks
+    dim3 grid((M + 15) / 16, (N + 15) / 16);
+#define GEMM_T16(AK, BK_)                                                                                    \
+  do {                                                                                                       \
+    if (K <= 128)                                                                                            \
+      hipLaunchKernelGGL((k_gemm_tile16<AK, BK_, 4>), grid, dim3(256), 0, 0, A, lda, B, ldb, C, ldc, M, N, K, \
+                         alpha, beta, epi);                                                                  \
+    else                                                                                                     \
+      hipLaunchKernelGGL((k_gemm_tile16<AK, BK_, 8>), grid, dim3(512), 0, 0, A, lda, B, ldb, C, ldc, M, N, K, \
+                         alpha, beta, epi);                                                                  \
+  } while (0)
+    if (a_kc && b_kc) GEMM_T16(true, true);
+    else if (a_kc) GEMM_T16(true, false);
+    else if (b_kc) GEMM_T16(false, true);
+    else GEMM_T16(false, false);
+#undef GEMM_T16
+    if (fused) *fused = true;
+    return dn_launch_status();
+  }
   if (tiles64 < cus && off32 && !heavy) {
     dim3 grid((M + 31) / 32, (N + 31) / 32);
 #define GEMM_SMALL(AK, BK_)                                                                                  \

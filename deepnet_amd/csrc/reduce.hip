@@ -782,6 +782,8 @@ static int rows_reduce_one(const float* M, int ld, int h, int w, const float* x,
   const bool stream = (long long)w * h >= DN_STREAM_MIN_ELEMS;
   if (cps <= 64)
     hipLaunchKernelGGL((k_rows_one<OP, 4, 4, false>), grid, dim3(256), 0, 0, M, ld, h, w, cps, x, y, ws.partial, ws.counters, alpha, beta);
+  else if ((long long)w * h <= (1 << 18))   // layer states (a few hundred units x a batch): 256 lanes start sooner than 1024
+    hipLaunchKernelGGL((k_rows_one<OP, 4, 8, false>), grid, dim3(256), 0, 0, M, ld, h, w, cps, x, y, ws.partial, ws.counters, alpha, beta);
   else if (stream)
     hipLaunchKernelGGL((k_rows_one<OP, 16, 8, true>), grid, dim3(1024), 0, 0, M, ld, h, w, cps, x, y, ws.partial, ws.counters, alpha, beta);
   else
