@@ -562,6 +562,16 @@ def main():
         secondary['rbm_cd1_fused_extension'] = {
             'steps_per_sec': round(1.0 / t, 1), 'us_per_step': round(t * 1e6, 1),
             'note': 'same step with dot_bias_act (an extension of this backend, not in the reference API): 10 launches instead of 16'}
+        def recorded(step, iters, warm):
+            # the step recorded once as a HIP graph (cm.Graph, an extension of this backend) and
+            # replayed with one launch per step: same kernels, same results
+            with cm.Graph() as g:
+                step()
+            tt = time_loop(cm, g.launch, iters, warm)
+            g.free()
+            return round(tt * 1e6, 1)
+        secondary['rbm_cd1']['us_per_step_recorded_graph'] = recorded(rbm.step, 200, 20)
+        secondary['rbm_cd1_fused_extension']['us_per_step_recorded_graph'] = recorded(rbm.step_fused, 200, 20)
         cm.CUDAMatrix.init_random(3)
         mlp = MLP(cm)
         t = time_loop(cm, mlp.step, 100, 10)
@@ -571,6 +581,8 @@ def main():
         secondary['mlp_fused_extensions'] = {
             'steps_per_sec': round(1.0 / t, 1), 'us_per_step': round(t * 1e6, 1),
             'note': 'same step with dot_bias_act, softmax_ce_grad and momentum_update (extensions of this backend, not in the reference API): 32 launches instead of 51'}
+        secondary['mlp_784_1024_1024_10']['us_per_step_recorded_graph'] = recorded(mlp.step, 100, 10)
+        secondary['mlp_fused_extensions']['us_per_step_recorded_graph'] = recorded(mlp.step_fused, 100, 10)
         net = net_mlp(cm)
         t = time_loop(cm, lambda: net.TrainOneBatch(0), 100, 10)
         secondary['mlp_through_neuralnet_classes'] = {

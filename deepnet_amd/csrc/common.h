@@ -15,6 +15,11 @@ void* dn_scratch(size_t bytes, int slot = 0);
 // Looks up (once per device) the fixed workspace of the entry points that allocate nothing.
 int dn_noalloc_setup();
 
+// The stream every kernel of the library is queued on: the NULL stream, or the stream a
+// caller is capturing into a HIP graph (graph_capture_begin .. graph_capture_end).
+hipStream_t dn_stream();
+bool dn_capturing();
+
 // Records the launch status of the kernel just queued; returns CUDA_ERROR or 0.
 static inline int dn_launch_status() {
   return hipPeekAtLastError() == hipSuccess ? 0 : CUDA_ERROR;

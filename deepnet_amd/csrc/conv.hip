@@ -1523,7 +1523,7 @@ static void launch_rowmajor(const ConvArgs& a0, long long rows, int cols, int gz
     const long long total4 = total / 4;            // (the batch is a multiple of 16)
     long long blocks = (total4 + 255) / 256;
     if (blocks > 8ll * cus) blocks = 8ll * cus;
-    hipLaunchKernelGGL(k_conv_sum_splits, dim3((unsigned)blocks), dim3(256), 0, 0, (const float*)a.partial, a.splits, total4,
+    hipLaunchKernelGGL(k_conv_sum_splits, dim3((unsigned)blocks), dim3(256), 0, dn_stream(), (const float*)a.partial, a.splits, total4,
                        a.out);
   }
 }
@@ -1548,10 +1548,10 @@ static void launch_uniform_rows(const ConvArgs& a, long long rows, int cols, int
   {
     const unsigned gx = (unsigned)(rows / 128);
     // (column counts that leave a 32-wide block half empty take 16-wide blocks)
-    if (cols <= 16) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 1, true, 1, false, LOCAL>), dim3(gx, 1, gz), dim3(256), 0, 0, a);
-    else if (cols <= 32) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 1, true, 0, false, LOCAL>), dim3(gx, (cols + 31) / 32, gz), dim3(256), 0, 0, a);
-    else if (cols <= 48) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 2, true, 3, false, LOCAL>), dim3(gx, 1, gz), dim3(256), 0, 0, a);
-    else if (cols <= 64) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 2, true, 0, false, LOCAL>), dim3(gx, (cols + 63) / 64, gz), dim3(256), 0, 0, a);
+    if (cols <= 16) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 1, true, 1, false, LOCAL>), dim3(gx, 1, gz), dim3(256), 0, dn_stream(), a);
+    else if (cols <= 32) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 1, true, 0, false, LOCAL>), dim3(gx, (cols + 31) / 32, gz), dim3(256), 0, dn_stream(), a);
+    else if (cols <= 48) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 2, true, 3, false, LOCAL>), dim3(gx, 1, gz), dim3(256), 0, dn_stream(), a);
+    else if (cols <= 64) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 2, true, 0, false, LOCAL>), dim3(gx, (cols + 63) / 64, gz), dim3(256), 0, dn_stream(), a);
     else {
       // More than 96 columns: 128-wide tiles (64 x 64 per wavefront) or 64-wide ones (32 x 64).
       // What decides is how full the column tiles are and how evenly the tiles spread over the
@@ -1563,8 +1563,8 @@ static void launch_uniform_rows(const ConvArgs& a, long long rows, int cols, int
       const int c128 = (cols + 127) / 128, c64 = (cols + 63) / 64;
       const double s128 = (double)cols / (128.0 * c128) * spread((long long)gx * c128 * gz);
       const double s64 = (double)cols / (64.0 * c64) * spread((long long)gx * c64 * gz) * (MODE == CONV_UP ? 0.82 : 1.0);
-      if (s64 > s128) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 2, true, 0, false, LOCAL>), dim3(gx, c64, gz), dim3(256), 0, 0, a);
-      else hipLaunchKernelGGL((k_conv_mfma<MODE, 2, 2, 2, true, 0, false, LOCAL>), dim3(gx, c128, gz), dim3(256), 0, 0, a);
+      if (s64 > s128) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 2, true, 0, false, LOCAL>), dim3(gx, c64, gz), dim3(256), 0, dn_stream(), a);
+      else hipLaunchKernelGGL((k_conv_mfma<MODE, 2, 2, 2, true, 0, false, LOCAL>), dim3(gx, c128, gz), dim3(256), 0, dn_stream(), a);
     }
   }
 }
@@ -1579,22 +1579,22 @@ static void launch_general_rows(const ConvArgs& a, long long rows, int cols, int
     const unsigned gx = (unsigned)((rows + 255) / 256);
     if constexpr (MODE == CONV_UP) {
       if (a.pad0 == 0 && (a.Mx - 1) * a.s + a.k <= a.H && rows % 256 == 0) {  // nothing to mask in the image gather
-        if (cols <= 32) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 2, 1, false, 0, true>), dim3(gx, (cols + 31) / 32, gz), dim3(256), 0, 0, a);
-        else if (cols <= 64) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 2, 2, false, 0, true>), dim3(gx, (cols + 63) / 64, gz), dim3(256), 0, 0, a);
-        else hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 2, 3, false, 0, true>), dim3(gx, (cols + 95) / 96, gz), dim3(256), 0, 0, a);
+        if (cols <= 32) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 2, 1, false, 0, true>), dim3(gx, (cols + 31) / 32, gz), dim3(256), 0, dn_stream(), a);
+        else if (cols <= 64) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 2, 2, false, 0, true>), dim3(gx, (cols + 63) / 64, gz), dim3(256), 0, dn_stream(), a);
+        else hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 2, 3, false, 0, true>), dim3(gx, (cols + 95) / 96, gz), dim3(256), 0, dn_stream(), a);
         return;
       }
     }
-    if (cols <= 32) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 2, 1>), dim3(gx, (cols + 31) / 32, gz), dim3(256), 0, 0, a);
-    else if (cols <= 64) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 2, 2>), dim3(gx, (cols + 63) / 64, gz), dim3(256), 0, 0, a);
-    else hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 2, 3>), dim3(gx, (cols + 95) / 96, gz), dim3(256), 0, 0, a);
+    if (cols <= 32) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 2, 1>), dim3(gx, (cols + 31) / 32, gz), dim3(256), 0, dn_stream(), a);
+    else if (cols <= 64) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 2, 2>), dim3(gx, (cols + 63) / 64, gz), dim3(256), 0, dn_stream(), a);
+    else hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 2, 3>), dim3(gx, (cols + 95) / 96, gz), dim3(256), 0, dn_stream(), a);
     return;
   }
   const unsigned gx = (unsigned)((rows + 127) / 128);
-  if (cols <= 32) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 1>), dim3(gx, (cols + 31) / 32, gz), dim3(256), 0, 0, a);
-  else if (cols <= 64) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 2>), dim3(gx, (cols + 63) / 64, gz), dim3(256), 0, 0, a);
-  else if (cols <= 96) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 3>), dim3(gx, (cols + 95) / 96, gz), dim3(256), 0, 0, a);
-  else hipLaunchKernelGGL((k_conv_mfma<MODE, 2, 2, 2>), dim3(gx, (cols + 127) / 128, gz), dim3(256), 0, 0, a);  // 64 x 64 per wavefront
+  if (cols <= 32) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 1>), dim3(gx, (cols + 31) / 32, gz), dim3(256), 0, dn_stream(), a);
+  else if (cols <= 64) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 2>), dim3(gx, (cols + 63) / 64, gz), dim3(256), 0, dn_stream(), a);
+  else if (cols <= 96) hipLaunchKernelGGL((k_conv_mfma<MODE, 4, 1, 3>), dim3(gx, (cols + 95) / 96, gz), dim3(256), 0, dn_stream(), a);
+  else hipLaunchKernelGGL((k_conv_mfma<MODE, 2, 2, 2>), dim3(gx, (cols + 127) / 128, gz), dim3(256), 0, dn_stream(), a);  // 64 x 64 per wavefront
 }
 
 static void conv_up_impl(cudamat* images, cudamat* filters, cudamat* targets, int numModulesX, int paddingStart,
@@ -1633,11 +1633,11 @@ static void conv_up_impl(cudamat* images, cudamat* filters, cudamat* targets, in
     a.dS = make_fastdiv((uint32_t)(N / 32));  // tile -> (module, image block)
     a.dSS = make_fastdiv((uint32_t)(blocks * 4)); // wavefronts of a group
     if (K <= 32) {
-      if (a.Fg <= 32) hipLaunchKernelGGL((k_conv_up_regs<16, 1>), grid, dim3(256), 0, 0, a);
-      else hipLaunchKernelGGL((k_conv_up_regs<16, 2>), grid, dim3(256), 0, 0, a);
+      if (a.Fg <= 32) hipLaunchKernelGGL((k_conv_up_regs<16, 1>), grid, dim3(256), 0, dn_stream(), a);
+      else hipLaunchKernelGGL((k_conv_up_regs<16, 2>), grid, dim3(256), 0, dn_stream(), a);
     } else {
-      if (a.Fg <= 32) hipLaunchKernelGGL((k_conv_up_regs<40, 1>), grid, dim3(256), 0, 0, a);
-      else hipLaunchKernelGGL((k_conv_up_regs<40, 2>), grid, dim3(256), 0, 0, a);
+      if (a.Fg <= 32) hipLaunchKernelGGL((k_conv_up_regs<40, 1>), grid, dim3(256), 0, dn_stream(), a);
+      else hipLaunchKernelGGL((k_conv_up_regs<40, 2>), grid, dim3(256), 0, dn_stream(), a);
     }
   } else if (!local && fast_ok(a)) {
     launch_rowmajor<CONV_UP>(a, (long long)M * N, a.Fg, numGroups);
@@ -1649,7 +1649,7 @@ static void conv_up_impl(cudamat* images, cudamat* filters, cudamat* targets, in
     const long long total = (long long)N * M * F;
     long long blocks = (total + 255) / 256;
     if (blocks > dn_num_cus() * 16ll) blocks = dn_num_cus() * 16ll;
-    hipLaunchKernelGGL(k_conv_up_direct, dim3((unsigned)blocks), dim3(256), 0, 0, a);
+    hipLaunchKernelGGL(k_conv_up_direct, dim3((unsigned)blocks), dim3(256), 0, dn_stream(), a);
   }
   if (dn_launch_status()) conv_set_error(where, hipGetErrorString(hipGetLastError()));
 }
@@ -1689,19 +1689,19 @@ static void conv_down_impl(cudamat* hidActs, cudamat* filters, cudamat* targets,
     const unsigned gx = (unsigned)((long long)a.yq * a.yq * N / 128);
     // column counts that leave a 32-wide block half empty take 16-wide blocks
     if (local) {
-      if (cols <= 16) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 1, true, 1, false, true>), dim3(gx, 1, numGroups), dim3(256), 0, 0, a);
-      else if (cols <= 32) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 1, true, 0, false, true>), dim3(gx, 1, numGroups), dim3(256), 0, 0, a);
-      else if (cols <= 48) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 2, true, 3, false, true>), dim3(gx, 1, numGroups), dim3(256), 0, 0, a);
-      else if (cols <= 64) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 2, true, 0, false, true>), dim3(gx, 1, numGroups), dim3(256), 0, 0, a);
-      else if (cols <= 96) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 3, true, 0, false, true>), dim3(gx, 1, numGroups), dim3(256), 0, 0, a);
-      else hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 2, 2, 2, true, 0, false, true>), dim3(gx, (cols + 127) / 128, numGroups), dim3(256), 0, 0, a);
+      if (cols <= 16) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 1, true, 1, false, true>), dim3(gx, 1, numGroups), dim3(256), 0, dn_stream(), a);
+      else if (cols <= 32) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 1, true, 0, false, true>), dim3(gx, 1, numGroups), dim3(256), 0, dn_stream(), a);
+      else if (cols <= 48) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 2, true, 3, false, true>), dim3(gx, 1, numGroups), dim3(256), 0, dn_stream(), a);
+      else if (cols <= 64) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 2, true, 0, false, true>), dim3(gx, 1, numGroups), dim3(256), 0, dn_stream(), a);
+      else if (cols <= 96) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 3, true, 0, false, true>), dim3(gx, 1, numGroups), dim3(256), 0, dn_stream(), a);
+      else hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 2, 2, 2, true, 0, false, true>), dim3(gx, (cols + 127) / 128, numGroups), dim3(256), 0, dn_stream(), a);
     } else {
-      if (cols <= 16) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 1, true, 1>), dim3(gx, 1, numGroups), dim3(256), 0, 0, a);
-      else if (cols <= 32) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 1, true>), dim3(gx, 1, numGroups), dim3(256), 0, 0, a);
-      else if (cols <= 48) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 2, true, 3>), dim3(gx, 1, numGroups), dim3(256), 0, 0, a);
-      else if (cols <= 64) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 2, true>), dim3(gx, 1, numGroups), dim3(256), 0, 0, a);
-      else if (cols <= 96) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 3, true>), dim3(gx, 1, numGroups), dim3(256), 0, 0, a);
-      else hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 2, 2, 2, true>), dim3(gx, (cols + 127) / 128, numGroups), dim3(256), 0, 0, a);
+      if (cols <= 16) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 1, true, 1>), dim3(gx, 1, numGroups), dim3(256), 0, dn_stream(), a);
+      else if (cols <= 32) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 1, true>), dim3(gx, 1, numGroups), dim3(256), 0, dn_stream(), a);
+      else if (cols <= 48) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 2, true, 3>), dim3(gx, 1, numGroups), dim3(256), 0, dn_stream(), a);
+      else if (cols <= 64) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 2, true>), dim3(gx, 1, numGroups), dim3(256), 0, dn_stream(), a);
+      else if (cols <= 96) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 3, true>), dim3(gx, 1, numGroups), dim3(256), 0, dn_stream(), a);
+      else hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 2, 2, 2, true>), dim3(gx, (cols + 127) / 128, numGroups), dim3(256), 0, dn_stream(), a);
     }
   } else if (!local && fast_ok(a) && dn_aligned16(a.out) && a.Cg <= 16) {
     // few colours: patch-matrix form
@@ -1720,7 +1720,7 @@ static void conv_down_impl(cudamat* hidActs, cudamat* filters, cudamat* targets,
         long long blocks = (prow / 32 + 3) / 4;
         if (blocks > dn_num_cus()) blocks = dn_num_cus();  // one wavefront per SIMD, looping over tiles
         const dim3 grid((unsigned)blocks);
-#define PATCH_REGS(KS, CT) hipLaunchKernelGGL((k_conv_patch_regs<KS, CT>), grid, dim3(256), 0, 0, hid_g, flt_g, P, (int)prow, a.Fg, F, pcols, pcols8)
+#define PATCH_REGS(KS, CT) hipLaunchKernelGGL((k_conv_patch_regs<KS, CT>), grid, dim3(256), 0, dn_stream(), hid_g, flt_g, P, (int)prow, a.Fg, F, pcols, pcols8)
         if (a.Fg <= 32) { if (pcols <= 32) PATCH_REGS(16, 1); else if (pcols <= 64) PATCH_REGS(16, 2); else PATCH_REGS(16, 3); }
         else { if (pcols <= 32) PATCH_REGS(32, 1); else if (pcols <= 64) PATCH_REGS(32, 2); else PATCH_REGS(32, 3); }
 #undef PATCH_REGS
@@ -1731,10 +1731,10 @@ static void conv_down_impl(cudamat* hidActs, cudamat* filters, cudamat* targets,
       const long long lanes = (long long)(N / 4) * a.HH * a.Cg;
       long long blocks = (lanes + 255) / 256;
       if (blocks > dn_num_cus() * 64ll) blocks = dn_num_cus() * 64ll;
-      if (a.s == 1 && a.k == 3) hipLaunchKernelGGL((k_conv_down_gather_s1<3>), dim3((unsigned)blocks), dim3(256), 0, 0, a, (const float*)P, g);
-      else if (a.s == 1 && a.k == 5) hipLaunchKernelGGL((k_conv_down_gather_s1<5>), dim3((unsigned)blocks), dim3(256), 0, 0, a, (const float*)P, g);
-      else if (a.s == 1 && a.k == 7) hipLaunchKernelGGL((k_conv_down_gather_s1<7>), dim3((unsigned)blocks), dim3(256), 0, 0, a, (const float*)P, g);
-      else hipLaunchKernelGGL(k_conv_down_gather, dim3((unsigned)blocks), dim3(256), 0, 0, a, (const float*)P, g);
+      if (a.s == 1 && a.k == 3) hipLaunchKernelGGL((k_conv_down_gather_s1<3>), dim3((unsigned)blocks), dim3(256), 0, dn_stream(), a, (const float*)P, g);
+      else if (a.s == 1 && a.k == 5) hipLaunchKernelGGL((k_conv_down_gather_s1<5>), dim3((unsigned)blocks), dim3(256), 0, dn_stream(), a, (const float*)P, g);
+      else if (a.s == 1 && a.k == 7) hipLaunchKernelGGL((k_conv_down_gather_s1<7>), dim3((unsigned)blocks), dim3(256), 0, dn_stream(), a, (const float*)P, g);
+      else hipLaunchKernelGGL(k_conv_down_gather, dim3((unsigned)blocks), dim3(256), 0, dn_stream(), a, (const float*)P, g);
     }
   } else if (!local && fast_ok(a) && dn_aligned16(a.out)) {
     const int q = (imgSize + moduleStride - 1) / moduleStride;
@@ -1747,7 +1747,7 @@ static void conv_down_impl(cudamat* hidActs, cudamat* filters, cudamat* targets,
     const long long total = (long long)N * a.HH * numImgColors;
     long long blocks = (total + 255) / 256;
     if (blocks > dn_num_cus() * 16ll) blocks = dn_num_cus() * 16ll;
-    hipLaunchKernelGGL(k_conv_down_direct, dim3((unsigned)blocks), dim3(256), 0, 0, a);
+    hipLaunchKernelGGL(k_conv_down_direct, dim3((unsigned)blocks), dim3(256), 0, dn_stream(), a);
   }
   if (dn_launch_status()) conv_set_error(where, hipGetErrorString(hipGetLastError()));
 }
@@ -1798,12 +1798,12 @@ static void conv_outp_impl(cudamat* images, cudamat* hidActs, cudamat* targets, 
       if (!a.partial) { conv_set_error(where, "out of device memory for the split-K workspace"); return; }
       const dim3 grid((unsigned)nblocks, 1, numGroups);
       const int rt = a.Fg <= 32 ? 1 : 2, ct = cols <= 32 ? 1 : cols <= 64 ? 2 : 3;
-#define OUTP_SMALL(RT, CT) hipLaunchKernelGGL((k_conv_outp_small<RT, CT>), grid, dim3(256), 0, 0, a)
+#define OUTP_SMALL(RT, CT) hipLaunchKernelGGL((k_conv_outp_small<RT, CT>), grid, dim3(256), 0, dn_stream(), a)
       if (rt == 1) { if (ct == 1) OUTP_SMALL(1, 1); else if (ct == 2) OUTP_SMALL(1, 2); else OUTP_SMALL(1, 3); }
       else { if (ct == 1) OUTP_SMALL(2, 1); else if (ct == 2) OUTP_SMALL(2, 2); else OUTP_SMALL(2, 3); }
 #undef OUTP_SMALL
       const int total = F * cols;
-      hipLaunchKernelGGL(k_conv_outp_finish, dim3((total + 15) / 16), dim3(256), 0, 0, a);
+      hipLaunchKernelGGL(k_conv_outp_finish, dim3((total + 15) / 16), dim3(256), 0, dn_stream(), a);
     } else if (fast) {
       // rows = filters of a group: pick the tile height that wastes least.
       const int Fg = a.Fg;
@@ -1823,19 +1823,19 @@ static void conv_outp_impl(cudamat* images, cudamat* hidActs, cudamat* targets, 
       if (!a.partial) { conv_set_error(where, "out of device memory for the split-K workspace"); return; }
       dim3 grid(gx, gy, numGroups * a.splits * a.chunks);
       if (paddingStart == 0 && (numModulesX - 1) * moduleStride + filterSize <= H) {  // nothing to mask in the image gather
-        if (BMs == 32) hipLaunchKernelGGL((k_conv_mfma<CONV_OUTP, 1, 1, 1, false, 0, true>), grid, dim3(256), 0, 0, a);
-        else if (BMs == 64) hipLaunchKernelGGL((k_conv_mfma<CONV_OUTP, 1, 2, 1, false, 0, true>), grid, dim3(256), 0, 0, a);
-        else if (BMs == 96) hipLaunchKernelGGL((k_conv_mfma<CONV_OUTP, 1, 3, 1, false, 0, true>), grid, dim3(256), 0, 0, a);
-        else hipLaunchKernelGGL((k_conv_mfma<CONV_OUTP, 2, 2, 2, false, 0, true>), grid, dim3(256), 0, 0, a);
+        if (BMs == 32) hipLaunchKernelGGL((k_conv_mfma<CONV_OUTP, 1, 1, 1, false, 0, true>), grid, dim3(256), 0, dn_stream(), a);
+        else if (BMs == 64) hipLaunchKernelGGL((k_conv_mfma<CONV_OUTP, 1, 2, 1, false, 0, true>), grid, dim3(256), 0, dn_stream(), a);
+        else if (BMs == 96) hipLaunchKernelGGL((k_conv_mfma<CONV_OUTP, 1, 3, 1, false, 0, true>), grid, dim3(256), 0, dn_stream(), a);
+        else hipLaunchKernelGGL((k_conv_mfma<CONV_OUTP, 2, 2, 2, false, 0, true>), grid, dim3(256), 0, dn_stream(), a);
       }
-      else if (BMs == 32) hipLaunchKernelGGL((k_conv_mfma<CONV_OUTP, 1, 1, 1>), grid, dim3(256), 0, 0, a);
-      else if (BMs == 64) hipLaunchKernelGGL((k_conv_mfma<CONV_OUTP, 1, 2, 1>), grid, dim3(256), 0, 0, a);
-      else if (BMs == 96) hipLaunchKernelGGL((k_conv_mfma<CONV_OUTP, 1, 3, 1>), grid, dim3(256), 0, 0, a);
-      else hipLaunchKernelGGL((k_conv_mfma<CONV_OUTP, 2, 2, 2>), grid, dim3(256), 0, 0, a);
+      else if (BMs == 32) hipLaunchKernelGGL((k_conv_mfma<CONV_OUTP, 1, 1, 1>), grid, dim3(256), 0, dn_stream(), a);
+      else if (BMs == 64) hipLaunchKernelGGL((k_conv_mfma<CONV_OUTP, 1, 2, 1>), grid, dim3(256), 0, dn_stream(), a);
+      else if (BMs == 96) hipLaunchKernelGGL((k_conv_mfma<CONV_OUTP, 1, 3, 1>), grid, dim3(256), 0, dn_stream(), a);
+      else hipLaunchKernelGGL((k_conv_mfma<CONV_OUTP, 2, 2, 2>), grid, dim3(256), 0, dn_stream(), a);
       const int total = F * cols;
-      hipLaunchKernelGGL(k_conv_outp_finish, dim3((total + 15) / 16, a.chunks), dim3(256), 0, 0, a);
+      hipLaunchKernelGGL(k_conv_outp_finish, dim3((total + 15) / 16, a.chunks), dim3(256), 0, dn_stream(), a);
     } else {
-      hipLaunchKernelGGL(k_conv_outp_direct, dim3((unsigned)(F * cols)), dim3(256), 0, 0, a);
+      hipLaunchKernelGGL(k_conv_outp_direct, dim3((unsigned)(F * cols)), dim3(256), 0, dn_stream(), a);
     }
   }
   if (dn_launch_status()) conv_set_error(where, hipGetErrorString(hipGetLastError()));
@@ -1888,7 +1888,7 @@ static void pad_batch(const float* src, float* dst, int N, int Np, long long col
   long long blocks = (total + 255) / 256;
   if (blocks > 16ll * dn_num_cus()) blocks = 16ll * dn_num_cus();
   const FastDiv fd = make_fastdiv((uint32_t)rows);
-  hipLaunchKernelGGL(k_pad_batch, dim3((unsigned)blocks), dim3(256), 0, 0, src, dst, N, Np, (unsigned)total, fd, unpad ? 1 : 0,
+  hipLaunchKernelGGL(k_pad_batch, dim3((unsigned)blocks), dim3(256), 0, dn_stream(), src, dst, N, Np, (unsigned)total, fd, unpad ? 1 : 0,
                      vec ? 1 : 0);
 }
 
@@ -1979,10 +1979,10 @@ static void conv_up_filters(cudamat* images, cudamat* filters, cudamat* targets,
     return;
   }
   cudamat fp = pad_standin(filters, Fp, Q, &ws), tp = pad_standin(targets, N, Fp * M, &ws);
-  hipLaunchKernelGGL(k_pad_filters, dim3(pad_grid(Fp * Q)), dim3(256), 0, 0, (const float*)filters->data_device, fp.data_device, F, Fp, Q, 0);
+  hipLaunchKernelGGL(k_pad_filters, dim3(pad_grid(Fp * Q)), dim3(256), 0, dn_stream(), (const float*)filters->data_device, fp.data_device, F, Fp, Q, 0);
   conv_up_impl(images, &fp, &tp, numModulesX, paddingStart, moduleStride, numImgColors, numGroups, "convUp");
   if (!conv_last_error())
-    hipLaunchKernelGGL(k_copy_prefix, dim3(pad_grid((long long)N * F * M)), dim3(256), 0, 0, (const float*)tp.data_device,
+    hipLaunchKernelGGL(k_copy_prefix, dim3(pad_grid((long long)N * F * M)), dim3(256), 0, dn_stream(), (const float*)tp.data_device,
                        targets->data_device, (long long)N * F * M, (long long)N * F * M);
 }
 
@@ -2000,8 +2000,8 @@ static void conv_down_filters(cudamat* hidActs, cudamat* filters, cudamat* targe
   }
   const long long M = hidActs->size[1] / F;
   cudamat fp = pad_standin(filters, Fp, Q, &ws), hp = pad_standin(hidActs, N, Fp * M, &ws);
-  hipLaunchKernelGGL(k_pad_filters, dim3(pad_grid(Fp * Q)), dim3(256), 0, 0, (const float*)filters->data_device, fp.data_device, F, Fp, Q, 0);
-  hipLaunchKernelGGL(k_copy_prefix, dim3(pad_grid((long long)N * Fp * M)), dim3(256), 0, 0, (const float*)hidActs->data_device,
+  hipLaunchKernelGGL(k_pad_filters, dim3(pad_grid(Fp * Q)), dim3(256), 0, dn_stream(), (const float*)filters->data_device, fp.data_device, F, Fp, Q, 0);
+  hipLaunchKernelGGL(k_copy_prefix, dim3(pad_grid((long long)N * Fp * M)), dim3(256), 0, dn_stream(), (const float*)hidActs->data_device,
                      hp.data_device, (long long)N * F * M, (long long)N * Fp * M);
   conv_down_impl(&hp, &fp, targets, imgSize, paddingStart, moduleStride, numImgColors, numGroups, "convDown");
 }
@@ -2023,12 +2023,12 @@ static void conv_outp_filters(cudamat* images, cudamat* hidActs, cudamat* target
     return;
   }
   cudamat tp = pad_standin(targets, Fp, Q, &ws), hp = pad_standin(hidActs, N, Fp * M, &ws);
-  hipLaunchKernelGGL(k_copy_prefix, dim3(pad_grid((long long)N * Fp * M)), dim3(256), 0, 0, (const float*)hidActs->data_device,
+  hipLaunchKernelGGL(k_copy_prefix, dim3(pad_grid((long long)N * Fp * M)), dim3(256), 0, dn_stream(), (const float*)hidActs->data_device,
                      hp.data_device, (long long)N * F * M, (long long)N * Fp * M);
   conv_outp_impl(images, &hp, &tp, numModulesX, filterSize, paddingStart, moduleStride, numImgColors, numGroups, partialSum,
                  "convOutp");
   if (!conv_last_error())
-    hipLaunchKernelGGL(k_pad_filters, dim3(pad_grid((long long)F * Q)), dim3(256), 0, 0, (const float*)tp.data_device,
+    hipLaunchKernelGGL(k_pad_filters, dim3(pad_grid((long long)F * Q)), dim3(256), 0, dn_stream(), (const float*)tp.data_device,
                        targets->data_device, F, Fp, Q, 1);
 }
 

@@ -19,6 +19,14 @@ int dn_num_cus() {
   return g_num_cus;
 }
 
+// ------------------------------------------------------------------ launch stream and graph capture
+static hipStream_t g_stream = nullptr;     // nullptr: the NULL stream
+static bool g_capturing = false;
+static hipStream_t g_capture_stream = nullptr;
+
+hipStream_t dn_stream() { return g_stream; }
+bool dn_capturing() { return g_capturing; }
+
 // ------------------------------------------------------------------ scratch
 // Grow-only device workspaces.  Slot 0: partials of two-stage reductions and
 // split-K products, scalar results.  Slot 1: the patch matrix of the col2im
@@ -30,6 +38,8 @@ static size_t g_scratch_bytes[4] = {0, 0, 0, 0};
 
 void* dn_scratch(size_t bytes, int slot) {
   if (bytes > g_scratch_bytes[slot]) {
+    if (g_capturing) return nullptr;   // growing means freeing and allocating: not while a graph is recorded
+
     if (g_scratch[slot]) {
       hipDeviceSynchronize();
       hipFree(g_scratch[slot]);
@@ -138,13 +148,75 @@ int cuda_set_device(int deviceId) {
   return 0;
 }
 
-void cuda_sync_threads(void) { hipDeviceSynchronize(); }
+void cuda_sync_threads(void) { if (!g_capturing) hipDeviceSynchronize(); }
+
+// ---- HIP graphs (no counterpart in the reference): record a fixed sequence of library calls
+// once and replay it with one launch, for steps whose cost is the launching itself.
+// graph_capture_begin() switches the library to a capturing stream: every call until
+// graph_capture_end() is recorded instead of run (with the pointers and scalars it was given).
+// What cannot be recorded fails with its usual error code: calls that wait for the device
+// (copy_to_host, vdot, euclid_norm), workspaces that would have to grow (run the sequence once
+// before recording it) and the split schedule of the random generator (matrices of more than
+// 32 * 12288 elements).  The random generator's state lives on the device, so every replay
+// draws fresh numbers.  graph_launch() queues a replay on the NULL stream, in order with
+// everything else the library does.
+void* graph_capture_begin(void) {
+  if (g_capturing) return nullptr;
+  if (!g_capture_stream && hipStreamCreateWithFlags(&g_capture_stream, hipStreamNonBlocking) != hipSuccess) {
+    g_capture_stream = nullptr;
+    hipGetLastError();
+    return nullptr;
+  }
+  if (hipDeviceSynchronize() != hipSuccess) return nullptr;        // recorded work starts from a quiet device
+  if (hipStreamBeginCapture(g_capture_stream, hipStreamCaptureModeThreadLocal) != hipSuccess) {
+    hipGetLastError();
+    return nullptr;
+  }
+  g_stream = g_capture_stream;
+  g_capturing = true;
+  return (void*)g_capture_stream;
+}
+
+// Ends the recording; returns an executable graph (NULL on failure) for graph_launch / graph_free.
+void* graph_capture_end(void) {
+  if (!g_capturing) return nullptr;
+  hipGraph_t graph = nullptr;
+  const hipError_t e = hipStreamEndCapture(g_capture_stream, &graph);
+  g_stream = nullptr;
+  g_capturing = false;
+  if (e != hipSuccess || !graph) { hipGetLastError(); return nullptr; }
+  hipGraphExec_t exec = nullptr;
+  const hipError_t e2 = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+  hipGraphDestroy(graph);
+  if (e2 != hipSuccess) { hipGetLastError(); return nullptr; }
+  return (void*)exec;
+}
+
+int graph_launch(void* exec) {
+  if (!exec || g_capturing) return ERROR_GENERIC;
+  return hipGraphLaunch((hipGraphExec_t)exec, nullptr) == hipSuccess ? 0 : CUDA_ERROR;
+}
+
+int graph_free(void* exec) {
+  if (!exec) return 0;
+  hipDeviceSynchronize();
+  return hipGraphExecDestroy((hipGraphExec_t)exec) == hipSuccess ? 0 : CUDA_ERROR;
+}
+
+// A second library of this package (the conv library has its own copy of this file) joins a
+// recording by queueing on the same stream; NULL afterwards.
+int graph_set_stream(void* stream, int capturing) {
+  g_stream = (hipStream_t)stream;
+  g_capturing = capturing != 0;
+  return 0;
+}
 
 int get_leading_dimension(cudamat* mat) { return mat->is_trans ? mat->size[1] : mat->size[0]; }
 int get_nonleading_dimension(cudamat* mat) { return mat->is_trans ? mat->size[0] : mat->size[1]; }
 void set_transpose(cudamat* mat, int is_trans) { mat->is_trans = is_trans; }
 
 int allocate_device_memory(cudamat* mat) {
+  if (g_capturing) return ERROR_UNSUPPORTED;      // (allocations and transfers are not recorded into a graph)
   const long long len = dn_len(mat);
   void* p = nullptr;
   // A 0-element matrix still gets a distinct, valid pointer.
@@ -160,6 +232,7 @@ int allocate_device_memory(cudamat* mat) {
 
 int copy_to_host(cudamat* mat) {
   if (!mat->on_device) return ERROR_NOT_ON_DEVICE;
+  if (g_capturing) return ERROR_UNSUPPORTED;
   const long long len = dn_len(mat);
   if (len > 0 &&
       hipMemcpy(mat->data_host, mat->data_device, (size_t)len * sizeof(float), hipMemcpyDeviceToHost) != hipSuccess)
@@ -168,6 +241,7 @@ int copy_to_host(cudamat* mat) {
 }
 
 int copy_to_device(cudamat* mat) {
+  if (g_capturing) return ERROR_UNSUPPORTED;
   if (!mat->on_device) {
     int err = allocate_device_memory(mat);
     if (err) return err;
@@ -184,12 +258,13 @@ int copy_on_device(cudamat* mat1, cudamat* mat2) {
   const long long len = dn_len(mat1);
   if (len > 0 && mat1->data_device != mat2->data_device &&
       hipMemcpyAsync(mat2->data_device, mat1->data_device, (size_t)len * sizeof(float), hipMemcpyDeviceToDevice,
-                     0) != hipSuccess)
+                     dn_stream()) != hipSuccess)
     return CUBLAS_ERROR;
   return 0;
 }
 
 int free_device_memory(cudamat* mat) {
+  if (g_capturing) return ERROR_UNSUPPORTED;
   if (mat->owns_data && mat->on_device) {
     hipError_t e = hipFree(mat->data_device);
     mat->on_device = 0;
@@ -285,7 +360,7 @@ int get_row_slice(cudamat* source, cudamat* target, unsigned int start, unsigned
   const int rows = end - start;
   if (width == 0) return 0;
   dim3 grid((rows + 255) / 256, width < 4096 ? width : 4096);
-  hipLaunchKernelGGL(k_copy_rows, grid, dim3(256), 0, 0, source->data_device, target->data_device, rows, width,
+  hipLaunchKernelGGL(k_copy_rows, grid, dim3(256), 0, dn_stream(), source->data_device, target->data_device, rows, width,
                      height, rows, (int)start, 0);
   return dn_launch_status();
 }
@@ -298,7 +373,7 @@ int set_row_slice(cudamat* source, cudamat* target, unsigned int start, unsigned
   const int rows = end - start;
   if (width == 0) return 0;
   dim3 grid((rows + 255) / 256, width < 4096 ? width : 4096);
-  hipLaunchKernelGGL(k_copy_rows, grid, dim3(256), 0, 0, source->data_device, target->data_device, rows, width, rows,
+  hipLaunchKernelGGL(k_copy_rows, grid, dim3(256), 0, dn_stream(), source->data_device, target->data_device, rows, width, rows,
                      height, 0, (int)start);
   return dn_launch_status();
 }
@@ -309,9 +384,9 @@ int copy_transpose(cudamat* source, cudamat* target) {
   if (height == 0 || width == 0) return 0;
   dim3 grid((height + TR_TILE - 1) / TR_TILE, (width + TR_TILE - 1) / TR_TILE);
   if (height % 4 == 0 && width % 4 == 0 && dn_aligned16(source->data_device) && dn_aligned16(target->data_device))
-    hipLaunchKernelGGL(k_transpose4, grid, dim3(256), 0, 0, source->data_device, target->data_device, height, width);
+    hipLaunchKernelGGL(k_transpose4, grid, dim3(256), 0, dn_stream(), source->data_device, target->data_device, height, width);
   else
-    hipLaunchKernelGGL(k_transpose, grid, dim3(256), 0, 0, source->data_device, target->data_device, height, width);
+    hipLaunchKernelGGL(k_transpose, grid, dim3(256), 0, dn_stream(), source->data_device, target->data_device, height, width);
   return dn_launch_status();
 }
 

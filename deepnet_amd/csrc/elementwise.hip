@@ -140,14 +140,14 @@ static int launch_ew(const float* a, const float* b, float* t, long long n, F f)
     if (blocks < 1) blocks = 1;
     if (blocks > 0x7fffffffll) return ERROR_UNSUPPORTED;
     if (n >= DN_STREAM_MIN_ELEMS)
-      hipLaunchKernelGGL((k_ew<NIN, true, F>), dim3((unsigned)blocks), dim3(EW_THREADS), 0, 0, a, b, t, n, head, n4, f);
+      hipLaunchKernelGGL((k_ew<NIN, true, F>), dim3((unsigned)blocks), dim3(EW_THREADS), 0, dn_stream(), a, b, t, n, head, n4, f);
     else
-      hipLaunchKernelGGL((k_ew<NIN, false, F>), dim3((unsigned)blocks), dim3(EW_THREADS), 0, 0, a, b, t, n, head, n4, f);
+      hipLaunchKernelGGL((k_ew<NIN, false, F>), dim3((unsigned)blocks), dim3(EW_THREADS), 0, dn_stream(), a, b, t, n, head, n4, f);
   } else {
     long long blocks = (n + EW_THREADS - 1) / EW_THREADS;
     const long long cap = (long long)cus * 32;
     if (blocks > cap) blocks = cap;
-    hipLaunchKernelGGL((k_ew_scalar<NIN, F>), dim3((unsigned)blocks), dim3(EW_THREADS), 0, 0, a, b, t, n, f);
+    hipLaunchKernelGGL((k_ew_scalar<NIN, F>), dim3((unsigned)blocks), dim3(EW_THREADS), 0, dn_stream(), a, b, t, n, f);
   }
   return dn_launch_status();
 }
@@ -219,7 +219,7 @@ static int launch_bcast(const float* a, const float* vec, float* t, int h, int w
     if (blocks < 1) blocks = 1;
     const bool vec4 = COLVEC && head == 0 && h % 4 == 0 && dn_aligned16(vec);
 #define BCAST_LAUNCH(ST, V4)                                                                                  \
-  hipLaunchKernelGGL((k_bcast<COLVEC, ST, V4, F>), dim3((unsigned)blocks), dim3(EW_THREADS), 0, 0, a, vec, t, n, \
+  hipLaunchKernelGGL((k_bcast<COLVEC, ST, V4, F>), dim3((unsigned)blocks), dim3(EW_THREADS), 0, dn_stream(), a, vec, t, n, \
                      head, n4, fd, f)
     if (n >= DN_STREAM_MIN_ELEMS) {
       if (vec4) BCAST_LAUNCH(true, COLVEC); else BCAST_LAUNCH(true, false);
@@ -231,7 +231,7 @@ static int launch_bcast(const float* a, const float* vec, float* t, int h, int w
     long long blocks = (n + EW_THREADS - 1) / EW_THREADS;
     const long long cap = (long long)cus * 32;
     if (blocks > cap) blocks = cap;
-    hipLaunchKernelGGL((k_bcast_scalar<COLVEC, F>), dim3((unsigned)blocks), dim3(EW_THREADS), 0, 0, a, vec, t, n, fd,
+    hipLaunchKernelGGL((k_bcast_scalar<COLVEC, F>), dim3((unsigned)blocks), dim3(EW_THREADS), 0, dn_stream(), a, vec, t, n, fd,
                        f);
   }
   return dn_launch_status();
@@ -250,7 +250,7 @@ __global__ void k_diag(const float* a, const float* vec, float* t, int w, F f) {
 template <class F>
 static int launch_diag(const float* a, const float* vec, float* t, int w, F f) {
   if (w <= 0) return 0;
-  hipLaunchKernelGGL((k_diag<F>), dim3((w + 255) / 256), dim3(256), 0, 0, a, vec, t, w, f);
+  hipLaunchKernelGGL((k_diag<F>), dim3((w + 255) / 256), dim3(256), 0, dn_stream(), a, vec, t, w, f);
   return dn_launch_status();
 }
 
@@ -564,11 +564,11 @@ extern "C" int momentum_update(cudamat* w, cudamat* w_delta, cudamat* gradient, 
   const long long blocks = (lanes + EW_THREADS - 1) / EW_THREADS;
   if (blocks > 0x7fffffffll) return ERROR_UNSUPPORTED;
   if (vec)
-    hipLaunchKernelGGL((k_momentum_update<true>), dim3((unsigned)blocks), dim3(EW_THREADS), 0, 0, w->data_device,
+    hipLaunchKernelGGL((k_momentum_update<true>), dim3((unsigned)blocks), dim3(EW_THREADS), 0, dn_stream(), w->data_device,
                        w_delta->data_device, gradient->data_device, n, momentum, l2_decay, l1_decay, epsilon, use_l2,
                        use_l1, reset);
   else
-    hipLaunchKernelGGL((k_momentum_update<false>), dim3((unsigned)blocks), dim3(EW_THREADS), 0, 0, w->data_device,
+    hipLaunchKernelGGL((k_momentum_update<false>), dim3((unsigned)blocks), dim3(EW_THREADS), 0, dn_stream(), w->data_device,
                        w_delta->data_device, gradient->data_device, n, momentum, l2_decay, l1_decay, epsilon, use_l2,
                        use_l1, reset);
   return dn_launch_status();

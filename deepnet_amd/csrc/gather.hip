@@ -140,7 +140,7 @@ int selectRows(cudamat* source, cudamat* target, cudamat* indices) {
   if (target->size[0] != source->size[0] || target->size[1] < n || indices->size[0] != 1)
     return ERROR_INCOMPATIBLE_DIMENSIONS;
   if (n == 0 || source->size[0] == 0) return 0;
-  hipLaunchKernelGGL(k_select_cols, col_grid(source->size[0], n), dim3(256), 0, 0, (const float*)source->data_device,
+  hipLaunchKernelGGL(k_select_cols, col_grid(source->size[0], n), dim3(256), 0, dn_stream(), (const float*)source->data_device,
                      target->data_device, (const float*)indices->data_device, n, source->size[0], source->size[1]);
   return dn_launch_status();
 }
@@ -151,7 +151,7 @@ int setSelectedRows(cudamat* target, cudamat* source, cudamat* indices) {
   if (target->size[0] != source->size[0] || source->size[1] < n || indices->size[0] != 1)
     return ERROR_INCOMPATIBLE_DIMENSIONS;
   if (n == 0 || source->size[0] == 0) return 0;
-  hipLaunchKernelGGL(k_set_selected_cols, col_grid(source->size[0], n), dim3(256), 0, 0, target->data_device,
+  hipLaunchKernelGGL(k_set_selected_cols, col_grid(source->size[0], n), dim3(256), 0, dn_stream(), target->data_device,
                      (const float*)source->data_device, (const float*)indices->data_device, n, target->size[0],
                      target->size[1]);
   return dn_launch_status();
@@ -164,7 +164,7 @@ int swapColumns(cudamat* source, cudamat* target, cudamat* indices1, cudamat* in
     return ERROR_NOT_ON_DEVICE;
   if (target->size[0] != h || indices2->size[0] * indices2->size[1] != cols) return ERROR_INCOMPATIBLE_DIMENSIONS;
   if (cols == 0 || h == 0) return 0;
-  hipLaunchKernelGGL(k_swap_cols, col_grid(h, cols), dim3(256), 0, 0, source->data_device, target->data_device,
+  hipLaunchKernelGGL(k_swap_cols, col_grid(h, cols), dim3(256), 0, dn_stream(), source->data_device, target->data_device,
                      (const float*)indices1->data_device, (const float*)indices2->data_device, cols, source->size[1],
                      target->size[1], h);
   return dn_launch_status();
@@ -179,7 +179,7 @@ int generate_translations_big_var_off(cudamat* source, cudamat* target, cudamat*
       off_y->size[0] * off_y->size[1] < imgs || target_w > source_w)
     return ERROR_INCOMPATIBLE_DIMENSIONS;
   if (imgs == 0) return 0;
-  hipLaunchKernelGGL(k_translate, dim3(imgs), dim3(512), 0, 0, (const float*)source->data_device, target->data_device,
+  hipLaunchKernelGGL(k_translate, dim3(imgs), dim3(512), 0, dn_stream(), (const float*)source->data_device, target->data_device,
                      (const float*)off_x->data_device, (const float*)off_y->data_device, source_w, target_w,
                      num_channels, (long long)imgs * source->size[0]);
   return dn_launch_status();
@@ -190,7 +190,7 @@ int blockify(cudamat* source, cudamat* target, int blocksize) {
   if (source->size[0] != target->size[0] || source->size[1] != target->size[1] || blocksize <= 0)
     return ERROR_INCOMPATIBLE_DIMENSIONS;
   if (source->size[1] == 0 || source->size[0] == 0) return 0;
-  hipLaunchKernelGGL(k_blockify, dim3(source->size[1]), dim3(512), 0, 0, (const float*)source->data_device,
+  hipLaunchKernelGGL(k_blockify, dim3(source->size[1]), dim3(512), 0, dn_stream(), (const float*)source->data_device,
                      target->data_device, source->size[0], blocksize, make_fastdiv((uint32_t)blocksize));
   return dn_launch_status();
 }
@@ -203,7 +203,7 @@ int accumulate_columns(cudamat* mat, cudamat* indices, cudamat* target, float mu
   if (indices->size[0] != 1 || indices->size[1] != w) return ERROR_INCOMPATIBLE_DIMENSIONS;
   if (512 < w2) return ERROR_INCOMPATIBLE_DIMENSIONS;  // the reference's one-lane-per-target-column limit
   if (h == 0 || w2 == 0) return 0;
-  hipLaunchKernelGGL(k_accumulate_cols, col_grid(h, w2), dim3(256), 0, 0, (const float*)mat->data_device,
+  hipLaunchKernelGGL(k_accumulate_cols, col_grid(h, w2), dim3(256), 0, dn_stream(), (const float*)mat->data_device,
                      (const float*)indices->data_device, target->data_device, w, w2, h, mult, avg);
   return dn_launch_status();
 }
@@ -215,7 +215,7 @@ int expand(cudamat* source, cudamat* indices, cudamat* target) {
   if (target->size[0] != h) return ERROR_INCOMPATIBLE_DIMENSIONS;
   if (indices->size[0] != 1 || indices->size[1] != w2) return ERROR_INCOMPATIBLE_DIMENSIONS;
   if (h == 0 || w2 == 0) return 0;
-  hipLaunchKernelGGL(k_expand, col_grid(h, w2), dim3(256), 0, 0, (const float*)source->data_device,
+  hipLaunchKernelGGL(k_expand, col_grid(h, w2), dim3(256), 0, dn_stream(), (const float*)source->data_device,
                      (const float*)indices->data_device, target->data_device, h, w, w2);
   return dn_launch_status();
 }
@@ -228,7 +228,7 @@ int expand_and_add(cudamat* source, cudamat* mat, cudamat* indices, cudamat* tar
   if (indices->size[0] != 1 || indices->size[1] != w) return ERROR_INCOMPATIBLE_DIMENSIONS;
   if (mat->size[0] != h) return ERROR_INCOMPATIBLE_DIMENSIONS;
   if (h == 0 || w == 0) return 0;
-  hipLaunchKernelGGL(k_expand_and_add, col_grid(h, w), dim3(256), 0, 0, (const float*)source->data_device,
+  hipLaunchKernelGGL(k_expand_and_add, col_grid(h, w), dim3(256), 0, dn_stream(), (const float*)source->data_device,
                      (const float*)mat->data_device, (const float*)indices->data_device, target->data_device, w, h,
                      mult, w2);
   return dn_launch_status();

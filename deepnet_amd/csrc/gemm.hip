@@ -624,7 +624,7 @@ static void launch_gemm(bool a_kc, bool b_kc, dim3 grid, const float* A, int lda
                         int ldc, int M, int N, int K, int kps, float alpha, float beta, float* partial, bool a_vec,
                         bool b_vec, GemmEpilogue epi) {
 #define GEMM_GO(AK, BK_)                                                                                         \
-  hipLaunchKernelGGL((k_gemm<WM, WN, AK, BK_>), grid, dim3(256), 0, 0, A, lda, B, ldb, C, ldc, M, N, K, kps, alpha, \
+  hipLaunchKernelGGL((k_gemm<WM, WN, AK, BK_>), grid, dim3(256), 0, dn_stream(), A, lda, B, ldb, C, ldc, M, N, K, kps, alpha, \
                      beta, partial, a_vec, b_vec, epi)
   if (a_kc && b_kc) GEMM_GO(true, true);
   else if (a_kc) GEMM_GO(true, false);
@@ -645,7 +645,7 @@ static int gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, co
   if (K <= 0) {
     size_t total = (size_t)M * N;
     unsigned blocks = (unsigned)((total + 255) / 256 < (size_t)cus * 8 ? (total + 255) / 256 : (size_t)cus * 8);
-    hipLaunchKernelGGL(k_scale, dim3(blocks), dim3(256), 0, 0, C, ldc, M, N, beta);
+    hipLaunchKernelGGL(k_scale, dim3(blocks), dim3(256), 0, dn_stream(), C, ldc, M, N, beta);
     return dn_launch_status();
   }
   const bool a_kc = a_trans, b_kc = !b_trans;
@@ -668,10 +668,10 @@ static int gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, co
 #define GEMM_T16(AK, BK_)                                                                                    \
   do {                                                                                                       \
     if (K <= 128)                                                                                            \
-      hipLaunchKernelGGL((k_gemm_tile16<AK, BK_, 4>), grid, dim3(256), 0, 0, A, lda, B, ldb, C, ldc, M, N, K, \
+      hipLaunchKernelGGL((k_gemm_tile16<AK, BK_, 4>), grid, dim3(256), 0, dn_stream(), A, lda, B, ldb, C, ldc, M, N, K, \
                          alpha, beta, epi);                                                                  \
     else                                                                                                     \
-      hipLaunchKernelGGL((k_gemm_tile16<AK, BK_, 8>), grid, dim3(512), 0, 0, A, lda, B, ldb, C, ldc, M, N, K, \
+      hipLaunchKernelGGL((k_gemm_tile16<AK, BK_, 8>), grid, dim3(512), 0, dn_stream(), A, lda, B, ldb, C, ldc, M, N, K, \
                          alpha, beta, epi);                                                                  \
   } while (0)
     if (a_kc && b_kc) GEMM_T16(true, true);
@@ -687,10 +687,10 @@ static int gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, co
 #define GEMM_SMALL(AK, BK_)                                                                                  \
   do {                                                                                                       \
     if (K <= 128)                                                                                            \
-      hipLaunchKernelGGL((k_gemm_small<AK, BK_, 4>), grid, dim3(256), 0, 0, A, lda, B, ldb, C, ldc, M, N, K,  \
+      hipLaunchKernelGGL((k_gemm_small<AK, BK_, 4>), grid, dim3(256), 0, dn_stream(), A, lda, B, ldb, C, ldc, M, N, K,  \
                          alpha, beta, a_vec, b_vec, epi);                                                    \
     else                                                                                                     \
-      hipLaunchKernelGGL((k_gemm_small<AK, BK_, 8>), grid, dim3(512), 0, 0, A, lda, B, ldb, C, ldc, M, N, K,  \
+      hipLaunchKernelGGL((k_gemm_small<AK, BK_, 8>), grid, dim3(512), 0, dn_stream(), A, lda, B, ldb, C, ldc, M, N, K,  \
                          alpha, beta, a_vec, b_vec, epi);                                                    \
   } while (0)
     if (a_kc && b_kc) GEMM_SMALL(true, true);
@@ -740,7 +740,7 @@ static int gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, co
   if (splits > 1) {
     size_t total = (size_t)M * N;
     unsigned blocks = (unsigned)((total + 255) / 256 < (size_t)cus * 8 ? (total + 255) / 256 : (size_t)cus * 8);
-    hipLaunchKernelGGL(k_gemm_splitk_finish, dim3(blocks), dim3(256), 0, 0, partial, splits, C, ldc, M, N, alpha, beta);
+    hipLaunchKernelGGL(k_gemm_splitk_finish, dim3(blocks), dim3(256), 0, dn_stream(), partial, splits, C, ldc, M, N, alpha, beta);
   }
   return dn_launch_status();
 }

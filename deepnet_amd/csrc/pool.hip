@@ -515,7 +515,7 @@ static void norm_lds_launch(int qb, bool same, const float* a0, const float* a1,
   const size_t lds = (size_t)2 * S * S * qb * sizeof(float4);
   const FastDiv dS = make_fastdiv((uint32_t)S);
 #define NORM_LDS_GO(QB, SM, SZ) \
-  hipLaunchKernelGGL((k_norm_lds<QB, UNDO, SM, SZ>), grid, block, lds, 0, a0, a1, a2, win, out0, out1, N, S, dS, nblk, size, addScale, powScale)
+  hipLaunchKernelGGL((k_norm_lds<QB, UNDO, SM, SZ>), grid, block, lds, dn_stream(), a0, a1, a2, win, out0, out1, N, S, dS, nblk, size, addScale, powScale)
 #define NORM_LDS_SZ(QB, SM) do { if (size == 3) NORM_LDS_GO(QB, SM, 3); else if (size == 5) NORM_LDS_GO(QB, SM, 5); \
                                  else if (size == 7) NORM_LDS_GO(QB, SM, 7); else NORM_LDS_GO(QB, SM, 0); } while (0)
 #define NORM_LDS_QB(QB) do { if (same && !UNDO) NORM_LDS_SZ(QB, true); else NORM_LDS_SZ(QB, false); } while (0)
@@ -577,11 +577,11 @@ static void pool_impl(cudamat* images, cudamat* rnd, cudamat* targets, int numFi
   const unsigned grid = grid_for(outs / (v4 ? 4 : 1));
   const float* r = rnd ? rnd->data_device : nullptr;
   if (!rnd) {
-    if (v4) hipLaunchKernelGGL((k_pool<4, 0>), dim3(grid), dim3(256), 0, 0, images->data_device, r, targets->data_device, g);
-    else hipLaunchKernelGGL((k_pool<1, 0>), dim3(grid), dim3(256), 0, 0, images->data_device, r, targets->data_device, g);
+    if (v4) hipLaunchKernelGGL((k_pool<4, 0>), dim3(grid), dim3(256), 0, dn_stream(), images->data_device, r, targets->data_device, g);
+    else hipLaunchKernelGGL((k_pool<1, 0>), dim3(grid), dim3(256), 0, dn_stream(), images->data_device, r, targets->data_device, g);
   } else {
-    if (v4) hipLaunchKernelGGL((k_pool<4, 1>), dim3(grid), dim3(256), 0, 0, images->data_device, r, targets->data_device, g);
-    else hipLaunchKernelGGL((k_pool<1, 1>), dim3(grid), dim3(256), 0, 0, images->data_device, r, targets->data_device, g);
+    if (v4) hipLaunchKernelGGL((k_pool<4, 1>), dim3(grid), dim3(256), 0, dn_stream(), images->data_device, r, targets->data_device, g);
+    else hipLaunchKernelGGL((k_pool<1, 1>), dim3(grid), dim3(256), 0, dn_stream(), images->data_device, r, targets->data_device, g);
   }
   if (dn_launch_status()) conv_set_error(where, hipGetErrorString(hipGetLastError()));
 }
@@ -605,12 +605,12 @@ static void cnorm_impl(cudamat* images, cudamat* meanDiffs, cudamat* denoms, cud
   make_geom(g, N, numFilters, S, S, 0, 0, 1, v4 ? 4 : 1);
   const unsigned grid = grid_for(total / (v4 ? 4 : 1));
 #define CNORM_GO(VW)                                                                                           \
-  hipLaunchKernelGGL((k_cnorm<VW>)    , dim3(grid), dim3(256), 0, 0, (const float*)images->data_device,         \
+  hipLaunchKernelGGL((k_cnorm<VW>)    , dim3(grid), dim3(256), 0, dn_stream(), (const float*)images->data_device,         \
                      (const float*)meanDiffs->data_device, denoms->data_device, targets->data_device, g, sizeX, \
                      addScale, powScale)
 #define CNORM_ROWS(SZ)                                                                                          \
   hipLaunchKernelGGL((k_norm_rows<4, SZ, NORM_SEG, false>), dim3(grid_for((long long)g.NV * S * nseg * numFilters)), \
-                     dim3(256), 0, 0, (const float*)images->data_device, (const float*)nullptr,                  \
+                     dim3(256), 0, dn_stream(), (const float*)images->data_device, (const float*)nullptr,                  \
                      (const float*)nullptr, (const float*)meanDiffs->data_device, denoms->data_device,           \
                      targets->data_device, g, nseg, make_fastdiv((uint32_t)nseg), addScale, powScale)
   const int nseg = (S + NORM_SEG - 1) / NORM_SEG;
@@ -658,11 +658,11 @@ static void rnorm_undo_impl(cudamat* outGrads, cudamat* denoms, cudamat* inputs,
     }
   }
   if (total % 4 == 0 && all_aligned16({acts->data_device, denoms->data_device, outGrads->data_device}))
-    hipLaunchKernelGGL((k_rnorm_undo_prelim<4>), dim3(grid_for(total / 4)), dim3(256), 0, 0, acts->data_device,
+    hipLaunchKernelGGL((k_rnorm_undo_prelim<4>), dim3(grid_for(total / 4)), dim3(256), 0, dn_stream(), acts->data_device,
                        (const float*)denoms->data_device, (const float*)outGrads->data_device, (size_t)(total / 4),
                        -2.f * addScale * powScale);
   else
-    hipLaunchKernelGGL((k_rnorm_undo_prelim<1>), dim3(grid_for(total)), dim3(256), 0, 0, acts->data_device,
+    hipLaunchKernelGGL((k_rnorm_undo_prelim<1>), dim3(grid_for(total)), dim3(256), 0, dn_stream(), acts->data_device,
                        (const float*)denoms->data_device, (const float*)outGrads->data_device, (size_t)total,
                        -2.f * addScale * powScale);
   const bool v4 = N % 4 == 0 && all_aligned16({outGrads->data_device, denoms->data_device, inputs->data_device,
@@ -671,12 +671,12 @@ static void rnorm_undo_impl(cudamat* outGrads, cudamat* denoms, cudamat* inputs,
   make_geom(g, N, numFilters, S, S, 0, 0, 1, v4 ? 4 : 1);
   const unsigned grid = grid_for(total / (v4 ? 4 : 1));
 #define RUNDO_GO(VW)                                                                                          \
-  hipLaunchKernelGGL((k_rnorm_undo<VW>)    , dim3(grid), dim3(256), 0, 0, (const float*)outGrads->data_device, \
+  hipLaunchKernelGGL((k_rnorm_undo<VW>)    , dim3(grid), dim3(256), 0, dn_stream(), (const float*)outGrads->data_device, \
                      (const float*)denoms->data_device, (const float*)inputs->data_device,                     \
                      (const float*)acts->data_device, targets->data_device, g, sizeX, powScale)
 #define RUNDO_ROWS(SZ)                                                                                         \
   hipLaunchKernelGGL((k_norm_rows<4, SZ, NORM_SEG, true>), dim3(grid_for((long long)g.NV * S * nseg * numFilters)), \
-                     dim3(256), 0, 0, (const float*)outGrads->data_device, (const float*)denoms->data_device,   \
+                     dim3(256), 0, dn_stream(), (const float*)outGrads->data_device, (const float*)denoms->data_device,   \
                      (const float*)inputs->data_device, (const float*)acts->data_device, (float*)nullptr,       \
                      targets->data_device, g, nseg, make_fastdiv((uint32_t)nseg), 0.f, powScale)
   const int nseg = (S + NORM_SEG - 1) / NORM_SEG;
@@ -729,16 +729,16 @@ void MaxPoolUndo(cudamat* images, cudamat* maxGrads, cudamat* maxActs, cudamat* 
   make_geom(g, N, F, S, outputsX, subsX, startX, strideX, v4 ? 4 : 1);
   const unsigned grid = grid_for(total / (v4 ? 4 : 1));
   if (v4 && g.subs == 3 && g.stride == 2)
-    hipLaunchKernelGGL((k_pool_undo_fixed<3, 2>), dim3(grid), dim3(256), 0, 0, (const float*)images->data_device,
+    hipLaunchKernelGGL((k_pool_undo_fixed<3, 2>), dim3(grid), dim3(256), 0, dn_stream(), (const float*)images->data_device,
                        (const float*)maxGrads->data_device, (const float*)maxActs->data_device, targets->data_device, g);
   else if (v4 && g.subs == 2 && g.stride == 2)
-    hipLaunchKernelGGL((k_pool_undo_fixed<2, 2>), dim3(grid), dim3(256), 0, 0, (const float*)images->data_device,
+    hipLaunchKernelGGL((k_pool_undo_fixed<2, 2>), dim3(grid), dim3(256), 0, dn_stream(), (const float*)images->data_device,
                        (const float*)maxGrads->data_device, (const float*)maxActs->data_device, targets->data_device, g);
   else if (v4)
-    hipLaunchKernelGGL((k_pool_undo<4>), dim3(grid), dim3(256), 0, 0, (const float*)images->data_device,
+    hipLaunchKernelGGL((k_pool_undo<4>), dim3(grid), dim3(256), 0, dn_stream(), (const float*)images->data_device,
                        (const float*)maxGrads->data_device, (const float*)maxActs->data_device, targets->data_device, g);
   else
-    hipLaunchKernelGGL((k_pool_undo<1>), dim3(grid), dim3(256), 0, 0, (const float*)images->data_device,
+    hipLaunchKernelGGL((k_pool_undo<1>), dim3(grid), dim3(256), 0, dn_stream(), (const float*)images->data_device,
                        (const float*)maxGrads->data_device, (const float*)maxActs->data_device, targets->data_device, g);
   if (dn_launch_status()) conv_set_error(where, hipGetErrorString(hipGetLastError()));
 }

@@ -511,11 +511,11 @@ static bool colblock_launch(const float* M, int ld, int h, int w, const float* x
   const bool stream = (long long)w * h >= DN_STREAM_MIN_ELEMS;
   if (w >= 8 * cus) {
     if (stream)
-      hipLaunchKernelGGL((k_colblock<4, OP, true>), dim3((w + 3) / 4), dim3(256), 0, 0, M, ld, h, w, x, y, alpha, beta);
+      hipLaunchKernelGGL((k_colblock<4, OP, true>), dim3((w + 3) / 4), dim3(256), 0, dn_stream(), M, ld, h, w, x, y, alpha, beta);
     else
-      hipLaunchKernelGGL((k_colblock<4, OP, false>), dim3((w + 3) / 4), dim3(256), 0, 0, M, ld, h, w, x, y, alpha, beta);
+      hipLaunchKernelGGL((k_colblock<4, OP, false>), dim3((w + 3) / 4), dim3(256), 0, dn_stream(), M, ld, h, w, x, y, alpha, beta);
   } else if (w >= 4 * cus) {
-    hipLaunchKernelGGL((k_colblock<2, OP, false>), dim3((w + 1) / 2), dim3(256), 0, 0, M, ld, h, w, x, y, alpha, beta);
+    hipLaunchKernelGGL((k_colblock<2, OP, false>), dim3((w + 1) / 2), dim3(256), 0, dn_stream(), M, ld, h, w, x, y, alpha, beta);
   } else {
     return false;
   }
@@ -781,13 +781,13 @@ static int rows_reduce_one(const float* M, int ld, int h, int w, const float* x,
   dim3 grid(bx, splits);
   const bool stream = (long long)w * h >= DN_STREAM_MIN_ELEMS;
   if (cps <= 64)
-    hipLaunchKernelGGL((k_rows_one<OP, 4, 4, false>), grid, dim3(256), 0, 0, M, ld, h, w, cps, x, y, ws.partial, ws.counters, alpha, beta);
+    hipLaunchKernelGGL((k_rows_one<OP, 4, 4, false>), grid, dim3(256), 0, dn_stream(), M, ld, h, w, cps, x, y, ws.partial, ws.counters, alpha, beta);
   else if ((long long)w * h <= (1 << 18))   // layer states (a few hundred units x a batch): 256 lanes start sooner than 1024
-    hipLaunchKernelGGL((k_rows_one<OP, 4, 8, false>), grid, dim3(256), 0, 0, M, ld, h, w, cps, x, y, ws.partial, ws.counters, alpha, beta);
+    hipLaunchKernelGGL((k_rows_one<OP, 4, 8, false>), grid, dim3(256), 0, dn_stream(), M, ld, h, w, cps, x, y, ws.partial, ws.counters, alpha, beta);
   else if (stream)
-    hipLaunchKernelGGL((k_rows_one<OP, 16, 8, true>), grid, dim3(1024), 0, 0, M, ld, h, w, cps, x, y, ws.partial, ws.counters, alpha, beta);
+    hipLaunchKernelGGL((k_rows_one<OP, 16, 8, true>), grid, dim3(1024), 0, dn_stream(), M, ld, h, w, cps, x, y, ws.partial, ws.counters, alpha, beta);
   else
-    hipLaunchKernelGGL((k_rows_one<OP, 16, 8, false>), grid, dim3(1024), 0, 0, M, ld, h, w, cps, x, y, ws.partial, ws.counters, alpha, beta);
+    hipLaunchKernelGGL((k_rows_one<OP, 16, 8, false>), grid, dim3(1024), 0, dn_stream(), M, ld, h, w, cps, x, y, ws.partial, ws.counters, alpha, beta);
   return dn_launch_status();
 }
 
@@ -804,6 +804,7 @@ static int rows_workspace(int h, int w, RowsWorkspace* ws) {
   const int splits = rows_one_splits(h, w);
   if (splits == 1) return 0;
   if (!counters) {
+    if (dn_capturing()) return CUDA_ERROR;
     if (hipMalloc(&counters, kCounters * sizeof(unsigned)) != hipSuccess) { counters = nullptr; hipGetLastError(); return CUDA_ERROR; }
     if (hipMemset(counters, 0, kCounters * sizeof(unsigned)) != hipSuccess) return CUDA_ERROR;
   }
@@ -842,20 +843,20 @@ static int rows_reduce(const float* M, int ld, int h, int w, const float* x, flo
   if (vec) {
     // 8 wavefronts x 8 columns in flight: a 64-column slice is one trip
     if (cps > 16 && (long long)w * h >= DN_STREAM_MIN_ELEMS)
-      hipLaunchKernelGGL((k_rows_stage1<true, OP, 8, 8, true>), grid, dim3(512), 0, 0, M, ld, h, w, cps, x, y, partial, alpha, beta);
+      hipLaunchKernelGGL((k_rows_stage1<true, OP, 8, 8, true>), grid, dim3(512), 0, dn_stream(), M, ld, h, w, cps, x, y, partial, alpha, beta);
     else if (cps > 16)
-      hipLaunchKernelGGL((k_rows_stage1<true, OP, 8, 8, false>), grid, dim3(512), 0, 0, M, ld, h, w, cps, x, y, partial, alpha, beta);
+      hipLaunchKernelGGL((k_rows_stage1<true, OP, 8, 8, false>), grid, dim3(512), 0, dn_stream(), M, ld, h, w, cps, x, y, partial, alpha, beta);
     else
-      hipLaunchKernelGGL((k_rows_stage1<true, OP, 4, 4, false>), grid, dim3(256), 0, 0, M, ld, h, w, cps, x, y, partial, alpha, beta);
+      hipLaunchKernelGGL((k_rows_stage1<true, OP, 4, 4, false>), grid, dim3(256), 0, dn_stream(), M, ld, h, w, cps, x, y, partial, alpha, beta);
   } else {
-    hipLaunchKernelGGL((k_rows_stage1<false, OP, 4, 4, false>), grid, dim3(256), 0, 0, M, ld, h, w, cps, x, y, partial, alpha, beta);
+    hipLaunchKernelGGL((k_rows_stage1<false, OP, 4, 4, false>), grid, dim3(256), 0, dn_stream(), M, ld, h, w, cps, x, y, partial, alpha, beta);
   }
   if (splits > 1) {
     if (h % 4 == 0)
-      hipLaunchKernelGGL((k_rows_stage2<true, OP>), dim3((h + 255) / 256), dim3(256), 0, 0, (const float*)partial, splits,
+      hipLaunchKernelGGL((k_rows_stage2<true, OP>), dim3((h + 255) / 256), dim3(256), 0, dn_stream(), (const float*)partial, splits,
                          h, y, alpha, beta);
     else
-      hipLaunchKernelGGL((k_rows_stage2<false, OP>), dim3((h + 63) / 64), dim3(256), 0, 0, (const float*)partial, splits,
+      hipLaunchKernelGGL((k_rows_stage2<false, OP>), dim3((h + 63) / 64), dim3(256), 0, dn_stream(), (const float*)partial, splits,
                          h, y, alpha, beta);
   }
   return dn_launch_status();
@@ -886,7 +887,7 @@ int dn_noalloc_setup() {
   if (g_noalloc_ptr[dev]) return 0;
   unsigned char* ptr = nullptr;
   if (hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return CUDA_ERROR;
-  hipLaunchKernelGGL(k_fill_u32, dim3((NOALLOC_COUNTERS + 255) / 256), dim3(256), 0, 0,
+  hipLaunchKernelGGL(k_fill_u32, dim3((NOALLOC_COUNTERS + 255) / 256), dim3(256), 0, dn_stream(),
                      reinterpret_cast<unsigned*>(ptr + (size_t)NOALLOC_PARTIAL_FLOATS * 4), NOALLOC_COUNTERS, 0u);
   if (dn_launch_status()) return CUDA_ERROR;
   g_noalloc_ptr[dev] = ptr;
@@ -899,9 +900,9 @@ int dn_gemv_cols(const float* M, int ld, int h, int w, const float* x, float* y,
   if (colblock_launch<COL_DOT>(M, ld, h, w, x, y, alpha, beta)) return dn_launch_status();
   const int cus = dn_num_cus();
   if (w < cus * 2 && h >= 4096) {
-    hipLaunchKernelGGL((k_gemv_cols<256>), dim3(w), dim3(256), 0, 0, M, ld, h, w, x, y, alpha, beta);
+    hipLaunchKernelGGL((k_gemv_cols<256>), dim3(w), dim3(256), 0, dn_stream(), M, ld, h, w, x, y, alpha, beta);
   } else {
-    hipLaunchKernelGGL((k_gemv_cols<64>), dim3((w + 3) / 4), dim3(256), 0, 0, M, ld, h, w, x, y, alpha, beta);
+    hipLaunchKernelGGL((k_gemv_cols<64>), dim3((w + 3) / 4), dim3(256), 0, dn_stream(), M, ld, h, w, x, y, alpha, beta);
   }
   return dn_launch_status();
 }
@@ -945,6 +946,7 @@ __global__ void __launch_bounds__(256) k_dot_finish(const double* partial, int n
 
 static int flat_dot(const float* a, const float* b, long long n, int take_sqrt, float* result) {
   *result = 0.f;
+  if (dn_capturing()) return ERROR_UNSUPPORTED;        // the result is read back: nothing to record
   if (n <= 0) return 0;
   long long nb = (n + 2047) / 2048;
   const long long cap = (long long)dn_num_cus() * 8;
@@ -953,8 +955,8 @@ static int flat_dot(const float* a, const float* b, long long n, int take_sqrt, 
   if (!ws) return CUDA_ERROR;
   double* partial = (double*)ws;
   float* out = (float*)(ws + (size_t)nb * sizeof(double));
-  hipLaunchKernelGGL(k_dot_partial, dim3((unsigned)nb), dim3(256), 0, 0, a, b, n, partial);
-  hipLaunchKernelGGL(k_dot_finish, dim3(1), dim3(256), 0, 0, partial, (int)nb, out, take_sqrt);
+  hipLaunchKernelGGL(k_dot_partial, dim3((unsigned)nb), dim3(256), 0, dn_stream(), a, b, n, partial);
+  hipLaunchKernelGGL(k_dot_finish, dim3(1), dim3(256), 0, dn_stream(), partial, (int)nb, out, take_sqrt);
   if (hipMemcpy(result, out, sizeof(float), hipMemcpyDeviceToHost) != hipSuccess) return CUDA_ERROR;
   return 0;
 }
@@ -965,9 +967,9 @@ template <class K64, class K256, class... Args>
 static int launch_cols(K64 k64, K256 k256, int w, int h, Args... args) {
   if (w <= 0) return 0;
   if (w < dn_num_cus() * 2 && h >= 4096)
-    hipLaunchKernelGGL(k256, dim3(w), dim3(256), 0, 0, args...);
+    hipLaunchKernelGGL(k256, dim3(w), dim3(256), 0, dn_stream(), args...);
   else
-    hipLaunchKernelGGL(k64, dim3((w + 3) / 4), dim3(256), 0, 0, args...);
+    hipLaunchKernelGGL(k64, dim3((w + 3) / 4), dim3(256), 0, dn_stream(), args...);
   return dn_launch_status();
 }
 
@@ -1018,7 +1020,7 @@ int max_by_axis_noalloc(cudamat* mat, cudamat* target, int axis) {
   if (!rows_one_ok(M, h, h) || rows_one_splits(h, w) == 0) {
     // unaligned operand, or few rows and very many columns: the 64-row kernel over all columns,
     // one launch and no partials
-    hipLaunchKernelGGL((k_rows_stage1<false, ROW_MAX, 4, 4, false>), dim3((h + 63) / 64, 1), dim3(256), 0, 0, M, h, h, w,
+    hipLaunchKernelGGL((k_rows_stage1<false, ROW_MAX, 4, 4, false>), dim3((h + 63) / 64, 1), dim3(256), 0, dn_stream(), M, h, h, w,
                        w, (const float*)nullptr, target->data_device, (float*)nullptr, 1.f, 0.f);
     return dn_launch_status();
   }
@@ -1050,7 +1052,7 @@ int argmax_by_axis(cudamat* mat, cudamat* target, int axis) {
   } else if (axis == 1) {
     if (target->size[0] != h || target->size[1] != 1) return ERROR_INCOMPATIBLE_DIMENSIONS;
     if (h <= 0) return 0;
-    hipLaunchKernelGGL(k_row_reduce, dim3((h + 63) / 64), dim3(256), 0, 0, (const float*)mat->data_device,
+    hipLaunchKernelGGL(k_row_reduce, dim3((h + 63) / 64), dim3(256), 0, dn_stream(), (const float*)mat->data_device,
                        target->data_device, w, h, 1, 0.f, 0.f);
     return dn_launch_status();
   }
@@ -1069,7 +1071,7 @@ int choose_max_by_axis(cudamat* mat, cudamat* target, int axis) {
                        target->data_device, (const float*)nullptr, w, h, 1);
   } else if (axis == 1) {
     if (h <= 0) return 0;
-    hipLaunchKernelGGL(k_row_reduce, dim3((h + 63) / 64), dim3(256), 0, 0, (const float*)mat->data_device,
+    hipLaunchKernelGGL(k_row_reduce, dim3((h + 63) / 64), dim3(256), 0, dn_stream(), (const float*)mat->data_device,
                        target->data_device, w, h, 2, 0.f, 0.f);
     return dn_launch_status();
   }
@@ -1109,7 +1111,7 @@ int normlimit_by_axis(cudamat* mat, cudamat* target, int axis, float norm) {
                        target->data_device, w, h, norm);
   } else if (axis == 1) {
     if (h <= 0) return 0;
-    hipLaunchKernelGGL(k_row_normlimit, dim3((h + 63) / 64), dim3(256), 0, 0, (const float*)mat->data_device,
+    hipLaunchKernelGGL(k_row_normlimit, dim3((h + 63) / 64), dim3(256), 0, dn_stream(), (const float*)mat->data_device,
                        target->data_device, w, h, norm);
     return dn_launch_status();
   }
@@ -1124,20 +1126,20 @@ static int softmax_impl(const float* in, float* out, int w, int h, SoftmaxExtras
     const int n4 = h / 4;
     dim3 grid((w + 3) / 4), block(256);
     const bool stream = (long long)w * h >= DN_STREAM_MIN_ELEMS;
-    if (n4 <= 512) hipLaunchKernelGGL((k_col_softmax_blk<2, 4, false>), grid, block, 0, 0, in, out, w, h, x);
-    else if (n4 <= 768) hipLaunchKernelGGL((k_col_softmax_blk<3, 4, false>), grid, block, 0, 0, in, out, w, h, x);
-    else if (stream) hipLaunchKernelGGL((k_col_softmax_blk<4, 4, true>), grid, block, 0, 0, in, out, w, h, x);
-    else hipLaunchKernelGGL((k_col_softmax_blk<4, 4, false>), grid, block, 0, 0, in, out, w, h, x);
+    if (n4 <= 512) hipLaunchKernelGGL((k_col_softmax_blk<2, 4, false>), grid, block, 0, dn_stream(), in, out, w, h, x);
+    else if (n4 <= 768) hipLaunchKernelGGL((k_col_softmax_blk<3, 4, false>), grid, block, 0, dn_stream(), in, out, w, h, x);
+    else if (stream) hipLaunchKernelGGL((k_col_softmax_blk<4, 4, true>), grid, block, 0, dn_stream(), in, out, w, h, x);
+    else hipLaunchKernelGGL((k_col_softmax_blk<4, 4, false>), grid, block, 0, dn_stream(), in, out, w, h, x);
     return dn_launch_status();
   }
   if (reg_ok) {
     const int n4 = h / 4;
     dim3 grid((w + 3) / 4), block(256);
-    if (n4 <= 64) hipLaunchKernelGGL((k_col_softmax_reg<1>), grid, block, 0, 0, in, out, w, h, x);
-    else if (n4 <= 128) hipLaunchKernelGGL((k_col_softmax_reg<2>), grid, block, 0, 0, in, out, w, h, x);
-    else if (n4 <= 256) hipLaunchKernelGGL((k_col_softmax_reg<4>), grid, block, 0, 0, in, out, w, h, x);
-    else if (n4 <= 512) hipLaunchKernelGGL((k_col_softmax_reg<8>), grid, block, 0, 0, in, out, w, h, x);
-    else hipLaunchKernelGGL((k_col_softmax_reg<16>), grid, block, 0, 0, in, out, w, h, x);
+    if (n4 <= 64) hipLaunchKernelGGL((k_col_softmax_reg<1>), grid, block, 0, dn_stream(), in, out, w, h, x);
+    else if (n4 <= 128) hipLaunchKernelGGL((k_col_softmax_reg<2>), grid, block, 0, dn_stream(), in, out, w, h, x);
+    else if (n4 <= 256) hipLaunchKernelGGL((k_col_softmax_reg<4>), grid, block, 0, dn_stream(), in, out, w, h, x);
+    else if (n4 <= 512) hipLaunchKernelGGL((k_col_softmax_reg<8>), grid, block, 0, dn_stream(), in, out, w, h, x);
+    else hipLaunchKernelGGL((k_col_softmax_reg<16>), grid, block, 0, dn_stream(), in, out, w, h, x);
     return dn_launch_status();
   }
   return launch_cols(k_col_softmax<64>, k_col_softmax<256>, w, h, in, out, w, h, x);
@@ -1181,7 +1183,7 @@ int apply_softmax_grad(cudamat* mat, cudamat* labels, cudamat* target) {
   if (n >= (1ll << 32)) return ERROR_UNSUPPORTED;
   long long blocks = (n + 255) / 256;
   if (blocks > dn_num_cus() * 32ll) blocks = dn_num_cus() * 32ll;
-  hipLaunchKernelGGL(k_softmax_grad, dim3((unsigned)blocks), dim3(256), 0, 0, (const float*)mat->data_device,
+  hipLaunchKernelGGL(k_softmax_grad, dim3((unsigned)blocks), dim3(256), 0, dn_stream(), (const float*)mat->data_device,
                      (const float*)labels->data_device, target->data_device, w, h, make_fastdiv((uint32_t)h));
   return dn_launch_status();
 }
@@ -1201,7 +1203,7 @@ int get_softmax_cross_entropy(cudamat* mat, cudamat* labels, cudamat* target, fl
   if (target->size[0] != 1 || target->size[1] != w) return ERROR_INCOMPATIBLE_DIMENSIONS;
   if (labels->size[0] != 1 || labels->size[1] != w) return ERROR_INCOMPATIBLE_DIMENSIONS;
   if (w <= 0) return 0;
-  hipLaunchKernelGGL(k_softmax_ce, dim3((w + 255) / 256), dim3(256), 0, 0, (const float*)mat->data_device,
+  hipLaunchKernelGGL(k_softmax_ce, dim3((w + 255) / 256), dim3(256), 0, dn_stream(), (const float*)mat->data_device,
                      (const float*)labels->data_device, target->data_device, w, h, tiny);
   return dn_launch_status();
 }

@@ -254,7 +254,7 @@ static int launch_rng(rnd_struct* st, size_t n, Op op) {
   if (n == 0) return 0;
   const size_t draws = (n + NUM_RND_STREAMS - 1) / NUM_RND_STREAMS;
   if (draws < RNG_SPLIT_MIN_DRAWS) {
-    hipLaunchKernelGGL((k_rng_serial<Op>), dim3(RNG_BLOCKS), dim3(RNG_BLOCK), 0, 0, st->dev_mults, st->dev_words, n,
+    hipLaunchKernelGGL((k_rng_serial<Op>), dim3(RNG_BLOCKS), dim3(RNG_BLOCK), 0, dn_stream(), st->dev_mults, st->dev_words, n,
                        op);
     return dn_launch_status();
   }
@@ -265,17 +265,20 @@ static int launch_rng(rnd_struct* st, size_t n, Op op) {
   int top = 0;
   while ((parts - 1) >> top) ++top;
   if (chbits + top > RNG_JUMP_BITS) {
-    hipLaunchKernelGGL((k_rng_serial<Op>), dim3(RNG_BLOCKS), dim3(RNG_BLOCK), 0, 0, st->dev_mults, st->dev_words, n,
+    hipLaunchKernelGGL((k_rng_serial<Op>), dim3(RNG_BLOCKS), dim3(RNG_BLOCK), 0, dn_stream(), st->dev_mults, st->dev_words, n,
                        op);
     return dn_launch_status();
   }
+  // (the split schedule publishes the new state by flipping dev_words on the host, which a
+  // recorded graph would not repeat)
+  if (dn_capturing()) return ERROR_UNSUPPORTED;
   unsigned long long* next = rng_other(st->dev_words);
   const unsigned grid = (unsigned)(parts * (NUM_RND_STREAMS / RNG_SPLIT_BLOCK));
   if (op.src)
-    hipLaunchKernelGGL((k_rng_split<Op, 16>), dim3(grid), dim3(RNG_SPLIT_BLOCK), 0, 0, st->dev_mults,
+    hipLaunchKernelGGL((k_rng_split<Op, 16>), dim3(grid), dim3(RNG_SPLIT_BLOCK), 0, dn_stream(), st->dev_mults,
                        (const unsigned long long*)st->dev_words, next, rng_table(st->dev_words), n, chbits, op);
   else
-    hipLaunchKernelGGL((k_rng_split<Op, 4>), dim3(grid), dim3(RNG_SPLIT_BLOCK), 0, 0, st->dev_mults,
+    hipLaunchKernelGGL((k_rng_split<Op, 4>), dim3(grid), dim3(RNG_SPLIT_BLOCK), 0, dn_stream(), st->dev_mults,
                        (const unsigned long long*)st->dev_words, next, rng_table(st->dev_words), n, chbits, op);
   st->dev_words = next;
   return dn_launch_status();
@@ -307,7 +310,7 @@ int init_random(rnd_struct* rnd_state, int seed, char* cudamatpath) {
   // align the region to 256 KiB inside the (never freed, as in the reference) allocation
   const uintptr_t base = (reinterpret_cast<uintptr_t>(dw) + 2 * RNG_BUF_BYTES - 1) & ~(uintptr_t)(2 * RNG_BUF_BYTES - 1);
   rnd_state->dev_words = reinterpret_cast<unsigned long long*>(base);
-  hipLaunchKernelGGL(k_seed, dim3(RNG_BLOCKS), dim3(RNG_BLOCK), 0, 0, rnd_state->dev_mults, rnd_state->dev_words,
+  hipLaunchKernelGGL(k_seed, dim3(RNG_BLOCKS), dim3(RNG_BLOCK), 0, dn_stream(), rnd_state->dev_mults, rnd_state->dev_words,
                      const_cast<unsigned long long*>(rng_table(rnd_state->dev_words)), (unsigned int)seed);
   return dn_launch_status();
 }
@@ -325,7 +328,7 @@ int fill_with_rand(rnd_struct* rnd_state, cudamat* mat) {
 int fill_with_randn(rnd_struct* rnd_state, cudamat* mat) {
   if (!mat->on_device) return ERROR_NOT_ON_DEVICE;
   if (!rng_ready(rnd_state)) return ERROR_GENERIC;
-  hipLaunchKernelGGL(k_rng_gauss, dim3(RNG_BLOCKS), dim3(RNG_BLOCK), 0, 0, rnd_state->dev_mults, rnd_state->dev_words,
+  hipLaunchKernelGGL(k_rng_gauss, dim3(RNG_BLOCKS), dim3(RNG_BLOCK), 0, dn_stream(), rnd_state->dev_mults, rnd_state->dev_words,
                      (const float*)nullptr, mat->data_device, (size_t)dn_len(mat), 1.f);
   return dn_launch_status();
 }
@@ -350,7 +353,7 @@ int sample_gaussian(rnd_struct* rnd_state, cudamat* mat, cudamat* target, float 
   if (mat->size[0] != target->size[0] || mat->size[1] != target->size[1]) return ERROR_INCOMPATIBLE_DIMENSIONS;
   if (!mat->on_device || !target->on_device) return ERROR_NOT_ON_DEVICE;
   if (!rng_ready(rnd_state)) return ERROR_GENERIC;
-  hipLaunchKernelGGL(k_rng_gauss, dim3(RNG_BLOCKS), dim3(RNG_BLOCK), 0, 0, rnd_state->dev_mults, rnd_state->dev_words,
+  hipLaunchKernelGGL(k_rng_gauss, dim3(RNG_BLOCKS), dim3(RNG_BLOCK), 0, dn_stream(), rnd_state->dev_mults, rnd_state->dev_words,
                      (const float*)mat->data_device, target->data_device, (size_t)dn_len(mat), mult);
   return dn_launch_status();
 }

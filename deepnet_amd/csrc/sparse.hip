@@ -120,12 +120,12 @@ int sparse_dot(cudamat_sparse* mat1, cudamat* mat2, cudamat* target, float beta,
   }
   const unsigned gx = (unsigned)((m + 63) / 64);
   if (n >= 16) {
-    hipLaunchKernelGGL((k_sparse_dot<4>), dim3(gx, (unsigned)((n + 15) / 16)), dim3(256), 0, 0, m, n, k, mat1->nnz,
+    hipLaunchKernelGGL((k_sparse_dot<4>), dim3(gx, (unsigned)((n + 15) / 16)), dim3(256), 0, dn_stream(), m, n, k, mat1->nnz,
                        (const float*)mat1->data_device.data, (const int*)mat1->data_device.indptr,
                        (const int*)mat1->data_device.indices, (const float*)mat2->data_device, target->data_device, beta,
                        alpha);
   } else {
-    hipLaunchKernelGGL((k_sparse_dot<1>), dim3(gx, (unsigned)((n + 3) / 4)), dim3(256), 0, 0, m, n, k, mat1->nnz,
+    hipLaunchKernelGGL((k_sparse_dot<1>), dim3(gx, (unsigned)((n + 3) / 4)), dim3(256), 0, dn_stream(), m, n, k, mat1->nnz,
                        (const float*)mat1->data_device.data, (const int*)mat1->data_device.indptr,
                        (const int*)mat1->data_device.indices, (const float*)mat2->data_device, target->data_device, beta,
                        alpha);

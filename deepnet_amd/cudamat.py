@@ -104,6 +104,8 @@ _SIGNATURES = {
     'dropout': (_i, [_R, _M, _f, _f]),
     'add_col_mult': (_i, [_M, _M, _M, _f]), 'add_row_mult': (_i, [_M, _M, _M, _f]),
     'mult_diagonal_scalar': (_i, [_M, _f, _M]), 'add_diagonal_scalar': (_i, [_M, _f, _M]),
+    'graph_capture_begin': (ct.c_void_p, []), 'graph_capture_end': (ct.c_void_p, []),
+    'graph_launch': (_i, [ct.c_void_p]), 'graph_free': (_i, [ct.c_void_p]), 'graph_set_stream': (_i, [ct.c_void_p, _i]),
     'max_by_axis': (_i, [_M, _M, _i]), 'max_by_axis_noalloc': (_i, [_M, _M, _i]), 'argmax_by_axis': (_i, [_M, _M, _i]),
     'choose_max_by_axis': (_i, [_M, _M, _i]), 'choose_max_and_accumulate': (_i, [_M, _M]),
     'sqsum_by_axis': (_i, [_M, _M, _i, _f, _f]), 'normlimit_by_axis': (_i, [_M, _M, _i, _f]),
@@ -807,6 +809,58 @@ def dot(m1, m2, mult=1.0, target=None):
 
 
 _ACTS = {None: 0, 'none': 0, 'linear': 0, 'sigmoid': 1, 'logistic': 1, 'relu': 2, 'rectified_linear': 2, 'tanh': 3}
+
+
+class Graph(object):
+    """A recorded sequence of library calls (an extension of this backend: a HIP graph).
+
+        step()                                  # once, eagerly: workspaces reach their sizes
+        with cm.Graph() as g:
+            step()                              # recorded, not run
+        for _ in range(n):
+            g.launch()                          # one launch replays the whole sequence
+
+    The calls are recorded with the matrices and scalars they were given; the random generator's
+    state lives on the device, so every replay draws fresh numbers.  Calls that wait for the
+    device (asarray, copy_to_host, vdot, euclid_norm), allocations (empty, CUDAMatrix(...)) and
+    random fills of more than 32 * 12288 elements raise CUDAMatException while recording."""
+
+    def __init__(self):
+        self._exec = None
+        self._others = []
+
+    def __enter__(self):
+        stream = _cudamat.graph_capture_begin()
+        if not stream:
+            raise CUDAMatException("could not start recording a graph")
+        # the conv library, when it is loaded, queues on the same stream
+        import sys
+        conv = sys.modules.get(__package__ + '.cudamat_conv' if __package__ else 'cudamat_conv')
+        if conv is not None:
+            conv._ConvNet.graph_set_stream.argtypes = [ct.c_void_p, ct.c_int]
+            conv._ConvNet.graph_set_stream(stream, 1)
+            self._others.append(conv._ConvNet)
+        return self
+
+    def __exit__(self, exc_type, exc, tb):
+        for lib in self._others:
+            lib.graph_set_stream(None, 0)
+        self._others = []
+        handle = _cudamat.graph_capture_end()
+        if exc_type is None and not handle:
+            raise CUDAMatException("recording the graph failed")
+        self._exec = handle
+        return False
+
+    def launch(self):
+        if not self._exec:
+            raise CUDAMatException("no recorded graph to launch")
+        _check(_cudamat.graph_launch(self._exec))
+
+    def free(self):
+        if self._exec:
+            _cudamat.graph_free(self._exec)
+            self._exec = None
 
 
 def dot_bias_act(m1, m2, bias=None, target=None, act='sigmoid'):

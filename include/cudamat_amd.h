@@ -251,6 +251,21 @@ int apply_softmax_grad(cudamat* mat, cudamat* labels, cudamat* target);
 int get_softmax_correct(cudamat* mat, cudamat* labels, cudamat* target);
 int get_softmax_cross_entropy(cudamat* mat, cudamat* labels, cudamat* target, float tiny);
 
+/* ---- HIP graphs: no counterpart in the reference.  graph_capture_begin() makes the library
+ * record every following call (with the pointers and scalars it is given) into a HIP graph
+ * instead of running it, until graph_capture_end() returns the executable graph;
+ * graph_launch() replays it with one launch on the NULL stream.  For step sequences that are
+ * bound by the cost of launching (the RBM and MLP steps).  Calls that wait for the device,
+ * workspaces that would have to grow and the random generator's split schedule fail with
+ * their error codes while recording; run the sequence once before recording it.
+ * graph_capture_begin returns the capturing stream (NULL on failure); graph_set_stream hands
+ * that stream to a second library of this package (stream NULL, capturing 0 afterwards). ---- */
+void* graph_capture_begin(void);
+void* graph_capture_end(void);
+int graph_launch(void* graph_exec);
+int graph_free(void* graph_exec);
+int graph_set_stream(void* stream, int capturing);
+
 #ifdef __cplusplus
 }
 #endif

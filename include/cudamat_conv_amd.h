@@ -27,6 +27,12 @@ extern "C" {
 /* No counterpart in the reference (it asserts): message of the last failed call, or NULL. */
 const char* conv_last_error(void);
 
+/* No counterpart in the reference: the stream this library queues its kernels on.  The matrix
+ * library's graph_capture_begin() returns the stream it records into; handing it over here
+ * (capturing = 1) makes the conv / pool / norm calls part of the same recording, and
+ * (NULL, 0) returns this library to the NULL stream (include/cudamat_amd.h, "HIP graphs"). */
+int graph_set_stream(void* stream, int capturing);
+
 /* ---- shared-filter convolution: cudamat_conv.cu:1404-1412 (filterActs :15-257, imgActs :265-640,
  * weightActs :642-1015).  paddingStart is <= 0 (the Python wrapper negates it). ---- */
 void convUp(cudamat* images, cudamat* filters, cudamat* targets, int numModulesX, int paddingStart, int moduleStride,

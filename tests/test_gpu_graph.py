@@ -1,0 +1,120 @@
+"""Recorded step sequences (cm.Graph: graph_capture_begin / _end / graph_launch of the C ABI)
+against the same steps run call by call: every replay is compared bit for bit, with eager
+work and synchronisations between the replays."""
+import os
+import sys
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, ROOT)
+import bench          # noqa: E402
+
+pytestmark = pytest.mark.gpu
+
+
+def _bits(m):
+    return m.asarray().view(np.uint32).copy()
+
+
+def _eager_between(cm, rng):
+    """Unrelated work and a synchronisation, as a program would do between two replays."""
+    a = cm.CUDAMatrix(np.asarray(rng.standard_normal((300, 70)), dtype=np.float32, order='F'))
+    b = cm.empty((300, 70))
+    a.apply_sigmoid(target=b)
+    s = b.sum(axis=1)
+    total = float(s.asarray().sum())
+    for m in (a, b, s):
+        m.free_device_memory()
+    return total
+
+
+@pytest.mark.parametrize("kind,fused", [('rbm', False), ('rbm', True), ('mlp', False), ('mlp', True)])
+def test_replays_equal_eager_steps(cm, kind, fused):
+    rng = np.random.default_rng(5)
+    make = (lambda: bench.RBM(cm)) if kind == 'rbm' else (lambda: bench.MLP(cm))
+    params = (lambda o: [o.W, o.bv, o.bh, o.h, o.v2]) if kind == 'rbm' else (lambda o: o.W + o.b + o.dW + [o.loss] + o.mask)
+    # reference: five steps call by call
+    cm.CUDAMatrix.init_random(11)
+    ref = make()
+    want = []
+    for _ in range(5):
+        (ref.step_fused if fused else ref.step)()
+        want.append([_bits(m) for m in params(ref)])
+    # same start: one eager step (workspaces reach their sizes), then the step is recorded once
+    # (recording runs nothing) and replayed four times
+    cm.CUDAMatrix.init_random(11)
+    obj = make()
+    step = obj.step_fused if fused else obj.step
+    step()
+    for got, w in zip([_bits(m) for m in params(obj)], want[0]):
+        assert np.array_equal(got, w)
+    with cm.Graph() as g:
+        step()
+    for got, w in zip([_bits(m) for m in params(obj)], want[0]):
+        assert np.array_equal(got, w)                   # recording changed nothing
+    for i in range(1, 5):
+        g.launch()
+        got = [_bits(m) for m in params(obj)]            # (reading back waits for the replay)
+        for a, w in zip(got, want[i]):
+            assert np.array_equal(a, w), (kind, fused, i)
+        _eager_between(cm, rng)
+    g.free()
+
+
+def test_conv_stage_is_recorded_with_the_matrix_ops(cm, cc):
+    rng = np.random.default_rng(6)
+    N, C, H, F, k, p = 128, 3, 16, 32, 5, 2
+    f = lambda a: cm.CUDAMatrix(np.asarray(a, dtype=np.float32, order='F'))
+    x, w = f(rng.standard_normal((N, C * H * H))), f(0.1 * rng.standard_normal((F, C * k * k)))
+    up, pooled = cm.empty((N, F * H * H)), cm.empty((N, F * 7 * 7))
+    den, normed = cm.empty(pooled.shape), cm.empty(pooled.shape)
+
+    def stage():
+        cc.convUp(x, w, up, H, p, 1, C)
+        up.lower_bound(0)
+        cc.MaxPool(up, pooled, F, 3, 0, 2, 7)
+        cc.ResponseNorm(pooled, den, normed, F, 5, 0.001, 0.75)
+    stage()
+    want = _bits(normed)
+    with cm.Graph() as g:
+        stage()
+    for i in range(3):
+        normed.assign(0)
+        x.mult(1.0)
+        g.launch()
+        assert np.array_equal(_bits(normed), want)
+    # new inputs in the same buffers: the replay works on what the buffers hold now
+    x.assign(f(rng.standard_normal((N, C * H * H))))
+    g.launch()
+    got = _bits(normed)
+    stage()
+    assert np.array_equal(got, _bits(normed)) and not np.array_equal(got, want)
+    g.free()
+
+
+def test_what_cannot_be_recorded_raises(cm):
+    a = cm.CUDAMatrix(np.ones((8, 8), dtype=np.float32))
+    big = cm.empty((1024, 512))                          # 524288 elements: the generator's split schedule
+    with pytest.raises(cm.CUDAMatException):
+        with cm.Graph():
+            a.asarray()
+    with pytest.raises(cm.CUDAMatException):
+        with cm.Graph():
+            cm.empty((4, 4))
+    with pytest.raises(cm.CUDAMatException):
+        with cm.Graph():
+            big.fill_with_rand()
+    with pytest.raises(cm.CUDAMatException):
+        with cm.Graph():
+            a.euclid_norm()
+    # the library is back on the NULL stream and works as before
+    a.add(1.0)
+    assert np.array_equal(a.asarray(), np.full((8, 8), 2.0, dtype=np.float32))
+    with cm.Graph() as g:
+        a.add(1.0)
+    assert np.array_equal(a.asarray(), np.full((8, 8), 2.0, dtype=np.float32))
+    g.launch(); g.launch()
+    assert np.array_equal(a.asarray(), np.full((8, 8), 4.0, dtype=np.float32))
+    g.free()
