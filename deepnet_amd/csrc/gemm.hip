@@ -496,8 +496,8 @@ k_gemm_small(const float* __restrict__ A, int lda, const float* __restrict__ B, 
 }
 
 // The same single-launch scheme on 16 x 16 output blocks (v_mfma_f32_16x16x4_f32), for products
-// whose 32 x 32 blocks would occupy less than half of the CUs (the forward passes of the RBM
-// and MLP configurations: 500 x 100 and 1024 x 128 outputs): four times the workgroups, so
+// whose 32 x 32 blocks would occupy less than two fifths of the CUs (the products of the RBM
+// configuration with 500 x 100 and 784 x 100 outputs): four times the workgroups, so
 // the matrix-core time of a block (K/32 chunks of 8 instructions) spreads over the whole chip.
 // Lane (i, kq) of a wavefront holds, for chunk c, row i of an operand at k = 32c + 8kq + j,
 // j < 8: two 16-byte loads when the operand is K-contiguous, 64-byte runs per 16 lanes when
@@ -662,18 +662,14 @@ static int gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, co
   // (measured: 4096 x 128 x 4096 66 us against 53 us, 2048 x 128 x 2048 17.7 against 21.4).
   const bool heavy = (double)M * (double)N * (double)K >= 1.5e9;
   const long long tiles32 = (long long)((M + 31) / 32) * ((N + 31) / 32);
-  if (tiles64 < cus && off32 && !heavy && tiles32 * 2 <= cus) {
-    // 32 x 32 blocks would leave more than half of the CUs idle: 16 x 16 blocks
+  if (tiles64 < cus && off32 && !heavy && tiles32 * 5 <= cus * 2) {
+    // 32 x 32 blocks would leave most of the CUs idle: 16 x 16 blocks, K over 4 wavefronts (measured
+    // against 32 x 32 blocks and against 8 wavefronts: 500 x 100 x 784 5.4 us / 7.7 / 6.0; with 128
+    // blocks of 32 x 32, 1024 x 128 x 784, the larger blocks win, 7.7 us against 8.8)
     dim3 grid((M + 15) / 16, (N + 15) / 16);
-#define GEMM_T16(AK, BK_)                                                                                    \
-  do {                                                                                                       \
-    if (K <= 128)                                                                                            \
-      hipLaunchKernelGGL((k_gemm_tile16<AK, BK_, 4>), grid, dim3(256), 0, dn_stream(), A, lda, B, ldb, C, ldc, M, N, K, \
-                         alpha, beta, epi);                                                                  \
-    else                                                                                                     \
-      hipLaunchKernelGGL((k_gemm_tile16<AK, BK_, 8>), grid, dim3(512), 0, dn_stream(), A, lda, B, ldb, C, ldc, M, N, K, \
-                         alpha, beta, epi);                                                                  \
-  } while (0)
+#define GEMM_T16(AK, BK_)                                                                                  \
+  hipLaunchKernelGGL((k_gemm_tile16<AK, BK_, 4>), grid, dim3(256), 0, dn_stream(), A, lda, B, ldb, C, ldc, M, N, K, \
+                     alpha, beta, epi)
     if (a_kc && b_kc) GEMM_T16(true, true);
     else if (a_kc) GEMM_T16(true, false);
     else if (b_kc) GEMM_T16(false, true);

@@ -286,3 +286,22 @@ def test_small_products_on_random_shapes(cm, rng, m, k, n, ta, tb, beta):
     assert np.max(np.abs(c.asarray() - want) / bound) < REL
     for h in (a, b, c):
         h.free_device_memory()
+
+
+@pytest.mark.parametrize("m,k,n", [(15, 31, 17), (16, 32, 16), (17, 33, 15), (48, 64, 80), (31, 65, 33), (100, 1029, 20),
+                                   (3, 2000, 5), (250, 96, 250)])
+@pytest.mark.parametrize("ta,tb", [(False, False), (True, False), (False, True), (True, True)])
+def test_small_products_around_the_16_wide_blocks(cm, rng, m, k, n, ta, tb):
+    """Shapes that take the 16 x 16 block kernel: edges at 15 / 16 / 17, a reduction that ends
+    inside, at and just past a 32-deep chunk, long reductions over few outputs; with alpha and
+    a beta that reads the target."""
+    A, B, C = _rand(rng, (m, k)), _rand(rng, (k, n)), _rand(rng, (m, n))
+    a = cm.CUDAMatrix(np.asfortranarray(A.T)) if ta else cm.CUDAMatrix(A)
+    b = cm.CUDAMatrix(np.asfortranarray(B.T)) if tb else cm.CUDAMatrix(B)
+    c = cm.CUDAMatrix(C)
+    cm._check(cm._cudamat.dot((a.T if ta else a).p_mat, (b.T if tb else b).p_mat, c.p_mat, -0.5, 2.0))
+    want = 2.0 * (A.astype(np.float64) @ B.astype(np.float64)) - 0.5 * C
+    bound = 2.0 * (np.abs(A).astype(np.float64) @ np.abs(B)) + 0.5 * np.abs(C) + 1e-30
+    assert np.max(np.abs(c.asarray() - want) / bound) < REL
+    for h in (a, b, c):
+        h.free_device_memory()
