@@ -1028,6 +1028,43 @@ __global__ void __launch_bounds__(256) k_conv_outp_finish(ConvArgs p) {
   }
 }
 
+// The same sum for many partial blocks (the small-output kernel leaves one per workgroup, up to
+// 256): 64 neighbouring outputs per workgroup, one per lane, so that a wavefront reads whole
+// 256-byte runs; the 16 wavefronts take every 16th block with all their loads in flight and
+// meet in LDS.  Fixed order of additions.
+__global__ void __launch_bounds__(1024) k_conv_outp_finish_wide(ConvArgs p) {
+  __shared__ float sv[16][64];
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int per_group = p.Fg * p.Cg * p.kk2;
+  const int total = p.G * per_group;
+  const int e = blockIdx.x * 64 + lane;
+  const float* part = p.partial + (size_t)blockIdx.y * p.splits * total;
+  float acc = 0.f;
+  if (e < total) {
+    for (int z0 = wv; z0 < p.splits; z0 += 16 * 16) {
+      float v[16];
+#pragma unroll
+      for (int u = 0; u < 16; ++u) {
+        const int z = z0 + 16 * u;
+        v[u] = z < p.splits ? part[(size_t)z * total + e] : 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < 16; ++u) acc += v[u];
+    }
+  }
+  sv[wv][lane] = acc;
+  __syncthreads();
+  if (wv == 0 && e < total) {
+    float sum = sv[0][lane];
+#pragma unroll
+    for (int w = 1; w < 16; ++w) sum += sv[w][lane];
+    const int g = e / per_group, rem = e - g * per_group;
+    const int q = rem / p.Fg, fl = rem - q * p.Fg;
+    float* t = p.out + (size_t)blockIdx.y * total + (size_t)p.F * q + g * p.Fg + fl;
+    *t = (p.scale_t == 0.f ? 0.f : p.scale_t * *t) + p.scale_o * sum;
+  }
+}
+
 // ------------------------------------------------------------------ convDown through a patch matrix
 // With few colours per group the implicit GEMM above has only Cg useful columns
 // in a 32-wide matrix-core block and re-reads the hidden activations once per
@@ -1807,7 +1844,8 @@ static void conv_outp_impl(cudamat* images, cudamat* hidActs, cudamat* targets, 
       else { if (ct == 1) OUTP_SMALL(2, 1); else if (ct == 2) OUTP_SMALL(2, 2); else OUTP_SMALL(2, 3); }
 #undef OUTP_SMALL
       const int total = F * cols;
-      hipLaunchKernelGGL(k_conv_outp_finish, dim3((total + 15) / 16), dim3(256), 0, dn_stream(), a);
+      if (a.splits >= 64) hipLaunchKernelGGL(k_conv_outp_finish_wide, dim3((total + 63) / 64), dim3(1024), 0, dn_stream(), a);
+      else hipLaunchKernelGGL(k_conv_outp_finish, dim3((total + 15) / 16), dim3(256), 0, dn_stream(), a);
     } else if (fast) {
       // rows = filters of a group: pick the tile height that wastes least.
       const int Fg = a.Fg;
