@@ -468,6 +468,8 @@ def main():
     ap.add_argument('--probe', action='store_true',
                     help='run only the roofline kernel (add_mult) and a copy-shaped calibration kernel '
                          '(mult by a scalar into a second matrix), for rocprofv3 --pmc runs')
+    ap.add_argument('--no-graph', action='store_true',
+                    help='skip the recorded-graph timings (rocprofv3 --kernel-trace crashes inside hipGraphLaunch)')
     ap.add_argument('--probe-c2', action='store_true',
                     help='launch every op of the 4096^2 list three times over the 8 operand sets, plus the copy-shaped '
                          'calibration kernel, and nothing else (for rocprofv3 --pmc runs)')
@@ -565,6 +567,8 @@ def main():
         def recorded(step, iters, warm):
             # the step recorded once as a HIP graph (cm.Graph, an extension of this backend) and
             # replayed with one launch per step: same kernels, same results
+            if args.no_graph:
+                return None
             with cm.Graph() as g:
                 step()
             tt = time_loop(cm, g.launch, iters, warm)
