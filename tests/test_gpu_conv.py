@@ -67,7 +67,13 @@ def _f(a):
 
 
 def _relerr(got, want, bound):
-    return np.max(np.abs(np.asarray(got, np.float64) - want) / (bound + 1e-30))
+    """The larger of two measures: every element against the bound |x| * |w| of its own sum
+    (robust to cancellation), and the whole result against its own size (Frobenius norms, ten
+    times stricter: REL / 10 = 1e-5 relative to the result itself)."""
+    got = np.asarray(got, np.float64)
+    elementwise = np.max(np.abs(got - want) / (bound + 1e-30))
+    whole = np.linalg.norm(got - want) / (np.linalg.norm(want) + 1e-30)
+    return max(elementwise, 10.0 * whole)
 
 
 @pytest.mark.parametrize("N,C,H,F,k,s,p,G", CASES)

@@ -15,9 +15,14 @@ def _rand(rng, shape):
 
 
 def _relerr(got, want, A, B):
-    """Error relative to |A|.|B| elementwise bound (robust to cancellation)."""
+    """The larger of two measures: every element against the bound |A|.|B| of its own sum (robust
+    to cancellation), and the whole product against its own size (Frobenius norms, ten times
+    stricter: 1e-5 relative to the result itself)."""
     bound = np.abs(A).astype(np.float64) @ np.abs(B).astype(np.float64)
-    return np.max(np.abs(np.asarray(got, np.float64) - want) / (bound + 1e-30))
+    got = np.asarray(got, np.float64)
+    elementwise = np.max(np.abs(got - want) / (bound + 1e-30))
+    whole = np.linalg.norm(got - want) / (np.linalg.norm(want) + 1e-30)
+    return max(elementwise, 10.0 * whole)
 
 
 # (m, k, n): test_cudamat.py:796-880 uses 128x256x64-like shapes, eigenmat/test.py:23-47
