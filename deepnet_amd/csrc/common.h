@@ -12,6 +12,9 @@ int dn_num_cus();
 // Grow-only device workspaces (slot 0: partials and scalar results; slot 1: conv patch matrix).
 void* dn_scratch(size_t bytes, int slot = 0);
 
+// n 32-bit words that are zero between kernels (arrival counters); null when they cannot be had.
+unsigned* dn_zero_words(int n);
+
 // Looks up (once per device) the fixed workspace of the entry points that allocate nothing.
 int dn_noalloc_setup();
 

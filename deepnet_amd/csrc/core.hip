@@ -56,6 +56,23 @@ void* dn_scratch(size_t bytes, int slot) {
   return g_scratch[slot];
 }
 
+// A block of 32-bit words that is zero whenever no kernel of the library is running (arrival
+// counters that their kernels return to zero); allocated and cleared on first use.
+static unsigned* g_zero_words = nullptr;
+static int g_zero_words_n = 0;
+
+unsigned* dn_zero_words(int n) {
+  if (n > g_zero_words_n) {
+    if (g_capturing) return nullptr;
+    if (g_zero_words) { hipDeviceSynchronize(); hipFree(g_zero_words); g_zero_words = nullptr; g_zero_words_n = 0; }
+    const int want = n < 16384 ? 16384 : n;
+    if (hipMalloc(&g_zero_words, (size_t)want * sizeof(unsigned)) != hipSuccess) { g_zero_words = nullptr; hipGetLastError(); return nullptr; }
+    if (hipMemset(g_zero_words, 0, (size_t)want * sizeof(unsigned)) != hipSuccess) return nullptr;
+    g_zero_words_n = want;
+  }
+  return g_zero_words;
+}
+
 // ------------------------------------------------------------------ kernels
 
 // Column-major row-band copy: dst(r, c) = src(r + row0, c) for a band of `rows`
@@ -143,8 +160,24 @@ int cublas_shutdown(void) {
 }
 
 int cuda_set_device(int deviceId) {
+  int before = -1;
+  hipGetDevice(&before);
   if (hipSetDevice(deviceId) != hipSuccess) return CUDA_ERROR;
   g_num_cus = 0;
+  if (before != deviceId && before >= 0) {
+    // the workspaces live in the memory of the device that was current when they were made
+    hipSetDevice(before);
+    hipDeviceSynchronize();
+    for (int slot = 0; slot < 4; ++slot) {
+      if (g_scratch[slot]) hipFree(g_scratch[slot]);
+      g_scratch[slot] = nullptr;
+      g_scratch_bytes[slot] = 0;
+    }
+    if (g_zero_words) hipFree(g_zero_words);
+    g_zero_words = nullptr;
+    g_zero_words_n = 0;
+    hipSetDevice(deviceId);
+  }
   return 0;
 }
 

@@ -795,19 +795,15 @@ static inline bool rows_one_ok(const float* M, int ld, int h) {
   return dn_aligned16(M) && (ld % 4 == 0) && (h % 4 == 0);
 }
 
-// The library's own workspace: counters for 16384 row blocks (zeroed once; matrices with
-// more rows than that have no column slices), partials from the grow-only scratch.
+// The library's own workspace: arrival counters for 16384 row blocks (matrices with more rows
+// than that have no column slices), partials from the grow-only scratch.
 static int rows_workspace(int h, int w, RowsWorkspace* ws) {
-  static unsigned* counters = nullptr;
   const int kCounters = 16384;
   ws->partial = nullptr; ws->partial_floats = 0; ws->counters = nullptr; ws->num_counters = 0;
   const int splits = rows_one_splits(h, w);
   if (splits == 1) return 0;
-  if (!counters) {
-    if (dn_capturing()) return CUDA_ERROR;
-    if (hipMalloc(&counters, kCounters * sizeof(unsigned)) != hipSuccess) { counters = nullptr; hipGetLastError(); return CUDA_ERROR; }
-    if (hipMemset(counters, 0, kCounters * sizeof(unsigned)) != hipSuccess) return CUDA_ERROR;
-  }
+  unsigned* counters = dn_zero_words(kCounters);
+  if (!counters) return CUDA_ERROR;
   ws->partial = (float*)dn_scratch((size_t)splits * h * sizeof(float));
   if (!ws->partial) return CUDA_ERROR;
   ws->partial_floats = (size_t)splits * h;

@@ -195,7 +195,8 @@ def test_prob_max_pool_follows_the_reference_scan(cm, cc, rng):
                                       # the image block; maps of 32 and 48 pixels a side (smaller image
                                       # blocks, and past what fits in LDS)
                                       (16, 4, 12, 6), (32, 2, 10, 8), (100, 8, 15, 5), (44, 3, 13, 7),
-                                      (16, 4, 32, 5), (8, 2, 48, 3), (16, 2, 22, 6), (4, 2, 45, 5)])
+                                      (16, 4, 32, 5), (8, 2, 48, 3), (16, 2, 22, 6), (4, 2, 45, 5),
+                                      (32, 2, 16, 5), (64, 3, 16, 7)])      # 16 x 16 maps of 32 images: LDS tiles of exactly 64 KiB
 def test_response_norm_and_undo(cm, cc, rng, N, F, S, size):
     a, p = 0.001, 0.75
     x = _f(rng.standard_normal((N, F * S * S)) * 3)
