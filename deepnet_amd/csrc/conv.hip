@@ -1822,7 +1822,7 @@ static void conv_outp_impl(cudamat* images, cudamat* hidActs, cudamat* targets, 
   const bool fast = fast_ok(a);
   // Several chunks (partial sums over groups of modules; one module each for a locally connected
   // layer): all of them in one launch of the general kernel, the chunk along grid z
-  const bool batched = fast && chunks > 1;
+  const bool batched = fast && chunks > 1 && (long long)chunks * numGroups <= 32767;   // (grid z: chunks x groups x splits)
   for (int ch = 0; ch < (batched ? 1 : chunks); ++ch) {
     a.m_begin = ch * partialSum; a.m_count = partialSum;
     a.chunks = batched ? chunks : 1;
