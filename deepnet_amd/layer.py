@@ -338,6 +338,18 @@ class SoftmaxLayer(Layer):
         return perf
 
 
+class SmoothReluLayer(ReluLayer):
+    """deepnet/smooth_relu_layer.py: softplus units log(1 + exp(x)).  The derivative is taken from the
+    output s as 1 - exp(-s), which equals sigmoid(x)."""
+    activation = P.RECTIFIED_LINEAR_SMOOTH
+
+    def ApplyActivation(self):
+        cm.log_1_plus_exp(self.state)
+
+    def ComputeDeriv(self):
+        self.deriv.apply_rectified_linear_smooth_deriv(self.state)
+
+
 class SinLayer(Layer):
     """deepnet/sin_layer.py: hidden units sin(x); the input is kept for the derivative."""
     activation = P.SIN
@@ -367,7 +379,7 @@ class CosLayer(SinLayer):
 
 
 LAYER_TYPES = {cls.activation: cls for cls in (LinearLayer, LogisticLayer, TanhLayer, ReluLayer, SoftmaxLayer, SinLayer,
-                                               CosLayer)}
+                                               CosLayer, SmoothReluLayer)}
 
 
 def CreateLayer(activation, *args, **kwargs):

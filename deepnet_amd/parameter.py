@@ -16,6 +16,7 @@ from .choose_matrix_library import cm
 NONE, INVERSE_T, EXPONENTIAL = 'NONE', 'INVERSE_T', 'EXPONENTIAL'
 LINEAR, LOGISTIC, TANH, RECTIFIED_LINEAR, SOFTMAX = 'LINEAR', 'LOGISTIC', 'TANH', 'RECTIFIED_LINEAR', 'SOFTMAX'
 SIN, COS = 'SIN', 'COS'
+RECTIFIED_LINEAR_SMOOTH = 'RECTIFIED_LINEAR_SMOOTH'
 SQUARED_LOSS, CROSS_ENTROPY = 'SQUARED_LOSS', 'CROSS_ENTROPY'
 
 

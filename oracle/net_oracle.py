@@ -89,6 +89,8 @@ def activate(act, x):
         return np.tanh(x)
     if act == 'RECTIFIED_LINEAR':
         return np.maximum(x, 0.0)
+    if act == 'RECTIFIED_LINEAR_SMOOTH':           # smooth_relu_layer.py:11-16
+        return cmo.apply_log_1_plus_exp(x)
     if act == 'SOFTMAX':
         e = np.exp(x - x.max(axis=0, keepdims=True))
         return e / e.sum(axis=0, keepdims=True)
@@ -167,6 +169,8 @@ class Net(object):
             return d * s * (1.0 - s)
         if act == 'RECTIFIED_LINEAR':
             return d * (s > 0)
+        if act == 'RECTIFIED_LINEAR_SMOOTH':        # smooth_relu_layer.py:18-20: from the output, not masked
+            return cmo.apply_rectified_linear_smooth_deriv(d, s)
         if act == 'SIN':                            # sin_layer.py:15-17, cos_layer.py:15-17: from the kept input
             return d * np.cos(self.pre[i])
         if act == 'COS':

@@ -191,6 +191,21 @@ def test_example_convnet_of_the_reference_at_its_batch_size(cm, dn):
     _train_and_compare(cm, net, onet, batches, rtol=2e-4, atol=2e-6)
 
 
+def test_smooth_relu_hidden_units(cm, dn):
+    """deepnet/smooth_relu_layer.py: softplus units whose derivative is taken from the output."""
+    rng = np.random.default_rng(15)
+    sizes, B = (24, 40, 6), 16
+    sgd = dict(base_epsilon=0.05, initial_momentum=0.5, final_momentum=0.5)
+    w = [_f(0.3 * rng.standard_normal((sizes[i], sizes[i + 1]))) for i in range(2)]
+    spec = [(dn.P.LINEAR, 24, sgd, None),
+            (dn.P.RECTIFIED_LINEAR_SMOOTH, 40, sgd, {'w': w[0], 'hyper': sgd}),
+            (dn.P.SOFTMAX, 6, sgd, {'w': w[1], 'hyper': sgd})]
+    net, onet = _build_chain(dn, spec, B, rng)
+    assert type(net.layer[1]).__name__ == 'SmoothReluLayer'
+    batches = [(3.0 * rng.standard_normal((24, B)), rng.integers(0, 6, (1, B)).astype(np.float64)) for _ in range(3)]
+    _train_and_compare(cm, net, onet, batches)
+
+
 def test_sin_and_cos_hidden_units(cm, dn):
     """deepnet/sin_layer.py, cos_layer.py: the pre-activation is kept and the derivative taken from it."""
     rng = np.random.default_rng(14)

@@ -27,11 +27,13 @@ def _half_slope_tanh(x):
 
 def _torch_act(act, x):
     return {'LOGISTIC': torch.sigmoid, 'TANH': _half_slope_tanh, 'RECTIFIED_LINEAR': torch.relu,
-            'LINEAR': lambda t: t, 'SIN': torch.sin, 'COS': torch.cos}[act](x)
+            'LINEAR': lambda t: t, 'SIN': torch.sin, 'COS': torch.cos,
+            'RECTIFIED_LINEAR_SMOOTH': torch.nn.functional.softplus}[act](x)
 
 
 @pytest.mark.parametrize("hidden,loss", [('RECTIFIED_LINEAR', 'softmax'), ('LOGISTIC', 'softmax'), ('TANH', 'logistic_ce'),
-                                         ('RECTIFIED_LINEAR', 'linear_sq'), ('SIN', 'softmax'), ('COS', 'linear_sq')])
+                                         ('RECTIFIED_LINEAR', 'linear_sq'), ('SIN', 'softmax'), ('COS', 'linear_sq'),
+                                         ('RECTIFIED_LINEAR_SMOOTH', 'softmax')])
 def test_dense_net_steps_equal_torch_sgd(rng, hidden, loss):
     sizes, B, steps = (12, 9, 7, 5), 6, 4
     mom, eps, l2 = 0.9, 0.05, 0.01
@@ -40,7 +42,7 @@ def test_dense_net_steps_equal_torch_sgd(rng, hidden, loss):
     he = no.Hyper(base_epsilon=eps, initial_momentum=mom, final_momentum=mom, apply_l2_decay=True, l2_decay=l2)
     hl = no.Hyper(base_epsilon=eps, initial_momentum=mom, final_momentum=mom)
     hd = no.Hyper(base_epsilon=eps, initial_momentum=mom, final_momentum=mom, dropout=True, dropout_prob=0.5)
-    if hidden in ('SIN', 'COS'):
+    if hidden in ('SIN', 'COS', 'RECTIFIED_LINEAR_SMOOTH'):
         hd = hl     # (sin_layer.py:15-17 does not mask its derivative, so with dropout it is not the gradient of anything)
     out_act = {'softmax': 'SOFTMAX', 'logistic_ce': 'LOGISTIC', 'linear_sq': 'LINEAR'}[loss]
     Ws = [0.3 * rng.standard_normal((sizes[i], sizes[i + 1])) for i in range(3)]
