@@ -7,6 +7,7 @@
 // (column views) are peeled to alignment when they share the same offset and
 // fall back to 4-byte accesses otherwise.
 #include "common.h"
+#include "rng.h"
 #include "wide_math.h"
 #include <math.h>
 
@@ -467,7 +468,53 @@ int add_diagonal(cudamat* mat, cudamat* vec, cudamat* target) {
 }  // extern "C"
 
 int dn_gemm_fused(bool a_trans, bool b_trans, int M, int N, int K, const float* A, int lda, const float* B, int ldb,
-                  float* C, int ldc, const float* bias, int act, bool* fused);
+                  float* C, int ldc, const float* bias, int act, bool* fused, const DnGemmSample* smp, bool* sampled);
+
+// target = act(op(mat1) * op(mat2) + bias) and, with a generator and a sample matrix,
+// sample = (uniform < target), in as few launches as the shapes allow.
+static int dot_bias_act_impl(rnd_struct* rnd, cudamat* mat1, cudamat* mat2, cudamat* bias, cudamat* target,
+                             cudamat* sample, int act) {
+  if (!mat1->on_device || !mat2->on_device || !target->on_device || (bias && !bias->on_device)) return ERROR_NOT_ON_DEVICE;
+  if (target->is_trans || (bias && bias->is_trans)) return ERROR_TRANSPOSED;
+  if (act < 0 || act > 3) return ERROR_UNSUPPORTED;
+  if (get_leading_dimension(mat1) != target->size[0] || get_nonleading_dimension(mat2) != target->size[1] ||
+      get_nonleading_dimension(mat1) != get_leading_dimension(mat2))
+    return ERROR_INCOMPATIBLE_DIMENSIONS;
+  if (bias && (bias->size[0] != target->size[0] || bias->size[1] != 1)) return ERROR_INCOMPATIBLE_DIMENSIONS;
+  if (sample) {
+    if (!rnd || !rnd->dev_mults || !rnd->dev_words) return ERROR_GENERIC;
+    if (!sample->on_device) return ERROR_NOT_ON_DEVICE;
+    if (sample->is_trans) return ERROR_TRANSPOSED;
+    if (sample->size[0] != target->size[0] || sample->size[1] != target->size[1]) return ERROR_INCOMPATIBLE_DIMENSIONS;
+    if (sample->data_device == target->data_device) return ERROR_UNSUPPORTED;     // both are written
+  }
+  const int m = target->size[0], n = target->size[1], k = get_leading_dimension(mat2);
+  if (m <= 0 || n <= 0) return 0;
+  bool fused = false, sampled = false;
+  int err;
+  if (n == 1 || k <= 0) {
+    err = dot(mat1, mat2, target, 0.f, 1.f);                 // vector-shaped: the streaming kernels
+  } else {
+    // (a recorded graph could not repeat the host's switch to the generator's other word buffer)
+    DnGemmSample smp = {nullptr, nullptr, nullptr, nullptr};
+    const bool try_sample = sample && !dn_capturing();
+    if (try_sample) smp = DnGemmSample{sample->data_device, rnd->dev_mults, rnd->dev_words, rng_other(rnd->dev_words)};
+    err = dn_gemm_fused(mat1->is_trans != 0, mat2->is_trans != 0, m, n, k, mat1->data_device, mat1->size[0],
+                        mat2->data_device, mat2->size[0], target->data_device, m, bias ? bias->data_device : nullptr,
+                        act, &fused, try_sample ? &smp : nullptr, &sampled);
+    if (!err && sampled) rnd->dev_words = rng_other(rnd->dev_words);
+  }
+  if (err) return err;
+  if (!fused) {
+    if (bias && (err = add_col_vec(target, bias, target))) return err;
+    if (act == 1) err = apply_sigmoid(target, target);
+    else if (act == 2) err = lower_bound_scalar(target, 0.f, target);
+    else if (act == 3) err = apply_tanh(target, target);
+    if (err) return err;
+  }
+  if (sample && !sampled) return sample_bernoulli(rnd, target, sample);
+  return 0;
+}
 
 extern "C" {
 
@@ -477,32 +524,19 @@ extern "C" {
 // launch where the product runs as a single kernel, bit-identical to the three calls.
 // bias: rows(target) x 1 or null.  act: 0 none, 1 sigmoid, 2 max(x, 0), 3 tanh.
 int dot_bias_act(cudamat* mat1, cudamat* mat2, cudamat* bias, cudamat* target, int act) {
-  if (!mat1->on_device || !mat2->on_device || !target->on_device || (bias && !bias->on_device)) return ERROR_NOT_ON_DEVICE;
-  if (target->is_trans || (bias && bias->is_trans)) return ERROR_TRANSPOSED;
-  if (act < 0 || act > 3) return ERROR_UNSUPPORTED;
-  if (get_leading_dimension(mat1) != target->size[0] || get_nonleading_dimension(mat2) != target->size[1] ||
-      get_nonleading_dimension(mat1) != get_leading_dimension(mat2))
-    return ERROR_INCOMPATIBLE_DIMENSIONS;
-  if (bias && (bias->size[0] != target->size[0] || bias->size[1] != 1)) return ERROR_INCOMPATIBLE_DIMENSIONS;
-  const int m = target->size[0], n = target->size[1], k = get_leading_dimension(mat2);
-  if (m <= 0 || n <= 0) return 0;
-  bool fused = false;
-  int err;
-  if (n == 1 || k <= 0) {
-    err = dot(mat1, mat2, target, 0.f, 1.f);                 // vector-shaped: the streaming kernels
-  } else {
-    err = dn_gemm_fused(mat1->is_trans != 0, mat2->is_trans != 0, m, n, k, mat1->data_device, mat1->size[0],
-                        mat2->data_device, mat2->size[0], target->data_device, m, bias ? bias->data_device : nullptr,
-                        act, &fused);
-  }
-  if (err || fused) return err;
-  if (bias && (err = add_col_vec(target, bias, target))) return err;
-  if (act == 1) return apply_sigmoid(target, target);
-  if (act == 2) return lower_bound_scalar(target, 0.f, target);
-  if (act == 3) return apply_tanh(target, target);
-  return 0;
+  return dot_bias_act_impl(nullptr, mat1, mat2, bias, target, nullptr, act);
 }
 
+// Extension: dot_bias_act followed by sample_bernoulli(rnd_state, target, sample), the
+// up-pass of an RBM with its hidden sample (deepnet/dbm.py:95-105), bit-identical to the two
+// calls (same states, same samples, same generator state afterwards).  One launch where the
+// product runs as a single kernel over at most 16 * 12288 outputs and no graph is being
+// recorded; otherwise the separate kernels.
+int dot_bias_act_sample(rnd_struct* rnd_state, cudamat* mat1, cudamat* mat2, cudamat* bias, cudamat* target,
+                        cudamat* sample, int act) {
+  if (!sample) return ERROR_GENERIC;
+  return dot_bias_act_impl(rnd_state, mat1, mat2, bias, target, sample, act);
+}
 
 }  // extern "C"
 

@@ -9,6 +9,7 @@
 // products (a single row or column on either side, which is how sum(axis) and
 // add_sums arrive) go to the streaming matrix-vector kernels instead.
 #include "common.h"
+#include "rng.h"
 #include "wide_math.h"
 
 int dn_gemv_cols(const float* M, int ld, int h, int w, const float* x, float* y, float alpha, float beta);
@@ -21,16 +22,52 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 // the separate calls it replaces (add_col_vec, then the activation), so that the fused
 // result is bit-identical to theirs: bias is a column vector over the rows of C or null.
 enum { GEMM_ACT_NONE = 0, GEMM_ACT_SIGMOID = 1, GEMM_ACT_RELU = 2, GEMM_ACT_TANH = 3 };
+// sample != null (dot_bias_act_sample): the kernels that finish every output in one launch also
+// draw sample(i) = uniform_i < C(i) for element i = n * ldc + m of a C without gaps (ldc = M),
+// with the uniform that sample_bernoulli would use: draw number i / 12288 of stream i % 12288,
+// counted from the words the call starts with.  Those words are only read; the lane that makes
+// a stream's last draw writes the stream's new word to `next`, and the host makes `next` the
+// generator's current buffer afterwards.
 struct GemmEpilogue {
   const float* bias;
   int act;
+  float* sample;
+  const unsigned int* mults;
+  const unsigned long long* words;
+  unsigned long long* next;
+  unsigned int total;            // M * N
 };
+#define GEMM_SAMPLE_MAX_DRAWS 16
 __device__ __forceinline__ float gemm_finish(float v, int m, const GemmEpilogue& e) {
   if (e.bias) v = v + e.bias[m];
   if (e.act == GEMM_ACT_SIGMOID) v = dn_sigmoid(v);
   else if (e.act == GEMM_ACT_RELU) v = v < 0.f ? 0.f : v;
   else if (e.act == GEMM_ACT_TANH) v = dn_tanh(v);
   return v;
+}
+// The generator's word and multiplier for element i, fetched early so that the loads are over
+// when the product is.
+struct GemmDraw { unsigned long long w; unsigned int mult; };
+__device__ __forceinline__ GemmDraw gemm_draw_fetch(unsigned int i, bool ok, const GemmEpilogue& e) {
+  GemmDraw d = {0ull, 0u};
+  if (e.sample && ok) {
+    const unsigned int s = i % NUM_RND_STREAMS;
+    d.w = e.words[s];
+    d.mult = e.mults[s];
+  }
+  return d;
+}
+__device__ __forceinline__ void gemm_draw_store(GemmDraw d, unsigned int i, float p, const GemmEpilogue& e) {
+  const unsigned int s = i % NUM_RND_STREAMS, nd = i / NUM_RND_STREAMS;
+  unsigned long long w = d.w;
+  for (unsigned int k = 0; k <= nd; ++k) w = mwc_step(w, d.mult);
+  e.sample[i] = mwc_uniform(w) < p ? 1.f : 0.f;
+  if (i + NUM_RND_STREAMS >= e.total) e.next[s] = w;
+}
+// Streams without a draw (fewer outputs than streams) keep their word: one workgroup copies them.
+__device__ __forceinline__ void gemm_draw_idle_streams(int tid, int nthreads, const GemmEpilogue& e) {
+  if (e.sample && blockIdx.x == 0 && blockIdx.y == 0)
+    for (unsigned int s = e.total + tid; s < NUM_RND_STREAMS; s += nthreads) e.next[s] = e.words[s];
 }
 
 struct __attribute__((packed, aligned(4))) gemm_f4u { float x, y, z, w; };   // four floats at any 4-byte boundary
@@ -490,9 +527,16 @@ k_gemm_small(const float* __restrict__ A, int lda, const float* __restrict__ B, 
     const int v = e >> 6;
     const float sum = (red[0][e] + red[1][e]) + (red[2][e] + red[3][e]);
     const int nn = blockIdx.y * 32 + 8 * (v >> 2) + 4 * lk + (v & 3);
-    if (m_ok && nn < N)
-      C[(size_t)nn * ldc + m] = gemm_finish((beta == 0.f ? 0.f : beta * cprev[u]) + alpha * sum, m, epi);
+    if (m_ok && nn < N) {
+      const float out = gemm_finish((beta == 0.f ? 0.f : beta * cprev[u]) + alpha * sum, m, epi);
+      C[(size_t)nn * ldc + m] = out;
+      if (epi.sample) {
+        const unsigned int i = (unsigned int)nn * ldc + m;
+        gemm_draw_store(gemm_draw_fetch(i, true, epi), i, out, epi);
+      }
+    }
   }
+  gemm_draw_idle_streams(tid, NW * 64, epi);
 }
 
 // The same single-launch scheme on 16 x 16 output blocks (v_mfma_f32_16x16x4_f32), for products
@@ -550,6 +594,8 @@ k_gemm_tile16(const float* __restrict__ A, int lda, const float* __restrict__ B,
   const int em = m0 + li, en = n0 + 4 * kq + ev;
   const bool e_ok = tid < 256 && em < M && en < N;
   const float cprev = (beta != 0.f && e_ok) ? C[(size_t)en * ldc + em] : 0.f;
+  const unsigned int ei = (unsigned int)en * ldc + em;
+  const GemmDraw draw = gemm_draw_fetch(ei, e_ok, epi);
 
   constexpr int DEPTH = 4;
   const int nfull = K >> 5;                                  // whole chunks; wavefront wv takes wv, wv + NW, ...
@@ -592,8 +638,11 @@ k_gemm_tile16(const float* __restrict__ A, int lda, const float* __restrict__ B,
     float sum = red[0][tid];
 #pragma unroll
     for (int w = 1; w < NW; ++w) sum += red[w][tid];
-    C[(size_t)en * ldc + em] = gemm_finish((beta == 0.f ? 0.f : beta * cprev) + alpha * sum, em, epi);
+    const float out = gemm_finish((beta == 0.f ? 0.f : beta * cprev) + alpha * sum, em, epi);
+    C[(size_t)en * ldc + em] = out;
+    if (epi.sample) gemm_draw_store(draw, ei, out, epi);
   }
+  gemm_draw_idle_streams(tid, NW * 64, epi);
 }
 
 __global__ void k_gemm_splitk_finish(const float* partial, int splits, float* C, int ldc, int M, int N, float alpha,
@@ -637,9 +686,10 @@ static void launch_gemm(bool a_kc, bool b_kc, dim3 grid, const float* A, int lda
 // epi: what to append to each output (bias / activation); *fused tells the caller whether
 // the launch could carry it (the split-K and empty-K paths cannot).
 static int gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, const float* A, int lda, const float* B,
-                int ldb, float beta, float* C, int ldc, GemmEpilogue epi = GemmEpilogue{nullptr, GEMM_ACT_NONE},
-                bool* fused = nullptr) {
+                int ldb, float beta, float* C, int ldc, GemmEpilogue epi = GemmEpilogue{nullptr, GEMM_ACT_NONE, nullptr, nullptr, nullptr, nullptr, 0u},
+                bool* fused = nullptr, bool* sampled = nullptr) {
   if (fused) *fused = false;
+  if (sampled) *sampled = false;
   if (M <= 0 || N <= 0) return 0;
   const int cus = dn_num_cus();
   if (K <= 0) {
@@ -676,6 +726,7 @@ static int gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, co
     else GEMM_T16(false, false);
 #undef GEMM_T16
     if (fused) *fused = true;
+    if (sampled) *sampled = epi.sample != nullptr;
     return dn_launch_status();
   }
   if (tiles64 < cus && off32 && !heavy) {
@@ -695,6 +746,7 @@ static int gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, co
     else GEMM_SMALL(false, false);
 #undef GEMM_SMALL
     if (fused) *fused = true;
+    if (sampled) *sampled = epi.sample != nullptr;
     return dn_launch_status();
   }
   const long long tiles_big = (long long)((M + 127) / 128) * ((N + 127) / 128);
@@ -729,7 +781,7 @@ static int gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, co
     if (!partial) return CUDA_ERROR;
   }
   dim3 grid(gx, gy, splits);
-  const GemmEpilogue none = {nullptr, GEMM_ACT_NONE};
+  const GemmEpilogue none = {nullptr, GEMM_ACT_NONE, nullptr, nullptr, nullptr, nullptr, 0u};
   if (big) launch_gemm<2, 2>(a_kc, b_kc, grid, A, lda, B, ldb, C, ldc, M, N, K, kps, alpha, beta, partial, a_vec, b_vec, splits > 1 ? none : epi);
   else launch_gemm<1, 1>(a_kc, b_kc, grid, A, lda, B, ldb, C, ldc, M, N, K, kps, alpha, beta, partial, a_vec, b_vec, splits > 1 ? none : epi);
   if (fused) *fused = splits == 1;
@@ -748,10 +800,21 @@ int dn_gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, const 
 }
 
 // C = act(op(A)*op(B) + bias) for dot_bias_act(); *fused: whether the launch carried bias and act.
+// smp (may be null): the sample to draw in the same launch; *sampled says whether it was drawn
+// (then the generator's next words are in smp->next and the caller publishes them).
 int dn_gemm_fused(bool a_trans, bool b_trans, int M, int N, int K, const float* A, int lda, const float* B, int ldb,
-                  float* C, int ldc, const float* bias, int act, bool* fused) {
-  const GemmEpilogue epi = {bias, act};
-  return gemm(a_trans, b_trans, M, N, K, 1.f, A, lda, B, ldb, 0.f, C, ldc, epi, fused);
+                  float* C, int ldc, const float* bias, int act, bool* fused, const DnGemmSample* smp, bool* sampled) {
+  GemmEpilogue epi = {bias, act, nullptr, nullptr, nullptr, nullptr, 0u};
+  const unsigned long long total = (unsigned long long)M * (unsigned long long)N;
+  if (smp && ldc == M && total <= (unsigned long long)GEMM_SAMPLE_MAX_DRAWS * NUM_RND_STREAMS) {
+    epi.sample = smp->sample;
+    epi.mults = smp->mults;
+    epi.words = smp->words;
+    epi.next = smp->next;
+    epi.total = (unsigned int)total;
+  }
+  // (only the kernels that finish every output in one launch look at epi.sample)
+  return gemm(a_trans, b_trans, M, N, K, 1.f, A, lda, B, ldb, 0.f, C, ldc, epi, fused, sampled);
 }
 
 extern "C" {

@@ -15,35 +15,13 @@
 //             its first draw by multiplying the stream's word with per-stream
 //             constants (2^32)^-(2^j) mod m, one per set bit of its part number.
 #include "common.h"
+#include "rng.h"
 #include <math.h>
 #include <stdio.h>
 #include <stdlib.h>
 
 #define RNG_PI 3.1415926535897932f
 
-__device__ __forceinline__ unsigned long long mwc_step(unsigned long long w, unsigned int mult) {
-  return (unsigned long long)mult * (w & 0xffffffffull) + (w >> 32);
-}
-
-// (lo32 + 1) / 2^32 with the conversion rounded to nearest even: a value in (0, 1].
-__device__ __forceinline__ float mwc_uniform(unsigned long long w) {
-  return ((float)(unsigned int)(w & 0xffffffffull) + 1.0f) * 2.3283064365386963e-10f;
-}
-
-// Layout of the allocation behind rnd_struct::dev_words (N = 12288 words of 8 bytes):
-// a region aligned to 256 KiB holds two word buffers A (offset 0) and B (offset
-// 128 KiB) and, from offset 256 KiB, the jump table: entry j of stream t multiplies
-// a word by (2^32)^-(2^j) modulo m_t, i.e. jumps 2^j draws ahead.  dev_words points
-// at whichever of A / B holds the current words; the split schedule reads one
-// buffer, writes the other and flips the pointer, so no lane can overwrite a word
-// another lane still has to read.  Bit 17 of the pointer tells the two apart.
-#define RNG_JUMP_BITS 21
-#define RNG_BUF_BYTES (128u << 10)
-#define RNG_REGION_BYTES ((size_t)2 * RNG_BUF_BYTES + (size_t)RNG_JUMP_BITS * NUM_RND_STREAMS * 8)
-
-static inline unsigned long long* rng_other(unsigned long long* w) {
-  return reinterpret_cast<unsigned long long*>(reinterpret_cast<uintptr_t>(w) ^ (uintptr_t)RNG_BUF_BYTES);
-}
 static inline const unsigned long long* rng_table(const unsigned long long* w) {
   return reinterpret_cast<const unsigned long long*>((reinterpret_cast<uintptr_t>(w) & ~(uintptr_t)(2 * RNG_BUF_BYTES - 1)) +
                                                      2 * RNG_BUF_BYTES);

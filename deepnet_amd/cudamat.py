@@ -115,6 +115,7 @@ _SIGNATURES = {
     'correct_preds': (_i, [_M, _M, _M, _f]),
     'dot': (_i, [_M, _M, _M, _f, _f]),
     'dot_bias_act': (_i, [_M, _M, _M, _M, ct.c_int]),
+    'dot_bias_act_sample': (_i, [ct.c_void_p, _M, _M, _M, _M, _M, ct.c_int]),
     'momentum_update': (_i, [_M, _M, _M, _f, _f, _f, _f, ct.c_int]),
     'softmax_ce_grad': (_i, [_M, _M, _M, _M, _M, _f]),
     'init_from_sparse_array': (None, [_S, ct.POINTER(ct.c_float), ct.POINTER(ct.c_int), ct.POINTER(ct.c_int),
@@ -863,19 +864,26 @@ class Graph(object):
             self._exec = None
 
 
-def dot_bias_act(m1, m2, bias=None, target=None, act='sigmoid'):
+def dot_bias_act(m1, m2, bias=None, target=None, act='sigmoid', sample=None):
     """Extension of this backend (not in the reference): target = act(m1 . m2 + bias) in
     one launch, bit-identical to
         cm.dot(m1, m2, target=target); target.add_col_vec(bias); target.apply_sigmoid()
-    (act: None, 'sigmoid', 'relu' = lower_bound(0), 'tanh'; bias: rows x 1 or None)."""
+    (act: None, 'sigmoid', 'relu' = lower_bound(0), 'tanh'; bias: rows x 1 or None).
+    With `sample` (a matrix of target's shape) the same launch also does
+        target.sample_bernoulli(target=sample)
+    with the same draws and the same generator state afterwards."""
     if act not in _ACTS:
         raise ValueError("act must be one of %s" % sorted(k for k in _ACTS if k))
     if target is None:
         m = _cudamat.get_leading_dimension(m1.p_mat)
         n = _cudamat.get_nonleading_dimension(m2.p_mat)
         target = empty((m, n))
-    _check(_cudamat.dot_bias_act(m1.p_mat, m2.p_mat, bias.p_mat if bias is not None else None, target.p_mat,
-                                 _ACTS[act]))
+    b = bias.p_mat if bias is not None else None
+    if sample is None:
+        _check(_cudamat.dot_bias_act(m1.p_mat, m2.p_mat, b, target.p_mat, _ACTS[act]))
+    else:
+        _check(_cudamat.dot_bias_act_sample(CUDAMatrix.rnd_state_p, m1.p_mat, m2.p_mat, b, target.p_mat, sample.p_mat,
+                                            _ACTS[act]))
     return target
 
 

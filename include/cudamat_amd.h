@@ -188,6 +188,13 @@ float euclid_norm(cudamat* mat, int* err_code);
  * apply_tanh (the sequence of deepnet/dbm.py:95-105, deepnet/neuralnet.py:138-160).
  * bias: rows(target) x 1 or NULL; act: 0 none, 1 sigmoid, 2 max(x,0), 3 tanh. */
 int dot_bias_act(cudamat* mat1, cudamat* mat2, cudamat* bias, cudamat* target, int act);
+/* Extension, no counterpart in cudamat.cu: dot_bias_act followed by
+ * sample_bernoulli(rnd_state, target, sample) (the up-pass of an RBM with its hidden sample,
+ * deepnet/dbm.py:95-105), bit-identical to the two calls including the generator's state
+ * afterwards; one launch for single-kernel products of at most 16 * 12288 outputs outside a
+ * graph recording, the separate kernels otherwise.  sample: target's shape, another buffer. */
+int dot_bias_act_sample(rnd_struct* rnd_state, cudamat* mat1, cudamat* mat2, cudamat* bias, cudamat* target,
+                        cudamat* sample, int act);
 
 /* Extension, no counterpart in cudamat.cu: the parameter update of deepnet/parameter.py:80-106
  * in one pass, the same bits as the calls it replaces:

@@ -186,6 +186,72 @@ def test_dot_bias_act_is_bit_identical_to_the_three_calls(cm, rng, m, n, k, ta, 
         x.free_device_memory()
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("m,n,k,ta,act", [
+    (500, 100, 784, True, 'sigmoid'),      # the RBM's up-pass: 16 x 16 blocks, 5 draws per stream
+    (37, 19, 50, False, 'sigmoid'),        # fewer outputs than streams: the idle streams keep their words
+    (1024, 128, 784, True, 'sigmoid'),     # 32 x 32 blocks, 11 draws per stream
+    (96, 128, 64, False, 'tanh'),          # exactly 12288 outputs
+    (1024, 200, 300, True, 'sigmoid'),     # more than 16 draws per stream: separate kernels
+    (2048, 2048, 64, False, 'sigmoid'),    # a product on the big tiles: separate sample kernel
+    (300, 1, 40, False, 'sigmoid'),        # one column: the vector kernels
+])
+def test_dot_bias_act_sample_is_bit_identical_to_the_separate_calls(cm, rng, m, n, k, ta, act):
+    A = _rand(rng, (k, m) if ta else (m, k))
+    a, b = cm.CUDAMatrix(A), cm.CUDAMatrix(_rand(rng, (k, n)))
+    bias = cm.CUDAMatrix(_rand(rng, (m, 1)))
+    opa = a.T if ta else a
+    want, want_s, want_next = cm.empty((m, n)), cm.empty((m, n)), cm.empty((300, 77))
+    got, got_s, got_next = cm.empty((m, n)), cm.empty((m, n)), cm.empty((300, 77))
+    for i in range(2):                       # twice: the second call starts from the words the first one left
+        cm.CUDAMatrix.init_random(40 + i)
+        want_next.fill_with_rand()           # (moves the generator off its seed state)
+        cm.dot_bias_act(opa, b, bias, target=want, act=act)
+        want.sample_bernoulli(target=want_s)
+        want.sample_bernoulli(target=want_s)
+        want_next.fill_with_rand()
+        cm.CUDAMatrix.init_random(40 + i)
+        got_next.fill_with_rand()
+        cm.dot_bias_act(opa, b, bias, target=got, act=act, sample=got_s)
+        r = cm.dot_bias_act(opa, b, bias, target=got, act=act, sample=got_s)
+        assert r is got
+        got_next.fill_with_rand()
+        for x, y in ((want, got), (want_s, got_s), (want_next, got_next)):
+            assert np.array_equal(x.asarray().view(np.uint32), y.asarray().view(np.uint32))
+    smp = got_s.asarray()
+    assert set(np.unique(smp)) <= {0.0, 1.0}
+    if act == 'sigmoid' and m * n > 1000:
+        assert abs(smp.mean() - got.asarray().mean()) < 0.05
+    cm.CUDAMatrix.init_random(1)
+
+
+@pytest.mark.gpu
+def test_dot_bias_act_sample_errors_and_recording(cm, rng):
+    a, b = cm.CUDAMatrix(_rand(rng, (64, 32))), cm.CUDAMatrix(_rand(rng, (32, 48)))
+    t, s = cm.empty((64, 48)), cm.empty((64, 48))
+    with pytest.raises(cm.CUDAMatException):
+        cm.dot_bias_act(a, b, None, target=t, sample=cm.empty((64, 47)))
+    with pytest.raises(cm.CUDAMatException):
+        cm.dot_bias_act(a, b, None, target=t, sample=t)              # the sample needs a buffer of its own
+    assert cm._cudamat.dot_bias_act_sample(cm.CUDAMatrix.rnd_state_p, a.p_mat, b.p_mat, None, t.p_mat, None, 1) != 0
+    # while a graph is recorded the sample comes from its own kernel (the generator keeps one word
+    # buffer); every replay draws on from where the last one stopped
+    cm.CUDAMatrix.init_random(9)
+    want = []
+    for _ in range(3):
+        cm.dot_bias_act(a, b, None, target=t, sample=s)
+        want.append(s.asarray().copy())
+    cm.CUDAMatrix.init_random(9)
+    cm.dot_bias_act(a, b, None, target=t, sample=s)
+    with cm.Graph() as g:
+        cm.dot_bias_act(a, b, None, target=t, sample=s)
+    for i in (1, 2):
+        g.launch()
+        assert np.array_equal(s.asarray(), want[i])
+    g.free()
+    cm.CUDAMatrix.init_random(1)
+
+
 def test_dot_bias_act_errors(cm, rng):
     A = cm.CUDAMatrix(np.zeros((8, 5), dtype=np.float32))
     B = cm.CUDAMatrix(np.zeros((5, 3), dtype=np.float32))
