@@ -603,23 +603,27 @@ k_gemm_tile16(const float* __restrict__ A, int lda, const float* __restrict__ B,
   if (nfull > 0) {
     float a[DEPTH][8], b[DEPTH][8];
     int c = wv;
-    // a set beyond the last chunk re-reads the last one and is never multiplied
+    // Only chunks that exist are asked for (the conditions are wave-uniform): a set that re-read
+    // the last chunk instead made every wavefront of the chip hit the same few lines at once,
+    // which cost 1 us of the 4.8 us of a 500 x 100 x 784 product.
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
-      const int cc = min(c + d * NW, nfull - 1);
-      tile16_load<A_KC>(A, lda, mc, cc, kq, a[d]);
-      tile16_load<B_KC>(B, ldb, nc, cc, kq, b[d]);
+      if (c + d * NW < nfull) {
+        tile16_load<A_KC>(A, lda, mc, c + d * NW, kq, a[d]);
+        tile16_load<B_KC>(B, ldb, nc, c + d * NW, kq, b[d]);
+      }
     }
     for (; c < nfull; c += DEPTH * NW) {
 #pragma unroll
       for (int d = 0; d < DEPTH; ++d) {
-        if (c + d * NW < nfull) {                            // wave-uniform
+        if (c + d * NW < nfull) {
 #pragma unroll
           for (int j = 0; j < 8; ++j) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(b[d][j], a[d][j], acc, 0, 0, 0);
         }
-        const int cc = min(c + (d + DEPTH) * NW, nfull - 1);
-        tile16_load<A_KC>(A, lda, mc, cc, kq, a[d]);
-        tile16_load<B_KC>(B, ldb, nc, cc, kq, b[d]);
+        if (c + (d + DEPTH) * NW < nfull) {
+          tile16_load<A_KC>(A, lda, mc, c + (d + DEPTH) * NW, kq, a[d]);
+          tile16_load<B_KC>(B, ldb, nc, c + (d + DEPTH) * NW, kq, b[d]);
+        }
       }
     }
   }
@@ -643,6 +647,135 @@ k_gemm_tile16(const float* __restrict__ A, int lda, const float* __restrict__ B,
     if (epi.sample) gemm_draw_store(draw, ei, out, epi);
   }
   gemm_draw_idle_streams(tid, NW * 64, epi);
+}
+
+// Short reductions (K <= 128) on 64 x 64 tiles: the whole K extent of a tile's two operands is
+// asked for at once (two 16-byte loads per lane and operand), written to LDS once and multiplied
+// without another wait.  The slab loop of k_gemm spends such a product waiting for one global
+// round trip after the other (its tiles have two slabs in flight; 128 deep is eight slabs).
+// Sixteen wavefronts: (2 x 2) blocks of 32 x 32 outputs times four interleaved quarters of K,
+// so a tile's matrix-core time is 16 instructions per wavefront; the quarters are added up
+// through LDS (in the space of the operands) in a fixed order, every lane finishing four outputs.
+// LDS layouts: a K-contiguous operand is kept [row][k] (pitch 132: 16-byte writes and 16-byte
+// fragment reads, both free of bank conflicts), the other kind [k][row] (pitch 68).  Step t
+// of the multiplication takes k = 8t + 4 (lane / 32) + j, j < 4, from both.
+#define BOX_K 128
+#define BOX_PITCH_KC 132
+#define BOX_PITCH_MC 68
+#define BOX_THREADS 1024
+#define BOX_KW 4
+// One operand's 64 x 128 block into registers; zero where k >= kn.  fast: every 16-byte group
+// is either whole or unused (see the host side); otherwise element by element with clamped
+// indices.  Rows beyond the matrix repeat valid ones and only reach outputs that are not stored.
+template <bool KC>
+__device__ __forceinline__ void box_fetch(const float* __restrict__ P, int ld, int row0, int rows, int kn, int tid, bool fast,
+                                          gemm_f4u (&r)[2]) {
+  if (fast) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int f = tid + u * BOX_THREADS;
+      if (KC) {
+        const int rr = min(row0 + (f >> 5), rows - 1), kq = (f & 31) << 2;
+        r[u] = *reinterpret_cast<const gemm_f4u*>(P + (size_t)rr * ld + (kq < kn ? kq : 0));
+        if (kq >= kn) r[u] = gemm_f4u{0.f, 0.f, 0.f, 0.f};
+      } else {
+        const int k = f >> 4, mq = min(row0 + ((f & 15) << 2), rows - 4);
+        r[u] = *reinterpret_cast<const gemm_f4u*>(P + (size_t)(k < kn ? k : 0) * ld + mq);
+        if (k >= kn) r[u] = gemm_f4u{0.f, 0.f, 0.f, 0.f};
+      }
+    }
+  } else {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int f = tid + u * BOX_THREADS;
+      float v[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        int rr, k;
+        if (KC) { rr = row0 + (f >> 5); k = ((f & 31) << 2) + j; }
+        else { k = f >> 4; rr = row0 + ((f & 15) << 2) + j; }
+        const int rc = min(rr, rows - 1), kc = min(k, kn - 1);
+        const float x = KC ? P[(size_t)rc * ld + kc] : P[(size_t)kc * ld + rc];
+        v[j] = k < kn ? x : 0.f;
+      }
+      r[u] = gemm_f4u{v[0], v[1], v[2], v[3]};
+    }
+  }
+}
+template <bool KC>
+__device__ __forceinline__ void box_stash(float* S, int tid, const gemm_f4u (&r)[2]) {
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const int f = tid + u * BOX_THREADS;
+    if (KC) *reinterpret_cast<gemm_f4u*>(S + (f >> 5) * BOX_PITCH_KC + ((f & 31) << 2)) = r[u];
+    else *reinterpret_cast<gemm_f4u*>(S + (f >> 4) * BOX_PITCH_MC + ((f & 15) << 2)) = r[u];
+  }
+}
+template <bool KC>
+__device__ __forceinline__ void box_frag(const float* S, int row, int lk, int t, float (&v)[4]) {
+  if (KC) {
+    const gemm_f4u x = *reinterpret_cast<const gemm_f4u*>(S + row * BOX_PITCH_KC + 8 * t + 4 * lk);
+    v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w;
+  } else {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) v[j] = S[(8 * t + 4 * lk + j) * BOX_PITCH_MC + row];
+  }
+}
+template <bool A_KC, bool B_KC>
+__global__ void __launch_bounds__(BOX_THREADS)
+k_gemm_box(const float* __restrict__ A, int lda, const float* __restrict__ B, int ldb, float* C, int ldc, int M, int N, int K,
+           float alpha, float beta, bool a_fast, bool b_fast, GemmEpilogue epi) {
+  constexpr int A_FLOATS = A_KC ? 64 * BOX_PITCH_KC : BOX_K * BOX_PITCH_MC;
+  constexpr int B_FLOATS = B_KC ? 64 * BOX_PITCH_KC : BOX_K * BOX_PITCH_MC;
+  static_assert(A_FLOATS + B_FLOATS >= BOX_KW * 4096, "the partial tiles reuse the operands' space");
+  __shared__ __attribute__((aligned(16))) float lds[A_FLOATS + B_FLOATS];
+  float* As = lds;
+  float* Bs = lds + A_FLOATS;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wv & 1, wn = (wv >> 1) & 1, wk = wv >> 2, li = lane & 31, lk = lane >> 5;
+  const int m0 = blockIdx.x * 64, n0 = blockIdx.y * 64;
+  gemm_f4u ra[2], rb[2];
+  box_fetch<A_KC>(A, lda, m0, M, K, tid, a_fast, ra);
+  box_fetch<B_KC>(B, ldb, n0, N, K, tid, b_fast, rb);
+  // the four outputs this lane finishes: e = tid + 1024 u is C(m0 + e % 64, n0 + e / 64)
+  const int em = m0 + (tid & 63);
+  float cold[4];
+  if (beta != 0.f) {    // asked for under the operand loads
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int en = n0 + (tid >> 6) + 16 * u;
+      cold[u] = (em < M && en < N) ? C[(size_t)en * ldc + em] : 0.f;
+    }
+  }
+  box_stash<A_KC>(As, tid, ra);
+  box_stash<B_KC>(Bs, tid, rb);
+  __syncthreads();
+  f32x16 acc;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+  const int steps = (K + 7) >> 3;
+  for (int t = wk; t < steps; t += BOX_KW) {
+    float a[4], b[4];
+    box_frag<A_KC>(As, wm * 32 + li, lk, t, a);
+    box_frag<B_KC>(Bs, wn * 32 + li, lk, t, b);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(b[j], a[j], acc, 0, 0, 0);
+  }
+  __syncthreads();                      // every wavefront is done with the operands
+  // acc[v] is the tile's (m, n) = (32 wm + li, 32 wn + 8 (v / 4) + 4 lk + v % 4); partial tiles are [n][m]
+  float* part = lds + wk * 4096;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) part[(wn * 32 + 8 * (v >> 2) + 4 * lk + (v & 3)) * 64 + wm * 32 + li] = acc[v];
+  __syncthreads();
+  if (em >= M) return;
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int e = tid + BOX_THREADS * u;
+    const int en = n0 + (tid >> 6) + 16 * u;
+    const float sum = (lds[e] + lds[4096 + e]) + (lds[8192 + e] + lds[12288 + e]);
+    if (en < N) C[(size_t)en * ldc + em] = gemm_finish((beta != 0.f ? beta * cold[u] : 0.f) + alpha * sum, em, epi);
+  }
 }
 
 __global__ void k_gemm_splitk_finish(const float* partial, int splits, float* C, int ldc, int M, int N, float alpha,
@@ -712,6 +845,29 @@ static int gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, co
   // (measured: 4096 x 128 x 4096 66 us against 53 us, 2048 x 128 x 2048 17.7 against 21.4).
   const bool heavy = (double)M * (double)N * (double)K >= 1.5e9;
   const long long tiles32 = (long long)((M + 31) / 32) * ((N + 31) / 32);
+  if (K <= BOX_K && tiles64 >= cus / 2 && tiles64 <= 2 * cus) {
+    // short reductions on about one 64 x 64 tile per CU: the whole K extent at once (measured against
+    // the kernels below: 784 x 1024 x 128 6.3 us against 8.4, 1024 x 1024 x 128 with beta = 1 6.1
+    // against 8.7, 1280 x 1280 x 128 9.4 against 10.8; fewer than half a tile per CU and the
+    // kernels that split K over wavefronts win, 640 x 640 x 128 4.6 us against 5.7; from about
+    // 2.3 tiles per CU on the slab loop does, 1536 x 1536 x 64 8.4 us against 9.6)
+    // 16-byte groups run along K for a K-contiguous operand (whole or unused when K % 4 == 0) and
+    // along the rows for the other kind (rows % 4 == 0; the last group of an edge tile then starts
+    // at rows - 4 or earlier)
+    const bool a_fast = a_kc ? K % 4 == 0 : (M % 4 == 0 && M >= 4);
+    const bool b_fast = b_kc ? K % 4 == 0 : (N % 4 == 0 && N >= 4);
+    dim3 grid((M + 63) / 64, (N + 63) / 64);
+#define GEMM_BOX(AK, BK_)                                                                                        \
+  hipLaunchKernelGGL((k_gemm_box<AK, BK_>), grid, dim3(BOX_THREADS), 0, dn_stream(), A, lda, B, ldb, C, ldc, M, N, K, alpha, \
+                     beta, a_fast, b_fast, epi)
+    if (a_kc && b_kc) GEMM_BOX(true, true);
+    else if (a_kc) GEMM_BOX(true, false);
+    else if (b_kc) GEMM_BOX(false, true);
+    else GEMM_BOX(false, false);
+#undef GEMM_BOX
+    if (fused) *fused = true;
+    return dn_launch_status();
+  }
   if (tiles64 < cus && off32 && !heavy && tiles32 * 5 <= cus * 2) {
     // 32 x 32 blocks would leave most of the CUs idle: 16 x 16 blocks, K over 4 wavefronts (measured
     // against 32 x 32 blocks and against 8 wavefronts: 500 x 100 x 784 5.4 us / 7.7 / 6.0; with 128

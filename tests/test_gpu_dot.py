@@ -359,6 +359,38 @@ def test_small_products_on_random_shapes(cm, rng, m, k, n, ta, tb, beta):
         h.free_device_memory()
 
 
+@pytest.mark.parametrize("m,k,n", [(1024, 128, 1024), (1000, 100, 1000), (1001, 97, 999), (777, 128, 1100), (784, 1, 1024),
+                                   (1022, 7, 1026), (650, 60, 1300)])
+@pytest.mark.parametrize("ta,tb", [(False, False), (True, False), (False, True), (True, True)])
+def test_short_reductions_on_about_one_tile_per_cu(cm, rng, m, k, n, ta, tb):
+    """Products with K <= 128 and 128 to 512 tiles of 64 x 64 (on 256 CUs) take the kernel that loads
+    the whole K extent at once: whole and ragged tiles, K a multiple of 4 and not (16-byte groups
+    or single elements), row counts that are and are not multiples of 4; alpha and a beta that
+    reads the target, and the bias / activation epilogue of dot_bias_act."""
+    A, B, C = _rand(rng, (m, k)), _rand(rng, (k, n)), _rand(rng, (m, n))
+    a = cm.CUDAMatrix(np.asfortranarray(A.T)) if ta else cm.CUDAMatrix(A)
+    b = cm.CUDAMatrix(np.asfortranarray(B.T)) if tb else cm.CUDAMatrix(B)
+    c = cm.CUDAMatrix(C)
+    opa, opb = (a.T if ta else a), (b.T if tb else b)
+    cm._check(cm._cudamat.dot(opa.p_mat, opb.p_mat, c.p_mat, -0.5, 2.0))
+    prod = A.astype(np.float64) @ B.astype(np.float64)
+    want = 2.0 * prod - 0.5 * C
+    bound = 2.0 * (np.abs(A).astype(np.float64) @ np.abs(B)) + 0.5 * np.abs(C) + 1e-30
+    assert np.max(np.abs(c.asarray() - want) / bound) < REL
+    # beta = 0 must not read the target
+    c.assign(np.nan)
+    cm.dot(opa, opb, target=c)
+    assert _relerr(c.asarray(), prod, A, B) < REL
+    # the epilogue: bit-identical to the separate calls
+    bias = cm.CUDAMatrix(_rand(rng, (m, 1)))
+    t1, t2 = cm.empty((m, n)), cm.empty((m, n))
+    cm.dot(opa, opb, target=t1); t1.add_col_vec(bias); cm.tanh(t1)
+    cm.dot_bias_act(opa, opb, bias, target=t2, act='tanh')
+    assert np.array_equal(t1.asarray().view(np.uint32), t2.asarray().view(np.uint32))
+    for h in (a, b, c, bias, t1, t2):
+        h.free_device_memory()
+
+
 @pytest.mark.parametrize("m,k,n", [(15, 31, 17), (16, 32, 16), (17, 33, 15), (48, 64, 80), (31, 65, 33), (100, 1029, 20),
                                    (3, 2000, 5), (250, 96, 250)])
 @pytest.mark.parametrize("ta,tb", [(False, False), (True, False), (False, True), (True, True)])
