@@ -314,6 +314,43 @@ def gemm_probe(cm, ev, n=4096, iters=10, warm_s=0.03):
     return out
 
 
+def gemm_layer_shapes(cm, ev, iters=200):
+    """The products of the RBM (config 1) and MLP (config 3) steps, one shape at a time: HIP
+    events around `iters` back-to-back launches (an empty kernel takes 2.4 us that way)."""
+    rng = np.random.default_rng(7)
+    f = lambda *s: cm.CUDAMatrix(np.asarray(rng.standard_normal(s), dtype=np.float32, order='F'))
+    out = {}
+
+    def timed(label, fn, flops):
+        for _ in range(20):
+            fn()
+        e0, e1 = ev.new(), ev.new()
+        ev.record(e0)
+        for _ in range(iters):
+            fn()
+        ev.record(e1)
+        us = ev.elapsed_ms(e0, e1) / iters * 1e3
+        tf = flops / (us * 1e-6) / 1e12
+        out[label] = {'us': round(us, 2), 'tflops': round(tf, 2), 'frac_mfma_fp32': round(tf / MFMA_FP32_PEAK_TFLOPS, 4)}
+    nv, nh, B = 784, 500, 100
+    W, v, h, v2 = f(nv, nh), f(nv, B), f(nh, B), cm.empty((nv, B))
+    hh = cm.empty((nh, B))
+    timed('rbm_up_500x100x784', lambda: cm.dot(W.T, v, target=hh), 2.0 * nv * nh * B)
+    timed('rbm_down_784x100x500', lambda: cm.dot(W, h, target=v2), 2.0 * nv * nh * B)
+    timed('rbm_stats_784x500x100', lambda: W.add_dot(v, h.T, mult=1e-6), 2.0 * nv * nh * B)
+    for m in (W, v, h, v2, hh):
+        m.free_device_memory()
+    for a, b in ((784, 1024), (1024, 1024), (1024, 10)):
+        Wm, x, y, d = f(a, b), f(a, 128), cm.empty((b, 128)), f(b, 128)
+        xb, g = cm.empty((a, 128)), cm.empty((a, b))
+        timed('mlp_fwd_%dx128x%d' % (b, a), lambda: cm.dot(Wm.T, x, target=y), 2.0 * a * b * 128)
+        timed('mlp_bwd_%dx128x%d' % (a, b), lambda: cm.dot(Wm, d, target=xb), 2.0 * a * b * 128)
+        timed('mlp_grad_%dx%dx128' % (a, b), lambda: g.add_dot(x, d.T, mult=0.01), 2.0 * a * b * 128)
+        for m in (Wm, x, y, d, xb, g):
+            m.free_device_memory()
+    return out
+
+
 # ---------------------------------------------------------------- CPU baseline
 
 def cpu_baseline_c2():
@@ -605,6 +642,7 @@ def main():
         t = time_loop(cm, lambda: convnet.TrainOneBatch(0), 50, 5)
         secondary['example_convnet_batch100']['us_per_step_fused_extensions'] = round(t * 1e6, 1)
         secondary['gemm_fp32_4096'] = gemm_probe(cm, ev)
+        secondary['gemm_layer_shapes'] = gemm_layer_shapes(cm, ev)
         try:
             import bench_conv
             secondary.update(bench_conv.run(cm, ev))
