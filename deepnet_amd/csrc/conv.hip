@@ -1540,11 +1540,23 @@ static void launch_rowmajor(const ConvArgs& a0, long long rows, int cols, int gz
   const long long total = MODE == CONV_UP ? (long long)a.N * a.M * a.F : (long long)a.N * a.HH * a.C;
   long long want = 1;
   // (the sum of the partial outputs writes 16-byte groups)
-  if ((MODE == CONV_UP || (MODE == CONV_DOWN && a.s == 1)) && tiles < cus && a.scale_t == 0.f && a.scale_o == 1.f &&
-      dn_aligned16(a.out)) {
-    want = (2ll * cus) / tiles;
-    if (want > nslabs / 8) want = nslabs / 8;
-    if (want > 16) want = 16;
+  if ((MODE == CONV_UP || (MODE == CONV_DOWN && a.s == 1)) && a.scale_t == 0.f && a.scale_o == 1.f && dn_aligned16(a.out)) {
+    if (tiles < cus && (2 * tiles < cus || nslabs < 40)) {
+      want = (2ll * cus) / tiles;
+      if (want > nslabs / 8) want = nslabs / 8;
+      if (want > 16) want = 16;
+    } else if (nslabs >= 40 && 10 * tiles <= (MODE == CONV_UP ? 25ll : 13ll) * cus) {
+      // Long reductions on about one tile per CU: a lone workgroup per CU leaves every wait of its
+      // slab loop exposed, so the reduction is cut until three to four workgroups share a CU, each
+      // keeping at least 20 slabs (measured on 64 -> 64 colours of 5 x 5, batch 128: 16 x 16 maps
+      // Up 98 -> 79 us and Down 74 -> 65 us, 18 x 18 maps Up 146 -> 96 us and Down 109 -> 89 us, 12 x 12
+      // maps Up 61 -> 53 us; convDown stops gaining at 1.3 tiles per CU, convUp at 2.5; short
+      // reductions lose to the extra pass over the output: 32 colours of 3 x 3, 22 -> 30 us)
+      const long long target = (MODE == CONV_UP ? 4ll : 3ll) * cus;
+      want = (target + tiles / 2) / tiles;
+      if (want > 8) want = 8;
+      while (want > 1 && nslabs / want < 20) --want;
+    }
     if (want < 1) want = 1;
   }
   if (want > 1) {
