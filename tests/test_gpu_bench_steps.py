@@ -53,9 +53,19 @@ def test_mlp_step_of_the_benchmark_against_the_oracle(cm, fused):
         layers.append({'act': act, 'hyper': hyp(dropout=i < 2, dropout_prob=0.5), 'bias': mlp.b[i].asarray(),
                        'edge': {'w': mlp.W[i].asarray(), 'hyper': hyp()}, 'loss': 'CROSS_ENTROPY'})
     onet = no.Net(layers)
+    twin_masks = []
+    if fused:
+        # the fused step draws its dropout decisions without writing masks: a twin run of the plain
+        # step from the same seed makes the same draws and leaves them in its masks
+        twin = bench.MLP(cm)
+        for step in range(3):
+            twin.step()
+            twin_masks.append([twin.mask[0].asarray().copy(), twin.mask[1].asarray().copy()])
+        cm.CUDAMatrix.init_random(3)
     for step in range(3):
         (mlp.step_fused if fused else mlp.step)()
-        masks = [None, mlp.mask[0].asarray(), mlp.mask[1].asarray(), None]
+        m01 = twin_masks[step] if fused else [mlp.mask[0].asarray(), mlp.mask[1].asarray()]
+        masks = [None, m01[0], m01[1], None]
         for m in masks[1:3]:
             assert set(np.unique(m)) <= {0.0, 1.0} and 0.45 < m.mean() < 0.55
         perf = onet.train_step(x, labels, step, masks=masks)
