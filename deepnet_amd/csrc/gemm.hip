@@ -549,8 +549,8 @@ k_gemm_small(const float* __restrict__ A, int lda, const float* __restrict__ B, 
 // every NW-th chunk, four in flight each, and add up through LDS in wavefront order.
 typedef float f32x4m __attribute__((ext_vector_type(4)));
 
-// One whole chunk: no conditions, so that every load of a wavefront's four chunks is in
-// flight before the first multiplication (16-byte requests are taken at 4-byte alignment).
+// One whole chunk, without lane-dependent conditions: the loads of a wavefront's first four chunks
+// are all in flight before its first multiplication (16-byte requests are taken at 4-byte alignment).
 template <bool KC>
 __device__ __forceinline__ void tile16_load(const float* __restrict__ P, unsigned ld, unsigned row, int chunk, int kq,
                                             float (&r)[8]) {
