@@ -183,8 +183,11 @@ __device__ __forceinline__ void down_axis(int ph, int s, int pad0, int H, int k,
 // an add and a load.  convUp: the rows fill their tiles, and a tap beyond the reduction
 // re-reads the last one against a zero filter row.  convOutp: rows and columns beyond
 // the output are computed on whatever valid data was read and never stored.
+// (the merged-phase convDown kernels are asked to fit four wavefronts per SIMD, 128 registers: the
+// 3 colours x 16 phases of config 5a then run 288 us instead of 307; the same request costs every
+// other variant time -- config 5b's convOutp 530 -> 675 us with 168 registers and spills)
 template <int MODE, int WAVES_M, int WM, int WN, bool UNI = false, int N16 = 0, bool INSIDE = false, bool LOCAL = false>
-__global__ void __launch_bounds__(256) k_conv_mfma(ConvArgs p) {
+__global__ void __launch_bounds__(256, (MODE == CONV_DOWNM && WM * WN <= 2 ? 4 : 0)) k_conv_mfma(ConvArgs p) {
   static_assert(!LOCAL || UNI, "one filter bank per module: uniform-row kernels only");
   static_assert(!INSIDE || ((MODE == CONV_UP || MODE == CONV_OUTP) && !UNI), "INSIDE: the general gathers of the image");
   constexpr int WAVES_N = 4 / WAVES_M;
