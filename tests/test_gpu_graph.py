@@ -95,6 +95,30 @@ def test_conv_stage_is_recorded_with_the_matrix_ops(cm, cc):
     g.free()
 
 
+def test_split_conv_layer_records_with_and_without_its_workspace(cm, cc):
+    """A conv layer whose reduction is split over workgroups (partial outputs in the grow-only
+    workspace): recorded after an eager call it replays the split form; recorded in a fresh
+    process state, where the workspace would have to grow, it records the unsplit form.  Both
+    give the eager result to rounding."""
+    rng = np.random.default_rng(9)
+    N, C, H, F, k, p = 128, 64, 16, 64, 5, 2
+    f = lambda a: cm.CUDAMatrix(np.asarray(a, dtype=np.float32, order='F'))
+    x, w = f(rng.standard_normal((N, C * H * H))), f(0.05 * rng.standard_normal((F, C * k * k)))
+    up1, up2, up3 = cm.empty((N, F * H * H)), cm.empty((N, F * H * H)), cm.empty((N, F * H * H))
+    with cm.Graph() as g_first:                       # whatever workspace earlier tests left: may or may not suffice
+        cc.convUp(x, w, up1, H, p, 1, C)
+    g_first.launch()
+    cc.convUp(x, w, up2, H, p, 1, C)                  # eager: the workspace has its size now
+    with cm.Graph() as g_second:
+        cc.convUp(x, w, up3, H, p, 1, C)
+    g_second.launch()
+    a, b, c = up1.asarray(), up2.asarray(), up3.asarray()
+    assert np.array_equal(b.view(np.uint32), c.view(np.uint32))
+    scale = np.abs(b).max()
+    assert np.max(np.abs(a - b)) <= 1e-5 * scale
+    g_first.free(); g_second.free()
+
+
 def test_what_cannot_be_recorded_raises(cm):
     a = cm.CUDAMatrix(np.ones((8, 8), dtype=np.float32))
     big = cm.empty((1024, 512))                          # 524288 elements: the generator's split schedule
