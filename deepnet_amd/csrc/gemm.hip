@@ -868,10 +868,15 @@ static int gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, co
     if (fused) *fused = true;
     return dn_launch_status();
   }
-  if (tiles64 < cus && off32 && !heavy && tiles32 * 5 <= cus * 2) {
-    // 32 x 32 blocks would leave most of the CUs idle: 16 x 16 blocks, K over 4 wavefronts (measured
-    // against 32 x 32 blocks and against 8 wavefronts: 500 x 100 x 784 5.4 us / 7.7 / 6.0; with 128
-    // blocks of 32 x 32, 1024 x 128 x 784, the larger blocks win, 7.7 us against 8.8)
+  // Two K-contiguous operands whose rows lie a multiple of 1 KiB apart: the 16 x 16 block kernel
+  // reads 16 such rows per load instruction and they meet in the same memory channels (measured
+  // 1024 x 128 x 1024 with both leading dimensions 1024: 9.2 us against 8.5 us on 32 x 32 blocks).
+  const bool kc_aliased = a_kc && b_kc && (lda % 256 == 0 || ldb % 256 == 0);
+  if (tiles64 < cus && off32 && !heavy && (tiles32 * 5 <= cus * 2 || (tiles32 * 2 <= cus && !kc_aliased))) {
+    // 32 x 32 blocks would leave half or more of the CUs idle: 16 x 16 blocks, K over 4 wavefronts
+    // (measured against 32 x 32 blocks: 500 x 100 x 784 4.4 us against 7.7, 1024 x 128 x 784 6.5 against
+    // 7.9, 1024 x 128 x 1024 with an M-contiguous first operand 7.2 against 8.8; against 8 wavefronts per
+    // block: 500 x 100 x 784 5.4 us against 6.0)
     dim3 grid((M + 15) / 16, (N + 15) / 16);
 #define GEMM_T16(AK, BK_)                                                                                  \
   hipLaunchKernelGGL((k_gemm_tile16<AK, BK_, 4>), grid, dim3(256), 0, dn_stream(), A, lda, B, ldb, C, ldc, M, N, K, \
