@@ -190,7 +190,9 @@ def test_dot_bias_act_is_bit_identical_to_the_three_calls(cm, rng, m, n, k, ta, 
 @pytest.mark.parametrize("m,n,k,ta,act", [
     (500, 100, 784, True, 'sigmoid'),      # the RBM's up-pass: 16 x 16 blocks, 5 draws per stream
     (37, 19, 50, False, 'sigmoid'),        # fewer outputs than streams: the idle streams keep their words
-    (1024, 128, 784, True, 'sigmoid'),     # 32 x 32 blocks, 11 draws per stream
+    (1024, 128, 784, True, 'sigmoid'),     # 16 x 16 blocks on 512 workgroups, 11 draws per stream
+    (768, 192, 300, True, 'sigmoid'),      # 32 x 32 blocks (144 of them), 12 draws per stream
+    (1024, 128, 512, True, 'relu'),        # 32 x 32 blocks: both operands K-contiguous, rows 2 KiB apart
     (96, 128, 64, False, 'tanh'),          # exactly 12288 outputs
     (1024, 200, 300, True, 'sigmoid'),     # more than 16 draws per stream: separate kernels
     (2048, 2048, 64, False, 'sigmoid'),    # a product on the big tiles: separate sample kernel
