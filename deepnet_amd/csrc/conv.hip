@@ -1533,7 +1533,7 @@ __global__ void __launch_bounds__(256) k_conv_sum_splits(const float* partial, i
   }
 }
 
-template <int MODE>
+template <int MODE, bool LOCAL = false>
 static void launch_rowmajor_tiles(const ConvArgs& a, long long rows, int cols, int gz);
 template <int MODE, bool LOCAL = false>
 static void launch_uniform_rows(const ConvArgs& a, long long rows, int cols, int gz);
@@ -1545,7 +1545,7 @@ static void launch_general_rows(const ConvArgs& a, long long rows, int cols, int
 // latency: split the reduction over up to 16 workgroups per tile (at least 8 slabs each)
 // and sum the partial outputs with a second kernel.  (32 -> 64 filters of 5 x 5 on 8 x 8
 // maps: convUp 51 -> 17 us.)
-template <int MODE>
+template <int MODE, bool LOCAL = false>
 static void launch_rowmajor(const ConvArgs& a0, long long rows, int cols, int gz) {
   ConvArgs a = a0;
   const int cus = dn_num_cus();
@@ -1582,7 +1582,7 @@ static void launch_rowmajor(const ConvArgs& a0, long long rows, int cols, int gz
     if (!a.partial) { a.splits = 1; a.slabs_per_split = 0; }
     else a.split_stride = total;
   }
-  launch_rowmajor_tiles<MODE>(a, rows, cols, gz * a.splits);
+  launch_rowmajor_tiles<MODE, LOCAL>(a, rows, cols, gz * a.splits);
   if (a.splits > 1) {
     const long long total4 = total / 4;            // (the batch is a multiple of 16)
     long long blocks = (total4 + 255) / 256;
@@ -1592,8 +1592,12 @@ static void launch_rowmajor(const ConvArgs& a0, long long rows, int cols, int gz
   }
 }
 
-template <int MODE>
+template <int MODE, bool LOCAL>
 static void launch_rowmajor_tiles(const ConvArgs& a, long long rows, int cols, int gz) {
+  if constexpr (LOCAL) {   // (the caller has checked what the uniform-row kernels need)
+    launch_uniform_rows<MODE, true>(a, rows, cols, gz);
+    return;
+  }
   // Batches that are multiples of 128: tiles of 128 rows never straddle a module / pixel.
   // Measured on the benchmark layers: the buffer-load kernels win for long reductions
   // with up to 64 or more than 96 columns; 65-96 columns and short reductions are
@@ -1711,7 +1715,7 @@ static void conv_up_impl(cudamat* images, cudamat* filters, cudamat* targets, in
   } else if (local && fast_ok(a) && N % 128 == 0 && a.a_bytes != 0 && a.b_bytes != 0) {
     // locally connected: a 128-row tile is one module, so the uniform-row kernels only add that
     // module's bank to the filter offset
-    launch_uniform_rows<CONV_UP, true>(a, (long long)M * N, a.Fg, numGroups);
+    launch_rowmajor<CONV_UP, true>(a, (long long)M * N, a.Fg, numGroups);
   } else {
     const long long total = (long long)N * M * F;
     long long blocks = (total + 255) / 256;
@@ -1809,7 +1813,7 @@ static void conv_down_impl(cudamat* hidActs, cudamat* filters, cudamat* targets,
   } else if (local_uni) {
     // locally connected: a 128-row tile is one pixel; every slab adds the bank of the module its tap reaches
     const int q = (imgSize + moduleStride - 1) / moduleStride;
-    launch_uniform_rows<CONV_DOWN, true>(a, (long long)q * q * N, a.Cg, numGroups * moduleStride * moduleStride);
+    launch_rowmajor<CONV_DOWN, true>(a, (long long)q * q * N, a.Cg, numGroups * moduleStride * moduleStride);
   } else {
     const long long total = (long long)N * a.HH * numImgColors;
     long long blocks = (total + 255) / 256;
