@@ -16,39 +16,63 @@ __device__ __forceinline__ int wrap_index(float f, int n) {
   return (i < 0 || i >= n) ? -1 : i;
 }
 
+// W consecutive rows of a column per lane: 1, or 4 as one 16-byte access (row counts that are
+// multiples of 4, aligned operands: 4096 x 4096 select_columns 53 -> 27 us).
+template <int W>
+__device__ __forceinline__ void rows_ld(const float* p, float (&v)[W]) {
+  if constexpr (W == 4) { const float4 t = *reinterpret_cast<const float4*>(p); v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w; }
+  else v[0] = *p;
+}
+template <int W>
+__device__ __forceinline__ void rows_st(float* p, const float (&v)[W]) {
+  if constexpr (W == 4) *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+  else *p = v[0];
+}
+
 // target(:, c) = source(:, idx[c])
+template <int W>
 __global__ void k_select_cols(const float* source, float* target, const float* indices, int n_idx, int h, int src_w) {
-  const int r = blockIdx.x * blockDim.x + threadIdx.x;
+  const int r = (blockIdx.x * blockDim.x + threadIdx.x) * W;
   if (r >= h) return;
   for (int c = blockIdx.y; c < n_idx; c += gridDim.y) {
     const int s = wrap_index(indices[c], src_w);
-    target[(size_t)c * h + r] = s < 0 ? NAN : source[(size_t)s * h + r];
+    float v[W];
+    if (s < 0) { for (int k = 0; k < W; ++k) v[k] = NAN; }
+    else rows_ld<W>(source + (size_t)s * h + r, v);
+    rows_st<W>(target + (size_t)c * h + r, v);
   }
 }
 
 // target(:, idx[c]) = source(:, c)
+template <int W>
 __global__ void k_set_selected_cols(float* target, const float* source, const float* indices, int n_idx, int h,
                                     int tgt_w) {
-  const int r = blockIdx.x * blockDim.x + threadIdx.x;
+  const int r = (blockIdx.x * blockDim.x + threadIdx.x) * W;
   if (r >= h) return;
   for (int c = blockIdx.y; c < n_idx; c += gridDim.y) {
     const int t = wrap_index(indices[c], tgt_w);
-    if (t >= 0) target[(size_t)t * h + r] = source[(size_t)c * h + r];
+    if (t < 0) continue;
+    float v[W];
+    rows_ld<W>(source + (size_t)c * h + r, v);
+    rows_st<W>(target + (size_t)t * h + r, v);
   }
 }
 
 // swap source(:, idx1[c]) with target(:, idx2[c])
+template <int W>
 __global__ void k_swap_cols(float* source, float* target, const float* idx1, const float* idx2, int cols, int src_w,
                             int tgt_w, int h) {
-  const int r = blockIdx.x * blockDim.x + threadIdx.x;
+  const int r = (blockIdx.x * blockDim.x + threadIdx.x) * W;
   if (r >= h) return;
   for (int c = blockIdx.y; c < cols; c += gridDim.y) {
     const int s = (int)idx1[c], t = (int)idx2[c];
     if (s < 0 || s >= src_w || t < 0 || t >= tgt_w) continue;
     const size_t ps = (size_t)s * h + r, pt = (size_t)t * h + r;
-    const float tmp = source[ps];
-    source[ps] = target[pt];
-    target[pt] = tmp;
+    float a[W], b[W];
+    rows_ld<W>(source + ps, a);
+    rows_ld<W>(target + pt, b);
+    rows_st<W>(source + ps, b);
+    rows_st<W>(target + pt, a);
   }
 }
 
@@ -88,24 +112,38 @@ __global__ void k_translate(const float* source, float* target, const float* off
 }
 
 // target(:, c) = source(:, idx[c]) for every target column, NaN when outside.
+template <int W>
 __global__ void k_expand(const float* source, const float* indices, float* target, int h, int w, int tw) {
-  const int r = blockIdx.x * blockDim.x + threadIdx.x;
+  const int r = (blockIdx.x * blockDim.x + threadIdx.x) * W;
   if (r >= h) return;
   for (int c = blockIdx.y; c < tw; c += gridDim.y) {
     const int s = (int)indices[c];
-    target[(size_t)c * h + r] = (s >= 0 && s < w) ? source[(size_t)s * h + r] : NAN;
+    float v[W];
+    if (s >= 0 && s < w) rows_ld<W>(source + (size_t)s * h + r, v);
+    else { for (int k = 0; k < W; ++k) v[k] = NAN; }
+    rows_st<W>(target + (size_t)c * h + r, v);
   }
 }
 
 // target(:, c) = source(:, c) + mult * mat(:, idx[c])
+template <int W>
 __global__ void k_expand_and_add(const float* source, const float* mat, const float* indices, float* target, int w,
                                  int h, float mult, int w2) {
-  const int r = blockIdx.x * blockDim.x + threadIdx.x;
+  const int r = (blockIdx.x * blockDim.x + threadIdx.x) * W;
   if (r >= h) return;
   for (int c = blockIdx.y; c < w; c += gridDim.y) {
     const int s = (int)indices[c];
     const size_t p = (size_t)c * h + r;
-    target[p] = (s >= 0 && s < w2) ? source[p] + mult * mat[(size_t)s * h + r] : NAN;
+    float v[W];
+    if (s >= 0 && s < w2) {
+      float x[W], y[W];
+      rows_ld<W>(source + p, x);
+      rows_ld<W>(mat + (size_t)s * h + r, y);
+      for (int k = 0; k < W; ++k) v[k] = x[k] + mult * y[k];
+    } else {
+      for (int k = 0; k < W; ++k) v[k] = NAN;
+    }
+    rows_st<W>(target + p, v);
   }
 }
 
@@ -128,8 +166,13 @@ __global__ void k_accumulate_cols(const float* mat, const float* indices, float*
   }
 }
 
-static inline dim3 col_grid(int h, int cols) {
-  return dim3((h + 255) / 256, cols < 8192 ? (cols > 0 ? cols : 1) : 8192);
+static inline dim3 col_grid(int h, int cols, int rows_per_lane = 1) {
+  const int lanes = (h + rows_per_lane - 1) / rows_per_lane;
+  return dim3((lanes + 255) / 256, cols < 8192 ? (cols > 0 ? cols : 1) : 8192);
+}
+// 16-byte accesses down the rows: every column of these matrices then starts on a 16-byte boundary
+static inline bool rows4(int h, const void* a, const void* b, const void* c = nullptr) {
+  return h % 4 == 0 && dn_aligned16(a) && dn_aligned16(b) && (!c || dn_aligned16(c));
 }
 
 extern "C" {
@@ -140,8 +183,12 @@ int selectRows(cudamat* source, cudamat* target, cudamat* indices) {
   if (target->size[0] != source->size[0] || target->size[1] < n || indices->size[0] != 1)
     return ERROR_INCOMPATIBLE_DIMENSIONS;
   if (n == 0 || source->size[0] == 0) return 0;
-  hipLaunchKernelGGL(k_select_cols, col_grid(source->size[0], n), dim3(256), 0, dn_stream(), (const float*)source->data_device,
-                     target->data_device, (const float*)indices->data_device, n, source->size[0], source->size[1]);
+  if (rows4(source->size[0], source->data_device, target->data_device))
+    hipLaunchKernelGGL(k_select_cols<4>, col_grid(source->size[0], n, 4), dim3(256), 0, dn_stream(), (const float*)source->data_device,
+                       target->data_device, (const float*)indices->data_device, n, source->size[0], source->size[1]);
+  else
+    hipLaunchKernelGGL(k_select_cols<1>, col_grid(source->size[0], n), dim3(256), 0, dn_stream(), (const float*)source->data_device,
+                       target->data_device, (const float*)indices->data_device, n, source->size[0], source->size[1]);
   return dn_launch_status();
 }
 
@@ -151,9 +198,14 @@ int setSelectedRows(cudamat* target, cudamat* source, cudamat* indices) {
   if (target->size[0] != source->size[0] || source->size[1] < n || indices->size[0] != 1)
     return ERROR_INCOMPATIBLE_DIMENSIONS;
   if (n == 0 || source->size[0] == 0) return 0;
-  hipLaunchKernelGGL(k_set_selected_cols, col_grid(source->size[0], n), dim3(256), 0, dn_stream(), target->data_device,
-                     (const float*)source->data_device, (const float*)indices->data_device, n, target->size[0],
-                     target->size[1]);
+  if (rows4(source->size[0], source->data_device, target->data_device))
+    hipLaunchKernelGGL(k_set_selected_cols<4>, col_grid(source->size[0], n, 4), dim3(256), 0, dn_stream(), target->data_device,
+                       (const float*)source->data_device, (const float*)indices->data_device, n, target->size[0],
+                       target->size[1]);
+  else
+    hipLaunchKernelGGL(k_set_selected_cols<1>, col_grid(source->size[0], n), dim3(256), 0, dn_stream(), target->data_device,
+                       (const float*)source->data_device, (const float*)indices->data_device, n, target->size[0],
+                       target->size[1]);
   return dn_launch_status();
 }
 
@@ -164,9 +216,14 @@ int swapColumns(cudamat* source, cudamat* target, cudamat* indices1, cudamat* in
     return ERROR_NOT_ON_DEVICE;
   if (target->size[0] != h || indices2->size[0] * indices2->size[1] != cols) return ERROR_INCOMPATIBLE_DIMENSIONS;
   if (cols == 0 || h == 0) return 0;
-  hipLaunchKernelGGL(k_swap_cols, col_grid(h, cols), dim3(256), 0, dn_stream(), source->data_device, target->data_device,
-                     (const float*)indices1->data_device, (const float*)indices2->data_device, cols, source->size[1],
-                     target->size[1], h);
+  if (rows4(h, source->data_device, target->data_device))
+    hipLaunchKernelGGL(k_swap_cols<4>, col_grid(h, cols, 4), dim3(256), 0, dn_stream(), source->data_device, target->data_device,
+                       (const float*)indices1->data_device, (const float*)indices2->data_device, cols, source->size[1],
+                       target->size[1], h);
+  else
+    hipLaunchKernelGGL(k_swap_cols<1>, col_grid(h, cols), dim3(256), 0, dn_stream(), source->data_device, target->data_device,
+                       (const float*)indices1->data_device, (const float*)indices2->data_device, cols, source->size[1],
+                       target->size[1], h);
   return dn_launch_status();
 }
 
@@ -215,8 +272,12 @@ int expand(cudamat* source, cudamat* indices, cudamat* target) {
   if (target->size[0] != h) return ERROR_INCOMPATIBLE_DIMENSIONS;
   if (indices->size[0] != 1 || indices->size[1] != w2) return ERROR_INCOMPATIBLE_DIMENSIONS;
   if (h == 0 || w2 == 0) return 0;
-  hipLaunchKernelGGL(k_expand, col_grid(h, w2), dim3(256), 0, dn_stream(), (const float*)source->data_device,
-                     (const float*)indices->data_device, target->data_device, h, w, w2);
+  if (rows4(h, source->data_device, target->data_device))
+    hipLaunchKernelGGL(k_expand<4>, col_grid(h, w2, 4), dim3(256), 0, dn_stream(), (const float*)source->data_device,
+                       (const float*)indices->data_device, target->data_device, h, w, w2);
+  else
+    hipLaunchKernelGGL(k_expand<1>, col_grid(h, w2), dim3(256), 0, dn_stream(), (const float*)source->data_device,
+                       (const float*)indices->data_device, target->data_device, h, w, w2);
   return dn_launch_status();
 }
 
@@ -228,9 +289,14 @@ int expand_and_add(cudamat* source, cudamat* mat, cudamat* indices, cudamat* tar
   if (indices->size[0] != 1 || indices->size[1] != w) return ERROR_INCOMPATIBLE_DIMENSIONS;
   if (mat->size[0] != h) return ERROR_INCOMPATIBLE_DIMENSIONS;
   if (h == 0 || w == 0) return 0;
-  hipLaunchKernelGGL(k_expand_and_add, col_grid(h, w), dim3(256), 0, dn_stream(), (const float*)source->data_device,
-                     (const float*)mat->data_device, (const float*)indices->data_device, target->data_device, w, h,
-                     mult, w2);
+  if (rows4(h, source->data_device, target->data_device, mat->data_device))
+    hipLaunchKernelGGL(k_expand_and_add<4>, col_grid(h, w, 4), dim3(256), 0, dn_stream(), (const float*)source->data_device,
+                       (const float*)mat->data_device, (const float*)indices->data_device, target->data_device, w, h,
+                       mult, w2);
+  else
+    hipLaunchKernelGGL(k_expand_and_add<1>, col_grid(h, w), dim3(256), 0, dn_stream(), (const float*)source->data_device,
+                       (const float*)mat->data_device, (const float*)indices->data_device, target->data_device, w, h,
+                       mult, w2);
   return dn_launch_status();
 }
 

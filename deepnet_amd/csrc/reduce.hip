@@ -361,6 +361,19 @@ __global__ void k_softmax_grad(const float* mat, const float* labels, float* tar
     target[i] = mat[i] - (((int)labels[q] == (int)r) ? 1.f : 0.f);
   }
 }
+// The same with 16-byte groups (h a multiple of 4, aligned operands: a group stays inside its
+// column), one group per lane.
+template <bool STREAM>
+__global__ void __launch_bounds__(256) k_softmax_grad4(const float* mat, const float* labels, float* target, long long n4, int h, FastDiv fd) {
+  const long long tid = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (tid >= n4) return;
+  const uint32_t e = (uint32_t)(4 * tid);
+  const uint32_t q = fd_div(e, fd);
+  const int r = (int)(e - q * (uint32_t)h), lab = (int)labels[q];
+  float4 v = dn_ld4<STREAM>(mat + e);
+  v.x -= lab == r ? 1.f : 0.f; v.y -= lab == r + 1 ? 1.f : 0.f; v.z -= lab == r + 2 ? 1.f : 0.f; v.w -= lab == r + 3 ? 1.f : 0.f;
+  dn_st4<STREAM>(target + e, v);
+}
 
 __global__ void k_softmax_ce(const float* mat, const float* labels, float* target, int w, int h, float tiny) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
@@ -410,20 +423,6 @@ k_row_reduce(const float* mat, float* target, int w, int h, int op, float mult, 
   else { for (int j = wv; j < w; j += 4) target[(size_t)j * h + row] = (j == bidx) ? 1.f : 0.f; }
 }
 
-__global__ void __launch_bounds__(256) k_row_normlimit(const float* mat, float* target, int w, int h, float norm) {
-  __shared__ float sv[4][64];
-  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-  const int row = blockIdx.x * 64 + lane;
-  float acc = 0.f;
-  if (row < h)
-    for (int j = wv; j < w; j += 4) { const float v = mat[(size_t)j * h + row]; acc += v * v; }
-  sv[wv][lane] = acc;
-  __syncthreads();
-  if (row >= h) return;
-  float scale = sqrtf((sv[0][lane] + sv[1][lane]) + (sv[2][lane] + sv[3][lane]));
-  scale = (scale < norm) ? 1.f : (norm / scale);
-  for (int j = wv; j < w; j += 4) target[(size_t)j * h + row] = mat[(size_t)j * h + row] * scale;
-}
 
 // ------------------------------------------------------------------ weighted sums (matrix-vector)
 
@@ -1098,6 +1097,36 @@ int sqsum_by_axis(cudamat* mat, cudamat* target, int axis, float mult, float p) 
   return ERROR_UNSUPPORTED;
 }
 
+}  // extern "C"
+
+// t(i, j) = a(i, j) * (n_i < norm ? 1 : norm / n_i) with n_i = sqrt(sq[i]): the second pass of
+// normlimit_by_axis along the rows (cudamat_kernels.cu:1100-1130), given the rows' sums of
+// squares.  A flat pass over the matrix; VEC: 16-byte groups (h a multiple of 4, aligned
+// operands), whose four rows are one 16-byte group of sq.
+template <bool VEC, bool STREAM>
+__global__ void __launch_bounds__(256)
+k_scale_rows_to_norm(const float* a, const float* sq, float* t, long long n, FastDiv fd, float norm) {
+  auto one = [&](float x, float s) {
+    const float nn = sqrtf(s);
+    return x * (nn < norm ? 1.f : norm / nn);
+  };
+  const long long tid = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (VEC) {
+    const long long e = tid * 4;
+    if (e >= n) return;
+    const uint32_t r = (uint32_t)e - fd_div((uint32_t)e, fd) * fd.d;
+    const float4 x = dn_ld4<STREAM>(a + e);
+    const float4 s = *reinterpret_cast<const float4*>(sq + r);
+    dn_st4<STREAM>(t + e, make_float4(one(x.x, s.x), one(x.y, s.y), one(x.z, s.z), one(x.w, s.w)));
+  } else {
+    if (tid >= n) return;
+    const uint32_t r = (uint32_t)tid - fd_div((uint32_t)tid, fd) * fd.d;
+    t[tid] = one(a[tid], sq[r]);
+  }
+}
+
+extern "C" {
+
 int normlimit_by_axis(cudamat* mat, cudamat* target, int axis, float norm) {
   const int h = mat->size[0], w = mat->size[1];
   if (int e = check_axis_common(mat, target)) return e;
@@ -1106,9 +1135,26 @@ int normlimit_by_axis(cudamat* mat, cudamat* target, int axis, float norm) {
     return launch_cols(k_col_normlimit<64>, k_col_normlimit<256>, w, h, (const float*)mat->data_device,
                        target->data_device, w, h, norm);
   } else if (axis == 1) {
-    if (h <= 0) return 0;
-    hipLaunchKernelGGL(k_row_normlimit, dim3((h + 63) / 64), dim3(256), 0, dn_stream(), (const float*)mat->data_device,
-                       target->data_device, w, h, norm);
+    if (h <= 0 || w <= 0) return 0;
+    // two passes, each at streaming rate: the rows' sums of squares (the axis-1 reduction), then the
+    // scaling as a column-vector broadcast (4096 x 4096: 37 us; one workgroup per 64 rows walking
+    // all columns twice took 640 us).  The sums live in scratch slot 1, which nothing else of the
+    // matrix library uses (slot 0 holds the reduction's own partials).
+    float* sq = (float*)dn_scratch((size_t)h * sizeof(float), 1);
+    if (!sq) return CUDA_ERROR;
+    if (int e = rows_reduce<ROW_SQSUM>(mat->data_device, h, h, w, nullptr, sq, 1.f, 0.f)) return e;
+    const long long n = (long long)h * w;
+    if (n >= (1ll << 32)) return ERROR_UNSUPPORTED;    // 32-bit element index inside the kernel
+    const FastDiv fd = make_fastdiv((uint32_t)h);
+    const float* a = mat->data_device;
+    float* t = target->data_device;
+    if (h % 4 == 0 && dn_aligned16(a) && dn_aligned16(t)) {
+      const unsigned blocks = (unsigned)((n / 4 + 255) / 256);
+      if (n >= DN_STREAM_MIN_ELEMS) hipLaunchKernelGGL((k_scale_rows_to_norm<true, true>), dim3(blocks), dim3(256), 0, dn_stream(), a, (const float*)sq, t, n, fd, norm);
+      else hipLaunchKernelGGL((k_scale_rows_to_norm<true, false>), dim3(blocks), dim3(256), 0, dn_stream(), a, (const float*)sq, t, n, fd, norm);
+    } else {
+      hipLaunchKernelGGL((k_scale_rows_to_norm<false, false>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, dn_stream(), a, (const float*)sq, t, n, fd, norm);
+    }
     return dn_launch_status();
   }
   return ERROR_UNSUPPORTED;
@@ -1178,10 +1224,22 @@ int apply_softmax_grad(cudamat* mat, cudamat* labels, cudamat* target) {
   const long long n = (long long)h * w;
   if (n <= 0) return 0;
   if (n >= (1ll << 32)) return ERROR_UNSUPPORTED;
+  const FastDiv fd = make_fastdiv((uint32_t)h);
+  if (h % 4 == 0 && dn_aligned16(mat->data_device) && dn_aligned16(target->data_device)) {
+    const long long n4 = n / 4;
+    const unsigned blocks4 = (unsigned)((n4 + 255) / 256);
+    if (n >= DN_STREAM_MIN_ELEMS)
+      hipLaunchKernelGGL((k_softmax_grad4<true>), dim3(blocks4), dim3(256), 0, dn_stream(), (const float*)mat->data_device,
+                         (const float*)labels->data_device, target->data_device, n4, h, fd);
+    else
+      hipLaunchKernelGGL((k_softmax_grad4<false>), dim3(blocks4), dim3(256), 0, dn_stream(), (const float*)mat->data_device,
+                         (const float*)labels->data_device, target->data_device, n4, h, fd);
+    return dn_launch_status();
+  }
   long long blocks = (n + 255) / 256;
   if (blocks > dn_num_cus() * 32ll) blocks = dn_num_cus() * 32ll;
   hipLaunchKernelGGL(k_softmax_grad, dim3((unsigned)blocks), dim3(256), 0, dn_stream(), (const float*)mat->data_device,
-                     (const float*)labels->data_device, target->data_device, w, h, make_fastdiv((uint32_t)h));
+                     (const float*)labels->data_device, target->data_device, w, h, fd);
   return dn_launch_status();
 }
 

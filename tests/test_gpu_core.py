@@ -98,17 +98,18 @@ def test_row_slices(cm, rng):
         a.get_row_slice(5, 500)
 
 
-def test_select_set_swap_columns(cm, rng):
-    x = _rand(rng, (37, 20))
+@pytest.mark.parametrize("h", [37, 40, 1028])          # one row per lane, and four (row counts that are multiples of 4)
+def test_select_set_swap_columns(cm, rng, h):
+    x = _rand(rng, (h, 20))
     a = cm.CUDAMatrix(x)
     idx = np.array([[0, 19, -1, 5, 5, 25, -21]], dtype=np.float32)
-    t = cm.empty((37, idx.size))
+    t = cm.empty((h, idx.size))
     a.select_columns(cm.CUDAMatrix(idx), t)
     want = orc.select_columns(x, idx)
     got = t.asarray()
     assert np.array_equal(np.isnan(got), np.isnan(want))
     assert np.array_equal(got[~np.isnan(want)], want[~np.isnan(want)].astype(np.float32))
-    src = _rand(rng, (37, 3))
+    src = _rand(rng, (h, 3))
     sidx = np.array([[4, -1, 7]], dtype=np.float32)
     a.set_selected_columns(cm.CUDAMatrix(sidx), cm.CUDAMatrix(src))
     assert np.array_equal(a.asarray(), orc.set_selected_columns(x, src, sidx).astype(np.float32))
