@@ -195,6 +195,13 @@ k_rng_split(const unsigned int* mults, const unsigned long long* words, unsigned
 }
 
 // Box-Muller pairs: two draws give elements i and i + 12288 (cudamat_kernels.cu:125-143, 192-211).
+__device__ __forceinline__ void box_muller(float r1, float r2, float& a, float& b) {
+  const float T = 2.f * RNG_PI * r2;
+  const float R = sqrtf(-2.f * logf(r1));
+  a = R * cosf(T);
+  b = R * sinf(T);
+}
+
 __global__ void __launch_bounds__(RNG_BLOCK)
 k_rng_gauss(const unsigned int* mults, unsigned long long* words, const float* in, float* out, size_t n, float mult_by) {
   const unsigned int idx = blockIdx.x * RNG_BLOCK + threadIdx.x;
@@ -205,14 +212,85 @@ k_rng_gauss(const unsigned int* mults, unsigned long long* words, const float* i
     const float r1 = mwc_uniform(w);
     w = mwc_step(w, mult);
     const float r2 = mwc_uniform(w);
-    const float T = 2.f * RNG_PI * r2;
-    const float R = sqrtf(-2.f * logf(r1));
-    const float a = R * cosf(T), b = R * sinf(T);
+    float a, b;
+    box_muller(r1, r2, a, b);
     out[i] = in ? in[i] + mult_by * a : a;
     const size_t i2 = i + NUM_RND_STREAMS;
     if (i2 < n) out[i2] = in ? in[i2] + mult_by * b : b;
   }
   words[idx] = w;
+}
+
+// The same pairs on the split schedule.  A stream with an odd number of elements still
+// takes both draws of its last pair, so its draw count is rounded up to even; parts are
+// 2^chbits >= 16 draws, so no pair straddles two lanes.
+#define RNG_GAUSS_PAIRS 4
+__global__ void __launch_bounds__(RNG_SPLIT_BLOCK)
+k_rng_gauss_split(const unsigned int* mults, const unsigned long long* words, unsigned long long* next,
+                  const unsigned long long* table, const float* in, float* out, size_t n, int chbits, float mult_by) {
+  constexpr int blocks_per_part = NUM_RND_STREAMS / RNG_SPLIT_BLOCK;
+  constexpr int P = RNG_GAUSS_PAIRS;
+  const unsigned int part = blockIdx.x / blocks_per_part;
+  const unsigned int idx = (blockIdx.x % blocks_per_part) * RNG_SPLIT_BLOCK + threadIdx.x;
+  if (idx >= n) {
+    if (part == 0) next[idx] = words[idx];
+    return;
+  }
+  const unsigned long long elems = (n - idx + NUM_RND_STREAMS - 1) / NUM_RND_STREAMS;  // of this stream
+  const unsigned long long draws = (elems + 1) & ~1ull;
+  const unsigned long long d0 = (unsigned long long)part << chbits;
+  if (d0 >= draws) return;
+  const unsigned long long d1 = d0 + (1ull << chbits) < draws ? d0 + (1ull << chbits) : draws;
+  size_t i = (size_t)d0 * NUM_RND_STREAMS + idx;
+  unsigned long long d = d0;
+  // A batch of P pairs whose 2 P elements all exist; its reads are requested before the
+  // jump-ahead arithmetic and before the previous batch is consumed.
+  float x[2 * P];
+  auto fetch = [&](size_t at) {
+#pragma unroll
+    for (int k = 0; k < 2 * P; ++k) x[k] = in ? __builtin_nontemporal_load(in + at + (size_t)k * NUM_RND_STREAMS) : 0.f;
+  };
+  const bool full0 = d + 2 * P <= d1 && d + 2 * P <= elems;
+  if (full0) fetch(i);
+  const unsigned int mult = mults[idx];
+  unsigned long long w = words[idx];
+  for (unsigned int b = 0, pp = part; pp; ++b, pp >>= 1)
+    if (pp & 1u) w = mwc_montmul(w, table[(size_t)(chbits + b) * NUM_RND_STREAMS + idx], mult);
+  auto pair = [&](float& a, float& b) {
+    w = mwc_step(w, mult);
+    const float r1 = mwc_uniform(w);
+    w = mwc_step(w, mult);
+    box_muller(r1, mwc_uniform(w), a, b);
+  };
+  if (full0) {
+    for (;;) {
+      const size_t inext = i + (size_t)(2 * P) * NUM_RND_STREAMS;
+      const bool more = d + 4 * P <= d1 && d + 4 * P <= elems;
+      float y[2 * P];
+#pragma unroll
+      for (int k = 0; k < 2 * P; ++k) y[k] = x[k];
+      if (more) fetch(inext);
+#pragma unroll
+      for (int k = 0; k < P; ++k) {
+        float a, b;
+        pair(a, b);
+        const size_t at = i + (size_t)(2 * k) * NUM_RND_STREAMS;
+        __builtin_nontemporal_store(in ? y[2 * k] + mult_by * a : a, out + at);
+        __builtin_nontemporal_store(in ? y[2 * k + 1] + mult_by * b : b, out + at + NUM_RND_STREAMS);
+      }
+      d += 2 * P;
+      i = inext;
+      if (!more) break;
+    }
+  }
+  for (; d < d1; d += 2, i += 2 * (size_t)NUM_RND_STREAMS) {
+    float a, b;
+    pair(a, b);
+    out[i] = in ? in[i] + mult_by * a : a;
+    const size_t i2 = i + NUM_RND_STREAMS;
+    if (d + 1 < elems) out[i2] = in ? in[i2] + mult_by * b : b;
+  }
+  if (d1 == draws) next[idx] = w;
 }
 
 // Calls with at least RNG_SPLIT_MIN_DRAWS draws per stream are cut into parts of 2^c
@@ -293,6 +371,32 @@ int init_random(rnd_struct* rnd_state, int seed, char* cudamatpath) {
   return dn_launch_status();
 }
 
+// Gaussian ops: parts of 16 draws (8 pairs, each a logf, sqrtf, sinf and cosf) while that
+// gives at most RNG_GAUSS_PARTS parts per stream.  Recording keeps the serial kernel: the
+// split schedule flips dev_words on the host, which a recorded graph would not repeat.
+#define RNG_GAUSS_PARTS 256
+static int launch_gauss(rnd_struct* st, const float* in, float* out, size_t n, float mult_by) {
+  if (n == 0) return 0;
+  const size_t elems = (n + NUM_RND_STREAMS - 1) / NUM_RND_STREAMS;
+  const size_t draws = (elems + 1) & ~(size_t)1;   // of the busiest stream
+  int chbits = 4;
+  while (((draws + (1ull << chbits) - 1) >> chbits) > (size_t)RNG_GAUSS_PARTS) ++chbits;
+  const size_t parts = (draws + (1ull << chbits) - 1) >> chbits;
+  int top = 0;
+  while ((parts - 1) >> top) ++top;
+  if (draws < RNG_SPLIT_MIN_DRAWS || chbits + top > RNG_JUMP_BITS || dn_capturing()) {
+    hipLaunchKernelGGL(k_rng_gauss, dim3(RNG_BLOCKS), dim3(RNG_BLOCK), 0, dn_stream(), st->dev_mults, st->dev_words, in, out, n,
+                       mult_by);
+    return dn_launch_status();
+  }
+  unsigned long long* next = rng_other(st->dev_words);
+  const unsigned grid = (unsigned)(parts * (NUM_RND_STREAMS / RNG_SPLIT_BLOCK));
+  hipLaunchKernelGGL(k_rng_gauss_split, dim3(grid), dim3(RNG_SPLIT_BLOCK), 0, dn_stream(), st->dev_mults,
+                     (const unsigned long long*)st->dev_words, next, rng_table(st->dev_words), in, out, n, chbits, mult_by);
+  st->dev_words = next;
+  return dn_launch_status();
+}
+
 // A generator that init_random() never set up (null handle or null state pointers): the
 // reference would dereference it; here the call is refused.
 static inline bool rng_ready(const rnd_struct* st) { return st && st->dev_mults && st->dev_words; }
@@ -306,9 +410,7 @@ int fill_with_rand(rnd_struct* rnd_state, cudamat* mat) {
 int fill_with_randn(rnd_struct* rnd_state, cudamat* mat) {
   if (!mat->on_device) return ERROR_NOT_ON_DEVICE;
   if (!rng_ready(rnd_state)) return ERROR_GENERIC;
-  hipLaunchKernelGGL(k_rng_gauss, dim3(RNG_BLOCKS), dim3(RNG_BLOCK), 0, dn_stream(), rnd_state->dev_mults, rnd_state->dev_words,
-                     (const float*)nullptr, mat->data_device, (size_t)dn_len(mat), 1.f);
-  return dn_launch_status();
+  return launch_gauss(rnd_state, nullptr, mat->data_device, (size_t)dn_len(mat), 1.f);
 }
 
 // The sampling wrappers check dims before residency (cudamat.cu:469-572).
@@ -331,9 +433,7 @@ int sample_gaussian(rnd_struct* rnd_state, cudamat* mat, cudamat* target, float 
   if (mat->size[0] != target->size[0] || mat->size[1] != target->size[1]) return ERROR_INCOMPATIBLE_DIMENSIONS;
   if (!mat->on_device || !target->on_device) return ERROR_NOT_ON_DEVICE;
   if (!rng_ready(rnd_state)) return ERROR_GENERIC;
-  hipLaunchKernelGGL(k_rng_gauss, dim3(RNG_BLOCKS), dim3(RNG_BLOCK), 0, dn_stream(), rnd_state->dev_mults, rnd_state->dev_words,
-                     (const float*)mat->data_device, target->data_device, (size_t)dn_len(mat), mult);
-  return dn_launch_status();
+  return launch_gauss(rnd_state, mat->data_device, target->data_device, (size_t)dn_len(mat), mult);
 }
 
 int dropout(rnd_struct* rnd_state, cudamat* mat, float dropprob, float val) {

@@ -105,7 +105,10 @@ def test_deepnet_dropout_mask_sequence(cm, mults):
     assert np.array_equal(s.asarray(), want)
 
 
-@pytest.mark.parametrize("n", [1, N, N + 1, 2 * N, 2 * N + 3, 5 * N + 17])
+# from 31 elements per stream on, lanes share a stream (parts of whole pairs); odd element
+# counts leave a last pair with one element that still takes two draws
+@pytest.mark.parametrize("n", [1, N, N + 1, 2 * N, 2 * N + 3, 5 * N + 17, 30 * N + 1, 31 * N + 7, 33 * N, 40 * N + 5,
+                               257 * N + 4321])
 def test_fill_with_randn_matches_box_muller_of_exact_uniforms(cm, mults, n):
     cm.CUDAMatrix.init_random(9)
     host = mwc.MWC(mults, 9)
@@ -131,6 +134,13 @@ def test_randn_moments_and_sample_gaussian(cm, mults):
     b.sample_gaussian(mult=0.5, target=t)
     want = 2.0 + 0.5 * host.randn(base.size).reshape(base.shape, order='F')
     assert np.max(np.abs(t.asarray() - want)) < 2e-5
+    # the same on the schedule that shares a stream among lanes, ragged at the end
+    big = np.asarray(np.arange(1031 * 613) % 17, dtype=np.float32).reshape((1031, 613), order='F')
+    b, t = cm.CUDAMatrix(big), cm.empty(big.shape)
+    b.sample_gaussian(mult=0.25, target=t)
+    want = big + 0.25 * host.randn(big.size).reshape(big.shape, order='F')
+    assert np.max(np.abs(t.asarray() - want)) < 2e-5
+    assert np.array_equal(_device_words(cm), host.words)
 
 
 def test_perturb_ops(cm, mults, rng):
