@@ -11,6 +11,7 @@
 #include "common.h"
 #include <float.h>
 #include <math.h>
+#include <string.h>
 
 
 // ------------------------------------------------------------------ column walkers
@@ -908,51 +909,157 @@ int dn_gemv_rows(const float* M, int ld, int h, int w, const float* x, float* y,
 
 // ------------------------------------------------------------------ flat dot / norm
 
-// partial[block] = sum over a grid-stride slice of a[i]*b[i], accumulated in
-// fp32 per lane and in fp64 across lanes and workgroups.
-__global__ void __launch_bounds__(256) k_dot_partial(const float* a, const float* b, long long n, double* partial) {
+// Sum of a[i] * b[i] over everything, returned to the host.  One launch: a workgroup sums
+// a grid-stride slice (fp32 per lane over four independent chains, fp64 across lanes and
+// workgroups; 16-byte loads when VEC, four of each operand in flight), publishes its partial
+// sum and counts itself in; the one that arrives last adds the partials in block order, so
+// the result does not depend on the order of arrival, and writes {value, tag} as one 8-byte
+// word into pinned host memory.  The counters (one of groups, then one per group of
+// workgroups) return to zero for the next launch.
+#define DOT_U 4
+#define DOT_GROUP 32
+#define DOT_COUNTER_PITCH 64   // words between two counters: every counter in a memory line of its own
+template <bool VEC, bool STREAM, bool SAME>
+__global__ void __launch_bounds__(256)
+k_dot_one(const float* a, const float* b, long long n, double* partial, unsigned* counter,
+          unsigned long long* result, unsigned tag, int take_sqrt) {
   __shared__ double lds[4];
+  __shared__ int s_last;
   const long long stride = (long long)gridDim.x * 256;
-  float s0 = 0.f, s1 = 0.f;
-  long long i = (long long)blockIdx.x * 256 + threadIdx.x;
-  for (; i + stride < n; i += 2 * stride) {
-    s0 += a[i] * b[i];
-    s1 += a[i + stride] * b[i + stride];
+  float s[DOT_U] = {0.f, 0.f, 0.f, 0.f};
+  if (VEC) {
+    const long long n4 = n >> 2;
+    for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n4; i += DOT_U * stride) {
+      float4 x[DOT_U], y[DOT_U];
+#pragma unroll
+      for (int u = 0; u < DOT_U; ++u) {
+        const long long j = i + u * stride;
+        const bool ok = j < n4;
+        x[u] = ok ? dn_ld4<STREAM>(a + 4 * j) : make_float4(0.f, 0.f, 0.f, 0.f);
+        y[u] = SAME ? x[u] : ok ? dn_ld4<STREAM>(b + 4 * j) : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+#pragma unroll
+      for (int u = 0; u < DOT_U; ++u) s[u] += (x[u].x * y[u].x + x[u].y * y[u].y) + (x[u].z * y[u].z + x[u].w * y[u].w);
+    }
+    if (blockIdx.x == 0 && (long long)threadIdx.x < n - 4 * n4) s[0] += a[4 * n4 + threadIdx.x] * b[4 * n4 + threadIdx.x];
+  } else {
+    for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += DOT_U * stride) {
+      float x[DOT_U], y[DOT_U];
+#pragma unroll
+      for (int u = 0; u < DOT_U; ++u) {
+        const long long j = i + u * stride;
+        x[u] = j < n ? a[j] : 0.f;
+        y[u] = SAME ? x[u] : j < n ? b[j] : 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < DOT_U; ++u) s[u] += x[u] * y[u];
+    }
   }
-  if (i < n) s0 += a[i] * b[i];
-  double s = wave_sum_d((double)s0 + (double)s1);
-  if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = s;
+  double t = wave_sum_d(((double)s[0] + (double)s[1]) + ((double)s[2] + (double)s[3]));
+  if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = t;
   __syncthreads();
-  if (threadIdx.x == 0) partial[blockIdx.x] = (lds[0] + lds[1]) + (lds[2] + lds[3]);
-}
-
-__global__ void __launch_bounds__(256) k_dot_finish(const double* partial, int nblocks, float* out, int take_sqrt) {
-  __shared__ double lds[4];
-  double s = 0.0;
-  for (int i = threadIdx.x; i < nblocks; i += 256) s += partial[i];
-  s = wave_sum_d(s);
-  if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = s;
-  __syncthreads();
+  const int nblocks = gridDim.x;
   if (threadIdx.x == 0) {
-    const double t = (lds[0] + lds[1]) + (lds[2] + lds[3]);
-    out[0] = (float)(take_sqrt ? sqrt(t) : t);
+    t = (lds[0] + lds[1]) + (lds[2] + lds[3]);
+    if (nblocks == 1) {
+      s_last = 1;
+      lds[0] = t;
+    } else {
+      __hip_atomic_store(partial + blockIdx.x, t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __builtin_amdgcn_s_waitcnt(0);   // the store has been acknowledged
+      // Arrivals at one address are served one after the other (about 15 ns each), so the
+      // workgroups count themselves in by groups of DOT_GROUP and only the last of a group
+      // goes on to the counter of groups.
+      const int g = blockIdx.x / DOT_GROUP;
+      const int ng = (nblocks + DOT_GROUP - 1) / DOT_GROUP;
+      const int gsize = nblocks - g * DOT_GROUP < DOT_GROUP ? nblocks - g * DOT_GROUP : DOT_GROUP;
+      int last = 0;
+      if (__hip_atomic_fetch_add(counter + DOT_COUNTER_PITCH * (1 + g), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (unsigned)gsize - 1u) {
+        __hip_atomic_store(counter + DOT_COUNTER_PITCH * (1 + g), 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (__hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (unsigned)ng - 1u) {
+          __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          last = 1;
+        }
+      }
+      s_last = last;
+    }
+  }
+  __syncthreads();
+  if (!s_last) return;
+  if (nblocks > 1) {
+    // (atomic loads would be served one at a time; after the fence plain loads see what the
+    // other workgroups' acknowledged stores left at the device's point of coherence)
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    double p = 0.0;
+    for (int i = threadIdx.x; i < nblocks; i += 256) p += partial[i];
+    p = wave_sum_d(p);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = p;
+    __syncthreads();
+    if (threadIdx.x == 0) lds[0] = (lds[0] + lds[1]) + (lds[2] + lds[3]);
+  }
+  if (threadIdx.x == 0) {
+    const float v = (float)(take_sqrt ? sqrt(lds[0]) : lds[0]);
+    __hip_atomic_store(result, ((unsigned long long)tag << 32) | __float_as_uint(v), __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_SYSTEM);
   }
 }
 
+// The host's side of the result word: pinned memory that the kernel writes directly, so a
+// scalar result costs no copy call.  The host polls the word for this call's tag for a
+// while (a result of a short kernel arrives within microseconds) and otherwise waits for
+// the stream.
+static unsigned long long* g_result_host = nullptr;
+static unsigned long long* g_result_dev = nullptr;
+static unsigned g_result_tag = 0;
+
+static bool result_word() {
+  if (g_result_host) return true;
+  void* h = nullptr;
+  void* d = nullptr;
+  if (hipHostMalloc(&h, 64, hipHostMallocDefault) != hipSuccess) { hipGetLastError(); return false; }
+  if (hipHostGetDevicePointer(&d, h, 0) != hipSuccess) { hipGetLastError(); hipHostFree(h); return false; }
+  g_result_host = (unsigned long long*)h;
+  g_result_dev = (unsigned long long*)d;
+  *g_result_host = 0ull;
+  return true;
+}
+
+#define DOT_POLLS (1 << 16)
 static int flat_dot(const float* a, const float* b, long long n, int take_sqrt, float* result) {
   *result = 0.f;
   if (dn_capturing()) return ERROR_UNSUPPORTED;        // the result is read back: nothing to record
   if (n <= 0) return 0;
-  long long nb = (n + 2047) / 2048;
-  const long long cap = (long long)dn_num_cus() * 8;
+  const bool vec = dn_aligned16(a) && dn_aligned16(b) && n >= 1024;
+  long long nb = (n + (vec ? 4095 : 1023)) / (vec ? 4096 : 1024);
+  const long long cap = (long long)dn_num_cus() * 2;   // (more workgroups: more arrivals; 4 per CU cost 2 us at 4096 x 4096)
   if (nb > cap) nb = cap;
-  char* ws = (char*)dn_scratch((size_t)nb * sizeof(double) + 16);
-  if (!ws) return CUDA_ERROR;
-  double* partial = (double*)ws;
-  float* out = (float*)(ws + (size_t)nb * sizeof(double));
-  hipLaunchKernelGGL(k_dot_partial, dim3((unsigned)nb), dim3(256), 0, dn_stream(), a, b, n, partial);
-  hipLaunchKernelGGL(k_dot_finish, dim3(1), dim3(256), 0, dn_stream(), partial, (int)nb, out, take_sqrt);
-  if (hipMemcpy(result, out, sizeof(float), hipMemcpyDeviceToHost) != hipSuccess) return CUDA_ERROR;
+  double* partial = (double*)dn_scratch((size_t)nb * sizeof(double));
+  unsigned* counter = dn_zero_words(DOT_COUNTER_PITCH * (1 + (int)((nb + DOT_GROUP - 1) / DOT_GROUP)));
+  if (!partial || !counter || !result_word()) return CUDA_ERROR;
+  const unsigned tag = ++g_result_tag ? g_result_tag : ++g_result_tag;   // never 0, the word's first content
+  const dim3 grid((unsigned)nb), block(256);
+#define DOT_GO(VEC, STREAM, SAME) \
+  hipLaunchKernelGGL((k_dot_one<VEC, STREAM, SAME>), grid, block, 0, dn_stream(), a, b, n, partial, counter, g_result_dev, tag, take_sqrt)
+#define DOT_SAME(VEC, STREAM) do { if (a == b) DOT_GO(VEC, STREAM, true); else DOT_GO(VEC, STREAM, false); } while (0)
+  if (vec && n >= DN_STREAM_MIN_ELEMS) DOT_SAME(true, true);
+  else if (vec) DOT_SAME(true, false);
+  else DOT_SAME(false, false);
+#undef DOT_SAME
+#undef DOT_GO
+  if (hipGetLastError() != hipSuccess) return CUDA_ERROR;
+  unsigned long long word = 0;
+  for (int i = 0; i < DOT_POLLS; ++i) {
+    word = __atomic_load_n(g_result_host, __ATOMIC_ACQUIRE);
+    if ((unsigned)(word >> 32) == tag) break;
+  }
+  if ((unsigned)(word >> 32) != tag) {
+    if (hipStreamSynchronize(dn_stream()) != hipSuccess) return CUDA_ERROR;
+    word = __atomic_load_n(g_result_host, __ATOMIC_ACQUIRE);
+    if ((unsigned)(word >> 32) != tag) return CUDA_ERROR;
+  }
+  const unsigned bits = (unsigned)word;
+  memcpy(result, &bits, sizeof(float));
   return 0;
 }
 

@@ -155,12 +155,21 @@ def test_softmax_loss_helpers(cm, rng):
 
 
 def test_vdot_and_euclid_norm(cm, rng):
-    for shape in [(1, 1), (37, 53), (1000, 999)]:
+    # one workgroup, the 4-byte path (< 1024 elements), 16-byte groups with a tail, many
+    # workgroups with several trips each
+    for shape in [(1, 1), (37, 53), (1023, 1), (1024, 1), (1000, 999), (2051, 2049)]:
         x, y = _rand(rng, shape), _rand(rng, shape)
         a, b = cm.CUDAMatrix(x), cm.CUDAMatrix(y)
         scale = np.abs(x.astype(np.float64) * y).sum()
-        assert abs(cm.vdot(a, b) - orc.vdot(x, y)) / scale < REL
+        first = cm.vdot(a, b)
+        assert abs(first - orc.vdot(x, y)) / scale < REL
         assert abs(a.euclid_norm() - orc.euclid_norm(x)) / orc.euclid_norm(x) < REL
+        assert cm.vdot(a, b) == first          # the order of the sum is fixed
+    # operands that start 20 bytes into an allocation
+    x, y = _rand(rng, (5, 400)), _rand(rng, (5, 400))
+    a, b = cm.CUDAMatrix(x).get_col_slice(1, 400), cm.CUDAMatrix(y).get_col_slice(1, 400)
+    scale = np.abs(x[:, 1:].astype(np.float64) * y[:, 1:]).sum()
+    assert abs(cm.vdot(a, b) - orc.vdot(x[:, 1:], y[:, 1:])) / scale < REL
     with pytest.raises(cm.CUDAMatException, match="Incompatible matrix dimensions"):
         cm.vdot(a, cm.CUDAMatrix(_rand(rng, (3, 3))))
 
