@@ -803,21 +803,21 @@ __global__ void __launch_bounds__(256, (MODE == CONV_DOWNM && WM * WN <= 2 ? 4 :
 // Weight gradients of a layer with at most 32*RT filters per group and at most 32*CT
 // patch columns (a first layer over RGB: 64 x 75).  Both operands are contiguous along
 // the images, which is the reduction index here, so a chunk of (one module, 64 images)
-// is read row by row in whole 256-byte runs and kept in LDS as [row][image] with an odd
-// pitch: an MFMA operand (lane = row, two neighbouring images) is then one conflict-free
-// LDS read.  The four wavefronts each hold the whole RT x CT block of accumulators and
+// is read row by row in whole 256-byte runs and kept in LDS as [row][image] with a pitch
+// of 68: the 16-byte groups go to LDS as they came, and a lane's operands of four MFMA
+// steps (lane = row, four neighbouring images) are one conflict-free 16-byte LDS read.  The four wavefronts each hold the whole RT x CT block of accumulators and
 // split the 32 steps of a chunk between them (no columns are padded to a wavefront
 // grid, one barrier per chunk); they are summed through LDS once, at the end, and every
 // workgroup writes one partial block for k_conv_outp_finish.
 template <int RT, int CT>
 __global__ void __launch_bounds__(256, 1) k_conv_outp_small(ConvArgs p) {
   constexpr unsigned FAR = 0x80000000u;  // beyond any buffer here: sizes are below 2^31 bytes
-  constexpr int PITCH = 65;              // 64 images + 1: rows land on different banks
+  constexpr int PITCH = 68;              // 64 images + 4: 16-byte groups stay aligned, 8 neighbouring rows on different banks
   constexpr int NAV = RT * 2, NBV = CT * 2;   // 16-byte loads per lane and chunk (32 rows x 16 = 512 = 2 x 256)
   // one LDS arena: the two operand tiles (double buffered) while chunks are multiplied,
   // the four wavefronts' accumulators when they are summed at the end
   constexpr int TILES = 2 * 32 * (RT + CT) * PITCH, SUMS = 4 * 16 * RT * CT * 64;
-  __shared__ float arena[TILES > SUMS ? TILES : SUMS];
+  __shared__ __attribute__((aligned(16))) float arena[TILES > SUMS ? TILES : SUMS];
   float (*As)[32 * RT][PITCH] = reinterpret_cast<float (*)[32 * RT][PITCH]>(arena);
   float (*Bs)[32 * CT][PITCH] = reinterpret_cast<float (*)[32 * CT][PITCH]>(arena + 2 * 32 * RT * PITCH);
   const int tid = threadIdx.x, lane = tid & 63, li = lane & 31, lk = lane >> 5;
@@ -888,21 +888,22 @@ __global__ void __launch_bounds__(256, 1) k_conv_outp_small(ConvArgs p) {
   auto multiply = [&](auto set_tag, auto stash_tag, int buf, int next) __attribute__((always_inline)) {
     constexpr int SET = decltype(set_tag)::value;
     constexpr bool STASH = decltype(stash_tag)::value;
-    constexpr int NW = 4 * (NAV + NBV);                 // LDS writes of a lane per chunk
+    constexpr int NW = NAV + NBV;                       // 16-byte LDS writes of a lane per chunk
     constexpr int WPS = (NW + 7) / 8;                   // ... per step
-    float av[8][RT], bv[8][CT];
-    auto read = [&](int t) __attribute__((always_inline)) {
-      const int kk = 2 * (8 * wv + t) + lk;
+    // Step t of this wavefront multiplies image 16*wv + 8*(t/4) + 4*lk + t%4 of the chunk (the
+    // sum over images takes them in any order), so a lane's operands of four steps are
+    // one 16-byte LDS read per row block.
+    f32x4 av[2][RT], bv[2][CT];
+    auto read = [&](int h) __attribute__((always_inline)) {
+      const int kk = 16 * wv + 8 * h + 4 * lk;
 #pragma unroll
-      for (int i = 0; i < RT; ++i) av[t][i] = As[buf][i * 32 + li][kk];
+      for (int i = 0; i < RT; ++i) av[h][i] = *reinterpret_cast<const f32x4*>(&As[buf][i * 32 + li][kk]);
 #pragma unroll
-      for (int j = 0; j < CT; ++j) bv[t][j] = Bs[buf][j * 32 + li][kk];
+      for (int j = 0; j < CT; ++j) bv[h][j] = *reinterpret_cast<const f32x4*>(&Bs[buf][j * 32 + li][kk]);
     };
-#pragma unroll
-    for (int t = 0; t < 4; ++t) read(t);
+    read(0);
     __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int t = 4; t < 8; ++t) read(t);
+    read(1);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int t = 0; t < 8; ++t) {
@@ -910,14 +911,13 @@ __global__ void __launch_bounds__(256, 1) k_conv_outp_small(ConvArgs p) {
       for (int j = 0; j < CT; ++j)
 #pragma unroll
         for (int i = 0; i < RT; ++i)
-          acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[t][j], av[t][i], acc[j][i], 0, 0, 0);
+          acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[t >> 2][j][t & 3], av[t >> 2][i][t & 3], acc[j][i], 0, 0, 0);
       if (t == 0 && next >= 0) fetch(std::integral_constant<int, SET ^ 1>(), next);
       if (STASH) {
 #pragma unroll
-        for (int w = t * WPS; w < (t + 1) * WPS && w < NW; ++w) {
-          const int u = w >> 2, jj = w & 3;
-          if (u < NAV) As[buf ^ 1][r16 + 16 * u][n4 + jj] = ra[SET][u][jj];
-          else Bs[buf ^ 1][r16 + 16 * (u - NAV)][n4 + jj] = rb[SET][u - NAV][jj];
+        for (int u = t * WPS; u < (t + 1) * WPS && u < NW; ++u) {
+          if (u < NAV) *reinterpret_cast<f32x4*>(&As[buf ^ 1][r16 + 16 * u][n4]) = ra[SET][u];
+          else *reinterpret_cast<f32x4*>(&Bs[buf ^ 1][r16 + 16 * (u - NAV)][n4]) = rb[SET][u - NAV];
         }
       }
       __builtin_amdgcn_sched_barrier(0);
@@ -926,13 +926,9 @@ __global__ void __launch_bounds__(256, 1) k_conv_outp_small(ConvArgs p) {
   auto stash = [&](auto set_tag, int buf) __attribute__((always_inline)) {
     constexpr int SET = decltype(set_tag)::value;
 #pragma unroll
-    for (int u = 0; u < NAV; ++u)
+    for (int u = 0; u < NAV; ++u) *reinterpret_cast<f32x4*>(&As[buf][r16 + 16 * u][n4]) = ra[SET][u];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) As[buf][r16 + 16 * u][n4 + j] = ra[SET][u][j];
-#pragma unroll
-    for (int u = 0; u < NBV; ++u)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) Bs[buf][r16 + 16 * u][n4 + j] = rb[SET][u][j];
+    for (int u = 0; u < NBV; ++u) *reinterpret_cast<f32x4*>(&Bs[buf][r16 + 16 * u][n4]) = rb[SET][u];
   };
   const int my_chunks = (int)blockIdx.x < p.m_count ? ((p.m_count - 1 - (int)blockIdx.x) / (int)gridDim.x + 1) * halves : 0;
   // While chunk i is multiplied, chunk i+1 (asked for one trip ago) is written to LDS and
