@@ -502,7 +502,7 @@ static int dot_bias_act_impl(rnd_struct* rnd, cudamat* mat1, cudamat* mat2, cuda
     err = dn_gemm_fused(mat1->is_trans != 0, mat2->is_trans != 0, m, n, k, mat1->data_device, mat1->size[0],
                         mat2->data_device, mat2->size[0], target->data_device, m, bias ? bias->data_device : nullptr,
                         act, &fused, try_sample ? &smp : nullptr, &sampled);
-    if (!err && sampled) rnd->dev_words = rng_other(rnd->dev_words);
+    if (!err && sampled) rng_publish(rnd);
   }
   if (err) return err;
   if (!fused) {

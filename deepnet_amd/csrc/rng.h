@@ -27,6 +27,12 @@ static inline unsigned long long* rng_other(unsigned long long* w) {
   return reinterpret_cast<unsigned long long*>(reinterpret_cast<uintptr_t>(w) ^ (uintptr_t)RNG_BUF_BYTES);
 }
 
+// A kernel has left the generator's next state in rng_other(st->dev_words): make it the
+// current one.  Normally the pointer is flipped; once a recorded graph refers to the current
+// buffer (rng.hip pins it) the words are copied back into it instead, so that replays and
+// eager calls keep drawing from one sequence.
+void rng_publish(rnd_struct* st);
+
 // What a product that also draws a Bernoulli sample of its output needs from the generator:
 // the sample's buffer, the multipliers, the current words (read only) and the buffer that
 // receives the words after the call.

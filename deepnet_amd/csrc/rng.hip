@@ -305,11 +305,47 @@ k_rng_gauss_split(const unsigned int* mults, const unsigned long long* words, un
 #define RNG_SPLIT_PARTS 24
 #define RNG_SPLIT_SRC_PARTS 96
 
+// Word buffers that a recorded graph refers to: its serial kernels carry the buffer's address,
+// so from then on the generator's state has to stay in that buffer.
+#define RNG_MAX_PINNED 16
+static unsigned long long* g_rng_pinned[RNG_MAX_PINNED];
+static int g_rng_npinned = 0;
+
+static bool rng_is_pinned(const unsigned long long* w) {
+  for (int i = 0; i < g_rng_npinned; ++i)
+    if (g_rng_pinned[i] == w) return true;
+  return false;
+}
+
+// Called before a kernel that reads and writes st->dev_words in place is launched; false
+// when the launch is being recorded and the buffer cannot be remembered any more.
+static bool rng_pin_if_recording(rnd_struct* st) {
+  if (!dn_capturing() || rng_is_pinned(st->dev_words)) return true;
+  if (g_rng_npinned == RNG_MAX_PINNED) return false;
+  g_rng_pinned[g_rng_npinned++] = st->dev_words;
+  return true;
+}
+
+__global__ void __launch_bounds__(256) k_rng_copy_words(const unsigned long long* from, unsigned long long* to) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < NUM_RND_STREAMS) to[i] = from[i];
+}
+
+void rng_publish(rnd_struct* st) {
+  unsigned long long* next = rng_other(st->dev_words);
+  if (rng_is_pinned(st->dev_words))
+    hipLaunchKernelGGL(k_rng_copy_words, dim3(NUM_RND_STREAMS / 256), dim3(256), 0, dn_stream(), (const unsigned long long*)next,
+                       st->dev_words);
+  else
+    st->dev_words = next;
+}
+
 template <class Op>
 static int launch_rng(rnd_struct* st, size_t n, Op op) {
   if (n == 0) return 0;
   const size_t draws = (n + NUM_RND_STREAMS - 1) / NUM_RND_STREAMS;
   if (draws < RNG_SPLIT_MIN_DRAWS) {
+    if (!rng_pin_if_recording(st)) return ERROR_UNSUPPORTED;
     hipLaunchKernelGGL((k_rng_serial<Op>), dim3(RNG_BLOCKS), dim3(RNG_BLOCK), 0, dn_stream(), st->dev_mults, st->dev_words, n,
                        op);
     return dn_launch_status();
@@ -321,12 +357,13 @@ static int launch_rng(rnd_struct* st, size_t n, Op op) {
   int top = 0;
   while ((parts - 1) >> top) ++top;
   if (chbits + top > RNG_JUMP_BITS) {
+    if (!rng_pin_if_recording(st)) return ERROR_UNSUPPORTED;
     hipLaunchKernelGGL((k_rng_serial<Op>), dim3(RNG_BLOCKS), dim3(RNG_BLOCK), 0, dn_stream(), st->dev_mults, st->dev_words, n,
                        op);
     return dn_launch_status();
   }
-  // (the split schedule publishes the new state by flipping dev_words on the host, which a
-  // recorded graph would not repeat)
+  // (the split schedule publishes the new state from the host, which a recorded graph would
+  // not repeat)
   if (dn_capturing()) return ERROR_UNSUPPORTED;
   unsigned long long* next = rng_other(st->dev_words);
   const unsigned grid = (unsigned)(parts * (NUM_RND_STREAMS / RNG_SPLIT_BLOCK));
@@ -336,7 +373,7 @@ static int launch_rng(rnd_struct* st, size_t n, Op op) {
   else
     hipLaunchKernelGGL((k_rng_split<Op, 4>), dim3(grid), dim3(RNG_SPLIT_BLOCK), 0, dn_stream(), st->dev_mults,
                        (const unsigned long long*)st->dev_words, next, rng_table(st->dev_words), n, chbits, op);
-  st->dev_words = next;
+  rng_publish(st);
   return dn_launch_status();
 }
 
@@ -385,6 +422,7 @@ static int launch_gauss(rnd_struct* st, const float* in, float* out, size_t n, f
   int top = 0;
   while ((parts - 1) >> top) ++top;
   if (draws < RNG_SPLIT_MIN_DRAWS || chbits + top > RNG_JUMP_BITS || dn_capturing()) {
+    if (!rng_pin_if_recording(st)) return ERROR_UNSUPPORTED;
     hipLaunchKernelGGL(k_rng_gauss, dim3(RNG_BLOCKS), dim3(RNG_BLOCK), 0, dn_stream(), st->dev_mults, st->dev_words, in, out, n,
                        mult_by);
     return dn_launch_status();
@@ -393,7 +431,7 @@ static int launch_gauss(rnd_struct* st, const float* in, float* out, size_t n, f
   const unsigned grid = (unsigned)(parts * (NUM_RND_STREAMS / RNG_SPLIT_BLOCK));
   hipLaunchKernelGGL(k_rng_gauss_split, dim3(grid), dim3(RNG_SPLIT_BLOCK), 0, dn_stream(), st->dev_mults,
                      (const unsigned long long*)st->dev_words, next, rng_table(st->dev_words), in, out, n, chbits, mult_by);
-  st->dev_words = next;
+  rng_publish(st);
   return dn_launch_status();
 }
 

@@ -206,3 +206,31 @@ def test_sampler_error_codes(cm, rng):
     host_only = cm.CUDAMatrix(np.zeros((4, 4), dtype=np.float32), copy_to_device=False)
     with pytest.raises(cm.CUDAMatException, match="not in device memory"):
         host_only.fill_with_rand()
+
+
+def test_recorded_draws_and_eager_calls_share_one_sequence(cm, mults):
+    """A recorded graph carries the address of the state words it draws from.  Calls that
+    move the state to the other buffer (large matrices, the sample of dot_bias_act) must
+    leave it where the graph finds it: replays and eager calls interleave like eager calls."""
+    cm.CUDAMatrix.init_random(21)
+    host = mwc.MWC(mults, 21)
+    small, big = cm.empty((300, 40)), cm.empty((1024, 512))
+    small.fill_with_rand(); host.uniform(small.shape[0] * small.shape[1])
+    with cm.Graph() as g:
+        small.fill_with_rand()
+    for step in range(3):
+        g.launch()
+        want = host.uniform(small.shape[0] * small.shape[1])
+        assert np.array_equal(small.asarray().ravel(order='F').view(np.uint32), want.view(np.uint32)), step
+        big.fill_with_rand()                                  # the split schedule
+        want = host.uniform(big.shape[0] * big.shape[1])
+        assert np.array_equal(big.asarray().ravel(order='F').view(np.uint32), want.view(np.uint32)), step
+        # a product that draws the sample of its own output
+        w = cm.CUDAMatrix(np.zeros((64, 96), dtype=np.float32)); v = cm.CUDAMatrix(np.ones((64, 100), dtype=np.float32))
+        h, hs = cm.empty((96, 100)), cm.empty((96, 100))
+        cm.dot_bias_act(w.T, v, None, target=h, act='sigmoid', sample=hs)
+        u = host.uniform(96 * 100).reshape((96, 100), order='F')
+        assert np.array_equal(hs.asarray(), (u < np.float32(0.5)).astype(np.float32)), step
+        big.fill_with_randn(); host.randn(big.shape[0] * big.shape[1])
+    assert np.array_equal(_device_words(cm), host.words)
+    g.free()
