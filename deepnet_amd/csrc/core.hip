@@ -35,6 +35,7 @@ bool dn_capturing() { return g_capturing; }
 // for operands padded to a multiple of 16 filters.
 static void* g_scratch[4] = {nullptr, nullptr, nullptr, nullptr};
 static size_t g_scratch_bytes[4] = {0, 0, 0, 0};
+static bool g_scratch_recorded[4] = {false, false, false, false};
 
 void* dn_scratch(size_t bytes, int slot) {
   if (bytes > g_scratch_bytes[slot]) {
@@ -42,7 +43,10 @@ void* dn_scratch(size_t bytes, int slot) {
 
     if (g_scratch[slot]) {
       hipDeviceSynchronize();
-      hipFree(g_scratch[slot]);
+      // A block that was handed out while a graph was being recorded stays allocated for
+      // the life of the process: the graph's kernels carry its address.
+      if (!g_scratch_recorded[slot]) hipFree(g_scratch[slot]);
+      g_scratch_recorded[slot] = false;
     }
     size_t want = bytes < (1u << 20) ? (1u << 20) : bytes;
     if (hipMalloc(&g_scratch[slot], want) != hipSuccess) {
@@ -53,6 +57,7 @@ void* dn_scratch(size_t bytes, int slot) {
     }
     g_scratch_bytes[slot] = want;
   }
+  if (g_capturing) g_scratch_recorded[slot] = true;
   return g_scratch[slot];
 }
 
@@ -60,16 +65,24 @@ void* dn_scratch(size_t bytes, int slot) {
 // counters that their kernels return to zero); allocated and cleared on first use.
 static unsigned* g_zero_words = nullptr;
 static int g_zero_words_n = 0;
+static bool g_zero_words_recorded = false;
 
 unsigned* dn_zero_words(int n) {
   if (n > g_zero_words_n) {
     if (g_capturing) return nullptr;
-    if (g_zero_words) { hipDeviceSynchronize(); hipFree(g_zero_words); g_zero_words = nullptr; g_zero_words_n = 0; }
+    if (g_zero_words) {
+      hipDeviceSynchronize();
+      if (!g_zero_words_recorded) hipFree(g_zero_words);   // (as for the scratch blocks)
+      g_zero_words_recorded = false;
+      g_zero_words = nullptr;
+      g_zero_words_n = 0;
+    }
     const int want = n < 16384 ? 16384 : n;
     if (hipMalloc(&g_zero_words, (size_t)want * sizeof(unsigned)) != hipSuccess) { g_zero_words = nullptr; hipGetLastError(); return nullptr; }
     if (hipMemset(g_zero_words, 0, (size_t)want * sizeof(unsigned)) != hipSuccess) return nullptr;
     g_zero_words_n = want;
   }
+  if (g_capturing) g_zero_words_recorded = true;
   return g_zero_words;
 }
 

@@ -756,6 +756,9 @@ def empty(shape):
 _ones_views = {}
 
 
+_ones_retired = []
+
+
 def _ones(n, trans=False):
     """View of the first n entries of the device vector of ones (grown on demand), as a
     column or, with trans, as a row.  Views are kept per (n, trans): the sums call this
@@ -763,7 +766,10 @@ def _ones(n, trans=False):
     if not isinstance(CUDAMatrix.ones, CUDAMatrix):
         raise CUDAMatException("cublas_init() has not been called.")
     if n > CUDAMatrix.ones.shape[0]:
-        CUDAMatrix.ones = CUDAMatrix(np.ones((n, 1), dtype=np.float32, order='F'))
+        # (a recorded graph may still sum with the old vector: it is kept, and the vector at
+        # least doubles, so all the kept ones together are smaller than the current one)
+        _ones_retired.append(CUDAMatrix.ones)
+        CUDAMatrix.ones = CUDAMatrix(np.ones((max(n, 2 * CUDAMatrix.ones.shape[0]), 1), dtype=np.float32, order='F'))
         _ones_views.clear()
     key = (n, trans)
     view = _ones_views.get(key)
@@ -1069,6 +1075,7 @@ init = cublas_init
 def cublas_shutdown():
     CUDAMatrix.ones = 0
     _ones_views.clear()
+    del _ones_retired[:]
     _cudamat.cublas_shutdown()
 
 

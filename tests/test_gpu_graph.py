@@ -143,3 +143,30 @@ def test_what_cannot_be_recorded_raises(cm):
     g.launch(); g.launch()
     assert np.array_equal(a.asarray(), np.full((8, 8), 4.0, dtype=np.float32))
     g.free()
+
+
+def test_replays_survive_growth_of_the_library_workspaces(cm):
+    """A recorded reduction carries the addresses of the workspace, the arrival counters and
+    the vector of ones it used.  Later eager calls that outgrow them get new ones; the old
+    blocks stay allocated, and the replay still gives the recorded result."""
+    rng = np.random.default_rng(3)
+    x = np.asarray(rng.uniform(-1, 1, (64, 8192)), dtype=np.float32, order='F')
+    a, r1, r0 = cm.CUDAMatrix(x), cm.empty((64, 1)), cm.empty((1, 8192))
+    a.sum(axis=1, target=r1); a.sum(axis=0, target=r0)            # eagerly once: the workspaces reach their sizes
+    want1, want0 = r1.asarray().copy(), r0.asarray().copy()
+    with cm.Graph() as g:
+        a.sum(axis=1, target=r1)
+        a.sum(axis=0, target=r0)
+    # a product whose split reduction needs a larger workspace, a sum that needs a longer vector of ones
+    p = cm.CUDAMatrix(np.asarray(rng.uniform(-1, 1, (256, 32768)), dtype=np.float32, order='F'))
+    q = cm.CUDAMatrix(np.asarray(rng.uniform(-1, 1, (32768, 256)), dtype=np.float32, order='F'))
+    pq = cm.dot(p, q)
+    ref = p.asarray().astype(np.float64) @ q.asarray().astype(np.float64)
+    assert np.max(np.abs(pq.asarray() - ref)) <= 1e-4 * np.max(np.abs(p.asarray()).astype(np.float64) @ np.abs(q.asarray()))
+    long = cm.CUDAMatrix(np.ones((cm.MAX_ONES + 4096, 2), dtype=np.float32))
+    assert np.array_equal(long.sum(axis=0).asarray(), np.full((1, 2), cm.MAX_ONES + 4096, dtype=np.float32))
+    for _ in range(2):
+        r1.assign(0); r0.assign(0)
+        g.launch()
+        assert np.array_equal(r1.asarray(), want1) and np.array_equal(r0.asarray(), want0)
+    g.free()
