@@ -185,10 +185,12 @@ int cuda_set_device(int deviceId) {
       if (g_scratch[slot]) hipFree(g_scratch[slot]);
       g_scratch[slot] = nullptr;
       g_scratch_bytes[slot] = 0;
+      g_scratch_recorded[slot] = false;
     }
     if (g_zero_words) hipFree(g_zero_words);
     g_zero_words = nullptr;
     g_zero_words_n = 0;
+    g_zero_words_recorded = false;
     hipSetDevice(deviceId);
   }
   return 0;
