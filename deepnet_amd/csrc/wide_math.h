@@ -2,8 +2,9 @@
 // error of about 2^-33, so that a whole formula (exp -> add -> divide, log of a
 // sum, a * cos(b) ...) is rounded to fp32 once, at its end.  The fp32 library
 // routines are each allowed a few ulp and a chain of them drifts past the
-// 2-ulp parity bar; fp64 FMAs issue at the fp32 rate on this part, so these cost
-// about as many issue slots as the fp32 versions.
+// 2-ulp parity bar.  fp64 instructions issue at half the fp32 rate, which a
+// streaming kernel mostly hides; exp and sigmoid, the two that showed it, have
+// fp32 routes of about 1 ulp for arguments of ordinary size.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <math.h>
@@ -89,10 +90,52 @@ __device__ __forceinline__ float dn_tanh(float x) {
   return (float)(em * dn_rcp_wide(em + 2.0));
 }
 
-__device__ __forceinline__ float dn_exp(float x) { return x != x ? x : (float)dn_exp_wide((double)x); }
+// The same split in fp32 for arguments of ordinary size (fp64 instructions issue at half the
+// fp32 rate here, and exp / sigmoid over a large matrix are otherwise issue-bound):
+// n = rint(t log2 e), g = t - n ln2 in two FMAs (the first is exact: n has at most 8 significant
+// bits, the high part of ln2 has 16), e^g - 1 = g + g^2 P(g) with P the Taylor sum through g^5
+// (remainder g^8/8! < 5.2e-9).  Returns e^g - 1 to about half an ulp of e^g.
+__device__ __forceinline__ float dn_exp_parts_f32(float t, float* n_out) {
+  const float n = rintf(t * 1.44269504088896341f);
+  float g = fmaf(n, -0.693145751953125f, t);
+  g = fmaf(n, -1.42860682030941723e-06f, g);
+  float p = 1.98412698412698413e-04f;      // 1/7!
+  p = fmaf(p, g, 1.38888888888888894e-03f);  // 1/6!
+  p = fmaf(p, g, 8.33333333333333322e-03f);  // 1/5!
+  p = fmaf(p, g, 4.16666666666666644e-02f);  // 1/4!
+  p = fmaf(p, g, 1.66666666666666657e-01f);  // 1/3!
+  p = fmaf(p, g, 0.5f);
+  *n_out = n;
+  return fmaf(g * g, p, g);
+}
 
-// 1/(1+exp(-x))
+// e^x: one rounding of 1 + (e^g - 1) and an exact scaling for |x| <= 80 (results between
+// 1.8e-35 and 5.5e34: about 1 ulp in all); the fp64 evaluation beyond, and for NaN.
+__device__ __forceinline__ float dn_exp(float x) {
+  if (fabsf(x) <= 80.f) {
+    float n;
+    const float q = dn_exp_parts_f32(x, &n);
+    return ldexpf(1.0f + q, (int)n);
+  }
+  return x != x ? x : (float)dn_exp_wide((double)x);
+}
+
+// 1/(1+exp(-x)).  For |x| <= 16: e^-x = 2^n (1 + q) with |n| <= 23, so the sum 1 + 2^n is
+// exact, s = 2^n q + (1 + 2^n) is rounded once and the rounding error kept (a result just
+// below a power of two would double it), and the reciprocal of the pair is the hardware
+// estimate with one Newton step (about 1 ulp in all).
+// The fp64 evaluation beyond, and for NaN.
 __device__ __forceinline__ float dn_sigmoid(float x) {
+  if (fabsf(x) <= 16.f) {
+    float n;
+    const float q = dn_exp_parts_f32(-x, &n);
+    const float p2 = ldexpf(1.0f, (int)n);
+    const float hi = 1.0f + p2;
+    const float s = fmaf(p2, q, hi);
+    const float s_lo = fmaf(p2, q, hi - s);          // what the rounding of s dropped (hi - s is exact)
+    const float r = __builtin_amdgcn_rcpf(s);
+    return fmaf(r, fmaf(-s_lo, r, fmaf(-s, r, 1.0f)), r);
+  }
   const double s = 1.0 + dn_exp_wide(-(double)x);   // in [1, inf]
   const float r = (s < 1e300) ? (float)dn_rcp_wide(s) : 0.f;
   return x != x ? x : r;
