@@ -153,3 +153,16 @@ def test_blockify_expand_accumulate_translations(cm, rng):
     tr = cm.CUDAMatrix(imgs).generate_translations(8, 6, cm.CUDAMatrix(ox), cm.CUDAMatrix(oy))
     want = orc.generate_translations(imgs, 8, 6, ox, oy, 3).astype(np.float32)
     assert np.array_equal(tr.asarray(), want) and (want[:, 4] == 0).any() and (want[:, 0] != 0).all()
+
+
+@pytest.mark.parametrize("n", [1, 3, 1023, 4096, 16384, 16385])
+def test_small_results_reach_the_host_after_the_work_queued_before_them(cm, n):
+    """Matrices of up to 16384 elements are read back through a pinned block that a kernel
+    fills and tags; every read must show the values of the kernel queued just before it."""
+    a = cm.empty((n, 1))
+    b = cm.CUDAMatrix(np.arange(n, dtype=np.float32).reshape(n, 1))
+    for i in range(300):
+        a.assign(float(i))
+        a.add(b)
+        got = a.asarray()
+        assert got[0, 0] == i and got[-1, 0] == i + n - 1 and np.array_equal(got[:, 0], np.arange(n, dtype=np.float32) + i), i
