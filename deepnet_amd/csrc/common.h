@@ -14,6 +14,8 @@ void* dn_scratch(size_t bytes, int slot = 0);
 
 // n 32-bit words that are zero between kernels (arrival counters); null when they cannot be had.
 unsigned* dn_zero_words(int n);
+// f is called when the last executable graph that this library made has been freed.
+void dn_set_no_graphs_hook(void (*f)());
 
 // Looks up (once per device) the fixed workspace of the entry points that allocate nothing.
 int dn_noalloc_setup();

@@ -24,6 +24,10 @@ static hipStream_t g_stream = nullptr;     // nullptr: the NULL stream
 static bool g_capturing = false;
 static hipStream_t g_capture_stream = nullptr;
 
+static int g_live_graphs = 0;
+static void (*g_no_graphs_hook)() = nullptr;
+void dn_set_no_graphs_hook(void (*f)()) { g_no_graphs_hook = f; }
+
 hipStream_t dn_stream() { return g_stream; }
 bool dn_capturing() { return g_capturing; }
 
@@ -251,10 +255,9 @@ static bool stage_out(const float* src, float* host, int n) {
 // graph_capture_begin() switches the library to a capturing stream: every call until
 // graph_capture_end() is recorded instead of run (with the pointers and scalars it was given).
 // What cannot be recorded fails with its usual error code: calls that wait for the device
-// (copy_to_host, vdot, euclid_norm), workspaces that would have to grow (run the sequence once
-// before recording it) and the split schedule of the random generator (matrices of more than
-// 32 * 12288 elements).  The random generator's state lives on the device, so every replay
-// draws fresh numbers.  graph_launch() queues a replay on the NULL stream, in order with
+// (copy_to_host, vdot, euclid_norm) and workspaces that would have to grow (run the sequence
+// once before recording it).  The random generator's state lives on the device, so every
+// replay draws fresh numbers.  graph_launch() queues a replay on the NULL stream, in order with
 // everything else the library does.
 void* graph_capture_begin(void) {
   if (g_capturing) return nullptr;
@@ -285,6 +288,7 @@ void* graph_capture_end(void) {
   const hipError_t e2 = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
   hipGraphDestroy(graph);
   if (e2 != hipSuccess) { hipGetLastError(); return nullptr; }
+  ++g_live_graphs;
   return (void*)exec;
 }
 
@@ -296,7 +300,9 @@ int graph_launch(void* exec) {
 int graph_free(void* exec) {
   if (!exec) return 0;
   hipDeviceSynchronize();
-  return hipGraphExecDestroy((hipGraphExec_t)exec) == hipSuccess ? 0 : CUDA_ERROR;
+  const hipError_t e = hipGraphExecDestroy((hipGraphExec_t)exec);
+  if (g_live_graphs > 0 && --g_live_graphs == 0 && g_no_graphs_hook) g_no_graphs_hook();
+  return e == hipSuccess ? 0 : CUDA_ERROR;
 }
 
 // A second library of this package (the conv library has its own copy of this file) joins a

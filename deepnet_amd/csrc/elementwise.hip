@@ -495,9 +495,8 @@ static int dot_bias_act_impl(rnd_struct* rnd, cudamat* mat1, cudamat* mat2, cuda
   if (n == 1 || k <= 0) {
     err = dot(mat1, mat2, target, 0.f, 1.f);                 // vector-shaped: the streaming kernels
   } else {
-    // (a recorded graph could not repeat the host's switch to the generator's other word buffer)
     DnGemmSample smp = {nullptr, nullptr, nullptr, nullptr};
-    const bool try_sample = sample && !dn_capturing();
+    const bool try_sample = sample && rng_pin_if_recording(rnd);
     if (try_sample) smp = DnGemmSample{sample->data_device, rnd->dev_mults, rnd->dev_words, rng_other(rnd->dev_words)};
     err = dn_gemm_fused(mat1->is_trans != 0, mat2->is_trans != 0, m, n, k, mat1->data_device, mat1->size[0],
                         mat2->data_device, mat2->size[0], target->data_device, m, bias ? bias->data_device : nullptr,
@@ -530,8 +529,8 @@ int dot_bias_act(cudamat* mat1, cudamat* mat2, cudamat* bias, cudamat* target, i
 // Extension: dot_bias_act followed by sample_bernoulli(rnd_state, target, sample), the
 // up-pass of an RBM with its hidden sample (deepnet/dbm.py:95-105), bit-identical to the two
 // calls (same states, same samples, same generator state afterwards).  One launch where the
-// product runs as a single kernel over at most 16 * 12288 outputs and no graph is being
-// recorded; otherwise the separate kernels.
+// product runs as a single kernel over at most 16 * 12288 outputs; otherwise the separate
+// kernels.
 int dot_bias_act_sample(rnd_struct* rnd_state, cudamat* mat1, cudamat* mat2, cudamat* bias, cudamat* target,
                         cudamat* sample, int act) {
   if (!sample) return ERROR_GENERIC;

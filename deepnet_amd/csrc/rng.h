@@ -29,9 +29,12 @@ static inline unsigned long long* rng_other(unsigned long long* w) {
 
 // A kernel has left the generator's next state in rng_other(st->dev_words): make it the
 // current one.  Normally the pointer is flipped; once a recorded graph refers to the current
-// buffer (rng.hip pins it) the words are copied back into it instead, so that replays and
-// eager calls keep drawing from one sequence.
+// buffer (rng.hip pins it until the last graph has been freed) the words are copied back into
+// it instead, so that replays and eager calls keep drawing from one sequence.
 void rng_publish(rnd_struct* st);
+// To be called before a kernel that uses st->dev_words is launched: while a graph is being
+// recorded it pins the buffer.  Always true (kept as a condition at the call sites).
+bool rng_pin_if_recording(rnd_struct* st);
 
 // What a product that also draws a Bernoulli sample of its output needs from the generator:
 // the sample's buffer, the multipliers, the current words (read only) and the buffer that

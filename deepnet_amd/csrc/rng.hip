@@ -16,6 +16,7 @@
 //             constants (2^32)^-(2^j) mod m, one per set bit of its part number.
 #include "common.h"
 #include "rng.h"
+#include <vector>
 #include <math.h>
 #include <stdio.h>
 #include <stdlib.h>
@@ -305,24 +306,27 @@ k_rng_gauss_split(const unsigned int* mults, const unsigned long long* words, un
 #define RNG_SPLIT_PARTS 24
 #define RNG_SPLIT_SRC_PARTS 96
 
-// Word buffers that a recorded graph refers to: its serial kernels carry the buffer's address,
-// so from then on the generator's state has to stay in that buffer.
-#define RNG_MAX_PINNED 16
-static unsigned long long* g_rng_pinned[RNG_MAX_PINNED];
-static int g_rng_npinned = 0;
+// Word buffers that a recorded graph refers to: its kernels carry the buffer's address, so
+// from then on the generator's state has to stay in that buffer.
+static std::vector<unsigned long long*>& rng_pinned() {
+  static std::vector<unsigned long long*> list;
+  return list;
+}
 
 static bool rng_is_pinned(const unsigned long long* w) {
-  for (int i = 0; i < g_rng_npinned; ++i)
-    if (g_rng_pinned[i] == w) return true;
+  for (const unsigned long long* p : rng_pinned())
+    if (p == w) return true;
   return false;
 }
 
-// Called before a kernel that reads and writes st->dev_words in place is launched; false
-// when the launch is being recorded and the buffer cannot be remembered any more.
-static bool rng_pin_if_recording(rnd_struct* st) {
-  if (!dn_capturing() || rng_is_pinned(st->dev_words)) return true;
-  if (g_rng_npinned == RNG_MAX_PINNED) return false;
-  g_rng_pinned[g_rng_npinned++] = st->dev_words;
+// (no graph is left: the state may move between the buffers again)
+static void rng_unpin_all() { rng_pinned().clear(); }
+
+bool rng_pin_if_recording(rnd_struct* st) {
+  if (dn_capturing() && !rng_is_pinned(st->dev_words)) {
+    rng_pinned().push_back(st->dev_words);
+    dn_set_no_graphs_hook(rng_unpin_all);
+  }
   return true;
 }
 
@@ -362,9 +366,9 @@ static int launch_rng(rnd_struct* st, size_t n, Op op) {
                        op);
     return dn_launch_status();
   }
-  // (the split schedule publishes the new state from the host, which a recorded graph would
-  // not repeat)
-  if (dn_capturing()) return ERROR_UNSUPPORTED;
+  // (while a graph is recorded the buffer is pinned, and rng_publish() records the copy of the
+  // new words back into it)
+  if (!rng_pin_if_recording(st)) return ERROR_UNSUPPORTED;
   unsigned long long* next = rng_other(st->dev_words);
   const unsigned grid = (unsigned)(parts * (NUM_RND_STREAMS / RNG_SPLIT_BLOCK));
   if (op.src)
@@ -409,8 +413,7 @@ int init_random(rnd_struct* rnd_state, int seed, char* cudamatpath) {
 }
 
 // Gaussian ops: parts of 16 draws (8 pairs, each a logf, sqrtf, sinf and cosf) while that
-// gives at most RNG_GAUSS_PARTS parts per stream.  Recording keeps the serial kernel: the
-// split schedule flips dev_words on the host, which a recorded graph would not repeat.
+// gives at most RNG_GAUSS_PARTS parts per stream.
 #define RNG_GAUSS_PARTS 256
 static int launch_gauss(rnd_struct* st, const float* in, float* out, size_t n, float mult_by) {
   if (n == 0) return 0;
@@ -421,8 +424,8 @@ static int launch_gauss(rnd_struct* st, const float* in, float* out, size_t n, f
   const size_t parts = (draws + (1ull << chbits) - 1) >> chbits;
   int top = 0;
   while ((parts - 1) >> top) ++top;
-  if (draws < RNG_SPLIT_MIN_DRAWS || chbits + top > RNG_JUMP_BITS || dn_capturing()) {
-    if (!rng_pin_if_recording(st)) return ERROR_UNSUPPORTED;
+  if (!rng_pin_if_recording(st)) return ERROR_UNSUPPORTED;
+  if (draws < RNG_SPLIT_MIN_DRAWS || chbits + top > RNG_JUMP_BITS) {
     hipLaunchKernelGGL(k_rng_gauss, dim3(RNG_BLOCKS), dim3(RNG_BLOCK), 0, dn_stream(), st->dev_mults, st->dev_words, in, out, n,
                        mult_by);
     return dn_launch_status();

@@ -829,8 +829,8 @@ class Graph(object):
 
     The calls are recorded with the matrices and scalars they were given; the random generator's
     state lives on the device, so every replay draws fresh numbers.  Calls that wait for the
-    device (asarray, copy_to_host, vdot, euclid_norm), allocations (empty, CUDAMatrix(...)) and
-    random fills of more than 32 * 12288 elements raise CUDAMatException while recording."""
+    device (asarray, copy_to_host, vdot, euclid_norm) and allocations (empty, CUDAMatrix(...))
+    raise CUDAMatException while recording."""
 
     def __init__(self):
         self._exec = None

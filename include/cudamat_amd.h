@@ -191,8 +191,8 @@ int dot_bias_act(cudamat* mat1, cudamat* mat2, cudamat* bias, cudamat* target, i
 /* Extension, no counterpart in cudamat.cu: dot_bias_act followed by
  * sample_bernoulli(rnd_state, target, sample) (the up-pass of an RBM with its hidden sample,
  * deepnet/dbm.py:95-105), bit-identical to the two calls including the generator's state
- * afterwards; one launch for single-kernel products of at most 16 * 12288 outputs outside a
- * graph recording, the separate kernels otherwise.  sample: target's shape, another buffer. */
+ * afterwards; one launch for single-kernel products of at most 16 * 12288 outputs, the
+ * separate kernels otherwise.  sample: target's shape, another buffer. */
 int dot_bias_act_sample(rnd_struct* rnd_state, cudamat* mat1, cudamat* mat2, cudamat* bias, cudamat* target,
                         cudamat* sample, int act);
 
@@ -262,9 +262,9 @@ int get_softmax_cross_entropy(cudamat* mat, cudamat* labels, cudamat* target, fl
  * record every following call (with the pointers and scalars it is given) into a HIP graph
  * instead of running it, until graph_capture_end() returns the executable graph;
  * graph_launch() replays it with one launch on the NULL stream.  For step sequences that are
- * bound by the cost of launching (the RBM and MLP steps).  Calls that wait for the device,
- * workspaces that would have to grow and the random generator's split schedule fail with
- * their error codes while recording; run the sequence once before recording it.
+ * bound by the cost of launching (the RBM and MLP steps).  Calls that wait for the device
+ * and workspaces that would have to grow fail with their error codes while recording; run
+ * the sequence once before recording it.
  * graph_capture_begin returns the capturing stream (NULL on failure); graph_set_stream hands
  * that stream to a second library of this package (stream NULL, capturing 0 afterwards). ---- */
 void* graph_capture_begin(void);

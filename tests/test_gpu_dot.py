@@ -236,8 +236,8 @@ def test_dot_bias_act_sample_errors_and_recording(cm, rng):
     with pytest.raises(cm.CUDAMatException):
         cm.dot_bias_act(a, b, None, target=t, sample=t)              # the sample needs a buffer of its own
     assert cm._cudamat.dot_bias_act_sample(cm.CUDAMatrix.rnd_state_p, a.p_mat, b.p_mat, None, t.p_mat, None, 1) != 0
-    # while a graph is recorded the sample comes from its own kernel (the generator keeps one word
-    # buffer); every replay draws on from where the last one stopped
+    # recorded, the call keeps the generator's state in one word buffer; every replay draws on
+    # from where the last one stopped
     cm.CUDAMatrix.init_random(9)
     want = []
     for _ in range(3):

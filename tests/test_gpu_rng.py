@@ -231,6 +231,46 @@ def test_recorded_draws_and_eager_calls_share_one_sequence(cm, mults):
         cm.dot_bias_act(w.T, v, None, target=h, act='sigmoid', sample=hs)
         u = host.uniform(96 * 100).reshape((96, 100), order='F')
         assert np.array_equal(hs.asarray(), (u < np.float32(0.5)).astype(np.float32)), step
+        here = ct.cast(cm.CUDAMatrix.rnd_state.dev_rnd_words, ct.c_void_p).value
         big.fill_with_randn(); host.randn(big.shape[0] * big.shape[1])
+        assert ct.cast(cm.CUDAMatrix.rnd_state.dev_rnd_words, ct.c_void_p).value == here      # the state stays put
+    assert np.array_equal(_device_words(cm), host.words)
+    g.free()
+    # no graph is left: the next large call moves the state to the other buffer again
+    here = ct.cast(cm.CUDAMatrix.rnd_state.dev_rnd_words, ct.c_void_p).value
+    big.fill_with_rand()
+    want = host.uniform(big.shape[0] * big.shape[1])
+    assert np.array_equal(big.asarray().ravel(order='F').view(np.uint32), want.view(np.uint32))
+    assert ct.cast(cm.CUDAMatrix.rnd_state.dev_rnd_words, ct.c_void_p).value != here
+    assert np.array_equal(_device_words(cm), host.words)
+
+
+def test_large_draws_are_recorded_too(cm, mults):
+    """Matrices large enough for the schedule that shares a stream among lanes (and the sample
+    of dot_bias_act) record like the small ones: every replay continues the host's sequence."""
+    cm.CUDAMatrix.init_random(33)
+    host = mwc.MWC(mults, 33)
+    big, drop = cm.empty((1024, 512)), cm.CUDAMatrix(np.ones((700, 600), dtype=np.float32))
+    gauss = cm.empty((512, 1024))
+    w = cm.CUDAMatrix(np.zeros((64, 512), dtype=np.float32)); v = cm.CUDAMatrix(np.ones((64, 1024), dtype=np.float32))
+    h, hs = cm.empty((512, 1024)), cm.empty((512, 1024))
+    with cm.Graph() as g:
+        big.fill_with_rand()
+        drop.dropout(0.5)
+        cm.dot_bias_act(w.T, v, None, target=h, act='sigmoid', sample=hs)
+        gauss.fill_with_randn()
+    keep = np.ones((700, 600), dtype=np.float32)
+    for step in range(3):
+        g.launch()
+        want = host.uniform(big.shape[0] * big.shape[1])
+        assert np.array_equal(big.asarray().ravel(order='F').view(np.uint32), want.view(np.uint32)), step
+        keep *= (host.uniform(700 * 600) > np.float32(0.5)).astype(np.float32).reshape((700, 600), order='F')
+        assert np.array_equal(drop.asarray(), keep), step
+        u = host.uniform(512 * 1024).reshape((512, 1024), order='F')
+        assert np.array_equal(hs.asarray(), (u < np.float32(0.5)).astype(np.float32)), step
+        want = host.randn(512 * 1024)
+        assert np.max(np.abs(gauss.asarray().ravel(order='F') - want)) < 2e-5, step
+        if step == 1:
+            big.fill_with_rand(); host.uniform(big.shape[0] * big.shape[1])      # an eager call in between
     assert np.array_equal(_device_words(cm), host.words)
     g.free()
