@@ -2,6 +2,7 @@
 // Replaces cudamat/cudamat.cu:25-53, 87-123, 153-186, 217-434 and the copy
 // kernels cudamat_kernels.cu:247-294.
 #include "common.h"
+#include <vector>
 #include <stdio.h>
 #include <string.h>
 
@@ -40,6 +41,7 @@ bool dn_capturing() { return g_capturing; }
 static void* g_scratch[4] = {nullptr, nullptr, nullptr, nullptr};
 static size_t g_scratch_bytes[4] = {0, 0, 0, 0};
 static bool g_scratch_recorded[4] = {false, false, false, false};
+static std::vector<void*> g_retired;   // outgrown blocks that a recorded graph may still use
 
 void* dn_scratch(size_t bytes, int slot) {
   if (bytes > g_scratch_bytes[slot]) {
@@ -47,9 +49,11 @@ void* dn_scratch(size_t bytes, int slot) {
 
     if (g_scratch[slot]) {
       hipDeviceSynchronize();
-      // A block that was handed out while a graph was being recorded stays allocated for
-      // the life of the process: the graph's kernels carry its address.
-      if (!g_scratch_recorded[slot]) hipFree(g_scratch[slot]);
+      // A block that was handed out while a graph was being recorded stays allocated: the
+      // graph's kernels carry its address (it is freed with the last graph of this library;
+      // a library that only joins recordings keeps it for the life of the process).
+      if (g_scratch_recorded[slot]) g_retired.push_back(g_scratch[slot]);
+      else hipFree(g_scratch[slot]);
       g_scratch_recorded[slot] = false;
     }
     size_t want = bytes < (1u << 20) ? (1u << 20) : bytes;
@@ -76,7 +80,8 @@ unsigned* dn_zero_words(int n) {
     if (g_capturing) return nullptr;
     if (g_zero_words) {
       hipDeviceSynchronize();
-      if (!g_zero_words_recorded) hipFree(g_zero_words);   // (as for the scratch blocks)
+      if (g_zero_words_recorded) g_retired.push_back(g_zero_words);   // (as for the scratch blocks)
+      else hipFree(g_zero_words);
       g_zero_words_recorded = false;
       g_zero_words = nullptr;
       g_zero_words_n = 0;
@@ -301,7 +306,13 @@ int graph_free(void* exec) {
   if (!exec) return 0;
   hipDeviceSynchronize();
   const hipError_t e = hipGraphExecDestroy((hipGraphExec_t)exec);
-  if (g_live_graphs > 0 && --g_live_graphs == 0 && g_no_graphs_hook) g_no_graphs_hook();
+  if (g_live_graphs > 0 && --g_live_graphs == 0) {
+    for (void* p : g_retired) hipFree(p);
+    g_retired.clear();
+    for (bool& r : g_scratch_recorded) r = false;
+    g_zero_words_recorded = false;
+    if (g_no_graphs_hook) g_no_graphs_hook();
+  }
   return e == hipSuccess ? 0 : CUDA_ERROR;
 }
 

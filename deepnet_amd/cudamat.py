@@ -854,10 +854,20 @@ class Graph(object):
             lib.graph_set_stream(None, 0)
         self._others = []
         handle = _cudamat.graph_capture_end()
-        if exc_type is None and not handle:
+        if exc_type is not None:
+            if handle:                              # a recording that was given up is not kept
+                _cudamat.graph_free(handle)
+            return False
+        if not handle:
             raise CUDAMatException("recording the graph failed")
         self._exec = handle
         return False
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
 
     def launch(self):
         if not self._exec:
