@@ -3,6 +3,7 @@
 // kernels cudamat_kernels.cu:247-294.
 #include "common.h"
 #include <vector>
+#include <unordered_map>
 #include <stdio.h>
 #include <string.h>
 
@@ -41,7 +42,7 @@ bool dn_capturing() { return g_capturing; }
 static void* g_scratch[4] = {nullptr, nullptr, nullptr, nullptr};
 static size_t g_scratch_bytes[4] = {0, 0, 0, 0};
 static bool g_scratch_recorded[4] = {false, false, false, false};
-static std::vector<void*> g_retired;   // outgrown blocks that a recorded graph may still use
+static std::vector<void*>& g_retired = *new std::vector<void*>;   // outgrown blocks that a recorded graph may still use
 
 void* dn_scratch(size_t bytes, int slot) {
   if (bytes > g_scratch_bytes[slot]) {
@@ -67,6 +68,56 @@ void* dn_scratch(size_t bytes, int slot) {
   }
   if (g_capturing) g_scratch_recorded[slot] = true;
   return g_scratch[slot];
+}
+
+// ------------------------------------------------------------------ matrix memory
+// Matrices come from hipMalloc, one allocation each, as in the reference (cublasAlloc).
+// hipFree waits for the device, which stalls code that makes a temporary per step
+// (x = cm.dot(a, b); ...; del x: 19 us for two launches and a temporary, 10 us without the wait),
+// so a freed block is kept for the next request of exactly its size instead: everything
+// the library does is queued on one stream, a block's next owner can only touch it after
+// the kernels of the previous one.  At most DN_CACHE_BYTES are kept (a block that would
+// exceed them is freed at once); an allocation that fails frees them all and tries again.
+#define DN_CACHE_BYTES ((size_t)4 << 30)
+// (on the heap and never destroyed: matrices may still be freed while the process exits)
+static std::unordered_map<void*, size_t>& g_block_bytes = *new std::unordered_map<void*, size_t>;   // blocks handed out by block_get
+static std::unordered_map<size_t, std::vector<void*>>& g_block_cache = *new std::unordered_map<size_t, std::vector<void*>>;   // free blocks by size
+static size_t g_cached_bytes = 0;
+
+static void block_flush() {
+  for (auto& kv : g_block_cache)
+    for (void* p : kv.second) hipFree(p);
+  g_block_cache.clear();
+  g_cached_bytes = 0;
+}
+
+static void* block_get(size_t bytes) {
+  void* p = nullptr;
+  auto it = g_block_cache.find(bytes);
+  if (it != g_block_cache.end() && !it->second.empty()) {
+    p = it->second.back();
+    it->second.pop_back();
+    g_cached_bytes -= bytes;
+  } else if (hipMalloc(&p, bytes) != hipSuccess) {
+    hipGetLastError();
+    hipDeviceSynchronize();
+    block_flush();
+    if (hipMalloc(&p, bytes) != hipSuccess) { hipGetLastError(); return nullptr; }
+  }
+  g_block_bytes[p] = bytes;
+  return p;
+}
+
+// false when the runtime refuses to free the block
+static bool block_put(void* p) {
+  auto it = g_block_bytes.find(p);
+  if (it == g_block_bytes.end()) return hipFree(p) == hipSuccess;      // not one of ours (a caller's own allocation)
+  const size_t bytes = it->second;
+  g_block_bytes.erase(it);
+  if (g_cached_bytes + bytes > DN_CACHE_BYTES) return hipFree(p) == hipSuccess;
+  g_block_cache[bytes].push_back(p);
+  g_cached_bytes += bytes;
+  return true;
 }
 
 // A block of 32-bit words that is zero whenever no kernel of the library is running (arrival
@@ -178,6 +229,7 @@ int cublas_init(void) {
 
 int cublas_shutdown(void) {
   hipDeviceSynchronize();
+  block_flush();
   return 0;
 }
 
@@ -190,6 +242,7 @@ int cuda_set_device(int deviceId) {
     // the workspaces live in the memory of the device that was current when they were made
     hipSetDevice(before);
     hipDeviceSynchronize();
+    block_flush();
     for (int slot = 0; slot < 4; ++slot) {
       if (g_scratch[slot]) hipFree(g_scratch[slot]);
       g_scratch[slot] = nullptr;
@@ -331,13 +384,10 @@ void set_transpose(cudamat* mat, int is_trans) { mat->is_trans = is_trans; }
 int allocate_device_memory(cudamat* mat) {
   if (g_capturing) return ERROR_UNSUPPORTED;      // (allocations and transfers are not recorded into a graph)
   const long long len = dn_len(mat);
-  void* p = nullptr;
   // A 0-element matrix still gets a distinct, valid pointer.
   const size_t bytes = (size_t)(len > 0 ? len : 1) * sizeof(float);
-  if (hipMalloc(&p, bytes) != hipSuccess) {
-    hipGetLastError();
-    return CUBLAS_ERROR;
-  }
+  void* p = block_get(bytes);
+  if (!p) return CUBLAS_ERROR;
   mat->data_device = (float*)p;
   mat->on_device = 1;
   return 0;
@@ -405,9 +455,9 @@ int copy_on_device(cudamat* mat1, cudamat* mat2) {
 int free_device_memory(cudamat* mat) {
   if (g_capturing) return ERROR_UNSUPPORTED;
   if (mat->owns_data && mat->on_device) {
-    hipError_t e = hipFree(mat->data_device);
+    const bool ok = block_put(mat->data_device);
     mat->on_device = 0;
-    if (e != hipSuccess) return CUBLAS_ERROR;
+    if (!ok) return CUBLAS_ERROR;
   }
   return 0;
 }

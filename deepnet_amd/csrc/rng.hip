@@ -309,8 +309,8 @@ k_rng_gauss_split(const unsigned int* mults, const unsigned long long* words, un
 // Word buffers that a recorded graph refers to: its kernels carry the buffer's address, so
 // from then on the generator's state has to stay in that buffer.
 static std::vector<unsigned long long*>& rng_pinned() {
-  static std::vector<unsigned long long*> list;
-  return list;
+  static std::vector<unsigned long long*>* list = new std::vector<unsigned long long*>;   // never destroyed
+  return *list;
 }
 
 static bool rng_is_pinned(const unsigned long long* w) {

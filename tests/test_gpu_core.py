@@ -166,3 +166,28 @@ def test_small_results_reach_the_host_after_the_work_queued_before_them(cm, n):
         a.add(b)
         got = a.asarray()
         assert got[0, 0] == i and got[-1, 0] == i + n - 1 and np.array_equal(got[:, 0], np.arange(n, dtype=np.float32) + i), i
+
+
+def test_freed_blocks_are_reused_without_disturbing_queued_work(cm, rng):
+    """free_device_memory keeps a block for the next matrix of its size; work queued on the old
+    owner finishes before the new owner's first kernel, so results do not change."""
+    x = np.asarray(rng.uniform(-1, 1, (257, 129)), dtype=np.float32, order='F')
+    a = cm.CUDAMatrix(x)
+    total = np.zeros_like(x)
+    for i in range(50):
+        t = cm.empty(x.shape)
+        a.mult(float(i), target=t)
+        u = cm.empty(x.shape)
+        t.add(a, target=u)
+        t.free_device_memory()                   # its block goes to the next empty() of this size
+        v = cm.empty(x.shape)
+        v.assign(1.0)
+        assert np.array_equal(u.asarray(), x * np.float32(i) + x)
+        assert np.array_equal(v.asarray(), np.ones_like(x))
+        u.free_device_memory(); v.free_device_memory()
+    # other sizes, empty matrices and a shape changed after allocation
+    w = cm.empty((64, 64)); w.reshape((32, 128)); w.free_device_memory()
+    z = cm.empty((0, 5)); z.free_device_memory()
+    big = cm.empty((2048, 2048)); big.assign(2.0)
+    assert float(big.sum()) == 2.0 * 2048 * 2048
+    big.free_device_memory()
