@@ -178,6 +178,7 @@ class MLP(object):
         self.mask = [cm.empty((sizes[i + 1], B)) for i in range(2)]
         self.delta = [cm.empty((sizes[i + 1], B)) for i in range(3)]
         self.loss = cm.empty((1, B))
+        self.updates = None
         self.flops = 3 * 2 * B * (sizes[0] * sizes[1] + sizes[1] * sizes[2] + sizes[2] * sizes[3])
 
     def step(self):
@@ -204,8 +205,8 @@ class MLP(object):
                 d.mult(self.mom); d.add_mult(g); p.add_mult(d, -self.lr)
 
     def step_fused(self):
-        """The same step in 22 launches instead of 51: this backend's extensions dot_bias_act,
-        softmax_ce_grad and momentum_update, and the one-call forms that the reference's own
+        """The same step in 17 launches instead of 51: this backend's extensions dot_bias_act,
+        softmax_ce_grad and momentum_update (all six parameters in one launch), and the one-call forms that the reference's own
         API has for what deepnet spells out in several (dropout() for fill_with_rand ->
         greater_than -> mult, dot() into the gradient for assign(0) -> add_dot, dot() with a
         column of ones for assign(0) -> add_sums).  Every parameter, momentum buffer and loss
@@ -227,9 +228,10 @@ class MLP(object):
             if i > 0:
                 cm.dot(W[i], self.delta[i], target=self.delta[i - 1])
                 self.delta[i - 1].apply_rectified_linear_deriv(act[i])
-        for i in range(3):
-            cm.momentum_update(W[i], self.dW[i], self.gW[i], self.mom, self.lr, reset_gradient=False)
-            cm.momentum_update(b[i], self.db[i], self.gb[i], self.mom, self.lr, reset_gradient=False)
+        if self.updates is None:
+            self.updates = cm.MomentumUpdates([(W[i], self.dW[i], self.gW[i]) for i in range(3)] +
+                                              [(b[i], self.db[i], self.gb[i]) for i in range(3)])
+        self.updates.apply(self.mom, self.lr, reset_gradient=False)
 
 
 def net_mlp(cm, sizes=(784, 1024, 1024, 10), B=128, seed=3, fused=False):
@@ -626,7 +628,7 @@ def main():
         t = time_loop(cm, mlp.step_fused, 100, 10)
         secondary['mlp_fused_extensions'] = {
             'steps_per_sec': round(1.0 / t, 1), 'us_per_step': round(t * 1e6, 1),
-            'note': 'same step with dot_bias_act, softmax_ce_grad and momentum_update (extensions of this backend, not in the reference API) and the one-call forms dropout / dot into the gradient of the reference API: 22 launches instead of 51, same bits in every parameter'}
+            'note': 'same step with dot_bias_act, softmax_ce_grad and the momentum update of all six parameters in one launch (extensions of this backend, not in the reference API) and the one-call forms dropout / dot into the gradient of the reference API: 17 launches instead of 51, same bits in every parameter'}
         secondary['mlp_784_1024_1024_10']['us_per_step_recorded_graph'] = recorded(mlp.step, 100, 10)
         secondary['mlp_fused_extensions']['us_per_step_recorded_graph'] = recorded(mlp.step_fused, 100, 10)
         net = net_mlp(cm)

@@ -606,3 +606,99 @@ extern "C" int momentum_update(cudamat* w, cudamat* w_delta, cudamat* gradient, 
                        use_l1, reset);
   return dn_launch_status();
 }
+
+// The same update of up to MOM_MANY parameters in one launch (a net's weights and biases after
+// a step): workgroup b works on the parameter whose range of workgroups holds b.  Every
+// element goes through the arithmetic of k_momentum_update, so the results are the same bits.
+#define MOM_MANY 8
+struct MomTable {
+  float* w[MOM_MANY];
+  float* wd[MOM_MANY];
+  float* g[MOM_MANY];
+  long long n[MOM_MANY];
+  float momentum[MOM_MANY], l2[MOM_MANY], l1[MOM_MANY], eps[MOM_MANY];
+  int flags[MOM_MANY];               // bit 0: l2, bit 1: l1, bit 2: reset the gradient, bit 3: 16-byte groups
+  unsigned first_block[MOM_MANY + 1];
+  int count;
+};
+
+__global__ void __launch_bounds__(EW_THREADS) k_momentum_update_many(MomTable t) {
+  int k = 0;
+  while (k + 1 < t.count && blockIdx.x >= t.first_block[k + 1]) ++k;   // (uniform over the workgroup)
+  float* w = t.w[k];
+  float* wd = t.wd[k];
+  float* g = t.g[k];
+  const long long n = t.n[k];
+  const float momentum = t.momentum[k], l2 = t.l2[k], l1 = t.l1[k], eps = t.eps[k];
+  const int flags = t.flags[k];
+  const bool use_l2 = flags & 1, use_l1 = flags & 2, reset = flags & 4;
+  auto one = [&](float wv, float dv, float gv, float& w_out, float& d_out) {
+    float d = __fmul_rn(momentum, dv);
+    if (use_l2) d = __fmaf_rn(l2, wv, d);
+    if (use_l1) d = __fadd_rn(d, (wv > 0.f) ? l1 : ((wv < 0.f) ? -l1 : 0.f));
+    d = __fmaf_rn(1.f, gv, d);
+    d_out = d;
+    w_out = __fmaf_rn(-eps, d, wv);
+  };
+  const long long tid = (long long)(blockIdx.x - t.first_block[k]) * EW_THREADS + threadIdx.x;
+  if (flags & 8) {
+    if (tid * 4 >= n) return;
+    const float4 wv = *reinterpret_cast<const float4*>(w + 4 * tid);
+    const float4 dv = *reinterpret_cast<const float4*>(wd + 4 * tid);
+    const float4 gv = *reinterpret_cast<const float4*>(g + 4 * tid);
+    float4 wo, dox;
+    one(wv.x, dv.x, gv.x, wo.x, dox.x);
+    one(wv.y, dv.y, gv.y, wo.y, dox.y);
+    one(wv.z, dv.z, gv.z, wo.z, dox.z);
+    one(wv.w, dv.w, gv.w, wo.w, dox.w);
+    *reinterpret_cast<float4*>(wd + 4 * tid) = dox;
+    *reinterpret_cast<float4*>(w + 4 * tid) = wo;
+    if (reset) *reinterpret_cast<float4*>(g + 4 * tid) = make_float4(0.f, 0.f, 0.f, 0.f);
+  } else {
+    if (tid >= n) return;
+    float wo, dox;
+    one(w[tid], wd[tid], g[tid], wo, dox);
+    wd[tid] = dox;
+    w[tid] = wo;
+    if (reset) g[tid] = 0.f;
+  }
+}
+
+// Extension (no counterpart in cudamat.cu): momentum_update over count parameters, arguments as
+// arrays of count entries.  All parameters are checked (as momentum_update checks one) before
+// anything is launched; more than MOM_MANY take several launches.
+extern "C" int momentum_update_many(int count, cudamat** w, cudamat** w_delta, cudamat** gradient, const float* momentum,
+                                    const float* l2_decay, const float* l1_decay, const float* epsilon, const int* flags) {
+  if (count < 0) return ERROR_GENERIC;
+  for (int i = 0; i < count; ++i) {
+    if (!w[i]->on_device || !w_delta[i]->on_device || !gradient[i]->on_device) return ERROR_NOT_ON_DEVICE;
+    if (w[i]->is_trans != w_delta[i]->is_trans || w[i]->is_trans != gradient[i]->is_trans) return ERROR_TRANSPOSEDNESS;
+    if (!same_dims(w[i], w_delta[i]) || !same_dims(w[i], gradient[i])) return ERROR_INCOMPATIBLE_DIMENSIONS;
+    const long long lanes = dn_len(w[i]);
+    if ((lanes + EW_THREADS - 1) / EW_THREADS > 0x0fffffffll) return ERROR_UNSUPPORTED;
+  }
+  for (int i0 = 0; i0 < count; i0 += MOM_MANY) {
+    MomTable t;
+    t.count = 0;
+    unsigned blocks = 0;
+    for (int i = i0; i < count && i < i0 + MOM_MANY; ++i) {
+      const long long n = dn_len(w[i]);
+      if (n <= 0) continue;
+      const int k = t.count++;
+      const bool vec = n % 4 == 0 && dn_aligned16(w[i]->data_device) && dn_aligned16(w_delta[i]->data_device) &&
+                       dn_aligned16(gradient[i]->data_device);
+      t.w[k] = w[i]->data_device; t.wd[k] = w_delta[i]->data_device; t.g[k] = gradient[i]->data_device;
+      t.n[k] = n;
+      t.momentum[k] = momentum[i]; t.l2[k] = l2_decay[i]; t.l1[k] = l1_decay[i]; t.eps[k] = epsilon[i];
+      t.flags[k] = (flags[i] & 7) | (vec ? 8 : 0);
+      t.first_block[k] = blocks;
+      const long long lanes = vec ? n / 4 : n;
+      blocks += (unsigned)((lanes + EW_THREADS - 1) / EW_THREADS);
+    }
+    if (t.count == 0) continue;
+    t.first_block[t.count] = blocks;
+    hipLaunchKernelGGL(k_momentum_update_many, dim3(blocks), dim3(EW_THREADS), 0, dn_stream(), t);
+    if (int e = dn_launch_status()) return e;
+  }
+  return 0;
+}

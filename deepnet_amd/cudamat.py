@@ -117,6 +117,8 @@ _SIGNATURES = {
     'dot_bias_act': (_i, [_M, _M, _M, _M, ct.c_int]),
     'dot_bias_act_sample': (_i, [ct.c_void_p, _M, _M, _M, _M, _M, ct.c_int]),
     'momentum_update': (_i, [_M, _M, _M, _f, _f, _f, _f, ct.c_int]),
+    'momentum_update_many': (_i, [ct.c_int, ct.c_void_p, ct.c_void_p, ct.c_void_p, ct.c_void_p, ct.c_void_p, ct.c_void_p,
+                                  ct.c_void_p, ct.c_void_p]),
     'softmax_ce_grad': (_i, [_M, _M, _M, _M, _M, _f]),
     'init_from_sparse_array': (None, [_S, ct.POINTER(ct.c_float), ct.POINTER(ct.c_int), ct.POINTER(ct.c_int),
                                       _i, _i, _i]),
@@ -925,6 +927,48 @@ def momentum_update(w, w_delta, gradient, momentum, epsilon, l2_decay=None, l1_d
     _check(_cudamat.momentum_update(w.p_mat, w_delta.p_mat, gradient.p_mat, ct.c_float(momentum),
                                     ct.c_float(l2_decay or 0.0), ct.c_float(l1_decay or 0.0), ct.c_float(epsilon), flags))
     return w
+
+
+class MomentumUpdates(object):
+    """Extension of this backend: momentum_update for a fixed list of parameters in one launch
+    per 8 of them.  updates: a list of (w, w_delta, gradient) triples; the argument arrays are
+    built once, each step passes the scalars:
+
+        upd = cm.MomentumUpdates([(W1, dW1, gW1), (b1, db1, gb1), ...])
+        upd.apply(momentum, epsilon)                 # the same bits as one momentum_update each
+
+    momentum, epsilon, l2_decay, l1_decay: one number for all parameters or a sequence with one
+    entry per parameter (l2_decay / l1_decay None: no such term)."""
+
+    def __init__(self, updates):
+        self._keep = [tuple(u) for u in updates]
+        n = len(self._keep)
+        ptrs = ct.POINTER(cudamat) * n
+        self._w = ptrs(*[u[0].p_mat for u in self._keep])
+        self._wd = ptrs(*[u[1].p_mat for u in self._keep])
+        self._g = ptrs(*[u[2].p_mat for u in self._keep])
+        self._n = n
+        self._cache = {}
+
+    def _floats(self, v):
+        seq = [0.0 if x is None else float(x) for x in (v if isinstance(v, (list, tuple)) else [v] * self._n)]
+        if len(seq) != self._n:
+            raise ValueError("one value per parameter expected")
+        return (ct.c_float * self._n)(*seq)
+
+    def apply(self, momentum, epsilon, l2_decay=None, l1_decay=None, reset_gradient=True):
+        key = (repr(momentum), repr(epsilon), repr(l2_decay), repr(l1_decay), bool(reset_gradient))
+        args = self._cache.get(key)
+        if args is None:
+            per = lambda v: list(v) if isinstance(v, (list, tuple)) else [v] * self._n
+            flags = [(1 if a is not None else 0) | (2 if b is not None else 0) | (4 if reset_gradient else 0)
+                     for a, b in zip(per(l2_decay), per(l1_decay))]
+            args = (self._floats(momentum), self._floats(l2_decay), self._floats(l1_decay), self._floats(epsilon),
+                    (ct.c_int * self._n)(*flags))
+            if len(self._cache) > 64:
+                self._cache.clear()
+            self._cache[key] = args
+        _check(_cudamat.momentum_update_many(self._n, self._w, self._wd, self._g, args[0], args[1], args[2], args[3], args[4]))
 
 
 class SparseCUDAMatrix(object):

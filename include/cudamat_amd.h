@@ -204,6 +204,14 @@ int dot_bias_act_sample(rnd_struct* rnd_state, cudamat* mat1, cudamat* mat2, cud
 int momentum_update(cudamat* w, cudamat* w_delta, cudamat* gradient, float momentum, float l2_decay, float l1_decay,
                     float epsilon, int flags);
 
+/* Extension, no counterpart in cudamat.cu: momentum_update for count parameters in one
+ * launch per 8 of them (the weights and biases of a net after a step, deepnet/neuralnet.py:
+ * UpdateEdgeParams / UpdateLayerParams call parameter.py:80-106 once per parameter); every
+ * argument is an array of count entries, results are the bits of count separate calls. */
+int momentum_update_many(int count, cudamat** w, cudamat** w_delta, cudamat** gradient, const float* momentum,
+                         const float* l2_decay, const float* l1_decay, const float* epsilon, const int* flags);
+
+
 /* Extension, no counterpart in cudamat.cu: softmax(mat) -> probs, and from the stored probs
  * loss = -log(probs[label] + tiny) (1 x cols, may be NULL) and grad = probs - onehot(label)
  * (may be NULL) in the same launch: the bits of softmax -> get_softmax_cross_entropy ->

@@ -406,3 +406,48 @@ def test_momentum_update_errors(cm, rng):
     assert lib.momentum_update(a.p_mat, a.p_mat, host.p_mat, 0.9, 0.0, 0.0, 0.01, 0) == -8
     assert lib.momentum_update(a.p_mat, b.T.p_mat, a.p_mat, 0.9, 0.0, 0.0, 0.01, 0) == -7
     assert lib.momentum_update(a.p_mat, b.p_mat, a.p_mat, 0.9, 0.0, 0.0, 0.01, 0) == -1
+
+
+def test_momentum_updates_of_many_parameters_in_one_launch(cm, rng):
+    """MomentumUpdates gives the bits of one momentum_update per parameter: 11 parameters of
+    assorted sizes (two launches), a view that starts 4 bytes into its parent, per-parameter
+    and shared scalars, and the checks of the single call."""
+    shapes = [(64, 48), (48, 1), (10, 1), (1, 1), (257, 33), (128, 128), (5, 7), (1024, 16), (3, 1), (100, 100), (31, 1)]
+    def make():
+        r = np.random.default_rng(5)
+        ws = [cm.CUDAMatrix(np.asarray(r.uniform(-1, 1, s), dtype=np.float32, order='F')) for s in shapes]
+        ds = [cm.CUDAMatrix(np.asarray(r.uniform(-1, 1, s), dtype=np.float32, order='F')) for s in shapes]
+        gs = [cm.CUDAMatrix(np.asarray(r.uniform(-1, 1, s), dtype=np.float32, order='F')) for s in shapes]
+        parent = cm.CUDAMatrix(np.asarray(r.uniform(-1, 1, (1, 41)), dtype=np.float32, order='F'))
+        ws.append(parent.slice(1, 41)); ds.append(cm.CUDAMatrix(np.zeros((1, 40), dtype=np.float32))); gs.append(cm.CUDAMatrix(np.ones((1, 40), dtype=np.float32)))
+        return ws, ds, gs, parent
+    n = len(shapes) + 1
+    moms = [0.5 + 0.03 * i for i in range(n)]
+    l2s = [None if i % 3 == 0 else 0.001 * i for i in range(n)]
+    l1s = [0.0005 * i if i % 4 == 1 else None for i in range(n)]
+    for shared in (False, True):
+        w1, d1, g1, p1 = make()
+        w2, d2, g2, p2 = make()
+        for step in range(2):
+            for i in range(n):
+                if shared:
+                    cm.momentum_update(w1[i], d1[i], g1[i], 0.9, 0.01, l2_decay=0.002, reset_gradient=(step == 1))
+                else:
+                    cm.momentum_update(w1[i], d1[i], g1[i], moms[i], 0.01 + 0.001 * i, l2_decay=l2s[i], l1_decay=l1s[i], reset_gradient=(step == 1))
+            upd = cm.MomentumUpdates(list(zip(w2, d2, g2)))
+            if shared:
+                upd.apply(0.9, 0.01, l2_decay=0.002, reset_gradient=(step == 1))
+            else:
+                upd.apply(moms, [0.01 + 0.001 * i for i in range(n)], l2_decay=l2s, l1_decay=l1s, reset_gradient=(step == 1))
+        for i in range(n):
+            assert np.array_equal(w1[i].asarray(), w2[i].asarray()), i
+            assert np.array_equal(d1[i].asarray(), d2[i].asarray()), i
+            assert np.array_equal(g1[i].asarray(), g2[i].asarray()), i
+        assert np.array_equal(p1.asarray(), p2.asarray())
+    a, b = cm.CUDAMatrix(np.zeros((4, 4), dtype=np.float32)), cm.CUDAMatrix(np.zeros((4, 5), dtype=np.float32))
+    before = a.asarray().copy()
+    with pytest.raises(cm.CUDAMatException):
+        cm.MomentumUpdates([(a, a, a), (a, b, a)]).apply(0.9, 0.01)
+    assert np.array_equal(a.asarray(), before)              # nothing ran
+    with pytest.raises(ValueError):
+        cm.MomentumUpdates([(a, a, a)]).apply([0.9, 0.8], 0.01)
