@@ -435,7 +435,7 @@ k_gemv_cols(const float* M, int ld, int h, int w, const float* x, float* y, floa
   COL_SETUP(TPC)
   const bool stream = (long long)w * h >= DN_STREAM_MIN_ELEMS;
   float s = 0.f;
-  if (active) for_each_in_col<TPC>(M + (size_t)col * ld, h, lane, [&](int r, float v) { s += v * x[r]; }, stream);
+  if (active) for_each_in_col<TPC>(M + (size_t)col * ld, h, lane, [&](int r, float v) { s += x ? v * x[r] : v; }, stream);   // (no weights: a plain sum)
   s = col_combine<TPC, false>(s, lds4);
   if (active && lane == 0) y[col] = (beta == 0.f ? 0.f : beta * y[col]) + alpha * s;
 }
@@ -447,7 +447,8 @@ k_gemv_cols(const float* M, int ld, int h, int w, const float* x, float* y, floa
 // columns (M aligned, ld % 4 == 0) and h % 4 == 0.
 //   COL_DOT: y[j] = beta*y[j] + alpha * sum_i M(i,j) x[i]    COL_SQSUM: the same over M(i,j)^2
 //   COL_MAX: y[j] = max_i M(i,j), starting from -FLT_MAX
-enum { COL_DOT = 0, COL_SQSUM = 1, COL_MAX = 2 };
+//   COL_SUM: COL_DOT with every x[i] = 1, the additions in the same order (so the same bits), no loads of x
+enum { COL_DOT = 0, COL_SQSUM = 1, COL_MAX = 2, COL_SUM = 3 };
 
 template <int CB, int OP, bool STREAM>
 __global__ void __launch_bounds__(256)
@@ -485,6 +486,7 @@ k_colblock(const float* M, int ld, int h, int w, const float* x, float* y, float
         const float4 t = v[k][cb];
         if (OP == COL_DOT) { acc[cb] += t.x * xv[k].x; acc[cb] += t.y * xv[k].y; acc[cb] += t.z * xv[k].z; acc[cb] += t.w * xv[k].w; }
         else if (OP == COL_SQSUM) { acc[cb] += t.x * t.x; acc[cb] += t.y * t.y; acc[cb] += t.z * t.z; acc[cb] += t.w * t.w; }
+        else if (OP == COL_SUM) { acc[cb] += t.x; acc[cb] += t.y; acc[cb] += t.z; acc[cb] += t.w; }
         else acc[cb] = fmaxf(fmaxf(acc[cb], fmaxf(t.x, t.y)), fmaxf(t.z, t.w));
       }
   }
@@ -533,7 +535,8 @@ static bool colblock_launch(const float* M, int ld, int h, int w, const float* x
 // 256*bx .. 256*bx+255 when VEC (4 rows per lane, one 16-byte load per column)
 // or 64*bx .. 64*bx+63 otherwise; its 4 wavefronts take every 4th column, four
 // loads in flight each, and meet in LDS.  With one split the result is final.
-enum { ROW_DOT = 0, ROW_SQSUM = 1, ROW_MAX = 2 };
+//   ROW_SUM:   ROW_DOT with every x[j] = 1 (the same additions in the same order)
+enum { ROW_DOT = 0, ROW_SQSUM = 1, ROW_MAX = 2, ROW_SUM = 3 };
 
 
 template <int OP>
@@ -563,6 +566,7 @@ k_rows_stage1(const float* M, int ld, int h, int w, int cps, const float* x, flo
   auto take = [&](int k, float v, float xj) {
     if (OP == ROW_DOT) acc[k] += v * xj;
     else if (OP == ROW_SQSUM) acc[k] += v * v;
+    else if (OP == ROW_SUM) acc[k] += v;
     else acc[k] = v > acc[k] ? v : acc[k];
   };
   if (row0 < h) {
@@ -698,6 +702,7 @@ k_rows_one(const float* M, int ld, int h, int w, int cps, const float* x, float*
   auto take = [&](int k, float v, float xj) {
     if (OP == ROW_DOT) acc[k] += v * xj;
     else if (OP == ROW_SQSUM) acc[k] += v * v;
+    else if (OP == ROW_SUM) acc[k] += v;
     else acc[k] = v > acc[k] ? v : acc[k];
   };
   if (row0 < h) {
@@ -898,7 +903,7 @@ int dn_noalloc_setup() {
 // Host entry points used by dot() for vector-shaped products.
 int dn_gemv_cols(const float* M, int ld, int h, int w, const float* x, float* y, float alpha, float beta) {
   if (w <= 0) return 0;
-  if (colblock_launch<COL_DOT>(M, ld, h, w, x, y, alpha, beta)) return dn_launch_status();
+  if (x && colblock_launch<COL_DOT>(M, ld, h, w, x, y, alpha, beta)) return dn_launch_status();   // (x NULL: plain sums)
   const int cus = dn_num_cus();
   if (w < cus * 2 && h >= 4096) {
     hipLaunchKernelGGL((k_gemv_cols<256>), dim3(w), dim3(256), 0, dn_stream(), M, ld, h, w, x, y, alpha, beta);
@@ -1208,6 +1213,31 @@ int sqsum_by_axis(cudamat* mat, cudamat* target, int axis, float mult, float p) 
   }
   return ERROR_UNSUPPORTED;
 }
+
+// target = beta * target + alpha * (sums of mat along axis), the kernels that dot() with a vector
+// of ones runs, without the vector: the same additions in the same order, so the same bits.
+// A transposed operand is summed along its other stored axis, as dot() would.
+static int sums_impl(cudamat* mat, cudamat* target, int axis, float beta, float alpha) {
+  if (!mat->on_device || !target->on_device) return ERROR_NOT_ON_DEVICE;
+  if (target->is_trans) return ERROR_TRANSPOSED;
+  if (axis != 0 && axis != 1) return ERROR_UNSUPPORTED;
+  const int h = mat->size[0], w = mat->size[1];
+  const bool along_stored_columns = (axis == 0) != (mat->is_trans != 0);   // one result per stored column
+  const int results = along_stored_columns ? w : h;
+  if (axis == 0 ? (target->size[0] != 1 || target->size[1] != results) : (target->size[0] != results || target->size[1] != 1))
+    return ERROR_INCOMPATIBLE_DIMENSIONS;
+  if (results <= 0) return 0;
+  if (along_stored_columns) {
+    if (colblock_launch<COL_SUM>(mat->data_device, h, h, w, nullptr, target->data_device, alpha, beta)) return dn_launch_status();
+    return dn_gemv_cols(mat->data_device, h, h, w, nullptr, target->data_device, alpha, beta);
+  }
+  return rows_reduce<ROW_SUM>(mat->data_device, h, h, w, nullptr, target->data_device, alpha, beta);
+}
+
+// eigenmat.cc:747-760 (the reference's CPU backend exports these; its cudamat.py spells them as
+// dot() with a vector of ones, cudamat.py:1546-1577 and 724-748).
+int sum_by_axis(cudamat* mat, cudamat* target, int axis) { return sums_impl(mat, target, axis, 0.f, 1.f); }
+int add_sum_by_axis(cudamat* mat, cudamat* target, int axis, float mult) { return sums_impl(mat, target, axis, 1.f, mult); }
 
 }  // extern "C"
 

@@ -108,6 +108,7 @@ _SIGNATURES = {
     'graph_launch': (_i, [ct.c_void_p]), 'graph_free': (_i, [ct.c_void_p]), 'graph_set_stream': (_i, [ct.c_void_p, _i]),
     'max_by_axis': (_i, [_M, _M, _i]), 'max_by_axis_noalloc': (_i, [_M, _M, _i]), 'argmax_by_axis': (_i, [_M, _M, _i]),
     'choose_max_by_axis': (_i, [_M, _M, _i]), 'choose_max_and_accumulate': (_i, [_M, _M]),
+    'sum_by_axis': (_i, [_M, _M, _i]), 'add_sum_by_axis': (_i, [_M, _M, _i, _f]),
     'sqsum_by_axis': (_i, [_M, _M, _i, _f, _f]), 'normlimit_by_axis': (_i, [_M, _M, _i, _f]),
     'apply_log': (_i, [_M, _M, _f]), 'apply_pow': (_i, [_M, _f, _M]),
     'compute_cross_entropy': (_i, [_M, _M, _M, _f]),
@@ -400,17 +401,11 @@ class CUDAMatrix(object):
 
     def add_sums(self, mat, axis, mult=1.):
         """self += mult * (sums of mat along axis)."""
-        sz = mat.mat.size                      # (what get_leading / get_nonleading_dimension return)
-        m, n = (sz[1], sz[0]) if mat.mat.is_trans else (sz[0], sz[1])
-        if axis == 0:
-            left = _ones(m, trans=True)
-            right = mat
-        elif axis == 1:
-            left = mat
-            right = _ones(n)
-        else:
+        if axis not in (0, 1):
             raise ValueError("axis must be 0 or 1.")
-        _check(_cudamat.dot(left.p_mat, right.p_mat, self.p_mat, 1., float(mult)))
+        # (the reference multiplies by a vector of ones, cudamat.py:724-748; add_sum_by_axis runs
+        # the same kernels without reading the vector and leaves the same bits)
+        _check(_cudamat.add_sum_by_axis(mat.p_mat, self.p_mat, int(axis), float(mult)))
         return self
 
     def cumsum(self, axis, temp=None, target=None):
@@ -787,23 +782,21 @@ def _ones(n, trans=False):
 
 
 def sum(mat, axis, target=None):
-    """Sum along axis: 0 = leading dimension, 1 = non-leading.  Goes through dot() with
-    a vector of ones, so a transposed operand is honoured (cudamat.py:1546-1577)."""
+    """Sum along axis: 0 = leading dimension, 1 = non-leading, of the matrix as it is seen (a
+    transposed operand is honoured).  The reference multiplies by a vector of ones
+    (cudamat.py:1546-1577); sum_by_axis runs the same kernels without reading the vector and
+    leaves the same bits."""
     m = _cudamat.get_leading_dimension(mat.p_mat)
     n = _cudamat.get_nonleading_dimension(mat.p_mat)
     if axis == 0:
-        left = _ones(m, trans=True)
-        right = mat
         if target is None:
             target = empty((1, n))
     elif axis == 1:
-        left = mat
-        right = _ones(n)
         if target is None:
             target = empty((m, 1))
     else:
         raise ValueError("axis must be 0 or 1.")
-    _check(_cudamat.dot(left.p_mat, right.p_mat, target.p_mat, 0., 1.))
+    _check(_cudamat.sum_by_axis(mat.p_mat, target.p_mat, int(axis)))
     return target
 
 

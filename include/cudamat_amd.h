@@ -153,6 +153,12 @@ int max_by_axis_noalloc(cudamat* mat, cudamat* target, int axis);
 int argmax_by_axis(cudamat* mat, cudamat* target, int axis);
 int choose_max_by_axis(cudamat* mat, cudamat* target, int axis);
 int choose_max_and_accumulate(cudamat* mat, cudamat* acc);
+/* eigenmat.cc:733-760 (exported by the reference's CPU backend; its cudamat.py spells them as
+ * dot() with a vector of ones, cudamat.py:724-748 and 1546-1577): target = sums of mat along
+ * axis (0: one per column, 1: one per row; the other axis for a transposed mat), or
+ * target += mult * sums.  The kernels of those dot() calls without the vector: same bits. */
+int sum_by_axis(cudamat* mat, cudamat* target, int axis);
+int add_sum_by_axis(cudamat* mat, cudamat* target, int axis, float mult);
 int sqsum_by_axis(cudamat* mat, cudamat* target, int axis, float mult, float p);
 int normlimit_by_axis(cudamat* mat, cudamat* target, int axis, float norm);
 

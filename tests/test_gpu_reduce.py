@@ -242,3 +242,28 @@ def test_softmax_ce_grad_errors(cm, rng):
     assert lib.softmax_ce_grad(X.T.p_mat, L.p_mat, X.p_mat, None, None, 0.0) == -5
     host = cm.CUDAMatrix(np.zeros((1, 4), dtype=np.float32), copy_to_device=False)
     assert lib.softmax_ce_grad(X.p_mat, host.p_mat, X.p_mat, None, None, 0.0) == -8
+
+
+@pytest.mark.parametrize("shape", [(1, 1), (37, 53), (500, 100), (784, 128), (10, 128), (1000, 999), (4096, 1100), (1100, 4096),
+                                   (2048, 2048), (4096, 64)])
+def test_sums_leave_the_bits_of_dot_with_a_vector_of_ones(cm, rng, shape):
+    """sum / add_sums run the kernels that dot() with a vector of ones would run (the reference's
+    spelling, cudamat.py:724-748 and 1546-1577) without reading the vector: the same bits, also
+    for a transposed operand and with an accumulating target."""
+    x = _rand(rng, shape)
+    a = cm.CUDAMatrix(x)
+    h, w = shape
+    ones_h = cm.CUDAMatrix(np.ones((h, 1), dtype=np.float32)); ones_w = cm.CUDAMatrix(np.ones((w, 1), dtype=np.float32))
+    assert np.array_equal(a.sum(axis=0).asarray(), cm.dot(ones_h.T, a).asarray())
+    assert np.array_equal(a.sum(axis=1).asarray(), cm.dot(a, ones_w).asarray())
+    assert np.array_equal(cm.sum(a.T, axis=0).asarray(), cm.dot(ones_w.T, a.T).asarray())
+    assert np.array_equal(cm.sum(a.T, axis=1).asarray(), cm.dot(a.T, ones_h).asarray())
+    base = _rand(rng, (h, 1))
+    t1, t2 = cm.CUDAMatrix(base), cm.CUDAMatrix(base)
+    t1.add_sums(a, axis=1, mult=0.25)
+    t2.add_dot(a, ones_w, mult=0.25)
+    assert np.array_equal(t1.asarray(), t2.asarray())
+    with pytest.raises(cm.CUDAMatException, match="Incompatible matrix dimensions"):
+        a.sum(axis=0, target=cm.empty((1, w + 1)))
+    with pytest.raises(cm.CUDAMatException, match="Incompatible matrix dimensions"):
+        cm.empty((h + 1, 1)).add_sums(a, axis=1)
