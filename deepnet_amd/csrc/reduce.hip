@@ -567,7 +567,7 @@ k_rows_stage1(const float* M, int ld, int h, int w, int cps, const float* x, flo
     if (OP == ROW_DOT) acc[k] += v * xj;
     else if (OP == ROW_SQSUM) acc[k] += v * v;
     else if (OP == ROW_SUM) acc[k] += v;
-    else acc[k] = v > acc[k] ? v : acc[k];
+    else acc[k] = fmaxf(acc[k], v);
   };
   if (row0 < h) {
     // U columns of this wavefront in flight per trip; a column past the range is
@@ -703,7 +703,7 @@ k_rows_one(const float* M, int ld, int h, int w, int cps, const float* x, float*
     if (OP == ROW_DOT) acc[k] += v * xj;
     else if (OP == ROW_SQSUM) acc[k] += v * v;
     else if (OP == ROW_SUM) acc[k] += v;
-    else acc[k] = v > acc[k] ? v : acc[k];
+    else acc[k] = fmaxf(acc[k], v);
   };
   if (row0 < h) {
     for (int j = j0 + wv * 4 + c; j < j1; j += NW * 4 * U) {
