@@ -774,10 +774,24 @@ struct RowsWorkspace {
 // (few rows, very many columns): such shapes keep the two-stage kernels.
 static int rows_one_splits(int h, int w) {
   const int bx = (h + 63) / 64;
-  int splits = (dn_num_cus() + bx / 2) / bx;
+  const int cus = dn_num_cus();
+  int splits = (cus + bx / 2) / bx;
   if (splits > w / 256) splits = w / 256;
   if (splits < 1) splits = 1;
-  return splits <= ROWS_ONE_MAX_SPLITS ? splits : 0;
+  if (splits > ROWS_ONE_MAX_SPLITS) return 0;
+  // A few workgroups more than CUs double the time of the busiest CU (65 row blocks x 4 slices on
+  // 256 CUs: 22.4 us where 64 x 4 take 13.3): among the slice counts allowed, take the one with
+  // the smallest (workgroups on the busiest CU) x (columns per workgroup).
+  if (bx * splits > cus) {
+    long long best = -1;
+    int best_s = splits;
+    for (int s = 1; s <= ROWS_ONE_MAX_SPLITS && s <= (w / 256 > 1 ? w / 256 : 1); ++s) {
+      const long long cost = (long long)((bx * s + cus - 1) / cus) * ((w + s - 1) / s);
+      if (best < 0 || cost < best) { best = cost; best_s = s; }
+    }
+    splits = best_s;
+  }
+  return splits;
 }
 
 template <int OP>
