@@ -1320,9 +1320,11 @@ static int softmax_impl(const float* in, float* out, int w, int h, SoftmaxExtras
   if (w <= 0 || h <= 0) return 0;
   const bool reg_ok = (h % 4 == 0) && dn_aligned16(in) && dn_aligned16(out) && h <= 64 * 4 * 16 &&
                       (!x.grad || dn_aligned16(x.grad));
-  // (columns of more than 3072 rows in a streamed matrix measured faster on one wavefront per
-  // column, 24.0 against 26.3 us at 4096 x 4096; every other tall shape on the workgroup kernel)
-  if (reg_ok && h > 1024 && w >= 8 * dn_num_cus() && !(h > 3072 && (long long)w * h >= DN_STREAM_MIN_ELEMS)) {
+  // (4096 x 4096 measured faster on one wavefront per column, 24.0 against 26.3 us; every
+  // other tall shape on the workgroup kernel: 4000 x 4224 29.4 against 34.2 us, 3400 x 5000 27.8
+  // against 32.7, 4096 x 8192 46.2 against 49.9)
+  const bool one_wave_per_column = h == 4096 && (long long)w * h >= DN_STREAM_MIN_ELEMS && (long long)w * h < (1ll << 25);
+  if (reg_ok && h > 1024 && w >= 8 * dn_num_cus() && !one_wave_per_column) {
     const int n4 = h / 4;
     dim3 grid((w + 3) / 4), block(256);
     const bool stream = (long long)w * h >= DN_STREAM_MIN_ELEMS;
