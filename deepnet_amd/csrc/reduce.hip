@@ -1343,6 +1343,13 @@ static int softmax_impl(const float* in, float* out, int w, int h, SoftmaxExtras
     else hipLaunchKernelGGL((k_col_softmax_reg<16>), grid, block, 0, dn_stream(), in, out, w, h, x);
     return dn_launch_status();
   }
+  // columns of 4097 to 16384 rows still fit the registers of a workgroup (two columns or one at
+  // a time): one read and one write instead of the three passes below
+  if ((h % 4 == 0) && dn_aligned16(in) && dn_aligned16(out) && (!x.grad || dn_aligned16(x.grad)) && h > 4096 && h <= 16384) {
+    if (h <= 8192) hipLaunchKernelGGL((k_col_softmax_blk<8, 2, false>), dim3((w + 1) / 2), dim3(256), 0, dn_stream(), in, out, w, h, x);
+    else hipLaunchKernelGGL((k_col_softmax_blk<16, 1, false>), dim3(w), dim3(256), 0, dn_stream(), in, out, w, h, x);
+    return dn_launch_status();
+  }
   return launch_cols(k_col_softmax<64>, k_col_softmax<256>, w, h, in, out, w, h, x);
 }
 

@@ -105,7 +105,9 @@ def test_choose_max_and_accumulate(cm, rng):
     assert np.array_equal(acc.asarray(), acc0 + orc.choose_max_by_axis(x, 0).astype(np.float32))
 
 
-@pytest.mark.parametrize("shape", [(100, 10), (10, 128), (4096, 64), (1000, 33), (37, 53), (5, 1), (20000, 3)])
+# (columns of up to 4096, 8192 and 16384 rows have kernels of their own, longer ones three passes)
+@pytest.mark.parametrize("shape", [(100, 10), (10, 128), (4096, 64), (1000, 33), (37, 53), (5, 1), (20000, 3), (4100, 37), (8192, 9),
+                                   (10000, 5), (16384, 3), (16388, 2), (5001, 4)])
 def test_softmax(cm, rng, shape):
     x = _rand(rng, shape, -8, 8)
     a, t = cm.CUDAMatrix(x), cm.empty(shape)
@@ -203,7 +205,7 @@ def test_full_size_4096_sum_max_softmax(cm, rng, axis):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("h,w", [(10, 128), (1000, 64), (4096, 33), (7, 5), (256, 256)])
+@pytest.mark.parametrize("h,w", [(10, 128), (1000, 64), (4096, 33), (7, 5), (256, 256), (2048, 2100), (4100, 40), (10000, 12), (16384, 2)])
 def test_softmax_ce_grad_is_bit_identical_to_the_three_calls(cm, rng, h, w):
     # both softmax kernels (columns held in registers: h % 4 == 0; generic otherwise)
     x = np.asarray(3.0 * rng.standard_normal((h, w)), dtype=np.float32, order='F')
