@@ -178,6 +178,71 @@ k_pool_undo_fixed(const float* imgs, const float* maxGrads, const float* maxActs
   }
 }
 
+// The same for stride 2 on larger maps, start 0: a lane takes a 2 x 2 block of pixels (rows
+// 2i, 2i+1, columns 2j, 2j+1).  The windows that cover any of them are (i-1 | i, j-1 | j), so
+// the block's four pixels share four loads of each pooled array where one pixel at a time
+// asks for four of its own: a quarter of the requests to the caches, which is what bounds
+// the one-pixel kernel (96 maps of 55 x 55 at batch 128: 95 -> 68 us).  Every
+// pixel adds its windows in the order of the one-pixel kernel, so the results are the same bits.
+template <int SUBS>
+__global__ void __launch_bounds__(256)
+k_pool_undo_block2(const float* imgs, const float* maxGrads, const float* maxActs, float* target, PoolGeom g, int B, FastDiv dB) {
+  const uint32_t total = (uint32_t)g.NV * B * B * g.F;
+  for (uint32_t e = blockIdx.x * 256u + threadIdx.x; e < total; e += gridDim.x * 256u) {
+    int nv, bx, by, f;
+    decode4(e, g.dNV, dB, B, &nv, &bx, &by, &f);
+    Vec<4> ma[2][2], mg[2][2];
+    bool in[2][2];
+#pragma unroll
+    for (int jy = 0; jy < 2; ++jy) {
+      const int oy = by - 1 + jy;
+      const int oyc = oy < 0 ? 0 : (oy >= g.O ? g.O - 1 : oy);
+#pragma unroll
+      for (int jx = 0; jx < 2; ++jx) {
+        const int ox = bx - 1 + jx;
+        const int oxc = ox < 0 ? 0 : (ox >= g.O ? g.O - 1 : ox);
+        in[jy][jx] = (oy >= 0) & (oy < g.O) & (ox >= 0) & (ox < g.O);
+        const size_t ooff = (size_t)g.N * ((size_t)(f * g.O + oyc) * g.O + oxc) + nv * 4;
+        ma[jy][jx] = Vec<4>::load(maxActs + ooff);
+        mg[jy][jx] = Vec<4>::load(maxGrads + ooff);
+      }
+    }
+    Vec<4> img[2][2];
+#pragma unroll
+    for (int dy = 0; dy < 2; ++dy)
+#pragma unroll
+      for (int dx = 0; dx < 2; ++dx) {
+        const int py = 2 * by + dy, px = 2 * bx + dx;
+        const int pyc = py < g.S ? py : g.S - 1, pxc = px < g.S ? px : g.S - 1;
+        img[dy][dx] = Vec<4>::load(imgs + (size_t)g.N * ((size_t)(f * g.S + pyc) * g.S + pxc) + nv * 4);
+      }
+#pragma unroll
+    for (int dy = 0; dy < 2; ++dy)
+#pragma unroll
+      for (int dx = 0; dx < 2; ++dx) {
+        const int py = 2 * by + dy, px = 2 * bx + dx;
+        if (py >= g.S || px >= g.S) continue;
+        Vec<4> acc;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc.v[i] = 0.f;
+#pragma unroll
+        for (int jy = 0; jy < 2; ++jy)
+#pragma unroll
+          for (int jx = 0; jx < 2; ++jx) {
+            // window (by - 1 + jy, bx - 1 + jx) starts at row 2*(by - 1 + jy): the pixel is inside it
+            // when its offset from that row, 2 - 2*jy + dy, is below SUBS (likewise along x)
+            const bool ok = in[jy][jx] & (2 - 2 * jy + dy < SUBS) & (2 - 2 * jx + dx < SUBS);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const float t = (img[dy][dx].v[i] == ma[jy][jx].v[i] ? 1.f : 0.f) * mg[jy][jx].v[i];
+              acc.v[i] += ok ? t : 0.f;
+            }
+          }
+        acc.store(target + (size_t)g.N * ((size_t)(f * g.S + py) * g.S + px) + nv * 4);
+      }
+  }
+}
+
 // x^y for the normalisation layers through the hardware log2 / exp2 (the reference uses
 // __powf there, cudamat_conv_kernels.cu:112-176); relative error below 1e-6 for the
 // denominators these layers see (1 <= x < ~1e3).
@@ -733,7 +798,20 @@ void MaxPoolUndo(cudamat* images, cudamat* maxGrads, cudamat* maxActs, cudamat* 
   PoolGeom g;
   make_geom(g, N, F, S, outputsX, subsX, startX, strideX, v4 ? 4 : 1);
   const unsigned grid = grid_for(total / (v4 ? 4 : 1));
-  if (v4 && g.subs == 3 && g.stride == 2)
+  // (measured against the one-pixel kernel at batch 128: 64 maps of 32 x 32 17.7 -> 16.2 us, of
+  // 24 x 24 12.8 -> 9.4 us, 256 of 27 x 27 56.9 -> 42.8 us, 96 of 55 x 55 95 -> 68 us; 64 maps of
+  // 32 x 32 at batch 256 30.5 -> 31.9 us)
+  if (v4 && g.stride == 2 && g.start == 0 && (g.subs == 2 || g.subs == 3) && g.S >= 4) {
+    const int B = (g.S + 1) / 2;
+    const FastDiv dB = make_fastdiv((uint32_t)B);
+    const unsigned grid2 = grid_for((long long)g.NV * B * B * g.F);
+    if (g.subs == 3)
+      hipLaunchKernelGGL((k_pool_undo_block2<3>), dim3(grid2), dim3(256), 0, dn_stream(), (const float*)images->data_device,
+                         (const float*)maxGrads->data_device, (const float*)maxActs->data_device, targets->data_device, g, B, dB);
+    else
+      hipLaunchKernelGGL((k_pool_undo_block2<2>), dim3(grid2), dim3(256), 0, dn_stream(), (const float*)images->data_device,
+                         (const float*)maxGrads->data_device, (const float*)maxActs->data_device, targets->data_device, g, B, dB);
+  } else if (v4 && g.subs == 3 && g.stride == 2)
     hipLaunchKernelGGL((k_pool_undo_fixed<3, 2>), dim3(grid), dim3(256), 0, dn_stream(), (const float*)images->data_device,
                        (const float*)maxGrads->data_device, (const float*)maxActs->data_device, targets->data_device, g);
   else if (v4 && g.subs == 2 && g.stride == 2)

@@ -153,6 +153,9 @@ POOLS = [  # N, F, S, subs, start, stride
     # the reference changes kernels (kLocalPool2, cudamat_conv.cu:1040-1089)
     (8, 4, 12, 6, 0, 1), (8, 4, 12, 6, 0, 2), (16, 2, 13, 7, 0, 1), (16, 2, 13, 7, -3, 2), (4, 3, 14, 6, -2, 2),
     (128, 16, 16, 7, -3, 1),
+    # larger maps with stride 2 from 0 (the gradient kernel that takes 2 x 2 pixels per lane: odd and
+    # even sizes, windows of 3 and 2, outputs that stop short of the last rows)
+    (8, 3, 55, 3, 0, 2), (4, 2, 40, 3, 0, 2), (4, 2, 41, 2, 0, 2), (8, 2, 44, 2, 0, 2), (4, 3, 47, 3, 0, 2),
 ]
 
 
@@ -410,3 +413,25 @@ def test_benchmark_layers_at_full_size_on_sampled_outputs(cm, cc, N, C, H, F, k,
     assert abs(a - b) / scale < 1e-5 and abs(a - c_) / scale < 1e-5
     for m in (X, W, Y, up, down, outp):
         m.free_device_memory()
+
+
+@pytest.mark.parametrize("S,subs,O", [(55, 3, 27), (40, 3, 20), (41, 2, 21), (48, 2, 24), (46, 3, 20), (5, 3, 2), (8, 2, 4), (9, 3, 4), (32, 3, 16)])
+def test_pool_gradient_in_blocks_has_the_bits_of_the_general_kernel(cm, cc, rng, S, subs, O):
+    """Windows of 2 or 3 with stride 2 from 0 take a kernel that handles 2 x 2 pixels per lane; it adds the same
+    terms in the same order as the general kernel, which the same images reach in a batch that is
+    not a multiple of 4."""
+    N, F = 8, 3
+    x = _f(rng.integers(-3, 4, (N, F * S * S)))          # small integers: plenty of ties
+    g = _f(rng.standard_normal((N, F * O * O)))
+    X, T = cm.CUDAMatrix(x), cm.empty((N, F * O * O))
+    cc.MaxPool(X, T, F, subs, 0, 2, O)
+    U = cm.empty((N, F * S * S))
+    cc.MaxPoolUndo(X, U, cm.CUDAMatrix(g), T, subs, 0, 2, O)
+    want = co.max_pool_undo(x, g, T.asarray(), subs, 0, 2, O)
+    assert np.allclose(U.asarray(), want, rtol=1e-6, atol=1e-6)
+    # one image more in front: N = 9 is not a multiple of 4, so the general kernel runs; its columns 1..8 are the same problem
+    x9 = np.vstack([x[:1], x]); g9 = np.vstack([g[:1], g])
+    X9, T9, U9 = cm.CUDAMatrix(_f(x9)), cm.empty((N + 1, F * O * O)), cm.empty((N + 1, F * S * S))
+    cc.MaxPool(X9, T9, F, subs, 0, 2, O)
+    cc.MaxPoolUndo(X9, U9, cm.CUDAMatrix(_f(g9)), T9, subs, 0, 2, O)
+    assert np.array_equal(U9.asarray()[1:], U.asarray())
