@@ -889,7 +889,13 @@ static int gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, co
   // reads 16 such rows per load instruction and they meet in the same memory channels (measured
   // 1024 x 128 x 1024 with both leading dimensions 1024: 9.2 us against 8.5 us on 32 x 32 blocks).
   const bool kc_aliased = a_kc && b_kc && (lda % 256 == 0 || ldb % 256 == 0);
-  if (tiles64 < cus && off32 && !heavy && (tiles32 * 5 <= cus * 2 || (tiles32 * 2 <= cus && !kc_aliased))) {
+  // With both operands K-contiguous a CU's time goes with the operand bytes it pulls through its L1:
+  // more 16 x 16 blocks than CUs then means a second round on some of them, and from K = 1024 on the
+  // 32 x 32 blocks below are faster (1536 x 64 x 4096: 30.3 us against 2048 x 64 x 4096 on them in 25.9).
+  const long long tiles16 = (long long)((M + 15) / 16) * ((N + 15) / 16);
+  const bool t16_second_round = a_kc && b_kc && tiles16 > cus && K >= 1024;
+  if (tiles64 < cus && off32 && !heavy && !t16_second_round &&
+      (tiles32 * 5 <= cus * 2 || (tiles32 * 2 <= cus && !kc_aliased))) {
     // 32 x 32 blocks would leave half or more of the CUs idle: 16 x 16 blocks, K over 4 wavefronts
     // (measured against 32 x 32 blocks: 500 x 100 x 784 4.4 us against 7.7, 1024 x 128 x 784 6.5 against
     // 7.9, 1024 x 128 x 1024 with an M-contiguous first operand 7.2 against 8.8; against 8 wavefronts per
