@@ -913,7 +913,14 @@ static int gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, co
     if (sampled) *sampled = epi.sample != nullptr;
     return dn_launch_status();
   }
-  if (tiles64 < cus && off32 && !heavy) {
+  // 32 x 32 blocks, K over 8 wavefronts: a CU takes them two at a time in rounds of about 5 us per 512
+  // of K, so up to two rounds they beat one 64 x 64 tile per CU (512 x 1024 x 512: 10.2 us against
+  // 15.0, x 1024: 17.2 against 25.4) and from the third round on they do not (784 x 1000 x 200: 14.8 us
+  // against 9.0, x 1024: 37.6 against 25.9; 832 x 832 x 2048: 53.3 against 37.2). Two rounds of long
+  // reductions over operands that are both contiguous along the rows of the product lose to tiles with
+  // a split K (512 x 1024 x 2048: 39.2 us against 27.5).
+  const bool mn_both = !a_kc && !b_kc;
+  if (tiles32 <= 2ll * cus && !(mn_both && K >= 2048 && tiles32 > cus) && off32 && !heavy) {
     dim3 grid((M + 31) / 32, (N + 31) / 32);
 #define GEMM_SMALL(AK, BK_)                                                                                  \
   do {                                                                                                       \
@@ -954,7 +961,9 @@ static int gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, co
     // The second kernel costs about 5 us and a split slice starts its pipeline anew: measured
     // on 1024 x 1024 outputs a split only pays from K = 2048 on (K = 128: 13 us split, 7.5 us
     // whole), and with 1.5 tiles per CU (1280 x 1280) it never does.
-    if ((K < 2048 && !(heavy && K >= 1024)) || tiles * 4 >= (long long)cus * 5) want = 1;
+    // With four slices or more (tiles on two thirds of the CUs at most) it pays from K = 1024 on
+    // (768 x 768 x 1024: 23.4 us against 25.9, x 1536: 29.9 against 36.3).
+    if ((K < 2048 && !(K >= 1024 && (heavy || want >= 4))) || tiles * 4 >= (long long)cus * 5) want = 1;
     if (want > 1) splits = (int)want;
   }
   int kps = ((K + splits - 1) / splits + GEMM_BK - 1) / GEMM_BK * GEMM_BK;
