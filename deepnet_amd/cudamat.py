@@ -126,7 +126,7 @@ _SIGNATURES = {
     'allocate_device_memory_sparse': (_i, [_S]), 'copy_sparse_to_device': (_i, [_S]),
     'free_device_memory_sparse': (_i, [_S]),
     'sparse_dot': (_i, [_S, _M, _M, _f, _f]),
-    'vdot': (_f, [_M, _M, ct.POINTER(_i)]), 'euclid_norm': (_f, [_M, ct.POINTER(_i)]),
+    'vdot': (_f, [_M, _M, ct.POINTER(_i)]), 'euclid_norm': (_f, [_M, ct.POINTER(_i)]), 'sum_all': (_f, [_M, ct.POINTER(_i)]),
     'add_mult': (_i, [_M, _M, _f]), 'add_mult_sign': (_i, [_M, _M, _f]),
     'assign_scalar': (_i, [_M, _f]),
     'selectRows': (_i, [_M, _M, _M]), 'setSelectedRows': (_i, [_M, _M, _M]),
@@ -396,7 +396,12 @@ class CUDAMatrix(object):
         """Sum along axis (0 = leading dimension, 1 = non-leading); None sums everything
         and returns a Python float."""
         if axis is None:
-            return vdot(self, _ones(self.shape[0] * self.shape[1]))
+            # (the reference takes vdot() with a vector of ones, cudamat.py:719-720; sum_all is that
+            # kernel without the reads of the vector and leaves the same bits)
+            err_code = ct.c_int(0)
+            res = _cudamat.sum_all(self.p_mat, ct.byref(err_code))
+            _check(err_code.value)
+            return res
         return sum(self, axis, target)
 
     def add_sums(self, mat, axis, mult=1.):

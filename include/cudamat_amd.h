@@ -159,6 +159,10 @@ int choose_max_and_accumulate(cudamat* mat, cudamat* acc);
  * target += mult * sums.  The kernels of those dot() calls without the vector: same bits. */
 int sum_by_axis(cudamat* mat, cudamat* target, int axis);
 int add_sum_by_axis(cudamat* mat, cudamat* target, int axis, float mult);
+/* eigenmat.cc:864 (sum of every element; cudamat.py:719-720 spells it vdot() with a vector of ones
+ * as long as the matrix).  vdot's kernel without the vector, same bits; the error code comes back
+ * the way vdot and euclid_norm hand it back. */
+float sum_all(cudamat* mat, int* err_code);
 int sqsum_by_axis(cudamat* mat, cudamat* target, int axis, float mult, float p);
 int normlimit_by_axis(cudamat* mat, cudamat* target, int axis, float norm);
 

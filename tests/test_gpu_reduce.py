@@ -97,6 +97,36 @@ def test_sqsum_and_norm_limit_and_choose_max(cm, rng, shape, axis):
     assert np.array_equal(a.asarray(), orc.choose_max_by_axis(x, axis).astype(np.float32))
 
 
+@pytest.mark.parametrize("shape", [(4, 3), (512, 37), (516, 9), (784, 1024), (1024, 130), (1028, 64), (2048, 70), (2052, 33), (4096, 600),
+                                   (4096, 12), (4100, 16), (1001, 40)])
+def test_norm_limit_of_columns_held_in_registers(cm, rng, shape):
+    """Columns of up to 4096 rows (a multiple of 4) are read once; taller or ragged ones take the
+    general kernel.  Against the oracle (cudamat_kernels.cu:1100-1130), in place as well, and against
+    the general kernel, which a view of the same column at an odd offset runs (other lanes add the
+    squares there, so the norms agree to rounding)."""
+    h, w = shape
+    x = _rand(rng, shape)
+    x[:, 0] *= 1e-3                     # a column under the limit stays as it is
+    a = cm.CUDAMatrix(x)
+    norm = float(np.median(np.sqrt((x.astype(np.float64) ** 2).sum(axis=0))))
+    lim = cm.empty(shape)
+    a.norm_limit(norm, 0, target=lim)
+    want = orc.normlimit_by_axis(x, 0, norm)
+    got = lim.asarray().copy()
+    assert np.allclose(got, want, rtol=1e-5, atol=1e-7)
+    assert np.array_equal(got[:, 0], x[:, 0])
+    # one column at a time out of a taller matrix, starting one row down: unaligned, general kernel
+    tall = np.zeros((h + 1, w), dtype=np.float32, order='F'); tall[1:, :] = x
+    T = cm.CUDAMatrix(tall)
+    for c in (0, w // 2, w - 1):
+        part = T.slice(c, c + 1).reshape((1, h + 1)).slice(1, h + 1).reshape((h, 1))   # a view, 4 bytes off
+        out = cm.empty((h, 1))
+        part.norm_limit(norm, 0, target=out)
+        assert np.allclose(out.asarray().ravel(), got[:, c], rtol=2e-6, atol=0), c
+    a.norm_limit(norm, 0)
+    assert np.array_equal(a.asarray(), got)
+
+
 def test_choose_max_and_accumulate(cm, rng):
     x = _rand(rng, (10, 40))
     acc0 = np.ones((10, 40), dtype=np.float32, order='F')
@@ -269,3 +299,7 @@ def test_sums_leave_the_bits_of_dot_with_a_vector_of_ones(cm, rng, shape):
         a.sum(axis=0, target=cm.empty((1, w + 1)))
     with pytest.raises(cm.CUDAMatException, match="Incompatible matrix dimensions"):
         cm.empty((h + 1, 1)).add_sums(a, axis=1)
+    # the sum of everything: vdot() with as many ones (cudamat.py:719-720), without reading them
+    ones_all = cm.CUDAMatrix(np.ones((h, w), dtype=np.float32))
+    assert np.float32(a.sum()).tobytes() == np.float32(cm.vdot(a, ones_all)).tobytes()
+    assert abs(a.sum() - x.astype(np.float64).sum()) <= 1e-5 * np.abs(x).astype(np.float64).sum()
