@@ -857,11 +857,18 @@ static int gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, co
   // its own wavefronts.
   const long long tiles64 = (long long)((M + 63) / 64) * ((N + 63) / 64);
   const bool off32 = (size_t)lda * (a_kc ? M : K) < (1u << 30) && (size_t)ldb * (b_kc ? N : K) < (1u << 30);
-  // That kernel re-reads its operands from L2 for every 32 x 32 block ((M/32)(N/32) 64 K floats):
-  // beyond about 1.5e9 multiply-adds that traffic costs more than LDS tiles with a split K
-  // (measured: 4096 x 128 x 4096 66 us against 53 us, 2048 x 128 x 2048 17.7 against 21.4).
-  const bool heavy = (double)M * (double)N * (double)K >= 1.5e9;
+  // The kernels that split K over the wavefronts of a workgroup read their operands straight from L2
+  // and L1, and a CU's time goes with what it pulls through: per 1024 of K about 4 us while the
+  // 16 x 16 blocks fit one round of the CUs, 6.2 us up to one 32 x 32 block per CU (or a second round
+  // of 16 x 16 blocks), 15.5 us up to two.  LDS tiles with a split K cost about 12 us plus 1.5 us per
+  // 1e8 multiply-adds, second kernel included, and take over where that is less (measured, us:
+  // 4096 x 128 x 4096 66 -> 53, 1024 x 128 x 8192 45 -> 29, 3000 x 128 x 3000 44 -> 36, 1024 x 128 x 4096
+  // 24.1 -> 19.5; they stay behind on 2048 x 128 x 2048, 15.1 against 20.3, and 4096 x 128 x 1024,
+  // 17.2 against 19.2).
   const long long tiles32 = (long long)((M + 31) / 32) * ((N + 31) / 32);
+  const long long tiles16 = (long long)((M + 15) / 16) * ((N + 15) / 16);
+  const double per_1024 = tiles16 <= cus ? 4.0 : tiles32 <= cus ? 6.2 : 15.5;
+  const bool heavy = 12.0 + 1.5e-8 * (double)M * (double)N * (double)K < per_1024 * (double)K / 1024.0;
   if (K <= BOX_K && tiles64 >= cus / 2 && tiles64 <= 2 * cus) {
     // short reductions on about one 64 x 64 tile per CU: the whole K extent at once (measured against
     // the kernels below: 784 x 1024 x 128 6.3 us against 8.4, 1024 x 1024 x 128 with beta = 1 6.1
@@ -892,7 +899,6 @@ static int gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, co
   // With both operands K-contiguous a CU's time goes with the operand bytes it pulls through its L1:
   // more 16 x 16 blocks than CUs then means a second round on some of them, and from K = 1024 on the
   // 32 x 32 blocks below are faster (1536 x 64 x 4096: 30.3 us against 2048 x 64 x 4096 on them in 25.9).
-  const long long tiles16 = (long long)((M + 15) / 16) * ((N + 15) / 16);
   const bool t16_second_round = a_kc && b_kc && tiles16 > cus && K >= 1024;
   if (tiles64 < cus && off32 && !heavy && !t16_second_round &&
       (tiles32 * 5 <= cus * 2 || (tiles32 * 2 <= cus && !kc_aliased))) {
