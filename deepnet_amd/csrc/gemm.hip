@@ -104,7 +104,9 @@ __device__ __forceinline__ f32x4 gemm_load4(const float* base, int c, int c_lim,
 // gridDim.z > 1 splits K; then each z-slice writes its raw partial tile to
 // `partial` (M x N, ld = M, one slab per slice) and a second kernel applies
 // alpha/beta.  K slices are multiples of GEMM_BK.
-template <int WM, int WN, bool A_KC, bool B_KC>
+// PF (even): the number of register sets that take slabs from global memory in the main loop, where the
+// fragments of a slab are read from LDS one iteration ahead of their MFMAs, into a second register set.
+template <int WM, int WN, bool A_KC, bool B_KC, int PF = 2>
 __global__ void __launch_bounds__(256)
 k_gemm(const float* __restrict__ A, int lda, const float* __restrict__ B, int ldb, float* C, int ldc, int M, int N,
        int K, int k_per_split, float alpha, float beta, float* partial, bool a_vec, bool b_vec, GemmEpilogue epi) {
@@ -265,7 +267,97 @@ k_gemm(const float* __restrict__ A, int lda, const float* __restrict__ B, int ld
   // the checked loop.
   const bool fast = a_fast && b_fast;
   int buf = 0, k0 = kbeg;
-  if (fast && kbeg + 2 * GEMM_BK <= kend) {
+#define GEMM_FRAGS(BUF, AV, BV)                                                                        \
+  do {                                                                                                 \
+    _Pragma("unroll") for (int kk = 0; kk < GEMM_BK / 2; ++kk) {                                       \
+      _Pragma("unroll") for (int i = 0; i < WM; ++i)                                                   \
+        AV[kk][i] = As[BUF][kk + (GEMM_BK / 2) * lk][wm * 32 * WM + i * 32 + li];                      \
+      _Pragma("unroll") for (int j = 0; j < WN; ++j)                                                   \
+        BV[kk][j] = Bs[BUF][kk + (GEMM_BK / 2) * lk][wn * 32 * WN + j * 32 + li];                      \
+    }                                                                                                  \
+  } while (0)
+#define GEMM_MFMAS(AV, BV)                                                                             \
+  do {                                                                                                 \
+    _Pragma("unroll") for (int kk = 0; kk < GEMM_BK / 2; ++kk)                                         \
+      _Pragma("unroll") for (int j = 0; j < WN; ++j)                                                   \
+        _Pragma("unroll") for (int i = 0; i < WM; ++i) {                                               \
+          if (TWO_ACC && (kk & 1))                                                                     \
+            accb[j][i] = __builtin_amdgcn_mfma_f32_32x32x2f32(BV[kk][j], AV[kk][i], accb[j][i], 0, 0, 0); \
+          else                                                                                         \
+            acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x2f32(BV[kk][j], AV[kk][i], acc[j][i], 0, 0, 0); \
+        }                                                                                              \
+  } while (0)
+  if (PF && fast && kbeg + (PF + 1) * GEMM_BK <= kend) {
+    // fa/fb[c]: fragments of the slab at k0; LDS[buf ^ 1]: the slab after it; ga/gb: the PF - 1 slabs after
+    // that, on their way from global memory (a workgroup alone on its CU has nobody to hide that
+    // latency behind: the requests run PF + 1 slabs ahead of the MFMAs).  Every fetch asks for a full
+    // slab inside [kbeg, kend).
+    float fa[2][GEMM_BK / 2][WM], fb[2][GEMM_BK / 2][WN];
+    // a wavefront alone on its SIMD issues its MFMAs one after the other: two chains of accumulators, so
+    // that an MFMA does not wait for the one before it
+    constexpr bool TWO_ACC = WM * WN == 1;
+    f32x16 accb[TWO_ACC ? WN : 1][TWO_ACC ? WM : 1];
+    if (TWO_ACC) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) accb[0][0][v] = 0.f;
+    }
+    constexpr int NS = PF > 0 ? PF : 1;   // (PF == 0 never runs this branch)
+    f32x4 ga[NS][A4], gb[NS][B4];
+    GEMM_FETCH_FAST(ga[0], gb[0]);
+    GEMM_STASH(0, ga[0], gb[0]);
+    GEMM_FETCH_FAST(ga[0], gb[0]);
+    __syncthreads();
+    GEMM_FRAGS(0, fa[0], fb[0]);
+    GEMM_STASH(1, ga[0], gb[0]);
+#pragma unroll
+    for (int q = 0; q < PF - 1; ++q) GEMM_FETCH_FAST(ga[q], gb[q]);
+    __syncthreads();
+    while (k0 + (2 * PF + 1) * GEMM_BK <= kend) {
+#pragma unroll
+      for (int q = 0; q < PF; ++q) {
+        // LDS traffic first, then the MFMAs (the fences keep the compiler from sinking the reads to
+        // their uses one phase later, behind a wait): the chain of MFMAs runs while LDS answers
+        GEMM_FETCH_FAST(ga[(q + NS - 1) % NS], gb[(q + NS - 1) % NS]);
+        GEMM_FRAGS(buf ^ 1, fa[(q + 1) % 2], fb[(q + 1) % 2]);
+        GEMM_STASH(buf, ga[q], gb[q]);
+        GEMM_MFMAS(fa[q % 2], fb[q % 2]);
+        {
+          // The order of issue: the global loads, then one LDS read (and, in the second half, one LDS
+          // write) in the shadow of every MFMA; left to itself the compiler sinks the reads to their uses
+          // one phase later, behind a wait.  (4096 x 4096 x 4096: 1068 -> 933 us, 2048^3: 153 -> 133 us,
+          // 1024^3 on one workgroup per CU: 26.6 -> 24 us; four register sets instead of two gain nothing.)
+          __builtin_amdgcn_sched_group_barrier(0x020, A4 + B4, 0);
+#pragma unroll
+          for (int g = 0; g < GEMM_BK / 2 * WM * WN; ++g) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            if (g >= GEMM_BK / 4 * WM * WN) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        buf ^= 1; k0 += GEMM_BK;
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < PF - 1; ++q) {
+      GEMM_FRAGS(buf ^ 1, fa[(q + 1) % 2], fb[(q + 1) % 2]);
+      GEMM_STASH(buf, ga[q], gb[q]);
+      __builtin_amdgcn_sched_barrier(0);
+      GEMM_MFMAS(fa[q % 2], fb[q % 2]);
+      __builtin_amdgcn_sched_barrier(0);
+      __syncthreads();
+      __builtin_amdgcn_sched_barrier(0);
+      buf ^= 1; k0 += GEMM_BK;
+    }
+    GEMM_MFMAS(fa[(PF - 1) % 2], fb[(PF - 1) % 2]);
+    if (TWO_ACC) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[0][0][v] += accb[0][0][v];
+    }
+    buf ^= 1; k0 += GEMM_BK;         // LDS[buf] holds the full slab at k0, nothing is in flight
+  } else if (fast && kbeg + 2 * GEMM_BK <= kend) {
     // Global loads run two slabs ahead of the MFMAs: while slab i is multiplied, slab
     // i+1 (asked for one iteration ago) is written to LDS and slab i+2 is requested.
     GEMM_FETCH_FAST(ra, rb);
@@ -358,6 +450,8 @@ k_gemm(const float* __restrict__ A, int lda, const float* __restrict__ B, int ld
 
 #undef GEMM_FETCH_FAST
 #undef GEMM_STASH
+#undef GEMM_FRAGS
+#undef GEMM_MFMAS
 
 // Products too small to fill the chip with 64 x 64 tiles (the RBM / MLP layer shapes):
 // a workgroup owns one 32 x 32 block of C; its NW wavefronts each take every NW-th
