@@ -306,14 +306,16 @@ k_gemm(const float* __restrict__ A, int lda, const float* __restrict__ B, int ld
     }
     constexpr int NS = PF > 0 ? PF : 1;   // (PF == 0 never runs this branch)
     f32x4 ga[NS][A4], gb[NS][B4];
-    GEMM_FETCH_FAST(ga[0], gb[0]);
-    GEMM_STASH(0, ga[0], gb[0]);
-    GEMM_FETCH_FAST(ga[0], gb[0]);
-    __syncthreads();
-    GEMM_FRAGS(0, fa[0], fb[0]);
-    GEMM_STASH(1, ga[0], gb[0]);
+    // (the first slabs are all asked for before the first wait: one trip to memory in front of the
+    // first MFMA instead of three)
+    GEMM_FETCH_FAST(ra, rb);
+    GEMM_FETCH_FAST(ga[NS - 1], gb[NS - 1]);
 #pragma unroll
     for (int q = 0; q < PF - 1; ++q) GEMM_FETCH_FAST(ga[q], gb[q]);
+    GEMM_STASH(0, ra, rb);
+    __syncthreads();
+    GEMM_FRAGS(0, fa[0], fb[0]);
+    GEMM_STASH(1, ga[NS - 1], gb[NS - 1]);
     __syncthreads();
     while (k0 + (2 * PF + 1) * GEMM_BK <= kend) {
 #pragma unroll
