@@ -122,6 +122,38 @@ def test_large_square_products(cm, rng, n):
         h.free_device_memory()
 
 
+@pytest.mark.parametrize("m,k,n", [(1000, 1001, 1000), (1001, 1000, 1000), (1000, 1000, 1001), (1003, 999, 1005), (1088, 50, 1088),
+                                   (1100, 48, 1000), (1100, 47, 1000), (2000, 130, 1300), (1004, 1030, 996)])
+@pytest.mark.parametrize("ta,tb", [(False, False), (True, False), (False, True)])
+def test_products_on_the_tile_loop_with_any_alignment(cm, rng, m, k, n, ta, tb):
+    """More 64 x 64 tiles than the single-launch kernels take: the loop over 16-deep slabs whose
+    loads are unconditional 16-byte requests.  Leading dimensions that are not multiples of four
+    floats, operands that start at an odd float of a parent buffer, tiles that hang over the edge,
+    reductions of exactly three slabs (the shortest that enter the loop) and of one float less."""
+    A = np.asarray(rng.uniform(-1, 1, (k, m) if ta else (m, k)), dtype=np.float32, order='F')
+    B = np.asarray(rng.uniform(-1, 1, (n, k) if tb else (k, n)), dtype=np.float32, order='F')
+    C = np.asarray(rng.uniform(-1, 1, (m, n)), dtype=np.float32, order='F')
+    opa = (A.T if ta else A).astype(np.float64); opb = (B.T if tb else B).astype(np.float64)
+    want = 0.5 * C.astype(np.float64) + 1.25 * (opa @ opb)
+    bound = 0.5 * np.abs(C).astype(np.float64) + 1.25 * (np.abs(opa) @ np.abs(opb))
+    # whole matrices, then the same operands as views one column into a parent with one more column
+    # (the view starts rows-of-the-parent floats into the buffer: any 4-byte alignment)
+    pa = np.asfortranarray(np.concatenate([np.zeros((A.shape[0], 1), np.float32), A], axis=1))
+    pb = np.asfortranarray(np.concatenate([np.zeros((B.shape[0], 1), np.float32), B], axis=1))
+    for view in (False, True):
+        if view:
+            ha, hb = cm.CUDAMatrix(pa), cm.CUDAMatrix(pb)
+            a, b = ha.slice(1, pa.shape[1]), hb.slice(1, pb.shape[1])
+        else:
+            ha, hb = cm.CUDAMatrix(A), cm.CUDAMatrix(B)
+            a, b = ha, hb
+        c = cm.CUDAMatrix(C)
+        cm._check(cm._cudamat.dot((a.T if ta else a).p_mat, (b.T if tb else b).p_mat, c.p_mat, 0.5, 1.25))
+        assert np.max(np.abs(c.asarray() - want) / bound) < REL, view
+        for h in (ha, hb, c):
+            h.free_device_memory()
+
+
 @pytest.mark.parametrize("ta,tb", [(False, False), (True, False), (False, True), (True, True)])
 def test_split_k_products(cm, rng, ta, tb):
     """About one 64 x 64 tile per CU and K >= 2048: the reduction is split over two workgroups
