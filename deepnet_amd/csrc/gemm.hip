@@ -907,6 +907,31 @@ __global__ void k_gemm_splitk_finish(const float* partial, int splits, float* C,
   }
 }
 
+// The same, four rows at a time (M and ldc multiples of 4, C on a 16-byte boundary): the sums and the
+// expression per element are those of the kernel above.
+__global__ void __launch_bounds__(256)
+k_gemm_splitk_finish4(const float* partial, int splits, float* C, int ldc, int M, int N, float alpha, float beta) {
+  const size_t total4 = (size_t)M * N / 4;
+  const size_t e4 = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (e4 >= total4) return;
+  const f32x4* p4 = reinterpret_cast<const f32x4*>(partial) + e4;
+  f32x4 s = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+  for (int z = 0; z < splits; ++z) s += p4[(size_t)z * total4];
+  const size_t e = e4 * 4, m = e % M, n = e / M;
+  f32x4* c = reinterpret_cast<f32x4*>(C + n * ldc + m);
+  f32x4 o;
+  if (beta == 0.f) {
+#pragma unroll
+    for (int v = 0; v < 4; ++v) o[v] = 0.f + alpha * s[v];
+  } else {
+    const f32x4 old = *c;
+#pragma unroll
+    for (int v = 0; v < 4; ++v) o[v] = beta * old[v] + alpha * s[v];
+  }
+  *c = o;
+}
+
 // C = beta*C where the product is empty (K == 0).
 __global__ void k_scale(float* C, int ldc, int M, int N, float beta) {
   const size_t total = (size_t)M * N;
@@ -1086,7 +1111,10 @@ static int gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, co
   if (splits > 1) {
     size_t total = (size_t)M * N;
     unsigned blocks = (unsigned)((total + 255) / 256 < (size_t)cus * 8 ? (total + 255) / 256 : (size_t)cus * 8);
-    hipLaunchKernelGGL(k_gemm_splitk_finish, dim3(blocks), dim3(256), 0, dn_stream(), partial, splits, C, ldc, M, N, alpha, beta);
+    if (M % 4 == 0 && ldc % 4 == 0 && dn_aligned16(C))
+      hipLaunchKernelGGL(k_gemm_splitk_finish4, dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0, dn_stream(), partial, splits, C, ldc, M, N, alpha, beta);
+    else
+      hipLaunchKernelGGL(k_gemm_splitk_finish, dim3(blocks), dim3(256), 0, dn_stream(), partial, splits, C, ldc, M, N, alpha, beta);
   }
   return dn_launch_status();
 }
