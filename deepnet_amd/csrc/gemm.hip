@@ -1073,10 +1073,14 @@ static int gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, co
   const long long tiles_big = (long long)((M + 127) / 128) * ((N + 127) / 128);
   // 128 x 128 tiles (two workgroups per CU) against 64 x 64 tiles (five), as measured:
   // short reductions are mostly prologue and epilogue, which more resident workgroups hide
-  // (4096 x 4096 x 128, beta = 1: 71 us against 60 us; up to K = 512 when C is also read); and
+  // (4096 x 4096 x 128, beta = 1: 71 us against 60 us; up to K = 512 when C is also read, K = 256 otherwise); and
   // a tile count that leaves the last round of a CU half empty costs more than the smaller
   // tile's lower matrix-core rate of about 0.92 (3072 x 3072 x 2048: 404 us against 336 us).
-  const int kmax64 = beta != 0.f ? 512 : 128;
+  // (with the present main loop: 4096 x 4096 x 256 84 us on 64 x 64 tiles against 88 us, x 512 even, x 1024 268 us
+  // against 254 us; fewer than two big tiles per CU leave the CU to one or two workgroups, and the small
+  // tiles win up to K = 1024: 2048 x 2048 x 256 24.2 us against 30.3 us, x 512 39.6 against 46.7, x 1024 71.4
+  // against 75.5)
+  const int kmax64 = tiles_big < 2ll * cus ? 1024 : beta != 0.f ? 512 : 256;
   auto fill = [&](long long t) { return (double)t / (double)(((t + cus - 1) / cus) * cus); };
   const bool big = tiles_big >= cus && K > kmax64 && fill(tiles_big) >= 0.92 * fill(tiles64);
   const int BM = big ? 128 : 64, BN = big ? 128 : 64;
