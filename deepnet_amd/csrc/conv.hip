@@ -35,6 +35,7 @@
 //                      wavefront holds the whole output block
 #include "common.h"
 #include <type_traits>
+
 #include "../../include/cudamat_conv_amd.h"
 #include <math.h>
 #include <stdio.h>
@@ -1297,6 +1298,176 @@ __global__ void __launch_bounds__(256) k_conv_down_gather(ConvArgs p, const floa
   }
 }
 
+// ------------------------------------------------------------------ convDown, stride 1, at most 4 colours
+// One launch, every pixel written once, no intermediate (the counterpart of the reference's
+// img_acts_color, cudamat_conv_kernels.cuh:419-554, dispatched at cudamat_conv.cu:375-405).
+// The implicit GEMM of this pass has only Cg <= 4 output columns, which 32- and 16-wide
+// matrix-core blocks waste; v_mfma_f32_4x4x1_16b_f32 runs at the same rate on 16
+// independent 4 x 4 blocks of rank 1:
+//   block rows    4 neighbouring images            (first operand: one hidden activation per lane,
+//                                                   read from memory as it lies, 128-byte runs)
+//   block columns the colours of the group (+ pad) (second operand: w[c, ky, kx, f] per lane)
+//   blocks 0-7    images 0..31 with filter 2i, blocks 8-15 the same images with filter 2i + 1
+// A wavefront owns a 4 x 4 tile of pixels for 32 images (16 accumulators of 4 registers, lane
+// (block b, colour c), register v = image 4b + v) and one of NWV parts of the group's filters;
+// per pair of filters it loads the (K + 3)^2 modules its pixels reach once (a module outside
+// the grid is an out-of-range buffer offset and reads as zero) and issues 16 * K * K MFMAs,
+// acc[pixel] += hid[module = pixel - tap] (x) w[tap], with the loads of the next pair and the
+// LDS reads of its weights issued between them.  The wavefronts of a workgroup (the parts of
+// the filters) and the two filter parities meet in LDS in a fixed order.
+// Measured on the part: with 16 independent accumulators this MFMA form runs at the rate of the
+// 32 x 32 x 2 form (149 against 155 TFLOP/s), but it occupies the pipe for 8 cycles only, and
+// every other instruction of the same wavefront between two of them (LDS read, buffer load)
+// costs about one such slot, where a 64-cycle MFMA hides a dozen; two wavefronts per SIMD halve
+// that cost but need the operand sets in 256 registers, which spills.
+template <int K, int FSC, int NWV>
+__global__ void __launch_bounds__(64 * NWV, 1) k_conv_down_px(ConvArgs p) {
+  constexpr int T = 4, HR = K + T - 1, KK = K * K, NA = HR * HR, NT = 64 * NWV;
+  constexpr int CS = KK * FSC + 8;          // floats between the colours' weight blocks: their banks differ by 8
+  constexpr int WSZ = 5 * CS;               // four colours and a block of zeros (lanes of the pad colours)
+  constexpr int RED = NWV * 64 * 64;        // the final sum reuses the weights' memory
+  constexpr unsigned FAR_V = 0x40000000u, FAR_S = 0x20000000u;   // either one is beyond the buffer, and so is their sum
+  __shared__ float lds[WSZ > RED ? WSZ : RED];
+  const int tid = threadIdx.x, lane = tid & 63, par = lane >> 5, li = lane & 31, c = lane & 3;
+  const int wq = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int g = blockIdx.z;
+  // workgroup -> (image block, pixel tile); consecutive workgroups go round the 8 XCDs, so every XCD
+  // is handed a contiguous run of tiles (neighbouring tiles share the modules between them in its L2)
+  const int tiles_x = (p.H + T - 1) / T, tiles = tiles_x * tiles_x;
+  const int total = (int)gridDim.x;
+  int wid = (int)blockIdx.x;
+  if ((total & 7) == 0) wid = (wid & 7) * (total >> 3) + (wid >> 3);
+  const int nb = wid / tiles, tile = wid - nb * tiles;
+  const int ty = tile / tiles_x, tx = tile - ty * tiles_x;
+  const int y0 = ty * T, x0 = tx * T;
+  const int my0 = y0 - p.pad0 - (K - 1), mx0 = x0 - p.pad0 - (K - 1);   // first module row / column of the halo
+  const int Fq = p.Fg / NWV, nit = Fq >> 1;
+  const int f0 = g * p.Fg + wq * Fq;                                     // first filter of this wavefront
+
+  __amdgpu_buffer_rsrc_t r_hid = __builtin_amdgcn_make_buffer_rsrc((void*)p.hid, 0, (int)p.a_bytes, 0x00020000);
+  __amdgpu_buffer_rsrc_t r_flt = __builtin_amdgcn_make_buffer_rsrc((void*)p.flt, 0, (int)p.b_bytes, 0x00020000);
+
+  const unsigned plane = (unsigned)p.M * (unsigned)p.N * 4u;            // bytes between filters
+  unsigned voff[HR], soff[HR], sstep[HR];
+#pragma unroll
+  for (int j = 0; j < HR; ++j) {
+    const int mx = mx0 + j;
+    voff[j] = mx >= 0 && mx < p.Mx ? (unsigned)li * 4u + (unsigned)par * plane + (unsigned)(mx * p.N) * 4u : FAR_V;
+  }
+#pragma unroll
+  for (int r = 0; r < HR; ++r) {
+    const int my = my0 + r;
+    const bool ok = my >= 0 && my < p.Mx;
+    soff[r] = ok ? (unsigned)f0 * plane + ((unsigned)(my * p.Mx) * (unsigned)p.N + (unsigned)(nb * 32)) * 4u : FAR_S;
+    sstep[r] = ok ? 2u * plane : 0u;
+  }
+  float a0[NA], a1[NA];
+  auto request = [&](float (&an)[NA], int idx) __attribute__((always_inline)) {
+    an[idx] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r_hid, (int)voff[idx % HR], (int)soff[idx / HR], 0));
+  };
+#pragma unroll
+  for (int i = 0; i < NA; ++i) request(a0, i);
+
+  // weights of the group: w(f, q = c*KK + tap) at f + F*q, read along f, kept as [c][tap][f]
+  {
+    constexpr int PER = (4 * KK * FSC + NT - 1) / NT;
+    float w[PER];
+#pragma unroll
+    for (int it = 0; it < PER; ++it) {
+      const int e = tid + it * NT, f = e & (FSC - 1), q = e / FSC;
+      const unsigned off = q < p.Cg * KK && f < p.Fg ? ((unsigned)(g * p.Fg + f) + (unsigned)p.F * (unsigned)q) * 4u : FAR_V;
+      w[it] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r_flt, (int)off, 0, 0));
+    }
+#pragma unroll
+    for (int it = 0; it < PER; ++it) {
+      const int e = tid + it * NT, f = e & (FSC - 1), q = e / FSC;
+      if (e < 4 * KK * FSC) lds[(q / KK) * CS + (q % KK) * FSC + f] = w[it];
+    }
+    for (int e = tid; e < KK * FSC; e += NT) lds[4 * CS + e] = 0.f;
+  }
+  __syncthreads();
+  const float* wl = lds + (c < p.Cg ? c : 4) * CS + wq * Fq + par;   // + 2 per pair of filters, + FSC per tap
+
+  f32x4 acc[T * T];
+#pragma unroll
+  for (int i = 0; i < T * T; ++i) acc[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+  // One pair of filters: multiply a and the pair's weights (at wc) into the accumulators.  Between
+  // the MFMAs: one request in GAP for the next pair's modules (into an; beyond the last pair the
+  // offsets are out of range and nothing is fetched), and the weights two taps ahead (at the end
+  // of the step those of the next pair, at wn), kept in a ring of three registers.
+  // Taps run in descending order, so module rows are first used in ascending order.
+  // One pair of filters: multiply (a, b) into the accumulators.  Between the MFMAs: one request
+  // in GAP for the next pair's modules (into an; beyond the last pair the offsets are out of range
+  // and nothing is fetched) and one LDS read per tap for the next pair's weights (into bn).
+  // Taps run in descending order, so module rows are first used in ascending order.
+  float b0[KK], b1[KK];
+#pragma unroll
+  for (int t = 0; t < KK; ++t) b0[t] = wl[t * FSC];
+  auto step = [&](const float (&a)[NA], const float (&b)[KK], float (&an)[NA], float (&bn)[KK], const float* wn)
+      __attribute__((always_inline)) {
+    constexpr int NM = T * T * KK, GAP = NM / NA;
+#pragma unroll
+    for (int gi = 0; gi < KK; ++gi) {
+      const int ky = K - 1 - gi / K, kx = K - 1 - gi % K;
+#pragma unroll
+      for (int yy = 0; yy < T; ++yy)
+#pragma unroll
+        for (int xx = 0; xx < T; ++xx) {
+          const int m = (gi * T + yy) * T + xx;
+          if (m % GAP == 0 && m / GAP < NA) {
+            __builtin_amdgcn_sched_barrier(0);
+            request(an, m / GAP);
+            __builtin_amdgcn_sched_barrier(0);
+          }
+          if (m % (T * T) == T * T / 2) {
+            __builtin_amdgcn_sched_barrier(0);
+            bn[gi] = wn[gi * FSC];
+            __builtin_amdgcn_sched_barrier(0);
+          }
+          acc[yy * T + xx] = __builtin_amdgcn_mfma_f32_4x4x1f32(a[(yy + K - 1 - ky) * HR + xx + K - 1 - kx], b[ky * K + kx],
+                                                                acc[yy * T + xx], 0, 0, 0);
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  int it = 0;
+#define DOWN_PX_STEP(A, B, AN, BN)                                                      \
+  _Pragma("unroll") for (int r = 0; r < HR; ++r) soff[r] = it + 1 < nit ? soff[r] + sstep[r] : FAR_S; \
+  step(A, B, AN, BN, wl + 2 * (it + 1 < nit ? it + 1 : it));                            \
+  if (++it >= nit) break;
+  while (true) {
+    DOWN_PX_STEP(a0, b0, a1, b1)
+    DOWN_PX_STEP(a1, b1, a0, b0)
+  }
+#undef DOWN_PX_STEP
+
+  // the parts of the filters and the two parities meet in LDS: red[wavefront][register][lane]
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < T * T; ++i)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const float val = acc[i][v];   // (through a scalar: a cast applied to the vector element itself reads element 0)
+      lds[(wq * 64 + i * 4 + v) * 64 + lane] = val;
+    }
+  __syncthreads();
+  const int outs = T * T * p.Cg * 32;
+  for (int o = tid; o < outs; o += NT) {
+    const int img = o & 31, rest = o >> 5;
+    const int pix = rest / p.Cg, cc = rest - pix * p.Cg;
+    const int reg = pix * 4 + (img & 3), ln = 4 * (img >> 2) + cc;
+    float s = 0.f;
+#pragma unroll
+    for (int w = 0; w < NWV; ++w) s += lds[(w * 64 + reg) * 64 + ln] + lds[(w * 64 + reg) * 64 + 32 + ln];
+    const int y = y0 + pix / T, x = x0 + pix % T;
+    if (y < p.H && x < p.H) {
+      float* t = p.out + ((size_t)(g * p.Cg + cc) * p.HH + (size_t)(y * p.H + x)) * p.N + nb * 32 + img;
+      *t = (p.scale_t == 0.f ? 0.f : p.scale_t * *t) + p.scale_o * s;
+    }
+  }
+}
+
 // ------------------------------------------------------------------ host side
 
 static char g_conv_err[256];
@@ -1788,6 +1959,16 @@ static void conv_down_impl(cudamat* hidActs, cudamat* filters, cudamat* targets,
       else if (cols <= 96) hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 4, 1, 3, true>), dim3(gx, 1, numGroups), dim3(256), 0, dn_stream(), a);
       else hipLaunchKernelGGL((k_conv_mfma<CONV_DOWNM, 2, 2, 2, true>), dim3(gx, (cols + 127) / 128, numGroups), dim3(256), 0, dn_stream(), a);
     }
+  } else if (!local && moduleStride == 1 && a.Cg <= 4 && (k == 3 || k == 5) && N % 32 == 0 && a.Fg % 8 == 0 &&
+             a.Fg <= 128 && a.a_bytes != 0 && a.a_bytes <= 0x20000000u && a.b_bytes != 0 && a.b_bytes <= 0x20000000u &&
+             (long long)N * a.HH * numImgColors * 4 < (1ll << 31)) {
+    // at most four colours, stride 1: pixels accumulate in registers on 4 x 4 x 1 matrix-core blocks
+    const int tiles_x = (imgSize + 3) / 4;
+    const dim3 grid((unsigned)(tiles_x * tiles_x * (N / 32)), 1, numGroups);
+#define DOWN_PX(KF, FS) hipLaunchKernelGGL((k_conv_down_px<KF, FS, 4>), grid, dim3(256), 0, dn_stream(), a)
+    if (a.Fg <= 64) { if (k == 3) DOWN_PX(3, 64); else DOWN_PX(5, 64); }
+    else { if (k == 3) DOWN_PX(3, 128); else DOWN_PX(5, 128); }
+#undef DOWN_PX
   } else if (!local && fast_ok(a) && dn_aligned16(a.out) && a.Cg <= 16) {
     // few colours: patch-matrix form
     const long long prow = (long long)a.M * N;

@@ -59,6 +59,12 @@ CASES = [  # N, C, H, F, k, stride, padding, groups
     (128, 20, 8, 50, 5, 1, 0, 1),    # 20 colours -> 50 filters (padded to 64)
     (100, 3, 8, 10, 3, 1, 1, 1),     # batch 100 and 10 filters: both paddings at once
     (64, 4, 9, 24, 3, 2, 1, 1),      # 24 filters, strided
+    # convDown of stride-1 layers with at most 4 colours (4 x 4 x 1 matrix-core blocks, pixels in registers):
+    (32, 4, 7, 8, 3, 1, 2, 1),       # 4 colours, 8 filters (one pair per wavefront), map not a multiple of the 4 x 4 tile
+    (96, 3, 13, 24, 5, 1, 4, 1),     # padding k - 1: the module grid is larger than the image
+    (64, 8, 6, 144, 3, 1, 0, 2),     # 2 groups of 4 colours / 72 filters, no padding
+    (32, 2, 9, 128, 5, 1, 1, 1),     # 128 filters in one group
+    (160, 1, 5, 40, 5, 1, 3, 1),     # one colour, 5 image blocks, a single tile row
 ]
 
 
