@@ -9,6 +9,9 @@
 // One CU count for launch sizing; MI355X has 256 CUs in 8 XCDs.  Queried once.
 int dn_num_cus();
 
+// hipMalloc that releases the library's cache of freed matrix blocks and retries when the device is full.
+hipError_t dn_malloc(void** p, size_t bytes);
+
 // Grow-only device workspaces (slot 0: partials and scalar results; slot 1: conv patch matrix).
 void* dn_scratch(size_t bytes, int slot = 0);
 

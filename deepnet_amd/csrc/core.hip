@@ -44,6 +44,22 @@ static size_t g_scratch_bytes[4] = {0, 0, 0, 0};
 static bool g_scratch_recorded[4] = {false, false, false, false};
 static std::vector<void*>& g_retired = *new std::vector<void*>;   // outgrown blocks that a recorded graph may still use
 
+static void block_flush();
+
+// hipMalloc for the library's own workspaces: when the device is out of memory, the blocks that
+// free_device_memory keeps for reuse are given back first and the request is made again.
+hipError_t dn_malloc(void** p, size_t bytes) {
+  hipError_t e = hipMalloc(p, bytes);
+  if (e != hipSuccess) {
+    hipGetLastError();
+    hipDeviceSynchronize();
+    block_flush();
+    e = hipMalloc(p, bytes);
+    if (e != hipSuccess) { hipGetLastError(); *p = nullptr; }
+  }
+  return e;
+}
+
 void* dn_scratch(size_t bytes, int slot) {
   if (bytes > g_scratch_bytes[slot]) {
     if (g_capturing) return nullptr;   // growing means freeing and allocating: not while a graph is recorded
@@ -58,10 +74,9 @@ void* dn_scratch(size_t bytes, int slot) {
       g_scratch_recorded[slot] = false;
     }
     size_t want = bytes < (1u << 20) ? (1u << 20) : bytes;
-    if (hipMalloc(&g_scratch[slot], want) != hipSuccess) {
+    if (dn_malloc(&g_scratch[slot], want) != hipSuccess) {
       g_scratch[slot] = nullptr;
       g_scratch_bytes[slot] = 0;
-      hipGetLastError();
       return nullptr;
     }
     g_scratch_bytes[slot] = want;
@@ -98,11 +113,8 @@ static void* block_get(size_t bytes) {
     p = it->second.back();
     it->second.pop_back();
     g_cached_bytes -= bytes;
-  } else if (hipMalloc(&p, bytes) != hipSuccess) {
-    hipGetLastError();
-    hipDeviceSynchronize();
-    block_flush();
-    if (hipMalloc(&p, bytes) != hipSuccess) { hipGetLastError(); return nullptr; }
+  } else if (dn_malloc(&p, bytes) != hipSuccess) {
+    return nullptr;
   }
   g_block_bytes[p] = bytes;
   return p;
@@ -138,7 +150,7 @@ unsigned* dn_zero_words(int n) {
       g_zero_words_n = 0;
     }
     const int want = n < 16384 ? 16384 : n;
-    if (hipMalloc(&g_zero_words, (size_t)want * sizeof(unsigned)) != hipSuccess) { g_zero_words = nullptr; hipGetLastError(); return nullptr; }
+    if (dn_malloc((void**)&g_zero_words, (size_t)want * sizeof(unsigned)) != hipSuccess) { g_zero_words = nullptr; return nullptr; }
     if (hipMemset(g_zero_words, 0, (size_t)want * sizeof(unsigned)) != hipSuccess) return nullptr;
     g_zero_words_n = want;
   }
@@ -291,7 +303,7 @@ static bool stage_out(const float* src, float* host, int n) {
   if (!g_stage_host) {
     void* h = nullptr;
     void* d = nullptr;
-    if (hipHostMalloc(&h, sizeof(DnStage), hipHostMallocDefault) != hipSuccess) { hipGetLastError(); return false; }
+    if (hipHostMalloc(&h, sizeof(DnStage), hipHostMallocCoherent | hipHostMallocMapped) != hipSuccess) { hipGetLastError(); return false; }
     if (hipHostGetDevicePointer(&d, h, 0) != hipSuccess) { hipGetLastError(); hipHostFree(h); return false; }
     g_stage_host = (DnStage*)h;
     g_stage_dev = (DnStage*)d;
@@ -369,8 +381,7 @@ int graph_free(void* exec) {
   return e == hipSuccess ? 0 : CUDA_ERROR;
 }
 
-// A second library of this package (the conv library has its own copy of this file) joins a
-// recording by queueing on the same stream; NULL afterwards.
+// Queue on a stream of the caller's (capturing != 0: the caller is capturing it); NULL, 0 afterwards.
 int graph_set_stream(void* stream, int capturing) {
   g_stream = (hipStream_t)stream;
   g_capturing = capturing != 0;

@@ -826,6 +826,18 @@ static int rows_one_splits(int h, int w) {
   return splits;
 }
 
+__global__ void k_fill_u32(unsigned* p, int n, unsigned v);
+
+// The arrival counters are zero between launches because every launch returns them to zero.  A
+// launch that the runtime reports as failed may not have done so: clear them with a kernel (best
+// effort; on a device that has gone away this fails like everything after it).
+static void rezero_counters(unsigned* counters, int n) {
+  if (!counters || n <= 0 || dn_capturing()) return;
+  hipGetLastError();
+  hipLaunchKernelGGL(k_fill_u32, dim3((n + 255) / 256), dim3(256), 0, dn_stream(), counters, n, 0u);
+  hipGetLastError();
+}
+
 template <int OP>
 static int rows_reduce_one(const float* M, int ld, int h, int w, const float* x, float* y, float alpha, float beta,
                            const RowsWorkspace& ws) {
@@ -844,7 +856,9 @@ static int rows_reduce_one(const float* M, int ld, int h, int w, const float* x,
     hipLaunchKernelGGL((k_rows_one<OP, 16, 8, true>), grid, dim3(1024), 0, dn_stream(), M, ld, h, w, cps, x, y, ws.partial, ws.counters, alpha, beta);
   else
     hipLaunchKernelGGL((k_rows_one<OP, 16, 8, false>), grid, dim3(1024), 0, dn_stream(), M, ld, h, w, cps, x, y, ws.partial, ws.counters, alpha, beta);
-  return dn_launch_status();
+  const int status = dn_launch_status();
+  if (status && splits > 1) rezero_counters(ws.counters, bx);
+  return status;
 }
 
 static inline bool rows_one_ok(const float* M, int ld, int h) {
@@ -1075,7 +1089,7 @@ static bool result_word() {
   if (g_result_host) return true;
   void* h = nullptr;
   void* d = nullptr;
-  if (hipHostMalloc(&h, 64, hipHostMallocDefault) != hipSuccess) { hipGetLastError(); return false; }
+  if (hipHostMalloc(&h, 64, hipHostMallocCoherent | hipHostMallocMapped) != hipSuccess) { hipGetLastError(); return false; }
   if (hipHostGetDevicePointer(&d, h, 0) != hipSuccess) { hipGetLastError(); hipHostFree(h); return false; }
   g_result_host = (unsigned long long*)h;
   g_result_dev = (unsigned long long*)d;
@@ -1105,16 +1119,17 @@ static int flat_dot(const float* a, const float* b, long long n, int take_sqrt, 
   else DOT_SAME(false, false);
 #undef DOT_SAME
 #undef DOT_GO
-  if (hipGetLastError() != hipSuccess) return CUDA_ERROR;
+  const int n_counters = DOT_COUNTER_PITCH * (1 + (int)((nb + DOT_GROUP - 1) / DOT_GROUP));
+  if (hipGetLastError() != hipSuccess) { rezero_counters(counter, n_counters); return CUDA_ERROR; }
   unsigned long long word = 0;
   for (int i = 0; i < DOT_POLLS; ++i) {
     word = __atomic_load_n(g_result_host, __ATOMIC_ACQUIRE);
     if ((unsigned)(word >> 32) == tag) break;
   }
   if ((unsigned)(word >> 32) != tag) {
-    if (hipStreamSynchronize(dn_stream()) != hipSuccess) return CUDA_ERROR;
+    if (hipStreamSynchronize(dn_stream()) != hipSuccess) { rezero_counters(counter, n_counters); return CUDA_ERROR; }
     word = __atomic_load_n(g_result_host, __ATOMIC_ACQUIRE);
-    if ((unsigned)(word >> 32) != tag) return CUDA_ERROR;
+    if ((unsigned)(word >> 32) != tag) { rezero_counters(counter, n_counters); return CUDA_ERROR; }
   }
   const unsigned bits = (unsigned)word;
   memcpy(result, &bits, sizeof(float));
@@ -1264,15 +1279,19 @@ int sqsum_by_axis(cudamat* mat, cudamat* target, int axis, float mult, float p) 
 
 // target = beta * target + alpha * (sums of mat along axis), the kernels that dot() with a vector
 // of ones runs, without the vector: the same additions in the same order, so the same bits.
-// A transposed operand is summed along its other stored axis, as dot() would.
+// A transposed operand is summed along its other stored axis, as dot() would.  The target is
+// checked the way dot() checks it (cudamat.cu:1675-1679: leading and non-leading dimension,
+// the target's is_trans otherwise ignored), so a vector handed over as the transposed view
+// of its other orientation is accepted as it is there; it is the same memory.
 static int sums_impl(cudamat* mat, cudamat* target, int axis, float beta, float alpha) {
   if (!mat->on_device || !target->on_device) return ERROR_NOT_ON_DEVICE;
-  if (target->is_trans) return ERROR_TRANSPOSED;
   if (axis != 0 && axis != 1) return ERROR_UNSUPPORTED;
   const int h = mat->size[0], w = mat->size[1];
   const bool along_stored_columns = (axis == 0) != (mat->is_trans != 0);   // one result per stored column
   const int results = along_stored_columns ? w : h;
-  if (axis == 0 ? (target->size[0] != 1 || target->size[1] != results) : (target->size[0] != results || target->size[1] != 1))
+  const int t_lead = target->is_trans ? target->size[1] : target->size[0];
+  const int t_nonlead = target->is_trans ? target->size[0] : target->size[1];
+  if (axis == 0 ? (t_lead != 1 || t_nonlead != results) : (t_lead != results || t_nonlead != 1))
     return ERROR_INCOMPATIBLE_DIMENSIONS;
   if (results <= 0) return 0;
   if (along_stored_columns) {
@@ -1290,8 +1309,10 @@ int add_sum_by_axis(cudamat* mat, cudamat* target, int axis, float mult) { retur
 }  // extern "C"
 
 // t(i, j) = a(i, j) * (n_i < norm ? 1 : norm / n_i) with n_i = sqrt(sq[i]): the second pass of
-// normlimit_by_axis along the rows (cudamat_kernels.cu:1100-1130), given the rows' sums of
-// squares.  A flat pass over the matrix; VEC: 16-byte groups (h a multiple of 4, aligned
+// normlimit_by_axis along the rows, given the rows' sums of squares.  Axis 1 is an extension:
+// the reference returns ERROR_UNSUPPORTED for it (cudamat.cu:1300-1311); the rule is that of its
+// column kernel (kNormLimitColumnwise, cudamat_kernels.cu:1068-1098) applied to rows, and is
+// checked against the host restatement only.  A flat pass over the matrix; VEC: 16-byte groups (h a multiple of 4, aligned
 // operands), whose four rows are one 16-byte group of sq.
 template <bool VEC, bool STREAM>
 __global__ void __launch_bounds__(256)

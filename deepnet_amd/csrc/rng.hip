@@ -396,8 +396,8 @@ int init_random(rnd_struct* rnd_state, int seed, char* cudamatpath) {
     return ERROR_GENERIC;
   }
   void *dm = nullptr, *dw = nullptr;
-  if (hipMalloc(&dm, NUM_RND_STREAMS * sizeof(unsigned int)) != hipSuccess ||
-      hipMalloc(&dw, RNG_REGION_BYTES + 2 * RNG_BUF_BYTES) != hipSuccess ||
+  if (dn_malloc(&dm, NUM_RND_STREAMS * sizeof(unsigned int)) != hipSuccess ||
+      dn_malloc(&dw, RNG_REGION_BYTES + 2 * RNG_BUF_BYTES) != hipSuccess ||
       hipMemcpy(dm, host_mults, NUM_RND_STREAMS * sizeof(unsigned int), hipMemcpyHostToDevice) != hipSuccess) {
     free(host_mults);
     return CUDA_ERROR;

@@ -78,9 +78,9 @@ int allocate_device_memory_sparse(cudamat_sparse* mat) {
   mat->data_device.indptr = nullptr;
   // (an empty matrix still gets distinct, valid pointers)
   const size_t vals = (size_t)(nnz > 0 ? nnz : 1);
-  if (hipMalloc((void**)&mat->data_device.data, vals * sizeof(float)) != hipSuccess ||
-      hipMalloc((void**)&mat->data_device.indices, vals * sizeof(int)) != hipSuccess ||
-      hipMalloc((void**)&mat->data_device.indptr, ((size_t)rows + 1) * sizeof(int)) != hipSuccess) {
+  if (dn_malloc((void**)&mat->data_device.data, vals * sizeof(float)) != hipSuccess ||
+      dn_malloc((void**)&mat->data_device.indices, vals * sizeof(int)) != hipSuccess ||
+      dn_malloc((void**)&mat->data_device.indptr, ((size_t)rows + 1) * sizeof(int)) != hipSuccess) {
     hipGetLastError();
     release(mat);
     return CUBLAS_ERROR;

@@ -116,6 +116,7 @@ _SIGNATURES = {
     'correct_preds': (_i, [_M, _M, _M, _f]),
     'dot': (_i, [_M, _M, _M, _f, _f]),
     'dot_bias_act': (_i, [_M, _M, _M, _M, ct.c_int]),
+    'cd_update': (_i, [_M, _M, _M, _M, _M, _M, _M, _f]),
     'dot_bias_act_sample': (_i, [ct.c_void_p, _M, _M, _M, _M, _M, ct.c_int]),
     'momentum_update': (_i, [_M, _M, _M, _f, _f, _f, _f, ct.c_int]),
     'momentum_update_many': (_i, [ct.c_int, ct.c_void_p, ct.c_void_p, ct.c_void_p, ct.c_void_p, ct.c_void_p, ct.c_void_p,
@@ -834,25 +835,15 @@ class Graph(object):
 
     def __init__(self):
         self._exec = None
-        self._others = []
 
     def __enter__(self):
         stream = _cudamat.graph_capture_begin()
         if not stream:
             raise CUDAMatException("could not start recording a graph")
-        # the conv library, when it is loaded, queues on the same stream
-        import sys
-        conv = sys.modules.get(__package__ + '.cudamat_conv' if __package__ else 'cudamat_conv')
-        if conv is not None:
-            conv._ConvNet.graph_set_stream.argtypes = [ct.c_void_p, ct.c_int]
-            conv._ConvNet.graph_set_stream(stream, 1)
-            self._others.append(conv._ConvNet)
+        # (the conv library links against this one and queues on the same stream)
         return self
 
     def __exit__(self, exc_type, exc, tb):
-        for lib in self._others:
-            lib.graph_set_stream(None, 0)
-        self._others = []
         handle = _cudamat.graph_capture_end()
         if exc_type is not None:
             if handle:                              # a recording that was given up is not kept
@@ -901,6 +892,20 @@ def dot_bias_act(m1, m2, bias=None, target=None, act='sigmoid', sample=None):
         _check(_cudamat.dot_bias_act_sample(CUDAMatrix.rnd_state_p, m1.p_mat, m2.p_mat, b, target.p_mat, sample.p_mat,
                                             _ACTS[act]))
     return target
+
+
+def cd_update(W, bv, bh, v, h, v2, h2, eps):
+    """Extension of this backend (not in the reference): the contrastive-divergence update
+        W.add_dot(v, h.T, mult=eps); W.add_dot(v2, h2.T, mult=-eps)
+        bv.add_sums(v, axis=1, mult=eps); bv.add_sums(v2, axis=1, mult=-eps)
+        bh.add_sums(h, axis=1, mult=eps); bh.add_sums(h2, axis=1, mult=-eps)
+    (cudamat/examples/rbm_cudamat.py:57-85) as one product over the concatenated reduction
+    [v | v2] . [h | -h2]^T with a row of ones appended to each operand, one launch.  The sums are
+    formed in one accumulation instead of two rounded updates, so the result equals the six calls
+    to rounding (about 1e-7 relative), not bit for bit.  bv / bh may be None."""
+    _check(_cudamat.cd_update(W.p_mat, bv.p_mat if bv is not None else None, bh.p_mat if bh is not None else None,
+                              v.p_mat, h.p_mat, v2.p_mat, h2.p_mat, float(eps)))
+    return W
 
 
 def softmax_ce_grad(mat, labels, probs=None, loss=None, grad=None, tiny=1e-10):

@@ -276,6 +276,14 @@ int apply_softmax_grad(cudamat* mat, cudamat* labels, cudamat* target);
 int get_softmax_correct(cudamat* mat, cudamat* labels, cudamat* target);
 int get_softmax_cross_entropy(cudamat* mat, cudamat* labels, cudamat* target, float tiny);
 
+/* ---- Extension: the contrastive-divergence update of an RBM in one launch,
+ *   W += eps (v h^T - v2 h2^T),  bv += eps (rowsums v - rowsums v2),  bh += eps (rowsums h - rowsums h2),
+ * the six calls (two add_dot, four add_sums) of cudamat/examples/rbm_cudamat.py:57-85 and the statistics
+ * of deepnet/edge.py:236-242, layer.py:206-211, as one product over the concatenated reduction with a
+ * row of ones appended to each operand.  W nv x nh, v / v2 nv x batch, h / h2 nh x batch, bv nv x 1,
+ * bh nh x 1 (bv, bh may be NULL); nothing transposed.  Equal to the six calls to rounding. ---- */
+int cd_update(cudamat* W, cudamat* bv, cudamat* bh, cudamat* v, cudamat* h, cudamat* v2, cudamat* h2, float eps);
+
 /* ---- HIP graphs: no counterpart in the reference.  graph_capture_begin() makes the library
  * record every following call (with the pointers and scalars it is given) into a HIP graph
  * instead of running it, until graph_capture_end() returns the executable graph;
@@ -283,8 +291,9 @@ int get_softmax_cross_entropy(cudamat* mat, cudamat* labels, cudamat* target, fl
  * bound by the cost of launching (the RBM and MLP steps).  Calls that wait for the device
  * and workspaces that would have to grow fail with their error codes while recording; run
  * the sequence once before recording it.
- * graph_capture_begin returns the capturing stream (NULL on failure); graph_set_stream hands
- * that stream to a second library of this package (stream NULL, capturing 0 afterwards). ---- */
+ * graph_capture_begin returns the capturing stream (NULL on failure).  graph_set_stream makes
+ * the library queue on a stream of the caller's (capturing = 1: that stream is being captured by
+ * the caller; NULL, 0 returns to the NULL stream). ---- */
 void* graph_capture_begin(void);
 void* graph_capture_end(void);
 int graph_launch(void* graph_exec);

@@ -2,7 +2,10 @@
  * C ABI of the MI355X convolution / pooling / normalisation backend
  * (libcudamat_conv.so).  Names, argument order and argument meaning are those of
  * the 13 exports of the reference's cudamat/cudamat_conv.cu:1402-1456, which
- * cudamat/cudamat_conv.py binds through ctypes.
+ * cudamat/cudamat_conv.py binds through ctypes.  These 13 and conv_last_error are the
+ * library's whole dynamic symbol table.  It links against libcudamat.so (found next to it),
+ * whose stream, workspaces and block cache it shares: calls of both libraries run in call
+ * order on one stream and are recorded into the same HIP graphs.
  *
  * Layout (cudamat/cudamat_conv.cu:9-13): every operand is a column-major cudamat
  * whose size[0] is the number of images, so the flat index of pixel (c, y, x) of
@@ -26,12 +29,6 @@ extern "C" {
 
 /* No counterpart in the reference (it asserts): message of the last failed call, or NULL. */
 const char* conv_last_error(void);
-
-/* No counterpart in the reference: the stream this library queues its kernels on.  The matrix
- * library's graph_capture_begin() returns the stream it records into; handing it over here
- * (capturing = 1) makes the conv / pool / norm calls part of the same recording, and
- * (NULL, 0) returns this library to the NULL stream (include/cudamat_amd.h, "HIP graphs"). */
-int graph_set_stream(void* stream, int capturing);
 
 /* ---- shared-filter convolution: cudamat_conv.cu:1404-1412 (filterActs :15-257, imgActs :265-640,
  * weightActs :642-1015).  paddingStart is <= 0 (the Python wrapper negates it). ---- */

@@ -350,21 +350,61 @@ def test_sparse_dot_errors(cm, rng):
 
 @pytest.mark.gpu
 def test_fused_training_steps_of_the_bench_match_the_reference_sequences(cm):
-    # bench.py's RBM and MLP steps through the extensions leave the same bits in every
-    # parameter as the reference call sequences (same seeds, three steps each)
+    # bench.py's MLP step through the extensions leaves the same bits in every parameter as the
+    # reference call sequence (same seed, three steps).  The RBM step's layer states and samples
+    # have the same bits too; its parameters come from cd_update, which forms the statistics in one
+    # accumulation where the six reference calls round twice: equal to rounding, step after step.
     import bench
-    def run(cls, seed, fused, params):
+    def run(cls, seed, fused, params, steps):
         cm.CUDAMatrix.init_random(seed)
         model = cls(cm)
-        for _ in range(3):
+        for _ in range(steps):
             (model.step_fused if fused else model.step)()
         return [p.asarray().copy() for p in params(model)]
-    for cls, seed, params in ((bench.RBM, 1, lambda m: [m.W, m.bv, m.bh]),
-                              (bench.MLP, 3, lambda m: m.W + m.b + m.dW + [m.loss])):
-        plain, fused = run(cls, seed, False, params), run(cls, seed, True, params)
-        for a, b in zip(plain, fused):
-            assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+    mlp = lambda m: m.W + m.b + m.dW + [m.loss]
+    for a, b in zip(run(bench.MLP, 3, False, mlp, 3), run(bench.MLP, 3, True, mlp, 3)):
+        assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+    states = lambda m: [m.h, m.hs, m.v2, m.h2]
+    for a, b in zip(run(bench.RBM, 1, False, states, 1), run(bench.RBM, 1, True, states, 1)):
+        assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+    rbm = lambda m: [m.W, m.bv, m.bh]
+    for steps in (1, 3):
+        for a, b in zip(run(bench.RBM, 1, False, rbm, steps), run(bench.RBM, 1, True, rbm, steps)):
+            assert np.allclose(a, b, rtol=2e-6, atol=2e-8)
     cm.CUDAMatrix.init_random(1)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("nv,nh,B", [(784, 500, 100), (33, 65, 7), (64, 32, 1), (5, 3, 2), (100, 257, 33), (31, 31, 128)])
+def test_cd_update_equals_the_six_reference_calls(cm, rng, nv, nh, B):
+    f = lambda a: np.asarray(a, dtype=np.float32, order='F')
+    w, bv, bh = f(0.1 * rng.standard_normal((nv, nh))), f(rng.standard_normal((nv, 1))), f(rng.standard_normal((nh, 1)))
+    v, v2 = f(rng.random((nv, B)) < 0.3), f(rng.random((nv, B)))
+    h, h2 = f(rng.random((nh, B))), f(rng.random((nh, B)))
+    eps = 0.01 / B
+    V, H, V2, H2 = (cm.CUDAMatrix(a) for a in (v, h, v2, h2))
+    W1, BV1, BH1 = cm.CUDAMatrix(w), cm.CUDAMatrix(bv), cm.CUDAMatrix(bh)
+    W1.add_dot(V, H.T, mult=eps); W1.add_dot(V2, H2.T, mult=-eps)
+    BV1.add_sums(V, axis=1, mult=eps); BV1.add_sums(V2, axis=1, mult=-eps)
+    BH1.add_sums(H, axis=1, mult=eps); BH1.add_sums(H2, axis=1, mult=-eps)
+    W2, BV2, BH2 = cm.CUDAMatrix(w), cm.CUDAMatrix(bv), cm.CUDAMatrix(bh)
+    cm.cd_update(W2, BV2, BH2, V, H, V2, H2, eps)
+    d = np.float64
+    want_w = w.astype(d) + eps * (v.astype(d) @ h.astype(d).T - v2.astype(d) @ h2.astype(d).T)
+    want_bv = bv.astype(d) + eps * (v.astype(d).sum(1, keepdims=True) - v2.astype(d).sum(1, keepdims=True))
+    want_bh = bh.astype(d) + eps * (h.astype(d).sum(1, keepdims=True) - h2.astype(d).sum(1, keepdims=True))
+    for got, ref, want in ((W2, W1, want_w), (BV2, BV1, want_bv), (BH2, BH1, want_bh)):
+        assert np.allclose(got.asarray(), want, rtol=1e-6, atol=1e-7)          # against float64
+        assert np.allclose(got.asarray(), ref.asarray(), rtol=2e-6, atol=2e-7)  # against the six calls
+    # without the bias vectors; a second call continues from the first
+    W3 = cm.CUDAMatrix(w)
+    cm.cd_update(W3, None, None, V, H, V2, H2, eps)
+    assert np.array_equal(W3.asarray().view(np.uint32), W2.asarray().view(np.uint32))
+    cm.cd_update(W3, None, None, V, H, V2, H2, eps)
+    assert np.allclose(W3.asarray(), 2 * want_w - w.astype(d), rtol=1e-6, atol=2e-7)
+    # shape and flag errors
+    assert cm._cudamat.cd_update(W3.p_mat, None, None, V.p_mat, H.p_mat, V2.p_mat, V2.p_mat, 0.1) == (0 if nv == nh else -1)
+    assert cm._cudamat.cd_update(W3.p_mat, None, None, V.T.p_mat, H.p_mat, V2.p_mat, H2.p_mat, 0.1) == -5
 
 
 def _random_small_products(seed, count):

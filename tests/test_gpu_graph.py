@@ -166,3 +166,24 @@ def test_replays_survive_growth_of_the_library_workspaces(cm):
         g.launch()
         assert np.array_equal(r1.asarray(), want1) and np.array_equal(r0.asarray(), want0)
     g.free()
+
+
+def test_the_entry_point_that_allocates_nothing_is_recorded(cm):
+    """max_by_axis_noalloc is meant for callers under graph capture: recorded along axis 1 on a
+    matrix wide enough for column slices (partials and arrival counters of the fixed workspace in
+    use), replayed with eager work in between on inputs that change between the replays, every
+    replay compared bit for bit with the eager call on the same input."""
+    rng = np.random.default_rng(17)
+    x = cm.CUDAMatrix(np.asarray(rng.uniform(-1, 1, (2048, 4096)), dtype=np.float32, order='F'))
+    got, want = cm.empty((2048, 1)), cm.empty((2048, 1))
+    x.max_noalloc(1, got)                   # once eagerly: the workspace's address is looked up here
+    with cm.Graph() as g:
+        x.mult(-0.75)                       # the input changes from replay to replay
+        x.max_noalloc(1, got)
+    for _ in range(4):
+        g.launch()
+        x.max(1, want)
+        assert np.array_equal(_bits(got), _bits(want))
+        assert np.array_equal(got.asarray()[:, 0], x.asarray().max(axis=1))
+        _eager_between(cm, rng)
+    g.free()
