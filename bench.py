@@ -603,7 +603,15 @@ def main():
         t = time_loop(cm, rbm.step, 200, 20)
         secondary['rbm_cd1'] = {'steps_per_sec': round(1.0 / t, 1), 'us_per_step': round(t * 1e6, 1),
                                 'gemm_tflops': round(rbm.flops / t / 1e12, 3),
-                                'config': '784 visible x 500 hidden, batch 100, fp32'}
+                                'config': '784 visible x 500 hidden, batch 100, fp32',
+                                'note': 'the 16 calls of the reference API (cudamat/examples/rbm_cudamat.py:46-89); the library '
+                                        'folds add_col_vec / apply_sigmoid / sample_bernoulli into the launch of the dot() they '
+                                        'follow (deferred epilogues, same bits): 9 launches',
+                                'iters': 200, 'warmup': 20}
+        cm.set_deferred_epilogues(False)
+        t = time_loop(cm, rbm.step, 200, 20)
+        cm.set_deferred_epilogues(True)
+        secondary['rbm_cd1']['us_per_step_every_call_a_launch'] = round(t * 1e6, 1)
         t = time_loop(cm, rbm.step_fused, 200, 20)
         secondary['rbm_cd1_fused_extension'] = {
             'steps_per_sec': round(1.0 / t, 1), 'us_per_step': round(t * 1e6, 1),
@@ -624,7 +632,12 @@ def main():
         mlp = MLP(cm)
         t = time_loop(cm, mlp.step, 100, 10)
         secondary['mlp_784_1024_1024_10'] = {'steps_per_sec': round(1.0 / t, 1), 'us_per_step': round(t * 1e6, 1),
-                                              'gemm_tflops': round(mlp.flops / t / 1e12, 3), 'batch': 128}
+                                              'gemm_tflops': round(mlp.flops / t / 1e12, 3), 'batch': 128,
+                                              'iters': 100, 'warmup': 10}
+        cm.set_deferred_epilogues(False)
+        t = time_loop(cm, mlp.step, 100, 10)
+        cm.set_deferred_epilogues(True)
+        secondary['mlp_784_1024_1024_10']['us_per_step_every_call_a_launch'] = round(t * 1e6, 1)
         t = time_loop(cm, mlp.step_fused, 100, 10)
         secondary['mlp_fused_extensions'] = {
             'steps_per_sec': round(1.0 / t, 1), 'us_per_step': round(t * 1e6, 1),
@@ -665,21 +678,36 @@ def main():
         'config': {'workload': 'elementwise+reduction+RNG microbench, 4096x4096 fp32 column-major, 13 ops x %d '
                                'operand sets per step' % NSETS, 'step_bytes': STEP_BYTES},
         'roofline': roofline, 'ops': ops, 'secondary': secondary,
-        'timing': 'value: wall time of the K steps between two device synchronisations; ops: HIP events around the %d '
-                  'launches of an op in a step, median over the K steps' % NSETS,
+        'timing': {'value': 'wall time of the K = %d steps between two device synchronisations, after %d warm-up steps, one run'
+                            % (args.steps, args.warmup),
+                   'ops': 'HIP events on the NULL stream around the %d launches of an op in a step; median over the K steps' % NSETS,
+                   'steps_per_sec': 'wall time of `iters` steps after `warmup` steps, device synchronised on both sides, one run',
+                   'gemm_conv': 'HIP events around 10 (4096^3, conv: median of 3 such groups) or 200 (layer shapes) back-to-back '
+                                'launches after 30 ms of matrix-core warm-up',
+                   'note': 'shorter than 100 iterations x 5 repeats; figures move by 1-3 % between runs and up to 5 % (host-bound '
+                           'step loops: 20 %) between boxes'},
     }
     if not args.no_cpu:
         cb = cpu_baseline_c2()
         if not args.only_c2:
             r = cpu_baseline_rbm()
             cb['rbm_cd1_steps_per_sec'] = {'threads_%d' % k: round(v, 2) for k, v in r.items()}
+            # what the port's products reach: 5 products of 78.4 MFLOP per step (eigenmat itself calls Eigen's
+            # blocked product, eigenmat/eigenmat.cc:1059-1086, which this image does not have; the port's is a
+            # plain blocked loop), so the ratios below say how far the GPU step is from THIS code, no more
+            cb['rbm_cd1_gemm_gflops'] = {'threads_%d' % k: round(5 * 2 * 784 * 500 * 100 * v / 1e9, 1) for k, v in r.items()}
+            cb['rbm_cd1_gemm_note'] = ('step rate x 392 MFLOP of products per step; the port multiplies with a blocked triple '
+                                       'loop, eigenmat with Eigen (not in this image), so a tuned CPU GEMM would be several times faster')
             if 'rbm_cd1' in secondary:
                 secondary['rbm_cd1']['vs_cpu_1thread'] = round(secondary['rbm_cd1']['steps_per_sec'] / r[1], 1)
+                secondary['rbm_cd1']['vs_cpu_%dthreads' % max(r)] = round(secondary['rbm_cd1']['steps_per_sec'] / r[max(r)], 1)
             r = cpu_baseline_mlp()
             cb['mlp_784_1024_1024_10_steps_per_sec'] = {'threads_%d' % k: round(v, 2) for k, v in r.items()}
             if 'mlp_784_1024_1024_10' in secondary:
                 secondary['mlp_784_1024_1024_10']['vs_cpu_1thread'] = round(
                     secondary['mlp_784_1024_1024_10']['steps_per_sec'] / r[1], 1)
+                secondary['mlp_784_1024_1024_10']['vs_cpu_%dthreads' % max(r)] = round(
+                    secondary['mlp_784_1024_1024_10']['steps_per_sec'] / r[max(r)], 1)
             cb['conv_numpy_f64_ms'] = cpu_baseline_conv()
         line['cpu_baseline'] = cb
     print(json.dumps(line))

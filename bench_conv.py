@@ -30,11 +30,14 @@ def _time(ev, fn, iters, sync):
             fn()
         sync()
     e0, e1 = ev.new(), ev.new()
-    ev.record(e0)
-    for _ in range(iters):
-        fn()
-    ev.record(e1)
-    return ev.elapsed_ms(e0, e1) / iters
+    reps = []
+    for _ in range(3):      # median of three groups of `iters` back-to-back launches
+        ev.record(e0)
+        for _ in range(iters):
+            fn()
+        ev.record(e1)
+        reps.append(ev.elapsed_ms(e0, e1) / iters)
+    return sorted(reps)[1]
 
 
 def run(cm, ev, iters=10):

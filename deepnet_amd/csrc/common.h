@@ -24,8 +24,17 @@ void dn_set_no_graphs_hook(void (*f)());
 int dn_noalloc_setup();
 
 // The stream every kernel of the library is queued on: the NULL stream, or the stream a
-// caller is capturing into a HIP graph (graph_capture_begin .. graph_capture_end).
+// caller is capturing into a HIP graph (graph_capture_begin .. graph_capture_end).  Launches a
+// held-back product first (dn_flush), so that work is queued in call order.
 hipStream_t dn_stream();
+// Deferred epilogues: dot() may hold its launch back (dn_defer_dot) so that the add_col_vec /
+// activation / sample calls that follow it run in the product's epilogue; dn_flush() launches what
+// is held back.  Called by everything that queues work, hands out workspaces, moves data or waits.
+void dn_flush();
+void dn_set_pending(bool on);
+void dn_set_flush_hook(void (*f)());
+bool dn_defer_dot(cudamat* mat1, cudamat* mat2, cudamat* target, float beta, float alpha, int m, int n, int k);
+bool dn_pending_sample(rnd_struct* rnd, cudamat* mat, cudamat* target, int* err);
 bool dn_capturing();
 
 // Records the launch status of the kernel just queued; returns CUDA_ERROR or 0.

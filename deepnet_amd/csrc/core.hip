@@ -30,7 +30,24 @@ static int g_live_graphs = 0;
 static void (*g_no_graphs_hook)() = nullptr;
 void dn_set_no_graphs_hook(void (*f)()) { g_no_graphs_hook = f; }
 
-hipStream_t dn_stream() { return g_stream; }
+// A product whose launch is held back so that the calls that follow it can ride in its
+// epilogue (see "deferred epilogues" in elementwise.hip).  Everything that queues work, hands
+// out a workspace, moves data or waits for the device comes through dn_flush() first.
+static bool g_pending = false;
+static void (*g_flush_hook)() = nullptr;
+void dn_set_flush_hook(void (*f)()) { g_flush_hook = f; }
+void dn_set_pending(bool on) { g_pending = on; }
+void dn_flush() {
+  if (g_pending) {
+    g_pending = false;
+    if (g_flush_hook) g_flush_hook();
+  }
+}
+
+hipStream_t dn_stream() {
+  if (g_pending) dn_flush();
+  return g_stream;
+}
 bool dn_capturing() { return g_capturing; }
 
 // ------------------------------------------------------------------ scratch
@@ -49,6 +66,7 @@ static void block_flush();
 // hipMalloc for the library's own workspaces: when the device is out of memory, the blocks that
 // free_device_memory keeps for reuse are given back first and the request is made again.
 hipError_t dn_malloc(void** p, size_t bytes) {
+  dn_flush();
   hipError_t e = hipMalloc(p, bytes);
   if (e != hipSuccess) {
     hipGetLastError();
@@ -61,6 +79,7 @@ hipError_t dn_malloc(void** p, size_t bytes) {
 }
 
 void* dn_scratch(size_t bytes, int slot) {
+  dn_flush();      // (a held-back product may take, and grow, a workspace of its own when it is launched)
   if (bytes > g_scratch_bytes[slot]) {
     if (g_capturing) return nullptr;   // growing means freeing and allocating: not while a graph is recorded
 
@@ -122,6 +141,7 @@ static void* block_get(size_t bytes) {
 
 // false when the runtime refuses to free the block
 static bool block_put(void* p) {
+  dn_flush();
   auto it = g_block_bytes.find(p);
   if (it == g_block_bytes.end()) return hipFree(p) == hipSuccess;      // not one of ours (a caller's own allocation)
   const size_t bytes = it->second;
@@ -139,6 +159,7 @@ static int g_zero_words_n = 0;
 static bool g_zero_words_recorded = false;
 
 unsigned* dn_zero_words(int n) {
+  dn_flush();
   if (n > g_zero_words_n) {
     if (g_capturing) return nullptr;
     if (g_zero_words) {
@@ -240,12 +261,14 @@ int cublas_init(void) {
 }
 
 int cublas_shutdown(void) {
+  dn_flush();
   hipDeviceSynchronize();
   block_flush();
   return 0;
 }
 
 int cuda_set_device(int deviceId) {
+  dn_flush();
   int before = -1;
   hipGetDevice(&before);
   if (hipSetDevice(deviceId) != hipSuccess) return CUDA_ERROR;
@@ -270,7 +293,10 @@ int cuda_set_device(int deviceId) {
   return 0;
 }
 
-void cuda_sync_threads(void) { if (!g_capturing) hipDeviceSynchronize(); }
+void cuda_sync_threads(void) {
+  dn_flush();
+  if (!g_capturing) hipDeviceSynchronize();
+}
 
 // ---- HIP graphs (no counterpart in the reference): record a fixed sequence of library calls
 // once and replay it with one launch, for steps whose cost is the launching itself.
@@ -310,7 +336,7 @@ static bool stage_out(const float* src, float* host, int n) {
     g_stage_host->tag = 0;
   }
   const unsigned long long tag = ++g_stage_tag;
-  hipLaunchKernelGGL(k_stage_out, dim3(1), dim3(1024), 0, g_stream, src, g_stage_dev, n, tag);
+  hipLaunchKernelGGL(k_stage_out, dim3(1), dim3(1024), 0, dn_stream(), src, g_stage_dev, n, tag);
   if (hipGetLastError() != hipSuccess) return false;
   bool seen = false;
   for (int i = 0; i < DN_STAGE_POLLS && !seen; ++i) seen = __atomic_load_n(&g_stage_host->tag, __ATOMIC_ACQUIRE) == tag;
@@ -331,6 +357,7 @@ static bool stage_out(const float* src, float* host, int n) {
 // everything else the library does.
 void* graph_capture_begin(void) {
   if (g_capturing) return nullptr;
+  dn_flush();
   if (!g_capture_stream && hipStreamCreateWithFlags(&g_capture_stream, hipStreamNonBlocking) != hipSuccess) {
     g_capture_stream = nullptr;
     hipGetLastError();
@@ -349,6 +376,7 @@ void* graph_capture_begin(void) {
 // Ends the recording; returns an executable graph (NULL on failure) for graph_launch / graph_free.
 void* graph_capture_end(void) {
   if (!g_capturing) return nullptr;
+  dn_flush();      // (a held-back product belongs to the recording)
   hipGraph_t graph = nullptr;
   const hipError_t e = hipStreamEndCapture(g_capture_stream, &graph);
   g_stream = nullptr;
@@ -364,11 +392,13 @@ void* graph_capture_end(void) {
 
 int graph_launch(void* exec) {
   if (!exec || g_capturing) return ERROR_GENERIC;
+  dn_flush();
   return hipGraphLaunch((hipGraphExec_t)exec, nullptr) == hipSuccess ? 0 : CUDA_ERROR;
 }
 
 int graph_free(void* exec) {
   if (!exec) return 0;
+  dn_flush();
   hipDeviceSynchronize();
   const hipError_t e = hipGraphExecDestroy((hipGraphExec_t)exec);
   if (g_live_graphs > 0 && --g_live_graphs == 0) {
@@ -383,6 +413,7 @@ int graph_free(void* exec) {
 
 // Queue on a stream of the caller's (capturing != 0: the caller is capturing it); NULL, 0 afterwards.
 int graph_set_stream(void* stream, int capturing) {
+  dn_flush();
   g_stream = (hipStream_t)stream;
   g_capturing = capturing != 0;
   return 0;
@@ -406,6 +437,7 @@ int allocate_device_memory(cudamat* mat) {
 
 int copy_to_host(cudamat* mat) {
   if (!mat->on_device) return ERROR_NOT_ON_DEVICE;
+  dn_flush();
   if (g_capturing) return ERROR_UNSUPPORTED;
   const long long len = dn_len(mat);
   if (len > 0 && len <= DN_STAGE_FLOATS && stage_out(mat->data_device, mat->data_host, (int)len)) return 0;
@@ -417,6 +449,7 @@ int copy_to_host(cudamat* mat) {
 
 int copy_to_device(cudamat* mat) {
   if (g_capturing) return ERROR_UNSUPPORTED;
+  dn_flush();
   if (!mat->on_device) {
     int err = allocate_device_memory(mat);
     if (err) return err;

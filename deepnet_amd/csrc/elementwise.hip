@@ -349,8 +349,6 @@ extern "C" {
 DN_UNARY(sign, check_unary_trans, FSign{})
 DN_UNARY(apply_cos, check_unary, FCos{})
 DN_UNARY(apply_sin, check_unary, FSin{})
-DN_UNARY(apply_sigmoid, check_unary, FSigmoid{})
-DN_UNARY(apply_tanh, check_unary, FTanh{})
 DN_UNARY(apply_abs, check_unary, FAbs{})
 DN_UNARY(apply_log_1_plus_exp, check_unary, FLog1pExp{})
 DN_UNARY(apply_exp, check_unary, FExp{})
@@ -371,7 +369,6 @@ DN_SCALAR(less_than_scalar, check_unary_trans, FLtS)
 DN_SCALAR(greater_than_eq_scalar, check_unary_trans, FGeS)
 DN_SCALAR(greater_than_scalar, check_unary_trans, FGtS)
 DN_SCALAR(upper_bound_scalar, check_unary_trans, FUpperS)
-DN_SCALAR(lower_bound_scalar, check_unary_trans, FLowerS)
 DN_SCALAR(mult_by_scalar, check_unary, FMulS)
 DN_SCALAR(divide_by_scalar, check_unary, FDivS)
 DN_SCALAR(add_scalar, check_unary, FAddS)
@@ -419,7 +416,6 @@ int add_mult_sign(cudamat* mat1, cudamat* mat2, float mult) {
 }
 
 // ---- broadcasts
-DN_COLVEC(add_col_vec, FAdd{})
 DN_COLVEC(mult_by_col_vec, FMul{})
 DN_COLVEC(div_by_col_vec, FDiv{})
 DN_ROWVEC(add_row_vec, FAdd{})
@@ -469,6 +465,129 @@ int add_diagonal(cudamat* mat, cudamat* vec, cudamat* target) {
 
 int dn_gemm_fused(bool a_trans, bool b_trans, int M, int N, int K, const float* A, int lda, const float* B, int ldb,
                   float* C, int ldc, const float* bias, int act, bool* fused, const DnGemmSample* smp, bool* sampled);
+
+// ------------------------------------------------------------------ deferred epilogues
+// Every layer of deepnet computes its state as  dot -> add_col_vec -> apply_sigmoid (or
+// lower_bound(0), apply_tanh) [-> sample_bernoulli]  (deepnet/dbm.py:95-105,
+// neuralnet.py:138-160, cudamat/examples/rbm_cudamat.py:46-70): three or four launches of 2-5 us
+// each, and as many trips through the runtime's launch path, which is what such a step spends its
+// time on.  The product kernels can carry the bias, the activation and the sample in their
+// epilogue (dot_bias_act), so dot() with alpha = 1, beta = 0 does not launch at once: it is held
+// back, and while the calls that follow are exactly the rest of that sequence on the product's
+// own target they are folded into it; the launch happens at the activation (tanh, lower_bound),
+// at the sample, or at the first call of any other kind (everything that queues work, hands out a
+// workspace, moves data or waits for the device passes through dn_flush()).  The arithmetic is
+// that of the separate calls, bit for bit (tests/test_gpu_deferred.py), work reaches the stream
+// in call order, and a sequence that does not continue costs one kernel as before.
+struct DnPending {
+  bool active;
+  cudamat a, b, t, bias;
+  bool has_bias;
+  int act;            // 0 none yet, 1 sigmoid (waiting for a possible sample)
+};
+static DnPending g_pend = {};
+static bool g_no_defer = false;      // the library is issuing the calls of a sequence itself
+static bool g_defer_enabled = true;
+
+static int dot_bias_act_impl(rnd_struct* rnd, cudamat* mat1, cudamat* mat2, cudamat* bias, cudamat* target,
+                             cudamat* sample, int act);
+
+// Launches the held-back sequence (with the sample, when one is given).
+static int run_pending(rnd_struct* rnd, cudamat* sample) {
+  DnPending p = g_pend;
+  g_pend.active = false;
+  dn_set_pending(false);
+  const bool saved = g_no_defer;
+  g_no_defer = true;
+  const int e = dot_bias_act_impl(rnd, &p.a, &p.b, p.has_bias ? &p.bias : nullptr, &p.t, sample, p.act);
+  g_no_defer = saved;
+  return e;
+}
+static void flush_pending() {
+  if (g_pend.active) run_pending(nullptr, nullptr);
+}
+static const int g_flush_registered = (dn_set_flush_hook(flush_pending), 0);
+
+bool dn_defer_dot(cudamat* mat1, cudamat* mat2, cudamat* target, float beta, float alpha, int m, int n, int k) {
+  if (g_no_defer || !g_defer_enabled) return false;
+  if (alpha != 1.f || beta != 0.f || target->is_trans || m <= 1 || n <= 1 || k <= 0) return false;
+  dn_flush();                         // at most one product is held back
+  g_pend.active = true;
+  g_pend.a = *mat1; g_pend.b = *mat2; g_pend.t = *target;
+  g_pend.has_bias = false;
+  g_pend.act = 0;
+  dn_set_pending(true);
+  return true;
+}
+
+// x is the held-back product's target, as it was handed to dot()
+static inline bool pend_is(const cudamat* x) {
+  return x->on_device && !x->is_trans && x->data_device == g_pend.t.data_device && x->size[0] == g_pend.t.size[0] &&
+         x->size[1] == g_pend.t.size[1];
+}
+static inline bool pend_open() { return g_pend.active && !g_no_defer; }
+
+extern "C" {
+
+// Extension: switches the deferred epilogues on or off (on by default); returns the previous setting.
+int set_deferred_epilogues(int on) {
+  dn_flush();
+  const int before = g_defer_enabled ? 1 : 0;
+  g_defer_enabled = on != 0;
+  return before;
+}
+
+int add_col_vec(cudamat* mat, cudamat* vec, cudamat* target) {
+  if (pend_open() && !g_pend.has_bias && g_pend.act == 0 && pend_is(mat) && pend_is(target) && vec->on_device &&
+      !vec->is_trans && vec->size[0] == mat->size[0] && vec->size[1] == 1 && vec->data_device != mat->data_device) {
+    g_pend.bias = *vec;
+    g_pend.has_bias = true;
+    return 0;
+  }
+  if (int e = check_colvec(mat, vec, target)) return e;
+  return launch_bcast<true>(mat->data_device, vec->data_device, target->data_device, mat->size[0], mat->size[1], FAdd{});
+}
+
+int apply_sigmoid(cudamat* mat, cudamat* target) {
+  if (pend_open() && g_pend.act == 0 && pend_is(mat) && pend_is(target)) {
+    g_pend.act = 1;                   // stays held back: a sample of it may follow
+    return 0;
+  }
+  if (int e = check_unary(mat, target)) return e;
+  return launch_ew<1>(mat->data_device, nullptr, target->data_device, dn_len(mat), FSigmoid{});
+}
+
+int apply_tanh(cudamat* mat, cudamat* target) {
+  if (pend_open() && g_pend.act == 0 && pend_is(mat) && pend_is(target)) {
+    g_pend.act = 3;
+    return run_pending(nullptr, nullptr);
+  }
+  if (int e = check_unary(mat, target)) return e;
+  return launch_ew<1>(mat->data_device, nullptr, target->data_device, dn_len(mat), FTanh{});
+}
+
+int lower_bound_scalar(cudamat* mat, float val, cudamat* target) {
+  if (pend_open() && g_pend.act == 0 && val == 0.f && !signbit(val) && pend_is(mat) && pend_is(target)) {
+    g_pend.act = 2;
+    return run_pending(nullptr, nullptr);
+  }
+  if (int e = check_unary_trans(mat, target)) return e;
+  return launch_ew<1>(mat->data_device, nullptr, target->data_device, dn_len(mat), FLowerS{val});
+}
+
+}  // extern "C"
+
+// sample_bernoulli(rnd, mat, target) right after the held-back product's sigmoid: drawn by the
+// product's own launch.  Returns true when it took the call (*err is its result).
+bool dn_pending_sample(rnd_struct* rnd, cudamat* mat, cudamat* target, int* err) {
+  if (!(pend_open() && g_pend.act == 1 && pend_is(mat))) return false;
+  if (!target->on_device || target->is_trans || target->size[0] != mat->size[0] || target->size[1] != mat->size[1] ||
+      target->data_device == mat->data_device || !rnd || !rnd->dev_mults || !rnd->dev_words)
+    return false;
+  *err = run_pending(rnd, target);
+  return true;
+}
+
 
 // target = act(op(mat1) * op(mat2) + bias) and, with a generator and a sample matrix,
 // sample = (uniform < target), in as few launches as the shapes allow.
@@ -523,7 +642,12 @@ extern "C" {
 // launch where the product runs as a single kernel, bit-identical to the three calls.
 // bias: rows(target) x 1 or null.  act: 0 none, 1 sigmoid, 2 max(x, 0), 3 tanh.
 int dot_bias_act(cudamat* mat1, cudamat* mat2, cudamat* bias, cudamat* target, int act) {
-  return dot_bias_act_impl(nullptr, mat1, mat2, bias, target, nullptr, act);
+  dn_flush();
+  const bool saved = g_no_defer;
+  g_no_defer = true;
+  const int e = dot_bias_act_impl(nullptr, mat1, mat2, bias, target, nullptr, act);
+  g_no_defer = saved;
+  return e;
 }
 
 // Extension: dot_bias_act followed by sample_bernoulli(rnd_state, target, sample), the
@@ -534,7 +658,12 @@ int dot_bias_act(cudamat* mat1, cudamat* mat2, cudamat* bias, cudamat* target, i
 int dot_bias_act_sample(rnd_struct* rnd_state, cudamat* mat1, cudamat* mat2, cudamat* bias, cudamat* target,
                         cudamat* sample, int act) {
   if (!sample) return ERROR_GENERIC;
-  return dot_bias_act_impl(rnd_state, mat1, mat2, bias, target, sample, act);
+  dn_flush();
+  const bool saved = g_no_defer;
+  g_no_defer = true;
+  const int e = dot_bias_act_impl(rnd_state, mat1, mat2, bias, target, sample, act);
+  g_no_defer = saved;
+  return e;
 }
 
 }  // extern "C"

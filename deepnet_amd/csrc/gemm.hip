@@ -1269,6 +1269,8 @@ int dot(cudamat* mat1, cudamat* mat2, cudamat* target, float beta, float alpha) 
   // The target's own is_trans is ignored and its size[0] is used as the leading
   // dimension; refuse the combinations where that would write past its buffer.
   if ((long long)(n - 1) * ldc + m > dn_len(target)) return ERROR_INCOMPATIBLE_DIMENSIONS;
+  // (held back when the calls that follow may ride in its epilogue)
+  if (dn_defer_dot(mat1, mat2, target, beta, alpha, m, n, k)) return 0;
 
   // One output column: C(:,0) = op(A) * b with b = op(B)(:,0), k contiguous
   // values of B whichever way it is flagged (a k x 1 or 1 x k array).

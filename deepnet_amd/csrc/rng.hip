@@ -464,7 +464,15 @@ int fill_with_randn(rnd_struct* rnd_state, cudamat* mat) {
     return launch_rng(rnd_state, (size_t)dn_len(mat), OP{mat->data_device, target->data_device});      \
   }
 
-DN_SAMPLER(sample_bernoulli, OpBernoulli)
+int sample_bernoulli(rnd_struct* rnd_state, cudamat* mat, cudamat* target) {
+  // (the sample of a product that is being held back with its sigmoid is drawn by the product's launch)
+  int err = 0;
+  if (dn_pending_sample(rnd_state, mat, target, &err)) return err;
+  if (mat->size[0] != target->size[0] || mat->size[1] != target->size[1]) return ERROR_INCOMPATIBLE_DIMENSIONS;
+  if (!mat->on_device || !target->on_device) return ERROR_NOT_ON_DEVICE;
+  if (!rng_ready(rnd_state)) return ERROR_GENERIC;
+  return launch_rng(rnd_state, (size_t)dn_len(mat), OpBernoulli{mat->data_device, target->data_device});
+}
 DN_SAMPLER(sample_bernoulli_tanh, OpBernoulliTanh)
 DN_SAMPLER(sample_poisson, OpCopy)
 DN_SAMPLER(perturb_energy, OpPerturbEnergy)

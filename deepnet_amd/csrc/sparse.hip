@@ -43,6 +43,7 @@ k_sparse_dot(int m, int n, int k, int nnz, const float* data, const int* indptr,
 }
 
 static void release(cudamat_sparse* mat) {
+  dn_flush();
   if (mat->data_device.data) hipFree(mat->data_device.data);
   if (mat->data_device.indices) hipFree(mat->data_device.indices);
   if (mat->data_device.indptr) hipFree(mat->data_device.indptr);
@@ -94,6 +95,7 @@ int copy_sparse_to_device(cudamat_sparse* mat) {
     if (int err = allocate_device_memory_sparse(mat)) return err;
   }
   const size_t nnz = (size_t)mat->nnz, rows = (size_t)mat->size[0];
+  dn_flush();
   if ((nnz && hipMemcpy(mat->data_device.data, mat->data_host.data, nnz * sizeof(float), hipMemcpyHostToDevice) != hipSuccess) ||
       (nnz && hipMemcpy(mat->data_device.indices, mat->data_host.indices, nnz * sizeof(int), hipMemcpyHostToDevice) != hipSuccess) ||
       hipMemcpy(mat->data_device.indptr, mat->data_host.indptr, (rows + 1) * sizeof(int), hipMemcpyHostToDevice) != hipSuccess)

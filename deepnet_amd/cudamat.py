@@ -116,7 +116,7 @@ _SIGNATURES = {
     'correct_preds': (_i, [_M, _M, _M, _f]),
     'dot': (_i, [_M, _M, _M, _f, _f]),
     'dot_bias_act': (_i, [_M, _M, _M, _M, ct.c_int]),
-    'cd_update': (_i, [_M, _M, _M, _M, _M, _M, _M, _f]),
+    'cd_update': (_i, [_M, _M, _M, _M, _M, _M, _M, _f]), 'set_deferred_epilogues': (_i, [_i]),
     'dot_bias_act_sample': (_i, [ct.c_void_p, _M, _M, _M, _M, _M, ct.c_int]),
     'momentum_update': (_i, [_M, _M, _M, _f, _f, _f, _f, ct.c_int]),
     'momentum_update_many': (_i, [ct.c_int, ct.c_void_p, ct.c_void_p, ct.c_void_p, ct.c_void_p, ct.c_void_p, ct.c_void_p,
@@ -892,6 +892,14 @@ def dot_bias_act(m1, m2, bias=None, target=None, act='sigmoid', sample=None):
         _check(_cudamat.dot_bias_act_sample(CUDAMatrix.rnd_state_p, m1.p_mat, m2.p_mat, b, target.p_mat, sample.p_mat,
                                             _ACTS[act]))
     return target
+
+
+def set_deferred_epilogues(on):
+    """Extension of this backend: `dot` holds its launch back so that an `add_col_vec`, an activation
+    (`apply_sigmoid`, `lower_bound(0)`, `apply_tanh`) and a `sample_bernoulli` that follow it on its
+    own target run in the product's epilogue - one launch for the three or four calls of a layer's
+    up-pass, same bits, same order of work.  On by default; returns the previous setting."""
+    return bool(_cudamat.set_deferred_epilogues(1 if on else 0))
 
 
 def cd_update(W, bv, bh, v, h, v2, h2, eps):

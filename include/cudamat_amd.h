@@ -276,6 +276,15 @@ int apply_softmax_grad(cudamat* mat, cudamat* labels, cudamat* target);
 int get_softmax_correct(cudamat* mat, cudamat* labels, cudamat* target);
 int get_softmax_cross_entropy(cudamat* mat, cudamat* labels, cudamat* target, float tiny);
 
+/* ---- Extension: deferred epilogues.  dot() with alpha = 1, beta = 0 into an untransposed target holds
+ * its launch back; add_col_vec(target, bias, target), then apply_sigmoid / apply_tanh /
+ * lower_bound_scalar(.., 0, ..) in place, then sample_bernoulli(rnd, target, sample) are folded into that
+ * launch while they follow it directly (the sequence of cudamat/examples/rbm_cudamat.py:46-70 and
+ * deepnet/neuralnet.py:138-160).  Any other call launches what is held back first, so work is queued in
+ * call order and results are those of the separate launches, bit for bit.  set_deferred_epilogues(0)
+ * makes every call launch at once; returns the previous setting (default 1). ---- */
+int set_deferred_epilogues(int on);
+
 /* ---- Extension: the contrastive-divergence update of an RBM in one launch,
  *   W += eps (v h^T - v2 h2^T),  bv += eps (rowsums v - rowsums v2),  bh += eps (rowsums h - rowsums h2),
  * the six calls (two add_dot, four add_sums) of cudamat/examples/rbm_cudamat.py:57-85 and the statistics
