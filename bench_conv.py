@@ -78,7 +78,20 @@ def run(cm, ev, iters=10):
                 ms = _time(ev, fn, iters, cm.cuda_sync_threads)
                 gbs = nbytes / (ms * 1e-3) / 1e9
                 res[label] = {'us': round(ms * 1e3, 2), 'gbs': round(gbs, 1), 'frac_hbm': round(gbs / HBM_PEAK_GBS, 4)}
+            # the two pairs deepnet issues back to back, each as one launch (extensions of this backend):
+            # algorithmic bytes = the un-pooled map in + three pooled-size arrays out; four pooled-size arrays and the
+            # un-pooled map in + the un-pooled gradient out
+            p2, d2, n2 = cm.empty((N, F * O * O)), cm.empty((N, F * O * O)), cm.empty((N, F * O * O))
+            for label, fn, nbytes in (
+                    ('MaxPoolResponseNorm', lambda: cc.MaxPoolResponseNorm(up, p2, d2, n2, F, 3, 0, 2, O, 5, 0.001, 0.75),
+                     e_in + 3 * e_out),
+                    ('ResponseNormUndoMaxPoolUndo', lambda: cc.ResponseNormUndoMaxPoolUndo(grad, d2, n2, p2, up, undo, F, 3, 0, 2, O,
+                                                                                          5, 0.001, 0.75), 2 * e_in + 4 * e_out)):
+                ms = _time(ev, fn, iters, cm.cuda_sync_threads)
+                gbs = nbytes / (ms * 1e-3) / 1e9
+                res[label] = {'us': round(ms * 1e3, 2), 'gbs': round(gbs, 1), 'frac_hbm': round(gbs / HBM_PEAK_GBS, 4)}
             res['stage_fwd_bwd'] = _stage(cm, ev, iters, L, W, rng)
+            res['stage_fwd_bwd_fused_pool_norm'] = _stage(cm, ev, iters, L, W, rng, fused=True)
         out[name] = res
         for m in (X, W, Y, up, down, dw):
             m.free_device_memory()
@@ -108,7 +121,7 @@ def _local(cm, cc, ev, iters, rng):
     return res
 
 
-def _stage(cm, ev, iters, L, W, rng):
+def _stage(cm, ev, iters, L, W, rng, fused=False):
     """The whole conv stage of a deepnet edge at this layer (transpose, convUp, pool 3x3/2,
     rnorm 5, transpose; then the backward pass and the weight gradient) through
     deepnet_amd/convolutions.py: twelve library calls per step."""
@@ -121,6 +134,7 @@ def _stage(cm, ev, iters, L, W, rng):
     f = lambda a: cm.CUDAMatrix(np.asarray(a, dtype=np.float32, order='F'))
     inputs, deriv = f(rng.standard_normal((C * H * H, N))), f(rng.standard_normal((F * O * O, N)))
     edge = cv_mod.ConvEdge(W, cv, inputs.shape, deriv.shape)
+    edge.fused = fused
     state, grad = cm.empty(deriv.shape), cm.empty(W.shape)
     layer = types.SimpleNamespace(dirty=False, is_input=False, deriv=cm.empty(inputs.shape))
 

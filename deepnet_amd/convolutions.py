@@ -108,6 +108,12 @@ def ConvolveUp(inputs, edge, target):
     up = cc.convUp if edge.conv else cc.localUp
     up(edge.input_t, w, after_conv, n_locs, cv.padding, cv.stride, cv.num_colors)
     last = after_conv
+    if cv.max_pool and cv.rnorm and not cv.prob and getattr(edge, 'fused', False):
+        # this backend's one-launch form of the two calls below (same results)
+        cc.MaxPoolResponseNorm(last, edge.unrnormalized_layer, edge.denoms, edge.output_t, cv.num_filters, cv.pool_size, 0,
+                               cv.pool_stride, n_pool, cv.norm_size, cv.add_scale, cv.pow_scale)
+        edge.output_t.transpose(target)
+        return
     if cv.max_pool:
         pooled = edge.unrnormalized_layer if cv.rnorm else edge.output_t
         if cv.prob:
@@ -138,13 +144,21 @@ def AccumulateConvDeriv(layer, edge, deriv):
 
     deriv.transpose(edge.output_t2)
     grads, acts = edge.output_t2, edge.output_t
-    if cv.rnorm:
+    if cv.rnorm and cv.max_pool and getattr(edge, 'fused', False):
+        # this backend's one-launch form of the copy and the two calls below (same gradient in
+        # unpooled_layer; rnorm_temp1 / rnorm_temp2 are not written)
+        unpooled = edge.unpooled_layer
+        cc.ResponseNormUndoMaxPoolUndo(grads, edge.denoms, acts, edge.unrnormalized_layer, unpooled, unpooled,
+                                       cv.num_filters, cv.pool_size, 0, cv.pool_stride, n_pool, cv.norm_size,
+                                       cv.add_scale, cv.pow_scale)
+        grads = unpooled
+    elif cv.rnorm:
         # ResponseNormUndo overwrites its `acts` operand: work on a copy of the un-normalised layer.
         edge.rnorm_temp1.assign(edge.unrnormalized_layer)
         cc.ResponseNormUndo(grads, edge.denoms, acts, edge.rnorm_temp1, edge.rnorm_temp2, cv.num_filters,
                             cv.norm_size, cv.add_scale, cv.pow_scale)
         grads, acts = edge.rnorm_temp2, edge.unrnormalized_layer
-    if cv.max_pool:
+    if cv.max_pool and grads is not edge.unpooled_layer:
         # in place: the un-pooled activations are not needed once their gradient is known
         unpooled = edge.unpooled_layer
         cc.MaxPoolUndo(unpooled, unpooled, grads, acts, cv.pool_size, 0, cv.pool_stride, n_pool)

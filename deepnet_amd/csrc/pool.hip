@@ -243,6 +243,14 @@ k_pool_undo_block2(const float* imgs, const float* maxGrads, const float* maxAct
   }
 }
 
+// Loads the 16 bytes at p when ok, else returns `other`: from an address that is valid either way
+// (`safe`), so that the compiler emits a global load and a select (a conditional expression over the
+// load itself becomes a load through a pointer that may point at a stack copy of `other`).
+__device__ __forceinline__ float4 load4_or(const float* p, const float* safe, bool ok, float4 other) {
+  const float4 v = *reinterpret_cast<const float4*>(ok ? p : safe);
+  return ok ? v : other;
+}
+
 // x^y for the normalisation layers through the hardware log2 / exp2 (the reference uses
 // __powf there, cudamat_conv_kernels.cu:112-176); relative error below 1e-6 for the
 // denominators these layers see (1 <= x < ~1e3).
@@ -460,13 +468,13 @@ k_norm_lds(const float* a0, const float* a1, const float* a2, const float* win, 
       const bool ok = i < groups && q < qn;
       const size_t off = map0 + (size_t)N * pix + 4 * q;
       const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
-      w[k] = ok ? *reinterpret_cast<const float4*>(win + off) : z;
+      w[k] = load4_or(win + off, win + map0, ok, z);
       if (UNDO) {
-        og[k] = ok ? *reinterpret_cast<const float4*>(a0 + off) : z;
-        den[k] = ok ? *reinterpret_cast<const float4*>(a1 + off) : make_float4(1.f, 1.f, 1.f, 1.f);
-        keep0[k] = ok ? *reinterpret_cast<const float4*>(a2 + off) : z;
+        og[k] = load4_or(a0 + off, a0 + map0, ok, z);
+        den[k] = load4_or(a1 + off, a1 + map0, ok, make_float4(1.f, 1.f, 1.f, 1.f));
+        keep0[k] = load4_or(a2 + off, a2 + map0, ok, z);
       } else if (!SAME) {
-        keep0[k] = ok ? *reinterpret_cast<const float4*>(a0 + off) : z;
+        keep0[k] = load4_or(a0 + off, a0 + map0, ok, z);
       }
     }
 #pragma unroll
@@ -559,6 +567,259 @@ k_norm_lds(const float* a0, const float* a1, const float* a2, const float* win, 
       const float4 in = keep0[k], pw = keep1[k];
       *reinterpret_cast<float4*>(out1 + off) =
           make_float4(in.x * acc.x + pw.x, in.y * acc.y + pw.y, in.z * acc.z + pw.z, in.w * acc.w + pw.w);
+    }
+  }
+}
+
+// ------------------------------------------------------------------ pooling and normalisation in one launch
+// deepnet runs MaxPool -> ResponseNorm on the way up and ResponseNormUndo -> MaxPoolUndo on the way
+// down (deepnet/convolutions.py:58-66, 120-134).  The pooled map of a block of images is small
+// (15 x 15 x 32 images = 28.8 KB), so both pairs run as one kernel with it in LDS: the pooled
+// values never make the round trip through memory between the two stages, and the four
+// launches of a conv stage (each a 7-41 MB kernel whose load, compute and store phases do not
+// overlap at one workgroup per CU) become two.  The arithmetic of each stage is that of the
+// separate kernels above (same expressions, same order of additions): same bits.
+//
+// Up: a workgroup owns one map of QB * 4 images; a lane pools its (pooled pixel, 4 images)
+// groups straight from the un-pooled map (all window loads in flight), stores them, and the
+// workgroup goes on as k_norm_lds does.
+template <int QB, int SUBS, int STRIDE, int SIZE>
+__global__ void __launch_bounds__(NORM_LDS_THREADS)
+k_pool_norm_lds(const float* imgs, float* pooled, float* denoms, float* target, int N, int Sin, int start, int S,
+                FastDiv dS, int nblk, float addScale, float powScale) {
+  extern __shared__ float4 lds[];
+  const int f = blockIdx.x / nblk, b = blockIdx.x - f * nblk;
+  const int n0 = b * (QB * 4);
+  const int qn = (N - n0) / 4 < QB ? (N - n0) / 4 : QB;      // image groups of this block that exist
+  const int SS = S * S;
+  const int groups = SS * QB;
+  float4* tileA = lds;
+  float4* tileB = lds + groups;
+  const size_t in0 = (size_t)N * ((size_t)f * Sin * Sin) + n0;
+  const size_t map0 = (size_t)N * ((size_t)f * SS) + n0;
+  constexpr int org = -(SIZE / 2);
+  float4 keep0[NORM_LDS_SLOTS];
+#pragma unroll
+  for (int k = 0; k < NORM_LDS_SLOTS; ++k) {
+    const int i = (int)threadIdx.x + NORM_LDS_THREADS * k;
+    const int pix = i / QB, q = i - pix * QB;
+    const bool ok = i < groups && q < qn;
+    const int oy = (int)fd_div((uint32_t)pix, dS), ox = pix - oy * S;
+    const int sy = start + oy * STRIDE, sx = start + ox * STRIDE;
+    float4 w[SUBS][SUBS];
+    bool in[SUBS][SUBS];
+#pragma unroll
+    for (int dy = 0; dy < SUBS; ++dy)
+#pragma unroll
+      for (int dx = 0; dx < SUBS; ++dx) {
+        const int y = sy + dy, x = sx + dx;
+        in[dy][dx] = ok && (unsigned)y < (unsigned)Sin && (unsigned)x < (unsigned)Sin;
+        const int yc = y < 0 ? 0 : (y >= Sin ? Sin - 1 : y), xc = x < 0 ? 0 : (x >= Sin ? Sin - 1 : x);
+        w[dy][dx] = load4_or(imgs + in0 + (size_t)N * (yc * Sin + xc) + 4 * q, imgs + in0, ok, make_float4(0.f, 0.f, 0.f, 0.f));
+      }
+    float4 acc = make_float4(-2e38f, -2e38f, -2e38f, -2e38f);    // the start value of the pooling kernel
+#pragma unroll
+    for (int dy = 0; dy < SUBS; ++dy)
+#pragma unroll
+      for (int dx = 0; dx < SUBS; ++dx) {
+        const float4 v = w[dy][dx];
+        if (in[dy][dx]) {
+          acc.x = acc.x > v.x ? acc.x : v.x; acc.y = acc.y > v.y ? acc.y : v.y;
+          acc.z = acc.z > v.z ? acc.z : v.z; acc.w = acc.w > v.w ? acc.w : v.w;
+        }
+      }
+    if (!ok) acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    keep0[k] = acc;
+    if (ok) *reinterpret_cast<float4*>(pooled + map0 + (size_t)N * pix + 4 * q) = acc;
+    if (i < groups) tileA[i] = make_float4(acc.x * acc.x, acc.y * acc.y, acc.z * acc.z, acc.w * acc.w);
+  }
+  __syncthreads();
+  // sums along x
+#pragma unroll
+  for (int k = 0; k < NORM_LDS_SLOTS; ++k) {
+    const int i = (int)threadIdx.x + NORM_LDS_THREADS * k;
+    if (i >= groups) continue;
+    const int pix = i / QB;
+    const int y = (int)fd_div((uint32_t)pix, dS), x = pix - y * S;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    float4 t[SIZE];
+#pragma unroll
+    for (int d = 0; d < SIZE; ++d) {
+      const bool ok = (unsigned)(x + org + d) < (unsigned)S;
+      t[d] = tileA[i + (ok ? (org + d) * QB : 0)];
+    }
+#pragma unroll
+    for (int d = 0; d < SIZE; ++d) {
+      const bool ok = (unsigned)(x + org + d) < (unsigned)S;
+      acc.x += ok ? t[d].x : 0.f; acc.y += ok ? t[d].y : 0.f; acc.z += ok ? t[d].z : 0.f; acc.w += ok ? t[d].w : 0.f;
+    }
+    tileB[i] = acc;
+  }
+  __syncthreads();
+  // sums along y, then the output
+#pragma unroll
+  for (int k = 0; k < NORM_LDS_SLOTS; ++k) {
+    const int i = (int)threadIdx.x + NORM_LDS_THREADS * k;
+    if (i >= groups) continue;
+    const int pix = i / QB, q = i - pix * QB;
+    if (q >= qn) continue;
+    const int y = (int)fd_div((uint32_t)pix, dS);
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    float4 t[SIZE];
+#pragma unroll
+    for (int d = 0; d < SIZE; ++d) {
+      const bool ok = (unsigned)(y + org + d) < (unsigned)S;
+      t[d] = tileB[i + (ok ? (org + d) * S * QB : 0)];
+    }
+#pragma unroll
+    for (int d = 0; d < SIZE; ++d) {
+      const bool ok = (unsigned)(y + org + d) < (unsigned)S;
+      acc.x += ok ? t[d].x : 0.f; acc.y += ok ? t[d].y : 0.f; acc.z += ok ? t[d].z : 0.f; acc.w += ok ? t[d].w : 0.f;
+    }
+    const size_t off = map0 + (size_t)N * pix + 4 * q;
+    const float4 d = make_float4(1.f + addScale * acc.x, 1.f + addScale * acc.y, 1.f + addScale * acc.z, 1.f + addScale * acc.w);
+    const float4 in = keep0[k];
+    *reinterpret_cast<float4*>(denoms + off) = d;
+    *reinterpret_cast<float4*>(target + off) = make_float4(in.x * norm_pow(d.x, -powScale), in.y * norm_pow(d.y, -powScale),
+                                                           in.z * norm_pow(d.z, -powScale), in.w * norm_pow(d.w, -powScale));
+  }
+}
+
+// Down: the gradient of the normalisation for the pooled map (the arithmetic of k_norm_lds's
+// backward form; `acts` is only read) stays in LDS next to the pooled activations, and every
+// pixel of the un-pooled map then collects it from the windows that hold the pixel and whose
+// maximum it is, in the order of k_pool_undo_fixed.  target may be imgs (a lane reads its pixel
+// before it writes it).
+template <int QB, int SUBS, int STRIDE, int SIZE>
+__global__ void __launch_bounds__(NORM_LDS_THREADS)
+k_normundo_poolundo_lds(const float* outGrads, const float* denoms, const float* inputs, const float* acts, const float* imgs,
+                        float* target, int N, int Sin, FastDiv dSin, int start, int S, FastDiv dS, int nblk, float scale,
+                        float powScale) {
+  constexpr int NC = (SUBS + STRIDE - 1) / STRIDE;
+  extern __shared__ float4 lds[];
+  const int f = blockIdx.x / nblk, b = blockIdx.x - f * nblk;
+  const int n0 = b * (QB * 4);
+  const int qn = (N - n0) / 4 < QB ? (N - n0) / 4 : QB;
+  const int SS = S * S;
+  const int groups = SS * QB;
+  float4* tileA = lds;                 // the prepared acts, later the pooled map's gradient
+  float4* tileB = lds + groups;        // sums along x
+  float4* tileC = lds + 2 * groups;    // the pooled activations
+  const size_t in0 = (size_t)N * ((size_t)f * Sin * Sin) + n0;
+  const size_t map0 = (size_t)N * ((size_t)f * SS) + n0;
+  constexpr int org = SIZE / 2 - SIZE + 1;
+  float4 keep0[NORM_LDS_SLOTS], keep1[NORM_LDS_SLOTS];
+#pragma unroll
+  for (int k = 0; k < NORM_LDS_SLOTS; ++k) keep1[k] = make_float4(0.f, 0.f, 0.f, 0.f);
+  {
+    float4 w[NORM_LDS_SLOTS], og[NORM_LDS_SLOTS], den[NORM_LDS_SLOTS];
+#pragma unroll
+    for (int k = 0; k < NORM_LDS_SLOTS; ++k) {
+      const int i = (int)threadIdx.x + NORM_LDS_THREADS * k;
+      const int pix = i / QB, q = i - pix * QB;
+      const bool ok = i < groups && q < qn;
+      const size_t off = map0 + (size_t)N * pix + 4 * q;
+      const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
+      w[k] = load4_or(acts + off, acts + map0, ok, z);
+      og[k] = load4_or(outGrads + off, outGrads + map0, ok, z);
+      den[k] = load4_or(denoms + off, denoms + map0, ok, make_float4(1.f, 1.f, 1.f, 1.f));
+      keep0[k] = load4_or(inputs + off, inputs + map0, ok, z);
+    }
+#pragma unroll
+    for (int k = 0; k < NORM_LDS_SLOTS; ++k) {
+      const int i = (int)threadIdx.x + NORM_LDS_THREADS * k;
+      if (i >= groups) continue;
+      float4 t;
+      t.x = (scale * og[k].x * w[k].x) / den[k].x; t.y = (scale * og[k].y * w[k].y) / den[k].y;
+      t.z = (scale * og[k].z * w[k].z) / den[k].z; t.w = (scale * og[k].w * w[k].w) / den[k].w;
+      tileA[i] = t;
+      tileC[i] = w[k];
+      keep1[k] = make_float4(og[k].x * norm_pow(den[k].x, -powScale), og[k].y * norm_pow(den[k].y, -powScale),
+                             og[k].z * norm_pow(den[k].z, -powScale), og[k].w * norm_pow(den[k].w, -powScale));
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < NORM_LDS_SLOTS; ++k) {
+    const int i = (int)threadIdx.x + NORM_LDS_THREADS * k;
+    if (i >= groups) continue;
+    const int pix = i / QB;
+    const int y = (int)fd_div((uint32_t)pix, dS), x = pix - y * S;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    float4 t[SIZE];
+#pragma unroll
+    for (int d = 0; d < SIZE; ++d) {
+      const bool ok = (unsigned)(x + org + d) < (unsigned)S;
+      t[d] = tileA[i + (ok ? (org + d) * QB : 0)];
+    }
+#pragma unroll
+    for (int d = 0; d < SIZE; ++d) {
+      const bool ok = (unsigned)(x + org + d) < (unsigned)S;
+      acc.x += ok ? t[d].x : 0.f; acc.y += ok ? t[d].y : 0.f; acc.z += ok ? t[d].z : 0.f; acc.w += ok ? t[d].w : 0.f;
+    }
+    tileB[i] = acc;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < NORM_LDS_SLOTS; ++k) {
+    const int i = (int)threadIdx.x + NORM_LDS_THREADS * k;
+    if (i >= groups) continue;
+    const int pix = i / QB;
+    const int y = (int)fd_div((uint32_t)pix, dS);
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    float4 t[SIZE];
+#pragma unroll
+    for (int d = 0; d < SIZE; ++d) {
+      const bool ok = (unsigned)(y + org + d) < (unsigned)S;
+      t[d] = tileB[i + (ok ? (org + d) * S * QB : 0)];
+    }
+#pragma unroll
+    for (int d = 0; d < SIZE; ++d) {
+      const bool ok = (unsigned)(y + org + d) < (unsigned)S;
+      acc.x += ok ? t[d].x : 0.f; acc.y += ok ? t[d].y : 0.f; acc.z += ok ? t[d].z : 0.f; acc.w += ok ? t[d].w : 0.f;
+    }
+    const float4 in = keep0[k], pw = keep1[k];
+    // (tileA was last read before the barrier above)
+    tileA[i] = make_float4(in.x * acc.x + pw.x, in.y * acc.y + pw.y, in.z * acc.z + pw.z, in.w * acc.w + pw.w);
+  }
+  __syncthreads();
+  // the un-pooled map: every (pixel, 4 images) group of it, four per trip with their loads in flight together
+  const int items = Sin * Sin * QB;
+  for (int j0 = (int)threadIdx.x; j0 < items; j0 += 4 * NORM_LDS_THREADS) {
+    float4 img[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int j = j0 + u * NORM_LDS_THREADS;
+      const int pin = j / QB, q = j - pin * QB;
+      const bool ok = j < items && q < qn;
+      img[u] = load4_or(imgs + in0 + (size_t)N * pin + 4 * q, imgs + in0, ok, make_float4(0.f, 0.f, 0.f, 0.f));
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int j = j0 + u * NORM_LDS_THREADS;
+      const int pin = j / QB, q = j - pin * QB;
+      if (j >= items || q >= qn) continue;
+      const int py = (int)fd_div((uint32_t)pin, dSin), px = pin - py * Sin;
+      const int ty = py - start, tx = px - start;
+      const int oy_hi = ty >= 0 ? ty / STRIDE : 0, ox_hi = tx >= 0 ? tx / STRIDE : 0;
+      float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+      for (int jy = 0; jy < NC; ++jy) {
+        const int oy = oy_hi - (NC - 1 - jy);                  // ascending, as the reference scans
+        const bool vy = (ty >= 0) & (oy >= 0) & (oy < S) & (ty - oy * STRIDE < SUBS);
+        const int oyc = oy < 0 ? 0 : (oy >= S ? S - 1 : oy);
+#pragma unroll
+        for (int jx = 0; jx < NC; ++jx) {
+          const int ox = ox_hi - (NC - 1 - jx);
+          const bool ok = vy & (tx >= 0) & (ox >= 0) & (ox < S) & (tx - ox * STRIDE < SUBS);
+          const int oxc = ox < 0 ? 0 : (ox >= S ? S - 1 : ox);
+          const float4 ma = tileC[(oyc * S + oxc) * QB + q], mg = tileA[(oyc * S + oxc) * QB + q];
+          const float tx_ = (img[u].x == ma.x ? 1.f : 0.f) * mg.x, ty_ = (img[u].y == ma.y ? 1.f : 0.f) * mg.y;
+          const float tz_ = (img[u].z == ma.z ? 1.f : 0.f) * mg.z, tw_ = (img[u].w == ma.w ? 1.f : 0.f) * mg.w;
+          acc.x += ok ? tx_ : 0.f; acc.y += ok ? ty_ : 0.f; acc.z += ok ? tz_ : 0.f; acc.w += ok ? tw_ : 0.f;
+        }
+      }
+      *reinterpret_cast<float4*>(target + in0 + (size_t)N * pin + 4 * q) = acc;
     }
   }
 }
@@ -845,6 +1106,120 @@ void ContrastNormUndo(cudamat* outGrads, cudamat* denoms, cudamat* meanDiffs, cu
                       int numFilters, int sizeX, float addScale, float powScale) {
   rnorm_undo_impl(outGrads, denoms, meanDiffs, acts, targets, numFilters, sizeX, addScale, powScale,
                   "ContrastNormUndo");
+}
+
+// ---- Extensions (no counterpart in cudamat_conv.cu): the two pairs of calls deepnet always makes
+// back to back (deepnet/convolutions.py:58-66, 120-134), each in one launch where the pooled map of
+// 32 (16, 8, 4) images fits in LDS, the separate kernels otherwise; the same results either way.
+
+// pooled = MaxPool(images); (denoms, targets) = ResponseNorm(pooled)
+void MaxPoolResponseNorm(cudamat* images, cudamat* pooled, cudamat* denoms, cudamat* targets, int numFilters, int subsX,
+                         int startX, int strideX, int outputsX, int sizeX, float addScale, float powScale) {
+  const char* where = "MaxPoolResponseNorm";
+  conv_clear_error();
+  POOL_REQUIRE(images->on_device && pooled->on_device && denoms->on_device && targets->on_device, where);
+  POOL_REQUIRE(numFilters > 0 && subsX > 0 && strideX > 0 && outputsX > 0 && sizeX > 0, where);
+  const int N = images->size[0];
+  POOL_REQUIRE(N > 0 && images->size[1] % numFilters == 0, where);
+  const int Sin = isqrt_exact_p(images->size[1] / numFilters);
+  POOL_REQUIRE(Sin > 0, where);
+  for (cudamat* m : {pooled, denoms, targets})
+    POOL_REQUIRE(m->size[0] == N && m->size[1] == numFilters * outputsX * outputsX, where);
+  const bool v4 = N % 4 == 0 && all_aligned16({images->data_device, pooled->data_device, denoms->data_device, targets->data_device});
+  const int qb = v4 ? norm_lds_qb(N, outputsX) : 0;
+  const bool shapes = (strideX == 2 && (subsX == 2 || subsX == 3)) && (sizeX == 3 || sizeX == 5 || sizeX == 7);
+  const bool distinct = pooled->data_device != denoms->data_device && pooled->data_device != targets->data_device &&
+                        denoms->data_device != targets->data_device && images->data_device != pooled->data_device &&
+                        images->data_device != denoms->data_device && images->data_device != targets->data_device;
+  if (qb > 0 && shapes && distinct && (long long)N * images->size[1] < (1ll << 31)) {
+    const int nblk = (N + qb * 4 - 1) / (qb * 4);
+    const dim3 grid((unsigned)(numFilters * nblk)), block(NORM_LDS_THREADS);
+    const size_t lds = (size_t)2 * outputsX * outputsX * qb * sizeof(float4);
+    const FastDiv dS = make_fastdiv((uint32_t)outputsX);
+#define PN_GO(QB, SU, SZ) \
+  hipLaunchKernelGGL((k_pool_norm_lds<QB, SU, 2, SZ>), grid, block, lds, dn_stream(), (const float*)images->data_device, \
+                     pooled->data_device, denoms->data_device, targets->data_device, N, Sin, startX, outputsX, dS, nblk, addScale, powScale)
+#define PN_SZ(QB, SU) do { if (sizeX == 3) PN_GO(QB, SU, 3); else if (sizeX == 5) PN_GO(QB, SU, 5); else PN_GO(QB, SU, 7); } while (0)
+#define PN_SU(QB) do { if (subsX == 3) PN_SZ(QB, 3); else PN_SZ(QB, 2); } while (0)
+    if (qb == 8) PN_SU(8); else if (qb == 4) PN_SU(4); else if (qb == 2) PN_SU(2); else PN_SU(1);
+#undef PN_SU
+#undef PN_SZ
+#undef PN_GO
+    if (dn_launch_status()) conv_set_error(where, hipGetErrorString(hipGetLastError()));
+    return;
+  }
+  pool_impl(images, nullptr, pooled, numFilters, subsX, startX, strideX, outputsX, where);
+  if (conv_last_error()) return;
+  cnorm_impl(pooled, pooled, denoms, targets, numFilters, sizeX, addScale, powScale, where);
+}
+
+// targets = MaxPoolUndo(images, maxGrads = ResponseNormUndo(outGrads, denoms, inputs, acts), maxActs = acts):
+// `acts` are the pooled activations, and unlike ResponseNormUndo this call leaves them as they are.
+// targets may be images.
+void ResponseNormUndoMaxPoolUndo(cudamat* outGrads, cudamat* denoms, cudamat* inputs, cudamat* acts, cudamat* images,
+                                 cudamat* targets, int numFilters, int subsX, int startX, int strideX, int outputsX, int sizeX,
+                                 float addScale, float powScale) {
+  const char* where = "ResponseNormUndoMaxPoolUndo";
+  conv_clear_error();
+  POOL_REQUIRE(outGrads->on_device && denoms->on_device && inputs->on_device && acts->on_device && images->on_device &&
+               targets->on_device, where);
+  POOL_REQUIRE(numFilters > 0 && subsX > 0 && strideX > 0 && outputsX > 0 && sizeX > 0, where);
+  const int N = images->size[0];
+  POOL_REQUIRE(N > 0 && images->size[1] % numFilters == 0, where);
+  const int Sin = isqrt_exact_p(images->size[1] / numFilters);
+  POOL_REQUIRE(Sin > 0, where);
+  for (cudamat* m : {outGrads, denoms, inputs, acts})
+    POOL_REQUIRE(m->size[0] == N && m->size[1] == numFilters * outputsX * outputsX, where);
+  POOL_REQUIRE(targets->size[0] == N && targets->size[1] == images->size[1], where);
+  const bool v4 = N % 4 == 0 && all_aligned16({outGrads->data_device, denoms->data_device, inputs->data_device, acts->data_device,
+                                               images->data_device, targets->data_device});
+  const int qb = v4 ? norm_lds_qb(N, outputsX) : 0;
+  const bool shapes = (strideX == 2 && (subsX == 2 || subsX == 3)) && (sizeX == 3 || sizeX == 5 || sizeX == 7);
+  const size_t lds = (size_t)3 * outputsX * outputsX * (qb > 0 ? qb : 1) * sizeof(float4);
+  if (qb > 0 && shapes && lds <= 144 * 1024 && (long long)N * images->size[1] < (1ll << 31)) {
+    const int nblk = (N + qb * 4 - 1) / (qb * 4);
+    const dim3 grid((unsigned)(numFilters * nblk)), block(NORM_LDS_THREADS);
+    const FastDiv dS = make_fastdiv((uint32_t)outputsX), dSin = make_fastdiv((uint32_t)Sin);
+    const float scale = -2.f * addScale * powScale;
+    bool attr_ok = true;
+#define NP_GO(QB, SU, SZ)                                                                                                    \
+  do {                                                                                                                       \
+    static bool raised = false;   /* more than 64 KiB of dynamic LDS has to be asked for once per kernel */                  \
+    if (!raised && lds > 64 * 1024) {                                                                                        \
+      attr_ok = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_normundo_poolundo_lds<QB, SU, 2, SZ>),                  \
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, 144 * 1024) == hipSuccess;                   \
+      raised = attr_ok;                                                                                                      \
+    }                                                                                                                        \
+    if (attr_ok)                                                                                                             \
+      hipLaunchKernelGGL((k_normundo_poolundo_lds<QB, SU, 2, SZ>), grid, block, lds, dn_stream(),                            \
+                         (const float*)outGrads->data_device, (const float*)denoms->data_device,                             \
+                         (const float*)inputs->data_device, (const float*)acts->data_device, (const float*)images->data_device, \
+                         targets->data_device, N, Sin, dSin, startX, outputsX, dS, nblk, scale, powScale);                   \
+  } while (0)
+#define NP_SZ(QB, SU) do { if (sizeX == 3) NP_GO(QB, SU, 3); else if (sizeX == 5) NP_GO(QB, SU, 5); else NP_GO(QB, SU, 7); } while (0)
+#define NP_SU(QB) do { if (subsX == 3) NP_SZ(QB, 3); else NP_SZ(QB, 2); } while (0)
+    if (qb == 8) NP_SU(8); else if (qb == 4) NP_SU(4); else if (qb == 2) NP_SU(2); else NP_SU(1);
+#undef NP_SU
+#undef NP_SZ
+#undef NP_GO
+    if (attr_ok) {
+      if (dn_launch_status()) conv_set_error(where, hipGetErrorString(hipGetLastError()));
+      return;
+    }
+    hipGetLastError();
+  }
+  // the separate kernels, on a copy of the pooled activations (ResponseNormUndo overwrites its acts) and a
+  // temporary for the pooled map's gradient
+  const size_t pooled_floats = (size_t)N * acts->size[1];
+  float* ws = (float*)dn_scratch(2 * pooled_floats * sizeof(float), 2);
+  if (!ws) { conv_set_error(where, "out of device memory for the temporaries"); return; }
+  cudamat acts_copy = *acts, grad = *acts;
+  acts_copy.data_device = ws; acts_copy.owns_data = 0; acts_copy.is_trans = 0;
+  grad.data_device = ws + pooled_floats; grad.owns_data = 0; grad.is_trans = 0;
+  if (copy_on_device(acts, &acts_copy)) { conv_set_error(where, "copy of the pooled activations failed"); return; }
+  rnorm_undo_impl(outGrads, denoms, inputs, &acts_copy, &grad, numFilters, sizeX, addScale, powScale, where);
+  if (conv_last_error()) return;
+  MaxPoolUndo(images, &grad, acts, targets, subsX, startX, strideX, outputsX);
 }
 
 }  // extern "C"

@@ -38,6 +38,8 @@ _SIGNATURES = {
     'MaxPool': [_M, _M, _i, _i, _i, _i, _i],
     'ProbMaxPool': [_M, _M, _M, _i, _i, _i, _i, _i],
     'MaxPoolUndo': [_M, _M, _M, _M, _i, _i, _i, _i],
+    'MaxPoolResponseNorm': [_M, _M, _M, _M, _i, _i, _i, _i, _i, _i, _f, _f],
+    'ResponseNormUndoMaxPoolUndo': [_M, _M, _M, _M, _M, _M, _i, _i, _i, _i, _i, _i, _f, _f],
 }
 for _n, _args in _SIGNATURES.items():
     _fn = getattr(_ConvNet, _n)
@@ -184,3 +186,27 @@ def ContrastNormUndo(outGrad, denoms, meanDiffs, acts, targets, numChannels, siz
     assert targets.shape == outGrad.shape == denoms.shape == meanDiffs.shape == acts.shape
     _call('ContrastNormUndo', outGrad.p_mat, denoms.p_mat, meanDiffs.p_mat, acts.p_mat, targets.p_mat, numChannels,
           sizeX, float(addScale), float(powScale))
+
+
+def MaxPoolResponseNorm(images, pooled, denoms, targets, numChannels, subsX, startX, strideX, outputsX, sizeX, addScale,
+                        powScale):
+    """Extension of this backend (not in the reference): MaxPool(images -> pooled) followed by
+    ResponseNorm(pooled -> denoms, targets), the pair deepnet/convolutions.py:58-66 always issues
+    together, in one launch (the pooled map stays in LDS between the two stages); same results."""
+    numImages = images.shape[0]
+    assert pooled.shape == (numImages, numChannels * outputsX * outputsX)
+    assert targets.shape == pooled.shape == denoms.shape
+    _call('MaxPoolResponseNorm', images.p_mat, pooled.p_mat, denoms.p_mat, targets.p_mat, numChannels, subsX, startX,
+          strideX, outputsX, sizeX, float(addScale), float(powScale))
+
+
+def ResponseNormUndoMaxPoolUndo(outGrad, denoms, inGrad, acts, images, targets, numChannels, subsX, startX, strideX,
+                                outputsX, sizeX, addScale, powScale):
+    """Extension of this backend (not in the reference): ResponseNormUndo(outGrad, denoms, inGrad, acts)
+    followed by MaxPoolUndo(images, its result, acts -> targets), the pair of
+    deepnet/convolutions.py:120-134, in one launch.  ``acts`` are the pooled activations and are left
+    unchanged (ResponseNormUndo alone overwrites its ``acts``); ``targets`` may be ``images``."""
+    assert targets.shape == images.shape
+    assert outGrad.shape == denoms.shape == inGrad.shape == acts.shape
+    _call('ResponseNormUndoMaxPoolUndo', outGrad.p_mat, denoms.p_mat, inGrad.p_mat, acts.p_mat, images.p_mat,
+          targets.p_mat, numChannels, subsX, startX, strideX, outputsX, sizeX, float(addScale), float(powScale))

@@ -2,8 +2,8 @@
  * C ABI of the MI355X convolution / pooling / normalisation backend
  * (libcudamat_conv.so).  Names, argument order and argument meaning are those of
  * the 13 exports of the reference's cudamat/cudamat_conv.cu:1402-1456, which
- * cudamat/cudamat_conv.py binds through ctypes.  These 13 and conv_last_error are the
- * library's whole dynamic symbol table.  It links against libcudamat.so (found next to it),
+ * cudamat/cudamat_conv.py binds through ctypes.  These 13, the two fused pooling +
+ * normalisation calls at the end and conv_last_error are the library's whole dynamic symbol table.  It links against libcudamat.so (found next to it),
  * whose stream, workspaces and block cache it shares: calls of both libraries run in call
  * order on one stream and are recorded into the same HIP graphs.
  *
@@ -66,6 +66,18 @@ void ProbMaxPool(cudamat* images, cudamat* rnd, cudamat* targets, int numFilters
                  int outputsX);
 void MaxPoolUndo(cudamat* images, cudamat* maxGrads, cudamat* maxActs, cudamat* targets, int subsX, int startX,
                  int strideX, int outputsX);
+
+/* ---- Extensions (no counterpart in the reference): the two pairs of calls that deepnet/convolutions.py:58-66
+ * and :120-134 always issue back to back, each in one launch (the pooled map of a block of images stays in LDS
+ * between the two stages); results are those of the separate calls.
+ * MaxPoolResponseNorm: pooled = MaxPool(images); (denoms, targets) = ResponseNorm(pooled).
+ * ResponseNormUndoMaxPoolUndo: targets = MaxPoolUndo(images, maxGrads = ResponseNormUndo(outGrads, denoms, inputs,
+ * acts), maxActs = acts); `acts` (the pooled activations) is left unchanged; targets may be images. ---- */
+void MaxPoolResponseNorm(cudamat* images, cudamat* pooled, cudamat* denoms, cudamat* targets, int numFilters, int subsX,
+                         int startX, int strideX, int outputsX, int sizeX, float addScale, float powScale);
+void ResponseNormUndoMaxPoolUndo(cudamat* outGrads, cudamat* denoms, cudamat* inputs, cudamat* acts, cudamat* images,
+                                 cudamat* targets, int numFilters, int subsX, int startX, int strideX, int outputsX, int sizeX,
+                                 float addScale, float powScale);
 
 #ifdef __cplusplus
 }

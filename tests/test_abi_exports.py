@@ -29,14 +29,15 @@ def test_every_declared_symbol_is_exported(header, lib):
 
 def test_conv_library_exports_its_entry_points_and_nothing_else():
     """The reference's conv library exports its 13 entry points (cudamat_conv.cu:1402-1456); this one
-    adds conv_last_error and takes stream, workspaces and contraction kernels from libcudamat.so, so a
+    adds conv_last_error and the two fused pooling + normalisation calls, and takes stream, workspaces and contraction kernels from libcudamat.so, so a
     program that links both gets one copy of that state and no second `dot`."""
     import subprocess
     lib = os.path.join(ROOT, 'deepnet_amd', 'libcudamat_conv.so')
     out = subprocess.run(['nm', '-D', '--defined-only', lib], check=True, capture_output=True, text=True).stdout
     exported = sorted(line.split()[-1] for line in out.splitlines() if line.strip())
     want = sorted("""convUp convDown convOutp localUp localDown localOutp ResponseNorm ResponseNormUndo ContrastNorm
-    ContrastNormUndo MaxPool ProbMaxPool MaxPoolUndo conv_last_error""".split())
+    ContrastNormUndo MaxPool ProbMaxPool MaxPoolUndo conv_last_error MaxPoolResponseNorm
+    ResponseNormUndoMaxPoolUndo""".split())
     assert exported == want
     needed = subprocess.run(['readelf', '-d', lib], check=True, capture_output=True, text=True).stdout
     assert 'libcudamat.so' in needed and '$ORIGIN' in needed

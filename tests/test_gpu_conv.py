@@ -441,3 +441,80 @@ def test_pool_gradient_in_blocks_has_the_bits_of_the_general_kernel(cm, cc, rng,
     cc.MaxPool(X9, T9, F, subs, 0, 2, O)
     cc.MaxPoolUndo(X9, U9, cm.CUDAMatrix(_f(g9)), T9, subs, 0, 2, O)
     assert np.array_equal(U9.asarray()[1:], U.asarray())
+
+
+FUSED_POOL_NORM = [  # N, F, S (un-pooled side), subs, start, stride, norm size
+    (128, 64, 32, 3, 0, 2, 5),      # config 4
+    (32, 8, 32, 3, 0, 2, 5), (64, 4, 24, 3, 0, 2, 3), (32, 3, 13, 2, 0, 2, 3), (16, 4, 20, 2, 0, 2, 7), (100, 6, 27, 3, 0, 2, 5),
+    (32, 2, 9, 3, -1, 2, 3), (36, 3, 11, 3, 0, 2, 7),
+    # shapes the one-launch kernels do not take (other strides / windows / norm sizes, odd batches, large
+    # pooled maps): the entry points run the separate kernels
+    (8, 3, 9, 3, 0, 3, 3), (16, 2, 12, 4, -1, 3, 5), (6, 3, 8, 2, 0, 2, 4), (5, 2, 9, 3, 0, 2, 3), (16, 2, 60, 3, 0, 2, 5),
+]
+
+
+@pytest.mark.parametrize("N,F,S,subs,start,stride,size", FUSED_POOL_NORM)
+def test_pool_and_norm_in_one_launch_equal_the_separate_calls(cm, cc, rng, N, F, S, subs, start, stride, size):
+    """MaxPoolResponseNorm / ResponseNormUndoMaxPoolUndo against MaxPool -> ResponseNorm and
+    ResponseNormUndo (on a copy of the pooled layer) -> MaxPoolUndo: pooled values bit for bit, the
+    rest to 1e-5 (the one-launch kernels repeat the arithmetic of the separate ones; shapes that take
+    other separate kernels may differ in the order of additions), and against the definition."""
+    a, p = 0.001, 0.75
+    O = (S - start - subs + stride - 1) // stride + 1
+    x = _f(rng.standard_normal((N, F * S * S)) * 2)
+    X = cm.CUDAMatrix(x)
+    shape = (N, F * O * O)
+    pooled1, den1, out1 = cm.empty(shape), cm.empty(shape), cm.empty(shape)
+    cc.MaxPool(X, pooled1, F, subs, start, stride, O)
+    cc.ResponseNorm(pooled1, den1, out1, F, size, a, p)
+    pooled2, den2, out2 = cm.empty(shape), cm.empty(shape), cm.empty(shape)
+    for m in (pooled2, den2, out2):
+        m.assign(np.nan)
+    cc.MaxPoolResponseNorm(X, pooled2, den2, out2, F, subs, start, stride, O, size, a, p)
+    assert np.array_equal(pooled2.asarray(), pooled1.asarray())
+    assert np.allclose(den2.asarray(), den1.asarray(), rtol=1e-6) and np.allclose(out2.asarray(), out1.asarray(), rtol=1e-5, atol=1e-7)
+    want_pool = co.max_pool(x, F, subs, start, stride, O)
+    want_out, want_den = co.response_norm(want_pool.astype(np.float32), F, size, a, p)
+    assert np.array_equal(pooled2.asarray(), want_pool.astype(np.float32))
+    assert np.allclose(den2.asarray(), want_den, rtol=2e-6) and np.allclose(out2.asarray(), want_out, rtol=1e-5, atol=1e-7)
+    # backward, with deepnet's operand order (the normalised outputs as `inputs`, convolutions.py:111-122)
+    g = _f(rng.standard_normal(shape))
+    G = cm.CUDAMatrix(g)
+    tmp_acts, tmp_grad, undo1 = cm.empty(shape), cm.empty(shape), cm.empty(x.shape)
+    tmp_acts.assign(pooled1)
+    cc.ResponseNormUndo(G, den1, out1, tmp_acts, tmp_grad, F, size, a, p)
+    cc.MaxPoolUndo(X, undo1, tmp_grad, pooled1, subs, start, stride, O)
+    undo2 = cm.empty(x.shape)
+    undo2.assign(np.nan)
+    before = pooled2.asarray().copy()
+    cc.ResponseNormUndoMaxPoolUndo(G, den2, out2, pooled2, X, undo2, F, subs, start, stride, O, size, a, p)
+    assert np.array_equal(pooled2.asarray(), before)                  # the pooled layer is only read
+    assert np.allclose(undo2.asarray(), undo1.asarray(), rtol=1e-5, atol=1e-6)
+    ng, _ = co.response_norm_undo(g, den1.asarray(), out1.asarray(), pooled1.asarray(), F, size, a, p)
+    want_undo = co.max_pool_undo(x, ng.astype(np.float32), pooled1.asarray(), subs, start, stride, O)
+    assert np.allclose(undo2.asarray(), want_undo, rtol=1e-5, atol=1e-5)
+    # in place over the un-pooled layer, as convolutions.py uses it
+    X2 = cm.CUDAMatrix(x)
+    cc.ResponseNormUndoMaxPoolUndo(G, den2, out2, pooled2, X2, X2, F, subs, start, stride, O, size, a, p)
+    assert np.array_equal(X2.asarray().view(np.uint32), undo2.asarray().view(np.uint32))
+
+
+def test_pool_and_norm_in_one_launch_keep_the_bits_at_the_benchmark_layer(cm, cc, rng):
+    """At config 4 (64 maps of 32 x 32 -> 15 x 15, batch 128, norm size 5) the separate calls run the
+    kernels whose arithmetic the one-launch kernels repeat: every output has the same bits."""
+    N, F, S, O = 128, 64, 32, 15
+    x = _f(rng.standard_normal((N, F * S * S)))
+    X = cm.CUDAMatrix(x)
+    shape = (N, F * O * O)
+    pooled1, den1, out1, pooled2, den2, out2 = (cm.empty(shape) for _ in range(6))
+    cc.MaxPool(X, pooled1, F, 3, 0, 2, O); cc.ResponseNorm(pooled1, den1, out1, F, 5, 0.001, 0.75)
+    cc.MaxPoolResponseNorm(X, pooled2, den2, out2, F, 3, 0, 2, O, 5, 0.001, 0.75)
+    for a, b in ((pooled1, pooled2), (den1, den2), (out1, out2)):
+        assert np.array_equal(a.asarray().view(np.uint32), b.asarray().view(np.uint32))
+    G = cm.CUDAMatrix(_f(rng.standard_normal(shape)))
+    tmp_acts, tmp_grad, undo1, undo2 = cm.empty(shape), cm.empty(shape), cm.empty(x.shape), cm.empty(x.shape)
+    tmp_acts.assign(pooled1)
+    cc.ResponseNormUndo(G, den1, out1, tmp_acts, tmp_grad, F, 5, 0.001, 0.75)
+    cc.MaxPoolUndo(X, undo1, tmp_grad, pooled1, 3, 0, 2, O)
+    cc.ResponseNormUndoMaxPoolUndo(G, den2, out2, pooled2, X, undo2, F, 3, 0, 2, O, 5, 0.001, 0.75)
+    assert np.array_equal(undo1.asarray().view(np.uint32), undo2.asarray().view(np.uint32))
