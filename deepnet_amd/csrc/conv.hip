@@ -1680,6 +1680,146 @@ __global__ void __launch_bounds__(256, 1) k_conv_up_regs(ConvArgs p) {
   }
 }
 
+// ------------------------------------------------------------------ convUp, short reductions, one tile per wavefront
+// The same layers as k_conv_up_regs (reductions of at most 80 taps, at most 64 filters per
+// group) when the batch is a multiple of 64: a wavefront computes one (module, 64 images) tile
+// for all filters of the group and ends; two such wavefronts share a SIMD.
+//   v_mfma_f32_32x32x1_2b_f32: two 32 x 32 blocks of rank 1 per instruction.  Block rows are 32
+//   filters (first operand, the same values in both halves of the wavefront: one LDS read of
+//   the filter bank, kept as [tap][filter]); block columns are the images, block b the images
+//   32b .. 32b + 31 (second operand: lane = image, so a tap of the whole tile is ONE 256-byte
+//   run of the image tensor, its position a scalar: module origin + tap offset in an SGPR, a tap
+//   in the padding an out-of-range offset that reads as zero -- no vector arithmetic, no masks).
+// All taps of the tile are requested up front (in-order return: the MFMAs of tap k start when
+// tap k has arrived), the reduction is exactly the taps (75, not 80), the first 32 filters are
+// finished before the second 32 are started, so that their stores run under the second half's
+// MFMAs.  Filter size and colours are compile-time, so a tap's offset is three scalar
+// multiply-adds (with run-time sizes the 75 address computations were 3400 scalar instructions
+// in front of the first MFMA: 28.9 us; with them 17.1 us; with non-temporal stores 15.0 us).
+// Measured with the MFMAs replaced by plain arithmetic: 11.6 us (the 33.5 MB of stores and the
+// loads); what remains exposed is the second half's stores, which no MFMA is left to cover.
+typedef float f32x32 __attribute__((ext_vector_type(32)));
+// cache policy of the output stores: non-temporal (the 33.5 MB of outputs of the 3 -> 64 filters layer are
+// not read again by this kernel; measured 16.9 -> 15.0 us against the default policy)
+#define ST_NT 2
+template <int FB, int CG, int KF>   // FB: blocks of 32 filters of the group (1 or 2); CG colours per group, KF x KF filters
+__global__ void __launch_bounds__(256, 2) k_conv_up_taps(ConvArgs p) {
+  constexpr int K = CG * KF * KF, KMAX = K;
+  constexpr unsigned FAR = 0x80000000u;
+  __shared__ float w_lds[KMAX * 64];
+  const int tid = threadIdx.x, lane = tid & 63, li = lane & 31, half = lane >> 5;
+  const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int g = blockIdx.z;
+  const int NB = p.N >> 6;                                   // tiles of 64 images per module
+  const int T = p.M * NB;
+  const int t = blockIdx.x * 4 + wv;
+  const bool live = t < T;
+  const int m = live ? t / NB : 0, nb = live ? t - m * NB : 0;
+  const int my = (int)fd_div((unsigned)m, p.dMx), mx = m - my * p.Mx;
+  const int y0 = my * p.s + p.pad0, x0 = mx * p.s + p.pad0;
+  __amdgpu_buffer_rsrc_t r_img = __builtin_amdgcn_make_buffer_rsrc((void*)p.img, 0, (int)p.a_bytes, 0x00020000);
+  __amdgpu_buffer_rsrc_t r_flt = __builtin_amdgcn_make_buffer_rsrc((void*)p.flt, 0, (int)p.b_bytes, 0x00020000);
+  __amdgpu_buffer_rsrc_t r_out =
+      __builtin_amdgcn_make_buffer_rsrc((void*)p.out, 0, (int)((unsigned)p.N * (unsigned)p.M * (unsigned)p.F * 4u), 0x00020000);
+
+  // the group's filter bank: w(f, k) at f + F*k, read along f, kept as [k][64].  Requested before
+  // the tile's taps: waiting for it then leaves the (younger) tap loads in flight.
+  constexpr int PER = (KMAX * 64 + 255) / 256;
+  float w[PER];
+#pragma unroll
+  for (int it = 0; it < PER; ++it) {
+    const int e = tid + it * 256, f = e & 63, k = e >> 6;
+    const unsigned off = k < K && f < p.Fg ? ((unsigned)(g * p.Fg + f) + (unsigned)p.F * (unsigned)k) * 4u : FAR;
+    w[it] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r_flt, (int)off, 0, 0));
+  }
+  // the tile's taps: lane = image; a tap's position is wave-uniform (scalar registers only)
+  float a[KMAX];
+  {
+    const unsigned lane_off = (unsigned)lane * 4u;
+    const unsigned sx = (unsigned)p.N * 4u, sy = (unsigned)p.H * sx, sc = (unsigned)p.H * sy;
+    const unsigned base = (unsigned)(g * CG) * sc + (unsigned)y0 * sy + (unsigned)x0 * sx + (unsigned)(nb * 256);   // (wraps for y0, x0 < 0; taps inside the image come out right)
+    bool yv[KF], xv[KF];
+#pragma unroll
+    for (int i = 0; i < KF; ++i) {
+      yv[i] = live && (unsigned)(y0 + i) < (unsigned)p.H;
+      xv[i] = (unsigned)(x0 + i) < (unsigned)p.H;
+    }
+#pragma unroll
+    for (int c = 0; c < CG; ++c)
+#pragma unroll
+      for (int ky = 0; ky < KF; ++ky)
+#pragma unroll
+        for (int kx = 0; kx < KF; ++kx) {
+          const unsigned so = yv[ky] && xv[kx] ? base + (unsigned)c * sc + (unsigned)ky * sy + (unsigned)kx * sx : FAR;
+          a[(c * KF + ky) * KF + kx] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r_img, (int)lane_off, (int)so, 0));
+        }
+  }
+#pragma unroll
+  for (int it = 0; it < PER; ++it)
+    if (tid + it * 256 < KMAX * 64) w_lds[tid + it * 256] = w[it];
+  __syncthreads();
+  if (!live) return;
+
+  const unsigned fstride = (unsigned)p.N * (unsigned)p.M * 4u;          // bytes between filters in the output
+  // register r of lane (li, half): filter 8*((r%16)/4) + 4*half + r%4 of the block, image 32*(r/16) + li
+  const unsigned out_lane = ((unsigned)(nb * 64 + li) + (unsigned)p.N * (unsigned)m) * 4u + (unsigned)(4 * half) * fstride;
+  f32x32 acc[FB];
+  // filters are read RB - 1 taps ahead of their MFMA
+  constexpr int RB = 6;
+  auto run_block = [&](int fb, const f32x32* prev, int prev_fb) __attribute__((always_inline)) {
+    const float* wl = w_lds + fb * 32 + li;
+    float wq[RB];
+#pragma unroll
+    for (int i = 0; i < RB - 1; ++i) wq[i] = wl[i * 64];
+    f32x32 c;
+#pragma unroll
+    for (int v = 0; v < 32; ++v) c[v] = 0.f;
+#pragma unroll
+    for (int k = 0; k < KMAX; ++k) {
+      if (k < K) {
+        if (k + RB - 1 < KMAX) wq[(k + RB - 1) % RB] = wl[(k + RB - 1) * 64];
+        c = __builtin_amdgcn_mfma_f32_32x32x1f32(wq[k % RB], a[k], c, 0, 0, 0);
+        // the previous block's outputs leave under these MFMAs, one store per tap
+        if (prev && k < 32) {
+          const float val = (*prev)[k];
+          const int f_in_block = 8 * ((k & 15) >> 2) + (k & 3);
+          const bool ok = prev_fb * 32 + f_in_block < p.Fg;   // (wave-uniform: filters per group are a multiple of 8, so lanes 32-63, four filters on, agree)
+          const unsigned so = ok ? (unsigned)(g * p.Fg + prev_fb * 32 + f_in_block) * fstride + (unsigned)(k >> 4) * 128u : FAR;
+          __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(val), r_out, (int)out_lane, (int)so, ST_NT);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    acc[fb] = c;
+  };
+  run_block(0, nullptr, 0);
+  if (FB == 2) run_block(1, &acc[0], 0);
+  // the last block's outputs
+  {
+    constexpr int last = FB - 1;
+#pragma unroll
+    for (int r = 0; r < 32; ++r) {
+      const float val = acc[last][r];
+      const int f_in_block = 8 * ((r & 15) >> 2) + (r & 3);
+      const bool ok = last * 32 + f_in_block < p.Fg;
+      const unsigned so = ok ? (unsigned)(g * p.Fg + last * 32 + f_in_block) * fstride + (unsigned)(r >> 4) * 128u : FAR;
+      __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(val), r_out, (int)out_lane, (int)so, ST_NT);
+    }
+  }
+  // (K < 32 taps: the first block's outputs that did not leave under the second block's MFMAs)
+  if (FB == 2 && K < 32) {
+#pragma unroll
+    for (int r = 0; r < 32; ++r)
+      if (r >= K) {
+        const float val = acc[0][r];
+        const int f_in_block = 8 * ((r & 15) >> 2) + (r & 3);
+        const bool ok = f_in_block < p.Fg;
+        const unsigned so = ok ? (unsigned)(g * p.Fg + f_in_block) * fstride + (unsigned)(r >> 4) * 128u : FAR;
+        __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(val), r_out, (int)out_lane, (int)so, ST_NT);
+      }
+  }
+}
+
 static bool fast_ok(const ConvArgs& a) {
   // (the gathers use 32-bit byte offsets that include a margin for the padding / tap shift)
   const long long margin = (long long)a.N * ((long long)(a.k + (a.pad0 < 0 ? -a.pad0 : 0)) * (a.H + a.Mx) + a.k + a.H);
@@ -1878,6 +2018,17 @@ static void conv_up_impl(cudamat* images, cudamat* filters, cudamat* targets, in
   const int K = a.Cg * a.kk2;
   if (!local && fast_ok(a) && K <= 80 && a.Fg <= 64 && N % 32 == 0 && a.a_bytes != 0 && a.b_bytes != 0 &&
       (long long)N * M * F * 4 < (1ll << 31)) {  // (32-bit offsets into the output, and an out-of-range offset beyond it)
+    if (N % 64 == 0 && (k == 3 || k == 5) && (a.Cg == 1 || a.Cg == 3)) {
+      // one (module, 64 images) tile per wavefront, two wavefronts per SIMD
+      const long long tiles64 = (long long)M * (N / 64);
+      const dim3 grid64((unsigned)((tiles64 + 3) / 4), 1, numGroups);
+#define UP_TAPS(CG, KF) do { if (a.Fg <= 32) hipLaunchKernelGGL((k_conv_up_taps<1, CG, KF>), grid64, dim3(256), 0, dn_stream(), a); \
+                             else hipLaunchKernelGGL((k_conv_up_taps<2, CG, KF>), grid64, dim3(256), 0, dn_stream(), a); } while (0)
+      if (a.Cg == 3 && k == 5) UP_TAPS(3, 5); else if (a.Cg == 3) UP_TAPS(3, 3); else if (k == 5) UP_TAPS(1, 5); else UP_TAPS(1, 3);
+#undef UP_TAPS
+      if (dn_launch_status()) conv_set_error(where, hipGetErrorString(hipGetLastError()));
+      return;
+    }
     // short reduction, few filters per group: filter bank in registers
     const long long tiles = (long long)M * (N / 32);
     long long blocks = (tiles + 3) / 4;

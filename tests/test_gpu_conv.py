@@ -65,6 +65,12 @@ CASES = [  # N, C, H, F, k, stride, padding, groups
     (64, 8, 6, 144, 3, 1, 0, 2),     # 2 groups of 4 colours / 72 filters, no padding
     (32, 2, 9, 128, 5, 1, 1, 1),     # 128 filters in one group
     (160, 1, 5, 40, 5, 1, 3, 1),     # one colour, 5 image blocks, a single tile row
+    # convUp with one (module, 64 images) tile per wavefront (1 or 3 colours, 3 x 3 or 5 x 5 filters, batch a multiple of 64):
+    (64, 3, 9, 16, 3, 2, 1, 1),      # stride 2, 16 filters (one block of 32, half used)
+    (192, 1, 7, 64, 3, 1, 2, 1),     # one colour, padding wider than half the filter, three image tiles per module
+    (64, 6, 8, 128, 5, 1, 2, 2),     # 2 groups of 3 colours / 64 filters
+    (128, 3, 6, 8, 5, 1, 4, 1),      # 8 filters, every module touches the padding
+    (64, 3, 11, 40, 5, 3, 0, 1),     # 40 filters (second block of 32 a quarter used), stride 3, last module short of the edge
 ]
 
 
