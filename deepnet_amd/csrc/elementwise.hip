@@ -369,14 +369,8 @@ DN_SCALAR(less_than_scalar, check_unary_trans, FLtS)
 DN_SCALAR(greater_than_eq_scalar, check_unary_trans, FGeS)
 DN_SCALAR(greater_than_scalar, check_unary_trans, FGtS)
 DN_SCALAR(upper_bound_scalar, check_unary_trans, FUpperS)
-DN_SCALAR(mult_by_scalar, check_unary, FMulS)
 DN_SCALAR(divide_by_scalar, check_unary, FDivS)
 DN_SCALAR(add_scalar, check_unary, FAddS)
-
-int assign_scalar(cudamat* mat, float alpha) {
-  if (!mat->on_device) return ERROR_NOT_ON_DEVICE;
-  return launch_ew<0>(nullptr, nullptr, mat->data_device, dn_len(mat), FAssignS{alpha});
-}
 
 // ---- binary
 DN_BINARY(less_than_eq, check_binary, FLe{})
@@ -399,21 +393,6 @@ DN_BINARY(apply_pow_matrix, check_binary_notrans, FPowMat{})
 DN_BINARY_PARAM(compute_cross_entropy, FCrossEntropy)
 DN_BINARY_PARAM(compute_cross_entropy_bernoulli, FCrossEntropyBernoulli)
 DN_BINARY_PARAM(correct_preds, FCorrectPreds)
-
-// mat1 += alpha * mat2 (cudamat.cu:1763-1781): device, transposedness, dims; no target.
-int add_mult(cudamat* mat1, cudamat* mat2, float alpha) {
-  if (!mat1->on_device || !mat2->on_device) return ERROR_NOT_ON_DEVICE;
-  if (mat1->is_trans != mat2->is_trans) return ERROR_TRANSPOSEDNESS;
-  if (!same_dims(mat1, mat2)) return ERROR_INCOMPATIBLE_DIMENSIONS;
-  return launch_ew<2>(mat1->data_device, mat2->data_device, mat1->data_device, dn_len(mat1), FAxpy{alpha});
-}
-
-int add_mult_sign(cudamat* mat1, cudamat* mat2, float mult) {
-  if (!mat1->on_device || !mat2->on_device) return ERROR_NOT_ON_DEVICE;
-  if (mat1->is_trans != mat2->is_trans) return ERROR_TRANSPOSEDNESS;
-  if (!same_dims(mat1, mat2)) return ERROR_INCOMPATIBLE_DIMENSIONS;
-  return launch_ew<2>(mat1->data_device, mat2->data_device, mat1->data_device, dn_len(mat1), FAddMultSign{mult});
-}
 
 // ---- broadcasts
 DN_COLVEC(mult_by_col_vec, FMul{})
@@ -503,8 +482,11 @@ static int run_pending(rnd_struct* rnd, cudamat* sample) {
   g_no_defer = saved;
   return e;
 }
+static int run_queue(bool reset);
+static int queued_calls();
 static void flush_pending() {
   if (g_pend.active) run_pending(nullptr, nullptr);
+  if (queued_calls() > 0) run_queue(false);
 }
 static const int g_flush_registered = (dn_set_flush_hook(flush_pending), 0);
 
@@ -573,6 +555,136 @@ int lower_bound_scalar(cudamat* mat, float val, cudamat* target) {
   }
   if (int e = check_unary_trans(mat, target)) return e;
   return launch_ew<1>(mat->data_device, nullptr, target->data_device, dn_len(mat), FLowerS{val});
+}
+
+}  // extern "C"
+
+
+// ---- the parameter update.  deepnet/parameter.py:80-106 spells it
+//   w_delta.mult(momentum) [; w_delta.add_mult(w, l2)] [; w_delta.add_mult_sign(w, l1)] ; w_delta.add_mult(gradient)
+//   ; w.add_mult(w_delta, -epsilon) [; gradient.assign(0)]
+// four to six launches over the same three arrays; k_momentum_update does it in one pass with the same
+// roundings.  An in-place mult_by_scalar is held back, the add_mult / add_mult_sign calls into the same
+// matrix that follow it are queued, and when the add_mult that reads that matrix arrives and the queue spells
+// the update, one launch does it all (an assign_scalar(gradient, 0) that follows directly rides along);
+// any other call, or a queue that spells something else, launches the queued calls one by one, in order.
+enum { EQ_MULS, EQ_AXPY, EQ_AXPYSIGN };
+struct EqOp {
+  int kind;
+  cudamat dst, src;
+  float s;
+};
+static EqOp g_eq[4];
+static int g_eqn = 0;
+static bool g_eq_ready = false;       // the queue spells an update; w, -epsilon and the roles are in g_up
+static struct {
+  cudamat w, g;
+  float eps, l2, l1;
+  int flags;
+} g_up;
+
+static inline bool same_mat(const cudamat* a, const cudamat* b) {
+  return a->data_device == b->data_device && a->size[0] == b->size[0] && a->size[1] == b->size[1] &&
+         a->is_trans == b->is_trans;
+}
+static inline bool eq_open() { return g_eqn > 0 && !g_no_defer; }
+static int queued_calls() { return g_eqn; }
+
+extern "C" int momentum_update(cudamat* w, cudamat* w_delta, cudamat* gradient, float momentum, float l2_decay,
+                               float l1_decay, float epsilon, int flags);
+
+// Launches what the queue holds: the one-pass update if it spells one, else its calls one by one.
+static int run_queue(bool reset) {
+  EqOp q[4];
+  const int n = g_eqn;
+  for (int i = 0; i < n; ++i) q[i] = g_eq[i];
+  const bool ready = g_eq_ready;
+  g_eqn = 0;
+  g_eq_ready = false;
+  dn_set_pending(false);
+  const bool saved = g_no_defer;
+  g_no_defer = true;
+  int e = 0;
+  if (ready) {
+    e = momentum_update(&g_up.w, &q[0].dst, &g_up.g, q[0].s, g_up.l2, g_up.l1, g_up.eps, g_up.flags | (reset ? 4 : 0));
+  } else {
+    for (int i = 0; i < n && !e; ++i) {
+      if (q[i].kind == EQ_MULS) e = mult_by_scalar(&q[i].dst, q[i].s, &q[i].dst);
+      else if (q[i].kind == EQ_AXPY) e = add_mult(&q[i].dst, &q[i].src, q[i].s);
+      else e = add_mult_sign(&q[i].dst, &q[i].src, q[i].s);
+    }
+  }
+  g_no_defer = saved;
+  return e;
+}
+
+// The add_mult that reads the scaled matrix has arrived (w += alpha * w_delta): does the queue spell the update?
+static bool queue_spells_update(const cudamat* w, float alpha) {
+  const cudamat* wd = &g_eq[0].dst;
+  if (same_mat(w, wd) || w->data_device == wd->data_device || !same_dims(w, wd) || w->is_trans != wd->is_trans) return false;
+  int i = 1;
+  g_up.flags = 0; g_up.l2 = 0.f; g_up.l1 = 0.f;
+  if (i < g_eqn - 1 && g_eq[i].kind == EQ_AXPY && same_mat(&g_eq[i].src, w)) { g_up.l2 = g_eq[i].s; g_up.flags |= 1; ++i; }
+  if (i < g_eqn - 1 && g_eq[i].kind == EQ_AXPYSIGN && same_mat(&g_eq[i].src, w)) { g_up.l1 = g_eq[i].s; g_up.flags |= 2; ++i; }
+  if (i != g_eqn - 1 || g_eq[i].kind != EQ_AXPY || g_eq[i].s != 1.f) return false;
+  const cudamat* g = &g_eq[i].src;
+  if (g->data_device == w->data_device || g->data_device == wd->data_device) return false;
+  g_up.w = *w;
+  g_up.g = *g;
+  g_up.eps = -alpha;
+  return true;
+}
+
+extern "C" {
+
+int mult_by_scalar(cudamat* mat, float val, cudamat* target) {
+  if (int e = check_unary(mat, target)) return e;
+  if (!g_no_defer && g_defer_enabled && mat->data_device == target->data_device && dn_len(mat) > 0) {
+    dn_flush();
+    g_eq[0].kind = EQ_MULS; g_eq[0].dst = *mat; g_eq[0].src = *mat; g_eq[0].s = val;
+    g_eqn = 1;
+    g_eq_ready = false;
+    dn_set_pending(true);
+    return 0;
+  }
+  return launch_ew<1>(mat->data_device, nullptr, target->data_device, dn_len(mat), FMulS{val});
+}
+
+int assign_scalar(cudamat* mat, float alpha) {
+  if (!mat->on_device) return ERROR_NOT_ON_DEVICE;
+  if (eq_open() && g_eq_ready && alpha == 0.f && !signbit(alpha) && same_mat(mat, &g_up.g)) return run_queue(true);
+  return launch_ew<0>(nullptr, nullptr, mat->data_device, dn_len(mat), FAssignS{alpha});
+}
+
+// mat1 += alpha * mat2 (cudamat.cu:1763-1781): device, transposedness, dims; no target.
+int add_mult(cudamat* mat1, cudamat* mat2, float alpha) {
+  if (!mat1->on_device || !mat2->on_device) return ERROR_NOT_ON_DEVICE;
+  if (mat1->is_trans != mat2->is_trans) return ERROR_TRANSPOSEDNESS;
+  if (!same_dims(mat1, mat2)) return ERROR_INCOMPATIBLE_DIMENSIONS;
+  if (eq_open() && !g_eq_ready) {
+    if (same_mat(mat1, &g_eq[0].dst) && mat2->data_device != mat1->data_device && g_eqn < 4) {
+      g_eq[g_eqn].kind = EQ_AXPY; g_eq[g_eqn].dst = *mat1; g_eq[g_eqn].src = *mat2; g_eq[g_eqn].s = alpha;
+      ++g_eqn;
+      return 0;
+    }
+    if (same_mat(mat2, &g_eq[0].dst) && g_eqn >= 2 && queue_spells_update(mat1, alpha)) {
+      g_eq_ready = true;          // held back one more call: the gradient's reset may follow
+      return 0;
+    }
+  }
+  return launch_ew<2>(mat1->data_device, mat2->data_device, mat1->data_device, dn_len(mat1), FAxpy{alpha});
+}
+
+int add_mult_sign(cudamat* mat1, cudamat* mat2, float mult) {
+  if (!mat1->on_device || !mat2->on_device) return ERROR_NOT_ON_DEVICE;
+  if (mat1->is_trans != mat2->is_trans) return ERROR_TRANSPOSEDNESS;
+  if (!same_dims(mat1, mat2)) return ERROR_INCOMPATIBLE_DIMENSIONS;
+  if (eq_open() && !g_eq_ready && same_mat(mat1, &g_eq[0].dst) && mat2->data_device != mat1->data_device && g_eqn < 4) {
+    g_eq[g_eqn].kind = EQ_AXPYSIGN; g_eq[g_eqn].dst = *mat1; g_eq[g_eqn].src = *mat2; g_eq[g_eqn].s = mult;
+    ++g_eqn;
+    return 0;
+  }
+  return launch_ew<2>(mat1->data_device, mat2->data_device, mat1->data_device, dn_len(mat1), FAddMultSign{mult});
 }
 
 }  // extern "C"

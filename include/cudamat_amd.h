@@ -281,8 +281,11 @@ int get_softmax_cross_entropy(cudamat* mat, cudamat* labels, cudamat* target, fl
  * lower_bound_scalar(.., 0, ..) in place, then sample_bernoulli(rnd, target, sample) are folded into that
  * launch while they follow it directly (the sequence of cudamat/examples/rbm_cudamat.py:46-70 and
  * deepnet/neuralnet.py:138-160).  Any other call launches what is held back first, so work is queued in
- * call order and results are those of the separate launches, bit for bit.  set_deferred_epilogues(0)
- * makes every call launch at once; returns the previous setting (default 1). ---- */
+ * call order and results are those of the separate launches, bit for bit.  Likewise an in-place
+ * mult_by_scalar is held back and the add_mult / add_mult_sign calls of a parameter update
+ * (deepnet/parameter.py:80-106: w_delta *= momentum [; w_delta += l2 w] [; w_delta += l1 sign(w)] ;
+ * w_delta += gradient ; w += -epsilon w_delta [; gradient = 0]) run as one pass when they spell it.
+ * set_deferred_epilogues(0) makes every call launch at once; returns the previous setting (default 1). ---- */
 int set_deferred_epilogues(int on);
 
 /* ---- Extension: the contrastive-divergence update of an RBM in one launch,

@@ -1,5 +1,7 @@
 """Deferred epilogues: dot() holds its launch back and the add_col_vec / activation / sample calls
-that follow it on its own target run in the product's epilogue.  Every sequence here is run with
+that follow it on its own target run in the product's epilogue; an in-place mult_by_scalar is held
+back likewise and the add_mult / add_mult_sign calls of a parameter update (deepnet/parameter.py:80-106)
+are folded into one pass.  Every sequence here is run with
 the deferral switched off (each call its own launch) and on, and must leave the same bits in every
 matrix it touches and the same generator state; sequences that must NOT be folded (another
 matrix in between, a second bias, operands that change between the calls, reads, frees) are
@@ -114,7 +116,85 @@ def seq_lower_bound_not_zero(cm, a, B, bias, other, T, S):
     cm.dot(a, B, target=T); T.add_col_vec(bias); T.lower_bound(0.25)
 
 
-SEQS = [seq_sigmoid, seq_sigmoid_sample, seq_relu, seq_tanh, seq_no_bias, seq_bias_only_then_read, seq_dot_alone_then_other_work,
+# ---- the parameter update of deepnet/parameter.py:80-106 (w = T, w_delta = S, gradient = other)
+
+def _params(T, S, other):
+    T.assign(0.25); S.assign(-0.5)                      # (the harness fills them with constants: make them vary)
+    T.add(other); S.subtract(other)
+    return T, S, other
+
+
+def seq_update_plain(cm, a, B, bias, other, T, S):
+    w, wd, g = _params(T, S, other)
+    wd.mult(0.9); wd.add_mult(g); w.add_mult(wd, -0.01)
+
+
+def seq_update_with_reset(cm, a, B, bias, other, T, S):
+    w, wd, g = _params(T, S, other)
+    wd.mult(0.9); wd.add_mult(g); w.add_mult(wd, -0.01); g.assign(0)
+
+
+def seq_update_l2_l1_reset(cm, a, B, bias, other, T, S):
+    w, wd, g = _params(T, S, other)
+    wd.mult(0.5); wd.add_mult(w, 0.001); wd.add_mult_sign(w, 0.0005); wd.add_mult(g); w.add_mult(wd, -0.1); g.assign(0)
+
+
+def seq_update_l2_only(cm, a, B, bias, other, T, S):
+    w, wd, g = _params(T, S, other)
+    wd.mult(0.5); wd.add_mult(w, 0.001); wd.add_mult(g); w.add_mult(wd, -0.1); g.assign(1.0)     # (not a reset)
+
+
+def seq_update_l1_only_twice(cm, a, B, bias, other, T, S):
+    w, wd, g = _params(T, S, other)
+    for _ in range(2):
+        wd.mult(0.5); wd.add_mult_sign(w, 0.0005); wd.add_mult(g); w.add_mult(wd, -0.1)
+
+
+def seq_update_not_spelled_scaled_gradient(cm, a, B, bias, other, T, S):
+    w, wd, g = _params(T, S, other)
+    wd.mult(0.9); wd.add_mult(g, 0.5); w.add_mult(wd, -0.01); g.assign(0)
+
+
+def seq_update_not_spelled_wrong_order(cm, a, B, bias, other, T, S):
+    w, wd, g = _params(T, S, other)
+    wd.mult(0.9); wd.add_mult(g); wd.add_mult(w, 0.001); w.add_mult(wd, -0.01)
+
+
+def seq_update_not_spelled_no_gradient(cm, a, B, bias, other, T, S):
+    w, wd, g = _params(T, S, other)
+    wd.mult(0.9); wd.add_mult(w, 0.001); w.add_mult(wd, -0.01)
+
+
+def seq_update_interrupted(cm, a, B, bias, other, T, S):
+    w, wd, g = _params(T, S, other)
+    wd.mult(0.9); g.mult(2.0); wd.add_mult(g); w.add_mult(wd, -0.01); wd.mult(0.5); bias.mult(3.0); wd.add_mult(g)
+
+
+def seq_update_reads_another_matrix(cm, a, B, bias, other, T, S):
+    w, wd, g = _params(T, S, other)
+    wd.mult(0.9); wd.add_mult(g); w.add_mult(g, -0.01); w.add_mult(wd, -0.01)
+
+
+def seq_update_too_many_terms(cm, a, B, bias, other, T, S):
+    w, wd, g = _params(T, S, other)
+    wd.mult(0.9); wd.add_mult(w, 0.001); wd.add_mult_sign(w, 0.0005); wd.add_mult(g); wd.add_mult(g); w.add_mult(wd, -0.01)
+
+
+def seq_update_then_product(cm, a, B, bias, other, T, S):
+    w, wd, g = _params(T, S, other)
+    wd.mult(0.9); wd.add_mult(g); w.add_mult(wd, -0.01)
+    cm.dot(a, B, target=g); g.add_col_vec(bias); g.apply_sigmoid(); wd.mult(0.5); wd.add_mult(g); w.add_mult(wd, 0.3); g.assign(0)
+
+
+def seq_scale_alone_then_read(cm, a, B, bias, other, T, S):
+    T.assign(2.0); T.add(other); T.mult(0.5)
+    return T.asarray().view(np.uint32).copy()
+
+
+SEQS = [seq_update_plain, seq_update_with_reset, seq_update_l2_l1_reset, seq_update_l2_only, seq_update_l1_only_twice,
+        seq_update_not_spelled_scaled_gradient, seq_update_not_spelled_wrong_order, seq_update_not_spelled_no_gradient,
+        seq_update_interrupted, seq_update_reads_another_matrix, seq_update_too_many_terms, seq_update_then_product,
+        seq_scale_alone_then_read, seq_sigmoid, seq_sigmoid_sample, seq_relu, seq_tanh, seq_no_bias, seq_bias_only_then_read, seq_dot_alone_then_other_work,
         seq_bias_on_another_matrix, seq_two_biases, seq_bias_changes_in_between, seq_operand_changes_in_between,
         seq_sigmoid_into_another_target, seq_sample_in_place, seq_scaled_and_accumulating_products, seq_two_products_in_a_row,
         seq_free_while_held_back, seq_lower_bound_not_zero]
