@@ -31,6 +31,8 @@
 //   k_conv_up_regs     convUp with colours*k*k <= 80: filter bank in registers
 //   k_conv_patch_regs  convDown, stride 1, <= 16 colours: P = hid * W in registers,
 //                      then k_conv_down_gather(_s1) sums the entries that land on a pixel
+//   k_conv_outp_regs   convOutp with <= 64 x 80 outputs: both operands straight from global
+//                      memory into 16 x 16 x 4 matrix-core operands, no LDS tiles
 //   k_conv_outp_small  convOutp with <= 64 x 96 outputs: [row][image] LDS tiles, every
 //                      wavefront holds the whole output block
 #include "common.h"
@@ -990,6 +992,131 @@ __global__ void __launch_bounds__(256, 1) k_conv_outp_small(ConvArgs p) {
     const int v = e & 15, ji = e >> 4, jt = ji / RT, it = ji - jt * RT;
     const int q = jt * 32 + 8 * (v >> 2) + 4 * lk + (v & 3), f = it * 32 + li;
     if (q < cols && f < Fg) part[(size_t)q * Fg + f] = sum;
+  }
+}
+
+// The same gradients for at most 16*RB filters per group and 16*CB patch columns, without
+// LDS tiles: on v_mfma_f32_16x16x4_f32 a lane holds one row (a filter, or a patch column) of
+// an operand at four of sixteen reduction indices, and the reduction runs over the images,
+// along which both arrays are contiguous.  So a lane's operands of four steps are ONE 16-byte
+// load (images 4*kq .. 4*kq + 3 of a group of 16; the sum over images takes them in any
+// order, as long as both operands take them alike), a wavefront's load covers 16 rows in
+// 64-byte runs, and nothing is staged or synchronised: a wavefront owns a run of chunks
+// (module, 16 images), keeps D chunks in flight and multiplies RB x CB blocks per step.
+// Taps on the padding and chunks past the end are out-of-range loads (zeros); every trip
+// issues the same number of loads, so that the waits the compiler places count alike on
+// every path.  The four wavefronts are summed through LDS in a fixed order and every
+// workgroup leaves one partial block for k_conv_outp_finish_*.
+template <int RB, int CB, int D>
+__global__ void __launch_bounds__(256, 1) k_conv_outp_regs(ConvArgs p) {
+  constexpr unsigned FAR = 0x80000000u;  // beyond any buffer here: sizes are below 2^31 bytes
+  constexpr int PF = 16 * RB + 4;
+  __shared__ float sums[4][16 * CB * PF];
+  const int tid = threadIdx.x, lane = tid & 63, li = lane & 15, kq = lane >> 4;
+  const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int g = blockIdx.z;
+  const int N = p.N, H = p.H, Fg = p.Fg, cols = p.Cg * p.kk2;
+  __amdgpu_buffer_rsrc_t r_img = __builtin_amdgcn_make_buffer_rsrc((void*)p.img, 0, (int)p.a_bytes, 0x00020000);
+  __amdgpu_buffer_rsrc_t r_hid = __builtin_amdgcn_make_buffer_rsrc((void*)p.hid, 0, (int)p.b_bytes, 0x00020000);
+  unsigned a_voff[RB];       // hid(f, module, image) at image + N*(module + M*f)
+  const int f0 = 16 * RB * (int)blockIdx.y;         // (grid y: slices of 16*RB filters of the group)
+#pragma unroll
+  for (int i = 0; i < RB; ++i) {
+    const int f = f0 + 16 * i + li;
+    a_voff[i] = f < Fg ? ((unsigned)(g * Fg + f) * (unsigned)p.M * (unsigned)N + 4u * (unsigned)kq) * 4u : FAR;
+  }
+  unsigned b_voff[CB], b_yx[CB];   // img(colour, y0 + ky, x0 + kx, image); bit ky | bit 16 + kx of the tap
+#pragma unroll
+  for (int j = 0; j < CB; ++j) {
+    const unsigned q = 16 * j + li;
+    const unsigned c = fd_div(q, p.dkk2), r = q - c * (unsigned)p.kk2;
+    const unsigned ky = fd_div(r, p.dk), kx = r - ky * (unsigned)p.k;
+    const bool live = (int)q < cols;
+    b_voff[j] = live ? ((((unsigned)(g * p.Cg) + c) * H + ky) * H + kx) * (unsigned)N * 4u + 16u * (unsigned)kq : FAR;
+    b_yx[j] = live ? (1u << ky) | (1u << (16 + kx)) : 0xffffffffu;
+  }
+  f32x4 acc[CB][RB];
+#pragma unroll
+  for (int j = 0; j < CB; ++j)
+#pragma unroll
+    for (int i = 0; i < RB; ++i) acc[j][i] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+  const int cpm = N >> 4;                               // chunks per module
+  const int total = p.m_count * cpm;
+  const int c0 = ((int)blockIdx.x * 4 + wv) * p.slabs_per_split;
+  const int c1 = c0 + p.slabs_per_split < total ? c0 + p.slabs_per_split : total;
+  int fm = c0 / cpm, fj = c0 - fm * cpm, fc = c0;       // the next chunk to ask for: module, group of 16 images, index
+  f32x4 ra[D][RB], rb[D][CB];
+  auto fetch = [&](auto set_tag) __attribute__((always_inline)) {
+    constexpr int SET = decltype(set_tag)::value;
+    const bool valid = fc < c1;
+    const int m = p.m_begin + fm;
+    const int my = (int)fd_div((unsigned)m, p.dMx), mx = m - my * p.Mx;
+    const int y0 = my * p.s + p.pad0, x0 = mx * p.s + p.pad0;
+    const unsigned a_so = ((unsigned)m * (unsigned)N + 16u * (unsigned)fj) * 4u;
+    const unsigned gone = valid ? 0u : FAR;
+#pragma unroll
+    for (int i = 0; i < RB; ++i)
+      ra[SET][i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r_hid, (int)(a_voff[i] | gone), (int)a_so, 0));
+    const int ylo = y0 < 0 ? -y0 : 0, yhi = H - y0 < p.k ? H - y0 : p.k;
+    const int xlo = x0 < 0 ? -x0 : 0, xhi = H - x0 < p.k ? H - x0 : p.k;
+    const unsigned ym = yhi > ylo ? ((1u << yhi) - 1u) & ~((1u << ylo) - 1u) : 0u;
+    const unsigned xm = xhi > xlo ? ((1u << xhi) - 1u) & ~((1u << xlo) - 1u) : 0u;
+    const unsigned bad = valid ? ~(ym | (xm << 16)) : 0xffffffffu;
+    const unsigned b_add = (unsigned)(((y0 * H + x0) * N + 16 * fj) * 4);
+#pragma unroll
+    for (int j = 0; j < CB; ++j) {
+      const unsigned voff = (b_yx[j] & bad) ? FAR : b_voff[j] + b_add;
+      rb[SET][j] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r_img, (int)voff, 0, 0));
+    }
+    ++fc;
+    if (++fj == cpm) { fj = 0; ++fm; }
+  };
+  auto multiply = [&](auto set_tag) __attribute__((always_inline)) {
+    constexpr int SET = decltype(set_tag)::value;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int j = 0; j < CB; ++j)
+#pragma unroll
+        for (int i = 0; i < RB; ++i)
+          acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x4f32(rb[SET][j][t], ra[SET][i][t], acc[j][i], 0, 0, 0);
+  };
+  auto each_set = [&](auto&& fn) __attribute__((always_inline)) {
+    fn(std::integral_constant<int, 0>());
+    if constexpr (D > 1) fn(std::integral_constant<int, 1>());
+    if constexpr (D > 2) fn(std::integral_constant<int, 2>());
+    if constexpr (D > 3) fn(std::integral_constant<int, 3>());
+  };
+  // (the scheduling barriers keep the requests in the order of their use: the waits count on it)
+  each_set([&](auto tag) __attribute__((always_inline)) { fetch(tag); __builtin_amdgcn_sched_barrier(0); });
+  for (int c = c0; c < c1; c += D) {
+    each_set([&](auto tag) __attribute__((always_inline)) {
+      multiply(tag);               // (a chunk past the end multiplies zeros)
+      __builtin_amdgcn_sched_barrier(0);
+      fetch(tag);
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  }
+  // acc[j][i][v] of lane (li, kq): filter 16*i + li, patch column 16*j + 4*kq + v.  LDS holds the
+  // blocks as [column][filter] with a pitch of 16*RB + 4 (the four column groups of a write land
+  // on different banks), so that a wavefront then reads, adds and stores one column of a
+  // partial block as one run.
+#pragma unroll
+  for (int j = 0; j < CB; ++j)
+#pragma unroll
+    for (int i = 0; i < RB; ++i)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) sums[wv][(16 * j + 4 * kq + v) * PF + 16 * i + li] = acc[j][i][v];
+  __syncthreads();
+  float* part = p.partial + (size_t)blockIdx.x * ((size_t)p.G * Fg * cols) + (size_t)g * Fg * cols;
+  const bool f_ok = lane < 16 * RB && f0 + lane < Fg;
+  const int fl = f_ok ? lane : 0;
+#pragma unroll
+  for (int u = 0; u < 4 * CB; ++u) {
+    const int q = wv + 4 * u;
+    const float sum = (sums[0][q * PF + fl] + sums[1][q * PF + fl]) + (sums[2][q * PF + fl] + sums[3][q * PF + fl]);
+    if (f_ok && q < cols) part[(size_t)q * Fg + f0 + lane] = sum;
   }
 }
 
@@ -2169,6 +2296,29 @@ static void conv_down_impl(cudamat* hidActs, cudamat* filters, cudamat* targets,
   if (dn_launch_status()) conv_set_error(where, hipGetErrorString(hipGetLastError()));
 }
 
+// Two chunks in flight per wavefront: with three or four, more of the first requests of the whole
+// chip queue up in front of the first multiplication (measured 19.8 us against 21.3 on 128 images
+// of 32 x 32 x 3 and 64 filters of 5 x 5).
+#define OUTP_D 2
+template <int RB>
+static void launch_outp_regs_row(int cb, dim3 grid, const ConvArgs& a) {
+  switch (cb) {
+    case 1: hipLaunchKernelGGL((k_conv_outp_regs<RB, 1, OUTP_D>), grid, dim3(256), 0, dn_stream(), a); break;
+    case 2: hipLaunchKernelGGL((k_conv_outp_regs<RB, 2, OUTP_D>), grid, dim3(256), 0, dn_stream(), a); break;
+    case 3: hipLaunchKernelGGL((k_conv_outp_regs<RB, 3, OUTP_D>), grid, dim3(256), 0, dn_stream(), a); break;
+    case 4: hipLaunchKernelGGL((k_conv_outp_regs<RB, 4, OUTP_D>), grid, dim3(256), 0, dn_stream(), a); break;
+    default: hipLaunchKernelGGL((k_conv_outp_regs<RB, 5, OUTP_D>), grid, dim3(256), 0, dn_stream(), a); break;
+  }
+}
+static void launch_outp_regs(int rb, int cb, dim3 grid, const ConvArgs& a) {
+  switch (rb) {
+    case 1: launch_outp_regs_row<1>(cb, grid, a); break;
+    case 2: launch_outp_regs_row<2>(cb, grid, a); break;
+    case 3: launch_outp_regs_row<3>(cb, grid, a); break;
+    default: launch_outp_regs_row<4>(cb, grid, a); break;
+  }
+}
+
 static void conv_outp_impl(cudamat* images, cudamat* hidActs, cudamat* targets, int numModulesX, int filterSize,
                            int paddingStart, int moduleStride, int numImgColors, int numGroups, int partialSum,
                            const char* where) {
@@ -2203,9 +2353,34 @@ static void conv_outp_impl(cudamat* images, cudamat* hidActs, cudamat* targets, 
     a.m_begin = ch * partialSum; a.m_count = partialSum;
     a.chunks = batched ? chunks : 1;
     a.out = targets->data_device + (size_t)ch * cols * F;
-    const bool small = fast && !batched && a.Fg <= 64 && cols <= 96 && N % 64 == 0 &&
-                       (long long)N * numImgColors * H * H * 4 < (1ll << 31) && (long long)N * M * F * 4 < (1ll << 31);
-    if (small) {
+    const bool few = fast && !batched && a.Fg <= 64 && cols <= 96 &&
+                     (long long)N * numImgColors * H * H * 4 < (1ll << 31) && (long long)N * M * F * 4 < (1ll << 31);
+    const bool small = few && N % 64 == 0;
+    if (few && cols <= 80 && N % 16 == 0) {
+      // operands straight into registers as 16 x 16 blocks: a wavefront owns a run of (module, 16 images) chunks
+      // With an even number of filter blocks a workgroup takes half of them over twice the chunks:
+      // half as many partial blocks to write and to sum (20.7 -> 19.8 us on the shape above; a
+      // quarter of the filters per workgroup asks the vector caches for too many loads: 27 us)
+      const int total_chunks = a.m_count * (N / 16);
+      const int rb_all = (a.Fg + 15) / 16;
+      const int ys = (rb_all % 2 == 0 && total_chunks >= 8 * dn_num_cus()) ? 2 : 1;
+      const int cus = dn_num_cus() / ys;
+      int nblocks = (total_chunks + 3) / 4 < cus ? (total_chunks + 3) / 4 : cus;
+      a.slabs_per_split = (total_chunks + 4 * nblocks - 1) / (4 * nblocks);
+      nblocks = (total_chunks + 4 * a.slabs_per_split - 1) / (4 * a.slabs_per_split);
+      a.splits = nblocks;
+      a.a_bytes = (unsigned)((long long)N * numImgColors * H * H * 4);
+      a.b_bytes = (unsigned)((long long)N * M * F * 4);
+      a.partial = (float*)dn_scratch((size_t)a.splits * F * cols * sizeof(float));
+      if (!a.partial) { conv_set_error(where, "out of device memory for the split-K workspace"); return; }
+      const dim3 grid((unsigned)nblocks, (unsigned)ys, numGroups);
+      const int rb = rb_all / ys, cb = (cols + 15) / 16;
+      launch_outp_regs(rb, cb, grid, a);
+      const int total = F * cols;
+      if (a.splits >= 64) hipLaunchKernelGGL(k_conv_outp_finish_wide, dim3((total + 63) / 64), dim3(1024), 0, dn_stream(), a);
+      else if (a.splits < 16) hipLaunchKernelGGL(k_conv_outp_finish_few, dim3((total + 255) / 256), dim3(256), 0, dn_stream(), a);
+      else hipLaunchKernelGGL(k_conv_outp_finish, dim3((total + 15) / 16), dim3(256), 0, dn_stream(), a);
+    } else if (small) {
       // few filters and few patch columns: every wavefront holds the whole output block
       int nblocks = a.m_count < dn_num_cus() ? a.m_count : dn_num_cus();
       a.splits = nblocks;

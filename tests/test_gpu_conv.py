@@ -71,6 +71,12 @@ CASES = [  # N, C, H, F, k, stride, padding, groups
     (64, 6, 8, 128, 5, 1, 2, 2),     # 2 groups of 3 colours / 64 filters
     (128, 3, 6, 8, 5, 1, 4, 1),      # 8 filters, every module touches the padding
     (64, 3, 11, 40, 5, 3, 0, 1),     # 40 filters (second block of 32 a quarter used), stride 3, last module short of the edge
+    # convOutp with at most 64 x 80 outputs (operands straight into 16 x 16 x 4 blocks, a wavefront per run of (module, 16 images) chunks):
+    (48, 2, 7, 8, 3, 1, 1, 1),       # 3 chunks per module (an odd number for two register sets), 8 filters, 18 columns
+    (16, 5, 6, 56, 4, 2, 3, 1),      # exactly 80 columns, 56 filters (last block half used), stride 2, padding 3
+    (80, 3, 5, 24, 3, 1, 1, 1),      # 5 chunks per module, fewer chunks than wavefronts
+    (64, 3, 40, 32, 3, 1, 1, 1),     # enough chunks for two filter slices per module range (grid y)
+    (32, 8, 9, 96, 3, 1, 1, 2),      # 2 groups of 4 colours / 48 filters
 ]
 
 
