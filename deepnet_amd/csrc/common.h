@@ -33,8 +33,19 @@ hipStream_t dn_stream();
 void dn_flush();
 void dn_set_pending(bool on);
 void dn_set_flush_hook(void (*f)());
-bool dn_defer_dot(cudamat* mat1, cudamat* mat2, cudamat* target, float beta, float alpha, int m, int n, int k);
+bool dn_defer_dot(cudamat* mat1, cudamat* mat2, cudamat* target, float beta, float alpha, int m, int n, int k, int* err);
 bool dn_pending_sample(rnd_struct* rnd, cudamat* mat, cudamat* target, int* err);
+// Sums along the rows, y = beta*y + alpha*rowsums(M) (M is h x w, leading dimension h), may be held back too
+// and launched together (dn_row_sum_jobs), and a product into C may wait for a second one into the same C
+// (dn_gemm_pair); each with the bits of the separate launches.
+struct DnRowSumJob { const float* M; float* y; int h, w; float alpha, beta; };
+bool dn_defer_row_sum(const float* M, float* y, int h, int w, float alpha, float beta, int* err);
+bool dn_row_sum_job_ok(const float* M, int h, int w);
+int dn_row_sum_jobs(const DnRowSumJob* jobs, int n);
+int dn_gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, const float* A, int lda, const float* B, int ldb,
+            float beta, float* C, int ldc);
+int dn_gemm_pair(bool a_trans, bool b_trans, int M, int N, int K, float alpha, const float* A, int lda, const float* B, int ldb,
+                 float beta, float alpha2, const float* A2, int lda2, const float* B2, int ldb2, float* C, int ldc);
 bool dn_capturing();
 
 // Records the launch status of the kernel just queued; returns CUDA_ERROR or 0.

@@ -484,21 +484,116 @@ static int run_pending(rnd_struct* rnd, cudamat* sample) {
 }
 static int run_queue(bool reset);
 static int queued_calls();
+
+// ---- products that accumulate into their target (add_dot / subtract_dot, beta = 1) and sums along
+// the rows added to a vector (add_sums).  A contrastive-divergence step ends with
+//   W.add_dot(v, h.T, eps); W.add_dot(v', h'.T, -eps); bv.add_sums(v, 1, eps); bv.add_sums(v', 1, -eps);
+//   bh.add_sums(h, 1, eps); bh.add_sums(h', 1, -eps)
+// (cudamat/examples/rbm_cudamat.py:73-86): six launches of 2-5 us.  A product with beta = 1 waits for
+// a second product of the same shape into the same target (then both run as one launch,
+// dn_gemm_pair), and up to four row sums onto at most two vectors wait for each other
+// (dn_row_sum_jobs); each result has the bits of the separate launches, and anything else that
+// arrives launches what is held back first, in call order.
+struct PendAcc {
+  bool active;
+  cudamat a, b, t;
+  float alpha, beta;
+  int m, n, k;
+};
+static PendAcc g_acc = {};
+static DnRowSumJob g_sums[4];
+static int g_nsums = 0;
+
+static int run_acc(const cudamat* a2, const cudamat* b2, float alpha2) {
+  const PendAcc p = g_acc;
+  g_acc.active = false;
+  dn_set_pending(false);
+  const bool ta = p.a.is_trans != 0, tb = p.b.is_trans != 0;
+  if (a2)
+    return dn_gemm_pair(ta, tb, p.m, p.n, p.k, p.alpha, p.a.data_device, p.a.size[0], p.b.data_device, p.b.size[0], p.beta, alpha2,
+                        a2->data_device, a2->size[0], b2->data_device, b2->size[0], p.t.data_device, p.t.size[0]);
+  return dn_gemm(ta, tb, p.m, p.n, p.k, p.alpha, p.a.data_device, p.a.size[0], p.b.data_device, p.b.size[0], p.beta,
+                 p.t.data_device, p.t.size[0]);
+}
+static int run_sums() {
+  DnRowSumJob jobs[4];
+  const int n = g_nsums;
+  for (int i = 0; i < n; ++i) jobs[i] = g_sums[i];
+  g_nsums = 0;
+  dn_set_pending(false);
+  return dn_row_sum_jobs(jobs, n);
+}
+
 static void flush_pending() {
   if (g_pend.active) run_pending(nullptr, nullptr);
   if (queued_calls() > 0) run_queue(false);
+  if (g_acc.active) run_acc(nullptr, nullptr, 0.f);
+  if (g_nsums > 0) run_sums();
 }
 static const int g_flush_registered = (dn_set_flush_hook(flush_pending), 0);
 
-bool dn_defer_dot(cudamat* mat1, cudamat* mat2, cudamat* target, float beta, float alpha, int m, int n, int k) {
+static inline bool overlap(const float* p, long long np, const float* q, long long nq) {
+  return p < q + nq && q < p + np;
+}
+
+bool dn_defer_dot(cudamat* mat1, cudamat* mat2, cudamat* target, float beta, float alpha, int m, int n, int k, int* err) {
+  *err = 0;
   if (g_no_defer || !g_defer_enabled) return false;
-  if (alpha != 1.f || beta != 0.f || target->is_trans || m <= 1 || n <= 1 || k <= 0) return false;
+  if (target->is_trans || m <= 1 || n <= 1 || k <= 0) return false;
+  if (beta == 1.f) {
+    // the second product of a pair: same target, same shapes and transposes, operands that the first does not write
+    if (g_acc.active && target->data_device == g_acc.t.data_device && target->size[0] == g_acc.t.size[0] && m == g_acc.m &&
+        n == g_acc.n && k == g_acc.k && (mat1->is_trans != 0) == (g_acc.a.is_trans != 0) &&
+        (mat2->is_trans != 0) == (g_acc.b.is_trans != 0) &&
+        !overlap(mat1->data_device, dn_len(mat1), target->data_device, dn_len(target)) &&
+        !overlap(mat2->data_device, dn_len(mat2), target->data_device, dn_len(target))) {
+      *err = run_acc(mat1, mat2, alpha);
+      return true;
+    }
+    dn_flush();
+    if (k > 128) return false;        // (pairs run as one launch only for short reductions)
+    g_acc.active = true;
+    g_acc.a = *mat1; g_acc.b = *mat2; g_acc.t = *target;
+    g_acc.alpha = alpha; g_acc.beta = beta;
+    g_acc.m = m; g_acc.n = n; g_acc.k = k;
+    dn_set_pending(true);
+    return true;
+  }
+  if (alpha != 1.f || beta != 0.f) return false;
   dn_flush();                         // at most one product is held back
   g_pend.active = true;
   g_pend.a = *mat1; g_pend.b = *mat2; g_pend.t = *target;
   g_pend.has_bias = false;
   g_pend.act = 0;
   dn_set_pending(true);
+  return true;
+}
+
+bool dn_defer_row_sum(const float* M, float* y, int h, int w, float alpha, float beta, int* err) {
+  *err = 0;
+  if (g_no_defer || !g_defer_enabled || beta != 1.f || !dn_row_sum_job_ok(M, h, w)) return false;
+  if (overlap(M, (long long)h * w, y, h)) return false;
+  // does the call join what is queued?  At most two vectors with two sums each; no vector may share
+  // memory with another one or with a matrix that a queued sum reads (the order of the launches
+  // would matter then)
+  bool fits = g_nsums > 0;
+  const float* ys[2] = {nullptr, nullptr};
+  int cnt[2] = {0, 0}, nys = 0, mine = -1;
+  for (int i = 0; i < g_nsums && fits; ++i) {
+    const DnRowSumJob& q = g_sums[i];
+    int t = -1;
+    for (int u = 0; u < nys; ++u) if (ys[u] == q.y) t = u;
+    if (t < 0) { t = nys; ys[nys++] = q.y; }
+    ++cnt[t];
+    if (q.y == y && q.h == h) mine = t;
+    else if (overlap(q.y, q.h, y, h)) fits = false;
+    if (overlap(q.M, (long long)q.h * q.w, y, h) || overlap(M, (long long)h * w, q.y, q.h)) fits = false;
+  }
+  if (fits && (mine >= 0 ? cnt[mine] >= 2 : nys >= 2)) fits = false;
+  if (!fits) dn_flush();
+  g_sums[g_nsums++] = DnRowSumJob{M, y, h, w, alpha, beta};
+  dn_set_pending(true);
+  if (g_nsums == 4) *err = run_sums();
   return true;
 }
 

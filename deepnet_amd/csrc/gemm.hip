@@ -553,6 +553,12 @@ __device__ __forceinline__ void small_restage(float (*tile)[33], int lane, float
   __builtin_amdgcn_wave_barrier();
 }
 
+// beta*c + alpha*s as one multiplication and one fused multiply-add, spelled out so that every
+// kernel that finishes an output this way rounds alike (beta = 0 ignores c, NaN or not).
+__device__ __forceinline__ float small_axpby(float beta, float c, float alpha, float s) {
+  return __fmaf_rn(alpha, s, beta == 0.f ? 0.f : __fmul_rn(beta, c));
+}
+
 template <bool A_KC, bool B_KC, int NW>
 __global__ void __launch_bounds__(NW * 64)
 k_gemm_small(const float* __restrict__ A, int lda, const float* __restrict__ B, int ldb, float* C, int ldc, int M, int N,
@@ -644,7 +650,7 @@ k_gemm_small(const float* __restrict__ A, int lda, const float* __restrict__ B, 
     const float sum = (red[0][e] + red[1][e]) + (red[2][e] + red[3][e]);
     const int nn = blockIdx.y * 32 + 8 * (v >> 2) + 4 * lk + (v & 3);
     if (m_ok && nn < N) {
-      const float out = gemm_finish((beta == 0.f ? 0.f : beta * cprev[u]) + alpha * sum, m, epi);
+      const float out = gemm_finish(small_axpby(beta, cprev[u], alpha, sum), m, epi);
       C[(size_t)nn * ldc + m] = out;
       if (epi.sample) {
         const unsigned int i = (unsigned int)nn * ldc + m;
@@ -653,6 +659,73 @@ k_gemm_small(const float* __restrict__ A, int lda, const float* __restrict__ B, 
     }
   }
   gemm_draw_idle_streams(tid, NW * 64, epi);
+}
+
+// Two products into the same C, one after the other, in one launch:
+//   C = beta*C + alpha*op(A)*op(B);  C = C + alpha2*op(A2)*op(B2)
+// for reductions of at most 128 terms (one chunk per wavefront and product).  Each product is
+// computed, summed over the wavefronts and rounded exactly as k_gemm_small<.., 4> does it alone,
+// so the result has the bits of the two launches (the statistics of a contrastive-divergence
+// step, W += eps * v h^T; W -= eps * v' h'^T: cudamat/examples/rbm_cudamat.py:73-74, 83-84).
+template <bool A_KC, bool B_KC>
+__global__ void __launch_bounds__(256)
+k_gemm_small_pair(const float* __restrict__ A, int lda, const float* __restrict__ B, int ldb, const float* __restrict__ A2,
+                  int lda2, const float* __restrict__ B2, int ldb2, float* C, int ldc, int M, int N, int K, float alpha,
+                  float beta, float alpha2, bool a_vec, bool b_vec, bool a2_vec, bool b2_vec) {
+  constexpr int NW = 4;
+  __shared__ float red[2][NW][16 * 64];
+  constexpr int NSTAGE = (A_KC ? 1 : 0) + (B_KC ? 1 : 0);
+  __shared__ float stage[NW][NSTAGE > 0 ? NSTAGE : 1][32][33];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int li = lane & 31, lk = lane >> 5;
+  const int m = blockIdx.x * 32 + li, n = blockIdx.y * 32 + li;
+  const bool m_ok = m < M;
+  const unsigned mc = min(m, M - 1), nc = min(n, N - 1);
+  constexpr int EPL = 1024 / (NW * 64);
+  float cprev[EPL];
+#pragma unroll
+  for (int u = 0; u < EPL; ++u) {
+    const int v = (tid + u * NW * 64) >> 6;
+    const int nn = blockIdx.y * 32 + 8 * (v >> 2) + 4 * lk + (v & 3);
+    cprev[u] = (beta != 0.f && m_ok && nn < N) ? C[(size_t)nn * ldc + m] : 0.f;
+  }
+  const int k0 = wv * 32;
+  float a[2][16], b[2][16];
+  // (the same requests as k_gemm_small: row-wise for a whole chunk of a K-contiguous operand)
+  auto load = [&](const float* __restrict__ Pa, int la, bool va, const float* __restrict__ Pb, int lb, bool vb, float (&ra)[16],
+                  float (&rb)[16]) __attribute__((always_inline)) {
+    if (A_KC && k0 + 32 <= K) small_load_rows(Pa, la, blockIdx.x * 32, M - 1, k0, lane, va, ra);
+    else small_load<A_KC>(Pa, la, mc, k0, lk, K, va, ra);
+    if (B_KC && k0 + 32 <= K) small_load_rows(Pb, lb, blockIdx.y * 32, N - 1, k0, lane, vb, rb);
+    else small_load<B_KC>(Pb, lb, nc, k0, lk, K, vb, rb);
+  };
+  load(A, lda, a_vec, B, ldb, b_vec, a[0], b[0]);
+  load(A2, lda2, a2_vec, B2, ldb2, b2_vec, a[1], b[1]);
+#pragma unroll
+  for (int pr = 0; pr < 2; ++pr) {
+    f32x16 acc;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+    if (k0 < K) {                                             // wave-uniform
+      if (A_KC && k0 + 32 <= K) small_restage(stage[wv][0], lane, a[pr]);
+      if (B_KC && k0 + 32 <= K) small_restage(stage[wv][NSTAGE - 1], lane, b[pr]);
+#pragma unroll
+      for (int q = 0; q < 16; ++q) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(b[pr][q], a[pr][q], acc, 0, 0, 0);
+    }
+#pragma unroll
+    for (int v = 0; v < 16; ++v) red[pr][wv][v * 64 + lane] = acc[v];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int u = 0; u < EPL; ++u) {
+    const int e = tid + u * NW * 64;
+    const int v = e >> 6;
+    const float sum1 = (red[0][0][e] + red[0][1][e]) + (red[0][2][e] + red[0][3][e]);
+    const float sum2 = (red[1][0][e] + red[1][1][e]) + (red[1][2][e] + red[1][3][e]);
+    const int nn = blockIdx.y * 32 + 8 * (v >> 2) + 4 * lk + (v & 3);
+    if (m_ok && nn < N) C[(size_t)nn * ldc + m] = small_axpby(1.f, small_axpby(beta, cprev[u], alpha, sum1), alpha2, sum2);
+  }
 }
 
 // The same single-launch scheme on 16 x 16 output blocks (v_mfma_f32_16x16x4_f32), for products
@@ -1123,6 +1196,50 @@ static int gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, co
   return dn_launch_status();
 }
 
+// Whether gemm() would hand this product to k_gemm_small<.., 4> (the conditions of its dispatch, in its order).
+static bool gemm_goes_small4(bool a_kc, bool b_kc, int M, int N, int K, int lda, int ldb) {
+  if (M <= 0 || N <= 0 || K <= 0 || K > 128) return false;
+  const int cus = dn_num_cus();
+  const long long tiles64 = (long long)((M + 63) / 64) * ((N + 63) / 64);
+  const bool off32 = (size_t)lda * (a_kc ? M : K) < (1u << 30) && (size_t)ldb * (b_kc ? N : K) < (1u << 30);
+  const long long tiles32 = (long long)((M + 31) / 32) * ((N + 31) / 32);
+  const long long tiles16 = (long long)((M + 15) / 16) * ((N + 15) / 16);
+  const double per_1024 = tiles16 <= cus ? 4.0 : tiles32 <= cus ? 6.2 : 15.5;
+  const bool heavy = 12.0 + 1.5e-8 * (double)M * (double)N * (double)K < per_1024 * (double)K / 1024.0;
+  if (K <= BOX_K && tiles64 >= cus / 2 && tiles64 <= 2 * cus) return false;            // k_gemm_box
+  const bool kc_aliased = a_kc && b_kc && (lda % 256 == 0 || ldb % 256 == 0);
+  const bool t16_second_round = a_kc && b_kc && tiles16 > cus && K >= 1024;
+  if (tiles64 < cus && off32 && !heavy && !t16_second_round &&
+      (tiles32 * 5 <= cus * 2 || (tiles32 * 2 <= cus && !kc_aliased)))
+    return false;                                                                      // k_gemm_tile16
+  const bool mn_both = !a_kc && !b_kc;
+  return tiles32 <= 2ll * cus && !(mn_both && K >= 2048 && tiles32 > cus) && off32 && !heavy;
+}
+
+// C = beta*C + alpha*op(A)*op(B), then C = C + alpha2*op(A2)*op(B2) (the second pair of operands has the
+// first pair's shapes and transposes).  One launch with the bits of the two when both products are
+// k_gemm_small's with one chunk per wavefront; otherwise the two launches.
+int dn_gemm_pair(bool a_trans, bool b_trans, int M, int N, int K, float alpha, const float* A, int lda, const float* B, int ldb,
+                 float beta, float alpha2, const float* A2, int lda2, const float* B2, int ldb2, float* C, int ldc) {
+  const bool a_kc = a_trans, b_kc = !b_trans;
+  if (gemm_goes_small4(a_kc, b_kc, M, N, K, lda, ldb) && gemm_goes_small4(a_kc, b_kc, M, N, K, lda2, ldb2)) {
+    const bool a_vec = dn_aligned16(A) && (lda % 4 == 0), b_vec = dn_aligned16(B) && (ldb % 4 == 0);
+    const bool a2_vec = dn_aligned16(A2) && (lda2 % 4 == 0), b2_vec = dn_aligned16(B2) && (ldb2 % 4 == 0);
+    dim3 grid((M + 31) / 32, (N + 31) / 32);
+#define GEMM_PAIR(AK, BK_)                                                                                              \
+  hipLaunchKernelGGL((k_gemm_small_pair<AK, BK_>), grid, dim3(256), 0, dn_stream(), A, lda, B, ldb, A2, lda2, B2, ldb2, C, ldc, M, \
+                     N, K, alpha, beta, alpha2, a_vec, b_vec, a2_vec, b2_vec)
+    if (a_kc && b_kc) GEMM_PAIR(true, true);
+    else if (a_kc) GEMM_PAIR(true, false);
+    else if (b_kc) GEMM_PAIR(false, true);
+    else GEMM_PAIR(false, false);
+#undef GEMM_PAIR
+    return dn_launch_status();
+  }
+  if (int e = gemm(a_trans, b_trans, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc)) return e;
+  return gemm(a_trans, b_trans, M, N, K, alpha2, A2, lda2, B2, ldb2, 1.f, C, ldc);
+}
+
 // C = beta*C + alpha*op(A)*op(B) on raw column-major buffers, for the other kernels of the library.
 int dn_gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, const float* A, int lda, const float* B,
             int ldb, float beta, float* C, int ldc) {
@@ -1270,7 +1387,8 @@ int dot(cudamat* mat1, cudamat* mat2, cudamat* target, float beta, float alpha) 
   // dimension; refuse the combinations where that would write past its buffer.
   if ((long long)(n - 1) * ldc + m > dn_len(target)) return ERROR_INCOMPATIBLE_DIMENSIONS;
   // (held back when the calls that follow may ride in its epilogue)
-  if (dn_defer_dot(mat1, mat2, target, beta, alpha, m, n, k)) return 0;
+  int held = 0;
+  if (dn_defer_dot(mat1, mat2, target, beta, alpha, m, n, k, &held)) return held;
 
   // One output column: C(:,0) = op(A) * b with b = op(B)(:,0), k contiguous
   // values of B whichever way it is flagged (a k x 1 or 1 x k array).

@@ -285,6 +285,10 @@ int get_softmax_cross_entropy(cudamat* mat, cudamat* labels, cudamat* target, fl
  * mult_by_scalar is held back and the add_mult / add_mult_sign calls of a parameter update
  * (deepnet/parameter.py:80-106: w_delta *= momentum [; w_delta += l2 w] [; w_delta += l1 sign(w)] ;
  * w_delta += gradient ; w += -epsilon w_delta [; gradient = 0]) run as one pass when they spell it.
+ * A product with beta = 1 (add_dot, subtract_dot) of at most 128 terms waits for a second one of the
+ * same shape into the same target, and up to four add_sum_by_axis calls along the rows onto at most two
+ * vectors wait for each other (the statistics of cudamat/examples/rbm_cudamat.py:73-86: six calls, two
+ * launches); same bits, call order kept wherever two calls touch the same memory.
  * set_deferred_epilogues(0) makes every call launch at once; returns the previous setting (default 1). ---- */
 int set_deferred_epilogues(int on);
 

@@ -210,6 +210,135 @@ def test_same_bits_with_and_without_deferral(cm, seq, shape):
     cm.CUDAMatrix.init_random(1)
 
 
+# ---- accumulating products and row sums (the statistics of a contrastive-divergence step,
+# cudamat/examples/rbm_cudamat.py:73-86): W nv x nh, v / v2 nv x B, h / h2 nh x B, bv nv x 1, bh nh x 1
+
+STAT_SHAPES = [(784, 500, 100), (500, 784, 100), (33, 17, 5), (1024, 1024, 128), (100, 60, 128), (2048, 64, 16), (256, 512, 200),
+               (36, 40, 7), (4, 4, 2)]          # nv, nh, batch
+
+
+def stat_cd(cm, o):
+    eps = 0.01
+    o.W.add_dot(o.v, o.h.T, mult=eps); o.W.add_dot(o.v2, o.h2.T, mult=-eps)
+    o.bv.add_sums(o.v, axis=1, mult=eps); o.bv.add_sums(o.v2, axis=1, mult=-eps)
+    o.bh.add_sums(o.h, axis=1, mult=eps); o.bh.add_sums(o.h2, axis=1, mult=-eps)
+
+
+def stat_cd_subtract_dot(cm, o):
+    o.W.add_dot(o.v, o.h.T); o.W.subtract_dot(o.v2, o.h2.T)
+    o.bh.add_sums(o.h, axis=1); o.bv.add_sums(o.v, axis=1, mult=0.5); o.bh.add_sums(o.h2, axis=1, mult=-1.0); o.bv.add_sums(o.v2, axis=1, mult=-0.5)
+
+
+def stat_pair_then_read(cm, o):
+    o.W.add_dot(o.v, o.h.T, mult=0.25); o.W.add_dot(o.v2, o.h2.T, mult=-0.75)
+    return o.W.asarray().view(np.uint32).copy()
+
+
+def stat_single_then_read(cm, o):
+    o.W.add_dot(o.v, o.h.T, mult=0.25)
+    return o.W.asarray().view(np.uint32).copy()
+
+
+def stat_three_products(cm, o):
+    o.W.add_dot(o.v, o.h.T, mult=0.25); o.W.add_dot(o.v2, o.h2.T, mult=-0.75); o.W.add_dot(o.v, o.h2.T, mult=0.125)
+
+
+def stat_products_into_two_targets(cm, o):
+    o.W.add_dot(o.v, o.h.T, mult=0.25); o.W2.add_dot(o.v2, o.h2.T, mult=-0.75); o.W.add_dot(o.v2, o.h.T); o.W2.add_dot(o.v, o.h2.T)
+
+
+def stat_second_product_reads_the_target(cm, o):
+    # the visible states are overwritten by a product of the weights, then used: nothing may be reordered
+    o.W.add_dot(o.v, o.h.T, mult=0.25); cm.dot(o.W, o.h, target=o.v2); o.W.add_dot(o.v2, o.h2.T, mult=-0.75)
+
+
+def stat_overwriting_product_after_accumulating(cm, o):
+    o.W.add_dot(o.v, o.h.T, mult=0.25); cm.dot(o.v2, o.h2.T, target=o.W); o.W.add_dot(o.v, o.h2.T); o.W.add_dot(o.v2, o.h.T, mult=2.0)
+
+
+def stat_transposed_operands(cm, o):
+    # the same statistics with the roles exchanged: W2t is nh x nv
+    o.W2t.add_dot(o.h, o.v.T, mult=0.5); o.W2t.add_dot(o.h2, o.v2.T, mult=-0.5)
+
+
+def stat_three_sums_on_one_vector(cm, o):
+    o.bv.add_sums(o.v, axis=1, mult=0.5); o.bv.add_sums(o.v2, axis=1, mult=-0.25); o.bv.add_sums(o.v, axis=1, mult=2.0)
+
+
+def stat_sums_on_three_vectors(cm, o):
+    o.bv.add_sums(o.v, axis=1); o.bh.add_sums(o.h, axis=1); o.bv2.add_sums(o.v2, axis=1); o.bv.add_sums(o.v2, axis=1, mult=-1.0)
+
+
+def stat_sum_of_a_queued_result(cm, o):
+    o.bv.add_sums(o.v, axis=1, mult=0.5); o.bv2.add_sums(o.bv, axis=1); o.bv.add_sums(o.v2, axis=1)
+
+
+def stat_sum_into_a_queued_source(cm, o):
+    col = o.v.slice(0, 1)                      # the first column of v as an nv x 1 vector
+    o.bv.add_sums(o.v, axis=1, mult=0.5); col.add_sums(o.v2, axis=1); o.bv.add_sums(o.v, axis=1)
+
+
+def stat_sums_other_axis_in_between(cm, o):
+    o.bv.add_sums(o.v, axis=1, mult=0.5); o.row.add_sums(o.v, axis=0); o.bv.add_sums(o.v2, axis=1)
+
+
+def stat_sums_then_read(cm, o):
+    o.bh.add_sums(o.h, axis=1, mult=0.5); o.bh.add_sums(o.h2, axis=1, mult=-0.5)
+    return o.bh.asarray().view(np.uint32).copy()
+
+
+def stat_sum_with_assignment(cm, o):
+    o.bv.assign(0); o.bv.add_sums(o.v, axis=1); o.bh.assign(1.0); o.bh.add_sums(o.h, axis=1, mult=3.0); o.bh.mult(0.5)
+
+
+def stat_sums_of_transposed_views(cm, o):
+    o.bh.add_sums(o.hT.T, axis=1, mult=0.5); o.bh.add_sums(o.h2, axis=1, mult=-0.5)      # hT is B x nh
+
+
+STATS = [stat_cd, stat_cd_subtract_dot, stat_pair_then_read, stat_single_then_read, stat_three_products, stat_products_into_two_targets,
+         stat_second_product_reads_the_target, stat_overwriting_product_after_accumulating, stat_transposed_operands,
+         stat_three_sums_on_one_vector, stat_sums_on_three_vectors, stat_sum_of_a_queued_result, stat_sum_into_a_queued_source,
+         stat_sums_other_axis_in_between, stat_sums_then_read, stat_sum_with_assignment, stat_sums_of_transposed_views]
+
+
+class _Stat(object):
+    def __init__(self, cm, shape, seed):
+        nv, nh, B = shape
+        rng = np.random.default_rng(seed)
+        g = lambda *d: cm.CUDAMatrix(_f(rng.standard_normal(d)))
+        self.W, self.W2, self.W2t = g(nv, nh), g(nv, nh), g(nh, nv)
+        self.v, self.v2, self.h, self.h2, self.hT = g(nv, B), g(nv, B), g(nh, B), g(nh, B), g(B, nh)
+        self.bv, self.bv2, self.bh, self.row = g(nv, 1), g(nv, 1), g(nh, 1), g(1, B)
+
+    def all(self):
+        return [self.W, self.W2, self.W2t, self.v, self.v2, self.h, self.h2, self.bv, self.bv2, self.bh, self.row]
+
+
+@pytest.mark.parametrize("seq", STATS, ids=lambda f: f.__name__)
+@pytest.mark.parametrize("shape", STAT_SHAPES, ids=lambda s: "%dx%dx%d" % s)
+def test_statistics_keep_their_bits(cm, seq, shape):
+    res = []
+    for deferred in (False, True):
+        cm.set_deferred_epilogues(deferred)
+        o = _Stat(cm, shape, 11)
+        out = seq(cm, o)
+        res.append([_bits(x) for x in o.all()] + ([out] if out is not None else []))
+    cm.set_deferred_epilogues(True)
+    for i, (w, g) in enumerate(zip(*res)):
+        assert np.array_equal(g, w), "matrix %d differs" % i
+
+
+def test_statistics_are_the_float64_definition(cm):
+    o = _Stat(cm, (784, 500, 100), 12)
+    w0, bv0, bh0 = o.W.asarray().astype(np.float64), o.bv.asarray().astype(np.float64), o.bh.asarray().astype(np.float64)
+    v, v2, h, h2 = (x.asarray().astype(np.float64) for x in (o.v, o.v2, o.h, o.h2))
+    stat_cd(cm, o)
+    eps = np.float64(np.float32(0.01))
+    assert np.allclose(o.W.asarray(), w0 + eps * (v @ h.T - v2 @ h2.T), rtol=1e-5, atol=1e-5)
+    assert np.allclose(o.bv.asarray(), bv0 + eps * (v.sum(1, keepdims=True) - v2.sum(1, keepdims=True)), rtol=1e-5, atol=1e-5)
+    assert np.allclose(o.bh.asarray(), bh0 + eps * (h.sum(1, keepdims=True) - h2.sum(1, keepdims=True)), rtol=1e-5, atol=1e-5)
+
+
 def test_the_folded_sequence_is_the_float64_definition(cm, rng):
     m, k, n = 500, 784, 100
     w, x, b = _f(0.05 * rng.standard_normal((k, m))), _f(rng.random((k, n))), _f(rng.standard_normal((m, 1)))
