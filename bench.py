@@ -635,8 +635,9 @@ def main():
         secondary['mlp_784_1024_1024_10'] = {'steps_per_sec': round(1.0 / t, 1), 'us_per_step': round(t * 1e6, 1),
                                               'gemm_tflops': round(mlp.flops / t / 1e12, 3), 'batch': 128,
                                               'note': 'the 51 calls of the reference API; the library folds bias / activation calls into the '
-                                                      'launch of the dot() they follow and the mult / add_mult calls of each parameter update '
-                                                      'into one pass (same bits): 34 launches',
+                                                      'launch of the dot() they follow, the mult / add_mult calls of each parameter update '
+                                                      'into one pass and fill_with_rand / greater_than / mult of a dropout mask into one pass '
+                                                      '(same bits): 30 launches',
                                               'iters': 100, 'warmup': 10}
         cm.set_deferred_epilogues(False)
         t = time_loop(cm, mlp.step, 100, 10)

@@ -38,6 +38,10 @@ bool dn_pending_sample(rnd_struct* rnd, cudamat* mat, cudamat* target, int* err)
 // Sums along the rows, y = beta*y + alpha*rowsums(M) (M is h x w, leading dimension h), may be held back too
 // and launched together (dn_row_sum_jobs), and a product into C may wait for a second one into the same C
 // (dn_gemm_pair); each with the bits of the separate launches.
+// fill_with_rand may be held back as well: greater_than_scalar(mask, p) and mult_elementwise(state, mask)
+// that follow it spell a dropout mask (deepnet/neuralnet.py:194-198) and run as one pass (dn_rng_dropmask).
+bool dn_defer_fill_rand(rnd_struct* rnd, cudamat* mat, int* err);
+int dn_rng_dropmask(rnd_struct* rnd, float* mask, float* state, size_t n, float p);
 struct DnRowSumJob { const float* M; float* y; int h, w; float alpha, beta; };
 bool dn_defer_row_sum(const float* M, float* y, int h, int w, float alpha, float beta, int* err);
 bool dn_row_sum_job_ok(const float* M, int h, int w);

@@ -367,7 +367,6 @@ DN_SCALAR(apply_pow, check_unary, FPow)
 DN_SCALAR(less_than_eq_scalar, check_unary_trans, FLeS)
 DN_SCALAR(less_than_scalar, check_unary_trans, FLtS)
 DN_SCALAR(greater_than_eq_scalar, check_unary_trans, FGeS)
-DN_SCALAR(greater_than_scalar, check_unary_trans, FGtS)
 DN_SCALAR(upper_bound_scalar, check_unary_trans, FUpperS)
 DN_SCALAR(divide_by_scalar, check_unary, FDivS)
 DN_SCALAR(add_scalar, check_unary, FAddS)
@@ -382,7 +381,6 @@ DN_BINARY(lower_bound, check_binary, FLower{})
 DN_BINARY(add_elementwise, check_binary, FAdd{})
 DN_BINARY(subtract_elementwise, check_binary, FSub{})
 DN_BINARY(divide_elementwise, check_binary, FDiv{})
-DN_BINARY(mult_elementwise, check_binary, FMul{})
 DN_BINARY(apply_sin_deriv, check_binary, FSinDeriv{})
 DN_BINARY(apply_cos_deriv, check_binary, FCosDeriv{})
 DN_BINARY(apply_logistic_deriv, check_binary, FLogisticDeriv{})
@@ -524,11 +522,38 @@ static int run_sums() {
   return dn_row_sum_jobs(jobs, n);
 }
 
+// ---- the dropout mask: mask.fill_with_rand(); mask.greater_than(p); state.mult(mask)
+// (deepnet/neuralnet.py:194-198) as one pass over the generator's streams.
+struct PendDrop {
+  int stage;            // 0 nothing, 1 fill_with_rand held back, 2 ... and its threshold
+  rnd_struct* rnd;
+  cudamat mask;
+  float p;
+};
+static PendDrop g_drop = {};
+
+extern "C" int fill_with_rand(rnd_struct* rnd_state, cudamat* mat);
+
+static int run_drop(cudamat* state) {
+  const PendDrop d = g_drop;
+  g_drop.stage = 0;
+  dn_set_pending(false);
+  const bool saved = g_no_defer;
+  g_no_defer = true;
+  int e;
+  cudamat mask = d.mask;
+  if (d.stage == 1) e = fill_with_rand(d.rnd, &mask);
+  else e = dn_rng_dropmask(d.rnd, mask.data_device, state ? state->data_device : nullptr, (size_t)dn_len(&mask), d.p);
+  g_no_defer = saved;
+  return e;
+}
+
 static void flush_pending() {
   if (g_pend.active) run_pending(nullptr, nullptr);
   if (queued_calls() > 0) run_queue(false);
   if (g_acc.active) run_acc(nullptr, nullptr, 0.f);
   if (g_nsums > 0) run_sums();
+  if (g_drop.stage) run_drop(nullptr);
 }
 static const int g_flush_registered = (dn_set_flush_hook(flush_pending), 0);
 
@@ -568,6 +593,46 @@ bool dn_defer_dot(cudamat* mat1, cudamat* mat2, cudamat* target, float beta, flo
   dn_set_pending(true);
   return true;
 }
+
+bool dn_defer_fill_rand(rnd_struct* rnd, cudamat* mat, int* err) {
+  *err = 0;
+  if (g_no_defer || !g_defer_enabled || mat->is_trans || dn_len(mat) <= 0) return false;
+  dn_flush();
+  g_drop.stage = 1;
+  g_drop.rnd = rnd;
+  g_drop.mask = *mat;
+  g_drop.p = 0.f;
+  dn_set_pending(true);
+  return true;
+}
+static inline bool drop_mask_is(const cudamat* x) {
+  return x->on_device && !x->is_trans && x->data_device == g_drop.mask.data_device && x->size[0] == g_drop.mask.size[0] &&
+         x->size[1] == g_drop.mask.size[1];
+}
+
+extern "C" {
+
+int greater_than_scalar(cudamat* mat, float val, cudamat* target) {
+  if (g_drop.stage == 1 && !g_no_defer && drop_mask_is(mat) && drop_mask_is(target)) {
+    g_drop.stage = 2;
+    g_drop.p = val;
+    return 0;
+  }
+  if (int e = check_unary_trans(mat, target)) return e;
+  return launch_ew<1>(mat->data_device, nullptr, target->data_device, dn_len(mat), FGtS{val});
+}
+
+int mult_elementwise(cudamat* mat1, cudamat* mat2, cudamat* target) {
+  if (g_drop.stage == 2 && !g_no_defer && drop_mask_is(mat2) && mat1->on_device && !mat1->is_trans && target->on_device &&
+      !target->is_trans && target->data_device == mat1->data_device && mat1->size[0] == mat2->size[0] &&
+      mat1->size[1] == mat2->size[1] && target->size[0] == mat1->size[0] && target->size[1] == mat1->size[1] &&
+      !overlap(mat1->data_device, dn_len(mat1), mat2->data_device, dn_len(mat2)))
+    return run_drop(mat1);
+  if (int e = check_binary(mat1, mat2, target)) return e;
+  return launch_ew<2>(mat1->data_device, mat2->data_device, target->data_device, dn_len(mat1), FMul{});
+}
+
+}  // extern "C"
 
 bool dn_defer_row_sum(const float* M, float* y, int h, int w, float alpha, float beta, int* err) {
   *err = 0;

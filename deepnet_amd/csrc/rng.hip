@@ -96,6 +96,21 @@ struct OpPerturbProb {
   const float* src; float* dst;
   __device__ __forceinline__ float value(float u, float x) const { return -x / logf(u); }
 };
+// fill_with_rand -> greater_than(p) -> mult by the mask (deepnet/neuralnet.py:194-198) in one pass:
+// dst gets the mask (u > p ? 1 : 0), and where a second array is given (src, read and written in
+// place) it is multiplied by the mask.
+struct OpDropMask {
+  const float* src; float* dst;
+  float p;
+  float* state;
+  __device__ __forceinline__ float value(float u, float) const { return u > p ? 1.f : 0.f; }
+};
+// what an op stores besides dst[i] (v: the value stored there, x: what was loaded from src[i])
+template <class Op>
+__device__ __forceinline__ void rng_side(const Op&, size_t, float, float) {}
+__device__ __forceinline__ void rng_side(const OpDropMask& op, size_t i, float v, float x) {
+  if (op.state) op.state[i] = x * v;
+}
 
 // Draws [d0, d1) of one stream: element index of draw d is d * 12288 + idx.
 // STREAM: the call is large, use non-temporal accesses.
@@ -113,13 +128,17 @@ __device__ __forceinline__ unsigned long long rng_walk(unsigned long long w, uns
 #pragma unroll
     for (int k = 0; k < RNG_BATCH; ++k) {
       w = mwc_step(w, mult);
-      dn_st1_rt(op.dst + i + (size_t)k * NUM_RND_STREAMS, op.value(mwc_uniform(w), x[k]), STREAM);
+      const float v = op.value(mwc_uniform(w), x[k]);
+      dn_st1_rt(op.dst + i + (size_t)k * NUM_RND_STREAMS, v, STREAM);
+      rng_side(op, i + (size_t)k * NUM_RND_STREAMS, v, x[k]);
     }
   }
   for (; d < d1; ++d, i += NUM_RND_STREAMS) {
     const float x = op.src ? op.src[i] : 0.f;
     w = mwc_step(w, mult);
-    op.dst[i] = op.value(mwc_uniform(w), x);
+    const float v = op.value(mwc_uniform(w), x);
+    op.dst[i] = v;
+    rng_side(op, i, v, x);
   }
   return w;
 }
@@ -171,7 +190,9 @@ k_rng_split(const unsigned int* mults, const unsigned long long* words, unsigned
     if (pp & 1u) w = mwc_montmul(w, table[(size_t)(chbits + b) * NUM_RND_STREAMS + idx], mult);
   auto emit = [&](size_t at, float xv) {
     w = mwc_step(w, mult);
-    __builtin_nontemporal_store(op.value(mwc_uniform(w), xv), op.dst + at);
+    const float v = op.value(mwc_uniform(w), xv);
+    __builtin_nontemporal_store(v, op.dst + at);
+    rng_side(op, at, v, xv);
   };
   if (full0) {
     for (;;) {
@@ -445,6 +466,9 @@ static inline bool rng_ready(const rnd_struct* st) { return st && st->dev_mults 
 int fill_with_rand(rnd_struct* rnd_state, cudamat* mat) {
   if (!mat->on_device) return ERROR_NOT_ON_DEVICE;
   if (!rng_ready(rnd_state)) return ERROR_GENERIC;
+  // (held back: the threshold and the product of a dropout mask may follow)
+  int held = 0;
+  if (dn_defer_fill_rand(rnd_state, mat, &held)) return held;
   return launch_rng(rnd_state, (size_t)dn_len(mat), OpUniform{nullptr, mat->data_device});
 }
 
@@ -484,6 +508,17 @@ int sample_gaussian(rnd_struct* rnd_state, cudamat* mat, cudamat* target, float 
   if (!rng_ready(rnd_state)) return ERROR_GENERIC;
   return launch_gauss(rnd_state, mat->data_device, target->data_device, (size_t)dn_len(mat), mult);
 }
+
+}  // extern "C"
+
+// mask = (uniform draw > p) ? 1 : 0 over n elements, and state *= mask when state is given
+// (fill_with_rand, greater_than_scalar and mult_elementwise in one pass, same draws, same values).
+int dn_rng_dropmask(rnd_struct* rnd_state, float* mask, float* state, size_t n, float p) {
+  if (!rng_ready(rnd_state)) return ERROR_GENERIC;
+  return launch_rng(rnd_state, n, OpDropMask{state, mask, p, state});
+}
+
+extern "C" {
 
 int dropout(rnd_struct* rnd_state, cudamat* mat, float dropprob, float val) {
   if (!mat->on_device) return ERROR_NOT_ON_DEVICE;

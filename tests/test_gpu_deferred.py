@@ -191,7 +191,50 @@ def seq_scale_alone_then_read(cm, a, B, bias, other, T, S):
     return T.asarray().view(np.uint32).copy()
 
 
-SEQS = [seq_update_plain, seq_update_with_reset, seq_update_l2_l1_reset, seq_update_l2_only, seq_update_l1_only_twice,
+# ---- the dropout mask of deepnet/neuralnet.py:194-198 (mask = S, state = T)
+
+def seq_dropout(cm, a, B, bias, other, T, S):
+    T.add(other); S.fill_with_rand(); S.greater_than(0.5); T.mult(S)
+
+
+def seq_dropout_after_a_layer(cm, a, B, bias, other, T, S):
+    cm.dot(a, B, target=T); T.add_col_vec(bias); T.lower_bound(0); S.fill_with_rand(); S.greater_than(0.3); T.mult(S)
+    other.fill_with_rand(); other.greater_than(0.7); T.mult(other)
+
+
+def seq_dropout_mask_then_read(cm, a, B, bias, other, T, S):
+    S.fill_with_rand(); S.greater_than(0.25)
+    return S.asarray().view(np.uint32).copy()
+
+
+def seq_dropout_into_another_target(cm, a, B, bias, other, T, S):
+    T.add(other); S.fill_with_rand(); S.greater_than(0.5); T.mult(S, target=other)
+
+
+def seq_dropout_threshold_into_another_target(cm, a, B, bias, other, T, S):
+    T.add(other); S.fill_with_rand(); S.greater_than(0.5, target=other); T.mult(S)
+
+
+def seq_dropout_mask_times_itself(cm, a, B, bias, other, T, S):
+    S.fill_with_rand(); S.greater_than(0.5); S.mult(S); T.fill_with_rand(); T.mult(T)
+
+
+def seq_dropout_roles_exchanged(cm, a, B, bias, other, T, S):
+    T.add(other); S.fill_with_rand(); S.greater_than(0.5); S.mult(T)
+
+
+def seq_fill_then_other_work(cm, a, B, bias, other, T, S):
+    S.fill_with_rand(); T.add(S); S.greater_than(0.5); T.mult(S)
+
+
+def seq_dropout_of_special_values(cm, a, B, bias, other, T, S):
+    T.assign(-0.0); other.assign(float('inf')); T.add_mult(other, -1.0)        # -inf everywhere: times a zero of the mask is NaN
+    S.fill_with_rand(); S.greater_than(0.5); T.mult(S)
+
+
+SEQS = [seq_dropout, seq_dropout_after_a_layer, seq_dropout_mask_then_read, seq_dropout_into_another_target,
+        seq_dropout_threshold_into_another_target, seq_dropout_mask_times_itself, seq_dropout_roles_exchanged,
+        seq_fill_then_other_work, seq_dropout_of_special_values, seq_update_plain, seq_update_with_reset, seq_update_l2_l1_reset, seq_update_l2_only, seq_update_l1_only_twice,
         seq_update_not_spelled_scaled_gradient, seq_update_not_spelled_wrong_order, seq_update_not_spelled_no_gradient,
         seq_update_interrupted, seq_update_reads_another_matrix, seq_update_too_many_terms, seq_update_then_product,
         seq_scale_alone_then_read, seq_sigmoid, seq_sigmoid_sample, seq_relu, seq_tanh, seq_no_bias, seq_bias_only_then_read, seq_dot_alone_then_other_work,
