@@ -172,8 +172,9 @@ class MLP(object):
         self.b = [f(np.zeros((sizes[i + 1], 1))) for i in range(3)]
         self.dW = [f(np.zeros((sizes[i], sizes[i + 1]))) for i in range(3)]
         self.db = [f(np.zeros((sizes[i + 1], 1))) for i in range(3)]
-        self.gW = [cm.empty((sizes[i], sizes[i + 1])) for i in range(3)]
-        self.gb = [cm.empty((sizes[i + 1], 1)) for i in range(3)]
+        # gradients accumulate and Update() leaves them at zero (neuralnet.py:269, 284, parameter.py:105)
+        self.gW = [f(np.zeros((sizes[i], sizes[i + 1]))) for i in range(3)]
+        self.gb = [f(np.zeros((sizes[i + 1], 1))) for i in range(3)]
         self.act = [self.x] + [cm.empty((sizes[i + 1], B)) for i in range(3)]
         self.mask = [cm.empty((sizes[i + 1], B)) for i in range(2)]
         self.delta = [cm.empty((sizes[i + 1], B)) for i in range(3)]
@@ -195,17 +196,17 @@ class MLP(object):
         act[3].get_softmax_cross_entropy(self.labels, self.loss)
         act[3].apply_softmax_grad(self.labels, target=self.delta[2])
         for i in (2, 1, 0):
-            self.gW[i].assign(0); self.gW[i].add_dot(act[i], self.delta[i].T, mult=1.0 / B)
-            self.gb[i].assign(0); self.gb[i].add_sums(self.delta[i], axis=1, mult=1.0 / B)
+            self.gW[i].add_dot(act[i], self.delta[i].T, mult=1.0 / B)
+            self.gb[i].add_sums(self.delta[i], axis=1, mult=1.0 / B)
             if i > 0:
                 cm.dot(W[i], self.delta[i], target=self.delta[i - 1])
                 self.delta[i - 1].apply_rectified_linear_deriv(act[i])
         for i in range(3):
             for p, d, g in ((W[i], self.dW[i], self.gW[i]), (b[i], self.db[i], self.gb[i])):
-                d.mult(self.mom); d.add_mult(g); p.add_mult(d, -self.lr)
+                d.mult(self.mom); d.add_mult(g); p.add_mult(d, -self.lr); g.assign(0)
 
     def step_fused(self):
-        """The same step in 17 launches instead of 51: this backend's extensions dot_bias_act,
+        """The same step in 17 launches instead of 51 calls: this backend's extensions dot_bias_act,
         softmax_ce_grad and momentum_update (all six parameters in one launch), and the one-call forms that the reference's own
         API has for what deepnet spells out in several (dropout() for fill_with_rand ->
         greater_than -> mult, dot() into the gradient for assign(0) -> add_dot, dot() with a
@@ -231,7 +232,7 @@ class MLP(object):
         if self.updates is None:
             self.updates = cm.MomentumUpdates([(W[i], self.dW[i], self.gW[i]) for i in range(3)] +
                                               [(b[i], self.db[i], self.gb[i]) for i in range(3)])
-        self.updates.apply(self.mom, self.lr, reset_gradient=False)
+        self.updates.apply(self.mom, self.lr, reset_gradient=True)
 
 
 def net_mlp(cm, sizes=(784, 1024, 1024, 10), B=128, seed=3, fused=False):
@@ -637,7 +638,7 @@ def main():
                                               'note': 'the 51 calls of the reference API; the library folds bias / activation calls into the '
                                                       'launch of the dot() they follow, the mult / add_mult calls of each parameter update '
                                                       'into one pass and fill_with_rand / greater_than / mult of a dropout mask into one pass '
-                                                      '(same bits): 30 launches',
+                                                      '(same bits): 24 launches',
                                               'iters': 100, 'warmup': 10}
         cm.set_deferred_epilogues(False)
         t = time_loop(cm, mlp.step, 100, 10)

@@ -314,9 +314,9 @@ void hb_mlp_step(int nl, const int* sizes, int B, float lr, float mom, float** W
   const float invB = 1.f / (float)B;
   for (int i = nl - 1; i >= 0; --i) {
     const int in = sizes[i], out = sizes[i + 1];
-    memset(gW[i], 0, sizeof(float) * (size_t)in * out);
+    /* gradients accumulate (neuralnet.py:269, 284); Update() leaves them at zero (parameter.py:105) */
     hb_gemm(0, 1, in, out, B, invB, act[i], in, delta[i], out, 1.f, gW[i], in);
-    hb_add_sums(delta[i], gb[i], out, B, 1, 0.f, invB);
+    hb_add_sums(delta[i], gb[i], out, B, 1, 1.f, invB);
     if (i > 0) {
       hb_gemm(0, 0, in, B, out, 1.f, W[i], in, delta[i], out, 0.f, delta[i - 1], in);
       hb_relu_deriv(delta[i - 1], act[i], delta[i - 1], (size_t)in * B);
@@ -326,5 +326,7 @@ void hb_mlp_step(int nl, const int* sizes, int B, float lr, float mom, float** W
     const size_t nw = (size_t)sizes[i] * sizes[i + 1], nb = (size_t)sizes[i + 1];
     hb_mult_scalar(dW[i], mom, dW[i], nw); hb_add_mult(dW[i], gW[i], 1.f, nw); hb_add_mult(W[i], dW[i], -lr, nw);
     hb_mult_scalar(db[i], mom, db[i], nb); hb_add_mult(db[i], gb[i], 1.f, nb); hb_add_mult(b[i], db[i], -lr, nb);
+    memset(gW[i], 0, sizeof(float) * nw);
+    memset(gb[i], 0, sizeof(float) * nb);
   }
 }
