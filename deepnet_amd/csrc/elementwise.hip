@@ -466,6 +466,8 @@ static DnPending g_pend = {};
 static bool g_no_defer = false;      // the library is issuing the calls of a sequence itself
 static bool g_defer_enabled = true;
 
+static void refresh_pending();      // tells the library whether anything is still held back
+
 static int dot_bias_act_impl(rnd_struct* rnd, cudamat* mat1, cudamat* mat2, cudamat* bias, cudamat* target,
                              cudamat* sample, int act);
 
@@ -473,7 +475,7 @@ static int dot_bias_act_impl(rnd_struct* rnd, cudamat* mat1, cudamat* mat2, cuda
 static int run_pending(rnd_struct* rnd, cudamat* sample) {
   DnPending p = g_pend;
   g_pend.active = false;
-  dn_set_pending(false);
+  refresh_pending();
   const bool saved = g_no_defer;
   g_no_defer = true;
   const int e = dot_bias_act_impl(rnd, &p.a, &p.b, p.has_bias ? &p.bias : nullptr, &p.t, sample, p.act);
@@ -482,6 +484,10 @@ static int run_pending(rnd_struct* rnd, cudamat* sample) {
 }
 static int run_queue(bool reset);
 static int queued_calls();
+static int run_batch();
+static int stash_ready(bool reset);
+static bool update_ready();
+static int batched_updates();
 
 // ---- products that accumulate into their target (add_dot / subtract_dot, beta = 1) and sums along
 // the rows added to a vector (add_sums).  A contrastive-divergence step ends with
@@ -505,7 +511,7 @@ static int g_nsums = 0;
 static int run_acc(const cudamat* a2, const cudamat* b2, float alpha2) {
   const PendAcc p = g_acc;
   g_acc.active = false;
-  dn_set_pending(false);
+  refresh_pending();
   const bool ta = p.a.is_trans != 0, tb = p.b.is_trans != 0;
   if (a2)
     return dn_gemm_pair(ta, tb, p.m, p.n, p.k, p.alpha, p.a.data_device, p.a.size[0], p.b.data_device, p.b.size[0], p.beta, alpha2,
@@ -518,7 +524,7 @@ static int run_sums() {
   const int n = g_nsums;
   for (int i = 0; i < n; ++i) jobs[i] = g_sums[i];
   g_nsums = 0;
-  dn_set_pending(false);
+  refresh_pending();
   return dn_row_sum_jobs(jobs, n);
 }
 
@@ -537,7 +543,7 @@ extern "C" int fill_with_rand(rnd_struct* rnd_state, cudamat* mat);
 static int run_drop(cudamat* state) {
   const PendDrop d = g_drop;
   g_drop.stage = 0;
-  dn_set_pending(false);
+  refresh_pending();
   const bool saved = g_no_defer;
   g_no_defer = true;
   int e;
@@ -548,12 +554,21 @@ static int run_drop(cudamat* state) {
   return e;
 }
 
+static bool g_flushing = false;
 static void flush_pending() {
+  // (the launches below come back here through dn_stream(): what is still held back is launched by this
+  // call, in order, not by theirs)
+  if (g_flushing) return;
+  g_flushing = true;
+  if (update_ready()) stash_ready(false);          // (a complete update joins the ones that wait)
+  if (batched_updates() > 0) run_batch();          // older than anything else that is held back
   if (g_pend.active) run_pending(nullptr, nullptr);
   if (queued_calls() > 0) run_queue(false);
   if (g_acc.active) run_acc(nullptr, nullptr, 0.f);
   if (g_nsums > 0) run_sums();
   if (g_drop.stage) run_drop(nullptr);
+  g_flushing = false;
+  refresh_pending();
 }
 static const int g_flush_registered = (dn_set_flush_hook(flush_pending), 0);
 
@@ -753,6 +768,79 @@ static int queued_calls() { return g_eqn; }
 extern "C" int momentum_update(cudamat* w, cudamat* w_delta, cudamat* gradient, float momentum, float l2_decay,
                                float l1_decay, float epsilon, int flags);
 
+// Updates that are complete wait for each other: deepnet updates all parameters of a net one after the
+// other (neuralnet.py:300-312), and up to MOM_MANY of them run as one launch (k_momentum_update_many, the
+// arithmetic of the single update).  An update that touches an array of one that waits launches those first.
+#define UPD_BATCH 8
+struct UpdSpec {
+  cudamat w, wd, g;
+  float mom, l2, l1, eps;
+  int flags;
+};
+static UpdSpec g_ub[UPD_BATCH];
+static int g_ubn = 0;
+
+static bool update_ready() { return g_eqn > 0 && g_eq_ready; }
+static int batched_updates() { return g_ubn; }
+static void refresh_pending() {
+  dn_set_pending(g_pend.active || g_eqn > 0 || g_ubn > 0 || g_acc.active || g_nsums > 0 || g_drop.stage != 0);
+}
+
+extern "C" int momentum_update_many(int count, cudamat** w, cudamat** w_delta, cudamat** gradient, const float* momentum,
+                                    const float* l2_decay, const float* l1_decay, const float* epsilon, const int* flags);
+
+static int run_batch() {
+  UpdSpec u[UPD_BATCH];
+  const int n = g_ubn;
+  for (int i = 0; i < n; ++i) u[i] = g_ub[i];
+  g_ubn = 0;
+  refresh_pending();
+  const bool saved = g_no_defer;
+  g_no_defer = true;
+  int e = 0;
+  if (n == 1) {
+    e = momentum_update(&u[0].w, &u[0].wd, &u[0].g, u[0].mom, u[0].l2, u[0].l1, u[0].eps, u[0].flags);
+  } else if (n > 1) {
+    cudamat *w[UPD_BATCH], *wd[UPD_BATCH], *g[UPD_BATCH];
+    float mom[UPD_BATCH], l2[UPD_BATCH], l1[UPD_BATCH], eps[UPD_BATCH];
+    int flags[UPD_BATCH];
+    for (int i = 0; i < n; ++i) {
+      w[i] = &u[i].w; wd[i] = &u[i].wd; g[i] = &u[i].g;
+      mom[i] = u[i].mom; l2[i] = u[i].l2; l1[i] = u[i].l1; eps[i] = u[i].eps; flags[i] = u[i].flags;
+    }
+    e = momentum_update_many(n, w, wd, g, mom, l2, l1, eps, flags);
+  }
+  g_no_defer = saved;
+  return e;
+}
+
+static inline bool mats_overlap(const cudamat* a, const cudamat* b) {
+  return overlap(a->data_device, dn_len(a), b->data_device, dn_len(b));
+}
+
+// The queue spells an update and nothing more belongs to it: it joins the updates that wait.
+static int stash_ready(bool reset) {
+  UpdSpec u;
+  u.w = g_up.w; u.wd = g_eq[0].dst; u.g = g_up.g;
+  u.mom = g_eq[0].s; u.l2 = g_up.l2; u.l1 = g_up.l1; u.eps = g_up.eps;
+  u.flags = g_up.flags | (reset ? 4 : 0);
+  g_eqn = 0;
+  g_eq_ready = false;
+  bool alone = g_ubn == UPD_BATCH;
+  for (int i = 0; i < g_ubn && !alone; ++i) {
+    const cudamat* mine[3] = {&u.w, &u.wd, &u.g};
+    const cudamat* theirs[3] = {&g_ub[i].w, &g_ub[i].wd, &g_ub[i].g};
+    for (int a = 0; a < 3; ++a)
+      for (int b = 0; b < 3; ++b)
+        if (mats_overlap(mine[a], theirs[b])) alone = true;
+  }
+  int e = 0;
+  if (alone) e = run_batch();
+  g_ub[g_ubn++] = u;
+  dn_set_pending(true);
+  return e;
+}
+
 // Launches what the queue holds: the one-pass update if it spells one, else its calls one by one.
 static int run_queue(bool reset) {
   EqOp q[4];
@@ -761,7 +849,7 @@ static int run_queue(bool reset) {
   const bool ready = g_eq_ready;
   g_eqn = 0;
   g_eq_ready = false;
-  dn_set_pending(false);
+  refresh_pending();
   const bool saved = g_no_defer;
   g_no_defer = true;
   int e = 0;
@@ -800,7 +888,11 @@ extern "C" {
 int mult_by_scalar(cudamat* mat, float val, cudamat* target) {
   if (int e = check_unary(mat, target)) return e;
   if (!g_no_defer && g_defer_enabled && mat->data_device == target->data_device && dn_len(mat) > 0) {
-    dn_flush();
+    // (a complete update before this one waits on; anything else that is held back is launched now)
+    int e = 0;
+    if (update_ready()) e = stash_ready(false);
+    if (g_pend.active || g_eqn > 0 || g_acc.active || g_nsums > 0 || g_drop.stage != 0) dn_flush();
+    if (e) return e;
     g_eq[0].kind = EQ_MULS; g_eq[0].dst = *mat; g_eq[0].src = *mat; g_eq[0].s = val;
     g_eqn = 1;
     g_eq_ready = false;
@@ -812,7 +904,7 @@ int mult_by_scalar(cudamat* mat, float val, cudamat* target) {
 
 int assign_scalar(cudamat* mat, float alpha) {
   if (!mat->on_device) return ERROR_NOT_ON_DEVICE;
-  if (eq_open() && g_eq_ready && alpha == 0.f && !signbit(alpha) && same_mat(mat, &g_up.g)) return run_queue(true);
+  if (eq_open() && g_eq_ready && alpha == 0.f && !signbit(alpha) && same_mat(mat, &g_up.g)) return stash_ready(true);
   return launch_ew<0>(nullptr, nullptr, mat->data_device, dn_len(mat), FAssignS{alpha});
 }
 

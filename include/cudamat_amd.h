@@ -284,7 +284,8 @@ int get_softmax_cross_entropy(cudamat* mat, cudamat* labels, cudamat* target, fl
  * call order and results are those of the separate launches, bit for bit.  Likewise an in-place
  * mult_by_scalar is held back and the add_mult / add_mult_sign calls of a parameter update
  * (deepnet/parameter.py:80-106: w_delta *= momentum [; w_delta += l2 w] [; w_delta += l1 sign(w)] ;
- * w_delta += gradient ; w += -epsilon w_delta [; gradient = 0]) run as one pass when they spell it.
+ * w_delta += gradient ; w += -epsilon w_delta [; gradient = 0]) run as one pass when they spell it, and
+ * updates that follow each other directly (up to eight, on arrays that do not overlap) as one launch.
  * A product with beta = 1 (add_dot, subtract_dot) of at most 128 terms waits for a second one of the
  * same shape into the same target, and up to four add_sum_by_axis calls along the rows onto at most two
  * vectors wait for each other (the statistics of cudamat/examples/rbm_cudamat.py:73-86: six calls, two

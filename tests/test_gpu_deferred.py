@@ -382,6 +382,90 @@ def test_statistics_are_the_float64_definition(cm):
     assert np.allclose(o.bh.asarray(), bh0 + eps * (h.sum(1, keepdims=True) - h2.sum(1, keepdims=True)), rtol=1e-5, atol=1e-5)
 
 
+# ---- consecutive parameter updates (deepnet updates every edge and layer of a net in turn, neuralnet.py:300-312)
+
+def _upd(p, d, g, mom=0.9, lr=0.01, l2=None, l1=None, reset=True):
+    d.mult(mom)
+    if l2 is not None:
+        d.add_mult(p, l2)
+    if l1 is not None:
+        d.add_mult_sign(p, l1)
+    d.add_mult(g); p.add_mult(d, -lr)
+    if reset:
+        g.assign(0)
+
+
+def upd_six_in_a_row(cm, P):
+    for i in range(6):
+        _upd(*P[i])
+
+
+def upd_without_resets(cm, P):
+    for i in range(4):
+        _upd(*P[i], reset=False)
+
+
+def upd_mixed_decays_and_resets(cm, P):
+    _upd(*P[0], l2=0.001); _upd(*P[1], reset=False); _upd(*P[2], l1=0.002, l2=0.0005); _upd(*P[3], mom=0.5, lr=0.1, l1=0.01)
+
+
+def upd_eleven(cm, P):
+    for i in range(11):
+        _upd(*P[i % 6], mom=0.9 - 0.05 * i)              # more than one launch holds; the same parameter again: in order
+
+
+def upd_tied(cm, P):
+    # the second update reads what the first wrote, the third writes what the second read (both are 1024 x 1)
+    _upd(*P[1]); _upd(P[3][0], P[3][1], P[1][0], reset=False); _upd(P[1][0], P[1][1], P[3][2])
+
+
+def upd_gradient_is_another_delta(cm, P):
+    _upd(*P[0]); _upd(P[1][0], P[1][1], P[1][2]); _upd(P[0][0], P[0][2], P[0][1])     # roles exchanged on the same arrays
+
+
+def upd_then_scale_that_is_no_update(cm, P):
+    _upd(*P[0]); _upd(*P[1]); P[2][0].mult(0.5); P[2][0].add_mult(P[2][2], 2.0); P[2][1].add(P[2][0])
+
+
+def upd_then_read(cm, P):
+    _upd(*P[0]); _upd(*P[1], reset=False)
+    return P[1][0].asarray().view(np.uint32).copy()
+
+
+def upd_interleaved_with_a_product(cm, P):
+    _upd(*P[0]); cm.dot(P[0][0], P[0][0].T, target=P[6]); _upd(*P[1]); _upd(*P[2])
+
+
+def upd_reset_of_another_gradient(cm, P):
+    P[0][1].mult(0.9); P[0][1].add_mult(P[0][2]); P[0][0].add_mult(P[0][1], -0.01); P[1][2].assign(0); _upd(*P[1])
+
+
+UPDS = [upd_six_in_a_row, upd_without_resets, upd_mixed_decays_and_resets, upd_eleven, upd_tied, upd_gradient_is_another_delta,
+        upd_then_scale_that_is_no_update, upd_then_read, upd_interleaved_with_a_product, upd_reset_of_another_gradient]
+
+
+def _params_of_a_net(cm, seed):
+    rng = np.random.default_rng(seed)
+    g = lambda *d: cm.CUDAMatrix(_f(rng.standard_normal(d)))
+    shapes = [(784, 1024), (1024, 1), (1024, 1024), (1024, 1), (37, 10), (10, 1)]
+    P = [(g(*sh), g(*sh), g(*sh)) for sh in shapes]
+    P.append(cm.empty((784, 784)))
+    return P
+
+
+@pytest.mark.parametrize("seq", UPDS, ids=lambda f: f.__name__)
+def test_consecutive_updates_keep_their_bits(cm, seq):
+    res = []
+    for deferred in (False, True):
+        cm.set_deferred_epilogues(deferred)
+        P = _params_of_a_net(cm, 21)
+        out = seq(cm, P)
+        res.append([_bits(x) for t in P[:6] for x in t] + [_bits(P[6])] + ([out] if out is not None else []))
+    cm.set_deferred_epilogues(True)
+    for i, (w, g) in enumerate(zip(*res)):
+        assert np.array_equal(g, w), "matrix %d differs" % i
+
+
 def test_the_folded_sequence_is_the_float64_definition(cm, rng):
     m, k, n = 500, 784, 100
     w, x, b = _f(0.05 * rng.standard_normal((k, m))), _f(rng.random((k, n))), _f(rng.standard_normal((m, 1)))
