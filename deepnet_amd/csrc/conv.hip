@@ -1452,7 +1452,7 @@ __global__ void __launch_bounds__(64 * NWV, 1) k_conv_down_px(ConvArgs p) {
   constexpr int T = 4, HR = K + T - 1, KK = K * K, NA = HR * HR, NT = 64 * NWV;
   constexpr int CS = KK * FSC + 8;          // floats between the colours' weight blocks: their banks differ by 8
   constexpr int WSZ = 5 * CS;               // four colours and a block of zeros (lanes of the pad colours)
-  constexpr int RED = NWV * 64 * 64;        // the final sum reuses the weights' memory
+  constexpr int RED = NWV * (T * T * 2) * 64;   // the final sum reuses the weights' memory
   constexpr unsigned FAR_V = 0x40000000u, FAR_S = 0x20000000u;   // either one is beyond the buffer, and so is their sum
   __shared__ float lds[WSZ > RED ? WSZ : RED];
   const int tid = threadIdx.x, lane = tid & 63, par = lane >> 5, li = lane & 31, c = lane & 3;
@@ -1569,24 +1569,26 @@ __global__ void __launch_bounds__(64 * NWV, 1) k_conv_down_px(ConvArgs p) {
   }
 #undef DOWN_PX_STEP
 
-  // the parts of the filters and the two parities meet in LDS: red[wavefront][register][lane]
+  // The two filter parities (lanes l and l + 32) are added inside the wavefront: v_permlane32_swap
+  // on two accumulator registers leaves, in lanes 0-31, both parities of the first and, in lanes
+  // 32-63, both parities of the second, so one addition finishes two registers.  The parts of the
+  // filters (the wavefronts) then meet in LDS in a fixed order: red[wavefront][register pair][lane].
   __syncthreads();
 #pragma unroll
-  for (int i = 0; i < T * T; ++i)
-#pragma unroll
-    for (int v = 0; v < 4; ++v) {
-      const float val = acc[i][v];   // (through a scalar: a cast applied to the vector element itself reads element 0)
-      lds[(wq * 64 + i * 4 + v) * 64 + lane] = val;
-    }
+  for (int j = 0; j < T * T * 2; ++j) {
+    const float r0 = acc[j >> 1][(j & 1) * 2], r1 = acc[j >> 1][(j & 1) * 2 + 1];   // registers 2j and 2j + 1 of the tile
+    const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(r0), __float_as_uint(r1), false, false);
+    lds[(wq * (T * T * 2) + j) * 64 + lane] = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
+  }
   __syncthreads();
   const int outs = T * T * p.Cg * 32;
   for (int o = tid; o < outs; o += NT) {
     const int img = o & 31, rest = o >> 5;
     const int pix = rest / p.Cg, cc = rest - pix * p.Cg;
-    const int reg = pix * 4 + (img & 3), ln = 4 * (img >> 2) + cc;
+    const int reg = pix * 4 + (img & 3), ln = 4 * (img >> 2) + cc + 32 * (reg & 1);
     float s = 0.f;
 #pragma unroll
-    for (int w = 0; w < NWV; ++w) s += lds[(w * 64 + reg) * 64 + ln] + lds[(w * 64 + reg) * 64 + 32 + ln];
+    for (int w = 0; w < NWV; ++w) s += lds[(w * (T * T * 2) + (reg >> 1)) * 64 + ln];
     const int y = y0 + pix / T, x = x0 + pix % T;
     if (y < p.H && x < p.H) {
       float* t = p.out + ((size_t)(g * p.Cg + cc) * p.HH + (size_t)(y * p.H + x)) * p.N + nb * 32 + img;
