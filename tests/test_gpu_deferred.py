@@ -497,3 +497,68 @@ def test_the_switch_reports_its_previous_setting(cm):
     assert cm.set_deferred_epilogues(False) is True
     assert cm.set_deferred_epilogues(True) is False
     assert cm.set_deferred_epilogues(True) is True
+
+
+# ---- random call sequences: whatever is held back, every matrix ends with the bits of the separate launches
+
+def _random_sequence(cm, rng_ops, pool, vecs, rows, n_ops):
+    """n_ops library calls on randomly chosen matrices of one shape family (m x n matrices, m x 1 and
+    1 x n vectors, a k x m and a k x n operand pair per product): the operand choice includes every
+    kind of aliasing the calls accept."""
+    M = lambda: pool[rng_ops.integers(len(pool))]
+    V = lambda: vecs[rng_ops.integers(len(vecs))]
+    scal = lambda: float(np.float32(rng_ops.choice([0.0, 1.0, -1.0, 0.5, 0.9, -0.01, 2.0, 0.3])))
+    reads = []
+    for _ in range(n_ops):
+        op = rng_ops.integers(22)
+        a, b, c = M(), M(), M()
+        if op == 0: cm.dot(pool.A.T, pool.B, target=a)
+        elif op == 1: a.add_dot(pool.A.T, pool.B, mult=scal())
+        elif op == 2: a.add_dot(pool.A2.T, pool.B2, mult=scal())
+        elif op == 3: a.subtract_dot(pool.A.T, pool.B2)
+        elif op == 4: a.add_col_vec(V())
+        elif op == 5: a.apply_sigmoid()
+        elif op == 6: a.lower_bound(0)
+        elif op == 7: a.sample_bernoulli(target=b)
+        elif op == 8: a.mult(scal())
+        elif op == 9: a.add_mult(b, scal())
+        elif op == 10: a.add_mult_sign(b, scal())
+        elif op == 11: a.assign(scal())
+        elif op == 12: a.fill_with_rand()
+        elif op == 13: a.greater_than(scal())
+        elif op == 14: a.mult(b)
+        elif op == 15: V().add_sums(a, axis=1, mult=scal())
+        elif op == 16: rows[rng_ops.integers(len(rows))].add_sums(a, axis=0, mult=scal())
+        elif op == 17: a.add(b, target=c)
+        elif op == 18: cm.tanh(a)
+        elif op == 19: reads.append(_bits(a))
+        elif op == 20: a.add_mult(b)               # factor 1: the gradient of an update
+        else: V().add_sums(a, axis=1)
+    return reads
+
+
+class _Pool(list):
+    pass
+
+
+@pytest.mark.parametrize("shape", [(500, 100, 784), (64, 128, 96), (33, 7, 20), (1024, 128, 128)], ids=lambda s: "%dx%dx%d" % s)
+@pytest.mark.parametrize("seed", range(12))
+def test_random_sequences_keep_their_bits(cm, shape, seed):
+    m, n, k = shape
+    res = []
+    for deferred in (False, True):
+        cm.set_deferred_epilogues(deferred)
+        cm.CUDAMatrix.init_random(3 + seed)
+        rng = np.random.default_rng(100 + seed)
+        g = lambda *d: cm.CUDAMatrix(_f(rng.standard_normal(d) * 0.5))
+        pool = _Pool(g(m, n) for _ in range(4))
+        pool.A, pool.A2, pool.B, pool.B2 = g(k, m), g(k, m), g(k, n), g(k, n)
+        vecs, rows = [g(m, 1) for _ in range(2)], [g(1, n) for _ in range(2)]
+        reads = _random_sequence(cm, np.random.default_rng(1000 + seed), pool, vecs, rows, 60)
+        after = cm.empty((64, 48)); after.fill_with_rand()
+        res.append([_bits(x) for x in list(pool) + vecs + rows + [after]] + reads)
+    cm.set_deferred_epilogues(True)
+    cm.CUDAMatrix.init_random(1)
+    assert len(res[0]) == len(res[1])
+    for i, (w, gt) in enumerate(zip(*res)):
+        assert np.array_equal(gt, w), "result %d differs" % i
