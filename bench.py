@@ -607,8 +607,8 @@ def main():
                                 'config': '784 visible x 500 hidden, batch 100, fp32',
                                 'note': 'the 16 calls of the reference API (cudamat/examples/rbm_cudamat.py:46-89); the library '
                                         'folds add_col_vec / apply_sigmoid / sample_bernoulli into the launch of the dot() they '
-                                        'follow, the two add_dot calls into one launch and the four add_sums calls into another '
-                                        '(deferred epilogues, same bits): 5 launches',
+                                        'follow, and the two add_dot and four add_sums calls of the statistics into one launch '
+                                        '(deferred epilogues, same bits): 4 launches',
                                 'iters': 200, 'warmup': 20}
         cm.set_deferred_epilogues(False)
         t = time_loop(cm, rbm.step, 200, 20)

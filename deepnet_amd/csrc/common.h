@@ -48,6 +48,9 @@ bool dn_row_sum_job_ok(const float* M, int h, int w);
 int dn_row_sum_jobs(const DnRowSumJob* jobs, int n);
 int dn_gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, const float* A, int lda, const float* B, int ldb,
             float beta, float* C, int ldc);
+int dn_gemm_pair_sums(bool a_trans, bool b_trans, int M, int N, int K, float alpha, const float* A, int lda, const float* B,
+                      int ldb, float beta, float alpha2, const float* A2, int lda2, const float* B2, int ldb2, float* C, int ldc,
+                      const DnRowSumJob* jobs, int njobs);
 int dn_gemm_pair(bool a_trans, bool b_trans, int M, int N, int K, float alpha, const float* A, int lda, const float* B, int ldb,
                  float beta, float alpha2, const float* A2, int lda2, const float* B2, int ldb2, float* C, int ldc);
 bool dn_capturing();

@@ -500,32 +500,34 @@ static int batched_updates();
 // arrives launches what is held back first, in call order.
 struct PendAcc {
   bool active;
-  cudamat a, b, t;
-  float alpha, beta;
+  bool paired;          // the second product has arrived: the pair waits for the sums that may follow
+  cudamat a, b, t, a2, b2;
+  float alpha, beta, alpha2;
   int m, n, k;
 };
 static PendAcc g_acc = {};
 static DnRowSumJob g_sums[4];
 static int g_nsums = 0;
 
-static int run_acc(const cudamat* a2, const cudamat* b2, float alpha2) {
+// Launches the held-back product (or pair), together with the queued row sums when both wait.
+static int run_stats() {
   const PendAcc p = g_acc;
-  g_acc.active = false;
-  refresh_pending();
-  const bool ta = p.a.is_trans != 0, tb = p.b.is_trans != 0;
-  if (a2)
-    return dn_gemm_pair(ta, tb, p.m, p.n, p.k, p.alpha, p.a.data_device, p.a.size[0], p.b.data_device, p.b.size[0], p.beta, alpha2,
-                        a2->data_device, a2->size[0], b2->data_device, b2->size[0], p.t.data_device, p.t.size[0]);
-  return dn_gemm(ta, tb, p.m, p.n, p.k, p.alpha, p.a.data_device, p.a.size[0], p.b.data_device, p.b.size[0], p.beta,
-                 p.t.data_device, p.t.size[0]);
-}
-static int run_sums() {
   DnRowSumJob jobs[4];
   const int n = g_nsums;
   for (int i = 0; i < n; ++i) jobs[i] = g_sums[i];
+  g_acc.active = false;
   g_nsums = 0;
   refresh_pending();
-  return dn_row_sum_jobs(jobs, n);
+  if (!p.active) return n > 0 ? dn_row_sum_jobs(jobs, n) : 0;
+  const bool ta = p.a.is_trans != 0, tb = p.b.is_trans != 0;
+  if (p.paired)
+    return dn_gemm_pair_sums(ta, tb, p.m, p.n, p.k, p.alpha, p.a.data_device, p.a.size[0], p.b.data_device, p.b.size[0], p.beta,
+                             p.alpha2, p.a2.data_device, p.a2.size[0], p.b2.data_device, p.b2.size[0], p.t.data_device,
+                             p.t.size[0], jobs, n);
+  if (int e = dn_gemm(ta, tb, p.m, p.n, p.k, p.alpha, p.a.data_device, p.a.size[0], p.b.data_device, p.b.size[0], p.beta,
+                      p.t.data_device, p.t.size[0]))
+    return e;
+  return n > 0 ? dn_row_sum_jobs(jobs, n) : 0;
 }
 
 // ---- the dropout mask: mask.fill_with_rand(); mask.greater_than(p); state.mult(mask)
@@ -564,8 +566,7 @@ static void flush_pending() {
   if (batched_updates() > 0) run_batch();          // older than anything else that is held back
   if (g_pend.active) run_pending(nullptr, nullptr);
   if (queued_calls() > 0) run_queue(false);
-  if (g_acc.active) run_acc(nullptr, nullptr, 0.f);
-  if (g_nsums > 0) run_sums();
+  if (g_acc.active || g_nsums > 0) run_stats();
   if (g_drop.stage) run_drop(nullptr);
   g_flushing = false;
   refresh_pending();
@@ -586,13 +587,15 @@ bool dn_defer_dot(cudamat* mat1, cudamat* mat2, cudamat* target, float beta, flo
         n == g_acc.n && k == g_acc.k && (mat1->is_trans != 0) == (g_acc.a.is_trans != 0) &&
         (mat2->is_trans != 0) == (g_acc.b.is_trans != 0) &&
         !overlap(mat1->data_device, dn_len(mat1), target->data_device, dn_len(target)) &&
-        !overlap(mat2->data_device, dn_len(mat2), target->data_device, dn_len(target))) {
-      *err = run_acc(mat1, mat2, alpha);
+        !overlap(mat2->data_device, dn_len(mat2), target->data_device, dn_len(target)) && !g_acc.paired && g_nsums == 0) {
+      g_acc.paired = true;            // (stays held back: the sums of the same statistics may follow)
+      g_acc.a2 = *mat1; g_acc.b2 = *mat2; g_acc.alpha2 = alpha;
       return true;
     }
     dn_flush();
     if (k > 128) return false;        // (pairs run as one launch only for short reductions)
     g_acc.active = true;
+    g_acc.paired = false;
     g_acc.a = *mat1; g_acc.b = *mat2; g_acc.t = *target;
     g_acc.alpha = alpha; g_acc.beta = beta;
     g_acc.m = m; g_acc.n = n; g_acc.k = k;
@@ -670,10 +673,21 @@ bool dn_defer_row_sum(const float* M, float* y, int h, int w, float alpha, float
     if (overlap(q.M, (long long)q.h * q.w, y, h) || overlap(M, (long long)h * w, q.y, q.h)) fits = false;
   }
   if (fits && (mine >= 0 ? cnt[mine] >= 2 : nys >= 2)) fits = false;
+  // the first sum may join a pair of products that waits, unless it writes what they read or write,
+  // or reads what they write
+  if (g_nsums == 0 && g_acc.active && g_acc.paired) {
+    const cudamat* ops[5] = {&g_acc.t, &g_acc.a, &g_acc.b, &g_acc.a2, &g_acc.b2};
+    fits = !overlap(M, (long long)h * w, g_acc.t.data_device, dn_len(&g_acc.t));
+    for (int i = 0; i < 5 && fits; ++i) fits = !overlap(y, h, ops[i]->data_device, dn_len(ops[i]));
+  } else if (g_nsums > 0 && g_acc.active && fits) {
+    const cudamat* ops[5] = {&g_acc.t, &g_acc.a, &g_acc.b, &g_acc.a2, &g_acc.b2};
+    fits = !overlap(M, (long long)h * w, g_acc.t.data_device, dn_len(&g_acc.t));
+    for (int i = 0; i < 5 && fits; ++i) fits = !overlap(y, h, ops[i]->data_device, dn_len(ops[i]));
+  }
   if (!fits) dn_flush();
   g_sums[g_nsums++] = DnRowSumJob{M, y, h, w, alpha, beta};
   dn_set_pending(true);
-  if (g_nsums == 4) *err = run_sums();
+  if (g_nsums == 4) *err = run_stats();
   return true;
 }
 

@@ -9,6 +9,7 @@
 // cross-lane shuffles; rows are reduced by tiles of 64 rows x 4 wavefronts with
 // the lanes running down the rows so every load is a 256-byte run.
 #include "common.h"
+#include "rowsum_jobs.h"
 #include <float.h>
 #include <math.h>
 #include <string.h>
@@ -578,9 +579,7 @@ __device__ __forceinline__ float row_combine(float a, float b) { return OP == RO
 template <int OP>
 __device__ __forceinline__ float row_finish(float yold, float s, float alpha, float beta) {
   if (OP == ROW_MAX) return s;
-  // one multiplication and one fused multiply-add, spelled out so that every kernel that
-  // finishes a row this way rounds alike
-  return __fmaf_rn(alpha, s, beta == 0.f ? 0.f : __fmul_rn(beta, yold));
+  return rowsum_finish(yold, s, alpha, beta);
 }
 
 template <bool VEC, int OP, int NW, int U, bool STREAM>
@@ -937,60 +936,7 @@ static int rows_reduce(const float* M, int ld, int h, int w, const float* x, flo
 // 75-76, 85-86).  Every sum is taken in the order of k_rows_one<ROW_SUM, 4, ., false> with one
 // column slice (lane groups on neighbouring columns, four wavefronts, fixed order in LDS) and
 // finished by the same expression, so the results have the bits of the separate launches.
-struct RowSumJob { const float* M; int w; float alpha, beta; };
-struct RowSumJobs {
-  float* y0; float* y1;
-  int h0, h1, n0, n1, bx0;
-  RowSumJob a0, a1, b0, b1;       // a*: jobs of y0, b*: jobs of y1
-};
-
-__global__ void __launch_bounds__(256) k_rows_sum_jobs(RowSumJobs J) {
-  __shared__ float sv[4][64];
-  const bool second = (int)blockIdx.x >= J.bx0;              // block-uniform
-  const int bx = (int)blockIdx.x - (second ? J.bx0 : 0);
-  const int h = second ? J.h1 : J.h0, nj = second ? J.n1 : J.n0;
-  float* y = second ? J.y1 : J.y0;
-  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-  const int r = lane & 15, c = lane >> 4;
-  const int row0 = (bx * 16 + r) * 4;
-  const int row = bx * 64 + (int)threadIdx.x;
-  const bool mine = threadIdx.x < 64 && row < h;
-  float yv = mine ? y[row] : 0.f;
-  constexpr int NW = 4, U = 8;
-#pragma unroll
-  for (int q = 0; q < 2; ++q) {
-    if (q >= nj) break;
-    const RowSumJob job = second ? (q ? J.b1 : J.b0) : (q ? J.a1 : J.a0);
-    const int w = job.w;
-    float acc[4] = {0.f, 0.f, 0.f, 0.f};
-    if (row0 < h) {
-      for (int j = wv * 4 + c; j < w; j += NW * 4 * U) {
-        float4 v[U];
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-          const int jj = j + NW * 4 * u;
-          v[u] = jj < w ? dn_ld4<false>(job.M + (size_t)jj * h + row0) : make_float4(0.f, 0.f, 0.f, 0.f);
-        }
-#pragma unroll
-        for (int u = 0; u < U; ++u) { acc[0] += v[u].x; acc[1] += v[u].y; acc[2] += v[u].z; acc[3] += v[u].w; }
-      }
-    }
-#pragma unroll
-    for (int o = 16; o < 64; o <<= 1)
-#pragma unroll
-      for (int k = 0; k < 4; ++k) acc[k] = row_combine<ROW_SUM>(acc[k], __shfl_xor(acc[k], o, WAVE));
-    if (c == 0) *reinterpret_cast<float4*>(&sv[wv][r * 4]) = make_float4(acc[0], acc[1], acc[2], acc[3]);
-    __syncthreads();
-    if (mine) {
-      float s = sv[0][threadIdx.x];
-#pragma unroll
-      for (int k = 1; k < NW; ++k) s = row_combine<ROW_SUM>(s, sv[k][threadIdx.x]);
-      yv = row_finish<ROW_SUM>(yv, s, job.alpha, job.beta);
-    }
-    __syncthreads();
-  }
-  if (mine) y[row] = yv;
-}
+__global__ void __launch_bounds__(256) k_rows_sum_jobs(RowSumJobs J) { rows_sum_jobs_body(J, (int)blockIdx.x); }
 
 // Whether sums along the rows of this h x w matrix run as k_rows_one<ROW_SUM, 4, ., false> with one column slice.
 bool dn_row_sum_job_ok(const float* M, int h, int w) {
@@ -1000,24 +946,10 @@ bool dn_row_sum_job_ok(const float* M, int h, int w) {
 
 // jobs in call order: at most two different y, at most two jobs each (the caller has checked that)
 int dn_row_sum_jobs(const DnRowSumJob* jobs, int n) {
-  RowSumJobs J = {};
-  for (int i = 0; i < n; ++i) {
-    const RowSumJob rj = {jobs[i].M, jobs[i].w, jobs[i].alpha, jobs[i].beta};
-    if (J.n0 == 0 || jobs[i].y == J.y0) {
-      if (J.n0 >= 2) return ERROR_GENERIC;
-      J.y0 = jobs[i].y; J.h0 = jobs[i].h;
-      (J.n0 == 0 ? J.a0 : J.a1) = rj;
-      ++J.n0;
-    } else {
-      if ((J.n1 > 0 && jobs[i].y != J.y1) || J.n1 >= 2) return ERROR_GENERIC;
-      J.y1 = jobs[i].y; J.h1 = jobs[i].h;
-      (J.n1 == 0 ? J.b0 : J.b1) = rj;
-      ++J.n1;
-    }
-  }
-  if (J.n0 == 0) return 0;
-  J.bx0 = (J.h0 + 63) / 64;
-  const int blocks = J.bx0 + (J.n1 ? (J.h1 + 63) / 64 : 0);
+  RowSumJobs J;
+  const int blocks = rows_sum_jobs_table(jobs, n, &J);
+  if (blocks < 0) return ERROR_GENERIC;
+  if (blocks == 0) return 0;
   hipLaunchKernelGGL(k_rows_sum_jobs, dim3(blocks), dim3(256), 0, dn_stream(), J);
   return dn_launch_status();
 }

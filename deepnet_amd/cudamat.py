@@ -914,7 +914,9 @@ def cd_update(W, bv, bh, v, h, v2, h2, eps):
     (cudamat/examples/rbm_cudamat.py:57-85) as one product over the concatenated reduction
     [v | v2] . [h | -h2]^T with a row of ones appended to each operand, one launch.  The sums are
     formed in one accumulation instead of two rounded updates, so the result equals the six calls
-    to rounding (about 1e-7 relative), not bit for bit.  bv / bh may be None."""
+    to rounding (about 1e-7 relative), not bit for bit; for batches of up to 128 the library runs
+    the two products and four sums of the six calls themselves in one launch, with their bits.
+    bv / bh may be None."""
     _check(_cudamat.cd_update(W.p_mat, bv.p_mat if bv is not None else None, bh.p_mat if bh is not None else None,
                               v.p_mat, h.p_mat, v2.p_mat, h2.p_mat, float(eps)))
     return W

@@ -300,7 +300,8 @@ int set_deferred_epilogues(int on);
  * the six calls (two add_dot, four add_sums) of cudamat/examples/rbm_cudamat.py:57-85 and the statistics
  * of deepnet/edge.py:236-242, layer.py:206-211, as one product over the concatenated reduction with a
  * row of ones appended to each operand.  W nv x nh, v / v2 nv x batch, h / h2 nh x batch, bv nv x 1,
- * bh nh x 1 (bv, bh may be NULL); nothing transposed.  Equal to the six calls to rounding. ---- */
+ * bh nh x 1 (bv, bh may be NULL); nothing transposed.  Equal to the six calls to rounding (for batches
+ * of up to 128 the products and sums of the six calls themselves, in one launch: the same bits). ---- */
 int cd_update(cudamat* W, cudamat* bv, cudamat* bh, cudamat* v, cudamat* h, cudamat* v2, cudamat* h2, float eps);
 
 /* ---- HIP graphs: no counterpart in the reference.  graph_capture_begin() makes the library

@@ -396,6 +396,8 @@ def test_cd_update_equals_the_six_reference_calls(cm, rng, nv, nh, B):
     for got, ref, want in ((W2, W1, want_w), (BV2, BV1, want_bv), (BH2, BH1, want_bh)):
         assert np.allclose(got.asarray(), want, rtol=1e-6, atol=1e-7)          # against float64
         assert np.allclose(got.asarray(), ref.asarray(), rtol=2e-6, atol=2e-7)  # against the six calls
+        if (nv, nh, B) == (784, 500, 100):      # (the shape of the benchmark runs the six calls' own kernels: same bits)
+            assert np.array_equal(got.asarray().view(np.uint32), ref.asarray().view(np.uint32))
     # without the bias vectors; a second call continues from the first
     W3 = cm.CUDAMatrix(w)
     cm.cd_update(W3, None, None, V, H, V2, H2, eps)
