@@ -368,6 +368,9 @@ void rng_publish(rnd_struct* st) {
 template <class Op>
 static int launch_rng(rnd_struct* st, size_t n, Op op) {
   if (n == 0) return 0;
+  // Work that is held back may use this generator (a fill_with_rand that waits for its threshold)
+  // and leave its next state in the other buffer: it is launched before the state is looked at.
+  dn_flush();
   const size_t draws = (n + NUM_RND_STREAMS - 1) / NUM_RND_STREAMS;
   if (draws < RNG_SPLIT_MIN_DRAWS) {
     if (!rng_pin_if_recording(st)) return ERROR_UNSUPPORTED;
@@ -438,6 +441,7 @@ int init_random(rnd_struct* rnd_state, int seed, char* cudamatpath) {
 #define RNG_GAUSS_PARTS 256
 static int launch_gauss(rnd_struct* st, const float* in, float* out, size_t n, float mult_by) {
   if (n == 0) return 0;
+  dn_flush();          // (as in launch_rng)
   const size_t elems = (n + NUM_RND_STREAMS - 1) / NUM_RND_STREAMS;
   const size_t draws = (elems + 1) & ~(size_t)1;   // of the busiest stream
   int chbits = 4;
