@@ -494,10 +494,11 @@ static int batched_updates();
 //   W.add_dot(v, h.T, eps); W.add_dot(v', h'.T, -eps); bv.add_sums(v, 1, eps); bv.add_sums(v', 1, -eps);
 //   bh.add_sums(h, 1, eps); bh.add_sums(h', 1, -eps)
 // (cudamat/examples/rbm_cudamat.py:73-86): six launches of 2-5 us.  A product with beta = 1 waits for
-// a second product of the same shape into the same target (then both run as one launch,
-// dn_gemm_pair), and up to four row sums onto at most two vectors wait for each other
-// (dn_row_sum_jobs); each result has the bits of the separate launches, and anything else that
-// arrives launches what is held back first, in call order.
+// a second product of the same shape into the same target, the pair waits for row sums, and up to
+// four row sums onto at most two vectors wait for each other: all of it runs as one launch
+// (dn_gemm_pair_sums; sums without a pair: dn_row_sum_jobs).  Each result has the bits of the
+// separate launches; sums that touch the pair's operands or target, and anything else that
+// arrives, launch what is held back first, in call order.
 struct PendAcc {
   bool active;
   bool paired;          // the second product has arrived: the pair waits for the sums that may follow
