@@ -77,6 +77,9 @@ CASES = [  # N, C, H, F, k, stride, padding, groups
     (80, 3, 5, 24, 3, 1, 1, 1),      # 5 chunks per module, fewer chunks than wavefronts
     (64, 3, 40, 32, 3, 1, 1, 1),     # enough chunks for two filter slices per module range (grid y)
     (32, 8, 9, 96, 3, 1, 1, 2),      # 2 groups of 4 colours / 48 filters
+    # convOutp with 81 to 96 patch columns and at most 64 filters ([row][image] LDS tiles, 32-wide column blocks):
+    (64, 6, 8, 32, 4, 1, 1, 1),      # 96 columns, 32 filters
+    (128, 9, 7, 64, 3, 1, 1, 1),     # 81 columns, 64 filters, two chunks of 64 images per module
 ]
 
 
