@@ -1289,11 +1289,6 @@ int dn_gemm_pair_sums(bool a_trans, bool b_trans, int M, int N, int K, float alp
   return njobs > 0 ? dn_row_sum_jobs(jobs, njobs) : 0;
 }
 
-int dn_gemm_pair(bool a_trans, bool b_trans, int M, int N, int K, float alpha, const float* A, int lda, const float* B, int ldb,
-                 float beta, float alpha2, const float* A2, int lda2, const float* B2, int ldb2, float* C, int ldc) {
-  return dn_gemm_pair_sums(a_trans, b_trans, M, N, K, alpha, A, lda, B, ldb, beta, alpha2, A2, lda2, B2, ldb2, C, ldc, nullptr, 0);
-}
-
 // C = beta*C + alpha*op(A)*op(B) on raw column-major buffers, for the other kernels of the library.
 int dn_gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, const float* A, int lda, const float* B,
             int ldb, float beta, float* C, int ldc) {
