@@ -33,6 +33,10 @@ hipStream_t dn_stream();
 void dn_flush();
 void dn_set_pending(bool on);
 void dn_set_flush_hook(void (*f)());
+void dn_set_ext_flush_hook(void (*f)());   // the conv library's held-back calls
+void dn_set_ext_pending(bool on);
+void dn_flush_ext();
+bool dn_defer_enabled();                    // set_deferred_epilogues()
 bool dn_defer_dot(cudamat* mat1, cudamat* mat2, cudamat* target, float beta, float alpha, int m, int n, int k, int* err);
 bool dn_pending_sample(rnd_struct* rnd, cudamat* mat, cudamat* target, int* err);
 // Sums along the rows, y = beta*y + alpha*rowsums(M) (M is h x w, leading dimension h), may be held back too

@@ -37,15 +37,29 @@ static bool g_pending = false;
 static void (*g_flush_hook)() = nullptr;
 void dn_set_flush_hook(void (*f)()) { g_flush_hook = f; }
 void dn_set_pending(bool on) { g_pending = on; }
+// The conv library holds calls back in the same way (a MaxPool that a ResponseNorm may follow); it
+// has its own flag and hook.  Whoever holds a call back launches what the other side holds first,
+// so at most one of the two is set at any time.
+static bool g_ext_pending = false;
+static void (*g_ext_flush_hook)() = nullptr;
+void dn_set_ext_flush_hook(void (*f)()) { g_ext_flush_hook = f; }
+void dn_set_ext_pending(bool on) { g_ext_pending = on; }
+void dn_flush_ext() {
+  if (g_ext_pending) {
+    g_ext_pending = false;
+    if (g_ext_flush_hook) g_ext_flush_hook();
+  }
+}
 void dn_flush() {
   if (g_pending) {
     g_pending = false;
     if (g_flush_hook) g_flush_hook();
   }
+  dn_flush_ext();
 }
 
 hipStream_t dn_stream() {
-  if (g_pending) dn_flush();
+  if (g_pending || g_ext_pending) dn_flush();
   return g_stream;
 }
 bool dn_capturing() { return g_capturing; }

@@ -699,6 +699,8 @@ static inline bool pend_is(const cudamat* x) {
 }
 static inline bool pend_open() { return g_pend.active && !g_no_defer; }
 
+bool dn_defer_enabled() { return g_defer_enabled && !g_no_defer; }
+
 extern "C" {
 
 // Extension: switches the deferred epilogues on or off (on by default); returns the previous setting.
@@ -906,6 +908,7 @@ int mult_by_scalar(cudamat* mat, float val, cudamat* target) {
     // (a complete update before this one waits on; anything else that is held back is launched now)
     int e = 0;
     if (update_ready()) e = stash_ready(false);
+    dn_flush_ext();
     if (g_pend.active || g_eqn > 0 || g_acc.active || g_nsums > 0 || g_drop.stage != 0) dn_flush();
     if (e) return e;
     g_eq[0].kind = EQ_MULS; g_eq[0].dst = *mat; g_eq[0].src = *mat; g_eq[0].s = val;

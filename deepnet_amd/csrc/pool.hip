@@ -928,6 +928,47 @@ static void pool_impl(cudamat* images, cudamat* rnd, cudamat* targets, int numFi
   if (dn_launch_status()) conv_set_error(where, hipGetErrorString(hipGetLastError()));
 }
 
+// ---- MaxPool held back.  deepnet's conv stage calls MaxPool and then ResponseNorm on the pooled map
+// (deepnet/convolutions.py:58-66): where the two can run as one launch (MaxPoolResponseNorm's LDS
+// kernel: the same bits in the pooled map, the denominators and the result), MaxPool does not
+// launch at once; a ResponseNorm of its target takes it along, and any other call -- of this
+// library or of the matrix library -- launches it first (every launch passes through dn_stream()).
+struct PendPool {
+  bool active;
+  cudamat images, targets;
+  int numFilters, subsX, startX, strideX, outputsX;
+};
+static PendPool g_pp = {};
+static int norm_lds_qb(int N, int S);
+
+static void pool_flush() {
+  if (!g_pp.active) return;
+  PendPool q = g_pp;
+  g_pp.active = false;
+  pool_impl(&q.images, nullptr, &q.targets, q.numFilters, q.subsX, q.startX, q.strideX, q.outputsX, "MaxPool");
+}
+static const int g_pool_flush_registered = (dn_set_ext_flush_hook(pool_flush), 0);
+
+// Holds the call back when MaxPoolResponseNorm's one-launch kernel could serve it (the conditions of
+// that entry point on the pooling side; anything else, errors included, takes the usual path).
+static bool pool_hold(cudamat* images, cudamat* targets, int numFilters, int subsX, int startX, int strideX, int outputsX) {
+  if (!dn_defer_enabled()) return false;
+  if (!images->on_device || !targets->on_device || numFilters <= 0 || outputsX <= 0) return false;
+  if (!(strideX == 2 && (subsX == 2 || subsX == 3))) return false;
+  const int N = images->size[0];
+  if (N <= 0 || N % 4 != 0 || images->size[1] % numFilters != 0 || isqrt_exact_p(images->size[1] / numFilters) <= 0) return false;
+  if (targets->size[0] != N || targets->size[1] != numFilters * outputsX * outputsX) return false;
+  if (!all_aligned16({images->data_device, targets->data_device}) || images->data_device == targets->data_device) return false;
+  if (norm_lds_qb(N, outputsX) <= 0 || (long long)N * images->size[1] >= (1ll << 31)) return false;
+  dn_flush();                       // (what either library holds back comes first)
+  conv_clear_error();
+  g_pp.active = true;
+  g_pp.images = *images; g_pp.targets = *targets;
+  g_pp.numFilters = numFilters; g_pp.subsX = subsX; g_pp.startX = startX; g_pp.strideX = strideX; g_pp.outputsX = outputsX;
+  dn_set_ext_pending(true);
+  return true;
+}
+
 static void cnorm_impl(cudamat* images, cudamat* meanDiffs, cudamat* denoms, cudamat* targets, int numFilters,
                        int sizeX, float addScale, float powScale, const char* where) {
   conv_clear_error();
@@ -1038,6 +1079,7 @@ static void rnorm_undo_impl(cudamat* outGrads, cudamat* denoms, cudamat* inputs,
 extern "C" {
 
 void MaxPool(cudamat* images, cudamat* targets, int numFilters, int subsX, int startX, int strideX, int outputsX) {
+  if (pool_hold(images, targets, numFilters, subsX, startX, strideX, outputsX)) return;
   pool_impl(images, nullptr, targets, numFilters, subsX, startX, strideX, outputsX, "MaxPool");
 }
 
@@ -1098,8 +1140,23 @@ void MaxPoolUndo(cudamat* images, cudamat* maxGrads, cudamat* maxActs, cudamat* 
   if (dn_launch_status()) conv_set_error(where, hipGetErrorString(hipGetLastError()));
 }
 
+void MaxPoolResponseNorm(cudamat* images, cudamat* pooled, cudamat* denoms, cudamat* targets, int numFilters, int subsX,
+                         int startX, int strideX, int outputsX, int sizeX, float addScale, float powScale);
+
 void ResponseNorm(cudamat* images, cudamat* denoms, cudamat* targets, int numFilters, int sizeX, float addScale,
                   float powScale) {
+  // (the normalisation of a pooled map whose MaxPool is being held back: both in one launch)
+  if (g_pp.active && images->on_device && images->data_device == g_pp.targets.data_device && images->size[0] == g_pp.targets.size[0] &&
+      images->size[1] == g_pp.targets.size[1] && numFilters == g_pp.numFilters && sizeX > 0 && denoms->on_device &&
+      targets->on_device && denoms->size[0] == images->size[0] && denoms->size[1] == images->size[1] &&
+      targets->size[0] == images->size[0] && targets->size[1] == images->size[1]) {
+    PendPool q = g_pp;
+    g_pp.active = false;
+    dn_set_ext_pending(false);
+    MaxPoolResponseNorm(&q.images, images, denoms, targets, numFilters, q.subsX, q.startX, q.strideX, q.outputsX, sizeX,
+                        addScale, powScale);
+    return;
+  }
   cnorm_impl(images, images, denoms, targets, numFilters, sizeX, addScale, powScale, "ResponseNorm");
 }
 

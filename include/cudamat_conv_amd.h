@@ -60,7 +60,10 @@ void ContrastNormUndo(cudamat* outGrads, cudamat* denoms, cudamat* meanDiffs, cu
                       int numFilters, int sizeX, float addScale, float powScale);
 
 /* ---- local pooling: cudamat_conv.cu:1442-1454 (convLocalPool :1021-1120, convLocalProbPool
- * :1189-1289, convLocalMaxUndo :1128-1182) ---- */
+ * :1189-1289, convLocalMaxUndo :1128-1182).  MaxPool may be held back (unless
+ * set_deferred_epilogues(0) of libcudamat.so is in force): a ResponseNorm of its target that follows
+ * directly runs with it as one launch, any other call of either library launches it first; same
+ * results in every array. ---- */
 void MaxPool(cudamat* images, cudamat* targets, int numFilters, int subsX, int startX, int strideX, int outputsX);
 void ProbMaxPool(cudamat* images, cudamat* rnd, cudamat* targets, int numFilters, int subsX, int startX, int strideX,
                  int outputsX);

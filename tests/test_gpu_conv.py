@@ -480,8 +480,10 @@ def test_pool_and_norm_in_one_launch_equal_the_separate_calls(cm, cc, rng, N, F,
     X = cm.CUDAMatrix(x)
     shape = (N, F * O * O)
     pooled1, den1, out1 = cm.empty(shape), cm.empty(shape), cm.empty(shape)
+    cm.set_deferred_epilogues(False)          # (each call its own launch: a held-back MaxPool would join the ResponseNorm)
     cc.MaxPool(X, pooled1, F, subs, start, stride, O)
     cc.ResponseNorm(pooled1, den1, out1, F, size, a, p)
+    cm.set_deferred_epilogues(True)
     pooled2, den2, out2 = cm.empty(shape), cm.empty(shape), cm.empty(shape)
     for m in (pooled2, den2, out2):
         m.assign(np.nan)
@@ -533,3 +535,32 @@ def test_pool_and_norm_in_one_launch_keep_the_bits_at_the_benchmark_layer(cm, cc
     cc.MaxPoolUndo(X, undo1, tmp_grad, pooled1, 3, 0, 2, O)
     cc.ResponseNormUndoMaxPoolUndo(G, den2, out2, pooled2, X, undo2, F, 3, 0, 2, O, 5, 0.001, 0.75)
     assert np.array_equal(undo1.asarray().view(np.uint32), undo2.asarray().view(np.uint32))
+
+
+@pytest.mark.parametrize("N,F,S,subs,start,stride,size", FUSED_POOL_NORM)
+def test_a_held_back_max_pool_joins_the_response_norm_that_follows(cm, cc, rng, N, F, S, subs, start, stride, size):
+    """deepnet/convolutions.py:58-66 calls MaxPool and then ResponseNorm on the pooled map: the library
+    holds the MaxPool back and runs both as one launch where its LDS kernel applies.  With the
+    deferral off and on: the same bits in the pooled map, the denominators and the result, whatever
+    comes between or after the two calls."""
+    a, p = 0.001, 0.75
+    O = (S - start - subs + stride - 1) // stride + 1
+    x = _f(rng.standard_normal((N, F * S * S)) * 2)
+    shape = (N, F * O * O)
+    res = []
+    for deferred in (False, True):
+        cm.set_deferred_epilogues(deferred)
+        X = cm.CUDAMatrix(x)
+        pooled, den, out, other, den2, out2 = (cm.empty(shape) for _ in range(6))
+        for m in (pooled, den, out, other, den2, out2):
+            m.assign(np.nan)
+        cc.MaxPool(X, pooled, F, subs, start, stride, O); cc.ResponseNorm(pooled, den, out, F, size, a, p)   # the pair
+        cc.MaxPool(X, other, F, subs, start, stride, O)                                                     # held back, then read
+        first = other.asarray().copy()
+        cc.MaxPool(X, other, F, subs, start, stride, O); other.mult(2.0)                  # ... then used by the matrix library
+        cc.MaxPool(X, other, F, subs, start, stride, O); cc.ResponseNorm(pooled, den2, out2, F, size, a, p)  # ... then a norm of another map
+        cc.MaxPool(X, other, F, subs, start, stride, O); cc.MaxPool(X, pooled, F, subs, start, stride, O)    # two in a row
+        res.append([m.asarray().view(np.uint32).copy() for m in (pooled, den, out, other, den2, out2)] + [first.view(np.uint32)])
+    cm.set_deferred_epilogues(True)
+    for i, (w, g) in enumerate(zip(*res)):
+        assert np.array_equal(w, g), "result %d differs" % i
