@@ -105,15 +105,15 @@ STEP_BYTES = NSETS * sum(b for _, b, _ in C2_OPS)
 
 
 def run_c2_step(cm, sets, ev=None, marks=None):
-    """One step.  With ev/marks, brackets each op's NSETS launches with events."""
+    """One step.  With ev/marks, brackets the NSETS launches of every op that has a pair of events in marks."""
     for name, _, fn in C2_OPS:
-        if ev is not None:
-            a, b = marks[name]
-            ev.record(a)
+        pair = marks.get(name) if ev is not None else None
+        if pair:
+            ev.record(pair[0])
         for s in sets:
             fn(cm, s)
-        if ev is not None:
-            ev.record(b)
+        if pair:
+            ev.record(pair[1])
 
 
 # ---------------------------------------------------------------- secondary workloads
@@ -558,19 +558,27 @@ def main():
         return
 
     sets = build_c2(cm)
-    marks = {name: (ev.new(), ev.new()) for name, _, _ in C2_OPS}
+    roof_op = 'add_mult'
     for _ in range(args.warmup):
         run_c2_step(cm, sets)
+    # The timed steps: nothing waits inside them; the launches of the roofline's kernel have their own pair
+    # of events in every step, read back after the last one.
+    roof_marks = [{roof_op: (ev.new(), ev.new())} for _ in range(args.steps)]
     cm.cuda_sync_threads()
-    per_op_ms = {name: [] for name, _, _ in C2_OPS}
     t0 = time.perf_counter()
+    for k in range(args.steps):
+        run_c2_step(cm, sets, ev, roof_marks[k])
+    cm.cuda_sync_threads()
+    step_s = (time.perf_counter() - t0) / args.steps
+    roof_ms = float(np.mean([ev.elapsed_ms(*m[roof_op]) / NSETS for m in roof_marks]))
+    # The per-op figures: the same steps once more with events around every op, read back after each step.
+    marks = {name: (ev.new(), ev.new()) for name, _, _ in C2_OPS}
+    per_op_ms = {name: [] for name, _, _ in C2_OPS}
     for _ in range(args.steps):
         run_c2_step(cm, sets, ev, marks)
-        # reading the events back waits for the step, which the next step would do anyway
         for name, _, _ in C2_OPS:
             per_op_ms[name].append(ev.elapsed_ms(*marks[name]) / NSETS)
     cm.cuda_sync_threads()
-    step_s = (time.perf_counter() - t0) / args.steps
 
     ops = {}
     for name, nbytes, _ in C2_OPS:
@@ -579,7 +587,6 @@ def main():
         ops[name] = {'us': round(ms * 1e3, 2), 'gbs': round(gbs, 1), 'frac_hbm': round(gbs / HBM_PEAK_GBS, 4)}
     value = STEP_BYTES / step_s / 1e9
 
-    roof_op = 'add_mult'
     traffic = None
     try:    # HBM bytes per launch from the committed rocprofv3 --pmc summary (FETCH_SIZE + WRITE_SIZE, calibrated)
         for ln in open(os.path.join(ROOT, 'profiles', 'k_ew_axpy_hbm_traffic.md')):
@@ -587,12 +594,13 @@ def main():
                 traffic = int(ln.split(':')[1])
     except OSError:
         pass
+    roof_gbs = round(12 * E / (roof_ms * 1e-3) / 1e9, 1)
     roofline = {'kernel': 'k_ew<2, true, FAxpy> (add_mult, 4096x4096)', 'bound': 'hbm',
-                'achieved': ops[roof_op]['gbs'], 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
-                'frac': round(ops[roof_op]['gbs'] / HBM_PEAK_GBS, 4), 'traffic': traffic,
+                'achieved': roof_gbs, 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
+                'frac': round(roof_gbs / HBM_PEAK_GBS, 4), 'traffic': traffic,
                 'traffic_source': 'profiles/k_ew_axpy_hbm_traffic.md (an earlier rocprofv3 --pmc run of bench.py --probe, '
                                   'not measured by this run)',
-                'algorithmic_bytes_per_launch': 12 * E, 'avg_launch_us': ops[roof_op]['us']}
+                'algorithmic_bytes_per_launch': 12 * E, 'avg_launch_us': round(roof_ms * 1e3, 2)}
 
     secondary = {}
     if not args.only_c2:
@@ -686,7 +694,10 @@ def main():
         'roofline': roofline, 'ops': ops, 'secondary': secondary,
         'timing': {'value': 'wall time of the K = %d steps between two device synchronisations, after %d warm-up steps, one run'
                             % (args.steps, args.warmup),
-                   'ops': 'HIP events on the NULL stream around the %d launches of an op in a step; median over the K steps' % NSETS,
+                   'roofline': 'HIP events on the NULL stream around the %d add_mult launches of every timed step, read back after the '
+                               'last step; mean over the K steps' % NSETS,
+                   'ops': 'the K steps once more, outside the timed region, with HIP events around the %d launches of every op, '
+                          'read back after each step; median over the K steps' % NSETS,
                    'steps_per_sec': 'wall time of `iters` steps after `warmup` steps, device synchronised on both sides, one run',
                    'gemm_conv': 'HIP events around 10 (4096^3, conv: median of 3 such groups) or 200 (layer shapes) back-to-back '
                                 'launches after 30 ms of matrix-core warm-up',
