@@ -39,7 +39,8 @@ NSETS = 8
 class HipEvents(object):
     """hipEvent timing on the NULL stream (the stream the library launches on)."""
 
-    def __init__(self):
+    def __init__(self, flush=None):
+        self.flush = flush      # queues what the library holds back (cm.launch_deferred)
         self.hip = ct.CDLL('libamdhip64.so')
         self.hip.hipEventCreate.argtypes = [ct.POINTER(ct.c_void_p)]
         self.hip.hipEventRecord.argtypes = [ct.c_void_p, ct.c_void_p]
@@ -54,6 +55,9 @@ class HipEvents(object):
         return ev
 
     def record(self, ev):
+        # (a call that the library holds back is not in the stream yet: it is queued first)
+        if self.flush is not None:
+            self.flush()
         assert self.hip.hipEventRecord(ev, None) == 0
 
     def elapsed_ms(self, a, b):
@@ -525,7 +529,7 @@ def main():
     from deepnet_amd import cudamat as cm
     cm.cublas_init()
     cm.CUDAMatrix.init_random(2)
-    ev = HipEvents()
+    ev = HipEvents(cm.launch_deferred)
 
     if args.probe_mfma:
         # the matrix-core kernels only, a few launches each and no clock warm-up: for counter runs

@@ -711,6 +711,11 @@ int set_deferred_epilogues(int on) {
   return before;
 }
 
+int launch_deferred(void) {
+  dn_flush();
+  return dn_launch_status();
+}
+
 int add_col_vec(cudamat* mat, cudamat* vec, cudamat* target) {
   if (pend_open() && !g_pend.has_bias && g_pend.act == 0 && pend_is(mat) && pend_is(target) && vec->on_device &&
       !vec->is_trans && vec->size[0] == mat->size[0] && vec->size[1] == 1 && vec->data_device != mat->data_device) {

@@ -116,7 +116,7 @@ _SIGNATURES = {
     'correct_preds': (_i, [_M, _M, _M, _f]),
     'dot': (_i, [_M, _M, _M, _f, _f]),
     'dot_bias_act': (_i, [_M, _M, _M, _M, ct.c_int]),
-    'cd_update': (_i, [_M, _M, _M, _M, _M, _M, _M, _f]), 'set_deferred_epilogues': (_i, [_i]),
+    'cd_update': (_i, [_M, _M, _M, _M, _M, _M, _M, _f]), 'set_deferred_epilogues': (_i, [_i]), 'launch_deferred': (_i, []),
     'dot_bias_act_sample': (_i, [ct.c_void_p, _M, _M, _M, _M, _M, ct.c_int]),
     'momentum_update': (_i, [_M, _M, _M, _f, _f, _f, _f, ct.c_int]),
     'momentum_update_many': (_i, [ct.c_int, ct.c_void_p, ct.c_void_p, ct.c_void_p, ct.c_void_p, ct.c_void_p, ct.c_void_p,
@@ -904,6 +904,13 @@ def set_deferred_epilogues(on):
     (the statistics of cudamat/examples/rbm_cudamat.py:73-86).  On by default; returns the previous
     setting."""
     return bool(_cudamat.set_deferred_epilogues(1 if on else 0))
+
+
+def launch_deferred():
+    """Extension of this backend: queues the calls that are held back (see `set_deferred_epilogues`)
+    and waits for nothing.  For a caller that records its own events on the NULL stream, or queues
+    other work behind the library's, and must have every call made so far in the stream."""
+    _check(_cudamat.launch_deferred())
 
 
 def cd_update(W, bv, bh, v, h, v2, h2, eps):

@@ -292,8 +292,11 @@ int get_softmax_cross_entropy(cudamat* mat, cudamat* labels, cudamat* target, fl
  * launches); same bits, call order kept wherever two calls touch the same memory.  fill_with_rand is held
  * back likewise: greater_than_scalar of that matrix in place and mult_elementwise of another matrix by it in
  * place (the dropout mask of deepnet/neuralnet.py:194-198) run with it as one pass, same draws and values.
- * set_deferred_epilogues(0) makes every call launch at once; returns the previous setting (default 1). ---- */
+ * set_deferred_epilogues(0) makes every call launch at once; returns the previous setting (default 1).
+ * launch_deferred() queues what is held back now and waits for nothing: for a caller that records its own
+ * events on the library's stream (the NULL stream) or queues other work behind the library's. ---- */
 int set_deferred_epilogues(int on);
+int launch_deferred(void);
 
 /* ---- Extension: the contrastive-divergence update of an RBM in one launch,
  *   W += eps (v h^T - v2 h2^T),  bv += eps (rowsums v - rowsums v2),  bh += eps (rowsums h - rowsums h2),

@@ -505,6 +505,29 @@ def test_the_switch_reports_its_previous_setting(cm):
     assert cm.set_deferred_epilogues(True) is True
 
 
+def test_launch_deferred_queues_what_is_held_back(cm, rng):
+    """A caller that goes on with its own work on the NULL stream (here: a plain hipMemcpy through the
+    runtime, which the library does not see) finds the results of every call it has made."""
+    import ctypes as ct
+    hip = ct.CDLL('libamdhip64.so')
+    hip.hipMemcpy.argtypes = [ct.c_void_p, ct.c_void_p, ct.c_size_t, ct.c_int]
+    a, b = _f(rng.standard_normal((96, 64)) * 0.1), _f(rng.standard_normal((64, 40)))
+    bias = _f(rng.standard_normal((96, 1)))
+    A, B, bv = cm.CUDAMatrix(a), cm.CUDAMatrix(b), cm.CUDAMatrix(bias)
+    T = cm.empty((96, 40)); T.assign(-3.0)
+    cm.cuda_sync_threads()
+    cm.dot(A, B, target=T)
+    T.add_col_vec(bv)                         # both calls are held back now
+    cm.launch_deferred()
+    got = np.empty((96, 40), dtype=np.float32, order='F')
+    assert hip.hipMemcpy(got.ctypes.data, ct.cast(T.p_mat.contents.data_device, ct.c_void_p), got.nbytes, 2) == 0
+    want = a.astype(np.float64) @ b.astype(np.float64) + bias
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-5)
+    T.apply_sigmoid()                         # and the library goes on from there
+    np.testing.assert_allclose(T.asarray(), 1.0 / (1.0 + np.exp(-want)), rtol=1e-5, atol=1e-6)
+    cm.launch_deferred()                      # nothing held back: no effect
+
+
 # ---- random call sequences: whatever is held back, every matrix ends with the bits of the separate launches
 
 def _random_sequence(cm, rng_ops, pool, vecs, rows, n_ops):
