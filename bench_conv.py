@@ -40,6 +40,20 @@ def _time(ev, fn, iters, sync):
     return sorted(reps)[1]
 
 
+C4_SETS = 10     # operand sets that config 4's figures rotate over (33.5 MB maps: one set would stay in the caches)
+
+
+def _rotate(sets):
+    """sets[0], sets[1], ... in turn, one per call."""
+    state = [0]
+
+    def nxt():
+        s = sets[state[0] % len(sets)]
+        state[0] += 1
+        return s
+    return nxt
+
+
 def run(cm, ev, iters=10):
     from deepnet_amd import cudamat_conv as cc
     rng = np.random.default_rng(5)
@@ -48,53 +62,85 @@ def run(cm, ev, iters=10):
     for name, L in LAYERS.items():
         N, C, H, F, k, s, p, G = (L[x] for x in ('N', 'C', 'H', 'F', 'k', 's', 'p', 'G'))
         Mx = (H + 2 * p - k) // s + 1
-        X = f(rng.standard_normal((N, C * H * H)))
-        W = f(0.01 * rng.standard_normal((F, (C // G) * k * k)))
-        Y = f(rng.standard_normal((N, F * Mx * Mx)))
-        up, down, dw = cm.empty((N, F * Mx * Mx)), cm.empty((N, C * H * H)), cm.empty((F, (C // G) * k * k))
+        c4 = name.startswith('c4')
+        # Config 4's largest operand is 33.5 MB: launched again and again on the same arrays, a kernel would find its
+        # inputs in the L2s and the 256 MB last-level cache.  Its figures rotate over C4_SETS sets (about 1.4 GB).
+        # Configs 5a / 5b are bound by the matrix cores (0.25-0.5 ms per pass against 30 us for their bytes): one set.
+        hx, hw, hy = rng.standard_normal((N, C * H * H)), 0.01 * rng.standard_normal((F, (C // G) * k * k)), \
+            rng.standard_normal((N, F * Mx * Mx))
+        sets = [dict(X=f(hx), W=f(hw), Y=f(hy), up=cm.empty((N, F * Mx * Mx)), down=cm.empty((N, C * H * H)),
+                     dw=cm.empty((F, (C // G) * k * k))) for _ in range(C4_SETS if c4 else 1)]
+        nxt = _rotate(sets)
+        W = sets[0]['W']
         flops = 2.0 * N * F * Mx * Mx * (C // G) * k * k
-        res = {'gflop_per_pass': round(flops / 1e9, 3)}
-        for label, fn in (('convUp', lambda: cc.convUp(X, W, up, Mx, p, s, C, G)),
-                          ('convDown', lambda: cc.convDown(Y, W, down, Mx, p, s, k, H, C, numGroups=G)),
-                          ('convOutp', lambda: cc.convOutp(X, Y, dw, Mx, p, k, s, C, numGroups=G))):
+        res = {'gflop_per_pass': round(flops / 1e9, 3), 'operand_sets': len(sets)}
+
+        def conv_up():
+            d = nxt(); cc.convUp(d['X'], d['W'], d['up'], Mx, p, s, C, G)
+
+        def conv_down():
+            d = nxt(); cc.convDown(d['Y'], d['W'], d['down'], Mx, p, s, k, H, C, numGroups=G)
+
+        def conv_outp():
+            d = nxt(); cc.convOutp(d['X'], d['Y'], d['dw'], Mx, p, k, s, C, numGroups=G)
+        for label, fn in (('convUp', conv_up), ('convDown', conv_down), ('convOutp', conv_outp)):
             ms = _time(ev, fn, iters, cm.cuda_sync_threads)
             tf = flops / (ms * 1e-3) / 1e12
             res[label] = {'ms': round(ms, 4), 'tflops': round(tf, 2),
                           'frac_mfma_fp32': round(tf / MFMA_FP32_PEAK_TFLOPS, 4)}
-        if name.startswith('c4'):
+        if c4:
             O = 15
-            pooled, grad = cm.empty((N, F * O * O)), f(rng.standard_normal((N, F * O * O)))
-            undo = cm.empty((N, F * Mx * Mx))
-            den, normed, nundo = cm.empty((N, F * O * O)), cm.empty((N, F * O * O)), cm.empty((N, F * O * O))
-            acts = cm.empty((N, F * O * O))
+            hgrad = rng.standard_normal((N, F * O * O))
+            for d in sets:       # (d['up'] holds the convUp result of its set by now)
+                d.update(grad=f(hgrad), undo=cm.empty((N, F * Mx * Mx)))
+                for key in ('pooled', 'den', 'normed', 'nundo', 'acts', 'p2', 'd2', 'n2'):
+                    d[key] = cm.empty((N, F * O * O))
             e_in, e_out = 4.0 * N * F * Mx * Mx, 4.0 * N * F * O * O
-            for label, fn, nbytes in (
-                    ('MaxPool', lambda: cc.MaxPool(up, pooled, F, 3, 0, 2, O), e_in + e_out),
-                    ('MaxPoolUndo', lambda: cc.MaxPoolUndo(up, undo, grad, pooled, 3, 0, 2, O), 2 * e_in + 2 * e_out),
-                    ('ResponseNorm', lambda: cc.ResponseNorm(pooled, den, normed, F, 5, 0.001, 0.75), 3 * e_out),
-                    ('ResponseNormUndo', lambda: (acts.assign(normed),
-                                                  cc.ResponseNormUndo(grad, den, pooled, acts, nundo, F, 5, 0.001, 0.75)),
-                     (2 + 7) * e_out)):
-                ms = _time(ev, fn, iters, cm.cuda_sync_threads)
-                gbs = nbytes / (ms * 1e-3) / 1e9
-                res[label] = {'us': round(ms * 1e3, 2), 'gbs': round(gbs, 1), 'frac_hbm': round(gbs / HBM_PEAK_GBS, 4)}
+
+            def max_pool():
+                d = nxt(); cc.MaxPool(d['up'], d['pooled'], F, 3, 0, 2, O)
+
+            def max_pool_undo():
+                d = nxt(); cc.MaxPoolUndo(d['up'], d['undo'], d['grad'], d['pooled'], 3, 0, 2, O)
+
+            def response_norm():
+                d = nxt(); cc.ResponseNorm(d['pooled'], d['den'], d['normed'], F, 5, 0.001, 0.75)
+
+            def response_norm_undo():
+                d = nxt(); d['acts'].assign(d['normed'])
+                cc.ResponseNormUndo(d['grad'], d['den'], d['pooled'], d['acts'], d['nundo'], F, 5, 0.001, 0.75)
+
             # the two pairs deepnet issues back to back, each as one launch (extensions of this backend):
             # algorithmic bytes = the un-pooled map in + three pooled-size arrays out; four pooled-size arrays and the
             # un-pooled map in + the un-pooled gradient out
-            p2, d2, n2 = cm.empty((N, F * O * O)), cm.empty((N, F * O * O)), cm.empty((N, F * O * O))
-            for label, fn, nbytes in (
-                    ('MaxPoolResponseNorm', lambda: cc.MaxPoolResponseNorm(up, p2, d2, n2, F, 3, 0, 2, O, 5, 0.001, 0.75),
-                     e_in + 3 * e_out),
-                    ('ResponseNormUndoMaxPoolUndo', lambda: cc.ResponseNormUndoMaxPoolUndo(grad, d2, n2, p2, up, undo, F, 3, 0, 2, O,
-                                                                                          5, 0.001, 0.75), 2 * e_in + 4 * e_out)):
+            def pool_norm():
+                d = nxt(); cc.MaxPoolResponseNorm(d['up'], d['p2'], d['d2'], d['n2'], F, 3, 0, 2, O, 5, 0.001, 0.75)
+
+            def norm_undo_pool_undo():
+                d = nxt(); cc.ResponseNormUndoMaxPoolUndo(d['grad'], d['d2'], d['n2'], d['p2'], d['up'], d['undo'], F, 3, 0, 2, O,
+                                                          5, 0.001, 0.75)
+            # (each op is warmed up for longer than C4_SETS calls, so every set has the results of the op before it)
+            for label, fn, nbytes in (('MaxPool', max_pool, e_in + e_out),
+                                      ('MaxPoolUndo', max_pool_undo, 2 * e_in + 2 * e_out),
+                                      ('ResponseNorm', response_norm, 3 * e_out),
+                                      ('ResponseNormUndo', response_norm_undo, (2 + 7) * e_out),
+                                      ('MaxPoolResponseNorm', pool_norm, e_in + 3 * e_out),
+                                      ('ResponseNormUndoMaxPoolUndo', norm_undo_pool_undo, 2 * e_in + 4 * e_out)):
+                for _ in range(len(sets)):
+                    fn()
                 ms = _time(ev, fn, iters, cm.cuda_sync_threads)
                 gbs = nbytes / (ms * 1e-3) / 1e9
                 res[label] = {'us': round(ms * 1e3, 2), 'gbs': round(gbs, 1), 'frac_hbm': round(gbs / HBM_PEAK_GBS, 4)}
+            for d in sets[1:]:
+                for m in d.values():
+                    m.free_device_memory()
+            del sets[1:]
             res['stage_fwd_bwd'] = _stage(cm, ev, iters, L, W, rng)
             res['stage_fwd_bwd_fused_pool_norm'] = _stage(cm, ev, iters, L, W, rng, fused=True)
         out[name] = res
-        for m in (X, W, Y, up, down, dw):
-            m.free_device_memory()
+        for d in sets:
+            for m in d.values():
+                m.free_device_memory()
     out['local_64x8x8_64f3'] = _local(cm, cc, ev, iters, rng)
     return {'conv': out}
 
