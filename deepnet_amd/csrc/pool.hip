@@ -701,6 +701,9 @@ k_pool_norm_lds(const float* imgs, float* pooled, float* denoms, float* target, 
 // pixel of the un-pooled map then collects it from the windows that hold the pixel and whose
 // maximum it is, in the order of k_pool_undo_fixed.  target may be imgs (a lane reads its pixel
 // before it writes it).
+#ifndef UNDO_PRE
+#define UNDO_PRE 2
+#endif
 template <int QB, int SUBS, int STRIDE, int SIZE>
 __global__ void __launch_bounds__(NORM_LDS_THREADS)
 k_normundo_poolundo_lds(const float* outGrads, const float* denoms, const float* inputs, const float* acts, const float* imgs,
@@ -722,6 +725,18 @@ k_normundo_poolundo_lds(const float* outGrads, const float* denoms, const float*
   float4 keep0[NORM_LDS_SLOTS], keep1[NORM_LDS_SLOTS];
 #pragma unroll
   for (int k = 0; k < NORM_LDS_SLOTS; ++k) keep1[k] = make_float4(0.f, 0.f, 0.f, 0.f);
+  // The un-pooled map does not depend on the normalisation's gradient: the groups of the first
+  // UNDO_PRE trips of the last phase are requested here, together with the pooled arrays.
+  const int items = Sin * Sin * QB;
+  float4 pre[4 * UNDO_PRE];
+#pragma unroll
+  for (int u = 0; u < 4 * UNDO_PRE; ++u) {
+    const int j = (int)threadIdx.x + u * NORM_LDS_THREADS;
+    const int pin = j / QB, q = j - pin * QB;
+    const bool ok = j < items && q < qn;
+    const float4 v4 = ld4_once(ok ? imgs + in0 + (size_t)N * pin + 4 * q : imgs + in0, POOL_NT & 4);
+    pre[u] = ok ? v4 : make_float4(0.f, 0.f, 0.f, 0.f);
+  }
   {
     float4 w[NORM_LDS_SLOTS], og[NORM_LDS_SLOTS], den[NORM_LDS_SLOTS];
 #pragma unroll
@@ -795,16 +810,7 @@ k_normundo_poolundo_lds(const float* outGrads, const float* denoms, const float*
   }
   __syncthreads();
   // the un-pooled map: every (pixel, 4 images) group of it, four per trip with their loads in flight together
-  const int items = Sin * Sin * QB;
-  for (int j0 = (int)threadIdx.x; j0 < items; j0 += 4 * NORM_LDS_THREADS) {
-    float4 img[4];
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int j = j0 + u * NORM_LDS_THREADS;
-      const int pin = j / QB, q = j - pin * QB;
-      const bool ok = j < items && q < qn;
-      { const float4 v4 = ld4_once(ok ? imgs + in0 + (size_t)N * pin + 4 * q : imgs + in0, POOL_NT & 4); img[u] = ok ? v4 : make_float4(0.f, 0.f, 0.f, 0.f); }
-    }
+  auto scatter = [&](int j0, const float4* img) {
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int j = j0 + u * NORM_LDS_THREADS;
@@ -832,6 +838,19 @@ k_normundo_poolundo_lds(const float* outGrads, const float* denoms, const float*
       }
       st4_once(target + in0 + (size_t)N * pin + 4 * q, acc, POOL_NT & 8);
     }
+  };
+#pragma unroll
+  for (int t = 0; t < UNDO_PRE; ++t) scatter((int)threadIdx.x + t * 4 * NORM_LDS_THREADS, pre + 4 * t);
+  for (int j0 = (int)threadIdx.x + UNDO_PRE * 4 * NORM_LDS_THREADS; j0 < items; j0 += 4 * NORM_LDS_THREADS) {
+    float4 img[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int j = j0 + u * NORM_LDS_THREADS;
+      const int pin = j / QB, q = j - pin * QB;
+      const bool ok = j < items && q < qn;
+      { const float4 v4 = ld4_once(ok ? imgs + in0 + (size_t)N * pin + 4 * q : imgs + in0, POOL_NT & 4); img[u] = ok ? v4 : make_float4(0.f, 0.f, 0.f, 0.f); }
+    }
+    scatter(j0, img);
   }
 }
 
