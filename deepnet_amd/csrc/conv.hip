@@ -1519,11 +1519,6 @@ __global__ void __launch_bounds__(64 * NWV, 1) k_conv_down_px(ConvArgs p) {
 #pragma unroll
   for (int i = 0; i < T * T; ++i) acc[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
-  // One pair of filters: multiply a and the pair's weights (at wc) into the accumulators.  Between
-  // the MFMAs: one request in GAP for the next pair's modules (into an; beyond the last pair the
-  // offsets are out of range and nothing is fetched), and the weights two taps ahead (at the end
-  // of the step those of the next pair, at wn), kept in a ring of three registers.
-  // Taps run in descending order, so module rows are first used in ascending order.
   // One pair of filters: multiply (a, b) into the accumulators.  Between the MFMAs: one request
   // in GAP for the next pair's modules (into an; beyond the last pair the offsets are out of range
   // and nothing is fetched) and one LDS read per tap for the next pair's weights (into bn).
