@@ -41,7 +41,8 @@ bool dn_defer_dot(cudamat* mat1, cudamat* mat2, cudamat* target, float beta, flo
 bool dn_pending_sample(rnd_struct* rnd, cudamat* mat, cudamat* target, int* err);
 // Sums along the rows, y = beta*y + alpha*rowsums(M) (M is h x w, leading dimension h), may be held back too
 // and launched together (dn_row_sum_jobs), and a product into C may wait for a second one into the same C
-// (dn_gemm_pair_sums, together with the sums); each with the bits of the separate launches.
+// (dn_gemm_pair_sums, together with the sums; a product that stays alone takes the sums along where its kernel
+// can, dn_gemm_sums); each with the bits of the separate launches.
 // fill_with_rand may be held back as well: greater_than_scalar(mask, p) and mult_elementwise(state, mask)
 // that follow it spell a dropout mask (deepnet/neuralnet.py:194-198) and run as one pass (dn_rng_dropmask).
 bool dn_defer_fill_rand(rnd_struct* rnd, cudamat* mat, int* err);
@@ -52,6 +53,8 @@ bool dn_row_sum_job_ok(const float* M, int h, int w);
 int dn_row_sum_jobs(const DnRowSumJob* jobs, int n);
 int dn_gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, const float* A, int lda, const float* B, int ldb,
             float beta, float* C, int ldc);
+int dn_gemm_sums(bool a_trans, bool b_trans, int M, int N, int K, float alpha, const float* A, int lda, const float* B, int ldb,
+                 float beta, float* C, int ldc, const DnRowSumJob* jobs, int njobs);
 int dn_gemm_pair_sums(bool a_trans, bool b_trans, int M, int N, int K, float alpha, const float* A, int lda, const float* B,
                       int ldb, float beta, float alpha2, const float* A2, int lda2, const float* B2, int ldb2, float* C, int ldc,
                       const DnRowSumJob* jobs, int njobs);

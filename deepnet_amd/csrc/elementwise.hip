@@ -525,10 +525,8 @@ static int run_stats() {
     return dn_gemm_pair_sums(ta, tb, p.m, p.n, p.k, p.alpha, p.a.data_device, p.a.size[0], p.b.data_device, p.b.size[0], p.beta,
                              p.alpha2, p.a2.data_device, p.a2.size[0], p.b2.data_device, p.b2.size[0], p.t.data_device,
                              p.t.size[0], jobs, n);
-  if (int e = dn_gemm(ta, tb, p.m, p.n, p.k, p.alpha, p.a.data_device, p.a.size[0], p.b.data_device, p.b.size[0], p.beta,
-                      p.t.data_device, p.t.size[0]))
-    return e;
-  return n > 0 ? dn_row_sum_jobs(jobs, n) : 0;
+  return dn_gemm_sums(ta, tb, p.m, p.n, p.k, p.alpha, p.a.data_device, p.a.size[0], p.b.data_device, p.b.size[0], p.beta,
+                      p.t.data_device, p.t.size[0], jobs, n);
 }
 
 // ---- the dropout mask: mask.fill_with_rand(); mask.greater_than(p); state.mult(mask)
@@ -674,16 +672,13 @@ bool dn_defer_row_sum(const float* M, float* y, int h, int w, float alpha, float
     if (overlap(q.M, (long long)q.h * q.w, y, h) || overlap(M, (long long)h * w, q.y, q.h)) fits = false;
   }
   if (fits && (mine >= 0 ? cnt[mine] >= 2 : nys >= 2)) fits = false;
-  // the first sum may join a pair of products that waits, unless it writes what they read or write,
-  // or reads what they write
-  if (g_nsums == 0 && g_acc.active && g_acc.paired) {
+  // a sum may join the product (or the pair of products) that waits, unless it writes what they read
+  // or write, or reads what they write
+  if (g_acc.active && (fits || g_nsums == 0)) {
     const cudamat* ops[5] = {&g_acc.t, &g_acc.a, &g_acc.b, &g_acc.a2, &g_acc.b2};
+    const int nops = g_acc.paired ? 5 : 3;
     fits = !overlap(M, (long long)h * w, g_acc.t.data_device, dn_len(&g_acc.t));
-    for (int i = 0; i < 5 && fits; ++i) fits = !overlap(y, h, ops[i]->data_device, dn_len(ops[i]));
-  } else if (g_nsums > 0 && g_acc.active && fits) {
-    const cudamat* ops[5] = {&g_acc.t, &g_acc.a, &g_acc.b, &g_acc.a2, &g_acc.b2};
-    fits = !overlap(M, (long long)h * w, g_acc.t.data_device, dn_len(&g_acc.t));
-    for (int i = 0; i < 5 && fits; ++i) fits = !overlap(y, h, ops[i]->data_device, dn_len(ops[i]));
+    for (int i = 0; i < nops && fits; ++i) fits = !overlap(y, h, ops[i]->data_device, dn_len(ops[i]));
   }
   if (!fits) dn_flush();
   g_sums[g_nsums++] = DnRowSumJob{M, y, h, w, alpha, beta};

@@ -798,9 +798,8 @@ __device__ __forceinline__ void tile16_load_tail(const float* __restrict__ P, un
 }
 
 template <bool A_KC, bool B_KC, int NW>
-__global__ void __launch_bounds__(NW * 64)
-k_gemm_tile16(const float* __restrict__ A, int lda, const float* __restrict__ B, int ldb, float* C, int ldc, int M, int N,
-              int K, float alpha, float beta, GemmEpilogue epi) {
+__device__ __forceinline__ void gemm_tile16_body(const float* __restrict__ A, int lda, const float* __restrict__ B, int ldb, float* C,
+                                                 int ldc, int M, int N, int K, float alpha, float beta, const GemmEpilogue& epi) {
   __shared__ float red[NW][4 * 64];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -865,6 +864,29 @@ k_gemm_tile16(const float* __restrict__ A, int lda, const float* __restrict__ B,
     if (epi.sample) gemm_draw_store(draw, ei, out, epi);
   }
   gemm_draw_idle_streams(tid, NW * 64, epi);
+}
+
+template <bool A_KC, bool B_KC, int NW>
+__global__ void __launch_bounds__(NW * 64)
+k_gemm_tile16(const float* __restrict__ A, int lda, const float* __restrict__ B, int ldb, float* C, int ldc, int M, int N,
+              int K, float alpha, float beta, GemmEpilogue epi) {
+  gemm_tile16_body<A_KC, B_KC, NW>(A, lda, B, ldb, C, ldc, M, N, K, alpha, beta, epi);
+}
+
+// A product and up to four sums along the rows (rowsum_jobs.h) in one launch: the rows of the grid
+// below gy are the blocks of the product, the workgroups behind them the row blocks of the sums
+// (a weight gradient and the bias gradient of the same layer: deepnet/edge.py:236-242,
+// layer.py:206-211).  Every workgroup runs the code it would run in the separate kernels.
+template <bool A_KC, bool B_KC, int NW>
+__global__ void __launch_bounds__(NW * 64)
+k_gemm_tile16_sums(const float* __restrict__ A, int lda, const float* __restrict__ B, int ldb, float* C, int ldc, int M, int N,
+                   int K, float alpha, float beta, GemmEpilogue epi, int gy, RowSumJobs J, int jblocks) {
+  if ((int)blockIdx.y < gy) {
+    gemm_tile16_body<A_KC, B_KC, NW>(A, lda, B, ldb, C, ldc, M, N, K, alpha, beta, epi);
+  } else {
+    const int b = ((int)blockIdx.y - gy) * (int)gridDim.x + (int)blockIdx.x;
+    if (b < jblocks) rows_sum_jobs_body(J, b);
+  }
 }
 
 // Short reductions (K <= 128) on 64 x 64 tiles: the whole K extent of a tile's two operands is
@@ -940,9 +962,9 @@ __device__ __forceinline__ void box_frag(const float* S, int row, int lk, int t,
   }
 }
 template <bool A_KC, bool B_KC>
-__global__ void __launch_bounds__(BOX_THREADS)
-k_gemm_box(const float* __restrict__ A, int lda, const float* __restrict__ B, int ldb, float* C, int ldc, int M, int N, int K,
-           float alpha, float beta, bool a_fast, bool b_fast, GemmEpilogue epi) {
+__device__ __forceinline__ void gemm_box_body(const float* __restrict__ A, int lda, const float* __restrict__ B, int ldb, float* C,
+                                              int ldc, int M, int N, int K, float alpha, float beta, bool a_fast, bool b_fast,
+                                              const GemmEpilogue& epi) {
   constexpr int A_FLOATS = A_KC ? 64 * BOX_PITCH_KC : BOX_K * BOX_PITCH_MC;
   constexpr int B_FLOATS = B_KC ? 64 * BOX_PITCH_KC : BOX_K * BOX_PITCH_MC;
   static_assert(A_FLOATS + B_FLOATS >= BOX_KW * 4096, "the partial tiles reuse the operands' space");
@@ -993,6 +1015,26 @@ k_gemm_box(const float* __restrict__ A, int lda, const float* __restrict__ B, in
     const int en = n0 + (tid >> 6) + 16 * u;
     const float sum = (lds[e] + lds[4096 + e]) + (lds[8192 + e] + lds[12288 + e]);
     if (en < N) C[(size_t)en * ldc + em] = gemm_finish((beta != 0.f ? beta * cold[u] : 0.f) + alpha * sum, em, epi);
+  }
+}
+
+template <bool A_KC, bool B_KC>
+__global__ void __launch_bounds__(BOX_THREADS)
+k_gemm_box(const float* __restrict__ A, int lda, const float* __restrict__ B, int ldb, float* C, int ldc, int M, int N, int K,
+           float alpha, float beta, bool a_fast, bool b_fast, GemmEpilogue epi) {
+  gemm_box_body<A_KC, B_KC>(A, lda, B, ldb, C, ldc, M, N, K, alpha, beta, a_fast, b_fast, epi);
+}
+
+// ... and beside the 1024-lane blocks of this kernel (the sums use the first 256 lanes of theirs)
+template <bool A_KC, bool B_KC>
+__global__ void __launch_bounds__(BOX_THREADS)
+k_gemm_box_sums(const float* __restrict__ A, int lda, const float* __restrict__ B, int ldb, float* C, int ldc, int M, int N, int K,
+                float alpha, float beta, bool a_fast, bool b_fast, GemmEpilogue epi, int gy, RowSumJobs J, int jblocks) {
+  if ((int)blockIdx.y < gy) {
+    gemm_box_body<A_KC, B_KC>(A, lda, B, ldb, C, ldc, M, N, K, alpha, beta, a_fast, b_fast, epi);
+  } else {
+    const int b = ((int)blockIdx.y - gy) * (int)gridDim.x + (int)blockIdx.x;
+    if (b < jblocks) rows_sum_jobs_body(J, b);
   }
 }
 
@@ -1061,6 +1103,14 @@ static void launch_gemm(bool a_kc, bool b_kc, dim3 grid, const float* A, int lda
 // Host-side dispatch shared with tests through dot().
 // epi: what to append to each output (bias / activation); *fused tells the caller whether
 // the launch could carry it (the split-K and empty-K paths cannot).
+// Sums along the rows that the next product may take along in its launch (dn_gemm_sums sets them;
+// the launch site that does so clears the count).
+static const RowSumJobs* g_side_jobs = nullptr;
+static int g_side_blocks = 0;
+static inline bool side_jobs_fit(const GemmEpilogue& epi) {
+  return g_side_blocks > 0 && g_side_jobs && !epi.bias && epi.act == GEMM_ACT_NONE && !epi.sample;
+}
+
 static int gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, const float* A, int lda, const float* B,
                 int ldb, float beta, float* C, int ldc, GemmEpilogue epi = GemmEpilogue{nullptr, GEMM_ACT_NONE, nullptr, nullptr, nullptr, nullptr, 0u},
                 bool* fused = nullptr, bool* sampled = nullptr) {
@@ -1110,10 +1160,22 @@ static int gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, co
 #define GEMM_BOX(AK, BK_)                                                                                        \
   hipLaunchKernelGGL((k_gemm_box<AK, BK_>), grid, dim3(BOX_THREADS), 0, dn_stream(), A, lda, B, ldb, C, ldc, M, N, K, alpha, \
                      beta, a_fast, b_fast, epi)
-    if (a_kc && b_kc) GEMM_BOX(true, true);
+#define GEMM_BOX_SUMS(AK, BK_)                                                                                    \
+  hipLaunchKernelGGL((k_gemm_box_sums<AK, BK_>), sgrid, dim3(BOX_THREADS), 0, dn_stream(), A, lda, B, ldb, C, ldc, M, N, K, \
+                     alpha, beta, a_fast, b_fast, epi, (int)grid.y, *g_side_jobs, g_side_blocks)
+    if (side_jobs_fit(epi)) {
+      const dim3 sgrid(grid.x, grid.y + (g_side_blocks + grid.x - 1) / grid.x);
+      if (a_kc && b_kc) GEMM_BOX_SUMS(true, true);
+      else if (a_kc) GEMM_BOX_SUMS(true, false);
+      else if (b_kc) GEMM_BOX_SUMS(false, true);
+      else GEMM_BOX_SUMS(false, false);
+      g_side_blocks = 0;                // taken along
+    }
+    else if (a_kc && b_kc) GEMM_BOX(true, true);
     else if (a_kc) GEMM_BOX(true, false);
     else if (b_kc) GEMM_BOX(false, true);
     else GEMM_BOX(false, false);
+#undef GEMM_BOX_SUMS
 #undef GEMM_BOX
     if (fused) *fused = true;
     return dn_launch_status();
@@ -1136,10 +1198,22 @@ static int gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, co
 #define GEMM_T16(AK, BK_)                                                                                  \
   hipLaunchKernelGGL((k_gemm_tile16<AK, BK_, 4>), grid, dim3(256), 0, dn_stream(), A, lda, B, ldb, C, ldc, M, N, K, \
                      alpha, beta, epi)
-    if (a_kc && b_kc) GEMM_T16(true, true);
+#define GEMM_T16_SUMS(AK, BK_)                                                                                   \
+  hipLaunchKernelGGL((k_gemm_tile16_sums<AK, BK_, 4>), sgrid, dim3(256), 0, dn_stream(), A, lda, B, ldb, C, ldc, M, N, K, \
+                     alpha, beta, epi, (int)grid.y, *g_side_jobs, g_side_blocks)
+    if (side_jobs_fit(epi)) {
+      const dim3 sgrid(grid.x, grid.y + (g_side_blocks + grid.x - 1) / grid.x);
+      if (a_kc && b_kc) GEMM_T16_SUMS(true, true);
+      else if (a_kc) GEMM_T16_SUMS(true, false);
+      else if (b_kc) GEMM_T16_SUMS(false, true);
+      else GEMM_T16_SUMS(false, false);
+      g_side_blocks = 0;                // taken along
+    }
+    else if (a_kc && b_kc) GEMM_T16(true, true);
     else if (a_kc) GEMM_T16(true, false);
     else if (b_kc) GEMM_T16(false, true);
     else GEMM_T16(false, false);
+#undef GEMM_T16_SUMS
 #undef GEMM_T16
     if (fused) *fused = true;
     if (sampled) *sampled = epi.sample != nullptr;
@@ -1223,6 +1297,23 @@ static int gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, co
       hipLaunchKernelGGL(k_gemm_splitk_finish, dim3(blocks), dim3(256), 0, dn_stream(), partial, splits, C, ldc, M, N, alpha, beta);
   }
   return dn_launch_status();
+}
+
+// C = beta*C + alpha*op(A)*op(B) and the sums of `jobs`, which touch nothing the product reads or writes:
+// one launch where the product's kernel can take the sums along, otherwise the product, then the sums.
+int dn_gemm_sums(bool a_trans, bool b_trans, int M, int N, int K, float alpha, const float* A, int lda, const float* B, int ldb,
+                 float beta, float* C, int ldc, const DnRowSumJob* jobs, int njobs) {
+  RowSumJobs J = {};
+  const int jblocks = njobs > 0 ? rows_sum_jobs_table(jobs, njobs, &J) : 0;
+  if (jblocks < 0) return ERROR_GENERIC;
+  g_side_jobs = &J;
+  g_side_blocks = jblocks;
+  const int e = gemm(a_trans, b_trans, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc);
+  const bool taken = g_side_blocks == 0;
+  g_side_jobs = nullptr;
+  g_side_blocks = 0;
+  if (e) return e;
+  return (taken || njobs <= 0) ? 0 : dn_row_sum_jobs(jobs, njobs);
 }
 
 // Whether gemm() would hand this product to k_gemm_small<.., 4> (the conditions of its dispatch, in its order).

@@ -21,9 +21,11 @@ __device__ __forceinline__ float rowsum_finish(float yold, float s, float alpha,
   return __fmaf_rn(alpha, s, beta == 0.f ? 0.f : __fmul_rn(beta, yold));
 }
 
-// Workgroup `block` (256 lanes) of the jobs: 64 rows of one of the vectors.
+// Workgroup `block` of the jobs: 64 rows of one of the vectors, on the first 256 lanes (a larger
+// workgroup's other lanes only keep the barriers company).
 __device__ __forceinline__ void rows_sum_jobs_body(const RowSumJobs& J, int block) {
   __shared__ float sv[4][64];
+  const bool live = threadIdx.x < 256;
   const bool second = block >= J.bx0;                        // block-uniform
   const int bx = block - (second ? J.bx0 : 0);
   const int h = second ? J.h1 : J.h0, nj = second ? J.n1 : J.n0;
@@ -41,7 +43,7 @@ __device__ __forceinline__ void rows_sum_jobs_body(const RowSumJobs& J, int bloc
     const RowSumJob job = second ? (q ? J.b1 : J.b0) : (q ? J.a1 : J.a0);
     const int w = job.w;
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
-    if (row0 < h) {
+    if (live && row0 < h) {
       for (int j = wv * 4 + c; j < w; j += NW * 4 * U) {
         float4 v[U];
 #pragma unroll
@@ -57,7 +59,7 @@ __device__ __forceinline__ void rows_sum_jobs_body(const RowSumJobs& J, int bloc
     for (int o = 16; o < 64; o <<= 1)
 #pragma unroll
       for (int k = 0; k < 4; ++k) acc[k] += __shfl_xor(acc[k], o, 64);
-    if (c == 0) *reinterpret_cast<float4*>(&sv[wv][r * 4]) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+    if (live && c == 0) *reinterpret_cast<float4*>(&sv[wv][r * 4]) = make_float4(acc[0], acc[1], acc[2], acc[3]);
     __syncthreads();
     if (mine) {
       float s = sv[0][threadIdx.x];

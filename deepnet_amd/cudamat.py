@@ -901,8 +901,9 @@ def set_deferred_epilogues(on):
     up-pass, same bits, same order of work.  Likewise the calls of a parameter update
     (deepnet/parameter.py:80-106) run as one pass, two `add_dot` calls of the same shape into one
     target as one launch, and up to four `add_sums(.., axis=1)` calls onto two vectors as one launch
-    (the statistics of cudamat/examples/rbm_cudamat.py:73-86).  On by default; returns the previous
-    setting."""
+    (the statistics of cudamat/examples/rbm_cudamat.py:73-86); an `add_dot` that stays alone takes the
+    `add_sums` calls that follow it along in its launch (the gradients of a layer, deepnet/edge.py:236-242,
+    layer.py:206-211).  On by default; returns the previous setting."""
     return bool(_cudamat.set_deferred_epilogues(1 if on else 0))
 
 

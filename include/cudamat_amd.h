@@ -289,7 +289,9 @@ int get_softmax_cross_entropy(cudamat* mat, cudamat* labels, cudamat* target, fl
  * A product with beta = 1 (add_dot, subtract_dot) of at most 128 terms waits for a second one of the
  * same shape into the same target, and up to four add_sum_by_axis calls along the rows onto at most two
  * vectors wait for each other (the statistics of cudamat/examples/rbm_cudamat.py:73-86: six calls, two
- * launches); same bits, call order kept wherever two calls touch the same memory.  fill_with_rand is held
+ * launches; a product that stays alone takes the sums along in its own launch where its kernel can: a weight
+ * gradient and the bias gradient of its layer, deepnet/edge.py:236-242, layer.py:206-211); same bits, call order
+ * kept wherever two calls touch the same memory.  fill_with_rand is held
  * back likewise: greater_than_scalar of that matrix in place and mult_elementwise of another matrix by it in
  * place (the dropout mask of deepnet/neuralnet.py:194-198) run with it as one pass, same draws and values.
  * set_deferred_epilogues(0) makes every call launch at once; returns the previous setting (default 1).

@@ -263,7 +263,7 @@ def test_same_bits_with_and_without_deferral(cm, seq, shape):
 # cudamat/examples/rbm_cudamat.py:73-86): W nv x nh, v / v2 nv x B, h / h2 nh x B, bv nv x 1, bh nh x 1
 
 STAT_SHAPES = [(784, 500, 100), (500, 784, 100), (33, 17, 5), (1024, 1024, 128), (100, 60, 128), (2048, 64, 16), (256, 512, 200),
-               (36, 40, 7), (4, 4, 2)]          # nv, nh, batch
+               (36, 40, 7), (4, 4, 2), (784, 1024, 128), (1024, 10, 128), (1280, 640, 64)]          # nv, nh, batch
 
 
 def stat_cd(cm, o):
@@ -344,7 +344,36 @@ def stat_sums_of_transposed_views(cm, o):
     o.bh.add_sums(o.hT.T, axis=1, mult=0.5); o.bh.add_sums(o.h2, axis=1, mult=-0.5)      # hT is B x nh
 
 
-STATS = [stat_cd, stat_cd_subtract_dot, stat_pair_then_read, stat_single_then_read, stat_three_products, stat_products_into_two_targets,
+# a weight gradient and the bias gradient of the same layer (deepnet/edge.py:236-242, layer.py:206-211): one
+# product with the sums that follow it
+def stat_gradient(cm, o):
+    o.W.add_dot(o.v, o.h.T); o.bh.add_sums(o.h, axis=1)
+
+
+def stat_gradient_two_sums(cm, o):
+    o.W.add_dot(o.v, o.h.T, mult=0.5); o.bv.add_sums(o.v, axis=1); o.bh.add_sums(o.h, axis=1, mult=0.25)
+
+
+def stat_gradient_sum_reads_the_target(cm, o):
+    o.W.add_dot(o.v, o.h.T, mult=0.5); o.bv.add_sums(o.W, axis=1)
+
+
+def stat_gradient_sum_into_an_operand(cm, o):
+    col = o.v.slice(0, 1)
+    o.W.add_dot(o.v, o.h.T, mult=0.5); col.add_sums(o.v2, axis=1); o.W.add_dot(o.v, o.h2.T)
+
+
+def stat_gradient_then_second_product(cm, o):
+    o.W.add_dot(o.v, o.h.T, mult=0.5); o.bh.add_sums(o.h, axis=1); o.W.add_dot(o.v2, o.h2.T, mult=-0.5); o.bh.add_sums(o.h2, axis=1)
+
+
+def stat_gradients_of_two_layers(cm, o):
+    o.W.add_dot(o.v, o.h.T); o.bh.add_sums(o.h, axis=1); o.W2t.add_dot(o.h2, o.v2.T); o.bv.add_sums(o.v2, axis=1)
+    return o.bv.asarray().view(np.uint32).copy()
+
+
+STATS = [stat_gradient, stat_gradient_two_sums, stat_gradient_sum_reads_the_target, stat_gradient_sum_into_an_operand,
+         stat_gradient_then_second_product, stat_gradients_of_two_layers, stat_cd, stat_cd_subtract_dot, stat_pair_then_read, stat_single_then_read, stat_three_products, stat_products_into_two_targets,
          stat_second_product_reads_the_target, stat_overwriting_product_after_accumulating, stat_transposed_operands,
          stat_three_sums_on_one_vector, stat_sums_on_three_vectors, stat_sum_of_a_queued_result, stat_sum_into_a_queued_source,
          stat_sums_other_axis_in_between, stat_sums_then_read, stat_sum_with_assignment, stat_sums_of_transposed_views]
