@@ -385,7 +385,8 @@ DN_BINARY(apply_sin_deriv, check_binary, FSinDeriv{})
 DN_BINARY(apply_cos_deriv, check_binary, FCosDeriv{})
 DN_BINARY(apply_logistic_deriv, check_binary, FLogisticDeriv{})
 DN_BINARY(apply_tanh_deriv, check_binary, FTanhDeriv{})
-DN_BINARY(apply_rectified_linear_deriv, check_binary, FReluDeriv{})
+// (defined with the deferred epilogues below: a held-back product may take it along)
+int apply_rectified_linear_deriv(cudamat* mat1, cudamat* mat2, cudamat* target);
 DN_BINARY(apply_rectified_linear_smooth_deriv, check_binary, FReluSmoothDeriv{})
 DN_BINARY(apply_pow_matrix, check_binary_notrans, FPowMat{})
 DN_BINARY_PARAM(compute_cross_entropy, FCrossEntropy)
@@ -441,7 +442,8 @@ int add_diagonal(cudamat* mat, cudamat* vec, cudamat* target) {
 }  // extern "C"
 
 int dn_gemm_fused(bool a_trans, bool b_trans, int M, int N, int K, const float* A, int lda, const float* B, int ldb,
-                  float* C, int ldc, const float* bias, int act, bool* fused, const DnGemmSample* smp, bool* sampled);
+                  float* C, int ldc, const float* bias, int act, bool* fused, const DnGemmSample* smp, bool* sampled,
+                  const float* gate);
 
 // ------------------------------------------------------------------ deferred epilogues
 // Every layer of deepnet computes its state as  dot -> add_col_vec -> apply_sigmoid (or
@@ -458,8 +460,8 @@ int dn_gemm_fused(bool a_trans, bool b_trans, int M, int N, int K, const float* 
 // in call order, and a sequence that does not continue costs one kernel as before.
 struct DnPending {
   bool active;
-  cudamat a, b, t, bias;
-  bool has_bias;
+  cudamat a, b, t, bias, gate;
+  bool has_bias, has_gate;
   int act;            // 0 none yet, 1 sigmoid (waiting for a possible sample)
 };
 static DnPending g_pend = {};
@@ -469,7 +471,7 @@ static bool g_defer_enabled = true;
 static void refresh_pending();      // tells the library whether anything is still held back
 
 static int dot_bias_act_impl(rnd_struct* rnd, cudamat* mat1, cudamat* mat2, cudamat* bias, cudamat* target,
-                             cudamat* sample, int act);
+                             cudamat* sample, int act, cudamat* gate = nullptr);
 
 // Launches the held-back sequence (with the sample, when one is given).
 static int run_pending(rnd_struct* rnd, cudamat* sample) {
@@ -478,7 +480,7 @@ static int run_pending(rnd_struct* rnd, cudamat* sample) {
   refresh_pending();
   const bool saved = g_no_defer;
   g_no_defer = true;
-  const int e = dot_bias_act_impl(rnd, &p.a, &p.b, p.has_bias ? &p.bias : nullptr, &p.t, sample, p.act);
+  const int e = dot_bias_act_impl(rnd, &p.a, &p.b, p.has_bias ? &p.bias : nullptr, &p.t, sample, p.act, p.has_gate ? &p.gate : nullptr);
   g_no_defer = saved;
   return e;
 }
@@ -606,6 +608,7 @@ bool dn_defer_dot(cudamat* mat1, cudamat* mat2, cudamat* target, float beta, flo
   g_pend.active = true;
   g_pend.a = *mat1; g_pend.b = *mat2; g_pend.t = *target;
   g_pend.has_bias = false;
+  g_pend.has_gate = false;
   g_pend.act = 0;
   dn_set_pending(true);
   return true;
@@ -738,6 +741,20 @@ int apply_tanh(cudamat* mat, cudamat* target) {
   }
   if (int e = check_unary(mat, target)) return e;
   return launch_ew<1>(mat->data_device, nullptr, target->data_device, dn_len(mat), FTanh{});
+}
+
+// deriv = dot(w, deriv_above); deriv.apply_rectified_linear_deriv(state): the backward pass of a layer of
+// rectified linear units (deepnet/neuralnet.py:203-222, layer.py:168-172) in the product's launch.
+int apply_rectified_linear_deriv(cudamat* mat1, cudamat* mat2, cudamat* target) {
+  if (pend_open() && g_pend.act == 0 && !g_pend.has_bias && pend_is(mat1) && pend_is(target) && mat2->on_device &&
+      !mat2->is_trans && mat2->size[0] == target->size[0] && mat2->size[1] == target->size[1] &&
+      !overlap(mat2->data_device, dn_len(mat2), target->data_device, dn_len(target))) {
+    g_pend.gate = *mat2;
+    g_pend.has_gate = true;
+    return run_pending(nullptr, nullptr);
+  }
+  if (int e = check_binary(mat1, mat2, target)) return e;
+  return launch_ew<2>(mat1->data_device, mat2->data_device, target->data_device, dn_len(mat1), FReluDeriv{});
 }
 
 int lower_bound_scalar(cudamat* mat, float val, cudamat* target) {
@@ -974,7 +991,7 @@ bool dn_pending_sample(rnd_struct* rnd, cudamat* mat, cudamat* target, int* err)
 // target = act(op(mat1) * op(mat2) + bias) and, with a generator and a sample matrix,
 // sample = (uniform < target), in as few launches as the shapes allow.
 static int dot_bias_act_impl(rnd_struct* rnd, cudamat* mat1, cudamat* mat2, cudamat* bias, cudamat* target,
-                             cudamat* sample, int act) {
+                             cudamat* sample, int act, cudamat* gate) {
   if (!mat1->on_device || !mat2->on_device || !target->on_device || (bias && !bias->on_device)) return ERROR_NOT_ON_DEVICE;
   if (target->is_trans || (bias && bias->is_trans)) return ERROR_TRANSPOSED;
   if (act < 0 || act > 3) return ERROR_UNSUPPORTED;
@@ -1001,7 +1018,7 @@ static int dot_bias_act_impl(rnd_struct* rnd, cudamat* mat1, cudamat* mat2, cuda
     if (try_sample) smp = DnGemmSample{sample->data_device, rnd->dev_mults, rnd->dev_words, rng_other(rnd->dev_words)};
     err = dn_gemm_fused(mat1->is_trans != 0, mat2->is_trans != 0, m, n, k, mat1->data_device, mat1->size[0],
                         mat2->data_device, mat2->size[0], target->data_device, m, bias ? bias->data_device : nullptr,
-                        act, &fused, try_sample ? &smp : nullptr, &sampled);
+                        act, &fused, try_sample ? &smp : nullptr, &sampled, gate ? gate->data_device : nullptr);
     if (!err && sampled) rng_publish(rnd);
   }
   if (err) return err;
@@ -1011,6 +1028,7 @@ static int dot_bias_act_impl(rnd_struct* rnd, cudamat* mat1, cudamat* mat2, cuda
     else if (act == 2) err = lower_bound_scalar(target, 0.f, target);
     else if (act == 3) err = apply_tanh(target, target);
     if (err) return err;
+    if (gate && (err = apply_rectified_linear_deriv(target, gate, target))) return err;
   }
   if (sample && !sampled) return sample_bernoulli(rnd, target, sample);
   return 0;

@@ -37,13 +37,16 @@ struct GemmEpilogue {
   const unsigned long long* words;
   unsigned long long* next;
   unsigned int total;            // M * N
+  const float* gate;             // an array laid out as C (or null): outputs are multiplied by (gate > 0 ? 1 : 0)
 };
 #define GEMM_SAMPLE_MAX_DRAWS 16
-__device__ __forceinline__ float gemm_finish(float v, int m, const GemmEpilogue& e) {
+// (m: the output's row; off: its offset in C)
+__device__ __forceinline__ float gemm_finish(float v, int m, size_t off, const GemmEpilogue& e) {
   if (e.bias) v = v + e.bias[m];
   if (e.act == GEMM_ACT_SIGMOID) v = dn_sigmoid(v);
   else if (e.act == GEMM_ACT_RELU) v = v < 0.f ? 0.f : v;
   else if (e.act == GEMM_ACT_TANH) v = dn_tanh(v);
+  if (e.gate) v = v * (e.gate[off] > 0.f ? 1.f : 0.f);      // apply_rectified_linear_deriv's expression
   return v;
 }
 // The generator's word and multiplier for element i, fetched early so that the loads are over
@@ -430,7 +433,7 @@ k_gemm(const float* __restrict__ A, int lda, const float* __restrict__ B, int ld
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           const int n = nb + 8 * (v >> 2) + (v & 3);
-          if (m < M && n < N) out[(size_t)n * ldo + m] = gemm_finish(beta * cold[i][v] + alpha * acc[j][i][v], m, epi);
+          if (m < M && n < N) out[(size_t)n * ldo + m] = gemm_finish(beta * cold[i][v] + alpha * acc[j][i][v], m, (size_t)n * ldo + m, epi);
         }
       }
     }
@@ -448,7 +451,7 @@ k_gemm(const float* __restrict__ A, int lda, const float* __restrict__ B, int ld
         if (n < N) {
           float* p = out + (size_t)n * ldo + m;
           if (split) *p = acc[j][i][v];
-          else *p = gemm_finish(alpha * acc[j][i][v], m, epi);
+          else *p = gemm_finish(alpha * acc[j][i][v], m, (size_t)n * ldo + m, epi);
         }
       }
     }
@@ -651,7 +654,7 @@ k_gemm_small(const float* __restrict__ A, int lda, const float* __restrict__ B, 
     const float sum = (red[0][e] + red[1][e]) + (red[2][e] + red[3][e]);
     const int nn = blockIdx.y * 32 + 8 * (v >> 2) + 4 * lk + (v & 3);
     if (m_ok && nn < N) {
-      const float out = gemm_finish(small_axpby(beta, cprev[u], alpha, sum), m, epi);
+      const float out = gemm_finish(small_axpby(beta, cprev[u], alpha, sum), m, (size_t)nn * ldc + m, epi);
       C[(size_t)nn * ldc + m] = out;
       if (epi.sample) {
         const unsigned int i = (unsigned int)nn * ldc + m;
@@ -859,7 +862,7 @@ __device__ __forceinline__ void gemm_tile16_body(const float* __restrict__ A, in
     float sum = red[0][tid];
 #pragma unroll
     for (int w = 1; w < NW; ++w) sum += red[w][tid];
-    const float out = gemm_finish((beta == 0.f ? 0.f : beta * cprev) + alpha * sum, em, epi);
+    const float out = gemm_finish((beta == 0.f ? 0.f : beta * cprev) + alpha * sum, em, (size_t)en * ldc + em, epi);
     C[(size_t)en * ldc + em] = out;
     if (epi.sample) gemm_draw_store(draw, ei, out, epi);
   }
@@ -1014,7 +1017,7 @@ __device__ __forceinline__ void gemm_box_body(const float* __restrict__ A, int l
     const int e = tid + BOX_THREADS * u;
     const int en = n0 + (tid >> 6) + 16 * u;
     const float sum = (lds[e] + lds[4096 + e]) + (lds[8192 + e] + lds[12288 + e]);
-    if (en < N) C[(size_t)en * ldc + em] = gemm_finish((beta != 0.f ? beta * cold[u] : 0.f) + alpha * sum, em, epi);
+    if (en < N) C[(size_t)en * ldc + em] = gemm_finish((beta != 0.f ? beta * cold[u] : 0.f) + alpha * sum, em, (size_t)en * ldc + em, epi);
   }
 }
 
@@ -1108,11 +1111,11 @@ static void launch_gemm(bool a_kc, bool b_kc, dim3 grid, const float* A, int lda
 static const RowSumJobs* g_side_jobs = nullptr;
 static int g_side_blocks = 0;
 static inline bool side_jobs_fit(const GemmEpilogue& epi) {
-  return g_side_blocks > 0 && g_side_jobs && !epi.bias && epi.act == GEMM_ACT_NONE && !epi.sample;
+  return g_side_blocks > 0 && g_side_jobs && !epi.bias && epi.act == GEMM_ACT_NONE && !epi.sample && !epi.gate;
 }
 
 static int gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, const float* A, int lda, const float* B,
-                int ldb, float beta, float* C, int ldc, GemmEpilogue epi = GemmEpilogue{nullptr, GEMM_ACT_NONE, nullptr, nullptr, nullptr, nullptr, 0u},
+                int ldb, float beta, float* C, int ldc, GemmEpilogue epi = GemmEpilogue{nullptr, GEMM_ACT_NONE, nullptr, nullptr, nullptr, nullptr, 0u, nullptr},
                 bool* fused = nullptr, bool* sampled = nullptr) {
   if (fused) *fused = false;
   if (sampled) *sampled = false;
@@ -1284,7 +1287,7 @@ static int gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, co
     if (!partial) return CUDA_ERROR;
   }
   dim3 grid(gx, gy, splits);
-  const GemmEpilogue none = {nullptr, GEMM_ACT_NONE, nullptr, nullptr, nullptr, nullptr, 0u};
+  const GemmEpilogue none = {nullptr, GEMM_ACT_NONE, nullptr, nullptr, nullptr, nullptr, 0u, nullptr};
   if (big) launch_gemm<2, 2>(a_kc, b_kc, grid, A, lda, B, ldb, C, ldc, M, N, K, kps, alpha, beta, partial, a_vec, b_vec, splits > 1 ? none : epi);
   else launch_gemm<1, 1>(a_kc, b_kc, grid, A, lda, B, ldb, C, ldc, M, N, K, kps, alpha, beta, partial, a_vec, b_vec, splits > 1 ? none : epi);
   if (fused) *fused = splits == 1;
@@ -1386,12 +1389,14 @@ int dn_gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, const 
   return gemm(a_trans, b_trans, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc);
 }
 
-// C = act(op(A)*op(B) + bias) for dot_bias_act(); *fused: whether the launch carried bias and act.
+// C = act(op(A)*op(B) + bias) [* (gate > 0)] for dot_bias_act(); *fused: whether the launch carried bias, act and gate
+// (gate, when given, is laid out as C with leading dimension ldc).
 // smp (may be null): the sample to draw in the same launch; *sampled says whether it was drawn
 // (then the generator's next words are in smp->next and the caller publishes them).
 int dn_gemm_fused(bool a_trans, bool b_trans, int M, int N, int K, const float* A, int lda, const float* B, int ldb,
-                  float* C, int ldc, const float* bias, int act, bool* fused, const DnGemmSample* smp, bool* sampled) {
-  GemmEpilogue epi = {bias, act, nullptr, nullptr, nullptr, nullptr, 0u};
+                  float* C, int ldc, const float* bias, int act, bool* fused, const DnGemmSample* smp, bool* sampled,
+                  const float* gate) {
+  GemmEpilogue epi = {bias, act, nullptr, nullptr, nullptr, nullptr, 0u, gate};
   const unsigned long long total = (unsigned long long)M * (unsigned long long)N;
   if (smp && ldc == M && total <= (unsigned long long)GEMM_SAMPLE_MAX_DRAWS * NUM_RND_STREAMS) {
     epi.sample = smp->sample;

@@ -238,7 +238,40 @@ def seq_fill_then_another_draw(cm, a, B, bias, other, T, S):
     S.fill_with_rand(); S.greater_than(0.5); other.sample_bernoulli()
 
 
-SEQS = [seq_fill_then_another_draw, seq_dropout, seq_dropout_after_a_layer, seq_dropout_mask_then_read, seq_dropout_into_another_target,
+# the backward pass of a layer of rectified linear units: deriv = dot(w, deriv_above);
+# deriv.apply_rectified_linear_deriv(state)  (deepnet/neuralnet.py:203-222, layer.py:168-172)
+def seq_relu_deriv(cm, a, B, bias, other, T, S):
+    cm.dot(a, B, target=T); T.apply_rectified_linear_deriv(other)
+
+
+def seq_relu_deriv_then_other_work(cm, a, B, bias, other, T, S):
+    cm.dot(a, B, target=T); T.apply_rectified_linear_deriv(other); T.mult(0.5); other.add(T)
+
+
+def seq_relu_deriv_into_another_target(cm, a, B, bias, other, T, S):
+    cm.dot(a, B, target=T); T.apply_rectified_linear_deriv(other, target=S)
+
+
+def seq_relu_deriv_by_itself(cm, a, B, bias, other, T, S):
+    cm.dot(a, B, target=T); T.apply_rectified_linear_deriv(T)
+
+
+def seq_relu_deriv_after_a_bias(cm, a, B, bias, other, T, S):
+    cm.dot(a, B, target=T); T.add_col_vec(bias); T.apply_rectified_linear_deriv(other)
+
+
+def seq_relu_deriv_of_another_matrix(cm, a, B, bias, other, T, S):
+    cm.dot(a, B, target=T); S.apply_rectified_linear_deriv(T); other.apply_rectified_linear_deriv(S)
+
+
+def seq_relu_deriv_with_special_values(cm, a, B, bias, other, T, S):
+    other.assign(0.0); S.assign(-0.0); other.subtract(S)                  # zeros of both signs in the gate
+    cm.dot(a, B, target=T); T.apply_rectified_linear_deriv(other)
+    S.assign(np.inf); cm.dot(a, B, target=T); T.apply_rectified_linear_deriv(S)
+
+
+SEQS = [seq_relu_deriv, seq_relu_deriv_then_other_work, seq_relu_deriv_into_another_target, seq_relu_deriv_by_itself,
+        seq_relu_deriv_after_a_bias, seq_relu_deriv_of_another_matrix, seq_relu_deriv_with_special_values, seq_fill_then_another_draw, seq_dropout, seq_dropout_after_a_layer, seq_dropout_mask_then_read, seq_dropout_into_another_target,
         seq_dropout_threshold_into_another_target, seq_dropout_mask_times_itself, seq_dropout_roles_exchanged,
         seq_fill_then_other_work, seq_dropout_of_special_values, seq_update_plain, seq_update_with_reset, seq_update_l2_l1_reset, seq_update_l2_only, seq_update_l1_only_twice,
         seq_update_not_spelled_scaled_gradient, seq_update_not_spelled_wrong_order, seq_update_not_spelled_no_gradient,
@@ -568,7 +601,7 @@ def _random_sequence(cm, rng_ops, pool, vecs, rows, n_ops):
     scal = lambda: float(np.float32(rng_ops.choice([0.0, 1.0, -1.0, 0.5, 0.9, -0.01, 2.0, 0.3])))
     reads = []
     for _ in range(n_ops):
-        op = rng_ops.integers(22)
+        op = rng_ops.integers(24)
         a, b, c = M(), M(), M()
         if op == 0: cm.dot(pool.A.T, pool.B, target=a)
         elif op == 1: a.add_dot(pool.A.T, pool.B, mult=scal())
@@ -591,6 +624,8 @@ def _random_sequence(cm, rng_ops, pool, vecs, rows, n_ops):
         elif op == 18: cm.tanh(a)
         elif op == 19: reads.append(_bits(a))
         elif op == 20: a.add_mult(b)               # factor 1: the gradient of an update
+        elif op == 22: a.apply_rectified_linear_deriv(b)
+        elif op == 23: a.apply_rectified_linear_deriv(b, target=c)
         else: V().add_sums(a, axis=1)
     return reads
 
