@@ -37,6 +37,9 @@ void dn_set_ext_flush_hook(void (*f)());   // the conv library's held-back calls
 void dn_set_ext_pending(bool on);
 void dn_flush_ext();
 bool dn_defer_enabled();                    // set_deferred_epilogues()
+void dn_refresh_pending();                  // recomputes whether anything is held back
+bool dn_softmax_held();                     // a softmax that waits for its loss and gradient (reduce.hip)
+void dn_softmax_flush();
 bool dn_defer_dot(cudamat* mat1, cudamat* mat2, cudamat* target, float beta, float alpha, int m, int n, int k, int* err);
 bool dn_pending_sample(rnd_struct* rnd, cudamat* mat, cudamat* target, int* err);
 // Sums along the rows, y = beta*y + alpha*rowsums(M) (M is h x w, leading dimension h), may be held back too

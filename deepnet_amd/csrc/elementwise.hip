@@ -469,6 +469,7 @@ static bool g_no_defer = false;      // the library is issuing the calls of a se
 static bool g_defer_enabled = true;
 
 static void refresh_pending();      // tells the library whether anything is still held back
+static bool held_besides_updates();
 
 static int dot_bias_act_impl(rnd_struct* rnd, cudamat* mat1, cudamat* mat2, cudamat* bias, cudamat* target,
                              cudamat* sample, int act, cudamat* gate = nullptr);
@@ -569,6 +570,7 @@ static void flush_pending() {
   if (queued_calls() > 0) run_queue(false);
   if (g_acc.active || g_nsums > 0) run_stats();
   if (g_drop.stage) run_drop(nullptr);
+  dn_softmax_flush();
   g_flushing = false;
   refresh_pending();
 }
@@ -816,9 +818,12 @@ static int g_ubn = 0;
 
 static bool update_ready() { return g_eqn > 0 && g_eq_ready; }
 static int batched_updates() { return g_ubn; }
-static void refresh_pending() {
-  dn_set_pending(g_pend.active || g_eqn > 0 || g_ubn > 0 || g_acc.active || g_nsums > 0 || g_drop.stage != 0);
+// anything held back besides complete updates that wait for more of their kind
+static bool held_besides_updates() {
+  return g_pend.active || g_eqn > 0 || g_acc.active || g_nsums > 0 || g_drop.stage != 0 || dn_softmax_held();
 }
+static void refresh_pending() { dn_set_pending(held_besides_updates() || g_ubn > 0); }
+void dn_refresh_pending() { refresh_pending(); }
 
 extern "C" int momentum_update_many(int count, cudamat** w, cudamat** w_delta, cudamat** gradient, const float* momentum,
                                     const float* l2_decay, const float* l1_decay, const float* epsilon, const int* flags);
@@ -926,7 +931,7 @@ int mult_by_scalar(cudamat* mat, float val, cudamat* target) {
     int e = 0;
     if (update_ready()) e = stash_ready(false);
     dn_flush_ext();
-    if (g_pend.active || g_eqn > 0 || g_acc.active || g_nsums > 0 || g_drop.stage != 0) dn_flush();
+    if (held_besides_updates()) dn_flush();
     if (e) return e;
     g_eq[0].kind = EQ_MULS; g_eq[0].dst = *mat; g_eq[0].src = *mat; g_eq[0].s = val;
     g_eqn = 1;

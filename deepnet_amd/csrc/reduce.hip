@@ -1448,10 +1448,94 @@ static int softmax_impl(const float* in, float* out, int w, int h, SoftmaxExtras
   return launch_cols(k_col_softmax<64>, k_col_softmax<256>, w, h, in, out, w, h, x);
 }
 
+}  // extern "C"
+
+// ---- softmax held back.  A softmax layer's loss is spelled  state.apply_softmax();
+// state.get_softmax_cross_entropy(labels, loss); state.apply_softmax_grad(labels, target=deriv)
+// (deepnet/softmax_layer.py:25-28, 40-62): the softmax does not launch at once, the loss and the
+// gradient of its result join it while they follow directly, and the three run as softmax_ce_grad's one
+// launch (same kernels, same bits).  Any other call launches what is held back first.
+struct PendSoftmax {
+  int stage;                      // 0 nothing, 1 the softmax waits, 2 ... and its loss
+  cudamat in, probs, labels, loss;
+  float tiny;
+};
+static PendSoftmax g_sm = {};
+
+bool dn_softmax_held() { return g_sm.stage != 0; }
+
+void dn_softmax_flush() {
+  if (g_sm.stage == 0) return;
+  const PendSoftmax p = g_sm;
+  g_sm.stage = 0;
+  dn_refresh_pending();
+  if (p.stage == 1) softmax_impl(p.in.data_device, p.probs.data_device, p.in.size[1], p.in.size[0]);
+  else softmax_impl(p.in.data_device, p.probs.data_device, p.in.size[1], p.in.size[0],
+                    SoftmaxExtras{p.labels.data_device, p.loss.data_device, nullptr, p.tiny});
+}
+
+static inline bool sm_overlap(const cudamat* a, const cudamat* b) {
+  const float *p = a->data_device, *q = b->data_device;
+  const long long np = dn_len(a), nq = dn_len(b);
+  return p < q + nq && q < p + np;
+}
+static inline bool sm_same(const cudamat* a, const cudamat* b) {
+  return a->data_device == b->data_device && a->size[0] == b->size[0] && a->size[1] == b->size[1] && !a->is_trans;
+}
+
+// (the arguments have passed the entry point's checks)
+static bool softmax_hold(cudamat* mat, cudamat* target) {
+  if (!dn_defer_enabled() || mat->size[0] <= 0 || mat->size[1] <= 0 || target->is_trans) return false;
+  if (mat->data_device != target->data_device && sm_overlap(mat, target)) return false;
+  dn_flush();                     // (what else is held back comes first)
+  g_sm.stage = 1;
+  g_sm.in = *mat; g_sm.probs = *target;
+  dn_set_pending(true);
+  return true;
+}
+
+// the loss of the held-back softmax: labels and loss are 1 x w vectors apart from everything else
+static bool softmax_join_loss(cudamat* mat, cudamat* labels, cudamat* target, float tiny) {
+  if (g_sm.stage != 1 || !dn_defer_enabled() || !sm_same(mat, &g_sm.probs)) return false;
+  const int w = mat->size[1];
+  if (!labels->on_device || !target->on_device || labels->size[0] != 1 || labels->size[1] != w || target->size[0] != 1 ||
+      target->size[1] != w)
+    return false;
+  for (const cudamat* m : {&g_sm.in, &g_sm.probs})
+    if (sm_overlap(labels, m) || sm_overlap(target, m)) return false;
+  if (sm_overlap(labels, target)) return false;
+  g_sm.labels = *labels; g_sm.loss = *target; g_sm.tiny = tiny;
+  g_sm.stage = 2;
+  return true;
+}
+
+// the gradient of the held-back softmax: launches the sequence
+static bool softmax_join_grad(cudamat* mat, cudamat* labels, cudamat* target, int* err) {
+  if (g_sm.stage == 0 || !dn_defer_enabled() || !sm_same(mat, &g_sm.probs)) return false;
+  const int h = mat->size[0], w = mat->size[1];
+  if (!labels->on_device || !target->on_device || target->is_trans || labels->size[0] != 1 || labels->size[1] != w ||
+      target->size[0] != h || target->size[1] != w || !dn_aligned16(target->data_device))
+    return false;
+  if (g_sm.stage == 2 && !(labels->data_device == g_sm.labels.data_device)) return false;
+  for (const cudamat* m : {&g_sm.in, &g_sm.probs})
+    if (sm_overlap(labels, m) || sm_overlap(target, m)) return false;
+  if (sm_overlap(labels, target) || (g_sm.stage == 2 && sm_overlap(target, &g_sm.loss))) return false;
+  const PendSoftmax p = g_sm;
+  g_sm.stage = 0;
+  dn_refresh_pending();
+  *err = softmax_impl(p.in.data_device, p.probs.data_device, w, h,
+                      SoftmaxExtras{labels->data_device, p.stage == 2 ? p.loss.data_device : nullptr, target->data_device,
+                                    p.stage == 2 ? p.tiny : 0.f});
+  return true;
+}
+
+extern "C" {
+
 int softmax(cudamat* mat, cudamat* target) {
   const int h = mat->size[0], w = mat->size[1];
   if (int e = check_axis_common(mat, target)) return e;
   if (target->size[0] != h || target->size[1] != w) return ERROR_INCOMPATIBLE_DIMENSIONS;
+  if (softmax_hold(mat, target)) return 0;
   return softmax_impl(mat->data_device, target->data_device, w, h);
 }
 
@@ -1473,6 +1557,7 @@ int softmax_ce_grad(cudamat* mat, cudamat* labels, cudamat* probs, cudamat* loss
 int softmax_overwrite(cudamat* mat) {
   if (!mat->on_device) return ERROR_NOT_ON_DEVICE;
   if (mat->is_trans) return ERROR_TRANSPOSED;
+  if (softmax_hold(mat, mat)) return 0;
   return softmax_impl(mat->data_device, mat->data_device, mat->size[1], mat->size[0]);
 }
 
@@ -1481,6 +1566,7 @@ int apply_softmax_grad(cudamat* mat, cudamat* labels, cudamat* target) {
   if (int e = check_axis_common(mat, target)) return e;
   if (target->size[0] != h || target->size[1] != w) return ERROR_INCOMPATIBLE_DIMENSIONS;
   if (labels->size[0] != 1 || labels->size[1] != w) return ERROR_INCOMPATIBLE_DIMENSIONS;
+  { int held = 0; if (softmax_join_grad(mat, labels, target, &held)) return held; }
   const long long n = (long long)h * w;
   if (n <= 0) return 0;
   if (n >= (1ll << 32)) return ERROR_UNSUPPORTED;
@@ -1517,6 +1603,7 @@ int get_softmax_cross_entropy(cudamat* mat, cudamat* labels, cudamat* target, fl
   if (int e = check_axis_common(mat, target)) return e;
   if (target->size[0] != 1 || target->size[1] != w) return ERROR_INCOMPATIBLE_DIMENSIONS;
   if (labels->size[0] != 1 || labels->size[1] != w) return ERROR_INCOMPATIBLE_DIMENSIONS;
+  if (softmax_join_loss(mat, labels, target, tiny)) return 0;
   if (w <= 0) return 0;
   hipLaunchKernelGGL(k_softmax_ce, dim3((w + 255) / 256), dim3(256), 0, dn_stream(), (const float*)mat->data_device,
                      (const float*)labels->data_device, target->data_device, w, h, tiny);

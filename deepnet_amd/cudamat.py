@@ -904,7 +904,8 @@ def set_deferred_epilogues(on):
     target as one launch, and up to four `add_sums(.., axis=1)` calls onto two vectors as one launch
     (the statistics of cudamat/examples/rbm_cudamat.py:73-86); an `add_dot` that stays alone takes the
     `add_sums` calls that follow it along in its launch (the gradients of a layer, deepnet/edge.py:236-242,
-    layer.py:206-211).  On by default; returns the previous setting."""
+    layer.py:206-211), and `apply_softmax` waits for the `get_softmax_cross_entropy` and `apply_softmax_grad`
+    of its result (deepnet/softmax_layer.py:25-62).  On by default; returns the previous setting."""
     return bool(_cudamat.set_deferred_epilogues(1 if on else 0))
 
 

@@ -296,6 +296,8 @@ int get_softmax_cross_entropy(cudamat* mat, cudamat* labels, cudamat* target, fl
  * kept wherever two calls touch the same memory.  fill_with_rand is held
  * back likewise: greater_than_scalar of that matrix in place and mult_elementwise of another matrix by it in
  * place (the dropout mask of deepnet/neuralnet.py:194-198) run with it as one pass, same draws and values.
+ * softmax / softmax_overwrite are held back too: get_softmax_cross_entropy and apply_softmax_grad (into another
+ * matrix) of the result join it and the three run as softmax_ce_grad's launch (deepnet/softmax_layer.py:25-62).
  * set_deferred_epilogues(0) makes every call launch at once; returns the previous setting (default 1).
  * launch_deferred() queues what is held back now and waits for nothing: for a caller that records its own
  * events on the library's stream (the NULL stream) or queues other work behind the library's. ---- */

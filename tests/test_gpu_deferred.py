@@ -270,7 +270,83 @@ def seq_relu_deriv_with_special_values(cm, a, B, bias, other, T, S):
     S.assign(np.inf); cm.dot(a, B, target=T); T.apply_rectified_linear_deriv(S)
 
 
-SEQS = [seq_relu_deriv, seq_relu_deriv_then_other_work, seq_relu_deriv_into_another_target, seq_relu_deriv_by_itself,
+# a softmax layer and its loss: state.apply_softmax(); state.get_softmax_cross_entropy(labels, loss);
+# state.apply_softmax_grad(labels, target=deriv)  (deepnet/softmax_layer.py:25-62)
+def _labels(cm, T, shift=0):
+    m, n = T.shape
+    return cm.CUDAMatrix(_f(((np.arange(n) * 7 + shift) % m).reshape(1, n))), cm.empty((1, n))
+
+
+def seq_softmax_loss_grad(cm, a, B, bias, other, T, S):
+    lab, loss = _labels(cm, T)
+    cm.dot(a, B, target=T); T.add_col_vec(bias); T.apply_softmax(); T.get_softmax_cross_entropy(lab, loss); T.apply_softmax_grad(lab, target=S)
+    return _bits(loss)
+
+
+def seq_softmax_grad_only(cm, a, B, bias, other, T, S):
+    lab, loss = _labels(cm, T)
+    cm.dot(a, B, target=T); T.apply_softmax(); T.apply_softmax_grad(lab, target=S)
+
+
+def seq_softmax_loss_only_then_read(cm, a, B, bias, other, T, S):
+    lab, loss = _labels(cm, T)
+    cm.dot(a, B, target=T); T.apply_softmax(); T.get_softmax_cross_entropy(lab, loss, tiny=1e-6)
+    return _bits(loss)
+
+
+def seq_softmax_alone_then_other_work(cm, a, B, bias, other, T, S):
+    cm.dot(a, B, target=T); T.apply_softmax(); other.add(T)
+
+
+def seq_softmax_grad_in_place(cm, a, B, bias, other, T, S):
+    lab, loss = _labels(cm, T)
+    cm.dot(a, B, target=T); T.apply_softmax(); T.get_softmax_cross_entropy(lab, loss); T.apply_softmax_grad(lab)
+    return _bits(loss)
+
+
+def seq_softmax_into_another_target(cm, a, B, bias, other, T, S):
+    lab, loss = _labels(cm, T)
+    cm.dot(a, B, target=T); T.apply_softmax(target=other); other.get_softmax_cross_entropy(lab, loss); other.apply_softmax_grad(lab, target=S)
+    return _bits(loss)
+
+
+def seq_softmax_loss_of_the_logits(cm, a, B, bias, other, T, S):
+    # the loss and the gradient are asked of the matrix the softmax read, not of its result: nothing joins
+    lab, loss = _labels(cm, T)
+    cm.dot(a, B, target=T); T.apply_sigmoid(); T.apply_softmax(target=other); T.get_softmax_cross_entropy(lab, loss); T.apply_softmax_grad(lab, target=S)
+    return _bits(loss)
+
+
+def seq_softmax_two_label_vectors(cm, a, B, bias, other, T, S):
+    lab, loss = _labels(cm, T)
+    lab2, _ = _labels(cm, T, shift=1)
+    cm.dot(a, B, target=T); T.apply_softmax(); T.get_softmax_cross_entropy(lab, loss); T.apply_softmax_grad(lab2, target=S)
+    return _bits(loss)
+
+
+def seq_softmax_correct_in_between(cm, a, B, bias, other, T, S):
+    lab, loss = _labels(cm, T)
+    hit = cm.empty(loss.shape)
+    cm.dot(a, B, target=T); T.apply_softmax(); T.get_softmax_correct(lab, hit); T.get_softmax_cross_entropy(lab, loss); T.apply_softmax_grad(lab, target=S)
+    return np.concatenate([_bits(loss).ravel(), _bits(hit).ravel()])
+
+
+def seq_softmax_then_scale_in_place(cm, a, B, bias, other, T, S):
+    # an in-place scale is held back itself and launches what waits before it
+    cm.dot(a, B, target=T); T.apply_softmax(); T.mult(0.9); other.mult(0.5); other.add_mult(T)
+
+
+def seq_softmax_gradient_over_the_logits_of_another(cm, a, B, bias, other, T, S):
+    # the gradient's target is the matrix a second softmax reads
+    lab, loss = _labels(cm, T)
+    cm.dot(a, B, target=T); T.apply_softmax(target=other); other.apply_softmax_grad(lab, target=T); T.apply_softmax(target=S)
+    S.get_softmax_cross_entropy(lab, loss)
+    return _bits(loss)
+
+
+SEQS = [seq_softmax_loss_grad, seq_softmax_grad_only, seq_softmax_loss_only_then_read, seq_softmax_alone_then_other_work,
+        seq_softmax_grad_in_place, seq_softmax_into_another_target, seq_softmax_loss_of_the_logits, seq_softmax_two_label_vectors,
+        seq_softmax_correct_in_between, seq_softmax_then_scale_in_place, seq_softmax_gradient_over_the_logits_of_another, seq_relu_deriv, seq_relu_deriv_then_other_work, seq_relu_deriv_into_another_target, seq_relu_deriv_by_itself,
         seq_relu_deriv_after_a_bias, seq_relu_deriv_of_another_matrix, seq_relu_deriv_with_special_values, seq_fill_then_another_draw, seq_dropout, seq_dropout_after_a_layer, seq_dropout_mask_then_read, seq_dropout_into_another_target,
         seq_dropout_threshold_into_another_target, seq_dropout_mask_times_itself, seq_dropout_roles_exchanged,
         seq_fill_then_other_work, seq_dropout_of_special_values, seq_update_plain, seq_update_with_reset, seq_update_l2_l1_reset, seq_update_l2_only, seq_update_l1_only_twice,
@@ -599,9 +675,12 @@ def _random_sequence(cm, rng_ops, pool, vecs, rows, n_ops):
     M = lambda: pool[rng_ops.integers(len(pool))]
     V = lambda: vecs[rng_ops.integers(len(vecs))]
     scal = lambda: float(np.float32(rng_ops.choice([0.0, 1.0, -1.0, 0.5, 0.9, -0.01, 2.0, 0.3])))
+    m_, n_ = pool[0].shape
+    lab, loss = cm.CUDAMatrix(_f(((np.arange(n_) * 5) % m_).reshape(1, n_))), cm.empty((1, n_))
+    loss.assign(0)
     reads = []
     for _ in range(n_ops):
-        op = rng_ops.integers(24)
+        op = rng_ops.integers(27)
         a, b, c = M(), M(), M()
         if op == 0: cm.dot(pool.A.T, pool.B, target=a)
         elif op == 1: a.add_dot(pool.A.T, pool.B, mult=scal())
@@ -626,7 +705,11 @@ def _random_sequence(cm, rng_ops, pool, vecs, rows, n_ops):
         elif op == 20: a.add_mult(b)               # factor 1: the gradient of an update
         elif op == 22: a.apply_rectified_linear_deriv(b)
         elif op == 23: a.apply_rectified_linear_deriv(b, target=c)
+        elif op == 24: a.apply_softmax() if rng_ops.integers(2) else a.apply_softmax(target=b)
+        elif op == 25: a.get_softmax_cross_entropy(lab, loss)
+        elif op == 26: a.apply_softmax_grad(lab, target=b)
         else: V().add_sums(a, axis=1)
+    reads.append(_bits(loss))
     return reads
 
 
