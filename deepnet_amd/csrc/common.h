@@ -50,9 +50,10 @@ bool dn_pending_sample(rnd_struct* rnd, cudamat* mat, cudamat* target, int* err)
 // that follow it spell a dropout mask (deepnet/neuralnet.py:194-198) and run as one pass (dn_rng_dropmask).
 bool dn_defer_fill_rand(rnd_struct* rnd, cudamat* mat, int* err);
 int dn_rng_dropmask(rnd_struct* rnd, float* mask, float* state, size_t n, float p);
-struct DnRowSumJob { const float* M; float* y; int h, w; float alpha, beta; };
+struct DnRowSumJob { const float* M; float* y; int h, w; float alpha, beta; int scalar; };   // scalar: dn_row_sum_job_kind() == 2
 bool dn_defer_row_sum(const float* M, float* y, int h, int w, float alpha, float beta, int* err);
-bool dn_row_sum_job_ok(const float* M, int h, int w);
+bool dn_row_sum_job_ok(const float* M, int h, int w);     // kind 1
+int dn_row_sum_job_kind(const float* M, int h, int w);    // 0: not as a job, 1: 16-byte loads of four rows, 2: one row per lane
 int dn_row_sum_jobs(const DnRowSumJob* jobs, int n);
 int dn_gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, const float* A, int lda, const float* B, int ldb,
             float beta, float* C, int ldc);

@@ -658,7 +658,8 @@ int mult_elementwise(cudamat* mat1, cudamat* mat2, cudamat* target) {
 
 bool dn_defer_row_sum(const float* M, float* y, int h, int w, float alpha, float beta, int* err) {
   *err = 0;
-  if (g_no_defer || !g_defer_enabled || beta != 1.f || !dn_row_sum_job_ok(M, h, w)) return false;
+  const int kind = (g_no_defer || !g_defer_enabled || beta != 1.f) ? 0 : dn_row_sum_job_kind(M, h, w);
+  if (kind == 0) return false;
   if (overlap(M, (long long)h * w, y, h)) return false;
   // does the call join what is queued?  At most two vectors with two sums each; no vector may share
   // memory with another one or with a matrix that a queued sum reads (the order of the launches
@@ -686,7 +687,7 @@ bool dn_defer_row_sum(const float* M, float* y, int h, int w, float alpha, float
     for (int i = 0; i < nops && fits; ++i) fits = !overlap(y, h, ops[i]->data_device, dn_len(ops[i]));
   }
   if (!fits) dn_flush();
-  g_sums[g_nsums++] = DnRowSumJob{M, y, h, w, alpha, beta};
+  g_sums[g_nsums++] = DnRowSumJob{M, y, h, w, alpha, beta, kind == 2 ? 1 : 0};
   dn_set_pending(true);
   if (g_nsums == 4) *err = run_stats();
   return true;

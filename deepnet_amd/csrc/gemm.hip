@@ -1516,12 +1516,12 @@ int cd_update(cudamat* W, cudamat* bv, cudamat* bh, cudamat* v, cudamat* h, cuda
     DnRowSumJob jobs[4];
     int nj = 0;
     if (bv) {
-      jobs[nj++] = DnRowSumJob{v->data_device, bv->data_device, nv, B, eps, 1.f};
-      jobs[nj++] = DnRowSumJob{v2->data_device, bv->data_device, nv, B, -eps, 1.f};
+      jobs[nj++] = DnRowSumJob{v->data_device, bv->data_device, nv, B, eps, 1.f, 0};
+      jobs[nj++] = DnRowSumJob{v2->data_device, bv->data_device, nv, B, -eps, 1.f, 0};
     }
     if (bh) {
-      jobs[nj++] = DnRowSumJob{h->data_device, bh->data_device, nh, B, eps, 1.f};
-      jobs[nj++] = DnRowSumJob{h2->data_device, bh->data_device, nh, B, -eps, 1.f};
+      jobs[nj++] = DnRowSumJob{h->data_device, bh->data_device, nh, B, eps, 1.f, 0};
+      jobs[nj++] = DnRowSumJob{h2->data_device, bh->data_device, nh, B, -eps, 1.f, 0};
     }
     return dn_gemm_pair_sums(false, true, nv, nh, B, eps, v->data_device, nv, h->data_device, nh, 1.f, -eps, v2->data_device, nv,
                              h2->data_device, nh, W->data_device, nv, jobs, nj);

@@ -943,6 +943,13 @@ bool dn_row_sum_job_ok(const float* M, int h, int w) {
   if (h <= 0 || w <= 0 || !rows_one_ok(M, h, h) || rows_one_splits(h, w) != 1) return false;
   return w <= 64 || (long long)w * h <= (1 << 18);
 }
+// 1: as above; 2: rows that do not come in aligned groups of four, small enough for rows_reduce() to take
+// k_rows_stage1<false, ROW_SUM, 4, 4, false> with one column slice; 0: neither.
+int dn_row_sum_job_kind(const float* M, int h, int w) {
+  if (dn_row_sum_job_ok(M, h, w)) return 1;
+  if (h <= 0 || w <= 0 || rows_one_ok(M, h, h)) return 0;
+  return (long long)w * h <= (1 << 18) ? 2 : 0;
+}
 
 // jobs in call order: at most two different y, at most two jobs each (the caller has checked that)
 int dn_row_sum_jobs(const DnRowSumJob* jobs, int n) {

@@ -3,12 +3,13 @@
 // products (gemm.hip).  A job adds alpha * rowsums(M) to a vector y (M is h x w, leading dimension
 // h); up to two vectors with up to two jobs each, applied in the order given.  Every sum is taken
 // in the order of k_rows_one<ROW_SUM, 4, ., false> with one column slice (lane groups on
-// neighbouring columns, four wavefronts, fixed order in LDS) and finished by the same expression,
+// neighbouring columns, four wavefronts, fixed order in LDS; a job marked scalar: in the order of
+// k_rows_stage1<false, ROW_SUM, 4, 4, false>) and finished by the same expression,
 // so the results have the bits of the separate launches.
 #pragma once
 #include "common.h"
 
-struct RowSumJob { const float* M; int w; float alpha, beta; };
+struct RowSumJob { const float* M; int w; float alpha, beta; int scalar; };
 struct RowSumJobs {
   float* y0; float* y1;
   int h0, h1, n0, n1, bx0;
@@ -43,6 +44,35 @@ __device__ __forceinline__ void rows_sum_jobs_body(const RowSumJobs& J, int bloc
     const RowSumJob job = second ? (q ? J.b1 : J.b0) : (q ? J.a1 : J.a0);
     const int w = job.w;
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    if (job.scalar) {
+      // matrices whose rows do not come in aligned groups of four: a lane owns one row, in the order of
+      // k_rows_stage1<false, ROW_SUM, 4, 4, false> with one column slice (wavefront v the columns v, v + 4, ..,
+      // four in flight; a column past the end adds a zero)
+      const int srow = bx * 64 + lane;
+      float a1 = 0.f;
+      if (live && srow < h) {
+        for (int j = wv; j < w; j += 16) {
+          float v[4];
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            const int jj = j + 4 * u;
+            v[u] = jj < w ? job.M[(size_t)jj * h + srow] : 0.f;
+          }
+#pragma unroll
+          for (int u = 0; u < 4; ++u) a1 += v[u];
+        }
+      }
+      if (live) sv[wv][lane] = a1;
+      __syncthreads();
+      if (mine) {
+        float s = sv[0][threadIdx.x];
+#pragma unroll
+        for (int k = 1; k < NW; ++k) s += sv[k][threadIdx.x];
+        yv = rowsum_finish(yv, s, job.alpha, job.beta);
+      }
+      __syncthreads();
+      continue;
+    }
     if (live && row0 < h) {
       for (int j = wv * 4 + c; j < w; j += NW * 4 * U) {
         float4 v[U];
@@ -77,7 +107,7 @@ __device__ __forceinline__ void rows_sum_jobs_body(const RowSumJobs& J, int bloc
 static inline int rows_sum_jobs_table(const DnRowSumJob* jobs, int n, RowSumJobs* out) {
   RowSumJobs J = {};
   for (int i = 0; i < n; ++i) {
-    const RowSumJob rj = {jobs[i].M, jobs[i].w, jobs[i].alpha, jobs[i].beta};
+    const RowSumJob rj = {jobs[i].M, jobs[i].w, jobs[i].alpha, jobs[i].beta, jobs[i].scalar};
     if (J.n0 == 0 || jobs[i].y == J.y0) {
       if (J.n0 >= 2) return -1;
       J.y0 = jobs[i].y; J.h0 = jobs[i].h;

@@ -372,7 +372,7 @@ def test_same_bits_with_and_without_deferral(cm, seq, shape):
 # cudamat/examples/rbm_cudamat.py:73-86): W nv x nh, v / v2 nv x B, h / h2 nh x B, bv nv x 1, bh nh x 1
 
 STAT_SHAPES = [(784, 500, 100), (500, 784, 100), (33, 17, 5), (1024, 1024, 128), (100, 60, 128), (2048, 64, 16), (256, 512, 200),
-               (36, 40, 7), (4, 4, 2), (784, 1024, 128), (1024, 10, 128), (1280, 640, 64)]          # nv, nh, batch
+               (36, 40, 7), (4, 4, 2), (784, 1024, 128), (1024, 10, 128), (1280, 640, 64), (1022, 10, 128), (66, 130, 31)]          # nv, nh, batch
 
 
 def stat_cd(cm, o):
