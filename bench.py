@@ -650,8 +650,8 @@ def main():
                                               'note': 'the 51 calls of the reference API; the library folds bias / activation calls into the '
                                                       'launch of the dot() they follow, the mult / add_mult calls of each parameter update '
                                                       'into one pass and fill_with_rand / greater_than / mult of a dropout mask into one pass '
-                                                      '(same bits), consecutive updates wait for each other and share a launch, a weight gradient takes the '
-                                                      'bias gradient that follows it along a backward product the apply_rectified_linear_deriv behind it, and the softmax its loss and gradient: 12 launches',
+                                                      '(same bits; behind a layer of rectified linear units in the layer\'s own launch), consecutive updates wait for each other and share a launch, a weight gradient takes the '
+                                                      'bias gradient that follows it along a backward product the apply_rectified_linear_deriv behind it, and the softmax its loss and gradient: 10 launches',
                                               'iters': 100, 'warmup': 10}
         cm.set_deferred_epilogues(False)
         t = time_loop(cm, mlp.step, 100, 10)

@@ -443,7 +443,7 @@ int add_diagonal(cudamat* mat, cudamat* vec, cudamat* target) {
 
 int dn_gemm_fused(bool a_trans, bool b_trans, int M, int N, int K, const float* A, int lda, const float* B, int ldb,
                   float* C, int ldc, const float* bias, int act, bool* fused, const DnGemmSample* smp, bool* sampled,
-                  const float* gate);
+                  const float* gate, int drop, float drop_p);
 
 // ------------------------------------------------------------------ deferred epilogues
 // Every layer of deepnet computes its state as  dot -> add_col_vec -> apply_sigmoid (or
@@ -470,9 +470,10 @@ static bool g_defer_enabled = true;
 
 static void refresh_pending();      // tells the library whether anything is still held back
 static bool held_besides_updates();
+static inline bool pend_is(const cudamat* x);
 
 static int dot_bias_act_impl(rnd_struct* rnd, cudamat* mat1, cudamat* mat2, cudamat* bias, cudamat* target,
-                             cudamat* sample, int act, cudamat* gate = nullptr);
+                             cudamat* sample, int act, cudamat* gate = nullptr, bool drop = false, float drop_p = 0.f);
 
 // Launches the held-back sequence (with the sample, when one is given).
 static int run_pending(rnd_struct* rnd, cudamat* sample) {
@@ -536,6 +537,7 @@ static int run_stats() {
 // (deepnet/neuralnet.py:194-198) as one pass over the generator's streams.
 struct PendDrop {
   int stage;            // 0 nothing, 1 fill_with_rand held back, 2 ... and its threshold
+  bool with_pend;       // ... behind a held-back product with max(x, 0), whose target the mask may be meant for
   rnd_struct* rnd;
   cudamat mask;
   float p;
@@ -619,8 +621,19 @@ bool dn_defer_dot(cudamat* mat1, cudamat* mat2, cudamat* target, float beta, flo
 bool dn_defer_fill_rand(rnd_struct* rnd, cudamat* mat, int* err) {
   *err = 0;
   if (g_no_defer || !g_defer_enabled || mat->is_trans || dn_len(mat) <= 0) return false;
-  dn_flush();
+  // behind a product with max(x, 0) that waits (and nothing else does): a mask of its target's shape, apart from
+  // its operands, may turn out to be its dropout mask; both wait then
+  bool with = g_pend.active && g_pend.act == 2 && !g_pend.has_gate && queued_calls() == 0 && batched_updates() == 0 && !g_acc.active && g_nsums == 0 &&
+              g_drop.stage == 0 && !dn_softmax_held() && rnd && rnd->dev_mults && rnd->dev_words &&
+              mat->size[0] == g_pend.t.size[0] && mat->size[1] == g_pend.t.size[1];
+  if (with) {
+    const cudamat* ops[4] = {&g_pend.t, &g_pend.a, &g_pend.b, &g_pend.bias};
+    for (int i = 0; i < (g_pend.has_bias ? 4 : 3) && with; ++i)
+      with = !overlap(mat->data_device, dn_len(mat), ops[i]->data_device, dn_len(ops[i]));
+  }
+  if (!with) dn_flush();
   g_drop.stage = 1;
+  g_drop.with_pend = with;
   g_drop.rnd = rnd;
   g_drop.mask = *mat;
   g_drop.p = 0.f;
@@ -648,8 +661,31 @@ int mult_elementwise(cudamat* mat1, cudamat* mat2, cudamat* target) {
   if (g_drop.stage == 2 && !g_no_defer && drop_mask_is(mat2) && mat1->on_device && !mat1->is_trans && target->on_device &&
       !target->is_trans && target->data_device == mat1->data_device && mat1->size[0] == mat2->size[0] &&
       mat1->size[1] == mat2->size[1] && target->size[0] == mat1->size[0] && target->size[1] == mat1->size[1] &&
-      !overlap(mat1->data_device, dn_len(mat1), mat2->data_device, dn_len(mat2)))
+      !overlap(mat1->data_device, dn_len(mat1), mat2->data_device, dn_len(mat2))) {
+    if (g_drop.with_pend && g_pend.active && g_pend.act == 2 && pend_is(mat1)) {
+      // the mask is for the product that waits: product, bias, max(x, 0), mask and masking in one launch
+      const PendDrop d = g_drop;
+      DnPending p = g_pend;
+      g_drop.stage = 0;
+      g_pend.active = false;
+      refresh_pending();
+      const bool saved = g_no_defer;
+      g_no_defer = true;
+      cudamat mask = d.mask;
+      const int e = dot_bias_act_impl(d.rnd, &p.a, &p.b, p.has_bias ? &p.bias : nullptr, &p.t, &mask, p.act, nullptr, true, d.p);
+      g_no_defer = saved;
+      return e;
+    }
+    if (g_pend.active) {              // (the product that waits is another matter: it comes first, by itself)
+      const PendDrop d = g_drop;
+      g_drop.stage = 0;
+      const int e = run_pending(nullptr, nullptr);
+      g_drop = d;
+      refresh_pending();
+      if (e) return e;
+    }
     return run_drop(mat1);
+  }
   if (int e = check_binary(mat1, mat2, target)) return e;
   return launch_ew<2>(mat1->data_device, mat2->data_device, target->data_device, dn_len(mat1), FMul{});
 }
@@ -762,8 +798,8 @@ int apply_rectified_linear_deriv(cudamat* mat1, cudamat* mat2, cudamat* target) 
 
 int lower_bound_scalar(cudamat* mat, float val, cudamat* target) {
   if (pend_open() && g_pend.act == 0 && val == 0.f && !signbit(val) && pend_is(mat) && pend_is(target)) {
-    g_pend.act = 2;
-    return run_pending(nullptr, nullptr);
+    g_pend.act = 2;                   // stays held back: a dropout mask for it may follow
+    return 0;
   }
   if (int e = check_unary_trans(mat, target)) return e;
   return launch_ew<1>(mat->data_device, nullptr, target->data_device, dn_len(mat), FLowerS{val});
@@ -996,8 +1032,9 @@ bool dn_pending_sample(rnd_struct* rnd, cudamat* mat, cudamat* target, int* err)
 
 // target = act(op(mat1) * op(mat2) + bias) and, with a generator and a sample matrix,
 // sample = (uniform < target), in as few launches as the shapes allow.
+// drop: the sample is a dropout mask instead, sample = (uniform > drop_p), and target is multiplied by it.
 static int dot_bias_act_impl(rnd_struct* rnd, cudamat* mat1, cudamat* mat2, cudamat* bias, cudamat* target,
-                             cudamat* sample, int act, cudamat* gate) {
+                             cudamat* sample, int act, cudamat* gate, bool drop, float drop_p) {
   if (!mat1->on_device || !mat2->on_device || !target->on_device || (bias && !bias->on_device)) return ERROR_NOT_ON_DEVICE;
   if (target->is_trans || (bias && bias->is_trans)) return ERROR_TRANSPOSED;
   if (act < 0 || act > 3) return ERROR_UNSUPPORTED;
@@ -1024,7 +1061,8 @@ static int dot_bias_act_impl(rnd_struct* rnd, cudamat* mat1, cudamat* mat2, cuda
     if (try_sample) smp = DnGemmSample{sample->data_device, rnd->dev_mults, rnd->dev_words, rng_other(rnd->dev_words)};
     err = dn_gemm_fused(mat1->is_trans != 0, mat2->is_trans != 0, m, n, k, mat1->data_device, mat1->size[0],
                         mat2->data_device, mat2->size[0], target->data_device, m, bias ? bias->data_device : nullptr,
-                        act, &fused, try_sample ? &smp : nullptr, &sampled, gate ? gate->data_device : nullptr);
+                        act, &fused, try_sample ? &smp : nullptr, &sampled, gate ? gate->data_device : nullptr,
+                        drop ? 1 : 0, drop_p);
     if (!err && sampled) rng_publish(rnd);
   }
   if (err) return err;
@@ -1036,7 +1074,9 @@ static int dot_bias_act_impl(rnd_struct* rnd, cudamat* mat1, cudamat* mat2, cuda
     if (err) return err;
     if (gate && (err = apply_rectified_linear_deriv(target, gate, target))) return err;
   }
-  if (sample && !sampled) return sample_bernoulli(rnd, target, sample);
+  if (sample && !sampled)
+    return drop ? dn_rng_dropmask(rnd, sample->data_device, target->data_device, (size_t)dn_len(target), drop_p)
+                : sample_bernoulli(rnd, target, sample);
   return 0;
 }
 

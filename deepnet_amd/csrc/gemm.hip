@@ -38,6 +38,8 @@ struct GemmEpilogue {
   unsigned long long* next;
   unsigned int total;            // M * N
   const float* gate;             // an array laid out as C (or null): outputs are multiplied by (gate > 0 ? 1 : 0)
+  int drop;                      // the draws make a dropout mask: sample = (uniform > drop_p), C = C * sample
+  float drop_p;
 };
 #define GEMM_SAMPLE_MAX_DRAWS 16
 // (m: the output's row; off: its offset in C)
@@ -67,6 +69,17 @@ __device__ __forceinline__ void gemm_draw_store(GemmDraw d, unsigned int i, floa
   for (unsigned int k = 0; k <= nd; ++k) w = mwc_step(w, d.mult);
   e.sample[i] = mwc_uniform(w) < p ? 1.f : 0.f;
   if (i + NUM_RND_STREAMS >= e.total) e.next[s] = w;
+}
+// The same draw as a dropout mask (fill_with_rand -> greater_than(drop_p), deepnet/neuralnet.py:194-198):
+// stores and returns (uniform > drop_p ? 1 : 0).
+__device__ __forceinline__ float gemm_draw_mask(GemmDraw d, unsigned int i, const GemmEpilogue& e) {
+  const unsigned int s = i % NUM_RND_STREAMS, nd = i / NUM_RND_STREAMS;
+  unsigned long long w = d.w;
+  for (unsigned int k = 0; k <= nd; ++k) w = mwc_step(w, d.mult);
+  const float mk = mwc_uniform(w) > e.drop_p ? 1.f : 0.f;
+  e.sample[i] = mk;
+  if (i + NUM_RND_STREAMS >= e.total) e.next[s] = w;
+  return mk;
 }
 // Streams without a draw (fewer outputs than streams) keep their word: one workgroup copies them.
 __device__ __forceinline__ void gemm_draw_idle_streams(int tid, int nthreads, const GemmEpilogue& e) {
@@ -654,12 +667,11 @@ k_gemm_small(const float* __restrict__ A, int lda, const float* __restrict__ B, 
     const float sum = (red[0][e] + red[1][e]) + (red[2][e] + red[3][e]);
     const int nn = blockIdx.y * 32 + 8 * (v >> 2) + 4 * lk + (v & 3);
     if (m_ok && nn < N) {
-      const float out = gemm_finish(small_axpby(beta, cprev[u], alpha, sum), m, (size_t)nn * ldc + m, epi);
+      float out = gemm_finish(small_axpby(beta, cprev[u], alpha, sum), m, (size_t)nn * ldc + m, epi);
+      const unsigned int i = (unsigned int)nn * ldc + m;
+      if (epi.sample && epi.drop) out = out * gemm_draw_mask(gemm_draw_fetch(i, true, epi), i, epi);
       C[(size_t)nn * ldc + m] = out;
-      if (epi.sample) {
-        const unsigned int i = (unsigned int)nn * ldc + m;
-        gemm_draw_store(gemm_draw_fetch(i, true, epi), i, out, epi);
-      }
+      if (epi.sample && !epi.drop) gemm_draw_store(gemm_draw_fetch(i, true, epi), i, out, epi);
     }
   }
   gemm_draw_idle_streams(tid, NW * 64, epi);
@@ -862,9 +874,10 @@ __device__ __forceinline__ void gemm_tile16_body(const float* __restrict__ A, in
     float sum = red[0][tid];
 #pragma unroll
     for (int w = 1; w < NW; ++w) sum += red[w][tid];
-    const float out = gemm_finish((beta == 0.f ? 0.f : beta * cprev) + alpha * sum, em, (size_t)en * ldc + em, epi);
+    float out = gemm_finish((beta == 0.f ? 0.f : beta * cprev) + alpha * sum, em, (size_t)en * ldc + em, epi);
+    if (epi.sample && epi.drop) out = out * gemm_draw_mask(draw, ei, epi);
     C[(size_t)en * ldc + em] = out;
-    if (epi.sample) gemm_draw_store(draw, ei, out, epi);
+    if (epi.sample && !epi.drop) gemm_draw_store(draw, ei, out, epi);
   }
   gemm_draw_idle_streams(tid, NW * 64, epi);
 }
@@ -1115,7 +1128,7 @@ static inline bool side_jobs_fit(const GemmEpilogue& epi) {
 }
 
 static int gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, const float* A, int lda, const float* B,
-                int ldb, float beta, float* C, int ldc, GemmEpilogue epi = GemmEpilogue{nullptr, GEMM_ACT_NONE, nullptr, nullptr, nullptr, nullptr, 0u, nullptr},
+                int ldb, float beta, float* C, int ldc, GemmEpilogue epi = GemmEpilogue{nullptr, GEMM_ACT_NONE, nullptr, nullptr, nullptr, nullptr, 0u, nullptr, 0, 0.f},
                 bool* fused = nullptr, bool* sampled = nullptr) {
   if (fused) *fused = false;
   if (sampled) *sampled = false;
@@ -1287,7 +1300,7 @@ static int gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, co
     if (!partial) return CUDA_ERROR;
   }
   dim3 grid(gx, gy, splits);
-  const GemmEpilogue none = {nullptr, GEMM_ACT_NONE, nullptr, nullptr, nullptr, nullptr, 0u, nullptr};
+  const GemmEpilogue none = {nullptr, GEMM_ACT_NONE, nullptr, nullptr, nullptr, nullptr, 0u, nullptr, 0, 0.f};
   if (big) launch_gemm<2, 2>(a_kc, b_kc, grid, A, lda, B, ldb, C, ldc, M, N, K, kps, alpha, beta, partial, a_vec, b_vec, splits > 1 ? none : epi);
   else launch_gemm<1, 1>(a_kc, b_kc, grid, A, lda, B, ldb, C, ldc, M, N, K, kps, alpha, beta, partial, a_vec, b_vec, splits > 1 ? none : epi);
   if (fused) *fused = splits == 1;
@@ -1390,13 +1403,14 @@ int dn_gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, const 
 }
 
 // C = act(op(A)*op(B) + bias) [* (gate > 0)] for dot_bias_act(); *fused: whether the launch carried bias, act and gate
-// (gate, when given, is laid out as C with leading dimension ldc).
+// (gate, when given, is laid out as C with leading dimension ldc).  drop: the sample is a dropout mask,
+// (uniform > drop_p), and C is multiplied by it.
 // smp (may be null): the sample to draw in the same launch; *sampled says whether it was drawn
 // (then the generator's next words are in smp->next and the caller publishes them).
 int dn_gemm_fused(bool a_trans, bool b_trans, int M, int N, int K, const float* A, int lda, const float* B, int ldb,
                   float* C, int ldc, const float* bias, int act, bool* fused, const DnGemmSample* smp, bool* sampled,
-                  const float* gate) {
-  GemmEpilogue epi = {bias, act, nullptr, nullptr, nullptr, nullptr, 0u, gate};
+                  const float* gate, int drop, float drop_p) {
+  GemmEpilogue epi = {bias, act, nullptr, nullptr, nullptr, nullptr, 0u, gate, drop, drop_p};
   const unsigned long long total = (unsigned long long)M * (unsigned long long)N;
   if (smp && ldc == M && total <= (unsigned long long)GEMM_SAMPLE_MAX_DRAWS * NUM_RND_STREAMS) {
     epi.sample = smp->sample;

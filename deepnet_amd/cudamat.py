@@ -899,7 +899,8 @@ def set_deferred_epilogues(on):
     (`apply_sigmoid`, `lower_bound(0)`, `apply_tanh`) and a `sample_bernoulli` that follow it on its
     own target run in the product's epilogue - one launch for the three or four calls of a layer's
     up-pass, same bits, same order of work; `apply_rectified_linear_deriv(state)` of the product's target
-    directly behind it (a layer's backward pass) runs there too.  Likewise the calls of a parameter update
+    directly behind it (a layer's backward pass) runs there too, and so does the dropout mask of a layer of
+    rectified linear units (`mask.fill_with_rand(); mask.greater_than(p); state.mult(mask)`).  Likewise the calls of a parameter update
     (deepnet/parameter.py:80-106) run as one pass, two `add_dot` calls of the same shape into one
     target as one launch, and up to four `add_sums(.., axis=1)` calls onto two vectors as one launch
     (the statistics of cudamat/examples/rbm_cudamat.py:73-86); an `add_dot` that stays alone takes the

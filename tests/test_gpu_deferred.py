@@ -202,6 +202,34 @@ def seq_dropout_after_a_layer(cm, a, B, bias, other, T, S):
     other.fill_with_rand(); other.greater_than(0.7); T.mult(other)
 
 
+def seq_layer_mask_for_another_matrix(cm, a, B, bias, other, T, S):
+    # the mask that follows the layer is meant for another matrix: the layer comes first, then the masking
+    cm.dot(a, B, target=T); T.add_col_vec(bias); T.lower_bound(0); S.fill_with_rand(); S.greater_than(0.3); other.mult(S); other.add(T)
+
+
+def seq_layer_mask_unfinished(cm, a, B, bias, other, T, S):
+    cm.dot(a, B, target=T); T.lower_bound(0); S.fill_with_rand(); other.add(T); S.greater_than(0.5); T.mult(S)
+
+
+def seq_layer_mask_is_an_operand(cm, a, B, bias, other, T, S):
+    # the mask is drawn into the matrix the product reads: the product must see the old values
+    cm.dot(a, B, target=T); T.lower_bound(0); B.fill_with_rand(); B.greater_than(0.5); cm.dot(a, B, target=S)
+
+
+def seq_layer_mask_then_sample(cm, a, B, bias, other, T, S):
+    cm.dot(a, B, target=T); T.add_col_vec(bias); T.lower_bound(0); S.fill_with_rand(); S.greater_than(0.5); T.mult(S)
+    T.apply_sigmoid(); T.sample_bernoulli(target=other)
+
+
+def seq_two_layers_with_masks(cm, a, B, bias, other, T, S):
+    cm.dot(a, B, target=T); T.add_col_vec(bias); T.lower_bound(0); S.fill_with_rand(); S.greater_than(0.5); T.mult(S)
+    cm.dot(a, B, target=other); other.lower_bound(0); S.fill_with_rand(); S.greater_than(0.25); other.mult(S)
+
+
+def seq_layer_without_mask_then_draw(cm, a, B, bias, other, T, S):
+    cm.dot(a, B, target=T); T.lower_bound(0); other.fill_with_randn(); S.fill_with_rand()
+
+
 def seq_dropout_mask_then_read(cm, a, B, bias, other, T, S):
     S.fill_with_rand(); S.greater_than(0.25)
     return S.asarray().view(np.uint32).copy()
@@ -344,7 +372,8 @@ def seq_softmax_gradient_over_the_logits_of_another(cm, a, B, bias, other, T, S)
     return _bits(loss)
 
 
-SEQS = [seq_softmax_loss_grad, seq_softmax_grad_only, seq_softmax_loss_only_then_read, seq_softmax_alone_then_other_work,
+SEQS = [seq_layer_mask_for_another_matrix, seq_layer_mask_unfinished, seq_layer_mask_is_an_operand, seq_layer_mask_then_sample,
+        seq_two_layers_with_masks, seq_layer_without_mask_then_draw, seq_softmax_loss_grad, seq_softmax_grad_only, seq_softmax_loss_only_then_read, seq_softmax_alone_then_other_work,
         seq_softmax_grad_in_place, seq_softmax_into_another_target, seq_softmax_loss_of_the_logits, seq_softmax_two_label_vectors,
         seq_softmax_correct_in_between, seq_softmax_then_scale_in_place, seq_softmax_gradient_over_the_logits_of_another, seq_relu_deriv, seq_relu_deriv_then_other_work, seq_relu_deriv_into_another_target, seq_relu_deriv_by_itself,
         seq_relu_deriv_after_a_bias, seq_relu_deriv_of_another_matrix, seq_relu_deriv_with_special_values, seq_fill_then_another_draw, seq_dropout, seq_dropout_after_a_layer, seq_dropout_mask_then_read, seq_dropout_into_another_target,
@@ -680,7 +709,7 @@ def _random_sequence(cm, rng_ops, pool, vecs, rows, n_ops):
     loss.assign(0)
     reads = []
     for _ in range(n_ops):
-        op = rng_ops.integers(27)
+        op = rng_ops.integers(29)
         a, b, c = M(), M(), M()
         if op == 0: cm.dot(pool.A.T, pool.B, target=a)
         elif op == 1: a.add_dot(pool.A.T, pool.B, mult=scal())
@@ -708,6 +737,23 @@ def _random_sequence(cm, rng_ops, pool, vecs, rows, n_ops):
         elif op == 24: a.apply_softmax() if rng_ops.integers(2) else a.apply_softmax(target=b)
         elif op == 25: a.get_softmax_cross_entropy(lab, loss)
         elif op == 26: a.apply_softmax_grad(lab, target=b)
+        elif op == 27:      # a layer as deepnet spells it, with the variations that do and do not fold
+            cm.dot(pool.A.T, pool.B, target=a)
+            if rng_ops.integers(2): a.add_col_vec(V())
+            kind = rng_ops.integers(4)
+            if kind == 0: a.apply_sigmoid()
+            elif kind == 1: a.lower_bound(0)
+            elif kind == 2: cm.tanh(a)
+            if rng_ops.integers(2):
+                b.fill_with_rand()
+                if rng_ops.integers(4): b.greater_than(scal())
+                (a if rng_ops.integers(2) else c).mult(b)
+            elif rng_ops.integers(2): a.sample_bernoulli(target=b)
+        elif op == 28:      # an output layer and its loss
+            a.apply_softmax() if rng_ops.integers(2) else a.apply_softmax(target=b)
+            src = a if rng_ops.integers(4) else b
+            if rng_ops.integers(2): src.get_softmax_cross_entropy(lab, loss)
+            if rng_ops.integers(4): src.apply_softmax_grad(lab, target=c)
         else: V().add_sums(a, axis=1)
     reads.append(_bits(loss))
     return reads
