@@ -453,16 +453,19 @@ int dn_gemm_fused(bool a_trans, bool b_trans, int M, int N, int K, const float* 
 // time on.  The product kernels can carry the bias, the activation and the sample in their
 // epilogue (dot_bias_act), so dot() with alpha = 1, beta = 0 does not launch at once: it is held
 // back, and while the calls that follow are exactly the rest of that sequence on the product's
-// own target they are folded into it; the launch happens at the activation (tanh, lower_bound),
-// at the sample, or at the first call of any other kind (everything that queues work, hands out a
-// workspace, moves data or waits for the device passes through dn_flush()).  The arithmetic is
+// own target they are folded into it; the launch happens at tanh, at the sample, or at the first
+// call of any other kind (everything that queues work, hands out a workspace, moves data or waits
+// for the device passes through dn_flush()).  Behind lower_bound(0) the product waits once more: the
+// dropout mask of its target (fill_with_rand -> greater_than -> mult, neuralnet.py:194-198) is drawn
+// in its epilogue when it follows.  apply_rectified_linear_deriv(target, state) directly behind the
+// product (a layer's backward pass, neuralnet.py:203-222) is folded likewise.  The arithmetic is
 // that of the separate calls, bit for bit (tests/test_gpu_deferred.py), work reaches the stream
 // in call order, and a sequence that does not continue costs one kernel as before.
 struct DnPending {
   bool active;
   cudamat a, b, t, bias, gate;
   bool has_bias, has_gate;
-  int act;            // 0 none yet, 1 sigmoid (waiting for a possible sample)
+  int act;            // 0 none yet, 1 sigmoid (waiting for a possible sample), 2 max(x, 0) (waiting for a possible mask)
 };
 static DnPending g_pend = {};
 static bool g_no_defer = false;      // the library is issuing the calls of a sequence itself
