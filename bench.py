@@ -204,13 +204,14 @@ class MLP(object):
             self.gb[i].add_sums(self.delta[i], axis=1, mult=1.0 / B)
             if i > 0:
                 cm.dot(W[i], self.delta[i], target=self.delta[i - 1])
+                self.delta[i - 1].mult(self.mask[i - 1])                      # the layer's dropout mask (neuralnet.py:212-213)
                 self.delta[i - 1].apply_rectified_linear_deriv(act[i])
         for i in range(3):
             for p, d, g in ((W[i], self.dW[i], self.gW[i]), (b[i], self.db[i], self.gb[i])):
                 d.mult(self.mom); d.add_mult(g); p.add_mult(d, -self.lr); g.assign(0)
 
     def step_fused(self):
-        """The same step in 17 launches instead of 51 calls: this backend's extensions dot_bias_act,
+        """The same step in 17 launches instead of 53 calls: this backend's extensions dot_bias_act,
         softmax_ce_grad and momentum_update (all six parameters in one launch), and the one-call forms that the reference's own
         API has for what deepnet spells out in several (dropout() for fill_with_rand ->
         greater_than -> mult, dot() into the gradient for assign(0) -> add_dot, dot() with a
@@ -647,7 +648,7 @@ def main():
         t = time_loop(cm, mlp.step, 100, 10)
         secondary['mlp_784_1024_1024_10'] = {'steps_per_sec': round(1.0 / t, 1), 'us_per_step': round(t * 1e6, 1),
                                               'gemm_tflops': round(mlp.flops / t / 1e12, 3), 'batch': 128,
-                                              'note': 'the 51 calls of the reference API; the library folds bias / activation calls into the '
+                                              'note': 'the 53 calls of the reference API; the library folds bias / activation calls into the '
                                                       'launch of the dot() they follow, the mult / add_mult calls of each parameter update '
                                                       'into one pass and fill_with_rand / greater_than / mult of a dropout mask into one pass '
                                                       '(same bits; behind a layer of rectified linear units in the layer\'s own launch), consecutive updates wait for each other and share a launch, a weight gradient takes the '

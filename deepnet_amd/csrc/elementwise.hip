@@ -443,7 +443,7 @@ int add_diagonal(cudamat* mat, cudamat* vec, cudamat* target) {
 
 int dn_gemm_fused(bool a_trans, bool b_trans, int M, int N, int K, const float* A, int lda, const float* B, int ldb,
                   float* C, int ldc, const float* bias, int act, bool* fused, const DnGemmSample* smp, bool* sampled,
-                  const float* gate, int drop, float drop_p);
+                  const float* gate, int drop, float drop_p, const float* mul);
 
 // ------------------------------------------------------------------ deferred epilogues
 // Every layer of deepnet computes its state as  dot -> add_col_vec -> apply_sigmoid (or
@@ -463,8 +463,8 @@ int dn_gemm_fused(bool a_trans, bool b_trans, int M, int N, int K, const float* 
 // in call order, and a sequence that does not continue costs one kernel as before.
 struct DnPending {
   bool active;
-  cudamat a, b, t, bias, gate;
-  bool has_bias, has_gate;
+  cudamat a, b, t, bias, gate, mul;
+  bool has_bias, has_gate, has_mul;
   int act;            // 0 none yet, 1 sigmoid (waiting for a possible sample), 2 max(x, 0) (waiting for a possible mask)
 };
 static DnPending g_pend = {};
@@ -474,9 +474,11 @@ static bool g_defer_enabled = true;
 static void refresh_pending();      // tells the library whether anything is still held back
 static bool held_besides_updates();
 static inline bool pend_is(const cudamat* x);
+static inline bool pend_open();
 
 static int dot_bias_act_impl(rnd_struct* rnd, cudamat* mat1, cudamat* mat2, cudamat* bias, cudamat* target,
-                             cudamat* sample, int act, cudamat* gate = nullptr, bool drop = false, float drop_p = 0.f);
+                             cudamat* sample, int act, cudamat* gate = nullptr, bool drop = false, float drop_p = 0.f,
+                             cudamat* mul = nullptr);
 
 // Launches the held-back sequence (with the sample, when one is given).
 static int run_pending(rnd_struct* rnd, cudamat* sample) {
@@ -485,7 +487,8 @@ static int run_pending(rnd_struct* rnd, cudamat* sample) {
   refresh_pending();
   const bool saved = g_no_defer;
   g_no_defer = true;
-  const int e = dot_bias_act_impl(rnd, &p.a, &p.b, p.has_bias ? &p.bias : nullptr, &p.t, sample, p.act, p.has_gate ? &p.gate : nullptr);
+  const int e = dot_bias_act_impl(rnd, &p.a, &p.b, p.has_bias ? &p.bias : nullptr, &p.t, sample, p.act, p.has_gate ? &p.gate : nullptr,
+                                  false, 0.f, p.has_mul ? &p.mul : nullptr);
   g_no_defer = saved;
   return e;
 }
@@ -616,6 +619,7 @@ bool dn_defer_dot(cudamat* mat1, cudamat* mat2, cudamat* target, float beta, flo
   g_pend.a = *mat1; g_pend.b = *mat2; g_pend.t = *target;
   g_pend.has_bias = false;
   g_pend.has_gate = false;
+  g_pend.has_mul = false;
   g_pend.act = 0;
   dn_set_pending(true);
   return true;
@@ -626,7 +630,7 @@ bool dn_defer_fill_rand(rnd_struct* rnd, cudamat* mat, int* err) {
   if (g_no_defer || !g_defer_enabled || mat->is_trans || dn_len(mat) <= 0) return false;
   // behind a product with max(x, 0) that waits (and nothing else does): a mask of its target's shape, apart from
   // its operands, may turn out to be its dropout mask; both wait then
-  bool with = g_pend.active && g_pend.act == 2 && !g_pend.has_gate && queued_calls() == 0 && batched_updates() == 0 && !g_acc.active && g_nsums == 0 &&
+  bool with = g_pend.active && g_pend.act == 2 && !g_pend.has_gate && !g_pend.has_mul && queued_calls() == 0 && batched_updates() == 0 && !g_acc.active && g_nsums == 0 &&
               g_drop.stage == 0 && !dn_softmax_held() && rnd && rnd->dev_mults && rnd->dev_words &&
               mat->size[0] == g_pend.t.size[0] && mat->size[1] == g_pend.t.size[1];
   if (with) {
@@ -688,6 +692,15 @@ int mult_elementwise(cudamat* mat1, cudamat* mat2, cudamat* target) {
       if (e) return e;
     }
     return run_drop(mat1);
+  }
+  // deriv = dot(w, deriv_above); deriv.mult(mask) [; deriv.apply_rectified_linear_deriv(state)]: the backward pass
+  // of a layer with dropout (deepnet/neuralnet.py:203-222): the factor rides in the product's epilogue
+  if (pend_open() && g_pend.act == 0 && !g_pend.has_bias && !g_pend.has_gate && !g_pend.has_mul && g_drop.stage == 0 &&
+      pend_is(mat1) && pend_is(target) && mat2->on_device && !mat2->is_trans && mat2->size[0] == target->size[0] &&
+      mat2->size[1] == target->size[1] && !overlap(mat2->data_device, dn_len(mat2), target->data_device, dn_len(target))) {
+    g_pend.mul = *mat2;
+    g_pend.has_mul = true;            // stays held back: the derivative of the activation may follow
+    return 0;
   }
   if (int e = check_binary(mat1, mat2, target)) return e;
   return launch_ew<2>(mat1->data_device, mat2->data_device, target->data_device, dn_len(mat1), FMul{});
@@ -757,7 +770,7 @@ int launch_deferred(void) {
 }
 
 int add_col_vec(cudamat* mat, cudamat* vec, cudamat* target) {
-  if (pend_open() && !g_pend.has_bias && g_pend.act == 0 && pend_is(mat) && pend_is(target) && vec->on_device &&
+  if (pend_open() && !g_pend.has_bias && !g_pend.has_mul && g_pend.act == 0 && pend_is(mat) && pend_is(target) && vec->on_device &&
       !vec->is_trans && vec->size[0] == mat->size[0] && vec->size[1] == 1 && vec->data_device != mat->data_device) {
     g_pend.bias = *vec;
     g_pend.has_bias = true;
@@ -768,7 +781,7 @@ int add_col_vec(cudamat* mat, cudamat* vec, cudamat* target) {
 }
 
 int apply_sigmoid(cudamat* mat, cudamat* target) {
-  if (pend_open() && g_pend.act == 0 && pend_is(mat) && pend_is(target)) {
+  if (pend_open() && g_pend.act == 0 && !g_pend.has_mul && pend_is(mat) && pend_is(target)) {
     g_pend.act = 1;                   // stays held back: a sample of it may follow
     return 0;
   }
@@ -777,7 +790,7 @@ int apply_sigmoid(cudamat* mat, cudamat* target) {
 }
 
 int apply_tanh(cudamat* mat, cudamat* target) {
-  if (pend_open() && g_pend.act == 0 && pend_is(mat) && pend_is(target)) {
+  if (pend_open() && g_pend.act == 0 && !g_pend.has_mul && pend_is(mat) && pend_is(target)) {
     g_pend.act = 3;
     return run_pending(nullptr, nullptr);
   }
@@ -800,7 +813,7 @@ int apply_rectified_linear_deriv(cudamat* mat1, cudamat* mat2, cudamat* target) 
 }
 
 int lower_bound_scalar(cudamat* mat, float val, cudamat* target) {
-  if (pend_open() && g_pend.act == 0 && val == 0.f && !signbit(val) && pend_is(mat) && pend_is(target)) {
+  if (pend_open() && g_pend.act == 0 && !g_pend.has_mul && val == 0.f && !signbit(val) && pend_is(mat) && pend_is(target)) {
     g_pend.act = 2;                   // stays held back: a dropout mask for it may follow
     return 0;
   }
@@ -1037,7 +1050,7 @@ bool dn_pending_sample(rnd_struct* rnd, cudamat* mat, cudamat* target, int* err)
 // sample = (uniform < target), in as few launches as the shapes allow.
 // drop: the sample is a dropout mask instead, sample = (uniform > drop_p), and target is multiplied by it.
 static int dot_bias_act_impl(rnd_struct* rnd, cudamat* mat1, cudamat* mat2, cudamat* bias, cudamat* target,
-                             cudamat* sample, int act, cudamat* gate, bool drop, float drop_p) {
+                             cudamat* sample, int act, cudamat* gate, bool drop, float drop_p, cudamat* mul) {
   if (!mat1->on_device || !mat2->on_device || !target->on_device || (bias && !bias->on_device)) return ERROR_NOT_ON_DEVICE;
   if (target->is_trans || (bias && bias->is_trans)) return ERROR_TRANSPOSED;
   if (act < 0 || act > 3) return ERROR_UNSUPPORTED;
@@ -1065,7 +1078,7 @@ static int dot_bias_act_impl(rnd_struct* rnd, cudamat* mat1, cudamat* mat2, cuda
     err = dn_gemm_fused(mat1->is_trans != 0, mat2->is_trans != 0, m, n, k, mat1->data_device, mat1->size[0],
                         mat2->data_device, mat2->size[0], target->data_device, m, bias ? bias->data_device : nullptr,
                         act, &fused, try_sample ? &smp : nullptr, &sampled, gate ? gate->data_device : nullptr,
-                        drop ? 1 : 0, drop_p);
+                        drop ? 1 : 0, drop_p, mul ? mul->data_device : nullptr);
     if (!err && sampled) rng_publish(rnd);
   }
   if (err) return err;
@@ -1075,6 +1088,7 @@ static int dot_bias_act_impl(rnd_struct* rnd, cudamat* mat1, cudamat* mat2, cuda
     else if (act == 2) err = lower_bound_scalar(target, 0.f, target);
     else if (act == 3) err = apply_tanh(target, target);
     if (err) return err;
+    if (mul && (err = mult_elementwise(target, mul, target))) return err;
     if (gate && (err = apply_rectified_linear_deriv(target, gate, target))) return err;
   }
   if (sample && !sampled)

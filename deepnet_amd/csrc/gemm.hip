@@ -40,6 +40,7 @@ struct GemmEpilogue {
   const float* gate;             // an array laid out as C (or null): outputs are multiplied by (gate > 0 ? 1 : 0)
   int drop;                      // the draws make a dropout mask: sample = (uniform > drop_p), C = C * sample
   float drop_p;
+  const float* mul;              // an array laid out as C (or null): outputs are multiplied by it, before the gate
 };
 #define GEMM_SAMPLE_MAX_DRAWS 16
 // (m: the output's row; off: its offset in C)
@@ -48,6 +49,7 @@ __device__ __forceinline__ float gemm_finish(float v, int m, size_t off, const G
   if (e.act == GEMM_ACT_SIGMOID) v = dn_sigmoid(v);
   else if (e.act == GEMM_ACT_RELU) v = v < 0.f ? 0.f : v;
   else if (e.act == GEMM_ACT_TANH) v = dn_tanh(v);
+  if (e.mul) v = v * e.mul[off];                            // mult_elementwise's expression
   if (e.gate) v = v * (e.gate[off] > 0.f ? 1.f : 0.f);      // apply_rectified_linear_deriv's expression
   return v;
 }
@@ -1124,11 +1126,11 @@ static void launch_gemm(bool a_kc, bool b_kc, dim3 grid, const float* A, int lda
 static const RowSumJobs* g_side_jobs = nullptr;
 static int g_side_blocks = 0;
 static inline bool side_jobs_fit(const GemmEpilogue& epi) {
-  return g_side_blocks > 0 && g_side_jobs && !epi.bias && epi.act == GEMM_ACT_NONE && !epi.sample && !epi.gate;
+  return g_side_blocks > 0 && g_side_jobs && !epi.bias && epi.act == GEMM_ACT_NONE && !epi.sample && !epi.gate && !epi.mul;
 }
 
 static int gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, const float* A, int lda, const float* B,
-                int ldb, float beta, float* C, int ldc, GemmEpilogue epi = GemmEpilogue{nullptr, GEMM_ACT_NONE, nullptr, nullptr, nullptr, nullptr, 0u, nullptr, 0, 0.f},
+                int ldb, float beta, float* C, int ldc, GemmEpilogue epi = GemmEpilogue{nullptr, GEMM_ACT_NONE, nullptr, nullptr, nullptr, nullptr, 0u, nullptr, 0, 0.f, nullptr},
                 bool* fused = nullptr, bool* sampled = nullptr) {
   if (fused) *fused = false;
   if (sampled) *sampled = false;
@@ -1300,7 +1302,7 @@ static int gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, co
     if (!partial) return CUDA_ERROR;
   }
   dim3 grid(gx, gy, splits);
-  const GemmEpilogue none = {nullptr, GEMM_ACT_NONE, nullptr, nullptr, nullptr, nullptr, 0u, nullptr, 0, 0.f};
+  const GemmEpilogue none = {nullptr, GEMM_ACT_NONE, nullptr, nullptr, nullptr, nullptr, 0u, nullptr, 0, 0.f, nullptr};
   if (big) launch_gemm<2, 2>(a_kc, b_kc, grid, A, lda, B, ldb, C, ldc, M, N, K, kps, alpha, beta, partial, a_vec, b_vec, splits > 1 ? none : epi);
   else launch_gemm<1, 1>(a_kc, b_kc, grid, A, lda, B, ldb, C, ldc, M, N, K, kps, alpha, beta, partial, a_vec, b_vec, splits > 1 ? none : epi);
   if (fused) *fused = splits == 1;
@@ -1403,14 +1405,14 @@ int dn_gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, const 
 }
 
 // C = act(op(A)*op(B) + bias) [* (gate > 0)] for dot_bias_act(); *fused: whether the launch carried bias, act and gate
-// (gate, when given, is laid out as C with leading dimension ldc).  drop: the sample is a dropout mask,
+// (gate and mul, when given, are laid out as C with leading dimension ldc: C = C * mul * (gate > 0)).  drop: the sample is a dropout mask,
 // (uniform > drop_p), and C is multiplied by it.
 // smp (may be null): the sample to draw in the same launch; *sampled says whether it was drawn
 // (then the generator's next words are in smp->next and the caller publishes them).
 int dn_gemm_fused(bool a_trans, bool b_trans, int M, int N, int K, const float* A, int lda, const float* B, int ldb,
                   float* C, int ldc, const float* bias, int act, bool* fused, const DnGemmSample* smp, bool* sampled,
-                  const float* gate, int drop, float drop_p) {
-  GemmEpilogue epi = {bias, act, nullptr, nullptr, nullptr, nullptr, 0u, gate, drop, drop_p};
+                  const float* gate, int drop, float drop_p, const float* mul) {
+  GemmEpilogue epi = {bias, act, nullptr, nullptr, nullptr, nullptr, 0u, gate, drop, drop_p, mul};
   const unsigned long long total = (unsigned long long)M * (unsigned long long)N;
   if (smp && ldc == M && total <= (unsigned long long)GEMM_SAMPLE_MAX_DRAWS * NUM_RND_STREAMS) {
     epi.sample = smp->sample;

@@ -280,8 +280,9 @@ int get_softmax_cross_entropy(cudamat* mat, cudamat* labels, cudamat* target, fl
  * its launch back; add_col_vec(target, bias, target), then apply_sigmoid / apply_tanh /
  * lower_bound_scalar(.., 0, ..) in place, then sample_bernoulli(rnd, target, sample) are folded into that
  * launch while they follow it directly (the sequence of cudamat/examples/rbm_cudamat.py:46-70 and
- * deepnet/neuralnet.py:138-160); so is apply_rectified_linear_deriv(target, state, target) directly behind the
- * product (the backward pass of a layer of rectified linear units, deepnet/neuralnet.py:203-222).  Any other
+ * deepnet/neuralnet.py:138-160); so are mult_elementwise(target, mask, target) and
+ * apply_rectified_linear_deriv(target, state, target) directly behind the product (the backward pass of a layer
+ * of rectified linear units with dropout, deepnet/neuralnet.py:203-222).  Any other
  * call launches what is held back first, so work is queued in
  * call order and results are those of the separate launches, bit for bit.  Likewise an in-place
  * mult_by_scalar is held back and the add_mult / add_mult_sign calls of a parameter update

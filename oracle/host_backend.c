@@ -319,6 +319,7 @@ void hb_mlp_step(int nl, const int* sizes, int B, float lr, float mom, float** W
     hb_add_sums(delta[i], gb[i], out, B, 1, 1.f, invB);
     if (i > 0) {
       hb_gemm(0, 0, in, B, out, 1.f, W[i], in, delta[i], out, 0.f, delta[i - 1], in);
+      hb_mult(delta[i - 1], mask[i - 1], delta[i - 1], (size_t)in * B);      /* the layer's dropout mask (neuralnet.py:212-213) */
       hb_relu_deriv(delta[i - 1], act[i], delta[i - 1], (size_t)in * B);
     }
   }

@@ -272,6 +272,36 @@ def seq_relu_deriv(cm, a, B, bias, other, T, S):
     cm.dot(a, B, target=T); T.apply_rectified_linear_deriv(other)
 
 
+def seq_masked_relu_deriv(cm, a, B, bias, other, T, S):
+    # ... of a layer with dropout: deriv.mult(mask) in between (neuralnet.py:212-213)
+    S.fill_with_rand(); S.greater_than(0.5); cm.dot(a, B, target=T); T.mult(S); T.apply_rectified_linear_deriv(other)
+
+
+def seq_masked_deriv_without_activation(cm, a, B, bias, other, T, S):
+    cm.dot(a, B, target=T); T.mult(other); S.add(T)
+
+
+def seq_factor_then_bias(cm, a, B, bias, other, T, S):
+    # a bias behind the factor is not the layer's sequence: nothing may be reordered
+    cm.dot(a, B, target=T); T.mult(other); T.add_col_vec(bias); T.apply_sigmoid()
+
+
+def seq_factor_twice(cm, a, B, bias, other, T, S):
+    cm.dot(a, B, target=T); T.mult(other); T.mult(other); T.apply_rectified_linear_deriv(S)
+
+
+def seq_factor_is_the_target(cm, a, B, bias, other, T, S):
+    cm.dot(a, B, target=T); T.mult(T); T.apply_rectified_linear_deriv(other)
+
+
+def seq_factor_into_another_target(cm, a, B, bias, other, T, S):
+    cm.dot(a, B, target=T); T.mult(other, target=S); T.apply_rectified_linear_deriv(S)
+
+
+def seq_factor_then_lower_bound(cm, a, B, bias, other, T, S):
+    cm.dot(a, B, target=T); T.mult(other); T.lower_bound(0); S.fill_with_rand(); S.greater_than(0.5); T.mult(S)
+
+
 def seq_relu_deriv_then_other_work(cm, a, B, bias, other, T, S):
     cm.dot(a, B, target=T); T.apply_rectified_linear_deriv(other); T.mult(0.5); other.add(T)
 
@@ -372,7 +402,8 @@ def seq_softmax_gradient_over_the_logits_of_another(cm, a, B, bias, other, T, S)
     return _bits(loss)
 
 
-SEQS = [seq_layer_mask_for_another_matrix, seq_layer_mask_unfinished, seq_layer_mask_is_an_operand, seq_layer_mask_then_sample,
+SEQS = [seq_masked_relu_deriv, seq_masked_deriv_without_activation, seq_factor_then_bias, seq_factor_twice, seq_factor_is_the_target,
+        seq_factor_into_another_target, seq_factor_then_lower_bound, seq_layer_mask_for_another_matrix, seq_layer_mask_unfinished, seq_layer_mask_is_an_operand, seq_layer_mask_then_sample,
         seq_two_layers_with_masks, seq_layer_without_mask_then_draw, seq_softmax_loss_grad, seq_softmax_grad_only, seq_softmax_loss_only_then_read, seq_softmax_alone_then_other_work,
         seq_softmax_grad_in_place, seq_softmax_into_another_target, seq_softmax_loss_of_the_logits, seq_softmax_two_label_vectors,
         seq_softmax_correct_in_between, seq_softmax_then_scale_in_place, seq_softmax_gradient_over_the_logits_of_another, seq_relu_deriv, seq_relu_deriv_then_other_work, seq_relu_deriv_into_another_target, seq_relu_deriv_by_itself,
