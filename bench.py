@@ -161,6 +161,44 @@ class RBM(object):
         self.bh.add_sums(h, axis=1, mult=eps); self.bh.add_sums(h2, axis=1, mult=-eps)
 
 
+class RBMExample(object):
+    """The loop body of cudamat/examples/rbm_cudamat.py:46-89, call for call (28 library calls per
+    minibatch: momentum on the three update buffers, positive phase with its statistics, the hidden sample
+    spelled fill_with_rand -> less_than, negative phase with its statistics, three parameter updates and the
+    reconstruction error, which the script reads back every step), on synthetic binary data."""
+
+    def __init__(self, cm, num_vis=784, num_hid=500, batch_size=100, num_batches=20, seed=1):
+        rng = np.random.default_rng(seed)
+        f = lambda a: cm.CUDAMatrix(np.asarray(a, dtype=np.float32, order='F'))
+        self.cm, self.bs, self.nb, self.nv = cm, batch_size, num_batches, num_vis
+        self.epsilon, self.momentum = 0.1, 0.9
+        self.dev_dat = f(rng.random((num_vis, batch_size * num_batches)) < 0.13)
+        self.w_vh, self.w_v, self.w_h = f(0.1 * rng.standard_normal((num_vis, num_hid))), f(np.zeros((num_vis, 1))), \
+            f(-4. * np.ones((num_hid, 1)))
+        self.wu_vh, self.wu_v, self.wu_h = f(np.zeros((num_vis, num_hid))), f(np.zeros((num_vis, 1))), f(np.zeros((num_hid, 1)))
+        self.v, self.h, self.r = cm.empty((num_vis, batch_size)), cm.empty((num_hid, batch_size)), cm.empty((num_hid, batch_size))
+        self.batch = 0
+
+    def step(self):
+        cm, bs = self.cm, self.bs
+        w_vh, w_v, w_h, wu_vh, wu_v, wu_h, v, h, r = (self.w_vh, self.w_v, self.w_h, self.wu_vh, self.wu_v, self.wu_h,
+                                                      self.v, self.h, self.r)
+        batch = self.batch
+        self.batch = (batch + 1) % self.nb
+        v_true = self.dev_dat.slice(batch * bs, (batch + 1) * bs)
+        v.assign(v_true)
+        wu_vh.mult(self.momentum); wu_v.mult(self.momentum); wu_h.mult(self.momentum)
+        cm.dot(w_vh.T, v, target=h); h.add_col_vec(w_h); h.apply_sigmoid()
+        wu_vh.add_dot(v, h.T); wu_v.add_sums(v, axis=1); wu_h.add_sums(h, axis=1)
+        r.fill_with_rand(); r.less_than(h, target=h)
+        cm.dot(w_vh, h, target=v); v.add_col_vec(w_v); v.apply_sigmoid()
+        cm.dot(w_vh.T, v, target=h); h.add_col_vec(w_h); h.apply_sigmoid()
+        wu_vh.subtract_dot(v, h.T); wu_v.add_sums(v, axis=1, mult=-1.); wu_h.add_sums(h, axis=1, mult=-1.)
+        w_vh.add_mult(wu_vh, self.epsilon / bs); w_v.add_mult(wu_v, self.epsilon / bs); w_h.add_mult(wu_h, self.epsilon / bs)
+        v.subtract(v_true)
+        return v.euclid_norm() ** 2 / (self.nv * bs)
+
+
 class MLP(object):
     """784-1024-1024-10 ReLU net, softmax cross-entropy, dropout 0.5 on the hidden
     layers (fill_with_rand -> greater_than -> mult), momentum SGD; batch 128, seed 3.
@@ -631,6 +669,16 @@ def main():
         secondary['rbm_cd1_fused_extension'] = {
             'steps_per_sec': round(1.0 / t, 1), 'us_per_step': round(t * 1e6, 1),
             'note': 'same step with dot_bias_act, its sample, and the weight / bias statistics as one product (cd_update): extensions of this backend, not in the reference API; 4 launches instead of 16'}
+        ex = RBMExample(cm)
+        t = time_loop(cm, ex.step, 200, 20)
+        secondary['rbm_example_script'] = {
+            'steps_per_sec': round(1.0 / t, 1), 'us_per_step': round(t * 1e6, 1),
+            'note': 'the loop body of cudamat/examples/rbm_cudamat.py:46-89 call for call (28 calls, the reconstruction error read '
+                    'back every step as the script does): 15 launches'}
+        cm.set_deferred_epilogues(False)
+        t = time_loop(cm, ex.step, 200, 20)
+        cm.set_deferred_epilogues(True)
+        secondary['rbm_example_script']['us_per_step_every_call_a_launch'] = round(t * 1e6, 1)
         def recorded(step, iters, warm):
             # the step recorded once as a HIP graph (cm.Graph, an extension of this backend) and
             # replayed with one launch per step: same kernels, same results

@@ -50,6 +50,8 @@ bool dn_pending_sample(rnd_struct* rnd, cudamat* mat, cudamat* target, int* err)
 // that follow it spell a dropout mask (deepnet/neuralnet.py:194-198) and run as one pass (dn_rng_dropmask).
 bool dn_defer_fill_rand(rnd_struct* rnd, cudamat* mat, int* err);
 int dn_rng_dropmask(rnd_struct* rnd, float* mask, float* state, size_t n, float p);
+// ... and less_than(mask, probs, target = probs) behind it a Bernoulli sample that keeps its uniforms (dn_rng_bernoulli_keep).
+int dn_rng_bernoulli_keep(rnd_struct* rnd, float* uni, float* probs, size_t n);
 struct DnRowSumJob { const float* M; float* y; int h, w; float alpha, beta; int scalar; };   // scalar: dn_row_sum_job_kind() == 2
 bool dn_defer_row_sum(const float* M, float* y, int h, int w, float alpha, float beta, int* err);
 bool dn_row_sum_job_ok(const float* M, int h, int w);     // kind 1

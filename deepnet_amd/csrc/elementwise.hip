@@ -373,7 +373,8 @@ DN_SCALAR(add_scalar, check_unary, FAddS)
 
 // ---- binary
 DN_BINARY(less_than_eq, check_binary, FLe{})
-DN_BINARY(less_than, check_binary, FLt{})
+// (defined with the held-back fill_with_rand below: r.fill_with_rand(); r.less_than(h, target = h) is a sample)
+int less_than(cudamat* mat1, cudamat* mat2, cudamat* target);
 DN_BINARY(greater_than_eq, check_binary, FGe{})
 DN_BINARY(greater_than, check_binary, FGt{})
 DN_BINARY(upper_bound, check_binary, FUpper{})
@@ -662,6 +663,25 @@ int greater_than_scalar(cudamat* mat, float val, cudamat* target) {
   }
   if (int e = check_unary_trans(mat, target)) return e;
   return launch_ew<1>(mat->data_device, nullptr, target->data_device, dn_len(mat), FGtS{val});
+}
+
+// r.fill_with_rand(); r.less_than(h, target = h): the hidden sample as cudamat/examples/rbm_cudamat.py:63-65
+// spells it, in one pass over the generator's streams (h gets the sample, r the uniforms).
+int less_than(cudamat* mat1, cudamat* mat2, cudamat* target) {
+  if (g_drop.stage == 1 && !g_no_defer && drop_mask_is(mat1) && mat2->on_device && !mat2->is_trans && target->on_device &&
+      !target->is_trans && target->data_device == mat2->data_device && mat2->size[0] == mat1->size[0] &&
+      mat2->size[1] == mat1->size[1] && target->size[0] == mat2->size[0] && target->size[1] == mat2->size[1] &&
+      !overlap(mat1->data_device, dn_len(mat1), mat2->data_device, dn_len(mat2))) {
+    const PendDrop d = g_drop;
+    g_drop.stage = 0;
+    if (g_pend.active) {              // (a product that waits with the fill comes first, by itself)
+      if (int e = run_pending(nullptr, nullptr)) return e;
+    }
+    refresh_pending();
+    return dn_rng_bernoulli_keep(d.rnd, d.mask.data_device, mat2->data_device, (size_t)dn_len(mat2));
+  }
+  if (int e = check_binary(mat1, mat2, target)) return e;
+  return launch_ew<2>(mat1->data_device, mat2->data_device, target->data_device, dn_len(mat1), FLt{});
 }
 
 int mult_elementwise(cudamat* mat1, cudamat* mat2, cudamat* target) {

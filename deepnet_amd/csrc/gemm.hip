@@ -579,9 +579,9 @@ __device__ __forceinline__ float small_axpby(float beta, float c, float alpha, f
 }
 
 template <bool A_KC, bool B_KC, int NW>
-__global__ void __launch_bounds__(NW * 64)
-k_gemm_small(const float* __restrict__ A, int lda, const float* __restrict__ B, int ldb, float* C, int ldc, int M, int N,
-             int K, float alpha, float beta, bool a_vec, bool b_vec, GemmEpilogue epi) {
+__device__ __forceinline__ void gemm_small_body(const float* __restrict__ A, int lda, const float* __restrict__ B, int ldb, float* C,
+                                                int ldc, int M, int N, int K, float alpha, float beta, bool a_vec, bool b_vec,
+                                                const GemmEpilogue& epi) {
   constexpr int RED = NW / 2 > 4 ? NW / 2 : 4;
   __shared__ float red[RED][16 * 64];
   constexpr int NSTAGE = (A_KC ? 1 : 0) + (B_KC ? 1 : 0);
@@ -677,6 +677,27 @@ k_gemm_small(const float* __restrict__ A, int lda, const float* __restrict__ B, 
     }
   }
   gemm_draw_idle_streams(tid, NW * 64, epi);
+}
+
+template <bool A_KC, bool B_KC, int NW>
+__global__ void __launch_bounds__(NW * 64)
+k_gemm_small(const float* __restrict__ A, int lda, const float* __restrict__ B, int ldb, float* C, int ldc, int M, int N,
+             int K, float alpha, float beta, bool a_vec, bool b_vec, GemmEpilogue epi) {
+  gemm_small_body<A_KC, B_KC, NW>(A, lda, B, ldb, C, ldc, M, N, K, alpha, beta, a_vec, b_vec, epi);
+}
+
+// The four-wavefront form with up to four sums along the rows (rowsum_jobs.h) behind its blocks, as
+// k_gemm_tile16_sums below.
+template <bool A_KC, bool B_KC>
+__global__ void __launch_bounds__(256)
+k_gemm_small_sums(const float* __restrict__ A, int lda, const float* __restrict__ B, int ldb, float* C, int ldc, int M, int N,
+                  int K, float alpha, float beta, bool a_vec, bool b_vec, GemmEpilogue epi, int gy, RowSumJobs J, int jblocks) {
+  if ((int)blockIdx.y < gy) {
+    gemm_small_body<A_KC, B_KC, 4>(A, lda, B, ldb, C, ldc, M, N, K, alpha, beta, a_vec, b_vec, epi);
+  } else {
+    const int b = ((int)blockIdx.y - gy) * (int)gridDim.x + (int)blockIdx.x;
+    if (b < jblocks) rows_sum_jobs_body(J, b);
+  }
 }
 
 // Two products into the same C, one after the other, in one launch:
@@ -1255,10 +1276,22 @@ static int gemm(bool a_trans, bool b_trans, int M, int N, int K, float alpha, co
       hipLaunchKernelGGL((k_gemm_small<AK, BK_, 8>), grid, dim3(512), 0, dn_stream(), A, lda, B, ldb, C, ldc, M, N, K,  \
                          alpha, beta, a_vec, b_vec, epi);                                                    \
   } while (0)
-    if (a_kc && b_kc) GEMM_SMALL(true, true);
+#define GEMM_SMALL_SUMS(AK, BK_)                                                                              \
+  hipLaunchKernelGGL((k_gemm_small_sums<AK, BK_>), sgrid, dim3(256), 0, dn_stream(), A, lda, B, ldb, C, ldc, M, N, K, \
+                     alpha, beta, a_vec, b_vec, epi, (int)grid.y, *g_side_jobs, g_side_blocks)
+    if (K <= 128 && side_jobs_fit(epi)) {
+      const dim3 sgrid(grid.x, grid.y + (g_side_blocks + grid.x - 1) / grid.x);
+      if (a_kc && b_kc) GEMM_SMALL_SUMS(true, true);
+      else if (a_kc) GEMM_SMALL_SUMS(true, false);
+      else if (b_kc) GEMM_SMALL_SUMS(false, true);
+      else GEMM_SMALL_SUMS(false, false);
+      g_side_blocks = 0;                // taken along
+    }
+    else if (a_kc && b_kc) GEMM_SMALL(true, true);
     else if (a_kc) GEMM_SMALL(true, false);
     else if (b_kc) GEMM_SMALL(false, true);
     else GEMM_SMALL(false, false);
+#undef GEMM_SMALL_SUMS
 #undef GEMM_SMALL
     if (fused) *fused = true;
     if (sampled) *sampled = epi.sample != nullptr;

@@ -105,12 +105,20 @@ struct OpDropMask {
   float* state;
   __device__ __forceinline__ float value(float u, float) const { return u > p ? 1.f : 0.f; }
 };
-// what an op stores besides dst[i] (v: the value stored there, x: what was loaded from src[i])
+// fill_with_rand(r) -> less_than(r, h, target = h) (the hidden sample of cudamat/examples/rbm_cudamat.py:63-65)
+// in one pass: dst gets (u < src ? 1 : 0), uni the uniforms themselves.
+struct OpBernoulliKeep {
+  const float* src; float* dst;
+  float* uni;
+  __device__ __forceinline__ float value(float u, float x) const { return u < x ? 1.f : 0.f; }
+};
+// what an op stores besides dst[i] (u: the draw, v: the value stored in dst[i], x: what was loaded from src[i])
 template <class Op>
-__device__ __forceinline__ void rng_side(const Op&, size_t, float, float) {}
-__device__ __forceinline__ void rng_side(const OpDropMask& op, size_t i, float v, float x) {
+__device__ __forceinline__ void rng_side(const Op&, size_t, float, float, float) {}
+__device__ __forceinline__ void rng_side(const OpDropMask& op, size_t i, float, float v, float x) {
   if (op.state) op.state[i] = x * v;
 }
+__device__ __forceinline__ void rng_side(const OpBernoulliKeep& op, size_t i, float u, float, float) { op.uni[i] = u; }
 
 // Draws [d0, d1) of one stream: element index of draw d is d * 12288 + idx.
 // STREAM: the call is large, use non-temporal accesses.
@@ -128,17 +136,17 @@ __device__ __forceinline__ unsigned long long rng_walk(unsigned long long w, uns
 #pragma unroll
     for (int k = 0; k < RNG_BATCH; ++k) {
       w = mwc_step(w, mult);
-      const float v = op.value(mwc_uniform(w), x[k]);
+      const float u = mwc_uniform(w), v = op.value(u, x[k]);
       dn_st1_rt(op.dst + i + (size_t)k * NUM_RND_STREAMS, v, STREAM);
-      rng_side(op, i + (size_t)k * NUM_RND_STREAMS, v, x[k]);
+      rng_side(op, i + (size_t)k * NUM_RND_STREAMS, u, v, x[k]);
     }
   }
   for (; d < d1; ++d, i += NUM_RND_STREAMS) {
     const float x = op.src ? op.src[i] : 0.f;
     w = mwc_step(w, mult);
-    const float v = op.value(mwc_uniform(w), x);
+    const float u = mwc_uniform(w), v = op.value(u, x);
     op.dst[i] = v;
-    rng_side(op, i, v, x);
+    rng_side(op, i, u, v, x);
   }
   return w;
 }
@@ -190,9 +198,9 @@ k_rng_split(const unsigned int* mults, const unsigned long long* words, unsigned
     if (pp & 1u) w = mwc_montmul(w, table[(size_t)(chbits + b) * NUM_RND_STREAMS + idx], mult);
   auto emit = [&](size_t at, float xv) {
     w = mwc_step(w, mult);
-    const float v = op.value(mwc_uniform(w), xv);
+    const float u = mwc_uniform(w), v = op.value(u, xv);
     __builtin_nontemporal_store(v, op.dst + at);
-    rng_side(op, at, v, xv);
+    rng_side(op, at, u, v, xv);
   };
   if (full0) {
     for (;;) {
@@ -520,6 +528,11 @@ int sample_gaussian(rnd_struct* rnd_state, cudamat* mat, cudamat* target, float 
 int dn_rng_dropmask(rnd_struct* rnd_state, float* mask, float* state, size_t n, float p) {
   if (!rng_ready(rnd_state)) return ERROR_GENERIC;
   return launch_rng(rnd_state, n, OpDropMask{state, mask, p, state});
+}
+
+int dn_rng_bernoulli_keep(rnd_struct* rnd_state, float* uni, float* probs, size_t n) {
+  if (!rng_ready(rnd_state)) return ERROR_GENERIC;
+  return launch_rng(rnd_state, n, OpBernoulliKeep{probs, probs, uni});
 }
 
 extern "C" {

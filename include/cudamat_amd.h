@@ -299,6 +299,7 @@ int get_softmax_cross_entropy(cudamat* mat, cudamat* labels, cudamat* target, fl
  * place (the dropout mask of deepnet/neuralnet.py:194-198) run with it as one pass, same draws and values.
  * Behind a held-back product with lower_bound_scalar(.., 0, ..) such a mask for the product's own target (at most
  * 16 * 12288 elements) is drawn in the product's epilogue: one launch for the six calls of a layer with dropout.
+ * less_than(r, h, h) behind a held-back fill_with_rand(r) is one pass as well (cudamat/examples/rbm_cudamat.py:63-65).
  * softmax / softmax_overwrite are held back too: get_softmax_cross_entropy and apply_softmax_grad (into another
  * matrix) of the result join it and the three run as softmax_ce_grad's launch (deepnet/softmax_layer.py:25-62).
  * set_deferred_epilogues(0) makes every call launch at once; returns the previous setting (default 1).

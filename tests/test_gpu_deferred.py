@@ -230,6 +230,23 @@ def seq_layer_without_mask_then_draw(cm, a, B, bias, other, T, S):
     cm.dot(a, B, target=T); T.lower_bound(0); other.fill_with_randn(); S.fill_with_rand()
 
 
+# the hidden sample as cudamat/examples/rbm_cudamat.py:63-65 spells it: r.fill_with_rand(); r.less_than(h, target=h)
+def seq_sample_by_uniforms(cm, a, B, bias, other, T, S):
+    cm.dot(a, B, target=T); T.add_col_vec(bias); T.apply_sigmoid(); S.fill_with_rand(); S.less_than(T, target=T)
+
+
+def seq_sample_by_uniforms_into_another_target(cm, a, B, bias, other, T, S):
+    T.apply_sigmoid(); S.fill_with_rand(); S.less_than(T, target=other); S.fill_with_rand(); T.less_than(S, target=S)
+
+
+def seq_sample_by_uniforms_behind_a_relu_layer(cm, a, B, bias, other, T, S):
+    cm.dot(a, B, target=T); T.lower_bound(0); S.fill_with_rand(); S.less_than(T, target=T); other.fill_with_rand()
+
+
+def seq_sample_by_uniforms_of_itself(cm, a, B, bias, other, T, S):
+    S.fill_with_rand(); S.less_than(S, target=S); T.fill_with_rand(); T.less_than(other)
+
+
 def seq_dropout_mask_then_read(cm, a, B, bias, other, T, S):
     S.fill_with_rand(); S.greater_than(0.25)
     return S.asarray().view(np.uint32).copy()
@@ -402,7 +419,8 @@ def seq_softmax_gradient_over_the_logits_of_another(cm, a, B, bias, other, T, S)
     return _bits(loss)
 
 
-SEQS = [seq_masked_relu_deriv, seq_masked_deriv_without_activation, seq_factor_then_bias, seq_factor_twice, seq_factor_is_the_target,
+SEQS = [seq_sample_by_uniforms, seq_sample_by_uniforms_into_another_target, seq_sample_by_uniforms_behind_a_relu_layer,
+        seq_sample_by_uniforms_of_itself, seq_masked_relu_deriv, seq_masked_deriv_without_activation, seq_factor_then_bias, seq_factor_twice, seq_factor_is_the_target,
         seq_factor_into_another_target, seq_factor_then_lower_bound, seq_layer_mask_for_another_matrix, seq_layer_mask_unfinished, seq_layer_mask_is_an_operand, seq_layer_mask_then_sample,
         seq_two_layers_with_masks, seq_layer_without_mask_then_draw, seq_softmax_loss_grad, seq_softmax_grad_only, seq_softmax_loss_only_then_read, seq_softmax_alone_then_other_work,
         seq_softmax_grad_in_place, seq_softmax_into_another_target, seq_softmax_loss_of_the_logits, seq_softmax_two_label_vectors,
@@ -682,7 +700,8 @@ def test_the_folded_sequence_is_the_float64_definition(cm, rng):
 def test_training_steps_of_the_bench_keep_their_bits(cm):
     import bench
     for cls, seed, params in ((bench.RBM, 1, lambda o: [o.W, o.bv, o.bh, o.h, o.hs, o.v2, o.h2]),
-                              (bench.MLP, 3, lambda o: o.W + o.b + o.dW + [o.loss] + o.mask)):
+                              (bench.MLP, 3, lambda o: o.W + o.b + o.dW + [o.loss] + o.mask),
+                              (bench.RBMExample, 1, lambda o: [o.w_vh, o.w_v, o.w_h, o.wu_vh, o.wu_v, o.wu_h, o.v, o.h, o.r])):
         res = []
         for deferred in (False, True):
             cm.set_deferred_epilogues(deferred)
@@ -740,7 +759,7 @@ def _random_sequence(cm, rng_ops, pool, vecs, rows, n_ops):
     loss.assign(0)
     reads = []
     for _ in range(n_ops):
-        op = rng_ops.integers(29)
+        op = rng_ops.integers(31)
         a, b, c = M(), M(), M()
         if op == 0: cm.dot(pool.A.T, pool.B, target=a)
         elif op == 1: a.add_dot(pool.A.T, pool.B, mult=scal())
@@ -780,6 +799,8 @@ def _random_sequence(cm, rng_ops, pool, vecs, rows, n_ops):
                 if rng_ops.integers(4): b.greater_than(scal())
                 (a if rng_ops.integers(2) else c).mult(b)
             elif rng_ops.integers(2): a.sample_bernoulli(target=b)
+        elif op == 29: a.less_than(b, target=b if rng_ops.integers(2) else c)
+        elif op == 30: a.fill_with_rand(); a.less_than(b, target=b)
         elif op == 28:      # an output layer and its loss
             a.apply_softmax() if rng_ops.integers(2) else a.apply_softmax(target=b)
             src = a if rng_ops.integers(4) else b
