@@ -1357,6 +1357,7 @@ int dn_gemm_sums(bool a_trans, bool b_trans, int M, int N, int K, float alpha, c
   RowSumJobs J = {};
   const int jblocks = njobs > 0 ? rows_sum_jobs_table(jobs, njobs, &J) : 0;
   if (jblocks < 0) return ERROR_GENERIC;
+  dn_flush();                     // (no other product may be launched from inside this one's launch and take the sums)
   g_side_jobs = &J;
   g_side_blocks = jblocks;
   const int e = gemm(a_trans, b_trans, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc);
